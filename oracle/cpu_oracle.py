@@ -1,0 +1,194 @@
+"""ctypes front-end of the CPU checker (test infrastructure only).
+
+Only tests, the smoke check and the benchmark's CPU-baseline leg load this
+module; the shipped library never does.  Arrays follow the NNTile tile layout:
+Fortran order, which in numpy C-order terms is ``[batch, seq, head]`` for
+K/Q/V/Y, ``[batch, seq]`` for logsumexp and ``[q_seq, k_seq]`` for the mask
+(element (k, q) of the reference's ``[k_seq, q_seq]`` mask sits at
+``k + q*k_seq``).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libnntile_cpu_oracle.so")
+_lib = None
+
+_i64 = ctypes.c_int64
+_f32 = ctypes.c_float
+_ptr = ctypes.c_void_p
+
+
+def build(force=False):
+    """Compile the checker with the Makefile beside this file."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-C", _HERE, "libnntile_cpu_oracle.so"])
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.nntile_oracle_gemm_f32.argtypes = [
+            ctypes.c_int, ctypes.c_int, _i64, _i64, _i64, _i64, _f32, _ptr,
+            _ptr, _f32, _ptr]
+        _lib.nntile_oracle_mask_scalar_f32.argtypes = [_i64, _i64, _ptr, _f32,
+                                                       _ptr]
+        _lib.nntile_oracle_maxsumexp_f32.argtypes = [_i64, _i64, _i64, _ptr,
+                                                     _ptr]
+        _lib.nntile_oracle_softmax_inplace_f32.argtypes = [
+            _i64, _i64, _i64, _ptr, _f32, _ptr]
+        _lib.nntile_oracle_logsumexp_f32.argtypes = [_i64, _ptr, _ptr]
+        _lib.nntile_oracle_accumulate_maxsumexp_f32.argtypes = [_i64, _ptr,
+                                                                _ptr]
+        for name in ("fp32", "bf16", "fp16"):
+            getattr(_lib, "nntile_oracle_accumulate_attn_output_" + name
+                    ).argtypes = [_i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr]
+        for name in ("f32_to_bf16", "bf16_to_f32", "f32_to_fp16",
+                     "fp16_to_f32"):
+            getattr(_lib, "nntile_oracle_" + name).argtypes = [_i64, _ptr,
+                                                               _ptr]
+        _lib.nntile_oracle_sdpa_vanilla_f32.argtypes = [
+            _i64, _i64, _i64, _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr,
+            _ptr, _ptr, ctypes.c_int]
+        _lib.nntile_oracle_sdpa_vanilla_f32.restype = ctypes.c_int
+        _lib.nntile_oracle_sdpa_bruteforce_f64.argtypes = [
+            _i64, _i64, _i64, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]
+        _lib.nntile_oracle_max_threads.restype = ctypes.c_int
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(_ptr)
+
+
+def _c(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def max_threads():
+    return int(lib().nntile_oracle_max_threads())
+
+
+# ---- 16-bit storage helpers (round to nearest even) -----------------------
+
+def f32_to_bf16(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().nntile_oracle_f32_to_bf16(x.size, _p(x), _p(out))
+    return out
+
+
+def bf16_to_f32(x):
+    x = _c(x, np.uint16)
+    out = np.empty(x.shape, np.float32)
+    lib().nntile_oracle_bf16_to_f32(x.size, _p(x), _p(out))
+    return out
+
+
+def f32_to_fp16(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().nntile_oracle_f32_to_fp16(x.size, _p(x), _p(out))
+    return out
+
+
+def fp16_to_f32(x):
+    x = _c(x, np.uint16)
+    out = np.empty(x.shape, np.float32)
+    lib().nntile_oracle_fp16_to_f32(x.size, _p(x), _p(out))
+    return out
+
+
+# ---- codelet-level restatements -------------------------------------------
+
+def gemm(transA, transB, m, n, k, batch, alpha, A, B, beta, C):
+    """Batched column-major GEMM on flat fp32 buffers, C updated in place."""
+    lib().nntile_oracle_gemm_f32(int(transA), int(transB), m, n, k, batch,
+                                 alpha, _p(A), _p(B), beta, _p(C))
+
+
+def mask_scalar(nrows, ncols, mask, val, data):
+    lib().nntile_oracle_mask_scalar_f32(nrows, ncols, _p(mask), val, _p(data))
+
+
+def maxsumexp(m, n, k, src, dst):
+    lib().nntile_oracle_maxsumexp_f32(m, n, k, _p(src), _p(dst))
+
+
+def softmax_inplace(m, n, k, stats, alpha, dst):
+    lib().nntile_oracle_softmax_inplace_f32(m, n, k, _p(stats), alpha, _p(dst))
+
+
+def logsumexp(nelems, stats, out):
+    lib().nntile_oracle_logsumexp_f32(nelems, _p(stats), _p(out))
+
+
+def accumulate_maxsumexp(nelems, src, dst):
+    lib().nntile_oracle_accumulate_maxsumexp_f32(nelems, _p(src), _p(dst))
+
+
+def accumulate_attn_output(dtype, head, seq, batch, src_lse, src_attn,
+                           dst_lse, dst_attn):
+    """dtype in {'fp32','bf16','fp16'}; 16-bit values are uint16 storage."""
+    fn = getattr(lib(), "nntile_oracle_accumulate_attn_output_" + dtype)
+    fn(head, seq, batch, _p(src_lse), _p(src_attn), _p(dst_lse), _p(dst_attn))
+
+
+# ---- the composition --------------------------------------------------------
+
+def sdpa_vanilla(K, Q, V, mask=None, k_tile=0, n_batch=None, kv_repeat=1,
+                 nthreads=0):
+    """gemm -> mask_scalar -> maxsumexp -> softmax_inplace -> gemm on fp32.
+
+    K, V: [kv_batch, k_seq, head]; Q: [batch, q_seq, head] (C-order views of
+    the Fortran tiles); mask: bool [q_seq, k_seq] C-order (= Fortran
+    [k_seq, q_seq]) or None.  Query batch entry b reads K/V entry
+    ``nb + n_batch*hkv`` with ``b = nb + n_batch*(g + kv_repeat*hkv)``.
+    Returns (Y [batch, q_seq, head] fp32, lse [batch, q_seq] fp32).
+    """
+    K = _c(K, np.float32)
+    Q = _c(Q, np.float32)
+    V = _c(V, np.float32)
+    batch, q_seq, head = Q.shape
+    kv_batch, k_seq, _ = K.shape
+    assert V.shape == K.shape and K.shape[2] == head
+    if n_batch is None:
+        if kv_repeat != 1:
+            raise ValueError("n_batch is required when kv_repeat > 1")
+        n_batch = batch
+    assert kv_batch * kv_repeat == batch and batch % (n_batch * kv_repeat) == 0
+    m = None
+    if mask is not None:
+        m = _c(mask, np.uint8)
+        assert m.shape == (q_seq, k_seq)
+    Y = np.empty((batch, q_seq, head), np.float32)
+    lse = np.empty((batch, q_seq), np.float32)
+    rc = lib().nntile_oracle_sdpa_vanilla_f32(
+        head, q_seq, k_seq, batch, n_batch, kv_repeat, k_tile, _p(K), _p(Q),
+        _p(m), _p(V), _p(Y), _p(lse), nthreads)
+    if rc != 0:
+        raise ValueError("bad sizes for sdpa_vanilla")
+    return Y, lse
+
+
+def sdpa_bruteforce_f64(K, Q, V, add_mask=None):
+    """fp64 brute force with an additive [q_seq, k_seq] fp32 mask."""
+    K = _c(K, np.float32)
+    Q = _c(Q, np.float32)
+    V = _c(V, np.float32)
+    batch, q_seq, head = Q.shape
+    k_seq = K.shape[1]
+    m = None if add_mask is None else _c(add_mask, np.float32)
+    A = np.empty((batch, q_seq, head), np.float64)
+    lse = np.empty((batch, q_seq), np.float64)
+    lib().nntile_oracle_sdpa_bruteforce_f64(q_seq, k_seq, head, batch, _p(K),
+                                            _p(Q), _p(m), _p(V), _p(A),
+                                            _p(lse))
+    return A, lse
