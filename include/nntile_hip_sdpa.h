@@ -1,0 +1,210 @@
+/* C ABI of the MI355X (gfx950) tile-level scaled-dot-product-attention forward.
+ *
+ * One shared library, libnntile_hip_sdpa.so, plain pointers and sizes only.
+ * Every entry point only ENQUEUES work on the HIP stream it is given: it never
+ * synchronises, never allocates and never frees.  Return value: 0 on success,
+ * a negative NNTILE_HIP_E* code otherwise (nothing is enqueued on error).
+ *
+ * Data layout (NNTile tiles are Fortran-ordered):
+ *   K, V       [head, k_seq, kv_batch]   element (h, s, b) at h + head*(s + k_seq*b)
+ *   Q, A       [head, q_seq, batch]      element (h, s, b) at h + head*(s + q_seq*b)
+ *   lse        [q_seq, batch]            fp32, natural-log units
+ *   mask       [k_seq, q_seq]            element (k, q) at k + q*k_seq
+ * 16-bit types are passed as their uint16 storage (bf16 / IEEE fp16).
+ * Scores are scaled by 1/sqrt(head) BEFORE the mask is applied.
+ *
+ * Semantics shared by all forward entry points: the call attends the given
+ * queries to the given keys and MERGES the result into the running pair
+ * (lse, A): lse <- logaddexp(lse, lse_new), A <- w_old*A + w_new*A_new.  A
+ * caller starts with lse = -inf (A may hold anything then, it is not read for
+ * such rows) and calls once per key tile, in any order.  A query that sees no
+ * key in this call leaves its lse and A row untouched.
+ */
+#ifndef NNTILE_HIP_SDPA_H
+#define NNTILE_HIP_SDPA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NNTILE_HIP_OK            0
+#define NNTILE_HIP_EINVAL       (-1)  /* null pointer / non-positive size / bad enum */
+#define NNTILE_HIP_EUNSUPPORTED (-2)  /* head size or combination without a kernel */
+#define NNTILE_HIP_ELAUNCH      (-3)  /* the HIP runtime refused the launch */
+#define NNTILE_HIP_EWORKSPACE   (-4)  /* workspace missing or too small */
+
+/* How visibility of key k to query q is given. */
+enum nntile_hip_mask_mode
+{
+    /* mask points at T values [k_seq, q_seq] that are ADDED to the scaled
+     * score: 0 = visible, -inf = hidden.  This is what the reference's flash
+     * codelet receives (src/kernel/flash_sdpa_fwd_cudnn/cuda.cc:103-109). */
+    NNTILE_HIP_MASK_ADDITIVE = 0,
+    /* no mask: every key is visible */
+    NNTILE_HIP_MASK_NONE = 1,
+    /* analytic: key at position k_pos0+k is visible to the query at position
+     * q_pos0+q iff k_pos0+k <= q_pos0+q+causal_offset.  No mask memory is
+     * read and key blocks that are hidden from a whole query block are
+     * skipped. */
+    NNTILE_HIP_MASK_CAUSAL = 2,
+    /* mask points at bytes [k_seq, q_seq]: non-zero = visible.  This is the
+     * reference's vanilla-path mask (src/kernel/mask_scalar/cpu.cc:21-49). */
+    NNTILE_HIP_MASK_BOOL = 3
+};
+
+/* ---- 1. drop-in for the reference kernel call -----------------------------
+ * Replaces kernel::flash_sdpa_fwd_cudnn::execute_graph<T>
+ * (include/nntile/kernel/flash_sdpa_fwd_cudnn/cuda.hh:61-76,
+ *  src/kernel/flash_sdpa_fwd_cudnn/cuda.cc:145-202): same argument order and
+ * meaning, the cuDNN handle/graph pair replaced by the stream.  One square
+ * tile: seq queries against seq keys, additive mask [seq, seq] in T.
+ * scratch_lse and scratch_A are accepted for signature compatibility and
+ * never touched (the merge is fused into the kernel); they may be null. */
+int nntile_hip_flash_sdpa_fwd_bf16(void *stream, int64_t seq, int64_t head,
+        int64_t batch, const uint16_t *K, const uint16_t *Q,
+        const uint16_t *mask, float *scratch_lse, const uint16_t *V,
+        uint16_t *scratch_A, float *lse, uint16_t *A);
+int nntile_hip_flash_sdpa_fwd_fp16(void *stream, int64_t seq, int64_t head,
+        int64_t batch, const uint16_t *K, const uint16_t *Q,
+        const uint16_t *mask, float *scratch_lse, const uint16_t *V,
+        uint16_t *scratch_A, float *lse, uint16_t *A);
+/* fp32 has no counterpart in the reference's flash pack
+ * (include/nntile/starpu/flash_sdpa_fwd_cudnn.hh:149-153 lists bf16, fp16);
+ * it is added so that fp32 models take the same path. */
+int nntile_hip_flash_sdpa_fwd_fp32(void *stream, int64_t seq, int64_t head,
+        int64_t batch, const float *K, const float *Q, const float *mask,
+        float *scratch_lse, const float *V, float *scratch_A, float *lse,
+        float *A);
+
+/* ---- 2. one (query tile, key tile) pair, general form ----------------------
+ * What tile::flash_sdpa_fwd_cudnn_async (src/tile/flash_sdpa_fwd_cudnn.cc:
+ * 161-196) would submit if tiles need not be square and the mask need not be
+ * materialised.  Query batch entry b reads key/value entry
+ *   (b % n_batch) + n_batch * (b / (n_batch*kv_group)),
+ * i.e. Q is [head, q_seq, n_batch, kv_group, n_head_kv] and K/V are
+ * [head, k_seq, n_batch, n_head_kv] without the per-group repeat of
+ * wrappers/python/nntile/model/llama_attention.py:579-580; kv_group = 1 and
+ * n_batch = batch give the plain one-to-one case. */
+typedef struct nntile_hip_sdpa_tile_args
+{
+    int64_t q_seq, k_seq, head;
+    int64_t batch;        /* flattened query batch */
+    int64_t n_batch;      /* size of the innermost batch axis shared by Q and K/V */
+    int64_t kv_group;     /* query heads per key/value head */
+    int32_t mask_mode;    /* enum nntile_hip_mask_mode */
+    int32_t reserved;
+    int64_t q_pos0, k_pos0, causal_offset;   /* NNTILE_HIP_MASK_CAUSAL only */
+    const void *K, *Q, *mask, *V;
+    float *lse;
+    void *A;
+} nntile_hip_sdpa_tile_args;
+
+int nntile_hip_sdpa_fwd_tile_bf16(void *stream, const nntile_hip_sdpa_tile_args *args);
+int nntile_hip_sdpa_fwd_tile_fp16(void *stream, const nntile_hip_sdpa_tile_args *args);
+int nntile_hip_sdpa_fwd_tile_fp32(void *stream, const nntile_hip_sdpa_tile_args *args);
+
+/* ---- 3. a whole grid of tiles in one launch ---------------------------------
+ * What tensor::flash_sdpa_fwd_cudnn_async (src/tensor/flash_sdpa_fwd_cudnn.cc:
+ * 210-279) computes when every tile of one (batch, head) slab is resident on
+ * this GPU: for each query tile, all key tiles are merged in one pass with the
+ * output kept in registers, instead of one task (and one round trip of A
+ * through T) per tile pair.  Tiles are separate allocations, as in NNTile;
+ * all query tiles hold q_tile rows and all key tiles k_tile rows, except the
+ * last of each, which holds the remainder of q_seq / k_seq.  Only the
+ * analytic masks (NONE, CAUSAL) are accepted; positions count from row 0 of
+ * tile 0 plus q_pos0 / k_pos0. */
+#define NNTILE_HIP_SDPA_MAX_TILES 64
+
+typedef struct nntile_hip_sdpa_grid_args
+{
+    int64_t q_seq, k_seq, q_tile, k_tile, head;
+    int64_t batch, n_batch, kv_group;
+    int32_t mask_mode, n_q_tiles, n_kv_tiles, reserved;
+    int64_t q_pos0, k_pos0, causal_offset;
+    const void *K[NNTILE_HIP_SDPA_MAX_TILES];
+    const void *V[NNTILE_HIP_SDPA_MAX_TILES];
+    const void *Q[NNTILE_HIP_SDPA_MAX_TILES];
+    float *lse[NNTILE_HIP_SDPA_MAX_TILES];
+    void *A[NNTILE_HIP_SDPA_MAX_TILES];
+} nntile_hip_sdpa_grid_args;
+
+int nntile_hip_sdpa_fwd_grid_bf16(void *stream, const nntile_hip_sdpa_grid_args *args);
+int nntile_hip_sdpa_fwd_grid_fp16(void *stream, const nntile_hip_sdpa_grid_args *args);
+int nntile_hip_sdpa_fwd_grid_fp32(void *stream, const nntile_hip_sdpa_grid_args *args);
+
+/* ---- 4. short-query / long-key decode ----------------------------------------
+ * The shape of LlamaAttention.forward_dynamic
+ * (wrappers/python/nntile/model/llama_attention.py:627-760), which in the
+ * reference repeats K/V per group and runs the vanilla composition.  Here the
+ * kv_group query heads of one key/value head share one pass over the cache,
+ * and the key axis is split over workgroups; partial results are merged with
+ * the accumulate_attn_output rule.  args->q_seq*kv_group must be <= 64.
+ * workspace: device memory of at least
+ * nntile_hip_sdpa_fwd_decode_workspace_bytes(args) bytes, private to the call
+ * until the stream has passed it (a STARPU_SCRATCH buffer in NNTile terms). */
+size_t nntile_hip_sdpa_fwd_decode_workspace_bytes(const nntile_hip_sdpa_tile_args *args);
+int nntile_hip_sdpa_fwd_decode_bf16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        void *workspace, size_t workspace_bytes);
+int nntile_hip_sdpa_fwd_decode_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        void *workspace, size_t workspace_bytes);
+
+/* ---- 5. the running-statistics hand-off on its own ---------------------------
+ * Replaces kernel::accumulate_attn_output::cuda<T>
+ * (src/kernel/accumulate_attn_output/cuda.cu:115-135; CPU statement
+ * src/kernel/accumulate_attn_output/cpu.cc:38-115): merges (src_lse, src_attn)
+ * into (dst_lse, dst_attn) for seq*batch rows of head values. */
+int nntile_hip_accumulate_attn_output_bf16(void *stream, int64_t head, int64_t seq,
+        int64_t batch, const float *src_lse, const uint16_t *src_attn,
+        float *dst_lse, uint16_t *dst_attn);
+int nntile_hip_accumulate_attn_output_fp16(void *stream, int64_t head, int64_t seq,
+        int64_t batch, const float *src_lse, const uint16_t *src_attn,
+        float *dst_lse, uint16_t *dst_attn);
+int nntile_hip_accumulate_attn_output_fp32(void *stream, int64_t head, int64_t seq,
+        int64_t batch, const float *src_lse, const float *src_attn,
+        float *dst_lse, float *dst_attn);
+
+/* ---- 6. StarPU codelet bodies ---------------------------------------------------
+ * Same shape as FlashSdpaFwdCudnn<T>::cuda(void *buffers[], void *cl_args)
+ * (src/starpu/flash_sdpa_fwd_cudnn.cc:60-155), to be placed in the codelet's
+ * hip_funcs[0] with STARPU_HIP_ASYNC.  buffers[i] point at StarPU variable
+ * interfaces in the reference's order: K(R) Q(R) mask(R) lse(RW) V(R) A(RW)
+ * scratch_lse(SCRATCH) scratch_A(SCRATCH); cl_args points at
+ * nntile_hip_flash_sdpa_cl_args, whose first four members are the
+ * reference's args_t (include/nntile/starpu/flash_sdpa_fwd_cudnn.hh:58-64).
+ * Errors are reported on stderr and the task becomes a no-op, as in the
+ * reference.  The stream comes from the function registered with
+ * nntile_hip_set_stream_provider (starpu_hip_get_local_stream in a StarPU
+ * build); without a provider the null stream is used. */
+typedef struct nntile_hip_variable_interface
+{
+    int id;              /* enum starpu_data_interface_id */
+    uintptr_t ptr;       /* device pointer of the tile */
+    uintptr_t dev_handle;
+    size_t offset;
+    size_t elemsize;
+} nntile_hip_variable_interface;
+
+typedef struct nntile_hip_flash_sdpa_cl_args
+{
+    void *owner;
+    int64_t seq, head, batch;
+} nntile_hip_flash_sdpa_cl_args;
+
+typedef void *(*nntile_hip_stream_provider)(void);
+void nntile_hip_set_stream_provider(nntile_hip_stream_provider fn);
+
+void nntile_hip_flash_sdpa_fwd_codelet_bf16(void *buffers[], void *cl_args);
+void nntile_hip_flash_sdpa_fwd_codelet_fp16(void *buffers[], void *cl_args);
+void nntile_hip_flash_sdpa_fwd_codelet_fp32(void *buffers[], void *cl_args);
+
+/* Library version and the ISA it was built for ("gfx950"). */
+const char *nntile_hip_sdpa_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NNTILE_HIP_SDPA_H */

@@ -1,0 +1,453 @@
+// C ABI of libnntile_hip_sdpa.so: argument checks and dispatch to the kernels.
+#include <cstdio>
+#include <cstring>
+
+#include "sdpa_common.hpp"
+
+namespace nntile_hip
+{
+
+template<typename T>
+int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head, int mode);
+int launch_prefill_fp32(hipStream_t stream, PrefillParams &p, int head, int mode);
+
+template<typename T>
+int launch_decode_16bit(hipStream_t stream, DecodeParams &p, int head, int mode);
+int decode_choose_splits(int units, int n_steps);
+size_t decode_workspace_bytes(int units, int n_splits, int rows, int head);
+
+struct F32Store;
+struct Bf16Store;
+struct Fp16Store;
+template<typename S>
+int launch_accumulate(hipStream_t stream, int64_t head, int64_t seq,
+        int64_t batch, const float *src_lse, const void *src_attn,
+        float *dst_lse, void *dst_attn);
+
+enum class DType { bf16, fp16, fp32 };
+
+static bool aligned16(const void *p)
+{
+    return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+static bool mode_ok(int mode)
+{
+    return mode >= NNTILE_HIP_MASK_ADDITIVE && mode <= NNTILE_HIP_MASK_BOOL;
+}
+
+static int dispatch_prefill(DType dt, hipStream_t stream, PrefillParams &p,
+        int64_t head, int mode)
+{
+    if(head != 32 && head != 64 && head != 128)
+    {
+        return NNTILE_HIP_EUNSUPPORTED;
+    }
+    p.scale = 1.0f / sqrtf(static_cast<float>(head));
+    switch(dt)
+    {
+        case DType::bf16:
+            return launch_prefill_16bit<Bf16>(stream, p, (int)head, mode);
+        case DType::fp16:
+            return launch_prefill_16bit<Fp16>(stream, p, (int)head, mode);
+        default:
+            return launch_prefill_fp32(stream, p, (int)head, mode);
+    }
+}
+
+static int tile_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a)
+{
+    if(a == nullptr || a->q_seq <= 0 || a->k_seq <= 0 || a->head <= 0
+            || a->batch <= 0 || a->n_batch <= 0 || a->kv_group <= 0
+            || !mode_ok(a->mask_mode) || a->K == nullptr || a->Q == nullptr
+            || a->V == nullptr || a->lse == nullptr || a->A == nullptr
+            || a->batch % (a->n_batch * a->kv_group) != 0
+            || a->batch > 0x7fffffff || a->q_seq > 0x7fffffff
+            || a->k_seq > 0x7fffffff)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    const bool explicit_mask = a->mask_mode == NNTILE_HIP_MASK_ADDITIVE
+        || a->mask_mode == NNTILE_HIP_MASK_BOOL;
+    if(explicit_mask && a->mask == nullptr)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(!aligned16(a->K) || !aligned16(a->Q) || !aligned16(a->V)
+            || !aligned16(a->A))
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    PrefillParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.q_seq = p.q_tile = a->q_seq;
+    p.k_seq = p.k_tile = a->k_seq;
+    p.q_pos0 = a->q_pos0;
+    p.k_pos0 = a->k_pos0;
+    p.causal_offset = a->causal_offset;
+    p.mask = a->mask;
+    p.mask_ld = a->k_seq;
+    p.n_q_tiles = p.n_kv_tiles = 1;
+    p.batch = (int32_t)a->batch;
+    p.n_batch = (int32_t)a->n_batch;
+    p.kv_group = (int32_t)a->kv_group;
+    p.K[0] = a->K;
+    p.V[0] = a->V;
+    p.Q[0] = a->Q;
+    p.lse[0] = a->lse;
+    p.A[0] = a->A;
+    return dispatch_prefill(dt, static_cast<hipStream_t>(stream), p, a->head,
+            a->mask_mode);
+}
+
+static int flash_call(DType dt, void *stream, int64_t seq, int64_t head,
+        int64_t batch, const void *K, const void *Q, const void *mask,
+        const void *V, float *lse, void *A)
+{
+    nntile_hip_sdpa_tile_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.q_seq = a.k_seq = seq;
+    a.head = head;
+    a.batch = batch;
+    a.n_batch = batch;
+    a.kv_group = 1;
+    a.mask_mode = NNTILE_HIP_MASK_ADDITIVE;
+    a.K = K;
+    a.Q = Q;
+    a.mask = mask;
+    a.V = V;
+    a.lse = lse;
+    a.A = A;
+    return tile_call(dt, stream, &a);
+}
+
+static int grid_call(DType dt, void *stream, const nntile_hip_sdpa_grid_args *a)
+{
+    if(a == nullptr || a->q_seq <= 0 || a->k_seq <= 0 || a->q_tile <= 0
+            || a->k_tile <= 0 || a->head <= 0 || a->batch <= 0
+            || a->n_batch <= 0 || a->kv_group <= 0
+            || a->batch % (a->n_batch * a->kv_group) != 0
+            || a->batch > 0x7fffffff || a->q_seq > 0x7fffffff
+            || a->k_seq > 0x7fffffff
+            || a->n_q_tiles <= 0 || a->n_q_tiles > NNTILE_HIP_SDPA_MAX_TILES
+            || a->n_kv_tiles <= 0 || a->n_kv_tiles > NNTILE_HIP_SDPA_MAX_TILES)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(a->mask_mode != NNTILE_HIP_MASK_NONE
+            && a->mask_mode != NNTILE_HIP_MASK_CAUSAL)
+    {
+        return mode_ok(a->mask_mode) ? NNTILE_HIP_EUNSUPPORTED
+            : NNTILE_HIP_EINVAL;
+    }
+    // the tile counts must match the extents
+    if((a->q_seq + a->q_tile - 1) / a->q_tile != a->n_q_tiles
+            || (a->k_seq + a->k_tile - 1) / a->k_tile != a->n_kv_tiles)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    PrefillParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.q_seq = a->q_seq;
+    p.k_seq = a->k_seq;
+    p.q_tile = a->q_tile;
+    p.k_tile = a->k_tile;
+    p.q_pos0 = a->q_pos0;
+    p.k_pos0 = a->k_pos0;
+    p.causal_offset = a->causal_offset;
+    p.n_q_tiles = a->n_q_tiles;
+    p.n_kv_tiles = a->n_kv_tiles;
+    p.batch = (int32_t)a->batch;
+    p.n_batch = (int32_t)a->n_batch;
+    p.kv_group = (int32_t)a->kv_group;
+    for(int t = 0; t < a->n_kv_tiles; ++t)
+    {
+        if(a->K[t] == nullptr || a->V[t] == nullptr || !aligned16(a->K[t])
+                || !aligned16(a->V[t]))
+        {
+            return NNTILE_HIP_EINVAL;
+        }
+        p.K[t] = a->K[t];
+        p.V[t] = a->V[t];
+    }
+    for(int t = 0; t < a->n_q_tiles; ++t)
+    {
+        if(a->Q[t] == nullptr || a->A[t] == nullptr || a->lse[t] == nullptr
+                || !aligned16(a->Q[t]) || !aligned16(a->A[t]))
+        {
+            return NNTILE_HIP_EINVAL;
+        }
+        p.Q[t] = a->Q[t];
+        p.A[t] = a->A[t];
+        p.lse[t] = a->lse[t];
+    }
+    return dispatch_prefill(dt, static_cast<hipStream_t>(stream), p, a->head,
+            a->mask_mode);
+}
+
+static bool decode_args_ok(const nntile_hip_sdpa_tile_args *a)
+{
+    return a != nullptr && a->q_seq > 0 && a->k_seq > 0 && a->head > 0
+        && a->batch > 0 && a->n_batch > 0 && a->kv_group > 0
+        && a->batch % (a->n_batch * a->kv_group) == 0
+        && a->batch <= 0x7fffffff && a->k_seq <= 0x7fffffff
+        && a->q_seq * a->kv_group <= 64;
+}
+
+static void decode_geometry(const nntile_hip_sdpa_tile_args *a, int &units,
+        int &n_steps, int &splits, int &rows)
+{
+    units = (int)(a->batch / a->kv_group);
+    n_steps = (int)((a->k_seq + 63) / 64);
+    splits = decode_choose_splits(units, n_steps);
+    rows = (int)(a->q_seq * a->kv_group);
+}
+
+static int decode_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a,
+        void *workspace, size_t workspace_bytes)
+{
+    if(!decode_args_ok(a) || !mode_ok(a->mask_mode) || a->K == nullptr
+            || a->Q == nullptr || a->V == nullptr || a->lse == nullptr
+            || a->A == nullptr || !aligned16(a->K) || !aligned16(a->Q)
+            || !aligned16(a->V) || !aligned16(a->A))
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    const bool explicit_mask = a->mask_mode == NNTILE_HIP_MASK_ADDITIVE
+        || a->mask_mode == NNTILE_HIP_MASK_BOOL;
+    if(explicit_mask && a->mask == nullptr)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(a->head != 64 && a->head != 128)
+    {
+        return NNTILE_HIP_EUNSUPPORTED;
+    }
+    int units, n_steps, splits, rows;
+    decode_geometry(a, units, n_steps, splits, rows);
+    const size_t need = decode_workspace_bytes(units, splits, rows, (int)a->head);
+    if(workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+    {
+        return NNTILE_HIP_EWORKSPACE;
+    }
+    DecodeParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.q_seq = a->q_seq;
+    p.k_seq = a->k_seq;
+    p.q_pos0 = a->q_pos0;
+    p.k_pos0 = a->k_pos0;
+    p.causal_offset = a->causal_offset;
+    p.mask = a->mask;
+    p.mask_ld = a->k_seq;
+    p.K = a->K;
+    p.V = a->V;
+    p.Q = a->Q;
+    p.lse = a->lse;
+    p.A = a->A;
+    p.part_o = static_cast<float *>(workspace);
+    p.part_ml = p.part_o + (size_t)units * splits * rows * a->head;
+    p.n_batch = (int32_t)a->n_batch;
+    p.kv_group = (int32_t)a->kv_group;
+    p.n_head_kv = (int32_t)(units / a->n_batch);
+    p.rows = rows;
+    p.n_splits = splits;
+    p.n_steps = n_steps;
+    p.steps_per_split = (n_steps + splits - 1) / splits;
+    p.scale = 1.0f / sqrtf(static_cast<float>(a->head));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dt == DType::bf16 ? launch_decode_16bit<Bf16>(s, p, (int)a->head, a->mask_mode)
+        : launch_decode_16bit<Fp16>(s, p, (int)a->head, a->mask_mode);
+}
+
+template<typename S>
+static int accumulate_call(void *stream, int64_t head, int64_t seq,
+        int64_t batch, const float *src_lse, const void *src_attn,
+        float *dst_lse, void *dst_attn)
+{
+    if(head <= 0 || seq <= 0 || batch <= 0)
+    {
+        return NNTILE_HIP_OK;   // the reference kernel returns silently
+    }
+    if(src_lse == nullptr || src_attn == nullptr || dst_lse == nullptr
+            || dst_attn == nullptr)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    return launch_accumulate<S>(static_cast<hipStream_t>(stream), head, seq,
+            batch, src_lse, src_attn, dst_lse, dst_attn);
+}
+
+static nntile_hip_stream_provider g_stream_provider = nullptr;
+
+static void codelet_call(DType dt, const char *name, void *buffers[],
+        void *cl_args)
+{
+    // Error behaviour of the reference body: report and return, the task
+    // becomes a no-op (src/starpu/flash_sdpa_fwd_cudnn.cc:69-115).
+    if(buffers == nullptr || cl_args == nullptr)
+    {
+        std::fprintf(stderr, "HIP Worker: %s: null buffers or arguments, "
+                "skipping task\n", name);
+        return;
+    }
+    const auto *args = static_cast<const nntile_hip_flash_sdpa_cl_args *>(cl_args);
+    auto **ifs = reinterpret_cast<nntile_hip_variable_interface **>(buffers);
+    for(int i = 0; i < 6; ++i)
+    {
+        if(ifs[i] == nullptr)
+        {
+            std::fprintf(stderr, "HIP Worker: %s: buffer %d is null, skipping "
+                    "task\n", name, i);
+            return;
+        }
+    }
+    void *stream = g_stream_provider ? g_stream_provider() : nullptr;
+    const int rc = flash_call(dt, stream, args->seq, args->head, args->batch,
+            reinterpret_cast<const void *>(ifs[0]->ptr),
+            reinterpret_cast<const void *>(ifs[1]->ptr),
+            reinterpret_cast<const void *>(ifs[2]->ptr),
+            reinterpret_cast<const void *>(ifs[4]->ptr),
+            reinterpret_cast<float *>(ifs[3]->ptr),
+            reinterpret_cast<void *>(ifs[5]->ptr));
+    if(rc != NNTILE_HIP_OK)
+    {
+        std::fprintf(stderr, "HIP Worker: %s: launch failed with code %d "
+                "(seq=%lld head=%lld batch=%lld), skipping task\n", name, rc,
+                (long long)args->seq, (long long)args->head,
+                (long long)args->batch);
+    }
+}
+
+} // namespace nntile_hip
+
+using namespace nntile_hip;
+
+extern "C"
+{
+
+int nntile_hip_flash_sdpa_fwd_bf16(void *stream, int64_t seq, int64_t head,
+        int64_t batch, const uint16_t *K, const uint16_t *Q,
+        const uint16_t *mask, float *, const uint16_t *V, uint16_t *,
+        float *lse, uint16_t *A)
+{
+    return flash_call(DType::bf16, stream, seq, head, batch, K, Q, mask, V, lse, A);
+}
+
+int nntile_hip_flash_sdpa_fwd_fp16(void *stream, int64_t seq, int64_t head,
+        int64_t batch, const uint16_t *K, const uint16_t *Q,
+        const uint16_t *mask, float *, const uint16_t *V, uint16_t *,
+        float *lse, uint16_t *A)
+{
+    return flash_call(DType::fp16, stream, seq, head, batch, K, Q, mask, V, lse, A);
+}
+
+int nntile_hip_flash_sdpa_fwd_fp32(void *stream, int64_t seq, int64_t head,
+        int64_t batch, const float *K, const float *Q, const float *mask,
+        float *, const float *V, float *, float *lse, float *A)
+{
+    return flash_call(DType::fp32, stream, seq, head, batch, K, Q, mask, V, lse, A);
+}
+
+int nntile_hip_sdpa_fwd_tile_bf16(void *stream, const nntile_hip_sdpa_tile_args *args)
+{
+    return tile_call(DType::bf16, stream, args);
+}
+
+int nntile_hip_sdpa_fwd_tile_fp16(void *stream, const nntile_hip_sdpa_tile_args *args)
+{
+    return tile_call(DType::fp16, stream, args);
+}
+
+int nntile_hip_sdpa_fwd_tile_fp32(void *stream, const nntile_hip_sdpa_tile_args *args)
+{
+    return tile_call(DType::fp32, stream, args);
+}
+
+int nntile_hip_sdpa_fwd_grid_bf16(void *stream, const nntile_hip_sdpa_grid_args *args)
+{
+    return grid_call(DType::bf16, stream, args);
+}
+
+int nntile_hip_sdpa_fwd_grid_fp16(void *stream, const nntile_hip_sdpa_grid_args *args)
+{
+    return grid_call(DType::fp16, stream, args);
+}
+
+int nntile_hip_sdpa_fwd_grid_fp32(void *stream, const nntile_hip_sdpa_grid_args *args)
+{
+    return grid_call(DType::fp32, stream, args);
+}
+
+size_t nntile_hip_sdpa_fwd_decode_workspace_bytes(const nntile_hip_sdpa_tile_args *args)
+{
+    if(!decode_args_ok(args))
+    {
+        return 0;
+    }
+    int units, n_steps, splits, rows;
+    decode_geometry(args, units, n_steps, splits, rows);
+    return decode_workspace_bytes(units, splits, rows, (int)args->head);
+}
+
+int nntile_hip_sdpa_fwd_decode_bf16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        void *workspace, size_t workspace_bytes)
+{
+    return decode_call(DType::bf16, stream, args, workspace, workspace_bytes);
+}
+
+int nntile_hip_sdpa_fwd_decode_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        void *workspace, size_t workspace_bytes)
+{
+    return decode_call(DType::fp16, stream, args, workspace, workspace_bytes);
+}
+
+int nntile_hip_accumulate_attn_output_bf16(void *stream, int64_t head, int64_t seq,
+        int64_t batch, const float *src_lse, const uint16_t *src_attn,
+        float *dst_lse, uint16_t *dst_attn)
+{
+    return accumulate_call<Bf16Store>(stream, head, seq, batch, src_lse, src_attn,
+            dst_lse, dst_attn);
+}
+
+int nntile_hip_accumulate_attn_output_fp16(void *stream, int64_t head, int64_t seq,
+        int64_t batch, const float *src_lse, const uint16_t *src_attn,
+        float *dst_lse, uint16_t *dst_attn)
+{
+    return accumulate_call<Fp16Store>(stream, head, seq, batch, src_lse, src_attn,
+            dst_lse, dst_attn);
+}
+
+int nntile_hip_accumulate_attn_output_fp32(void *stream, int64_t head, int64_t seq,
+        int64_t batch, const float *src_lse, const float *src_attn,
+        float *dst_lse, float *dst_attn)
+{
+    return accumulate_call<F32Store>(stream, head, seq, batch, src_lse, src_attn,
+            dst_lse, dst_attn);
+}
+
+void nntile_hip_set_stream_provider(nntile_hip_stream_provider fn)
+{
+    g_stream_provider = fn;
+}
+
+void nntile_hip_flash_sdpa_fwd_codelet_bf16(void *buffers[], void *cl_args)
+{
+    codelet_call(DType::bf16, "nntile_flash_sdpa_fwd_hip_bf16", buffers, cl_args);
+}
+
+void nntile_hip_flash_sdpa_fwd_codelet_fp16(void *buffers[], void *cl_args)
+{
+    codelet_call(DType::fp16, "nntile_flash_sdpa_fwd_hip_fp16", buffers, cl_args);
+}
+
+void nntile_hip_flash_sdpa_fwd_codelet_fp32(void *buffers[], void *cl_args)
+{
+    codelet_call(DType::fp32, "nntile_flash_sdpa_fwd_hip_fp32", buffers, cl_args);
+}
+
+const char *nntile_hip_sdpa_version(void)
+{
+    return "nntile_hip_sdpa 0.1 (gfx950)";
+}
+
+} // extern "C"

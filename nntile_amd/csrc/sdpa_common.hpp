@@ -1,0 +1,154 @@
+// Shared device-side definitions of the gfx950 attention kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/nntile_hip_sdpa.h"
+
+namespace nntile_hip
+{
+
+constexpr int kMaxTiles = NNTILE_HIP_SDPA_MAX_TILES;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+// Kernel arguments of the prefill kernels (passed by value in the kernarg
+// segment).  Query tile t holds rows [t*q_tile, min((t+1)*q_tile, q_seq)),
+// the same for key tiles.
+struct PrefillParams
+{
+    int64_t q_seq, k_seq, q_tile, k_tile;
+    int64_t q_pos0, k_pos0, causal_offset;
+    int64_t mask_ld;              // = k_seq of the single key tile (explicit masks)
+    const void *mask;
+    int32_t n_q_tiles, n_kv_tiles;
+    int32_t batch, n_batch, kv_group;
+    int32_t q_blocks_per_tile;    // ceil(q_tile / rows per workgroup)
+    int32_t k_blocks_per_tile;    // ceil(k_tile / keys per step)
+    int32_t xcd_remap;            // 1: regroup workgroups so a slab stays on one XCD
+    float scale;                  // 1/sqrt(head)
+    const void *K[kMaxTiles];
+    const void *V[kMaxTiles];
+    const void *Q[kMaxTiles];
+    float *lse[kMaxTiles];
+    void *A[kMaxTiles];
+};
+
+// Kernel arguments of the decode kernels.  K, V: [head, k_seq, n_batch,
+// n_head_kv]; Q, A: [head, q_seq, n_batch, kv_group, n_head_kv].
+struct DecodeParams
+{
+    int64_t q_seq, k_seq;
+    int64_t q_pos0, k_pos0, causal_offset;
+    int64_t mask_ld;
+    const void *mask;
+    const void *K, *V, *Q;
+    float *lse;
+    void *A;
+    float *part_o;      // [unit][split][rows][HEAD]
+    float *part_ml;     // [unit][split][rows][2]
+    int32_t n_batch, kv_group, n_head_kv;
+    int32_t rows;       // kv_group * q_seq
+    int32_t n_splits, steps_per_split, n_steps;
+    float scale;
+};
+
+__device__ __forceinline__ float fast_exp2(float x)
+{
+    return __builtin_amdgcn_exp2f(x);
+}
+
+__device__ __forceinline__ float neg_inf()
+{
+    return -__builtin_huge_valf();
+}
+
+// Storage <-> float for the 16-bit tile types.
+struct Bf16
+{
+    typedef bf16x8 vec8;
+    static __device__ __forceinline__ float to_float(uint16_t v)
+    {
+        return __uint_as_float(static_cast<uint32_t>(v) << 16);
+    }
+    static __device__ __forceinline__ uint16_t from_float(float f)
+    {
+        __bf16 h = static_cast<__bf16>(f);   // round to nearest even
+        return __builtin_bit_cast(uint16_t, h);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+        typedef __attribute__((ext_vector_type(2))) float f32x2;
+        f32x2 v = {lo, hi};
+        bf16x2 h = __builtin_convertvector(v, bf16x2);
+        return __builtin_bit_cast(uint32_t, h);
+    }
+    static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
+struct Fp16
+{
+    typedef f16x8 vec8;
+    static __device__ __forceinline__ float to_float(uint16_t v)
+    {
+        return static_cast<float>(__builtin_bit_cast(_Float16, v));
+    }
+    static __device__ __forceinline__ uint16_t from_float(float f)
+    {
+        _Float16 h = static_cast<_Float16>(f);
+        return __builtin_bit_cast(uint16_t, h);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+        typedef __attribute__((ext_vector_type(2))) float f32x2;
+        f32x2 v = {lo, hi};
+        f16x2 h = __builtin_convertvector(v, f16x2);
+        return __builtin_bit_cast(uint32_t, h);
+    }
+    static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// Key/value batch entry read by query batch entry b.
+__device__ __forceinline__ int kv_entry(int b, int n_batch, int kv_group)
+{
+    return (b % n_batch) + n_batch * (b / (n_batch * kv_group));
+}
+
+// Merge of a fresh (lse_new, value) into the running pair, per row:
+// returns the weights and the merged lse.  lse_new must be finite.
+__device__ __forceinline__ void merge_weights(float lse_old, float lse_new,
+        float &w_old, float &w_new, float &lse_out)
+{
+    if(lse_old == neg_inf())
+    {
+        w_old = 0.0f;
+        w_new = 1.0f;
+        lse_out = lse_new;
+        return;
+    }
+    const float top = fmaxf(lse_old, lse_new);
+    const float e_old = __expf(lse_old - top), e_new = __expf(lse_new - top);
+    const float sum = e_old + e_new;
+    const float inv = 1.0f / sum;
+    w_old = e_old * inv;
+    w_new = e_new * inv;
+    lse_out = top + __logf(sum);
+}
+
+} // namespace nntile_hip

@@ -1,0 +1,525 @@
+// Prefill attention forward for 16-bit tiles (bf16 / fp16) on gfx950.
+//
+// One workgroup = 4 wavefronts = 128 queries of one (batch entry, query tile);
+// each wavefront owns 32 queries.  Keys are walked in steps of 64.
+//
+//   S^T = K Q^T    v_mfma_f32_32x32x16: A = 32 keys x 16 head values read from
+//                  LDS, B = 16 head values x 32 queries held in registers for
+//                  the whole kernel.  In the 32x32 accumulator layout a lane
+//                  holds ONE query (lane % 32) and 16 of the 32 keys, so the
+//                  row maximum and the row sum of the softmax are reductions
+//                  over the lane's own registers plus one exchange with lane^32.
+//   O^T += V^T P^T A = 32 head values x 16 keys read from LDS, B = P^T taken
+//                  straight from the S^T accumulators (converted to 16 bit) -
+//                  the accumulator layout of the first product IS the B layout
+//                  of the second, up to a fixed permutation of the 16 keys,
+//                  and V^T is stored in LDS in that permuted key order.
+//
+// V arrives with the head axis contiguous but the second product contracts
+// over keys, so V is transposed on its way into LDS: a thread fetches 4 keys x
+// 8 head values, regroups them in registers and writes 8 x (4 keys) so that
+// every MFMA operand is a single 16-byte LDS read.
+//
+// The running (max, sum) pair lives in registers across all key tiles of a
+// query tile; the epilogue merges the result into the (lse, A) pair in memory
+// (the hand-off between NNTile tasks), so one launch can stand for one task or
+// for a whole row of tasks.
+#include "sdpa_common.hpp"
+
+namespace nntile_hip
+{
+
+constexpr int kQRows = 128;     // queries per workgroup
+constexpr int kKeys = 64;       // keys per step
+constexpr int kThreads = 256;
+
+template<typename T, int HEAD, int MODE>
+__global__ __launch_bounds__(kThreads, 2)
+void sdpa_prefill_16bit_kernel(const PrefillParams p)
+{
+    typedef typename T::vec8 vec8;
+    constexpr int KSTEPS = HEAD / 16;       // MFMA steps along head for S
+    constexpr int DBLOCKS = HEAD / 32;      // 32-row blocks of O^T
+    constexpr int KPAD = HEAD + 8;          // K row stride in LDS (elements)
+    constexpr int VPAD = kKeys + 8;         // V^T row stride in LDS
+    constexpr int CHUNKS = HEAD / 8;        // 16-byte chunks per row
+    constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
+            || MODE == NNTILE_HIP_MASK_BOOL);
+
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[kKeys * KPAD];
+    __shared__ __attribute__((aligned(16))) uint16_t Vt[HEAD * VPAD];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int col = lane & 31;      // query within the wavefront / row of a block
+    const int half = lane >> 5;
+
+    // ---- which queries --------------------------------------------------
+    const int q_blocks = p.n_q_tiles * p.q_blocks_per_tile;
+    int wg = blockIdx.x;
+    if(p.xcd_remap)
+    {
+        // Workgroups are dealt round-robin to the 8 XCDs; regroup them so that
+        // the query blocks of one batch entry (which share K and V) meet in
+        // one XCD's L2.
+        const int per_xcd = gridDim.x >> 3;
+        wg = (wg & 7) * per_xcd + (wg >> 3);
+    }
+    const int b = wg / q_blocks;
+    // heaviest (last) query blocks first
+    const int qblk = q_blocks - 1 - (wg % q_blocks);
+    const int qt = qblk / p.q_blocks_per_tile;
+    const int qb = qblk % p.q_blocks_per_tile;
+    const int64_t q_len = min(p.q_tile, p.q_seq - (int64_t)qt * p.q_tile);
+    const int64_t q_row0 = (int64_t)qb * kQRows;            // within the tile
+    if(q_row0 >= q_len)
+    {
+        return;
+    }
+    const int kvb = kv_entry(b, p.n_batch, p.kv_group);
+
+    const uint16_t *Qt = static_cast<const uint16_t *>(p.Q[qt])
+        + (int64_t)b * q_len * HEAD;
+    const int64_t my_q = q_row0 + wave * 32 + col;          // row within tile
+    const bool q_ok = my_q < q_len;
+    const int64_t my_qpos = p.q_pos0 + (int64_t)qt * p.q_tile + my_q;
+
+    // Q fragments, resident for the whole kernel.
+    vec8 qf[KSTEPS];
+    {
+        const uint16_t *src = Qt + (q_ok ? my_q : 0) * HEAD + half * 8;
+#pragma unroll
+        for(int ks = 0; ks < KSTEPS; ++ks)
+        {
+            u32x4 raw = *reinterpret_cast<const u32x4 *>(src + ks * 16);
+            if(!q_ok)
+            {
+                raw = u32x4{0, 0, 0, 0};
+            }
+            qf[ks] = __builtin_bit_cast(vec8, raw);
+        }
+    }
+
+    // ---- which keys --------------------------------------------------------
+    // Steps are numbered over all key tiles; step g covers keys
+    // [kb*64, kb*64+64) of tile kt = g / k_blocks_per_tile.
+    const int64_t last_k_len = p.k_seq - (int64_t)(p.n_kv_tiles - 1) * p.k_tile;
+    int n_steps = (p.n_kv_tiles - 1) * p.k_blocks_per_tile
+        + (int)((last_k_len + kKeys - 1) / kKeys);
+    // Positions of the first/last query of this workgroup and wavefront.
+    const int64_t wg_qpos_hi = p.q_pos0 + (int64_t)qt * p.q_tile
+        + min(q_row0 + kQRows, q_len) - 1;
+    const int64_t wave_qpos_lo = p.q_pos0 + (int64_t)qt * p.q_tile + q_row0
+        + wave * 32;
+    const int64_t wave_qpos_hi = wave_qpos_lo + 31;
+
+    // Cooperative load assignment.
+    // K: 64 rows x CHUNKS chunks of 16 B, thread t takes chunk t % CHUNKS of
+    //    rows t / CHUNKS + i * (256 / CHUNKS).
+    constexpr int K_ROWS_PER_PASS = kThreads / CHUNKS;
+    constexpr int K_PASSES = kKeys / K_ROWS_PER_PASS;
+    const int k_chunk = tid % CHUNKS;
+    const int k_row = tid / CHUNKS;
+    // V: 16 groups of 4 keys x CHUNKS chunks; thread u takes key group
+    //    u % 16 and chunk u / 16 (lanes walk the key axis so that the
+    //    transposed 8-byte LDS writes of 16 lanes fill one 128-byte row).
+    constexpr int V_UNITS = 16 * CHUNKS;
+    const bool v_active = tid < V_UNITS;
+    const int v_kg = tid & 15;
+    const int v_chunk = tid >> 4;
+    // LDS position of keys 4*kg..4*kg+3: within each group of 16 keys the
+    // order is [h][a][c] for key = 8a + 4h + c, which is the order in which
+    // the S^T accumulators of lane half h list their keys.
+    const int v_pos = 16 * (v_kg >> 2) + 8 * (v_kg & 1) + 4 * ((v_kg & 3) >> 1);
+
+    u32x4 k_regs[K_PASSES];
+    u32x4 v_regs[4];
+
+    auto fetch = [&](int g)
+    {
+        const int kt = g / p.k_blocks_per_tile;
+        const int kb = g % p.k_blocks_per_tile;
+        const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
+        const int64_t row0 = (int64_t)kb * kKeys;
+        const uint16_t *Kt = static_cast<const uint16_t *>(p.K[kt])
+            + ((int64_t)kvb * k_len) * HEAD;
+        const uint16_t *Vtile = static_cast<const uint16_t *>(p.V[kt])
+            + ((int64_t)kvb * k_len) * HEAD;
+#pragma unroll
+        for(int i = 0; i < K_PASSES; ++i)
+        {
+            const int64_t r = row0 + k_row + i * K_ROWS_PER_PASS;
+            k_regs[i] = (r < k_len)
+                ? *reinterpret_cast<const u32x4 *>(Kt + r * HEAD + k_chunk * 8)
+                : u32x4{0, 0, 0, 0};
+        }
+        if(v_active)
+        {
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+            {
+                const int64_t r = row0 + 4 * v_kg + j;
+                v_regs[j] = (r < k_len)
+                    ? *reinterpret_cast<const u32x4 *>(Vtile + r * HEAD
+                            + v_chunk * 8)
+                    : u32x4{0, 0, 0, 0};
+            }
+        }
+    };
+
+    auto stage = [&]()
+    {
+#pragma unroll
+        for(int i = 0; i < K_PASSES; ++i)
+        {
+            *reinterpret_cast<u32x4 *>(&Ks[(k_row + i * K_ROWS_PER_PASS) * KPAD
+                    + k_chunk * 8]) = k_regs[i];
+        }
+        if(v_active)
+        {
+#pragma unroll
+            for(int w = 0; w < 4; ++w)
+            {
+                // word w of each row holds head values 2w (low) and 2w+1 (high)
+                const uint32_t r0 = v_regs[0][w], r1 = v_regs[1][w],
+                      r2 = v_regs[2][w], r3 = v_regs[3][w];
+                u32x2 even, odd;
+                even[0] = __builtin_amdgcn_perm(r1, r0, 0x05040100u);
+                even[1] = __builtin_amdgcn_perm(r3, r2, 0x05040100u);
+                odd[0] = __builtin_amdgcn_perm(r1, r0, 0x07060302u);
+                odd[1] = __builtin_amdgcn_perm(r3, r2, 0x07060302u);
+                const int d = v_chunk * 8 + 2 * w;
+                *reinterpret_cast<u32x2 *>(&Vt[d * VPAD + v_pos]) = even;
+                *reinterpret_cast<u32x2 *>(&Vt[(d + 1) * VPAD + v_pos]) = odd;
+            }
+        }
+    };
+
+    // In CAUSAL mode steps past the last visible key of the workgroup are
+    // never run.
+    if(MODE == NNTILE_HIP_MASK_CAUSAL)
+    {
+        const int64_t hi = wg_qpos_hi + p.causal_offset - p.k_pos0; // last visible key row overall
+        if(hi < 0)
+        {
+            return;
+        }
+        const int64_t kt_hi = hi / p.k_tile;
+        if(kt_hi < p.n_kv_tiles)
+        {
+            const int64_t in_tile = hi - kt_hi * p.k_tile;
+            const int steps = (int)(kt_hi * p.k_blocks_per_tile + in_tile / kKeys + 1);
+            n_steps = min(n_steps, steps);
+        }
+    }
+
+    // Score units: in the analytic modes the raw dot product is kept and the
+    // scale is folded into the exponent; with an explicit mask the score is
+    // scaled first and the mask value added.
+    const float c = EXPLICIT ? kLog2e : p.scale * kLog2e;
+
+    f32x16 o[DBLOCKS];
+#pragma unroll
+    for(int db = 0; db < DBLOCKS; ++db)
+    {
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+        {
+            o[db][r] = 0.0f;
+        }
+    }
+    float m_run = neg_inf();
+    float l_run = 0.0f;      // this lane half's share of the row sum
+
+    fetch(0);
+    for(int g = 0; g < n_steps; ++g)
+    {
+        __syncthreads();            // previous step's LDS reads are done
+        stage();
+        __syncthreads();
+        if(g + 1 < n_steps)
+        {
+            fetch(g + 1);           // in flight during the arithmetic below
+        }
+
+        const int kt = g / p.k_blocks_per_tile;
+        const int kb = g % p.k_blocks_per_tile;
+        const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
+        const int64_t k_row0 = (int64_t)kb * kKeys;          // within the tile
+        const int64_t k_pos_base = p.k_pos0 + (int64_t)kt * p.k_tile + k_row0;
+        const int keys_here = (int)min((int64_t)kKeys, k_len - k_row0);
+
+        if(MODE == NNTILE_HIP_MASK_CAUSAL
+                && k_pos_base > wave_qpos_hi + p.causal_offset)
+        {
+            continue;               // nothing visible to this wavefront
+        }
+
+        // ---- S^T = K Q^T ---------------------------------------------------
+        f32x16 s[2];
+#pragma unroll
+        for(int mb = 0; mb < 2; ++mb)
+        {
+#pragma unroll
+            for(int r = 0; r < 16; ++r)
+            {
+                s[mb][r] = 0.0f;
+            }
+#pragma unroll
+            for(int ks = 0; ks < KSTEPS; ++ks)
+            {
+                const vec8 a = *reinterpret_cast<const vec8 *>(
+                        &Ks[(mb * 32 + col) * KPAD + ks * 16 + half * 8]);
+                s[mb] = T::mfma(a, qf[ks], s[mb]);
+            }
+        }
+
+        // ---- mask -----------------------------------------------------------
+        // register r of block mb holds key  mb*32 + 8*(r/4) + 4*half + r%4
+        if(EXPLICIT)
+        {
+            const int64_t qrow = q_ok ? my_q : 0;
+#pragma unroll
+            for(int mb = 0; mb < 2; ++mb)
+            {
+#pragma unroll
+                for(int rg = 0; rg < 4; ++rg)
+                {
+                    const int key0 = mb * 32 + 8 * rg + 4 * half;
+                    const int64_t krow = k_row0 + key0;
+                    float add[4];
+                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                    {
+                        const uint16_t *mp = static_cast<const uint16_t *>(p.mask)
+                            + qrow * p.mask_ld + krow;
+#pragma unroll
+                        for(int e = 0; e < 4; ++e)
+                        {
+                            add[e] = (key0 + e < keys_here)
+                                ? T::to_float(mp[e]) : neg_inf();
+                        }
+                    }
+                    else
+                    {
+                        const uint8_t *mp = static_cast<const uint8_t *>(p.mask)
+                            + qrow * p.mask_ld + krow;
+#pragma unroll
+                        for(int e = 0; e < 4; ++e)
+                        {
+                            add[e] = (key0 + e < keys_here && mp[e] != 0)
+                                ? 0.0f : neg_inf();
+                        }
+                    }
+#pragma unroll
+                    for(int e = 0; e < 4; ++e)
+                    {
+                        const float v = s[mb][4 * rg + e] * p.scale + add[e];
+                        // a hidden key stays hidden whatever the score is
+                        s[mb][4 * rg + e] = (add[e] == neg_inf()) ? neg_inf() : v;
+                    }
+                }
+            }
+        }
+        else
+        {
+            const bool ragged = keys_here < kKeys;
+            const bool diagonal = (MODE == NNTILE_HIP_MASK_CAUSAL)
+                && (k_pos_base + kKeys - 1 > wave_qpos_lo + p.causal_offset);
+            if(ragged || diagonal)
+            {
+                const int64_t vis = (MODE == NNTILE_HIP_MASK_CAUSAL)
+                    ? (my_qpos + p.causal_offset - k_pos_base)   // last visible key in step
+                    : (int64_t)kKeys;
+                const int lim = (int)max((int64_t)-1,
+                        min(vis, (int64_t)keys_here - 1));
+#pragma unroll
+                for(int mb = 0; mb < 2; ++mb)
+                {
+#pragma unroll
+                    for(int r = 0; r < 16; ++r)
+                    {
+                        const int key = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                        if(key > lim)
+                        {
+                            s[mb][r] = neg_inf();
+                        }
+                    }
+                }
+            }
+        }
+
+        // ---- online softmax ---------------------------------------------------
+        float mx = neg_inf();
+#pragma unroll
+        for(int mb = 0; mb < 2; ++mb)
+        {
+#pragma unroll
+            for(int r = 0; r < 16; ++r)
+            {
+                mx = fmaxf(mx, s[mb][r]);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+        const float alpha = fast_exp2((m_run - m_use) * c);
+        const float mc = m_use * c;
+        m_run = m_new;
+
+        float rs = 0.0f;
+        uint32_t pk[2][8];
+#pragma unroll
+        for(int mb = 0; mb < 2; ++mb)
+        {
+#pragma unroll
+            for(int r = 0; r < 16; r += 2)
+            {
+                const float p0 = fast_exp2(fmaf(s[mb][r], c, -mc));
+                const float p1 = fast_exp2(fmaf(s[mb][r + 1], c, -mc));
+                rs += p0 + p1;
+                pk[mb][r >> 1] = T::pack2(p0, p1);
+            }
+        }
+        l_run = l_run * alpha + rs;
+#pragma unroll
+        for(int db = 0; db < DBLOCKS; ++db)
+        {
+#pragma unroll
+            for(int r = 0; r < 16; ++r)
+            {
+                o[db][r] *= alpha;
+            }
+        }
+
+        // ---- O^T += V^T P^T ----------------------------------------------------
+#pragma unroll
+        for(int t = 0; t < 4; ++t)
+        {
+            const int mb = t >> 1, tt = t & 1;
+            const u32x4 praw = {pk[mb][4 * tt], pk[mb][4 * tt + 1],
+                pk[mb][4 * tt + 2], pk[mb][4 * tt + 3]};
+            const vec8 pb = __builtin_bit_cast(vec8, praw);
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+                const vec8 a = *reinterpret_cast<const vec8 *>(
+                        &Vt[(db * 32 + col) * VPAD + 16 * t + 8 * half]);
+                o[db] = T::mfma(a, pb, o[db]);
+            }
+        }
+    }
+
+    // ---- epilogue: normalise, merge into the running (lse, A) ----------------
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if(!q_ok || !(l_tot > 0.0f))
+    {
+        return;     // no visible key: leave lse and A as they are
+    }
+    const float to_ln = EXPLICIT ? 1.0f : p.scale;
+    const float lse_new = m_run * to_ln + __logf(l_tot);
+    float *lse_ptr = p.lse[qt] + (int64_t)b * q_len + my_q;
+    const float lse_old = *lse_ptr;
+    float w_old, w_new, lse_out;
+    merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
+    if(half == 0)
+    {
+        *lse_ptr = lse_out;
+    }
+    const float w_o = w_new / l_tot;
+    uint16_t *Arow = static_cast<uint16_t *>(p.A[qt])
+        + ((int64_t)b * q_len + my_q) * HEAD;
+    // register r of block db holds head value  db*32 + 8*(r/4) + 4*half + r%4
+#pragma unroll
+    for(int db = 0; db < DBLOCKS; ++db)
+    {
+#pragma unroll
+        for(int rg = 0; rg < 4; ++rg)
+        {
+            uint16_t *dst = Arow + db * 32 + 8 * rg + 4 * half;
+            float v[4];
+#pragma unroll
+            for(int e = 0; e < 4; ++e)
+            {
+                v[e] = o[db][4 * rg + e] * w_o;
+            }
+            if(w_old != 0.0f)
+            {
+                const u32x2 old = *reinterpret_cast<const u32x2 *>(dst);
+                v[0] += w_old * T::to_float((uint16_t)(old[0] & 0xffffu));
+                v[1] += w_old * T::to_float((uint16_t)(old[0] >> 16));
+                v[2] += w_old * T::to_float((uint16_t)(old[1] & 0xffffu));
+                v[3] += w_old * T::to_float((uint16_t)(old[1] >> 16));
+            }
+            u32x2 out;
+            out[0] = T::pack2(v[0], v[1]);
+            out[1] = T::pack2(v[2], v[3]);
+            *reinterpret_cast<u32x2 *>(dst) = out;
+        }
+    }
+}
+
+template<typename T, int HEAD>
+static int launch_mode(hipStream_t stream, const PrefillParams &p, int mode,
+        dim3 grid)
+{
+    switch(mode)
+    {
+        case NNTILE_HIP_MASK_ADDITIVE:
+            hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
+                        NNTILE_HIP_MASK_ADDITIVE>), grid, dim3(kThreads), 0,
+                    stream, p);
+            break;
+        case NNTILE_HIP_MASK_NONE:
+            hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
+                        NNTILE_HIP_MASK_NONE>), grid, dim3(kThreads), 0,
+                    stream, p);
+            break;
+        case NNTILE_HIP_MASK_CAUSAL:
+            hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
+                        NNTILE_HIP_MASK_CAUSAL>), grid, dim3(kThreads), 0,
+                    stream, p);
+            break;
+        case NNTILE_HIP_MASK_BOOL:
+            hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
+                        NNTILE_HIP_MASK_BOOL>), grid, dim3(kThreads), 0,
+                    stream, p);
+            break;
+        default:
+            return NNTILE_HIP_EINVAL;
+    }
+    return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
+}
+
+// Host launcher shared by the tile and grid entry points.  p must be fully
+// filled except for the block counts and the remap flag.
+template<typename T>
+int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
+        int mode)
+{
+    p.q_blocks_per_tile = (int)((p.q_tile + kQRows - 1) / kQRows);
+    p.k_blocks_per_tile = (int)((p.k_tile + kKeys - 1) / kKeys);
+    const int64_t n_wg = (int64_t)p.batch * p.n_q_tiles * p.q_blocks_per_tile;
+    if(n_wg <= 0 || n_wg > 0x7fffffff)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    p.xcd_remap = (n_wg % 8 == 0) ? 1 : 0;
+    const dim3 grid((unsigned)n_wg);
+    switch(head)
+    {
+        case 32:
+            return launch_mode<T, 32>(stream, p, mode, grid);
+        case 64:
+            return launch_mode<T, 64>(stream, p, mode, grid);
+        case 128:
+            return launch_mode<T, 128>(stream, p, mode, grid);
+        default:
+            return NNTILE_HIP_EUNSUPPORTED;
+    }
+}
+
+template int launch_prefill_16bit<Bf16>(hipStream_t, PrefillParams &, int, int);
+template int launch_prefill_16bit<Fp16>(hipStream_t, PrefillParams &, int, int);
+
+} // namespace nntile_hip

@@ -1,0 +1,410 @@
+// Prefill attention forward for fp32 tiles on gfx950.
+//
+// Same decomposition as the 16-bit kernel (one workgroup = 4 wavefronts = 128
+// queries, S^T = K Q^T and O^T += V^T P^T with a lane owning one query), but
+// on v_mfma_f32_32x32x2_f32: operands and products are true fp32, which the
+// 1e-4 tolerance of the fp32 configurations needs.  Keys are walked in steps
+// of 32.  With a 2-deep contraction per MFMA the lane half h supplies the
+// operand element k = h, so:
+//   S^T: 4 consecutive MFMAs consume one 16-byte read K[key][8j+4h .. +3]
+//        against the matching 4 query values held in registers;
+//   O^T: the B operand is the S^T accumulator register itself (key
+//        8*(r/4) + 4h + r%4), the A operand is V[that key][d] read from LDS
+//        with the head axis across lanes - no transposition is needed.
+#include "sdpa_common.hpp"
+
+namespace nntile_hip
+{
+
+constexpr int kQRows32 = 128;
+constexpr int kKeys32 = 32;
+constexpr int kThreads32 = 256;
+
+template<int HEAD, int MODE>
+__global__ __launch_bounds__(kThreads32, 2)
+void sdpa_prefill_fp32_kernel(const PrefillParams p)
+{
+    constexpr int QSTEPS = HEAD / 8;        // 16-byte groups per lane half along head
+    constexpr int DBLOCKS = HEAD / 32;
+    constexpr int PAD = HEAD + 4;           // row stride in LDS (floats)
+    constexpr int CHUNKS = HEAD / 4;        // 16-byte chunks per row
+    constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
+            || MODE == NNTILE_HIP_MASK_BOOL);
+
+    __shared__ __attribute__((aligned(16))) float Ks[kKeys32 * PAD];
+    __shared__ __attribute__((aligned(16))) float Vs[kKeys32 * PAD];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int col = lane & 31;
+    const int half = lane >> 5;
+
+    const int q_blocks = p.n_q_tiles * p.q_blocks_per_tile;
+    int wg = blockIdx.x;
+    if(p.xcd_remap)
+    {
+        const int per_xcd = gridDim.x >> 3;
+        wg = (wg & 7) * per_xcd + (wg >> 3);
+    }
+    const int b = wg / q_blocks;
+    const int qblk = q_blocks - 1 - (wg % q_blocks);
+    const int qt = qblk / p.q_blocks_per_tile;
+    const int qb = qblk % p.q_blocks_per_tile;
+    const int64_t q_len = min(p.q_tile, p.q_seq - (int64_t)qt * p.q_tile);
+    const int64_t q_row0 = (int64_t)qb * kQRows32;
+    if(q_row0 >= q_len)
+    {
+        return;
+    }
+    const int kvb = kv_entry(b, p.n_batch, p.kv_group);
+
+    const float *Qt = static_cast<const float *>(p.Q[qt])
+        + (int64_t)b * q_len * HEAD;
+    const int64_t my_q = q_row0 + wave * 32 + col;
+    const bool q_ok = my_q < q_len;
+    const int64_t my_qpos = p.q_pos0 + (int64_t)qt * p.q_tile + my_q;
+
+    // Q values of this lane: for group j, head values 8j + 4*half .. +3.
+    f32x4 qf[QSTEPS];
+    {
+        const float *src = Qt + (q_ok ? my_q : 0) * HEAD + half * 4;
+#pragma unroll
+        for(int j = 0; j < QSTEPS; ++j)
+        {
+            qf[j] = q_ok ? *reinterpret_cast<const f32x4 *>(src + j * 8)
+                : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+
+    const int64_t last_k_len = p.k_seq - (int64_t)(p.n_kv_tiles - 1) * p.k_tile;
+    int n_steps = (p.n_kv_tiles - 1) * p.k_blocks_per_tile
+        + (int)((last_k_len + kKeys32 - 1) / kKeys32);
+    const int64_t wg_qpos_hi = p.q_pos0 + (int64_t)qt * p.q_tile
+        + min(q_row0 + kQRows32, q_len) - 1;
+    const int64_t wave_qpos_lo = p.q_pos0 + (int64_t)qt * p.q_tile + q_row0
+        + wave * 32;
+    const int64_t wave_qpos_hi = wave_qpos_lo + 31;
+
+    // Cooperative loads: 32 rows x CHUNKS chunks for K and for V.
+    constexpr int ROWS_PER_PASS = kThreads32 / CHUNKS;
+    constexpr int PASSES = kKeys32 / ROWS_PER_PASS;
+    const int ld_chunk = tid % CHUNKS;
+    const int ld_row = tid / CHUNKS;
+    f32x4 k_regs[PASSES], v_regs[PASSES];
+
+    auto fetch = [&](int g)
+    {
+        const int kt = g / p.k_blocks_per_tile;
+        const int kb = g % p.k_blocks_per_tile;
+        const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
+        const int64_t row0 = (int64_t)kb * kKeys32;
+        const float *Kt = static_cast<const float *>(p.K[kt])
+            + ((int64_t)kvb * k_len) * HEAD;
+        const float *Vtile = static_cast<const float *>(p.V[kt])
+            + ((int64_t)kvb * k_len) * HEAD;
+#pragma unroll
+        for(int i = 0; i < PASSES; ++i)
+        {
+            const int64_t r = row0 + ld_row + i * ROWS_PER_PASS;
+            const bool ok = r < k_len;
+            const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+            k_regs[i] = ok ? *reinterpret_cast<const f32x4 *>(
+                    Kt + r * HEAD + ld_chunk * 4) : zero;
+            v_regs[i] = ok ? *reinterpret_cast<const f32x4 *>(
+                    Vtile + r * HEAD + ld_chunk * 4) : zero;
+        }
+    };
+
+    auto stage = [&]()
+    {
+#pragma unroll
+        for(int i = 0; i < PASSES; ++i)
+        {
+            const int off = (ld_row + i * ROWS_PER_PASS) * PAD + ld_chunk * 4;
+            *reinterpret_cast<f32x4 *>(&Ks[off]) = k_regs[i];
+            *reinterpret_cast<f32x4 *>(&Vs[off]) = v_regs[i];
+        }
+    };
+
+    if(MODE == NNTILE_HIP_MASK_CAUSAL)
+    {
+        const int64_t hi = wg_qpos_hi + p.causal_offset - p.k_pos0;
+        if(hi < 0)
+        {
+            return;
+        }
+        const int64_t kt_hi = hi / p.k_tile;
+        if(kt_hi < p.n_kv_tiles)
+        {
+            const int64_t in_tile = hi - kt_hi * p.k_tile;
+            const int steps = (int)(kt_hi * p.k_blocks_per_tile
+                    + in_tile / kKeys32 + 1);
+            n_steps = min(n_steps, steps);
+        }
+    }
+
+    const float c = EXPLICIT ? kLog2e : p.scale * kLog2e;
+
+    f32x16 o[DBLOCKS];
+#pragma unroll
+    for(int db = 0; db < DBLOCKS; ++db)
+    {
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+        {
+            o[db][r] = 0.0f;
+        }
+    }
+    float m_run = neg_inf();
+    float l_run = 0.0f;
+
+    fetch(0);
+    for(int g = 0; g < n_steps; ++g)
+    {
+        __syncthreads();
+        stage();
+        __syncthreads();
+        if(g + 1 < n_steps)
+        {
+            fetch(g + 1);
+        }
+
+        const int kt = g / p.k_blocks_per_tile;
+        const int kb = g % p.k_blocks_per_tile;
+        const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
+        const int64_t k_row0 = (int64_t)kb * kKeys32;
+        const int64_t k_pos_base = p.k_pos0 + (int64_t)kt * p.k_tile + k_row0;
+        const int keys_here = (int)min((int64_t)kKeys32, k_len - k_row0);
+
+        if(MODE == NNTILE_HIP_MASK_CAUSAL
+                && k_pos_base > wave_qpos_hi + p.causal_offset)
+        {
+            continue;
+        }
+
+        // ---- S^T = K Q^T ---------------------------------------------------
+        f32x16 s;
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+        {
+            s[r] = 0.0f;
+        }
+#pragma unroll
+        for(int j = 0; j < QSTEPS; ++j)
+        {
+            const f32x4 a = *reinterpret_cast<const f32x4 *>(
+                    &Ks[col * PAD + j * 8 + half * 4]);
+#pragma unroll
+            for(int e = 0; e < 4; ++e)
+            {
+                s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], qf[j][e], s,
+                        0, 0, 0);
+            }
+        }
+
+        // ---- mask: register r holds key 8*(r/4) + 4*half + r%4 ---------------
+        if(EXPLICIT)
+        {
+            const int64_t qrow = q_ok ? my_q : 0;
+#pragma unroll
+            for(int rg = 0; rg < 4; ++rg)
+            {
+                const int key0 = 8 * rg + 4 * half;
+                const int64_t krow = k_row0 + key0;
+#pragma unroll
+                for(int e = 0; e < 4; ++e)
+                {
+                    float add;
+                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                    {
+                        add = (key0 + e < keys_here)
+                            ? static_cast<const float *>(p.mask)[
+                                qrow * p.mask_ld + krow + e]
+                            : neg_inf();
+                    }
+                    else
+                    {
+                        add = (key0 + e < keys_here
+                                && static_cast<const uint8_t *>(p.mask)[
+                                    qrow * p.mask_ld + krow + e] != 0)
+                            ? 0.0f : neg_inf();
+                    }
+                    const float v = s[4 * rg + e] * p.scale + add;
+                    s[4 * rg + e] = (add == neg_inf()) ? neg_inf() : v;
+                }
+            }
+        }
+        else
+        {
+            const bool ragged = keys_here < kKeys32;
+            const bool diagonal = (MODE == NNTILE_HIP_MASK_CAUSAL)
+                && (k_pos_base + kKeys32 - 1 > wave_qpos_lo + p.causal_offset);
+            if(ragged || diagonal)
+            {
+                const int64_t vis = (MODE == NNTILE_HIP_MASK_CAUSAL)
+                    ? (my_qpos + p.causal_offset - k_pos_base)
+                    : (int64_t)kKeys32;
+                const int lim = (int)max((int64_t)-1,
+                        min(vis, (int64_t)keys_here - 1));
+#pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    const int key = 8 * (r >> 2) + 4 * half + (r & 3);
+                    if(key > lim)
+                    {
+                        s[r] = neg_inf();
+                    }
+                }
+            }
+        }
+
+        // ---- online softmax ---------------------------------------------------
+        float mx = neg_inf();
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+        {
+            mx = fmaxf(mx, s[r]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+        const float alpha = fast_exp2((m_run - m_use) * c);
+        const float mc = m_use * c;
+        m_run = m_new;
+        float rs = 0.0f;
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+        {
+            s[r] = fast_exp2(fmaf(s[r], c, -mc));
+            rs += s[r];
+        }
+        l_run = l_run * alpha + rs;
+#pragma unroll
+        for(int db = 0; db < DBLOCKS; ++db)
+        {
+#pragma unroll
+            for(int r = 0; r < 16; ++r)
+            {
+                o[db][r] *= alpha;
+            }
+        }
+
+        // ---- O^T += V^T P^T ----------------------------------------------------
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+        {
+            const int key = 8 * (r >> 2) + 4 * half + (r & 3);
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+                const float a = Vs[key * PAD + db * 32 + col];
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s[r], o[db],
+                        0, 0, 0);
+            }
+        }
+    }
+
+    // ---- epilogue --------------------------------------------------------------
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if(!q_ok || !(l_tot > 0.0f))
+    {
+        return;
+    }
+    const float to_ln = EXPLICIT ? 1.0f : p.scale;
+    const float lse_new = m_run * to_ln + __logf(l_tot);
+    float *lse_ptr = p.lse[qt] + (int64_t)b * q_len + my_q;
+    const float lse_old = *lse_ptr;
+    float w_old, w_new, lse_out;
+    merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
+    if(half == 0)
+    {
+        *lse_ptr = lse_out;
+    }
+    const float w_o = w_new / l_tot;
+    float *Arow = static_cast<float *>(p.A[qt])
+        + ((int64_t)b * q_len + my_q) * HEAD;
+#pragma unroll
+    for(int db = 0; db < DBLOCKS; ++db)
+    {
+#pragma unroll
+        for(int rg = 0; rg < 4; ++rg)
+        {
+            float *dst = Arow + db * 32 + 8 * rg + 4 * half;
+            f32x4 v;
+#pragma unroll
+            for(int e = 0; e < 4; ++e)
+            {
+                v[e] = o[db][4 * rg + e] * w_o;
+            }
+            if(w_old != 0.0f)
+            {
+                const f32x4 old = *reinterpret_cast<const f32x4 *>(dst);
+#pragma unroll
+                for(int e = 0; e < 4; ++e)
+                {
+                    v[e] += w_old * old[e];
+                }
+            }
+            *reinterpret_cast<f32x4 *>(dst) = v;
+        }
+    }
+}
+
+template<int HEAD>
+static int launch_mode32(hipStream_t stream, const PrefillParams &p, int mode,
+        dim3 grid)
+{
+    switch(mode)
+    {
+        case NNTILE_HIP_MASK_ADDITIVE:
+            hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
+                        NNTILE_HIP_MASK_ADDITIVE>), grid, dim3(kThreads32), 0,
+                    stream, p);
+            break;
+        case NNTILE_HIP_MASK_NONE:
+            hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
+                        NNTILE_HIP_MASK_NONE>), grid, dim3(kThreads32), 0,
+                    stream, p);
+            break;
+        case NNTILE_HIP_MASK_CAUSAL:
+            hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
+                        NNTILE_HIP_MASK_CAUSAL>), grid, dim3(kThreads32), 0,
+                    stream, p);
+            break;
+        case NNTILE_HIP_MASK_BOOL:
+            hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
+                        NNTILE_HIP_MASK_BOOL>), grid, dim3(kThreads32), 0,
+                    stream, p);
+            break;
+        default:
+            return NNTILE_HIP_EINVAL;
+    }
+    return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
+}
+
+int launch_prefill_fp32(hipStream_t stream, PrefillParams &p, int head, int mode)
+{
+    p.q_blocks_per_tile = (int)((p.q_tile + kQRows32 - 1) / kQRows32);
+    p.k_blocks_per_tile = (int)((p.k_tile + kKeys32 - 1) / kKeys32);
+    const int64_t n_wg = (int64_t)p.batch * p.n_q_tiles * p.q_blocks_per_tile;
+    if(n_wg <= 0 || n_wg > 0x7fffffff)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    p.xcd_remap = (n_wg % 8 == 0) ? 1 : 0;
+    const dim3 grid((unsigned)n_wg);
+    switch(head)
+    {
+        case 32:
+            return launch_mode32<32>(stream, p, mode, grid);
+        case 64:
+            return launch_mode32<64>(stream, p, mode, grid);
+        case 128:
+            return launch_mode32<128>(stream, p, mode, grid);
+        default:
+            return NNTILE_HIP_EUNSUPPORTED;
+    }
+}
+
+} // namespace nntile_hip

@@ -1,0 +1,259 @@
+"""ctypes binding of libnntile_hip_sdpa.so plus thin torch-tensor front-ends.
+
+torch is used for device memory and streams only; every computation goes
+through the C ABI declared in include/nntile_hip_sdpa.h.  There is no fallback:
+if the library is missing, loading fails.
+
+Tensor convention: torch tensors are C-ordered views of NNTile's Fortran
+tiles, i.e. K/V ``[kv_batch, k_seq, head]``, Q/A ``[batch, q_seq, head]``,
+lse ``[batch, q_seq]`` fp32, mask ``[q_seq, k_seq]``.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libnntile_hip_sdpa.so")
+
+MASK_ADDITIVE, MASK_NONE, MASK_CAUSAL, MASK_BOOL = 0, 1, 2, 3
+MAX_TILES = 64
+
+OK, EINVAL, EUNSUPPORTED, ELAUNCH, EWORKSPACE = 0, -1, -2, -3, -4
+_ERR = {EINVAL: "invalid argument", EUNSUPPORTED: "unsupported configuration",
+        ELAUNCH: "HIP launch failed", EWORKSPACE: "workspace missing or too small"}
+
+_i64 = ctypes.c_int64
+_vp = ctypes.c_void_p
+
+
+class TileArgs(ctypes.Structure):
+    _fields_ = [("q_seq", _i64), ("k_seq", _i64), ("head", _i64),
+                ("batch", _i64), ("n_batch", _i64), ("kv_group", _i64),
+                ("mask_mode", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("q_pos0", _i64), ("k_pos0", _i64), ("causal_offset", _i64),
+                ("K", _vp), ("Q", _vp), ("mask", _vp), ("V", _vp),
+                ("lse", _vp), ("A", _vp)]
+
+
+class GridArgs(ctypes.Structure):
+    _fields_ = [("q_seq", _i64), ("k_seq", _i64), ("q_tile", _i64),
+                ("k_tile", _i64), ("head", _i64), ("batch", _i64),
+                ("n_batch", _i64), ("kv_group", _i64),
+                ("mask_mode", ctypes.c_int32), ("n_q_tiles", ctypes.c_int32),
+                ("n_kv_tiles", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("q_pos0", _i64), ("k_pos0", _i64), ("causal_offset", _i64),
+                ("K", _vp * MAX_TILES), ("V", _vp * MAX_TILES),
+                ("Q", _vp * MAX_TILES), ("lse", _vp * MAX_TILES),
+                ("A", _vp * MAX_TILES)]
+
+
+class VariableInterface(ctypes.Structure):
+    _fields_ = [("id", ctypes.c_int), ("ptr", ctypes.c_size_t),
+                ("dev_handle", ctypes.c_size_t), ("offset", ctypes.c_size_t),
+                ("elemsize", ctypes.c_size_t)]
+
+
+class FlashClArgs(ctypes.Structure):
+    _fields_ = [("owner", _vp), ("seq", _i64), ("head", _i64), ("batch", _i64)]
+
+
+STREAM_PROVIDER = ctypes.CFUNCTYPE(_vp)
+
+EXPORTS = (
+    ["nntile_hip_flash_sdpa_fwd_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_sdpa_fwd_tile_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_sdpa_fwd_grid_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_sdpa_fwd_decode_" + t for t in ("bf16", "fp16")]
+    + ["nntile_hip_sdpa_fwd_decode_workspace_bytes"]
+    + ["nntile_hip_accumulate_attn_output_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_flash_sdpa_fwd_codelet_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_set_stream_provider", "nntile_hip_sdpa_version"])
+
+_lib = None
+
+
+def lib():
+    """The loaded C-ABI library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libnntile_hip_sdpa.so is missing: run `python -m nntile_amd.build`")
+        L = ctypes.CDLL(LIB_PATH)
+        for t in ("bf16", "fp16", "fp32"):
+            f = getattr(L, "nntile_hip_flash_sdpa_fwd_" + t)
+            f.argtypes = [_vp, _i64, _i64, _i64] + [_vp] * 8
+            f.restype = ctypes.c_int
+            f = getattr(L, "nntile_hip_sdpa_fwd_tile_" + t)
+            f.argtypes = [_vp, ctypes.POINTER(TileArgs)]
+            f.restype = ctypes.c_int
+            f = getattr(L, "nntile_hip_sdpa_fwd_grid_" + t)
+            f.argtypes = [_vp, ctypes.POINTER(GridArgs)]
+            f.restype = ctypes.c_int
+            f = getattr(L, "nntile_hip_accumulate_attn_output_" + t)
+            f.argtypes = [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp]
+            f.restype = ctypes.c_int
+            f = getattr(L, "nntile_hip_flash_sdpa_fwd_codelet_" + t)
+            f.argtypes = [ctypes.POINTER(_vp), _vp]
+            f.restype = None
+        for t in ("bf16", "fp16"):
+            f = getattr(L, "nntile_hip_sdpa_fwd_decode_" + t)
+            f.argtypes = [_vp, ctypes.POINTER(TileArgs), _vp, ctypes.c_size_t]
+            f.restype = ctypes.c_int
+        L.nntile_hip_sdpa_fwd_decode_workspace_bytes.argtypes = [ctypes.POINTER(TileArgs)]
+        L.nntile_hip_sdpa_fwd_decode_workspace_bytes.restype = ctypes.c_size_t
+        L.nntile_hip_set_stream_provider.argtypes = [_vp]
+        L.nntile_hip_set_stream_provider.restype = None
+        L.nntile_hip_sdpa_version.restype = ctypes.c_char_p
+        _lib = L
+    return _lib
+
+
+class SdpaError(RuntimeError):
+    def __init__(self, code, what):
+        super().__init__("%s: %s (code %d)" % (what, _ERR.get(code, "error"), code))
+        self.code = code
+
+
+def _check(code, what):
+    if code != OK:
+        raise SdpaError(code, what)
+
+
+def dtype_name(t):
+    if t.dtype == torch.bfloat16:
+        return "bf16"
+    if t.dtype == torch.float16:
+        return "fp16"
+    if t.dtype == torch.float32:
+        return "fp32"
+    raise TypeError("unsupported tile dtype %s" % t.dtype)
+
+
+def _stream(stream):
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _dev(*tensors):
+    for t in tensors:
+        if t is not None and not (t.is_cuda and t.is_contiguous()):
+            raise ValueError("tiles must be contiguous device tensors")
+
+
+def flash_sdpa_fwd(K, Q, mask, lse, V, A, stream=None):
+    """One square tile with an additive mask: the reference kernel call
+    (execute_graph) with its argument order K, Q, mask, lse, V, A."""
+    _dev(K, Q, mask, lse, V, A)
+    batch, seq, head = Q.shape
+    fn = getattr(lib(), "nntile_hip_flash_sdpa_fwd_" + dtype_name(Q))
+    _check(fn(_stream(stream), seq, head, batch, _ptr(K), _ptr(Q), _ptr(mask),
+              None, _ptr(V), None, _ptr(lse), _ptr(A)), "flash_sdpa_fwd")
+
+
+def _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0,
+               k_pos0, causal_offset):
+    batch, q_seq, head = Q.shape
+    k_seq = K.shape[1]
+    a = TileArgs()
+    a.q_seq, a.k_seq, a.head, a.batch = q_seq, k_seq, head, batch
+    a.n_batch = batch if n_batch is None else n_batch
+    a.kv_group = kv_group
+    a.mask_mode = mask_mode
+    a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
+    a.K, a.Q, a.V = K.data_ptr(), Q.data_ptr(), V.data_ptr()
+    a.mask = None if mask is None else mask.data_ptr()
+    a.lse, a.A = lse.data_ptr(), A.data_ptr()
+    return a
+
+
+def sdpa_fwd_tile(K, Q, mask, lse, V, A, mask_mode, n_batch=None, kv_group=1,
+                  q_pos0=0, k_pos0=0, causal_offset=0, stream=None):
+    _dev(K, Q, mask, lse, V, A)
+    a = _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0,
+                   k_pos0, causal_offset)
+    fn = getattr(lib(), "nntile_hip_sdpa_fwd_tile_" + dtype_name(Q))
+    _check(fn(_stream(stream), ctypes.byref(a)), "sdpa_fwd_tile")
+
+
+def sdpa_fwd_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq,
+                  q_tile, k_tile, mask_mode, n_batch=None, kv_group=1,
+                  q_pos0=0, k_pos0=0, causal_offset=0, stream=None):
+    """All key tiles merged into all query tiles in one launch.  Tiles are
+    lists of separately allocated tensors [batch, rows, head]."""
+    _dev(*K_tiles, *Q_tiles, *lse_tiles, *V_tiles, *A_tiles)
+    batch, _, head = Q_tiles[0].shape
+    a = GridArgs()
+    a.q_seq, a.k_seq, a.q_tile, a.k_tile, a.head = q_seq, k_seq, q_tile, k_tile, head
+    a.batch = batch
+    a.n_batch = batch if n_batch is None else n_batch
+    a.kv_group = kv_group
+    a.mask_mode = mask_mode
+    a.n_q_tiles, a.n_kv_tiles = len(Q_tiles), len(K_tiles)
+    a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
+    if len(Q_tiles) > MAX_TILES or len(K_tiles) > MAX_TILES:
+        raise SdpaError(EINVAL, "sdpa_fwd_grid")
+    for i, (k, v) in enumerate(zip(K_tiles, V_tiles)):
+        a.K[i], a.V[i] = k.data_ptr(), v.data_ptr()
+    for i, (q, l, o) in enumerate(zip(Q_tiles, lse_tiles, A_tiles)):
+        a.Q[i], a.lse[i], a.A[i] = q.data_ptr(), l.data_ptr(), o.data_ptr()
+    fn = getattr(lib(), "nntile_hip_sdpa_fwd_grid_" + dtype_name(Q_tiles[0]))
+    _check(fn(_stream(stream), ctypes.byref(a)), "sdpa_fwd_grid")
+    return a
+
+
+def decode_workspace_bytes(K, Q, n_batch, kv_group):
+    a = _tile_args(K, Q, None, Q, K, Q, MASK_NONE, n_batch, kv_group, 0, 0, 0)
+    return int(lib().nntile_hip_sdpa_fwd_decode_workspace_bytes(ctypes.byref(a)))
+
+
+def sdpa_fwd_decode(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group,
+                    workspace, q_pos0=0, k_pos0=0, causal_offset=0, stream=None):
+    """K, V: [n_head_kv*n_batch, k_seq, head]; Q, A:
+    [n_head_kv*kv_group*n_batch, q_seq, head]; workspace: a device byte
+    tensor of at least decode_workspace_bytes()."""
+    _dev(K, Q, mask, lse, V, A, workspace)
+    a = _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0,
+                   k_pos0, causal_offset)
+    fn = getattr(lib(), "nntile_hip_sdpa_fwd_decode_" + dtype_name(Q))
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _check(fn(_stream(stream), ctypes.byref(a), _ptr(workspace), nbytes),
+           "sdpa_fwd_decode")
+
+
+def accumulate_attn_output(src_lse, src_attn, dst_lse, dst_attn, stream=None):
+    """dst <- merge(dst, src) row by row; attn tiles [batch, seq, head]."""
+    _dev(src_lse, src_attn, dst_lse, dst_attn)
+    batch, seq, head = dst_attn.shape
+    fn = getattr(lib(), "nntile_hip_accumulate_attn_output_" + dtype_name(dst_attn))
+    _check(fn(_stream(stream), head, seq, batch, _ptr(src_lse), _ptr(src_attn),
+              _ptr(dst_lse), _ptr(dst_attn)), "accumulate_attn_output")
+
+
+def flash_sdpa_fwd_codelet(K, Q, mask, lse, V, A, scratch_lse=None, scratch_A=None,
+                           seq=None, head=None, batch=None):
+    """Calls the StarPU-shaped codelet body with look-alike variable
+    interfaces, as a StarPU HIP worker would (null stream unless a provider
+    was registered)."""
+    tensors = [K, Q, mask, lse, V, A, scratch_lse, scratch_A]
+    ifs = []
+    for t in tensors:
+        v = VariableInterface()
+        v.id = 2
+        v.ptr = 0 if t is None else t.data_ptr()
+        v.dev_handle = v.ptr
+        v.offset = 0
+        v.elemsize = 0 if t is None else t.numel() * t.element_size()
+        ifs.append(v)
+    bufs = (_vp * 8)(*[ctypes.addressof(v) for v in ifs])
+    b, s, h = Q.shape
+    args = FlashClArgs(None, s if seq is None else seq, h if head is None else head,
+                       b if batch is None else batch)
+    fn = getattr(lib(), "nntile_hip_flash_sdpa_fwd_codelet_" + dtype_name(Q))
+    fn(bufs, ctypes.addressof(args))

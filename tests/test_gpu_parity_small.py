@@ -1,0 +1,254 @@
+"""GPU parity of the HIP path against the CPU checker, through the C ABI, on
+shapes the checker finishes in well under a second.  Covers every entry point,
+every mask mode, the three dtypes, ragged and tiny extents, hidden rows and
+the running (lse, A) hand-off."""
+import numpy as np
+import pytest
+import torch
+
+from nntile_amd import hip_sdpa, synth
+from . import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle(oracle, f32, mask_bool, **kw):
+    qf, kf, vf = f32
+    return oracle.sdpa_vanilla(kf, qf, vf, mask_bool, **kw)
+
+
+def _mask(kind, q_seq, k_seq):
+    if kind == "causal":
+        return synth.causal_mask(q_seq, k_seq)
+    if kind == "full":
+        return np.ones((q_seq, k_seq), bool)
+    if kind == "window":      # tests/tile/flash_sdpa_fwd_cudnn.cc:57-86
+        return np.abs(np.arange(q_seq)[:, None] - np.arange(k_seq)[None, :]) <= 32
+    raise ValueError(kind)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("seq,head,batch", [(32, 32, 1), (64, 64, 2), (128, 64, 3),
+                                            (256, 128, 2), (96, 128, 1), (200, 64, 2),
+                                            (1, 64, 1), (33, 32, 5)])
+@pytest.mark.parametrize("kind", ["causal", "full", "window"])
+def test_flash_entry_matches_oracle(oracle, dtype, seq, head, batch, kind):
+    print("case", dtype, seq, head, batch, kind, flush=True)
+    (Q, K, V), f32 = H.make_qkv(42, batch, seq, seq, head, dtype)
+    mask = _mask(kind, seq, seq)
+    want, want_lse = _oracle(oracle, f32, mask)
+    lse, A = H.fresh_outputs(batch, seq, head, dtype)
+    hip_sdpa.flash_sdpa_fwd(K.cuda(), Q.cuda(), H.additive_mask(mask, dtype).cuda(),
+                            lse, V.cuda(), A)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+def test_reference_preset_data(oracle, dtype):
+    # tests/kernel/flash_sdpa_fwd_cudnn.cc:211-219: K=(i%20-10)*0.1, Q=0.8K, V=1.2K
+    seq, head, batch = 128, 64, 3
+    i = np.arange(batch * seq * head)
+    k = ((i % 20 - 10) * 0.1).astype(np.float32).reshape(batch, seq, head)
+    (K, kf), (Q, qf), (V, vf) = H.rounded(k, dtype), H.rounded(k * np.float32(0.8), dtype), \
+        H.rounded(k * np.float32(1.2), dtype)
+    mask = synth.causal_mask(seq, seq)
+    want, want_lse = oracle.sdpa_bruteforce_f64(kf, qf, vf,
+                                                np.where(mask, 0, -np.inf).astype(np.float32))
+    lse, A = H.fresh_outputs(batch, seq, head, dtype)
+    hip_sdpa.flash_sdpa_fwd(K.cuda(), Q.cuda(), H.additive_mask(mask, dtype).cuda(),
+                            lse, V.cuda(), A)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+@pytest.mark.parametrize("q_seq,k_seq,offset", [(128, 128, 0), (100, 260, 160), (64, 300, 100),
+                                                (130, 70, -20), (16, 512, 496)])
+def test_mask_modes_agree(oracle, dtype, q_seq, k_seq, offset):
+    """Analytic causal, boolean and additive masks give the oracle's answer on
+    non-square tiles, including queries that see nothing (negative offset)."""
+    print("case", dtype, q_seq, k_seq, offset, flush=True)
+    head, batch = 64, 2
+    (Q, K, V), f32 = H.make_qkv(7, batch, q_seq, k_seq, head, dtype)
+    mask = synth.causal_mask(q_seq, k_seq, offset)
+    want, want_lse = _oracle(oracle, f32, mask)
+    Kd, Qd, Vd = K.cuda(), Q.cuda(), V.cuda()
+    outs = []
+    for mode, m in [(hip_sdpa.MASK_CAUSAL, None),
+                    (hip_sdpa.MASK_BOOL, torch.from_numpy(mask).cuda()),
+                    (hip_sdpa.MASK_ADDITIVE, H.additive_mask(mask, dtype).cuda())]:
+        lse, A = H.fresh_outputs(batch, q_seq, head, dtype, poison=False)
+        hip_sdpa.sdpa_fwd_tile(Kd, Qd, m, lse, Vd, A, mode, causal_offset=offset)
+        torch.cuda.synchronize()
+        assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+        assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+        outs.append((H.to_np(lse), H.to_np(A)))
+    hidden = ~mask.any(axis=1)
+    if hidden.any():       # hidden queries: lse stays -inf, A untouched (0 here)
+        assert np.all(np.isneginf(outs[0][0][:, hidden])) and np.all(outs[0][1][:, hidden] == 0)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+def test_no_mask_mode(oracle, dtype):
+    (Q, K, V), f32 = H.make_qkv(9, 3, 70, 150, 128, dtype)
+    want, want_lse = _oracle(oracle, f32, None)
+    lse, A = H.fresh_outputs(3, 70, 128, dtype)
+    hip_sdpa.sdpa_fwd_tile(K.cuda(), Q.cuda(), None, lse, V.cuda(), A, hip_sdpa.MASK_NONE)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
+def test_running_merge_over_key_tiles(oracle, dtype):
+    """One call per key tile, (lse, A) carried in memory between calls as
+    between NNTile tasks (src/tensor/flash_sdpa_fwd_cudnn.cc:246-274), in a
+    shuffled order: equals attention over all keys at once."""
+    seq, head, batch, tile = 256, 64, 2, 64
+    (Q, K, V), f32 = H.make_qkv(11, batch, seq, seq, head, dtype)
+    mask = synth.causal_mask(seq, seq)
+    want, want_lse = _oracle(oracle, f32, mask)
+    lse, A = H.fresh_outputs(batch, seq, head, dtype)
+    Qd = Q.cuda()
+    for t in [2, 0, 3, 1]:
+        Kt = K[:, t * tile:(t + 1) * tile].contiguous().cuda()
+        Vt = V[:, t * tile:(t + 1) * tile].contiguous().cuda()
+        mt = H.additive_mask(mask[:, t * tile:(t + 1) * tile], dtype).contiguous().cuda()
+        hip_sdpa.sdpa_fwd_tile(Kt, Qd, mt, lse, Vt, A, hip_sdpa.MASK_ADDITIVE)
+    torch.cuda.synchronize()
+    # each hand-off rounds A to the tile dtype once more
+    assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+@pytest.mark.parametrize("q_seq,k_seq,q_tile,k_tile", [(256, 256, 64, 64), (300, 300, 128, 96),
+                                                       (200, 520, 200, 128), (512, 512, 128, 256)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_grid_entry_matches_oracle(oracle, dtype, q_seq, k_seq, q_tile, k_tile, causal):
+    print("case", dtype, q_seq, k_seq, q_tile, k_tile, causal, flush=True)
+    head, batch = 64, 3
+    offset = k_seq - q_seq
+    (Q, K, V), f32 = H.make_qkv(13, batch, q_seq, k_seq, head, dtype)
+    mask = synth.causal_mask(q_seq, k_seq, offset) if causal else None
+    want, want_lse = _oracle(oracle, f32, mask, k_tile=k_tile)
+    Kt = [K[:, s:s + k_tile].contiguous().cuda() for s in range(0, k_seq, k_tile)]
+    Vt = [V[:, s:s + k_tile].contiguous().cuda() for s in range(0, k_seq, k_tile)]
+    Qt = [Q[:, s:s + q_tile].contiguous().cuda() for s in range(0, q_seq, q_tile)]
+    outs = [H.fresh_outputs(batch, q.shape[1], head, dtype) for q in Qt]
+    hip_sdpa.sdpa_fwd_grid(Kt, Qt, [o[0] for o in outs], Vt, [o[1] for o in outs], q_seq, k_seq,
+                           q_tile, k_tile, hip_sdpa.MASK_CAUSAL if causal else hip_sdpa.MASK_NONE,
+                           causal_offset=offset)
+    torch.cuda.synchronize()
+    A = np.concatenate([H.to_np(o[1]) for o in outs], axis=1)
+    lse = np.concatenate([H.to_np(o[0]) for o in outs], axis=1)
+    assert H.rel_fro(A, want) < H.TOL[dtype]
+    assert H.rel_fro(lse, want_lse) < H.TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("q_seq,k_seq,n_batch,group,n_kv,head", [
+    (16, 512, 2, 4, 2, 128), (1, 300, 3, 4, 2, 128), (16, 1000, 1, 4, 1, 64),
+    (5, 77, 2, 8, 3, 128), (16, 64, 1, 2, 2, 128), (64, 200, 2, 1, 2, 64)])
+@pytest.mark.parametrize("mode", ["causal", "bool", "none"])
+def test_decode_entry_matches_oracle(oracle, dtype, q_seq, k_seq, n_batch, group, n_kv, head, mode):
+    print("case", dtype, q_seq, k_seq, n_batch, group, n_kv, head, mode, flush=True)
+    batch = n_batch * group * n_kv
+    (Q, K, V), f32 = H.make_qkv(17, batch, q_seq, k_seq, head, dtype, kv_batch=n_batch * n_kv)
+    offset = k_seq - q_seq            # layer/sdpa.py:516-531: new tokens are the last keys
+    mask = None if mode == "none" else synth.causal_mask(q_seq, k_seq, offset)
+    want, want_lse = _oracle(oracle, f32, mask, n_batch=n_batch, kv_repeat=group)
+    Kd, Qd, Vd = K.cuda(), Q.cuda(), V.cuda()
+    ws = torch.empty(hip_sdpa.decode_workspace_bytes(Kd, Qd, n_batch, group), dtype=torch.uint8,
+                     device="cuda")
+    lse, A = H.fresh_outputs(batch, q_seq, head, dtype)
+    m, mm = {"causal": (None, hip_sdpa.MASK_CAUSAL), "none": (None, hip_sdpa.MASK_NONE),
+             "bool": (None if mask is None else torch.from_numpy(mask).cuda(), hip_sdpa.MASK_BOOL)}[mode]
+    hip_sdpa.sdpa_fwd_decode(Kd, Qd, m, lse, Vd, A, mm, n_batch, group, ws, causal_offset=offset)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+
+
+def test_decode_merges_into_running_pair(oracle):
+    """Two decode calls over two halves of the cache == one call over all of it."""
+    dtype, q_seq, k_seq, n_batch, group, n_kv, head = "bf16", 16, 512, 2, 4, 2, 128
+    batch = n_batch * group * n_kv
+    (Q, K, V), f32 = H.make_qkv(19, batch, q_seq, k_seq, head, dtype, kv_batch=n_batch * n_kv)
+    offset = k_seq - q_seq
+    want, want_lse = _oracle(oracle, f32, synth.causal_mask(q_seq, k_seq, offset),
+                             n_batch=n_batch, kv_repeat=group)
+    Qd = Q.cuda()
+    lse, A = H.fresh_outputs(batch, q_seq, head, dtype)
+    for lo, hi in [(256, 512), (0, 256)]:
+        Kd, Vd = K[:, lo:hi].contiguous().cuda(), V[:, lo:hi].contiguous().cuda()
+        ws = torch.empty(hip_sdpa.decode_workspace_bytes(Kd, Qd, n_batch, group),
+                         dtype=torch.uint8, device="cuda")
+        hip_sdpa.sdpa_fwd_decode(Kd, Qd, None, lse, Vd, A, hip_sdpa.MASK_CAUSAL, n_batch, group,
+                                 ws, k_pos0=lo, causal_offset=offset)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("head,seq,batch", [(8, 5, 3), (64, 33, 2), (128, 7, 4), (5, 9, 1), (128, 1024, 8)])
+def test_accumulate_attn_output_preset(oracle, dtype, head, seq, batch):
+    # data formulas of tests/kernel/accumulate_attn_output.cc:98-128
+    lin = np.arange(seq * batch)
+    base = -3.0 + 0.25 * (lin % 17)
+    d_on, s_on = ((lin + 1) % 3) != 0, ((lin + 2) % 4) != 0
+    dst_lse = np.where(d_on, base, -np.inf).astype(np.float32)
+    src_lse = np.where(s_on, base + 0.5, -np.inf).astype(np.float32)
+    h = np.arange(head)[None, :]
+    dst = np.where(d_on[:, None], 0.1 * ((lin[:, None] + h) % 11) - 1.0, 0.0).astype(np.float32)
+    src = np.where(s_on[:, None], 0.2 * ((lin[:, None] + h + 3) % 13) - 0.5, 0.0).astype(np.float32)
+    (D, df), (S, sf) = H.rounded(dst.reshape(batch, seq, head), dtype), \
+        H.rounded(src.reshape(batch, seq, head), dtype)
+    want_lse, want = dst_lse.copy(), df.copy()
+    oracle.accumulate_attn_output("fp32", head, seq, batch, src_lse, sf, want_lse, want)
+    Dd, dl = D.cuda(), torch.from_numpy(dst_lse.reshape(batch, seq)).cuda()
+    hip_sdpa.accumulate_attn_output(torch.from_numpy(src_lse.reshape(batch, seq)).cuda(), S.cuda(), dl, Dd)
+    torch.cuda.synchronize()
+    tol = 1e-5 if dtype == "fp32" else 5e-3       # :176-184
+    assert np.max(np.abs(H.to_np(Dd) - want)) < tol * max(1.0, np.abs(want).max())
+    got_lse = H.to_np(dl).ravel()
+    assert np.array_equal(np.isneginf(got_lse), np.isneginf(want_lse))
+    fin = np.isfinite(want_lse)
+    assert np.max(np.abs(got_lse[fin] - want_lse[fin])) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+def test_codelet_body(oracle, dtype):
+    """The StarPU-shaped body with the reference's buffer order, run twice on
+    two key tiles; a bad argument makes the task a no-op."""
+    seq, head, batch = 64, 64, 2
+    (Q, K, V), f32 = H.make_qkv(23, batch, seq, seq, head, dtype)
+    mask = synth.causal_mask(seq, seq)
+    want, want_lse = _oracle(oracle, f32, mask)
+    lse, A = H.fresh_outputs(batch, seq, head, dtype)
+    Kd, Qd, Vd, md = K.cuda(), Q.cuda(), V.cuda(), H.additive_mask(mask, dtype).cuda()
+    s_lse, s_A = torch.empty_like(lse), torch.empty_like(A)
+    torch.cuda.synchronize()
+    hip_sdpa.flash_sdpa_fwd_codelet(Kd, Qd, md, lse, Vd, A, s_lse, s_A, head=48)   # unsupported head
+    torch.cuda.synchronize()
+    assert torch.isneginf(lse).all()
+    hip_sdpa.flash_sdpa_fwd_codelet(Kd, Qd, md, lse, Vd, A, s_lse, s_A)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+
+
+def test_inputs_are_not_modified():
+    # tests/kernel/flash_sdpa_fwd_cudnn.cc:345-362 asserts bit-identical inputs afterwards
+    (Q, K, V), _ = H.make_qkv(29, 2, 128, 128, 64, "bf16")
+    mask = H.additive_mask(synth.causal_mask(128, 128), "bf16")
+    Kd, Qd, Vd, md = K.cuda(), Q.cuda(), V.cuda(), mask.cuda()
+    lse, A = H.fresh_outputs(2, 128, 64, "bf16")
+    hip_sdpa.flash_sdpa_fwd(Kd, Qd, md, lse, Vd, A)
+    torch.cuda.synchronize()
+    for d, h in [(Kd, K), (Qd, Q), (Vd, V), (md, mask)]:
+        assert torch.equal(d.cpu().view(torch.int16), h.view(torch.int16))
