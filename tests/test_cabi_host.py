@@ -1,0 +1,105 @@
+"""CPU-side checks of the C-ABI library: it loads without a GPU, exports every
+symbol the header declares, and rejects bad arguments before touching HIP."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from nntile_amd import hip_sdpa as h
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "nntile_hip_sdpa.h")).read()
+    declared = set(re.findall(r"\b(nntile_hip_[a-z0-9_]+)\s*\(", header))
+    declared -= {"nntile_hip_stream_provider"}
+    assert len(declared) >= 20
+    L = h.lib()
+    for name in sorted(declared):
+        assert hasattr(L, name), name
+    assert set(h.EXPORTS) == declared
+    assert b"gfx950" in L.nntile_hip_sdpa_version()
+
+
+def test_struct_layouts_match_header():
+    assert ctypes.sizeof(h.TileArgs) == 6 * 8 + 8 + 3 * 8 + 6 * 8
+    assert ctypes.sizeof(h.GridArgs) == 8 * 8 + 16 + 3 * 8 + 5 * 64 * 8
+    assert ctypes.sizeof(h.FlashClArgs) == 32
+    assert ctypes.sizeof(h.VariableInterface) == 40
+
+
+def _tile(**kw):
+    a = h.TileArgs()
+    a.q_seq = a.k_seq = 64
+    a.head, a.batch, a.n_batch, a.kv_group = 64, 2, 2, 1
+    a.mask_mode = h.MASK_NONE
+    a.K = a.Q = a.V = a.lse = a.A = 4096       # never dereferenced on these paths
+    for k, v in kw.items():
+        setattr(a, k, v)
+    return a
+
+
+@pytest.mark.parametrize("t", ["bf16", "fp16", "fp32"])
+def test_bad_arguments_are_rejected_before_launch(t):
+    L = h.lib()
+    tile = getattr(L, "nntile_hip_sdpa_fwd_tile_" + t)
+    assert tile(None, None) == h.EINVAL
+    assert tile(None, ctypes.byref(_tile(q_seq=0))) == h.EINVAL
+    assert tile(None, ctypes.byref(_tile(K=None))) == h.EINVAL
+    assert tile(None, ctypes.byref(_tile(K=4100))) == h.EINVAL            # misaligned
+    assert tile(None, ctypes.byref(_tile(mask_mode=7))) == h.EINVAL
+    assert tile(None, ctypes.byref(_tile(mask_mode=h.MASK_ADDITIVE))) == h.EINVAL   # mask missing
+    assert tile(None, ctypes.byref(_tile(kv_group=3))) == h.EINVAL        # batch % (n_batch*group)
+    assert tile(None, ctypes.byref(_tile(head=48))) == h.EUNSUPPORTED
+    flash = getattr(L, "nntile_hip_flash_sdpa_fwd_" + t)
+    assert flash(None, 64, 64, 2, 4096, 4096, None, None, 4096, None, 4096, 4096) == h.EINVAL
+    assert flash(None, -1, 64, 2, 4096, 4096, 4096, None, 4096, None, 4096, 4096) == h.EINVAL
+    grid = getattr(L, "nntile_hip_sdpa_fwd_grid_" + t)
+    g = h.GridArgs()
+    assert grid(None, ctypes.byref(g)) == h.EINVAL
+    g.q_seq = g.k_seq = 256
+    g.q_tile = g.k_tile = 64
+    g.head, g.batch, g.n_batch, g.kv_group = 64, 2, 2, 1
+    g.n_q_tiles, g.n_kv_tiles = 4, 3                                        # 3 != ceil(256/64)
+    g.mask_mode = h.MASK_CAUSAL
+    assert grid(None, ctypes.byref(g)) == h.EINVAL
+    g.n_kv_tiles = 4
+    g.mask_mode = h.MASK_ADDITIVE
+    assert grid(None, ctypes.byref(g)) == h.EUNSUPPORTED
+    g.mask_mode = h.MASK_CAUSAL
+    assert grid(None, ctypes.byref(g)) == h.EINVAL                         # null tile pointers
+
+
+def test_decode_argument_checks():
+    L = h.lib()
+    a = _tile(q_seq=16, k_seq=512, head=128, batch=16, n_batch=2, kv_group=4)
+    need = L.nntile_hip_sdpa_fwd_decode_workspace_bytes(ctypes.byref(a))
+    assert need > 0
+    assert L.nntile_hip_sdpa_fwd_decode_bf16(None, ctypes.byref(a), None, 0) == h.EWORKSPACE
+    assert L.nntile_hip_sdpa_fwd_decode_bf16(None, ctypes.byref(a), 4096, need - 1) == h.EWORKSPACE
+    a.q_seq = 17                                                            # 17*4 rows > 64
+    assert L.nntile_hip_sdpa_fwd_decode_bf16(None, ctypes.byref(a), 4096, 1 << 30) == h.EINVAL
+    assert L.nntile_hip_sdpa_fwd_decode_workspace_bytes(ctypes.byref(a)) == 0
+    a.q_seq, a.head = 16, 32
+    assert L.nntile_hip_sdpa_fwd_decode_bf16(None, ctypes.byref(a), 4096, 1 << 30) == h.EUNSUPPORTED
+
+
+def test_codelet_body_swallows_bad_input(capfd):
+    """Errors in the codelet body are printed and the task becomes a no-op
+    (src/starpu/flash_sdpa_fwd_cudnn.cc:69-115)."""
+    L = h.lib()
+    L.nntile_hip_flash_sdpa_fwd_codelet_bf16(None, None)
+    bufs = (ctypes.c_void_p * 8)()
+    args = h.FlashClArgs(None, 64, 64, 2)
+    L.nntile_hip_flash_sdpa_fwd_codelet_bf16(bufs, ctypes.addressof(args))
+    err = capfd.readouterr().err
+    assert "skipping task" in err
+
+
+def test_accumulate_zero_sizes_return_silently():
+    # src/kernel/accumulate_attn_output/cuda.cu:123-126
+    L = h.lib()
+    assert L.nntile_hip_accumulate_attn_output_fp32(None, 0, 4, 4, None, None, None, None) == h.OK
+    assert L.nntile_hip_accumulate_attn_output_fp32(None, 8, 4, 4, None, None, None, None) == h.EINVAL
