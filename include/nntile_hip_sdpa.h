@@ -36,6 +36,13 @@ extern "C" {
 #define NNTILE_HIP_ELAUNCH      (-3)  /* the HIP runtime refused the launch */
 #define NNTILE_HIP_EWORKSPACE   (-4)  /* workspace missing or too small */
 
+/* flags (tile, grid and decode entry points) */
+/* The running pair is taken to be empty: lse and A are not read, every query
+ * row of the call is written, rows without a visible key get lse = -inf and
+ * A = 0.  Saves the fill of lse (wrappers/python/nntile/layer/sdpa.py:538-539)
+ * and one read of A when the caller knows this is the first key tile. */
+#define NNTILE_HIP_SDPA_OVERWRITE 1
+
 /* How visibility of key k to query q is given. */
 enum nntile_hip_mask_mode
 {
@@ -95,7 +102,7 @@ typedef struct nntile_hip_sdpa_tile_args
     int64_t n_batch;      /* size of the innermost batch axis shared by Q and K/V */
     int64_t kv_group;     /* query heads per key/value head */
     int32_t mask_mode;    /* enum nntile_hip_mask_mode */
-    int32_t reserved;
+    int32_t flags;        /* 0 or NNTILE_HIP_SDPA_OVERWRITE */
     int64_t q_pos0, k_pos0, causal_offset;   /* NNTILE_HIP_MASK_CAUSAL only */
     const void *K, *Q, *mask, *V;
     float *lse;
@@ -122,7 +129,7 @@ typedef struct nntile_hip_sdpa_grid_args
 {
     int64_t q_seq, k_seq, q_tile, k_tile, head;
     int64_t batch, n_batch, kv_group;
-    int32_t mask_mode, n_q_tiles, n_kv_tiles, reserved;
+    int32_t mask_mode, n_q_tiles, n_kv_tiles, flags;
     int64_t q_pos0, k_pos0, causal_offset;
     const void *K[NNTILE_HIP_SDPA_MAX_TILES];
     const void *V[NNTILE_HIP_SDPA_MAX_TILES];

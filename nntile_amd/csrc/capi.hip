@@ -91,6 +91,7 @@ static int tile_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a)
     p.batch = (int32_t)a->batch;
     p.n_batch = (int32_t)a->n_batch;
     p.kv_group = (int32_t)a->kv_group;
+    p.overwrite = (a->flags & NNTILE_HIP_SDPA_OVERWRITE) ? 1 : 0;
     p.K[0] = a->K;
     p.V[0] = a->V;
     p.Q[0] = a->Q;
@@ -160,6 +161,7 @@ static int grid_call(DType dt, void *stream, const nntile_hip_sdpa_grid_args *a)
     p.batch = (int32_t)a->batch;
     p.n_batch = (int32_t)a->n_batch;
     p.kv_group = (int32_t)a->kv_group;
+    p.overwrite = (a->flags & NNTILE_HIP_SDPA_OVERWRITE) ? 1 : 0;
     for(int t = 0; t < a->n_kv_tiles; ++t)
     {
         if(a->K[t] == nullptr || a->V[t] == nullptr || !aligned16(a->K[t])
@@ -252,6 +254,7 @@ static int decode_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *
     p.rows = rows;
     p.n_splits = splits;
     p.n_steps = n_steps;
+    p.overwrite = (a->flags & NNTILE_HIP_SDPA_OVERWRITE) ? 1 : 0;
     p.steps_per_split = (n_steps + splits - 1) / splits;
     p.scale = 1.0f / sqrtf(static_cast<float>(a->head));
     hipStream_t s = static_cast<hipStream_t>(stream);

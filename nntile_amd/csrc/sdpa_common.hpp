@@ -34,6 +34,7 @@ struct PrefillParams
     int32_t q_blocks_per_tile;    // ceil(q_tile / rows per workgroup)
     int32_t k_blocks_per_tile;    // ceil(k_tile / keys per step)
     int32_t xcd_remap;            // 1: regroup workgroups so a slab stays on one XCD
+    int32_t overwrite;            // 1: ignore the running pair, write every row
     float scale;                  // 1/sqrt(head)
     const void *K[kMaxTiles];
     const void *V[kMaxTiles];
@@ -58,6 +59,7 @@ struct DecodeParams
     int32_t n_batch, kv_group, n_head_kv;
     int32_t rows;       // kv_group * q_seq
     int32_t n_splits, steps_per_split, n_steps;
+    int32_t overwrite;
     float scale;
 };
 

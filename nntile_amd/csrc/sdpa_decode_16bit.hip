@@ -18,7 +18,7 @@
 namespace nntile_hip
 {
 
-constexpr int kDecRows = 64;      // query rows per workgroup (4 wavefronts x 16)
+
 constexpr int kDecKeys = 64;      // keys per step
 constexpr int kDecThreads = 256;
 
@@ -366,9 +366,21 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
     {
         top = fmaxf(top, p.part_ml[2 * (base + (int64_t)s * p.rows)]);
     }
+    const int64_t row = qb * p.q_seq + tok;
+    uint16_t *Arow = static_cast<uint16_t *>(p.A) + row * HEAD;
     if(top == neg_inf())
     {
-        return;         // no visible key at all: leave lse and A untouched
+        // no visible key at all: leave lse and A untouched, or write the
+        // empty row when the running pair is being overwritten
+        if(p.overwrite)
+        {
+            Arow[d] = 0;
+            if(d == 0)
+            {
+                p.lse[row] = neg_inf();
+            }
+        }
+        return;
     }
     float l = 0.0f, acc = 0.0f;
     for(int s = 0; s < p.n_splits; ++s)
@@ -384,11 +396,9 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
         acc += w * p.part_o[prow * HEAD + d];
     }
     const float lse_new = top + __logf(l);
-    const int64_t row = qb * p.q_seq + tok;
-    const float lse_old = p.lse[row];
+    const float lse_old = p.overwrite ? neg_inf() : p.lse[row];
     float w_old, w_new, lse_out;
     merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
-    uint16_t *Arow = static_cast<uint16_t *>(p.A) + row * HEAD;
     float v = acc * (w_new / l);
     if(w_old != 0.0f)
     {

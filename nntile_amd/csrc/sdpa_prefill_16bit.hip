@@ -20,10 +20,12 @@
 // 8 head values, regroups them in registers and writes 8 x (4 keys) so that
 // every MFMA operand is a single 16-byte LDS read.
 //
-// The running (max, sum) pair lives in registers across all key tiles of a
-// query tile; the epilogue merges the result into the (lse, A) pair in memory
-// (the hand-off between NNTile tasks), so one launch can stand for one task or
-// for a whole row of tasks.
+// K and V steps are double-buffered in LDS (one barrier per step); the global
+// loads of step g+1 are in flight while step g is computed.  The running
+// (max, sum) pair lives in registers across all key tiles of a query tile;
+// the epilogue merges the result into the (lse, A) pair in memory (the
+// hand-off between NNTile tasks), so one launch can stand for one task or for
+// a whole row of tasks.
 #include "sdpa_common.hpp"
 
 namespace nntile_hip
@@ -32,6 +34,13 @@ namespace nntile_hip
 constexpr int kQRows = 128;     // queries per workgroup
 constexpr int kKeys = 64;       // keys per step
 constexpr int kThreads = 256;
+
+// Walks the key steps of all key tiles in order: tile kt, step kb within the
+// tile, rows left in the tile from this step on.
+struct StepCursor
+{
+    int kt, kb, rows_left;
+};
 
 template<typename T, int HEAD, int MODE>
 __global__ __launch_bounds__(kThreads, 2)
@@ -43,11 +52,12 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     constexpr int KPAD = HEAD + 8;          // K row stride in LDS (elements)
     constexpr int VPAD = kKeys + 8;         // V^T row stride in LDS
     constexpr int CHUNKS = HEAD / 8;        // 16-byte chunks per row
+    constexpr int K_ELEMS = kKeys * KPAD;
+    constexpr int BUF_ELEMS = K_ELEMS + HEAD * VPAD;
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
 
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[kKeys * KPAD];
-    __shared__ __attribute__((aligned(16))) uint16_t Vt[HEAD * VPAD];
+    __shared__ __attribute__((aligned(16))) uint16_t lds[2 * BUF_ELEMS];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -56,23 +66,29 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     const int half = lane >> 5;
 
     // ---- which queries --------------------------------------------------
+    // Workgroups are dealt round-robin to the 8 XCDs.  With xcd_remap every
+    // XCD gets a contiguous range of batch entries (their query blocks share
+    // K and V in that XCD's L2); in both layouts the query blocks are handed
+    // out last-first, all batch entries of a block before the next block, so
+    // that under a causal mask the longest workgroups start first.
     const int q_blocks = p.n_q_tiles * p.q_blocks_per_tile;
-    int wg = blockIdx.x;
+    int b, qblk;
     if(p.xcd_remap)
     {
-        // Workgroups are dealt round-robin to the 8 XCDs; regroup them so that
-        // the query blocks of one batch entry (which share K and V) meet in
-        // one XCD's L2.
-        const int per_xcd = gridDim.x >> 3;
-        wg = (wg & 7) * per_xcd + (wg >> 3);
+        const int b_per_xcd = p.batch >> 3;
+        const int i = (int)(blockIdx.x >> 3);
+        b = (int)(blockIdx.x & 7) * b_per_xcd + i % b_per_xcd;
+        qblk = q_blocks - 1 - i / b_per_xcd;
     }
-    const int b = wg / q_blocks;
-    // heaviest (last) query blocks first
-    const int qblk = q_blocks - 1 - (wg % q_blocks);
+    else
+    {
+        b = (int)blockIdx.x % p.batch;
+        qblk = q_blocks - 1 - (int)blockIdx.x / p.batch;
+    }
     const int qt = qblk / p.q_blocks_per_tile;
     const int qb = qblk % p.q_blocks_per_tile;
-    const int64_t q_len = min(p.q_tile, p.q_seq - (int64_t)qt * p.q_tile);
-    const int64_t q_row0 = (int64_t)qb * kQRows;            // within the tile
+    const int q_len = (int)min(p.q_tile, p.q_seq - (int64_t)qt * p.q_tile);
+    const int q_row0 = qb * kQRows;                     // within the tile
     if(q_row0 >= q_len)
     {
         return;
@@ -81,14 +97,13 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
 
     const uint16_t *Qt = static_cast<const uint16_t *>(p.Q[qt])
         + (int64_t)b * q_len * HEAD;
-    const int64_t my_q = q_row0 + wave * 32 + col;          // row within tile
+    const int my_q = q_row0 + wave * 32 + col;          // row within tile
     const bool q_ok = my_q < q_len;
-    const int64_t my_qpos = p.q_pos0 + (int64_t)qt * p.q_tile + my_q;
 
     // Q fragments, resident for the whole kernel.
     vec8 qf[KSTEPS];
     {
-        const uint16_t *src = Qt + (q_ok ? my_q : 0) * HEAD + half * 8;
+        const uint16_t *src = Qt + (int64_t)(q_ok ? my_q : 0) * HEAD + half * 8;
 #pragma unroll
         for(int ks = 0; ks < KSTEPS; ++ks)
         {
@@ -102,19 +117,41 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     }
 
     // ---- which keys --------------------------------------------------------
-    // Steps are numbered over all key tiles; step g covers keys
-    // [kb*64, kb*64+64) of tile kt = g / k_blocks_per_tile.
-    const int64_t last_k_len = p.k_seq - (int64_t)(p.n_kv_tiles - 1) * p.k_tile;
+    // rel0: position of the workgroup's first query minus the position of key
+    // row 0, plus the causal offset; key row kg is visible to query row
+    // (q_row0 + r) iff kg <= rel0 + r.  Clamped so that the 32-bit arithmetic
+    // below cannot overflow.
+    const int k_seq = (int)p.k_seq, k_tile = (int)p.k_tile;
+    int rel0 = 0;
+    const int last_k_len = k_seq - (p.n_kv_tiles - 1) * k_tile;
     int n_steps = (p.n_kv_tiles - 1) * p.k_blocks_per_tile
-        + (int)((last_k_len + kKeys - 1) / kKeys);
-    // Positions of the first/last query of this workgroup and wavefront.
-    const int64_t wg_qpos_hi = p.q_pos0 + (int64_t)qt * p.q_tile
-        + min(q_row0 + kQRows, q_len) - 1;
-    const int64_t wave_qpos_lo = p.q_pos0 + (int64_t)qt * p.q_tile + q_row0
-        + wave * 32;
-    const int64_t wave_qpos_hi = wave_qpos_lo + 31;
+        + (last_k_len + kKeys - 1) / kKeys;
+    if(MODE == NNTILE_HIP_MASK_CAUSAL)
+    {
+        int64_t rel = p.q_pos0 + (int64_t)qt * p.q_tile + q_row0
+            + p.causal_offset - p.k_pos0;
+        rel = max((int64_t)-(1 << 30), min(rel, (int64_t)(1 << 30)));
+        rel0 = (int)rel;
+        const int hi = min(rel0 + min(kQRows, q_len - q_row0) - 1, k_seq - 1);
+        if(hi < 0)
+        {
+            if(!p.overwrite)
+            {
+                return;
+            }
+            n_steps = 0;    // nothing visible: the epilogue writes empty rows
+        }
+        else
+        {
+            const int kt_hi = hi / k_tile;
+            n_steps = min(n_steps, kt_hi * p.k_blocks_per_tile
+                    + (hi - kt_hi * k_tile) / kKeys + 1);
+        }
+    }
+    const int wave_rel_lo = rel0 + wave * 32;       // first query of the wavefront
+    const int my_rel = wave_rel_lo + col;
 
-    // Cooperative load assignment.
+    // ---- cooperative load assignment ----------------------------------------
     // K: 64 rows x CHUNKS chunks of 16 B, thread t takes chunk t % CHUNKS of
     //    rows t / CHUNKS + i * (256 / CHUNKS).
     constexpr int K_ROWS_PER_PASS = kThreads / CHUNKS;
@@ -132,49 +169,93 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // order is [h][a][c] for key = 8a + 4h + c, which is the order in which
     // the S^T accumulators of lane half h list their keys.
     const int v_pos = 16 * (v_kg >> 2) + 8 * (v_kg & 1) + 4 * ((v_kg & 3) >> 1);
+    // Byte offsets of this thread's loads within a full 64-row step.
+    const uint32_t k_goff = (uint32_t)(k_row * HEAD + k_chunk * 8) * 2u;
+    const uint32_t v_goff = (uint32_t)(4 * v_kg * HEAD + v_chunk * 8) * 2u;
+    // LDS element offsets of this thread's stores.
+    const int k_soff = k_row * KPAD + k_chunk * 8;
+    const int v_soff = K_ELEMS + (v_chunk * 8) * VPAD + v_pos;
 
     u32x4 k_regs[K_PASSES];
     u32x4 v_regs[4];
 
-    auto fetch = [&](int g)
+    auto tile_rows = [&](int kt) -> int
     {
-        const int kt = g / p.k_blocks_per_tile;
-        const int kb = g % p.k_blocks_per_tile;
-        const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
-        const int64_t row0 = (int64_t)kb * kKeys;
-        const uint16_t *Kt = static_cast<const uint16_t *>(p.K[kt])
-            + ((int64_t)kvb * k_len) * HEAD;
-        const uint16_t *Vtile = static_cast<const uint16_t *>(p.V[kt])
-            + ((int64_t)kvb * k_len) * HEAD;
-#pragma unroll
-        for(int i = 0; i < K_PASSES; ++i)
-        {
-            const int64_t r = row0 + k_row + i * K_ROWS_PER_PASS;
-            k_regs[i] = (r < k_len)
-                ? *reinterpret_cast<const u32x4 *>(Kt + r * HEAD + k_chunk * 8)
-                : u32x4{0, 0, 0, 0};
-        }
-        if(v_active)
+        return min(k_tile, k_seq - kt * k_tile);
+    };
+
+    // Global loads of one step into registers.  Rows past the end of the tile
+    // are clamped to its last row: their scores are masked and their
+    // probabilities are exactly 0, so any finite stand-in value works.
+    auto fetch = [&](const StepCursor &cur)
+    {
+        const int k_len = tile_rows(cur.kt);
+        const int64_t base = ((int64_t)kvb * k_len + (int64_t)cur.kb * kKeys)
+            * HEAD * 2;
+        const char *Kp = static_cast<const char *>(p.K[cur.kt]) + base;
+        const char *Vp = static_cast<const char *>(p.V[cur.kt]) + base;
+        if(cur.rows_left >= kKeys)
         {
 #pragma unroll
-            for(int j = 0; j < 4; ++j)
+            for(int i = 0; i < K_PASSES; ++i)
             {
-                const int64_t r = row0 + 4 * v_kg + j;
-                v_regs[j] = (r < k_len)
-                    ? *reinterpret_cast<const u32x4 *>(Vtile + r * HEAD
-                            + v_chunk * 8)
-                    : u32x4{0, 0, 0, 0};
+                k_regs[i] = *reinterpret_cast<const u32x4 *>(Kp + k_goff
+                        + (uint32_t)(i * K_ROWS_PER_PASS * HEAD * 2));
+            }
+            if(v_active)
+            {
+#pragma unroll
+                for(int j = 0; j < 4; ++j)
+                {
+                    v_regs[j] = *reinterpret_cast<const u32x4 *>(Vp + v_goff
+                            + (uint32_t)(j * HEAD * 2));
+                }
+            }
+        }
+        else
+        {
+            const int last = cur.rows_left - 1;
+#pragma unroll
+            for(int i = 0; i < K_PASSES; ++i)
+            {
+                const int r = min(k_row + i * K_ROWS_PER_PASS, last);
+                k_regs[i] = *reinterpret_cast<const u32x4 *>(Kp
+                        + (uint32_t)(r * HEAD + k_chunk * 8) * 2u);
+            }
+            if(v_active)
+            {
+#pragma unroll
+                for(int j = 0; j < 4; ++j)
+                {
+                    const int r = min(4 * v_kg + j, last);
+                    v_regs[j] = *reinterpret_cast<const u32x4 *>(Vp
+                            + (uint32_t)(r * HEAD + v_chunk * 8) * 2u);
+                }
             }
         }
     };
 
-    auto stage = [&]()
+    auto advance = [&](StepCursor &cur)
     {
+        cur.kb += 1;
+        cur.rows_left -= kKeys;
+        if(cur.rows_left <= 0)
+        {
+            cur.kt += 1;
+            cur.kb = 0;
+            cur.rows_left = (cur.kt < p.n_kv_tiles) ? tile_rows(cur.kt) : 0;
+        }
+    };
+
+    // Registers -> LDS buffer `buf`: K as is, V regrouped to [head][key].
+    auto stage = [&](int buf)
+    {
+        uint16_t *base = lds + buf * BUF_ELEMS;
 #pragma unroll
         for(int i = 0; i < K_PASSES; ++i)
         {
-            *reinterpret_cast<u32x4 *>(&Ks[(k_row + i * K_ROWS_PER_PASS) * KPAD
-                    + k_chunk * 8]) = k_regs[i];
+            *reinterpret_cast<u32x4 *>(base + k_soff
+                    + i * K_ROWS_PER_PASS * KPAD) = k_regs[i];
         }
         if(v_active)
         {
@@ -189,30 +270,11 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 even[1] = __builtin_amdgcn_perm(r3, r2, 0x05040100u);
                 odd[0] = __builtin_amdgcn_perm(r1, r0, 0x07060302u);
                 odd[1] = __builtin_amdgcn_perm(r3, r2, 0x07060302u);
-                const int d = v_chunk * 8 + 2 * w;
-                *reinterpret_cast<u32x2 *>(&Vt[d * VPAD + v_pos]) = even;
-                *reinterpret_cast<u32x2 *>(&Vt[(d + 1) * VPAD + v_pos]) = odd;
+                *reinterpret_cast<u32x2 *>(base + v_soff + (2 * w) * VPAD) = even;
+                *reinterpret_cast<u32x2 *>(base + v_soff + (2 * w + 1) * VPAD) = odd;
             }
         }
     };
-
-    // In CAUSAL mode steps past the last visible key of the workgroup are
-    // never run.
-    if(MODE == NNTILE_HIP_MASK_CAUSAL)
-    {
-        const int64_t hi = wg_qpos_hi + p.causal_offset - p.k_pos0; // last visible key row overall
-        if(hi < 0)
-        {
-            return;
-        }
-        const int64_t kt_hi = hi / p.k_tile;
-        if(kt_hi < p.n_kv_tiles)
-        {
-            const int64_t in_tile = hi - kt_hi * p.k_tile;
-            const int steps = (int)(kt_hi * p.k_blocks_per_tile + in_tile / kKeys + 1);
-            n_steps = min(n_steps, steps);
-        }
-    }
 
     // Score units: in the analytic modes the raw dot product is kept and the
     // scale is folded into the exponent; with an explicit mask the score is
@@ -232,201 +294,239 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     float m_run = neg_inf();
     float l_run = 0.0f;      // this lane half's share of the row sum
 
-    fetch(0);
+    StepCursor cur = {0, 0, tile_rows(0)};      // step being computed
+    StepCursor nxt = cur;                        // step being fetched
+    if(n_steps > 0)
+    {
+        fetch(nxt);
+        advance(nxt);
+        stage(0);
+        if(n_steps > 1)
+        {
+            fetch(nxt);
+            advance(nxt);
+        }
+    }
+    __syncthreads();
+
     for(int g = 0; g < n_steps; ++g)
     {
-        __syncthreads();            // previous step's LDS reads are done
-        stage();
-        __syncthreads();
-        if(g + 1 < n_steps)
-        {
-            fetch(g + 1);           // in flight during the arithmetic below
-        }
+        const int buf = g & 1;
+        const uint16_t *Ks = lds + buf * BUF_ELEMS;
+        const uint16_t *Vt = Ks + K_ELEMS;
+        const int k_row0 = cur.kb * kKeys;                   // within the tile
+        const int kg0 = cur.kt * k_tile + k_row0;            // key row overall
+        const int keys_here = min(kKeys, cur.rows_left);
+        // nothing of this step is visible to this wavefront
+        const bool idle = (MODE == NNTILE_HIP_MASK_CAUSAL)
+            && (kg0 > wave_rel_lo + 31);
 
-        const int kt = g / p.k_blocks_per_tile;
-        const int kb = g % p.k_blocks_per_tile;
-        const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
-        const int64_t k_row0 = (int64_t)kb * kKeys;          // within the tile
-        const int64_t k_pos_base = p.k_pos0 + (int64_t)kt * p.k_tile + k_row0;
-        const int keys_here = (int)min((int64_t)kKeys, k_len - k_row0);
-
-        if(MODE == NNTILE_HIP_MASK_CAUSAL
-                && k_pos_base > wave_qpos_hi + p.causal_offset)
+        uint32_t pk[2][8];
+        if(!idle)
         {
-            continue;               // nothing visible to this wavefront
-        }
-
-        // ---- S^T = K Q^T ---------------------------------------------------
-        f32x16 s[2];
-#pragma unroll
-        for(int mb = 0; mb < 2; ++mb)
-        {
-#pragma unroll
-            for(int r = 0; r < 16; ++r)
-            {
-                s[mb][r] = 0.0f;
-            }
-#pragma unroll
-            for(int ks = 0; ks < KSTEPS; ++ks)
-            {
-                const vec8 a = *reinterpret_cast<const vec8 *>(
-                        &Ks[(mb * 32 + col) * KPAD + ks * 16 + half * 8]);
-                s[mb] = T::mfma(a, qf[ks], s[mb]);
-            }
-        }
-
-        // ---- mask -----------------------------------------------------------
-        // register r of block mb holds key  mb*32 + 8*(r/4) + 4*half + r%4
-        if(EXPLICIT)
-        {
-            const int64_t qrow = q_ok ? my_q : 0;
+            // ---- S^T = K Q^T -------------------------------------------------
+            f32x16 s[2];
 #pragma unroll
             for(int mb = 0; mb < 2; ++mb)
             {
 #pragma unroll
-                for(int rg = 0; rg < 4; ++rg)
+                for(int r = 0; r < 16; ++r)
                 {
-                    const int key0 = mb * 32 + 8 * rg + 4 * half;
-                    const int64_t krow = k_row0 + key0;
-                    float add[4];
-                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
-                    {
-                        const uint16_t *mp = static_cast<const uint16_t *>(p.mask)
-                            + qrow * p.mask_ld + krow;
+                    s[mb][r] = 0.0f;
+                }
 #pragma unroll
-                        for(int e = 0; e < 4; ++e)
-                        {
-                            add[e] = (key0 + e < keys_here)
-                                ? T::to_float(mp[e]) : neg_inf();
-                        }
-                    }
-                    else
-                    {
-                        const uint8_t *mp = static_cast<const uint8_t *>(p.mask)
-                            + qrow * p.mask_ld + krow;
-#pragma unroll
-                        for(int e = 0; e < 4; ++e)
-                        {
-                            add[e] = (key0 + e < keys_here && mp[e] != 0)
-                                ? 0.0f : neg_inf();
-                        }
-                    }
-#pragma unroll
-                    for(int e = 0; e < 4; ++e)
-                    {
-                        const float v = s[mb][4 * rg + e] * p.scale + add[e];
-                        // a hidden key stays hidden whatever the score is
-                        s[mb][4 * rg + e] = (add[e] == neg_inf()) ? neg_inf() : v;
-                    }
+                for(int ks = 0; ks < KSTEPS; ++ks)
+                {
+                    const vec8 a = *reinterpret_cast<const vec8 *>(
+                            &Ks[(mb * 32 + col) * KPAD + ks * 16 + half * 8]);
+                    s[mb] = T::mfma(a, qf[ks], s[mb]);
                 }
             }
-        }
-        else
-        {
-            const bool ragged = keys_here < kKeys;
-            const bool diagonal = (MODE == NNTILE_HIP_MASK_CAUSAL)
-                && (k_pos_base + kKeys - 1 > wave_qpos_lo + p.causal_offset);
-            if(ragged || diagonal)
+
+            // ---- mask ---------------------------------------------------------
+            // register r of block mb holds key  mb*32 + 8*(r/4) + 4*half + r%4
+            if(EXPLICIT)
             {
-                const int64_t vis = (MODE == NNTILE_HIP_MASK_CAUSAL)
-                    ? (my_qpos + p.causal_offset - k_pos_base)   // last visible key in step
-                    : (int64_t)kKeys;
-                const int lim = (int)max((int64_t)-1,
-                        min(vis, (int64_t)keys_here - 1));
+                const int64_t qrow = q_ok ? my_q : 0;
 #pragma unroll
                 for(int mb = 0; mb < 2; ++mb)
                 {
 #pragma unroll
-                    for(int r = 0; r < 16; ++r)
+                    for(int rg = 0; rg < 4; ++rg)
                     {
-                        const int key = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                        if(key > lim)
+                        const int key0 = mb * 32 + 8 * rg + 4 * half;
+                        const int64_t krow = k_row0 + key0;
+                        float add[4];
+                        if(MODE == NNTILE_HIP_MASK_ADDITIVE)
                         {
-                            s[mb][r] = neg_inf();
+                            const uint16_t *mp = static_cast<const uint16_t *>(
+                                    p.mask) + qrow * p.mask_ld + krow;
+#pragma unroll
+                            for(int e = 0; e < 4; ++e)
+                            {
+                                add[e] = (key0 + e < keys_here)
+                                    ? T::to_float(mp[e]) : neg_inf();
+                            }
+                        }
+                        else
+                        {
+                            const uint8_t *mp = static_cast<const uint8_t *>(
+                                    p.mask) + qrow * p.mask_ld + krow;
+#pragma unroll
+                            for(int e = 0; e < 4; ++e)
+                            {
+                                add[e] = (key0 + e < keys_here && mp[e] != 0)
+                                    ? 0.0f : neg_inf();
+                            }
+                        }
+#pragma unroll
+                        for(int e = 0; e < 4; ++e)
+                        {
+                            const float v = s[mb][4 * rg + e] * p.scale + add[e];
+                            // a hidden key stays hidden whatever the score is
+                            s[mb][4 * rg + e] = (add[e] == neg_inf())
+                                ? neg_inf() : v;
                         }
                     }
                 }
             }
+            else
+            {
+                const bool ragged = keys_here < kKeys;
+                const bool diagonal = (MODE == NNTILE_HIP_MASK_CAUSAL)
+                    && (kg0 + kKeys - 1 > wave_rel_lo);
+                if(ragged || diagonal)
+                {
+                    // last visible key of this step for this lane's query
+                    int lim = keys_here - 1;
+                    if(MODE == NNTILE_HIP_MASK_CAUSAL)
+                    {
+                        lim = min(lim, my_rel - kg0);
+                    }
+#pragma unroll
+                    for(int mb = 0; mb < 2; ++mb)
+                    {
+#pragma unroll
+                        for(int r = 0; r < 16; ++r)
+                        {
+                            const int key = mb * 32 + 8 * (r >> 2) + 4 * half
+                                + (r & 3);
+                            if(key > lim)
+                            {
+                                s[mb][r] = neg_inf();
+                            }
+                        }
+                    }
+                }
+            }
+
+            // ---- online softmax -------------------------------------------------
+            float mx = neg_inf();
+#pragma unroll
+            for(int mb = 0; mb < 2; ++mb)
+            {
+#pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    mx = fmaxf(mx, s[mb][r]);
+                }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run, mx);
+            const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+            const float mc = m_use * c;
+            // The running maximum rarely moves after the first steps; the
+            // rescale of the 16*DBLOCKS output registers is skipped unless
+            // some query of the wavefront needs it.
+            if(__builtin_amdgcn_ballot_w64(m_new != m_run) != 0)
+            {
+                const float alpha = fast_exp2((m_run - m_use) * c);
+                l_run *= alpha;
+#pragma unroll
+                for(int db = 0; db < DBLOCKS; ++db)
+                {
+#pragma unroll
+                    for(int r = 0; r < 16; ++r)
+                    {
+                        o[db][r] *= alpha;
+                    }
+                }
+                m_run = m_new;
+            }
+
+            float rs = 0.0f;
+#pragma unroll
+            for(int mb = 0; mb < 2; ++mb)
+            {
+#pragma unroll
+                for(int r = 0; r < 16; r += 2)
+                {
+                    const float p0 = fast_exp2(fmaf(s[mb][r], c, -mc));
+                    const float p1 = fast_exp2(fmaf(s[mb][r + 1], c, -mc));
+                    rs += p0 + p1;
+                    pk[mb][r >> 1] = T::pack2(p0, p1);
+                }
+            }
+            l_run += rs;
         }
 
-        // ---- online softmax ---------------------------------------------------
-        float mx = neg_inf();
-#pragma unroll
-        for(int mb = 0; mb < 2; ++mb)
+        // ---- next step: registers -> the other LDS buffer, then new loads -----
+        // (every wavefront passed the barrier that ended step g-1, so nobody
+        // still reads that buffer)
+        if(g + 1 < n_steps)
         {
-#pragma unroll
-            for(int r = 0; r < 16; ++r)
+            stage(buf ^ 1);
+            if(g + 2 < n_steps)
             {
-                mx = fmaxf(mx, s[mb][r]);
-            }
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
-        const float alpha = fast_exp2((m_run - m_use) * c);
-        const float mc = m_use * c;
-        m_run = m_new;
-
-        float rs = 0.0f;
-        uint32_t pk[2][8];
-#pragma unroll
-        for(int mb = 0; mb < 2; ++mb)
-        {
-#pragma unroll
-            for(int r = 0; r < 16; r += 2)
-            {
-                const float p0 = fast_exp2(fmaf(s[mb][r], c, -mc));
-                const float p1 = fast_exp2(fmaf(s[mb][r + 1], c, -mc));
-                rs += p0 + p1;
-                pk[mb][r >> 1] = T::pack2(p0, p1);
-            }
-        }
-        l_run = l_run * alpha + rs;
-#pragma unroll
-        for(int db = 0; db < DBLOCKS; ++db)
-        {
-#pragma unroll
-            for(int r = 0; r < 16; ++r)
-            {
-                o[db][r] *= alpha;
+                fetch(nxt);
+                advance(nxt);
             }
         }
 
-        // ---- O^T += V^T P^T ----------------------------------------------------
-#pragma unroll
-        for(int t = 0; t < 4; ++t)
+        // ---- O^T += V^T P^T ------------------------------------------------------
+        if(!idle)
         {
-            const int mb = t >> 1, tt = t & 1;
-            const u32x4 praw = {pk[mb][4 * tt], pk[mb][4 * tt + 1],
-                pk[mb][4 * tt + 2], pk[mb][4 * tt + 3]};
-            const vec8 pb = __builtin_bit_cast(vec8, praw);
 #pragma unroll
-            for(int db = 0; db < DBLOCKS; ++db)
+            for(int t = 0; t < 4; ++t)
             {
-                const vec8 a = *reinterpret_cast<const vec8 *>(
-                        &Vt[(db * 32 + col) * VPAD + 16 * t + 8 * half]);
-                o[db] = T::mfma(a, pb, o[db]);
+                const int mb = t >> 1, tt = t & 1;
+                const u32x4 praw = {pk[mb][4 * tt], pk[mb][4 * tt + 1],
+                    pk[mb][4 * tt + 2], pk[mb][4 * tt + 3]};
+                const vec8 pb = __builtin_bit_cast(vec8, praw);
+#pragma unroll
+                for(int db = 0; db < DBLOCKS; ++db)
+                {
+                    const vec8 a = *reinterpret_cast<const vec8 *>(
+                            &Vt[(db * 32 + col) * VPAD + 16 * t + 8 * half]);
+                    o[db] = T::mfma(a, pb, o[db]);
+                }
             }
         }
+        advance(cur);
+        __syncthreads();
     }
 
     // ---- epilogue: normalise, merge into the running (lse, A) ----------------
     const float l_tot = l_run + __shfl_xor(l_run, 32);
-    if(!q_ok || !(l_tot > 0.0f))
+    const bool empty = !(l_tot > 0.0f);     // no visible key for this query
+    if(!q_ok || (empty && !p.overwrite))
     {
-        return;     // no visible key: leave lse and A as they are
+        return;     // leave lse and A as they are
     }
     const float to_ln = EXPLICIT ? 1.0f : p.scale;
-    const float lse_new = m_run * to_ln + __logf(l_tot);
+    const float lse_new = empty ? neg_inf() : m_run * to_ln + __logf(l_tot);
     float *lse_ptr = p.lse[qt] + (int64_t)b * q_len + my_q;
-    const float lse_old = *lse_ptr;
-    float w_old, w_new, lse_out;
-    merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
+    const float lse_old = p.overwrite ? neg_inf() : *lse_ptr;
+    float w_old = 0.0f, w_new = 0.0f, lse_out = neg_inf();
+    if(!empty)
+    {
+        merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
+    }
     if(half == 0)
     {
         *lse_ptr = lse_out;
     }
-    const float w_o = w_new / l_tot;
+    const float w_o = empty ? 0.0f : w_new / l_tot;
     uint16_t *Arow = static_cast<uint16_t *>(p.A[qt])
         + ((int64_t)b * q_len + my_q) * HEAD;
     // register r of block db holds head value  db*32 + 8*(r/4) + 4*half + r%4
@@ -441,7 +541,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
 #pragma unroll
             for(int e = 0; e < 4; ++e)
             {
-                v[e] = o[db][4 * rg + e] * w_o;
+                v[e] = empty ? 0.0f : o[db][4 * rg + e] * w_o;
             }
             if(w_old != 0.0f)
             {
@@ -504,7 +604,7 @@ int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
     {
         return NNTILE_HIP_EINVAL;
     }
-    p.xcd_remap = (n_wg % 8 == 0) ? 1 : 0;
+    p.xcd_remap = (p.batch % 8 == 0) ? 1 : 0;
     const dim3 grid((unsigned)n_wg);
     switch(head)
     {

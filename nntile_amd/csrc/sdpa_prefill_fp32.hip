@@ -132,9 +132,13 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         const int64_t hi = wg_qpos_hi + p.causal_offset - p.k_pos0;
         if(hi < 0)
         {
-            return;
+            if(!p.overwrite)
+            {
+                return;
+            }
+            n_steps = 0;    // nothing visible: the epilogue writes empty rows
         }
-        const int64_t kt_hi = hi / p.k_tile;
+        const int64_t kt_hi = hi < 0 ? (int64_t)p.n_kv_tiles : hi / p.k_tile;
         if(kt_hi < p.n_kv_tiles)
         {
             const int64_t in_tile = hi - kt_hi * p.k_tile;
@@ -159,7 +163,10 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     float m_run = neg_inf();
     float l_run = 0.0f;
 
-    fetch(0);
+    if(n_steps > 0)
+    {
+        fetch(0);
+    }
     for(int g = 0; g < n_steps; ++g)
     {
         __syncthreads();
@@ -307,21 +314,25 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
 
     // ---- epilogue --------------------------------------------------------------
     const float l_tot = l_run + __shfl_xor(l_run, 32);
-    if(!q_ok || !(l_tot > 0.0f))
+    const bool empty = !(l_tot > 0.0f);     // no visible key for this query
+    if(!q_ok || (empty && !p.overwrite))
     {
-        return;
+        return;     // leave lse and A as they are
     }
     const float to_ln = EXPLICIT ? 1.0f : p.scale;
-    const float lse_new = m_run * to_ln + __logf(l_tot);
+    const float lse_new = empty ? neg_inf() : m_run * to_ln + __logf(l_tot);
     float *lse_ptr = p.lse[qt] + (int64_t)b * q_len + my_q;
-    const float lse_old = *lse_ptr;
-    float w_old, w_new, lse_out;
-    merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
+    const float lse_old = p.overwrite ? neg_inf() : *lse_ptr;
+    float w_old = 0.0f, w_new = 0.0f, lse_out = neg_inf();
+    if(!empty)
+    {
+        merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
+    }
     if(half == 0)
     {
         *lse_ptr = lse_out;
     }
-    const float w_o = w_new / l_tot;
+    const float w_o = empty ? 0.0f : w_new / l_tot;
     float *Arow = static_cast<float *>(p.A[qt])
         + ((int64_t)b * q_len + my_q) * HEAD;
 #pragma unroll
@@ -335,7 +346,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
 #pragma unroll
             for(int e = 0; e < 4; ++e)
             {
-                v[e] = o[db][4 * rg + e] * w_o;
+                v[e] = empty ? 0.0f : o[db][4 * rg + e] * w_o;
             }
             if(w_old != 0.0f)
             {

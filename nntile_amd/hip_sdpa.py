@@ -18,6 +18,7 @@ LIB_PATH = os.path.join(_HERE, "libnntile_hip_sdpa.so")
 
 MASK_ADDITIVE, MASK_NONE, MASK_CAUSAL, MASK_BOOL = 0, 1, 2, 3
 MAX_TILES = 64
+OVERWRITE = 1
 
 OK, EINVAL, EUNSUPPORTED, ELAUNCH, EWORKSPACE = 0, -1, -2, -3, -4
 _ERR = {EINVAL: "invalid argument", EUNSUPPORTED: "unsupported configuration",
@@ -30,7 +31,7 @@ _vp = ctypes.c_void_p
 class TileArgs(ctypes.Structure):
     _fields_ = [("q_seq", _i64), ("k_seq", _i64), ("head", _i64),
                 ("batch", _i64), ("n_batch", _i64), ("kv_group", _i64),
-                ("mask_mode", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("mask_mode", ctypes.c_int32), ("flags", ctypes.c_int32),
                 ("q_pos0", _i64), ("k_pos0", _i64), ("causal_offset", _i64),
                 ("K", _vp), ("Q", _vp), ("mask", _vp), ("V", _vp),
                 ("lse", _vp), ("A", _vp)]
@@ -41,7 +42,7 @@ class GridArgs(ctypes.Structure):
                 ("k_tile", _i64), ("head", _i64), ("batch", _i64),
                 ("n_batch", _i64), ("kv_group", _i64),
                 ("mask_mode", ctypes.c_int32), ("n_q_tiles", ctypes.c_int32),
-                ("n_kv_tiles", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("n_kv_tiles", ctypes.c_int32), ("flags", ctypes.c_int32),
                 ("q_pos0", _i64), ("k_pos0", _i64), ("causal_offset", _i64),
                 ("K", _vp * MAX_TILES), ("V", _vp * MAX_TILES),
                 ("Q", _vp * MAX_TILES), ("lse", _vp * MAX_TILES),
@@ -158,7 +159,7 @@ def flash_sdpa_fwd(K, Q, mask, lse, V, A, stream=None):
 
 
 def _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0,
-               k_pos0, causal_offset):
+               k_pos0, causal_offset, flags=0):
     batch, q_seq, head = Q.shape
     k_seq = K.shape[1]
     a = TileArgs()
@@ -166,6 +167,7 @@ def _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0,
     a.n_batch = batch if n_batch is None else n_batch
     a.kv_group = kv_group
     a.mask_mode = mask_mode
+    a.flags = flags
     a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
     a.K, a.Q, a.V = K.data_ptr(), Q.data_ptr(), V.data_ptr()
     a.mask = None if mask is None else mask.data_ptr()
@@ -174,17 +176,17 @@ def _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0,
 
 
 def sdpa_fwd_tile(K, Q, mask, lse, V, A, mask_mode, n_batch=None, kv_group=1,
-                  q_pos0=0, k_pos0=0, causal_offset=0, stream=None):
+                  q_pos0=0, k_pos0=0, causal_offset=0, flags=0, stream=None):
     _dev(K, Q, mask, lse, V, A)
     a = _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0,
-                   k_pos0, causal_offset)
+                   k_pos0, causal_offset, flags)
     fn = getattr(lib(), "nntile_hip_sdpa_fwd_tile_" + dtype_name(Q))
     _check(fn(_stream(stream), ctypes.byref(a)), "sdpa_fwd_tile")
 
 
 def sdpa_fwd_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq,
                   q_tile, k_tile, mask_mode, n_batch=None, kv_group=1,
-                  q_pos0=0, k_pos0=0, causal_offset=0, stream=None):
+                  q_pos0=0, k_pos0=0, causal_offset=0, flags=0, stream=None):
     """All key tiles merged into all query tiles in one launch.  Tiles are
     lists of separately allocated tensors [batch, rows, head]."""
     _dev(*K_tiles, *Q_tiles, *lse_tiles, *V_tiles, *A_tiles)
@@ -195,6 +197,7 @@ def sdpa_fwd_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq,
     a.n_batch = batch if n_batch is None else n_batch
     a.kv_group = kv_group
     a.mask_mode = mask_mode
+    a.flags = flags
     a.n_q_tiles, a.n_kv_tiles = len(Q_tiles), len(K_tiles)
     a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
     if len(Q_tiles) > MAX_TILES or len(K_tiles) > MAX_TILES:
@@ -214,13 +217,14 @@ def decode_workspace_bytes(K, Q, n_batch, kv_group):
 
 
 def sdpa_fwd_decode(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group,
-                    workspace, q_pos0=0, k_pos0=0, causal_offset=0, stream=None):
+                    workspace, q_pos0=0, k_pos0=0, causal_offset=0, flags=0,
+                    stream=None):
     """K, V: [n_head_kv*n_batch, k_seq, head]; Q, A:
     [n_head_kv*kv_group*n_batch, q_seq, head]; workspace: a device byte
     tensor of at least decode_workspace_bytes()."""
     _dev(K, Q, mask, lse, V, A, workspace)
     a = _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0,
-                   k_pos0, causal_offset)
+                   k_pos0, causal_offset, flags)
     fn = getattr(lib(), "nntile_hip_sdpa_fwd_decode_" + dtype_name(Q))
     nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _check(fn(_stream(stream), ctypes.byref(a), _ptr(workspace), nbytes),

@@ -252,3 +252,48 @@ def test_inputs_are_not_modified():
     torch.cuda.synchronize()
     for d, h in [(Kd, K), (Qd, Q), (Vd, V), (md, mask)]:
         assert torch.equal(d.cpu().view(torch.int16), h.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+def test_overwrite_flag_ignores_running_pair(oracle, dtype):
+    """OVERWRITE: lse and A hold garbage on entry, every row is written; rows
+    that see no key get lse = -inf and A = 0."""
+    q_seq, k_seq, head, batch, offset = 200, 150, 64, 2, -70
+    (Q, K, V), f32 = H.make_qkv(31, batch, q_seq, k_seq, head, dtype)
+    mask = synth.causal_mask(q_seq, k_seq, offset)
+    want, want_lse = _oracle(oracle, f32, mask)
+    hidden = ~mask.any(axis=1)
+    assert hidden.sum() >= 64          # a whole wavefront and more sees nothing
+    for entry in ("tile", "grid"):
+        lse = torch.full((batch, q_seq), 123.0, device="cuda")
+        A = torch.full((batch, q_seq, head), float("nan"), dtype=H.TORCH_DT[dtype], device="cuda")
+        if entry == "tile":
+            hip_sdpa.sdpa_fwd_tile(K.cuda(), Q.cuda(), None, lse, V.cuda(), A, hip_sdpa.MASK_CAUSAL,
+                                   causal_offset=offset, flags=hip_sdpa.OVERWRITE)
+        else:
+            hip_sdpa.sdpa_fwd_grid([K.cuda()], [Q.cuda()], [lse], [V.cuda()], [A], q_seq, k_seq,
+                                   q_seq, k_seq, hip_sdpa.MASK_CAUSAL, causal_offset=offset,
+                                   flags=hip_sdpa.OVERWRITE)
+        torch.cuda.synchronize()
+        assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+        assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+        assert np.all(H.to_np(A)[:, hidden] == 0)
+
+
+def test_overwrite_flag_decode(oracle):
+    dtype, q_seq, k_seq, n_batch, group, n_kv, head = "bf16", 16, 300, 2, 4, 2, 128
+    batch = n_batch * group * n_kv
+    (Q, K, V), f32 = H.make_qkv(37, batch, q_seq, k_seq, head, dtype, kv_batch=n_batch * n_kv)
+    offset = -8                         # tokens 0..7 see nothing
+    mask = synth.causal_mask(q_seq, k_seq, offset)
+    want, want_lse = _oracle(oracle, f32, mask, n_batch=n_batch, kv_repeat=group)
+    Kd, Qd, Vd = K.cuda(), Q.cuda(), V.cuda()
+    ws = torch.empty(hip_sdpa.decode_workspace_bytes(Kd, Qd, n_batch, group), dtype=torch.uint8,
+                     device="cuda")
+    lse = torch.full((batch, q_seq), 5.0, device="cuda")
+    A = torch.full((batch, q_seq, head), float("nan"), dtype=torch.bfloat16, device="cuda")
+    hip_sdpa.sdpa_fwd_decode(Kd, Qd, None, lse, Vd, A, hip_sdpa.MASK_CAUSAL, n_batch, group, ws,
+                             causal_offset=offset, flags=hip_sdpa.OVERWRITE)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < 1e-2
+    assert H.rel_fro(H.to_np(lse), want_lse) < 1e-2
