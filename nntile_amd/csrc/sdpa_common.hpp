@@ -6,6 +6,17 @@
 
 #include "../../include/nntile_hip_sdpa.h"
 
+// Developer hook: a diagnostic build may define these to record cycle counters
+// at the phase boundaries of a kernel's main loop; they expand to nothing in
+// the library.
+#ifndef NNTILE_PHASE
+#define NNTILE_PHASE(n)
+#define NNTILE_PHASE_DUMP()
+#endif
+#ifndef PHASE_DECL
+#define PHASE_DECL
+#endif
+
 namespace nntile_hip
 {
 

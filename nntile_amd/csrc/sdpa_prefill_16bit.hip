@@ -13,19 +13,24 @@
 //                  straight from the S^T accumulators (converted to 16 bit) -
 //                  the accumulator layout of the first product IS the B layout
 //                  of the second, up to a fixed permutation of the 16 keys,
-//                  and V^T is stored in LDS in that permuted key order.
+//                  and the V operand is gathered in that permuted key order.
 //
+// K and V steps go from global memory straight into LDS (global_load_lds,
+// 16 bytes per lane, no register round trip), double-buffered, one barrier per
+// step; the loads of step g+1 are issued at the top of step g.  A load
+// instruction fills 1 KB of LDS contiguously, so rows cannot be padded; bank
+// conflicts are avoided by XOR-swizzling the 16-byte chunks of a row instead
+// (each lane picks the global chunk that belongs at its LDS position).
 // V arrives with the head axis contiguous but the second product contracts
-// over keys, so V is transposed on its way into LDS: a thread fetches 4 keys x
-// 8 head values, regroups them in registers and writes 8 x (4 keys) so that
-// every MFMA operand is a single 16-byte LDS read.
+// over keys: its MFMA operand is read with ds_read_b64_tr_b16, which hands
+// each lane 4 keys of one head value from a 4 x 16 block.
 //
-// K and V steps are double-buffered in LDS (one barrier per step); the global
-// loads of step g+1 are in flight while step g is computed.  The running
-// (max, sum) pair lives in registers across all key tiles of a query tile;
-// the epilogue merges the result into the (lse, A) pair in memory (the
-// hand-off between NNTile tasks), so one launch can stand for one task or for
-// a whole row of tasks.
+// The running (max, sum) pair lives in registers across all key tiles of a
+// query tile; the epilogue merges the result into the (lse, A) pair in memory
+// (the hand-off between NNTile tasks), so one launch can stand for one task or
+// for a whole row of tasks.
+#include <type_traits>
+
 #include "sdpa_common.hpp"
 
 namespace nntile_hip
@@ -40,7 +45,19 @@ constexpr int kThreads = 256;
 struct StepCursor
 {
     int kt, kb, rows_left;
+    const char *Kp, *Vp;    // first row of the step in the current key tile
 };
+
+// ds_read_b64_tr_b16: within each block of 16 lanes, lane i supplies the
+// address of 4 consecutive 16-bit values of row i/4 (values 4*(i%4)..+3 of
+// 16) and receives value i of rows 0..3.
+__device__ __forceinline__ u32x2 lds_read_tr16(const char *lds_ptr)
+{
+    typedef __attribute__((ext_vector_type(4))) short s16x4;
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(lds_ptr));
+    return __builtin_bit_cast(u32x2, v);
+}
 
 template<typename T, int HEAD, int MODE>
 __global__ __launch_bounds__(kThreads, 2)
@@ -49,15 +66,19 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     typedef typename T::vec8 vec8;
     constexpr int KSTEPS = HEAD / 16;       // MFMA steps along head for S
     constexpr int DBLOCKS = HEAD / 32;      // 32-row blocks of O^T
-    constexpr int KPAD = HEAD + 8;          // K row stride in LDS (elements)
-    constexpr int VPAD = kKeys + 8;         // V^T row stride in LDS
-    constexpr int CHUNKS = HEAD / 8;        // 16-byte chunks per row
-    constexpr int K_ELEMS = kKeys * KPAD;
-    constexpr int BUF_ELEMS = K_ELEMS + HEAD * VPAD;
+    constexpr int RB = HEAD * 2;            // bytes per K/V row
+    constexpr int CPR = HEAD / 8;           // 16-byte chunks per row
+    constexpr int RPL = 16 / CPR;           // rows per 256-byte line of LDS banks
+    constexpr int ROWS_PER_LOAD = 1024 / RB;   // rows one load instruction fills
+    constexpr int LOADS = kKeys / ROWS_PER_LOAD;  // load instructions per K (or V) step
+    constexpr int LOADS_PER_WAVE = LOADS / 4;
+    constexpr int K_BYTES = kKeys * RB;
+    constexpr int BUF_BYTES = 2 * K_BYTES;  // K then V
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
+    static_assert(LOADS_PER_WAVE >= 1, "head size too small for this tiling");
 
-    __shared__ __attribute__((aligned(16))) uint16_t lds[2 * BUF_ELEMS];
+    __shared__ __attribute__((aligned(1024))) char lds[2 * BUF_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -151,127 +172,131 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     const int wave_rel_lo = rel0 + wave * 32;       // first query of the wavefront
     const int my_rel = wave_rel_lo + col;
 
-    // ---- cooperative load assignment ----------------------------------------
-    // K: 64 rows x CHUNKS chunks of 16 B, thread t takes chunk t % CHUNKS of
-    //    rows t / CHUNKS + i * (256 / CHUNKS).
-    constexpr int K_ROWS_PER_PASS = kThreads / CHUNKS;
-    constexpr int K_PASSES = kKeys / K_ROWS_PER_PASS;
-    const int k_chunk = tid % CHUNKS;
-    const int k_row = tid / CHUNKS;
-    // V: 16 groups of 4 keys x CHUNKS chunks; thread u takes key group
-    //    u % 16 and chunk u / 16 (lanes walk the key axis so that the
-    //    transposed 8-byte LDS writes of 16 lanes fill one 128-byte row).
-    constexpr int V_UNITS = 16 * CHUNKS;
-    const bool v_active = tid < V_UNITS;
-    const int v_kg = tid & 15;
-    const int v_chunk = tid >> 4;
-    // LDS position of keys 4*kg..4*kg+3: within each group of 16 keys the
-    // order is [h][a][c] for key = 8a + 4h + c, which is the order in which
-    // the S^T accumulators of lane half h list their keys.
-    const int v_pos = 16 * (v_kg >> 2) + 8 * (v_kg & 1) + 4 * ((v_kg & 3) >> 1);
-    // Byte offsets of this thread's loads within a full 64-row step.
-    const uint32_t k_goff = (uint32_t)(k_row * HEAD + k_chunk * 8) * 2u;
-    const uint32_t v_goff = (uint32_t)(4 * v_kg * HEAD + v_chunk * 8) * 2u;
-    // LDS element offsets of this thread's stores.
-    const int k_soff = k_row * KPAD + k_chunk * 8;
-    const int v_soff = K_ELEMS + (v_chunk * 8) * VPAD + v_pos;
-
-    u32x4 k_regs[K_PASSES];
-    u32x4 v_regs[4];
+    // ---- LDS layout and the lane's fixed addresses ---------------------------
+    // A step's K (and V) block is kKeys rows of RB bytes, unpadded.  The
+    // 16-byte chunk c of row r is stored at chunk position
+    //   K:  c ^ ((r / RPL) % CPR)        16 consecutive rows, same c -> 16 bank groups
+    //   V:  c ^ (4 * ((r / RPL) % (CPR/4)))   4 consecutive rows x 64 B -> 4 quarters
+    // Load instruction `ld` fills rows [ld*ROWS_PER_LOAD, +ROWS_PER_LOAD): lane
+    // L lands on row ld*ROWS_PER_LOAD + L/CPR, chunk position L%CPR, and so must
+    // fetch the logical chunk that belongs there.
+    uint32_t k_goff[LOADS_PER_WAVE], v_goff[LOADS_PER_WAVE];
+    int ld_row[LOADS_PER_WAVE];
+    const int ld_cpos = lane % CPR;
+#pragma unroll
+    for(int i = 0; i < LOADS_PER_WAVE; ++i)
+    {
+        const int ld = wave * LOADS_PER_WAVE + i;
+        const int r = ld * ROWS_PER_LOAD + lane / CPR;
+        ld_row[i] = r;
+        k_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ ((r / RPL) % CPR)) * 16);
+        v_goff[i] = (uint32_t)(r * RB
+                + (ld_cpos ^ (4 * ((r / RPL) % (CPR >= 4 ? CPR / 4 : 1)))) * 16);
+    }
+    // S operand: lane (col, half) reads row mb*32+col, logical chunk 2*ks+half.
+    uint32_t k_raddr[2][KSTEPS];
+#pragma unroll
+    for(int mb = 0; mb < 2; ++mb)
+    {
+        const int r = mb * 32 + col;
+#pragma unroll
+        for(int ks = 0; ks < KSTEPS; ++ks)
+        {
+            k_raddr[mb][ks] = (uint32_t)(r * RB
+                    + ((2 * ks + half) ^ ((r / RPL) % CPR)) * 16);
+        }
+    }
+    // PV operand through the transposing read: within a 16-lane block, lane i
+    // addresses key j = i/4 and head values 4*(i%4)..+3 of the block's 16 head
+    // values, and receives keys 0..3 of head value i.  Blocks: lanes 16..31
+    // take the upper 16 head values of a 32-row block, lanes 32..63 the keys
+    // 4..7 (lane half h).  For step t (16 keys) and instruction a (keys
+    // 8a + 4h + j) the row is 16t + 8a + 4h + j; 16t + 8a goes into the
+    // instruction's immediate offset.
+    uint32_t v_raddr[DBLOCKS];
+    {
+        const int i16 = lane & 15, dblk = (lane >> 4) & 1;
+        const int j = i16 >> 2, r4 = i16 & 3;
+        const int r = 4 * half + j;         // row modulo 8: enough for the swizzle
+        const int swz = 4 * ((r / RPL) % (CPR >= 4 ? CPR / 4 : 1));
+#pragma unroll
+        for(int db = 0; db < DBLOCKS; ++db)
+        {
+            const int c = 4 * db + 2 * dblk + (r4 >> 1);
+            v_raddr[db] = (uint32_t)(K_BYTES + r * RB + (c ^ swz) * 16
+                    + 8 * (r4 & 1));
+        }
+    }
 
     auto tile_rows = [&](int kt) -> int
     {
         return min(k_tile, k_seq - kt * k_tile);
     };
 
-    // Global loads of one step into registers.  Rows past the end of the tile
-    // are clamped to its last row: their scores are masked and their
-    // probabilities are exactly 0, so any finite stand-in value works.
-    auto fetch = [&](const StepCursor &cur)
+    // Byte offset of batch entry kvb's slab inside key tile kt.
+    auto slab = [&](int kt) -> int64_t
     {
-        const int k_len = tile_rows(cur.kt);
-        const int64_t base = ((int64_t)kvb * k_len + (int64_t)cur.kb * kKeys)
-            * HEAD * 2;
-        const char *Kp = static_cast<const char *>(p.K[cur.kt]) + base;
-        const char *Vp = static_cast<const char *>(p.V[cur.kt]) + base;
+        return (int64_t)kvb * tile_rows(kt) * HEAD * 2;
+    };
+
+    // Global -> LDS loads of one step into buffer `buf`.  Rows past the end of
+    // the tile are clamped to its last row: their scores are masked and their
+    // probabilities are exactly 0, so any finite stand-in value works.
+    auto fetch = [&](const StepCursor &cur, int buf)
+    {
+        char *kdst = lds + buf * BUF_BYTES + wave * LOADS_PER_WAVE * 1024;
+        char *vdst = kdst + K_BYTES;
+        typedef const void __attribute__((address_space(1))) *gptr;
+        typedef void __attribute__((address_space(3))) *lptr;
         if(cur.rows_left >= kKeys)
         {
 #pragma unroll
-            for(int i = 0; i < K_PASSES; ++i)
+            for(int i = 0; i < LOADS_PER_WAVE; ++i)
             {
-                k_regs[i] = *reinterpret_cast<const u32x4 *>(Kp + k_goff
-                        + (uint32_t)(i * K_ROWS_PER_PASS * HEAD * 2));
-            }
-            if(v_active)
-            {
-#pragma unroll
-                for(int j = 0; j < 4; ++j)
-                {
-                    v_regs[j] = *reinterpret_cast<const u32x4 *>(Vp + v_goff
-                            + (uint32_t)(j * HEAD * 2));
-                }
+                __builtin_amdgcn_global_load_lds((gptr)(cur.Kp + k_goff[i]),
+                        (lptr)(kdst + i * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr)(cur.Vp + v_goff[i]),
+                        (lptr)(vdst + i * 1024), 16, 0, 0);
             }
         }
         else
         {
             const int last = cur.rows_left - 1;
 #pragma unroll
-            for(int i = 0; i < K_PASSES; ++i)
+            for(int i = 0; i < LOADS_PER_WAVE; ++i)
             {
-                const int r = min(k_row + i * K_ROWS_PER_PASS, last);
-                k_regs[i] = *reinterpret_cast<const u32x4 *>(Kp
-                        + (uint32_t)(r * HEAD + k_chunk * 8) * 2u);
-            }
-            if(v_active)
-            {
-#pragma unroll
-                for(int j = 0; j < 4; ++j)
-                {
-                    const int r = min(4 * v_kg + j, last);
-                    v_regs[j] = *reinterpret_cast<const u32x4 *>(Vp
-                            + (uint32_t)(r * HEAD + v_chunk * 8) * 2u);
-                }
+                // same chunk, clamped row
+                const uint32_t back = (uint32_t)(max(ld_row[i] - last, 0) * RB);
+                __builtin_amdgcn_global_load_lds(
+                        (gptr)(cur.Kp + (k_goff[i] - back)),
+                        (lptr)(kdst + i * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(
+                        (gptr)(cur.Vp + (v_goff[i] - back)),
+                        (lptr)(vdst + i * 1024), 16, 0, 0);
             }
         }
     };
 
+    // Next step; the tile base pointers are re-read only when the tile changes.
     auto advance = [&](StepCursor &cur)
     {
         cur.kb += 1;
         cur.rows_left -= kKeys;
+        cur.Kp += kKeys * RB;
+        cur.Vp += kKeys * RB;
         if(cur.rows_left <= 0)
         {
             cur.kt += 1;
             cur.kb = 0;
-            cur.rows_left = (cur.kt < p.n_kv_tiles) ? tile_rows(cur.kt) : 0;
-        }
-    };
-
-    // Registers -> LDS buffer `buf`: K as is, V regrouped to [head][key].
-    auto stage = [&](int buf)
-    {
-        uint16_t *base = lds + buf * BUF_ELEMS;
-#pragma unroll
-        for(int i = 0; i < K_PASSES; ++i)
-        {
-            *reinterpret_cast<u32x4 *>(base + k_soff
-                    + i * K_ROWS_PER_PASS * KPAD) = k_regs[i];
-        }
-        if(v_active)
-        {
-#pragma unroll
-            for(int w = 0; w < 4; ++w)
+            if(cur.kt < p.n_kv_tiles)
             {
-                // word w of each row holds head values 2w (low) and 2w+1 (high)
-                const uint32_t r0 = v_regs[0][w], r1 = v_regs[1][w],
-                      r2 = v_regs[2][w], r3 = v_regs[3][w];
-                u32x2 even, odd;
-                even[0] = __builtin_amdgcn_perm(r1, r0, 0x05040100u);
-                even[1] = __builtin_amdgcn_perm(r3, r2, 0x05040100u);
-                odd[0] = __builtin_amdgcn_perm(r1, r0, 0x07060302u);
-                odd[1] = __builtin_amdgcn_perm(r3, r2, 0x07060302u);
-                *reinterpret_cast<u32x2 *>(base + v_soff + (2 * w) * VPAD) = even;
-                *reinterpret_cast<u32x2 *>(base + v_soff + (2 * w + 1) * VPAD) = odd;
+                cur.rows_left = tile_rows(cur.kt);
+                cur.Kp = static_cast<const char *>(p.K[cur.kt]) + slab(cur.kt);
+                cur.Vp = static_cast<const char *>(p.V[cur.kt]) + slab(cur.kt);
+            }
+            else
+            {
+                cur.rows_left = 0;
             }
         }
     };
@@ -294,32 +319,41 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     float m_run = neg_inf();
     float l_run = 0.0f;      // this lane half's share of the row sum
 
-    StepCursor cur = {0, 0, tile_rows(0)};      // step being computed
+    PHASE_DECL
+    StepCursor cur = {0, 0, tile_rows(0),
+        static_cast<const char *>(p.K[0]) + slab(0),
+        static_cast<const char *>(p.V[0]) + slab(0)};     // step being computed
     StepCursor nxt = cur;                        // step being fetched
     if(n_steps > 0)
     {
-        fetch(nxt);
+        fetch(nxt, 0);
         advance(nxt);
-        stage(0);
-        if(n_steps > 1)
-        {
-            fetch(nxt);
-            advance(nxt);
-        }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    for(int g = 0; g < n_steps; ++g)
+    // One key step on LDS buffer BUF (a compile-time constant, so that every
+    // LDS address is a fixed register plus an immediate).
+    auto step = [&](int g, auto buf_tag)
     {
-        const int buf = g & 1;
-        const uint16_t *Ks = lds + buf * BUF_ELEMS;
-        const uint16_t *Vt = Ks + K_ELEMS;
+        constexpr int BUF = decltype(buf_tag)::value;
+        const char *Ks = lds + BUF * BUF_BYTES;
         const int k_row0 = cur.kb * kKeys;                   // within the tile
         const int kg0 = cur.kt * k_tile + k_row0;            // key row overall
         const int keys_here = min(kKeys, cur.rows_left);
         // nothing of this step is visible to this wavefront
         const bool idle = (MODE == NNTILE_HIP_MASK_CAUSAL)
             && (kg0 > wave_rel_lo + 31);
+
+        // ---- loads of the next step into the other buffer ----------------------
+        // (every wavefront passed the barrier that ended step g-1, so nobody
+        // still reads that buffer)
+        NNTILE_PHASE(0)
+        if(g + 1 < n_steps)
+        {
+            fetch(nxt, BUF ^ 1);
+            advance(nxt);
+        }
 
         uint32_t pk[2][8];
         if(!idle)
@@ -338,10 +372,11 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 for(int ks = 0; ks < KSTEPS; ++ks)
                 {
                     const vec8 a = *reinterpret_cast<const vec8 *>(
-                            &Ks[(mb * 32 + col) * KPAD + ks * 16 + half * 8]);
+                            Ks + k_raddr[mb][ks]);
                     s[mb] = T::mfma(a, qf[ks], s[mb]);
                 }
             }
+            NNTILE_PHASE(1)
 
             // ---- mask ---------------------------------------------------------
             // register r of block mb holds key  mb*32 + 8*(r/4) + 4*half + r%4
@@ -469,19 +504,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             }
             l_run += rs;
         }
-
-        // ---- next step: registers -> the other LDS buffer, then new loads -----
-        // (every wavefront passed the barrier that ended step g-1, so nobody
-        // still reads that buffer)
-        if(g + 1 < n_steps)
-        {
-            stage(buf ^ 1);
-            if(g + 2 < n_steps)
-            {
-                fetch(nxt);
-                advance(nxt);
-            }
-        }
+        NNTILE_PHASE(2)
 
         // ---- O^T += V^T P^T ------------------------------------------------------
         if(!idle)
@@ -496,15 +519,32 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
 #pragma unroll
                 for(int db = 0; db < DBLOCKS; ++db)
                 {
-                    const vec8 a = *reinterpret_cast<const vec8 *>(
-                            &Vt[(db * 32 + col) * VPAD + 16 * t + 8 * half]);
+                    const char *src = Ks + v_raddr[db] + (16 * t) * RB;
+                    const u32x2 lo = lds_read_tr16(src);
+                    const u32x2 hi = lds_read_tr16(src + 8 * RB);
+                    const u32x4 araw = {lo[0], lo[1], hi[0], hi[1]};
+                    const vec8 a = __builtin_bit_cast(vec8, araw);
                     o[db] = T::mfma(a, pb, o[db]);
                 }
             }
         }
         advance(cur);
+        NNTILE_PHASE(3)
+        // this wavefront's loads of the next step have landed in LDS
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+        NNTILE_PHASE(4)
+    };
+
+    for(int g = 0; g < n_steps; g += 2)
+    {
+        step(g, std::integral_constant<int, 0>{});
+        if(g + 1 < n_steps)
+        {
+            step(g + 1, std::integral_constant<int, 1>{});
+        }
     }
+    NNTILE_PHASE_DUMP()
 
     // ---- epilogue: normalise, merge into the running (lse, A) ----------------
     const float l_tot = l_run + __shfl_xor(l_run, 32);
