@@ -109,6 +109,14 @@ struct Bf16
     {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
+    // acc + lo + hi of a packed pair, in fp32
+    static __device__ __forceinline__ float add_pair(uint32_t packed, float acc)
+    {
+        typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+        const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+        return __builtin_amdgcn_fdot2_f32_bf16(
+                __builtin_bit_cast(bf16x2, packed), ones, acc, false);
+    }
 };
 
 struct Fp16
@@ -135,7 +143,32 @@ struct Fp16
     {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
+    static __device__ __forceinline__ float add_pair(uint32_t packed, float acc)
+    {
+        typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+        const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, packed), ones,
+                acc, false);
+    }
 };
+
+// max(x, value of x in lane ^ 32): v_permlane32_swap exchanges the upper half
+// of one register with the lower half of another without going through LDS.
+__device__ __forceinline__ float max_across_halves(float x)
+{
+    typedef __attribute__((ext_vector_type(2))) uint32_t pair;
+    const uint32_t u = __float_as_uint(x);
+    const pair r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+__device__ __forceinline__ float sum_across_halves(float x)
+{
+    typedef __attribute__((ext_vector_type(2))) uint32_t pair;
+    const uint32_t u = __float_as_uint(x);
+    const pair r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
 // Key/value batch entry read by query batch entry b.
 __device__ __forceinline__ int kv_entry(int b, int n_batch, int kv_group)

@@ -244,7 +244,9 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // probabilities are exactly 0, so any finite stand-in value works.
     auto fetch = [&](const StepCursor &cur, int buf)
     {
-        char *kdst = lds + buf * BUF_BYTES + wave * LOADS_PER_WAVE * 1024;
+        // (wave index made visibly uniform: the LDS target goes into M0)
+        char *kdst = lds + buf * BUF_BYTES
+            + __builtin_amdgcn_readfirstlane(wave) * LOADS_PER_WAVE * 1024;
         char *vdst = kdst + K_BYTES;
         typedef const void __attribute__((address_space(1))) *gptr;
         typedef void __attribute__((address_space(3))) *lptr;
@@ -466,7 +468,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                     mx = fmaxf(mx, s[mb][r]);
                 }
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            mx = max_across_halves(mx);
             const float m_new = fmaxf(m_run, mx);
             const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
             const float mc = m_use * c;
@@ -498,8 +500,10 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 {
                     const float p0 = fast_exp2(fmaf(s[mb][r], c, -mc));
                     const float p1 = fast_exp2(fmaf(s[mb][r + 1], c, -mc));
-                    rs += p0 + p1;
                     pk[mb][r >> 1] = T::pack2(p0, p1);
+                    // the row sum runs over the ROUNDED probabilities, the
+                    // values the second product actually uses
+                    rs = T::add_pair(pk[mb][r >> 1], rs);
                 }
             }
             l_run += rs;
@@ -547,7 +551,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     NNTILE_PHASE_DUMP()
 
     // ---- epilogue: normalise, merge into the running (lse, A) ----------------
-    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float l_tot = sum_across_halves(l_run);
     const bool empty = !(l_tot > 0.0f);     // no visible key for this query
     if(!q_ok || (empty && !p.overwrite))
     {
