@@ -9,19 +9,29 @@
 //    workgroups so that every CU streams; each workgroup writes an
 //    un-normalised partial (max, sum, O) and a second small kernel merges the
 //    partials and folds them into the running (lse, A) pair;
-//  * global loads are 16 bytes per lane over contiguous rows, staged through
-//    LDS; a wavefront owns 16 rows and uses v_mfma_f32_16x16x32 (S^T = K Q^T,
-//    O^T += V^T P^T with P^T taken from the S^T accumulators; V is transposed
-//    on its way into LDS, keys stored in the order the accumulators list them).
+//  * K and V steps go from global memory straight into LDS (global_load_lds,
+//    16 bytes per lane, 1 KB contiguous per instruction, no registers in
+//    between) through a ring of STAGES buffers, so that STAGES-1 steps of 32 KB
+//    are in flight per workgroup while one is consumed;
+//  * a wavefront owns 16 rows and uses v_mfma_f32_16x16x32 (S^T = K Q^T,
+//    O^T += V^T P^T with P^T taken from the S^T accumulators); LDS rows are
+//    unpadded and XOR-swizzled by 16-byte chunks against bank conflicts, and
+//    the V operand is gathered with the transposing ds_read_b64_tr_b16.
+#include <type_traits>
+
 #include "sdpa_common.hpp"
 
 namespace nntile_hip
 {
 
+// Cache policy of the K/V stream: non-temporal (each byte is used once).
+#ifndef NNTILE_DMA_AUX
+#define NNTILE_DMA_AUX 2
+#endif
 
 constexpr int kDecKeys = 64;      // keys per step
-constexpr int kDecThreads = 256;
-
+constexpr int kDecThreads = 256;  // 4 wavefronts x 16 query rows
+constexpr int kDecodeCUs = 256;   // MI355X
 
 typedef __attribute__((ext_vector_type(4))) float acc4;
 
@@ -41,21 +51,58 @@ template<> struct Mfma16<Fp16>
     }
 };
 
-template<typename T, int HEAD, int MODE>
-__global__ __launch_bounds__(kDecThreads, 3)
+__device__ __forceinline__ u32x2 dec_lds_read_tr16(const char *lds_ptr)
+{
+    typedef __attribute__((ext_vector_type(4))) short s16x4;
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(lds_ptr));
+    return __builtin_bit_cast(u32x2, v);
+}
+
+template<int N> __device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    // s_waitcnt simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14]
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+    asm volatile("" ::: "memory");
+}
+
+template<typename T, int HEAD, int MODE, int STAGES>
+__global__ __launch_bounds__(kDecThreads, 2)
 void sdpa_decode_16bit_kernel(const DecodeParams p)
 {
     typedef typename T::vec8 vec8;
     constexpr int KSTEPS = HEAD / 32;       // MFMA steps along head for S
     constexpr int DBLOCKS = HEAD / 16;      // 16-row blocks of O^T
-    constexpr int KPAD = HEAD + 8;
-    constexpr int VPAD = kDecKeys + 8;
-    constexpr int CHUNKS = HEAD / 8;
+    constexpr int RB = HEAD * 2;            // bytes per K/V row
+    constexpr int CPR = HEAD / 8;           // 16-byte chunks per row
+    constexpr int RPL = 16 / CPR;           // rows per 256-byte line of LDS banks
+    constexpr int ROWS_PER_LOAD = 1024 / RB;
+    constexpr int LOADS = kDecKeys / ROWS_PER_LOAD;     // per K (or V) step
+    constexpr int LOADS_PER_WAVE = LOADS / 4;
+    constexpr int K_BYTES = kDecKeys * RB;
+    constexpr int STAGE_BYTES = 2 * K_BYTES;            // K then V
+    constexpr int VM_PER_STEP = 2 * LOADS_PER_WAVE;     // load instructions a wave issues per step
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
+    static_assert(LOADS_PER_WAVE >= 1, "head size too small for this tiling");
 
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[kDecKeys * KPAD];
-    __shared__ __attribute__((aligned(16))) uint16_t Vt[HEAD * VPAD];
+    // One array per ring slot, not one array for all: the compiler then knows
+    // that loads streaming into one slot cannot alias the reads of another and
+    // does not make those reads wait for the loads.  (Unused slots of a
+    // shallower ring are dropped.)
+    __shared__ __attribute__((aligned(1024))) char ring0[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring1[STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char ring2[STAGES > 2 ? STAGE_BYTES : 16];
+    __shared__ __attribute__((aligned(1024))) char ring3[STAGES > 3 ? STAGE_BYTES : 16];
+    auto ring = [&](auto tag) -> char *
+    {
+        constexpr int I = decltype(tag)::value % STAGES;
+        if constexpr(I == 0) { return ring0; }
+        else if constexpr(I == 1) { return ring1; }
+        else if constexpr(I == 2) { return ring2; }
+        else { return ring3; }
+    };
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -91,76 +138,89 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         }
     }
 
-    const uint16_t *Kb = static_cast<const uint16_t *>(p.K)
-        + (int64_t)unit * p.k_seq * HEAD;
-    const uint16_t *Vb = static_cast<const uint16_t *>(p.V)
-        + (int64_t)unit * p.k_seq * HEAD;
+    const char *Kb = static_cast<const char *>(p.K) + (int64_t)unit * p.k_seq * RB;
+    const char *Vb = static_cast<const char *>(p.V) + (int64_t)unit * p.k_seq * RB;
 
-    // Cooperative loads (see the prefill kernel): K plain, V regrouped.
-    constexpr int K_ROWS_PER_PASS = kDecThreads / CHUNKS;
-    constexpr int K_PASSES = kDecKeys / K_ROWS_PER_PASS;
-    const int k_chunk = tid % CHUNKS;
-    const int k_row = tid / CHUNKS;
-    constexpr int V_UNITS = 16 * CHUNKS;
-    const bool v_active = tid < V_UNITS;
-    const int v_kg = tid & 15;
-    const int v_chunk = tid >> 4;
-    // LDS position of keys 4*kg..4*kg+3: within each group of 32 keys the
-    // order is [quad][a][c] for key = 16a + 4*quad + c.
-    const int v_pos = 32 * (v_kg >> 3) + 8 * (v_kg & 3) + 4 * ((v_kg & 7) >> 2);
+    // ---- LDS layout and the lane's fixed addresses ---------------------------
+    // chunk c of row r sits at chunk position
+    //   K:  c ^ ((r / RPL) % CPR)          16 consecutive rows, same c -> 16 bank groups
+    //   V:  c ^ (2 * ((r / RPL) % (CPR/2)))  8 consecutive rows x 32 B -> 8 bank groups
+    // Load instruction `ld` fills rows [ld*ROWS_PER_LOAD, +ROWS_PER_LOAD): lane L
+    // lands on row ld*ROWS_PER_LOAD + L/CPR, chunk position L % CPR.
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    uint32_t k_goff[LOADS_PER_WAVE], v_goff[LOADS_PER_WAVE];
+    int ld_row[LOADS_PER_WAVE];
+    const int ld_cpos = lane % CPR;
+#pragma unroll
+    for(int i = 0; i < LOADS_PER_WAVE; ++i)
+    {
+        const int r = (wave * LOADS_PER_WAVE + i) * ROWS_PER_LOAD + lane / CPR;
+        ld_row[i] = r;
+        k_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ ((r / RPL) % CPR)) * 16);
+        v_goff[i] = (uint32_t)(r * RB
+                + (ld_cpos ^ (2 * ((r / RPL) % (CPR / 2)))) * 16);
+    }
+    // S operand: lane (col, quad) reads row 16*kb + col, logical chunk 4*ks + quad;
+    // 16*kb goes into the immediate offset.
+    uint32_t k_raddr[KSTEPS];
+#pragma unroll
+    for(int ks = 0; ks < KSTEPS; ++ks)
+    {
+        k_raddr[ks] = (uint32_t)(col * RB + ((4 * ks + quad) ^ ((col / RPL) % CPR)) * 16);
+    }
+    // PV operand through the transposing read: a 16-lane block is one quad;
+    // lane i addresses key j = i/4 and head values 4*(i%4)..+3 of the block's
+    // 16 head values and receives keys 0..3 of head value i.  For the 32-key
+    // step t and instruction a the row is 32t + 16a + 4*quad + j; 32t + 16a goes
+    // into the immediate offset.
+    uint32_t v_raddr[DBLOCKS];
+    {
+        const int j = col >> 2, r4 = col & 3;
+        const int r = 4 * quad + j;
+        const int swz = 2 * ((r / RPL) % (CPR / 2));
+#pragma unroll
+        for(int db = 0; db < DBLOCKS; ++db)
+        {
+            const int c = 2 * db + (r4 >> 1);
+            v_raddr[db] = (uint32_t)(K_BYTES + r * RB + (c ^ swz) * 16 + 8 * (r4 & 1));
+        }
+    }
 
-    u32x4 k_regs[K_PASSES];
-    u32x4 v_regs[4];
+    typedef const void __attribute__((address_space(1))) *gptr;
+    typedef void __attribute__((address_space(3))) *lptr;
 
-    auto fetch = [&](int step)
+    // Loads of key step `step` into ring slot `slot`; rows past the end of the
+    // cache are clamped to its last row (their probabilities are exactly 0).
+    auto fetch = [&](int step, char *slot_base)
     {
         const int64_t row0 = (int64_t)step * kDecKeys;
-#pragma unroll
-        for(int i = 0; i < K_PASSES; ++i)
-        {
-            const int64_t r = row0 + k_row + i * K_ROWS_PER_PASS;
-            k_regs[i] = (r < p.k_seq)
-                ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(
-                            Kb + r * HEAD + k_chunk * 8))
-                : u32x4{0, 0, 0, 0};
-        }
-        if(v_active)
+        const char *Kp = Kb + row0 * RB;
+        const char *Vp = Vb + row0 * RB;
+        char *kdst = slot_base + wave_u * LOADS_PER_WAVE * 1024;
+        char *vdst = kdst + K_BYTES;
+        const int rows_left = (int)min((int64_t)kDecKeys, p.k_seq - row0);
+        if(rows_left >= kDecKeys)
         {
 #pragma unroll
-            for(int j = 0; j < 4; ++j)
+            for(int i = 0; i < LOADS_PER_WAVE; ++i)
             {
-                const int64_t r = row0 + 4 * v_kg + j;
-                v_regs[j] = (r < p.k_seq)
-                    ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(
-                                Vb + r * HEAD + v_chunk * 8))
-                    : u32x4{0, 0, 0, 0};
+                __builtin_amdgcn_global_load_lds((gptr)(Kp + k_goff[i]),
+                        (lptr)(kdst + i * 1024), 16, 0, NNTILE_DMA_AUX);
+                __builtin_amdgcn_global_load_lds((gptr)(Vp + v_goff[i]),
+                        (lptr)(vdst + i * 1024), 16, 0, NNTILE_DMA_AUX);
             }
         }
-    };
-
-    auto stage = [&]()
-    {
-#pragma unroll
-        for(int i = 0; i < K_PASSES; ++i)
+        else
         {
-            *reinterpret_cast<u32x4 *>(&Ks[(k_row + i * K_ROWS_PER_PASS) * KPAD
-                    + k_chunk * 8]) = k_regs[i];
-        }
-        if(v_active)
-        {
+            const int last = rows_left - 1;
 #pragma unroll
-            for(int w = 0; w < 4; ++w)
+            for(int i = 0; i < LOADS_PER_WAVE; ++i)
             {
-                const uint32_t r0 = v_regs[0][w], r1 = v_regs[1][w],
-                      r2 = v_regs[2][w], r3 = v_regs[3][w];
-                u32x2 even, odd;
-                even[0] = __builtin_amdgcn_perm(r1, r0, 0x05040100u);
-                even[1] = __builtin_amdgcn_perm(r3, r2, 0x05040100u);
-                odd[0] = __builtin_amdgcn_perm(r1, r0, 0x07060302u);
-                odd[1] = __builtin_amdgcn_perm(r3, r2, 0x07060302u);
-                const int d = v_chunk * 8 + 2 * w;
-                *reinterpret_cast<u32x2 *>(&Vt[d * VPAD + v_pos]) = even;
-                *reinterpret_cast<u32x2 *>(&Vt[(d + 1) * VPAD + v_pos]) = odd;
+                const uint32_t back = (uint32_t)(max(ld_row[i] - last, 0) * RB);
+                __builtin_amdgcn_global_load_lds((gptr)(Kp + (k_goff[i] - back)),
+                        (lptr)(kdst + i * 1024), 16, 0, NNTILE_DMA_AUX);
+                __builtin_amdgcn_global_load_lds((gptr)(Vp + (v_goff[i] - back)),
+                        (lptr)(vdst + i * 1024), 16, 0, NNTILE_DMA_AUX);
             }
         }
     };
@@ -178,19 +238,57 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
     float m_run = neg_inf();
     float l_run = 0.0f;
 
-    if(step_lo < step_hi)
+    // The workgroups of a launch advance through their key ranges at the same
+    // pace and the ranges start a power-of-two number of bytes apart, which
+    // would keep all of them on the same few memory channels at any moment.
+    // Each workgroup therefore starts at its own rotation of its range (the
+    // online softmax does not care about the order of the steps).
+    const int n_local = step_hi - step_lo;
+    const int rot = n_local > 0 ? (int)((blockIdx.x * 7u + (blockIdx.x >> 3)) % (unsigned)n_local) : 0;
+    auto actual = [&](int i) -> int
     {
-        fetch(step_lo);
-    }
-    for(int step = step_lo; step < step_hi; ++step)
+        const int j = i + rot;
+        return step_lo + (j >= n_local ? j - n_local : j);
+    };
+
+    // prologue: STAGES-1 steps in flight
+    if(0 < n_local) { fetch(actual(0), ring(std::integral_constant<int, 0>{})); }
+    if(STAGES > 2 && 1 < n_local) { fetch(actual(1), ring(std::integral_constant<int, 1>{})); }
+    if(STAGES > 3 && 2 < n_local) { fetch(actual(2), ring(std::integral_constant<int, 2>{})); }
+
+    // One key step on ring slot SLOT (a compile-time constant).
+    auto body = [&](int it, auto slot_tag)
     {
-        __syncthreads();
-        stage();
-        __syncthreads();
-        if(step + 1 < step_hi)
+        constexpr int SLOT = decltype(slot_tag)::value;
+        const int step = actual(it);
+        // this step's data has landed: everything but the loads of the later
+        // steps in flight is complete (in the tail fewer steps are in flight)
+        if(it + STAGES - 1 <= n_local)
         {
-            fetch(step + 1);
+            wait_vmcnt<(STAGES - 2) * VM_PER_STEP>();
         }
+        else
+        {
+            wait_vmcnt<0>();
+        }
+        // ... for every wavefront, and everyone is done with the previous step.
+        // A bare barrier: __syncthreads() would also drain the loads of the
+        // later steps (its release fence waits for every outstanding store,
+        // and a global->LDS load counts as one), which is exactly what the
+        // ring is there to avoid.  LDS reads are ordered by lgkmcnt, the
+        // loads by the explicit vmcnt above.
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        {
+            const int ahead = it + STAGES - 1;
+            if(ahead < n_local)
+            {
+                // into the slot the previous step used
+                fetch(actual(ahead),
+                        ring(std::integral_constant<int, SLOT + STAGES - 1>{}));
+            }
+        }
+        const char *Ks = ring(slot_tag);
+
         const int64_t k_row0 = (int64_t)step * kDecKeys;
         const int64_t k_pos_base = p.k_pos0 + k_row0;
         const int keys_here = (int)min((int64_t)kDecKeys, p.k_seq - k_row0);
@@ -205,7 +303,7 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
             for(int ks = 0; ks < KSTEPS; ++ks)
             {
                 const vec8 a = *reinterpret_cast<const vec8 *>(
-                        &Ks[(kb * 16 + col) * KPAD + ks * 32 + quad * 8]);
+                        Ks + k_raddr[ks] + kb * 16 * RB);
                 s[kb] = Mfma16<T>::run(a, qf[ks], s[kb]);
             }
         }
@@ -279,12 +377,21 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
             }
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        mx = max_across_halves(mx);
         const float m_new = fmaxf(m_run, mx);
         const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
-        const float alpha = fast_exp2((m_run - m_use) * c);
         const float mc = m_use * c;
-        m_run = m_new;
+        if(__builtin_amdgcn_ballot_w64(m_new != m_run) != 0)
+        {
+            const float alpha = fast_exp2((m_run - m_use) * c);
+            l_run *= alpha;
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+                o[db] *= alpha;
+            }
+            m_run = m_new;
+        }
         float rs = 0.0f;
         uint32_t pk[4][2];
 #pragma unroll
@@ -294,16 +401,12 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
             const float p1 = fast_exp2(fmaf(s[kb][1], c, -mc));
             const float p2 = fast_exp2(fmaf(s[kb][2], c, -mc));
             const float p3 = fast_exp2(fmaf(s[kb][3], c, -mc));
-            rs += (p0 + p1) + (p2 + p3);
             pk[kb][0] = T::pack2(p0, p1);
             pk[kb][1] = T::pack2(p2, p3);
+            rs = T::add_pair(pk[kb][0], rs);
+            rs = T::add_pair(pk[kb][1], rs);
         }
-        l_run = l_run * alpha + rs;
-#pragma unroll
-        for(int db = 0; db < DBLOCKS; ++db)
-        {
-            o[db] *= alpha;
-        }
+        l_run += rs;
 
         // ---- O^T += V^T P^T: 2 steps of 32 keys ----------------------------------
 #pragma unroll
@@ -312,19 +415,36 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
             const u32x4 praw = {pk[2 * t][0], pk[2 * t][1], pk[2 * t + 1][0],
                 pk[2 * t + 1][1]};
             const vec8 pb = __builtin_bit_cast(vec8, praw);
+            // all operand reads of this 32-key step first, then the MFMAs, so
+            // that the LDS latency is paid once and not once per MFMA
+            u32x4 araw[DBLOCKS];
 #pragma unroll
             for(int db = 0; db < DBLOCKS; ++db)
             {
-                const vec8 a = *reinterpret_cast<const vec8 *>(
-                        &Vt[(db * 16 + col) * VPAD + 32 * t + 8 * quad]);
-                o[db] = Mfma16<T>::run(a, pb, o[db]);
+                const char *src = Ks + v_raddr[db] + (32 * t) * RB;
+                const u32x2 lo = dec_lds_read_tr16(src);
+                const u32x2 hi = dec_lds_read_tr16(src + 16 * RB);
+                araw[db] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+                o[db] = Mfma16<T>::run(__builtin_bit_cast(vec8, araw[db]), pb, o[db]);
             }
         }
+    };
+
+    for(int it = 0; it < n_local; it += STAGES)
+    {
+        body(it, std::integral_constant<int, 0>{});
+        if(it + 1 < n_local) { body(it + 1, std::integral_constant<int, 1>{}); }
+        if(STAGES > 2 && it + 2 < n_local) { body(it + 2, std::integral_constant<int, 2>{}); }
+        if(STAGES > 3 && it + 3 < n_local) { body(it + 3, std::integral_constant<int, 3>{}); }
     }
 
     // ---- write the partial ---------------------------------------------------------
     float l_tot = l_run + __shfl_xor(l_run, 16);
-    l_tot += __shfl_xor(l_tot, 32);
+    l_tot = sum_across_halves(l_tot);
     if(!row_ok)
     {
         return;
@@ -347,18 +467,27 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
 }
 
 // Merge the split partials of each row and fold the result into (lse, A).
-// One workgroup of HEAD threads per (unit, row).
+// A thread handles 4 head values of one row; a workgroup of 256 threads
+// handles 1024/HEAD rows.
 template<typename T, int HEAD>
-__global__ __launch_bounds__(HEAD)
+__global__ __launch_bounds__(256)
 void sdpa_decode_reduce_kernel(const DecodeParams p)
 {
-    const int rr = blockIdx.x % p.rows;
-    const int unit = blockIdx.x / p.rows;
+    constexpr int TPR = HEAD / 4;               // threads per row
+    constexpr int ROWS_PER_WG = 256 / TPR;
+    const int64_t total_rows = (int64_t)p.n_batch * p.n_head_kv * p.rows;
+    const int64_t grow = (int64_t)blockIdx.x * ROWS_PER_WG + threadIdx.x / TPR;
+    if(grow >= total_rows)
+    {
+        return;
+    }
+    const int d4 = (threadIdx.x % TPR) * 4;
+    const int rr = (int)(grow % p.rows);
+    const int unit = (int)(grow / p.rows);
     const int nb = unit % p.n_batch;
     const int hkv = unit / p.n_batch;
     const int g = rr / (int)p.q_seq, tok = rr % (int)p.q_seq;
     const int64_t qb = nb + (int64_t)p.n_batch * (g + (int64_t)p.kv_group * hkv);
-    const int d = threadIdx.x;
 
     const int64_t base = (int64_t)unit * p.n_splits * p.rows + rr;
     float top = neg_inf();
@@ -367,22 +496,23 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
         top = fmaxf(top, p.part_ml[2 * (base + (int64_t)s * p.rows)]);
     }
     const int64_t row = qb * p.q_seq + tok;
-    uint16_t *Arow = static_cast<uint16_t *>(p.A) + row * HEAD;
+    uint16_t *Adst = static_cast<uint16_t *>(p.A) + row * HEAD + d4;
     if(top == neg_inf())
     {
         // no visible key at all: leave lse and A untouched, or write the
         // empty row when the running pair is being overwritten
         if(p.overwrite)
         {
-            Arow[d] = 0;
-            if(d == 0)
+            *reinterpret_cast<u32x2 *>(Adst) = u32x2{0, 0};
+            if(d4 == 0)
             {
                 p.lse[row] = neg_inf();
             }
         }
         return;
     }
-    float l = 0.0f, acc = 0.0f;
+    float l = 0.0f;
+    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
     for(int s = 0; s < p.n_splits; ++s)
     {
         const int64_t prow = base + (int64_t)s * p.rows;
@@ -393,51 +523,60 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
         }
         const float w = __expf(m - top);
         l += w * p.part_ml[2 * prow + 1];
-        acc += w * p.part_o[prow * HEAD + d];
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(p.part_o + prow * HEAD + d4);
+        acc += w * v;
     }
     const float lse_new = top + __logf(l);
     const float lse_old = p.overwrite ? neg_inf() : p.lse[row];
     float w_old, w_new, lse_out;
     merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
-    float v = acc * (w_new / l);
+    const float sc = w_new / l;
+    float v[4] = {acc[0] * sc, acc[1] * sc, acc[2] * sc, acc[3] * sc};
     if(w_old != 0.0f)
     {
-        v += w_old * T::to_float(Arow[d]);
+        const u32x2 old = *reinterpret_cast<const u32x2 *>(Adst);
+        v[0] += w_old * T::to_float((uint16_t)(old[0] & 0xffffu));
+        v[1] += w_old * T::to_float((uint16_t)(old[0] >> 16));
+        v[2] += w_old * T::to_float((uint16_t)(old[1] & 0xffffu));
+        v[3] += w_old * T::to_float((uint16_t)(old[1] >> 16));
     }
-    Arow[d] = T::from_float(v);
-    __syncthreads();    // every thread has read lse_old before it changes
-    if(d == 0)
+    u32x2 out;
+    out[0] = T::pack2(v[0], v[1]);
+    out[1] = T::pack2(v[2], v[3]);
+    *reinterpret_cast<u32x2 *>(Adst) = out;
+    // The threads of a row sit in one wavefront (TPR <= 32 divides 64) and
+    // run in lock step: all of them have read lse_old by now.
+    if(d4 == 0)
     {
         p.lse[row] = lse_out;
     }
 }
 
-template<typename T, int HEAD>
-static int launch_decode_head(hipStream_t stream, const DecodeParams &p, int mode)
+template<typename T, int HEAD, int MODE, int STAGES>
+static void launch_decode_main(hipStream_t stream, const DecodeParams &p, dim3 grid)
+{
+    auto kernel = sdpa_decode_16bit_kernel<T, HEAD, MODE, STAGES>;
+    hipLaunchKernelGGL(kernel, grid, dim3(kDecThreads), 0, stream, p);
+}
+
+template<typename T, int HEAD, int STAGES>
+static int launch_decode_stages(hipStream_t stream, const DecodeParams &p, int mode)
 {
     const int units = p.n_batch * p.n_head_kv;
     const dim3 grid((unsigned)(units * p.n_splits));
     switch(mode)
     {
         case NNTILE_HIP_MASK_ADDITIVE:
-            hipLaunchKernelGGL((sdpa_decode_16bit_kernel<T, HEAD,
-                        NNTILE_HIP_MASK_ADDITIVE>), grid, dim3(kDecThreads), 0,
-                    stream, p);
+            launch_decode_main<T, HEAD, NNTILE_HIP_MASK_ADDITIVE, STAGES>(stream, p, grid);
             break;
         case NNTILE_HIP_MASK_NONE:
-            hipLaunchKernelGGL((sdpa_decode_16bit_kernel<T, HEAD,
-                        NNTILE_HIP_MASK_NONE>), grid, dim3(kDecThreads), 0,
-                    stream, p);
+            launch_decode_main<T, HEAD, NNTILE_HIP_MASK_NONE, STAGES>(stream, p, grid);
             break;
         case NNTILE_HIP_MASK_CAUSAL:
-            hipLaunchKernelGGL((sdpa_decode_16bit_kernel<T, HEAD,
-                        NNTILE_HIP_MASK_CAUSAL>), grid, dim3(kDecThreads), 0,
-                    stream, p);
+            launch_decode_main<T, HEAD, NNTILE_HIP_MASK_CAUSAL, STAGES>(stream, p, grid);
             break;
         case NNTILE_HIP_MASK_BOOL:
-            hipLaunchKernelGGL((sdpa_decode_16bit_kernel<T, HEAD,
-                        NNTILE_HIP_MASK_BOOL>), grid, dim3(kDecThreads), 0,
-                    stream, p);
+            launch_decode_main<T, HEAD, NNTILE_HIP_MASK_BOOL, STAGES>(stream, p, grid);
             break;
         default:
             return NNTILE_HIP_EINVAL;
@@ -446,17 +585,30 @@ static int launch_decode_head(hipStream_t stream, const DecodeParams &p, int mod
     {
         return NNTILE_HIP_ELAUNCH;
     }
-    hipLaunchKernelGGL((sdpa_decode_reduce_kernel<T, HEAD>),
-            dim3((unsigned)(units * p.rows)), dim3(HEAD), 0, stream, p);
+    {
+        constexpr int rows_per_wg = 256 / (HEAD / 4);
+        const int64_t total_rows = (int64_t)units * p.rows;
+        hipLaunchKernelGGL((sdpa_decode_reduce_kernel<T, HEAD>),
+                dim3((unsigned)((total_rows + rows_per_wg - 1) / rows_per_wg)),
+                dim3(256), 0, stream, p);
+    }
     return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
 }
 
-// Number of key splits per unit: enough workgroups to give every CU several
-// resident streams, never more than one split per key step.
+// Ring depth 2 (64 KB of LDS at head 128) lets two workgroups share a CU, which
+// measured faster than one workgroup with a deeper ring.
+template<typename T, int HEAD>
+static int launch_decode_head(hipStream_t stream, const DecodeParams &p, int mode)
+{
+    return launch_decode_stages<T, HEAD, 2>(stream, p, mode);
+}
+
+// Number of key splits per unit: two workgroups per CU when the units allow
+// it, never more than one split per key step.  Fewer splits mean fewer
+// partials to write and merge.
 int decode_choose_splits(int units, int n_steps)
 {
-    const int target_wg = 1024;     // 256 CUs x 4 resident workgroups
-    int splits = (target_wg + units - 1) / units;
+    int splits = (2 * kDecodeCUs + units - 1) / units;
     splits = splits < 1 ? 1 : splits;
     splits = splits > n_steps ? n_steps : splits;
     splits = splits > 64 ? 64 : splits;

@@ -78,7 +78,11 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             || MODE == NNTILE_HIP_MASK_BOOL);
     static_assert(LOADS_PER_WAVE >= 1, "head size too small for this tiling");
 
-    __shared__ __attribute__((aligned(1024))) char lds[2 * BUF_BYTES];
+    // Two separate arrays, not one: the compiler then knows that the loads
+    // streaming into one buffer cannot alias the reads of the other and does
+    // not make those reads wait for the loads.
+    __shared__ __attribute__((aligned(1024))) char lds_a[BUF_BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_b[BUF_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -242,10 +246,10 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // Global -> LDS loads of one step into buffer `buf`.  Rows past the end of
     // the tile are clamped to its last row: their scores are masked and their
     // probabilities are exactly 0, so any finite stand-in value works.
-    auto fetch = [&](const StepCursor &cur, int buf)
+    auto fetch = [&](const StepCursor &cur, char *buf_base)
     {
         // (wave index made visibly uniform: the LDS target goes into M0)
-        char *kdst = lds + buf * BUF_BYTES
+        char *kdst = buf_base
             + __builtin_amdgcn_readfirstlane(wave) * LOADS_PER_WAVE * 1024;
         char *vdst = kdst + K_BYTES;
         typedef const void __attribute__((address_space(1))) *gptr;
@@ -328,7 +332,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     StepCursor nxt = cur;                        // step being fetched
     if(n_steps > 0)
     {
-        fetch(nxt, 0);
+        fetch(nxt, lds_a);
         advance(nxt);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -339,7 +343,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     auto step = [&](int g, auto buf_tag)
     {
         constexpr int BUF = decltype(buf_tag)::value;
-        const char *Ks = lds + BUF * BUF_BYTES;
+        const char *Ks = BUF ? lds_b : lds_a;
         const int k_row0 = cur.kb * kKeys;                   // within the tile
         const int kg0 = cur.kt * k_tile + k_row0;            // key row overall
         const int keys_here = min(kKeys, cur.rows_left);
@@ -353,7 +357,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         NNTILE_PHASE(0)
         if(g + 1 < n_steps)
         {
-            fetch(nxt, BUF ^ 1);
+            fetch(nxt, BUF ? lds_a : lds_b);
             advance(nxt);
         }
 

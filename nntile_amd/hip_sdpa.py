@@ -211,6 +211,65 @@ def sdpa_fwd_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq,
     return a
 
 
+class Plan:
+    """A fully prepared call: argument block built once, launched many times.
+    NNTile tiles keep their addresses from step to step, so a layer prepares
+    its calls once; `launch` costs one foreign call."""
+
+    def __init__(self, fn, args, what, extra=(), keep=()):
+        self._fn, self._args, self._what, self._extra = fn, args, what, extra
+        self._keep = keep          # tensors whose memory the call refers to
+
+    def launch(self, stream=None):
+        rc = self._fn(_stream(stream), ctypes.byref(self._args), *self._extra)
+        if rc != OK:
+            raise SdpaError(rc, self._what)
+
+
+def plan_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq, q_tile, k_tile,
+              mask_mode, n_batch=None, kv_group=1, q_pos0=0, k_pos0=0, causal_offset=0, flags=0):
+    _dev(*K_tiles, *Q_tiles, *lse_tiles, *V_tiles, *A_tiles)
+    batch, _, head = Q_tiles[0].shape
+    if len(Q_tiles) > MAX_TILES or len(K_tiles) > MAX_TILES:
+        raise SdpaError(EINVAL, "sdpa_fwd_grid")
+    a = GridArgs()
+    a.q_seq, a.k_seq, a.q_tile, a.k_tile, a.head = q_seq, k_seq, q_tile, k_tile, head
+    a.batch = batch
+    a.n_batch = batch if n_batch is None else n_batch
+    a.kv_group = kv_group
+    a.mask_mode = mask_mode
+    a.flags = flags
+    a.n_q_tiles, a.n_kv_tiles = len(Q_tiles), len(K_tiles)
+    a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
+    for i, (k, v) in enumerate(zip(K_tiles, V_tiles)):
+        a.K[i], a.V[i] = k.data_ptr(), v.data_ptr()
+    for i, (q, l, o) in enumerate(zip(Q_tiles, lse_tiles, A_tiles)):
+        a.Q[i], a.lse[i], a.A[i] = q.data_ptr(), l.data_ptr(), o.data_ptr()
+    fn = getattr(lib(), "nntile_hip_sdpa_fwd_grid_" + dtype_name(Q_tiles[0]))
+    return Plan(fn, a, "sdpa_fwd_grid",
+                keep=(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles))
+
+
+def plan_tile(K, Q, mask, lse, V, A, mask_mode, n_batch=None, kv_group=1, q_pos0=0, k_pos0=0,
+              causal_offset=0, flags=0):
+    _dev(K, Q, mask, lse, V, A)
+    a = _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0, k_pos0,
+                   causal_offset, flags)
+    fn = getattr(lib(), "nntile_hip_sdpa_fwd_tile_" + dtype_name(Q))
+    return Plan(fn, a, "sdpa_fwd_tile", keep=(K, Q, mask, lse, V, A))
+
+
+def plan_decode(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, workspace, q_pos0=0,
+                k_pos0=0, causal_offset=0, flags=0):
+    _dev(K, Q, mask, lse, V, A, workspace)
+    a = _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0, k_pos0,
+                   causal_offset, flags)
+    fn = getattr(lib(), "nntile_hip_sdpa_fwd_decode_" + dtype_name(Q))
+    nbytes = workspace.numel() * workspace.element_size()
+    return Plan(fn, a, "sdpa_fwd_decode", extra=(_ptr(workspace), nbytes),
+                keep=(K, Q, mask, lse, V, A, workspace))
+
+
 def decode_workspace_bytes(K, Q, n_batch, kv_group):
     a = _tile_args(K, Q, None, Q, K, Q, MASK_NONE, n_batch, kv_group, 0, 0, 0)
     return int(lib().nntile_hip_sdpa_fwd_decode_workspace_bytes(ctypes.byref(a)))
