@@ -1,0 +1,199 @@
+// Flat C interface over the host-side mirror, for tests and scripts: tensors
+// are created from shapes and Fortran-ordered host arrays, the operations are
+// the mirror's tile::/tensor:: functions, exceptions come back as messages.
+#include <cstring>
+#include <string>
+
+#include "nntile_host.hh"
+
+using namespace nntile;
+
+namespace
+{
+
+enum DType { DT_BF16 = 0, DT_FP16 = 1, DT_FP32 = 2 };
+
+struct AnyTensor
+{
+    int dtype;
+    std::unique_ptr<tensor::Tensor<bf16_t>> bf16;
+    std::unique_ptr<tensor::Tensor<fp16_t>> fp16;
+    std::unique_ptr<tensor::Tensor<fp32_t>> fp32;
+};
+
+int fail(char *err, int errlen, const std::exception &e)
+{
+    if(err != nullptr && errlen > 0)
+    {
+        std::strncpy(err, e.what(), static_cast<size_t>(errlen) - 1);
+        err[errlen - 1] = '\0';
+    }
+    return 1;
+}
+
+std::vector<Index> vec(const int64_t *p, int n)
+{
+    return std::vector<Index>(p, p + n);
+}
+
+template<typename T> tensor::Tensor<T> &get(AnyTensor *t);
+template<> tensor::Tensor<bf16_t> &get<bf16_t>(AnyTensor *t) { return *t->bf16; }
+template<> tensor::Tensor<fp16_t> &get<fp16_t>(AnyTensor *t) { return *t->fp16; }
+template<> tensor::Tensor<fp32_t> &get<fp32_t>(AnyTensor *t) { return *t->fp32; }
+
+template<typename T>
+void run_op(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *mask, AnyTensor *lse,
+        AnyTensor *V, AnyTensor *A, int mask_mode, int64_t offset, int overwrite)
+{
+    switch(op)
+    {
+        case 0:     // tensor-level, per-tile tasks, blocking
+            tensor::flash_sdpa_fwd_cudnn<T>(get<T>(K), get<T>(Q), get<T>(mask),
+                    get<fp32_t>(lse), get<T>(V), get<T>(A));
+            break;
+        case 1:     // tile-level on single-tile tensors, blocking
+            tile::flash_sdpa_fwd_cudnn<T>(get<T>(K).get_tile(0), get<T>(Q).get_tile(0),
+                    get<T>(mask).get_tile(0), get<fp32_t>(lse).get_tile(0),
+                    get<T>(V).get_tile(0), get<T>(A).get_tile(0));
+            break;
+        case 2:     // tensor-level, one launch per slab, analytic mask
+            tensor::flash_sdpa_fwd_hip_async<T>(get<T>(K), get<T>(Q), mask_mode,
+                    offset, get<fp32_t>(lse), get<T>(V), get<T>(A), overwrite != 0);
+            starpu::task_wait_for_all();
+            break;
+        default:
+            throw std::runtime_error("unknown operation");
+    }
+}
+
+} // namespace
+
+extern "C"
+{
+
+void *nntile_host_tensor_create(int dtype, int ndim, const int64_t *shape,
+        const int64_t *basetile, char *err, int errlen)
+{
+    try
+    {
+        auto *t = new AnyTensor;
+        t->dtype = dtype;
+        if(dtype == DT_BF16) t->bf16.reset(new tensor::Tensor<bf16_t>(vec(shape, ndim), vec(basetile, ndim)));
+        else if(dtype == DT_FP16) t->fp16.reset(new tensor::Tensor<fp16_t>(vec(shape, ndim), vec(basetile, ndim)));
+        else t->fp32.reset(new tensor::Tensor<fp32_t>(vec(shape, ndim), vec(basetile, ndim)));
+        return t;
+    }
+    catch(const std::exception &e)
+    {
+        fail(err, errlen, e);
+        return nullptr;
+    }
+}
+
+void nntile_host_tensor_free(void *t)
+{
+    delete static_cast<AnyTensor *>(t);
+}
+
+int nntile_host_tensor_from_array(void *t_, const void *src, char *err, int errlen)
+{
+    auto *t = static_cast<AnyTensor *>(t_);
+    try
+    {
+        if(t->dtype == DT_BF16) t->bf16->from_array(static_cast<const uint16_t *>(src));
+        else if(t->dtype == DT_FP16) t->fp16->from_array(static_cast<const uint16_t *>(src));
+        else t->fp32->from_array(static_cast<const float *>(src));
+        return 0;
+    }
+    catch(const std::exception &e) { return fail(err, errlen, e); }
+}
+
+int nntile_host_tensor_to_array(void *t_, void *dst, char *err, int errlen)
+{
+    auto *t = static_cast<AnyTensor *>(t_);
+    try
+    {
+        if(t->dtype == DT_BF16) t->bf16->to_array(static_cast<uint16_t *>(dst));
+        else if(t->dtype == DT_FP16) t->fp16->to_array(static_cast<uint16_t *>(dst));
+        else t->fp32->to_array(static_cast<float *>(dst));
+        return 0;
+    }
+    catch(const std::exception &e) { return fail(err, errlen, e); }
+}
+
+int64_t nntile_host_tensor_ntiles(void *t_)
+{
+    auto *t = static_cast<AnyTensor *>(t_);
+    if(t->dtype == DT_BF16) return t->bf16->grid.nelems;
+    if(t->dtype == DT_FP16) return t->fp16->grid.nelems;
+    return t->fp32->grid.nelems;
+}
+
+// op: 0 tensor::flash_sdpa_fwd_cudnn, 1 tile::flash_sdpa_fwd_cudnn (single-tile
+// tensors), 2 tensor::flash_sdpa_fwd_hip_async + wait (mask may be null)
+int nntile_host_flash_sdpa_fwd(int op, int dtype, void *K, void *Q, void *mask,
+        void *lse, void *V, void *A, int mask_mode, int64_t offset, int overwrite,
+        char *err, int errlen)
+{
+    try
+    {
+        auto k = static_cast<AnyTensor *>(K), q = static_cast<AnyTensor *>(Q),
+             m = static_cast<AnyTensor *>(mask), l = static_cast<AnyTensor *>(lse),
+             v = static_cast<AnyTensor *>(V), a = static_cast<AnyTensor *>(A);
+        if(dtype == DT_BF16) run_op<bf16_t>(op, k, q, m, l, v, a, mask_mode, offset, overwrite);
+        else if(dtype == DT_FP16) run_op<fp16_t>(op, k, q, m, l, v, a, mask_mode, offset, overwrite);
+        else run_op<fp32_t>(op, k, q, m, l, v, a, mask_mode, offset, overwrite);
+        return 0;
+    }
+    catch(const std::exception &e) { return fail(err, errlen, e); }
+}
+
+// Shape rules only (no device memory): level 0 = tile, 1 = tensor.  Shapes are
+// given as 6 x (ndim, dims..., basetile dims...) blocks in the order
+// K, Q, mask, logsumexp, V, A.
+int nntile_host_check_shapes(int level, const int64_t *desc, char *err, int errlen)
+{
+    try
+    {
+        std::vector<tensor::TensorTraits> tt;
+        const int64_t *p = desc;
+        for(int i = 0; i < 6; ++i)
+        {
+            const int nd = static_cast<int>(*p++);
+            auto shape = vec(p, nd); p += nd;
+            auto base = vec(p, nd); p += nd;
+            tt.emplace_back(shape, base);
+        }
+        if(level == 0)
+        {
+            tile::flash_sdpa_fwd_cudnn_check(tt[0], tt[1], tt[2], tt[3], tt[4], tt[5]);
+        }
+        else
+        {
+            tensor::flash_sdpa_fwd_cudnn_check(tt[0], tt[1], tt[2], tt[3], tt[4], tt[5]);
+        }
+        return 0;
+    }
+    catch(const std::exception &e) { return fail(err, errlen, e); }
+}
+
+uint32_t nntile_host_footprint(int64_t seq, int64_t head, int64_t batch)
+{
+    return starpu::FlashSdpaFwdCudnn<std::tuple<bf16_t>>::hash_parameters(seq, head, batch);
+}
+
+int64_t nntile_host_tasks_submitted(int dtype)
+{
+    if(dtype == DT_BF16) return starpu::flash_sdpa_fwd_cudnn<bf16_t>().submitted;
+    if(dtype == DT_FP16) return starpu::flash_sdpa_fwd_cudnn<fp16_t>().submitted;
+    return starpu::flash_sdpa_fwd_cudnn<fp32_t>().submitted;
+}
+
+const char *nntile_host_codelet_name(int dtype)
+{
+    if(dtype == DT_BF16) return starpu::flash_sdpa_fwd_cudnn<bf16_t>().name.c_str();
+    if(dtype == DT_FP16) return starpu::flash_sdpa_fwd_cudnn<fp16_t>().name.c_str();
+    return starpu::flash_sdpa_fwd_cudnn<fp32_t>().name.c_str();
+}
+
+} // extern "C"

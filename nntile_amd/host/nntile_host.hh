@@ -1,0 +1,217 @@
+// Host-side mirror of the NNTile layers the attention hot path crosses
+// (tile -> starpu codelet -> kernel), on a minimal stand-in runtime.
+//
+// Names, argument order, shape rules and error messages follow the reference:
+//   TileTraits / TensorTraits     include/nntile/tile/traits.hh:27-195,
+//                                 include/nntile/tensor/traits.hh:23-116
+//   starpu::FlashSdpaFwdCudnn     include/nntile/starpu/flash_sdpa_fwd_cudnn.hh:44-145,
+//                                 src/starpu/flash_sdpa_fwd_cudnn.cc:37-296
+//   tile::flash_sdpa_fwd_cudnn*   src/tile/flash_sdpa_fwd_cudnn.cc:25-213
+//   tensor::flash_sdpa_fwd_cudnn* src/tensor/flash_sdpa_fwd_cudnn.cc:23-297
+// What differs, on purpose: the codelet carries a HIP body (the C-ABI entry
+// point nntile_hip_flash_sdpa_fwd_codelet_<T>) next to the empty CPU list, the
+// pack gains fp32, and tensor:: gains flash_sdpa_fwd_hip_async, which merges
+// all key tiles of a slab in one launch when the mask is analytic.
+//
+// The runtime here is NOT StarPU: a Handle is a device allocation, submit()
+// runs the codelet body at once on the context's stream (in-order execution
+// gives the sequential consistency that StarPU derives from access modes).
+#pragma once
+
+#include <array>
+#include <cstdint>
+#include <cstdlib>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <tuple>
+#include <vector>
+
+#include "../../include/nntile_hip_sdpa.h"
+
+namespace nntile
+{
+
+using Index = std::int64_t;     // include/nntile/base_types.hh:45
+using Scalar = float;           // include/nntile/base_types.hh:48
+
+// Tile value types: storage only (include/nntile/base_types.hh:241-737).
+struct fp32_t { using storage_t = float; static constexpr const char *short_name = "fp32"; };
+struct bf16_t { using storage_t = std::uint16_t; static constexpr const char *short_name = "bf16"; };
+struct fp16_t { using storage_t = std::uint16_t; static constexpr const char *short_name = "fp16"; };
+
+namespace tile
+{
+
+//! Integer properties of a contiguous Fortran-ordered tile
+class TileTraits
+{
+public:
+    Index ndim;
+    std::vector<Index> shape;
+    std::vector<Index> stride;      // stride[0] = 1, stride[i+1] = stride[i]*shape[i]
+    Index nelems;
+    std::vector<std::array<Index, 2>> matrix_shape;
+    explicit TileTraits(const std::vector<Index> &shape_);
+    //! Linear offset of an element
+    Index index_to_linear(const std::vector<Index> &index) const;
+    std::vector<Index> linear_to_index(Index linear) const;
+};
+
+} // namespace tile
+
+namespace starpu
+{
+
+//! Device allocation standing in for a StarPU variable handle
+class Handle
+{
+    std::shared_ptr<void> mem;
+    std::size_t nbytes = 0;
+public:
+    Handle() = default;
+    explicit Handle(std::size_t size);      // allocates device memory
+    void *get_ptr() const { return mem.get(); }
+    std::size_t size() const { return nbytes; }
+    //! Blocking copies (the analogue of acquire/release on the host)
+    void from_host(const void *src) const;
+    void to_host(void *dst) const;
+    //! The reference's scratch handles are unregistered right after the
+    //! submission (src/tile/flash_sdpa_fwd_cudnn.cc:194-195)
+    void unregister_submit() { mem.reset(); nbytes = 0; }
+};
+
+using VariableHandle = Handle;
+
+//! Stream every codelet body of this process enqueues on
+void *get_local_stream();
+void task_wait_for_all();
+
+//! Wrapper of the attention codelet for one value type
+template<typename T> class FlashSdpaFwdCudnn;
+
+template<typename T>
+class FlashSdpaFwdCudnn<std::tuple<T>>
+{
+public:
+    std::string name;       // "nntile_flash_sdpa_fwd_cudnn_<type>"
+    //! Arguments handed to the body (reference args_t, same leading members)
+    struct args_t
+    {
+        FlashSdpaFwdCudnn<std::tuple<T>> *owner;
+        Index seq;
+        Index head;
+        Index batch;
+    };
+    FlashSdpaFwdCudnn();
+    static std::uint32_t hash_parameters(Index seq, Index head, Index batch);
+    //! No CPU implementation, as in the reference
+    static constexpr std::array<void (*)(void **, void *), 1> cpu_funcs = {nullptr};
+    //! The HIP body, same shape as the reference's cuda(buffers, cl_args)
+    static void hip(void *buffers[], void *cl_args) noexcept;
+    void submit(Index seq, Index head, Index batch, Handle K, Handle Q,
+            Handle mask, Handle logsumexp, Handle V, Handle A,
+            Handle scratch_logsumexp, Handle scratch_A);
+    //! Number of tasks submitted so far (for tests)
+    Index submitted = 0;
+};
+
+//! One codelet object per value type, looked up by type
+template<typename T> FlashSdpaFwdCudnn<std::tuple<T>> &flash_sdpa_fwd_cudnn();
+
+} // namespace starpu
+
+namespace tile
+{
+
+template<typename T>
+class Tile: public TileTraits, public starpu::Handle
+{
+public:
+    explicit Tile(const std::vector<Index> &shape_):
+        TileTraits(shape_),
+        starpu::Handle(sizeof(typename T::storage_t) * nelems)
+    {
+    }
+    explicit Tile(const TileTraits &traits):
+        TileTraits(traits),
+        starpu::Handle(sizeof(typename T::storage_t) * nelems)
+    {
+    }
+};
+
+//! Shape rules of one tile task; throws std::runtime_error
+void flash_sdpa_fwd_cudnn_check(const TileTraits &K, const TileTraits &Q,
+        const TileTraits &mask, const TileTraits &logsumexp,
+        const TileTraits &V, const TileTraits &A);
+
+template<typename T>
+void flash_sdpa_fwd_cudnn_async(const Tile<T> &K, const Tile<T> &Q,
+        const Tile<T> &mask, const Tile<fp32_t> &logsumexp, const Tile<T> &V,
+        const Tile<T> &A);
+
+template<typename T>
+void flash_sdpa_fwd_cudnn(const Tile<T> &K, const Tile<T> &Q,
+        const Tile<T> &mask, const Tile<fp32_t> &logsumexp, const Tile<T> &V,
+        const Tile<T> &A);
+
+} // namespace tile
+
+namespace tensor
+{
+
+class TensorTraits: public tile::TileTraits
+{
+public:
+    std::vector<Index> basetile_shape;
+    tile::TileTraits grid;
+    std::vector<Index> leftover_shape;
+    TensorTraits(const std::vector<Index> &shape_,
+            const std::vector<Index> &basetile_shape_);
+    std::vector<Index> get_tile_shape(const std::vector<Index> &tile_index) const;
+};
+
+template<typename T>
+class Tensor: public TensorTraits
+{
+    std::vector<tile::Tile<T>> tiles;
+public:
+    Tensor(const std::vector<Index> &shape_, const std::vector<Index> &basetile_shape_);
+    const tile::Tile<T> &get_tile(Index linear) const { return tiles.at(linear); }
+    const tile::Tile<T> &get_tile(const std::vector<Index> &tile_index) const
+    {
+        return tiles.at(grid.index_to_linear(tile_index));
+    }
+    //! Whole-tensor Fortran-ordered host array <-> tiles (blocking)
+    void from_array(const typename T::storage_t *src) const;
+    void to_array(typename T::storage_t *dst) const;
+};
+
+//! Shape and tiling rules of the tensor-level operation; throws
+void flash_sdpa_fwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
+        const TensorTraits &mask, const TensorTraits &logsumexp,
+        const TensorTraits &V, const TensorTraits &A);
+
+//! One tile task per (output tile, key tile) pair, in the reference's order
+template<typename T>
+void flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &V, const Tensor<T> &A);
+
+template<typename T>
+void flash_sdpa_fwd_cudnn(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &V, const Tensor<T> &A);
+
+//! Same result with an analytic mask (mask_mode NNTILE_HIP_MASK_NONE or
+//! NNTILE_HIP_MASK_CAUSAL with `causal_offset`): for every (batch, group,
+//! head) slab all key tiles are merged into all query tiles in ONE launch.
+//! `overwrite` = the running pair need not be initialised by the caller.
+template<typename T>
+void flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
+        int mask_mode, Index causal_offset, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &V, const Tensor<T> &A, bool overwrite);
+
+} // namespace tensor
+
+} // namespace nntile

@@ -1,0 +1,117 @@
+"""ctypes front-end of libnntile_host.so, the C++ mirror of the NNTile
+tile/tensor/codelet layers for the attention path.  Arrays are numpy,
+Fortran-ordered, in the reference's axis order [head, seq, batch, group, kv]."""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "host", "libnntile_host.so")
+DTYPES = {"bf16": 0, "fp16": 1, "fp32": 2}
+OP_TENSOR, OP_TILE, OP_HIP = 0, 1, 2
+_lib = None
+
+
+class HostError(RuntimeError):
+    """A std::runtime_error thrown by the C++ layer."""
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libnntile_host.so is missing: run `make -C nntile_amd/host`")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i64 = ctypes.c_void_p, ctypes.c_int64
+        L.nntile_host_tensor_create.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(i64),
+                                                ctypes.POINTER(i64), ctypes.c_char_p, ctypes.c_int]
+        L.nntile_host_tensor_create.restype = vp
+        L.nntile_host_tensor_free.argtypes = [vp]
+        L.nntile_host_tensor_from_array.argtypes = [vp, vp, ctypes.c_char_p, ctypes.c_int]
+        L.nntile_host_tensor_to_array.argtypes = [vp, vp, ctypes.c_char_p, ctypes.c_int]
+        L.nntile_host_tensor_ntiles.argtypes = [vp]
+        L.nntile_host_tensor_ntiles.restype = i64
+        L.nntile_host_flash_sdpa_fwd.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp,
+                                                 ctypes.c_int, i64, ctypes.c_int, ctypes.c_char_p,
+                                                 ctypes.c_int]
+        L.nntile_host_check_shapes.argtypes = [ctypes.c_int, ctypes.POINTER(i64), ctypes.c_char_p,
+                                               ctypes.c_int]
+        L.nntile_host_footprint.argtypes = [i64, i64, i64]
+        L.nntile_host_footprint.restype = ctypes.c_uint32
+        L.nntile_host_tasks_submitted.argtypes = [ctypes.c_int]
+        L.nntile_host_tasks_submitted.restype = i64
+        L.nntile_host_codelet_name.argtypes = [ctypes.c_int]
+        L.nntile_host_codelet_name.restype = ctypes.c_char_p
+        _lib = L
+    return _lib
+
+
+def _arr(v):
+    return (ctypes.c_int64 * len(v))(*v)
+
+
+def _call(fn, *args):
+    err = ctypes.create_string_buffer(256)
+    rc = fn(*args, err, 256)
+    if rc != 0:
+        raise HostError(err.value.decode())
+
+
+class Tensor:
+    """nntile::tensor::Tensor<T>: a grid of separately allocated device tiles."""
+
+    def __init__(self, dtype, shape, basetile):
+        self.dtype, self.shape, self.basetile = dtype, tuple(shape), tuple(basetile)
+        err = ctypes.create_string_buffer(256)
+        self.h = lib().nntile_host_tensor_create(DTYPES[dtype], len(shape), _arr(shape),
+                                                 _arr(basetile), err, 256)
+        if not self.h:
+            raise HostError(err.value.decode())
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().nntile_host_tensor_free(self.h)
+            self.h = None
+
+    @property
+    def ntiles(self):
+        return int(lib().nntile_host_tensor_ntiles(self.h))
+
+    def from_array(self, a):
+        np_dt = np.float32 if self.dtype == "fp32" else np.uint16
+        a = np.asfortranarray(a, dtype=np_dt)
+        assert a.shape == self.shape
+        _call(lib().nntile_host_tensor_from_array, self.h, a.ctypes.data_as(ctypes.c_void_p))
+        return self
+
+    def to_array(self):
+        np_dt = np.float32 if self.dtype == "fp32" else np.uint16
+        out = np.empty(self.shape, dtype=np_dt, order="F")
+        _call(lib().nntile_host_tensor_to_array, self.h, out.ctypes.data_as(ctypes.c_void_p))
+        return out
+
+
+def flash_sdpa_fwd(op, K, Q, mask, lse, V, A, mask_mode=0, offset=0, overwrite=False):
+    _call(lib().nntile_host_flash_sdpa_fwd, op, DTYPES[Q.dtype], K.h, Q.h,
+          None if mask is None else mask.h, lse.h, V.h, A.h, mask_mode, offset, int(overwrite))
+
+
+def check_shapes(level, specs):
+    """specs: six (shape, basetile) pairs in the order K, Q, mask, logsumexp, V, A."""
+    flat = []
+    for shape, base in specs:
+        flat += [len(shape)] + list(shape) + list(base)
+    _call(lib().nntile_host_check_shapes, level, _arr(flat))
+
+
+def footprint(seq, head, batch):
+    return int(lib().nntile_host_footprint(seq, head, batch))
+
+
+def tasks_submitted(dtype):
+    return int(lib().nntile_host_tasks_submitted(DTYPES[dtype]))
+
+
+def codelet_name(dtype):
+    return lib().nntile_host_codelet_name(DTYPES[dtype]).decode()
