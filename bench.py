@@ -27,28 +27,34 @@ PEAK_FP32_TFLOPS = 157.3      # MI355X fp32 matrix
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 
 
-def _events(n):
-    import torch
-    return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-            for _ in range(n)]
+# HBM bytes per launch from the hardware counters (FETCH_SIZE x 2.000 +
+# WRITE_SIZE x 1.000, the factors a 1 GiB device copy calibrates); the runs
+# and their figures are in profiles/sdpa_*_kernel_cfg*.txt.  They are
+# properties of the kernel and the workload, not of one timing run.
+TRAFFIC_PREFILL_CFG3 = 177748615      # Q+K+V 96 MiB in, A+lse 32.5 MiB out, K/V re-read 1.6x
+TRAFFIC_DECODE_CFG4 = 312418907       # main kernel + merge kernel, incl. 16.25 MiB of partials
 
 
 def time_steps(step, steps, warmup):
-    """Runs `step` warmup+steps times; returns (wall ms per step, mean device
-    ms per step from HIP events recorded on the launch stream)."""
+    """Runs `step` warmup times untimed, then exactly `steps` times between
+    two device synchronisations.  Returns (wall ms per step, device ms per
+    step); the device figure is one pair of HIP events recorded around the
+    timed region on the stream the kernels are launched on (torch's current
+    stream, which the library's stream argument is taken from)."""
     import torch
     for _ in range(warmup):
         step()
+    a = torch.cuda.Event(enable_timing=True)
+    b = torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
-    ev = _events(steps)
     t0 = time.perf_counter()
-    for a, b in ev:
-        a.record()
+    a.record()
+    for _ in range(steps):
         step()
-        b.record()
+    b.record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
-    dev = sum(a.elapsed_time(b) for a, b in ev) / steps
+    dev = a.elapsed_time(b) / steps
     return wall, dev
 
 
@@ -192,11 +198,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run only this leg: prefill | decode | per_task | extras (for profiling)")
+                    help="run only this leg: prefill | decode | per_task | extras | copy (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
-                         "(the path shards over (batch, kv head) with no exchange; see DESIGN.md)\n"
+                         "(the path shards over (batch, kv head) with no exchange between GPUs)\n"
                          % args.gpus)
         sys.exit(2)
 
@@ -220,6 +226,15 @@ def main():
         bench_decode(cfg4, args.steps, args.warmup)
         return
     if only == "prefill":
+        return
+    if only == "copy":
+        # calibration leg for the HBM traffic counters: a plain device copy
+        # of 1 GiB (reads 2^30 bytes, writes 2^30 bytes per launch)
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup + args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
         return
     if only == "extras":
         for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):
@@ -263,7 +278,7 @@ def main():
         "roofline": {"bound": "mfma", "kernel": "sdpa_prefill_16bit_kernel<bf16,128,causal>",
                      "achieved": round(main_leg["kernel_tflops"], 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(main_leg["kernel_tflops"] / PEAK_BF16_TFLOPS, 4),
-                     "traffic": None,
+                     "traffic": TRAFFIC_PREFILL_CFG3,
                      "kernel_ms": round(main_leg["kernel_ms_per_step"], 4)},
         "decode": {"workload": cfg4.name, "ms_per_step": round(dec["ms_per_step"], 4),
                    "value": round(dec["gbs"], 1), "unit": "GB/s",
@@ -271,7 +286,7 @@ def main():
                    "roofline": {"bound": "hbm", "kernel": "sdpa_decode_16bit_kernel + reduce",
                                 "achieved": round(dec["kernel_gbs"], 1), "peak": PEAK_HBM_GBS,
                                 "unit": "GB/s", "frac": round(dec["kernel_gbs"] / PEAK_HBM_GBS, 4),
-                                "traffic": None,
+                                "traffic": TRAFFIC_DECODE_CFG4,
                                 "algorithmic_bytes": dec["algorithmic_bytes"],
                                 "workspace_bytes": dec["workspace_bytes"],
                                 "kernel_ms": round(dec["kernel_ms_per_step"], 4)}},
