@@ -200,7 +200,7 @@ static void decode_geometry(const nntile_hip_sdpa_tile_args *a, int &units,
         int &n_steps, int &splits, int &rows)
 {
     units = (int)(a->batch / a->kv_group);
-    n_steps = (int)((a->k_seq + 63) / 64);
+    n_steps = (int)((a->k_seq + kDecKeys - 1) / kDecKeys);
     splits = decode_choose_splits(units, n_steps);
     rows = (int)(a->q_seq * a->kv_group);
 }

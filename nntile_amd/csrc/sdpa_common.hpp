@@ -21,6 +21,7 @@ namespace nntile_hip
 {
 
 constexpr int kMaxTiles = NNTILE_HIP_SDPA_MAX_TILES;
+constexpr int kDecKeys = 64;    // keys per step of the decode kernel
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -88,6 +89,7 @@ __device__ __forceinline__ float neg_inf()
 struct Bf16
 {
     typedef bf16x8 vec8;
+    static constexpr uint32_t kNegInfPair = 0xFF80FF80u;    // two -inf values
     static __device__ __forceinline__ float to_float(uint16_t v)
     {
         return __uint_as_float(static_cast<uint32_t>(v) << 16);
@@ -122,6 +124,7 @@ struct Bf16
 struct Fp16
 {
     typedef f16x8 vec8;
+    static constexpr uint32_t kNegInfPair = 0xFC00FC00u;    // two -inf values
     static __device__ __forceinline__ float to_float(uint16_t v)
     {
         return static_cast<float>(__builtin_bit_cast(_Float16, v));

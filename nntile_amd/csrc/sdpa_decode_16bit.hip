@@ -29,7 +29,6 @@ namespace nntile_hip
 #define NNTILE_DMA_AUX 2
 #endif
 
-constexpr int kDecKeys = 64;      // keys per step
 constexpr int kDecThreads = 256;  // 4 wavefronts x 16 query rows
 constexpr int kDecodeCUs = 256;   // MI355X
 
@@ -74,6 +73,7 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
     typedef typename T::vec8 vec8;
     constexpr int KSTEPS = HEAD / 32;       // MFMA steps along head for S
     constexpr int DBLOCKS = HEAD / 16;      // 16-row blocks of O^T
+    constexpr int KB = kDecKeys / 16;       // 16-key blocks of S^T per step
     constexpr int RB = HEAD * 2;            // bytes per K/V row
     constexpr int CPR = HEAD / 8;           // 16-byte chunks per row
     constexpr int RPL = 16 / CPR;           // rows per 256-byte line of LDS banks
@@ -294,9 +294,9 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         const int keys_here = (int)min((int64_t)kDecKeys, p.k_seq - k_row0);
 
         // ---- S^T = K Q^T: 4 blocks of 16 keys ----------------------------------
-        acc4 s[4];
+        acc4 s[KB];
 #pragma unroll
-        for(int kb = 0; kb < 4; ++kb)
+        for(int kb = 0; kb < KB; ++kb)
         {
             s[kb] = acc4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -313,7 +313,7 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         {
             // the mask is [k_seq, q_seq]: row index = token
 #pragma unroll
-            for(int kb = 0; kb < 4; ++kb)
+            for(int kb = 0; kb < KB; ++kb)
             {
                 const int key0 = 16 * kb + 4 * quad;
 #pragma unroll
@@ -351,7 +351,7 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
                 const int lim = (int)max((int64_t)-1,
                         min(vis, (int64_t)keys_here - 1));
 #pragma unroll
-                for(int kb = 0; kb < 4; ++kb)
+                for(int kb = 0; kb < KB; ++kb)
                 {
 #pragma unroll
                     for(int e = 0; e < 4; ++e)
@@ -368,7 +368,7 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         // ---- online softmax ---------------------------------------------------
         float mx = neg_inf();
 #pragma unroll
-        for(int kb = 0; kb < 4; ++kb)
+        for(int kb = 0; kb < KB; ++kb)
         {
 #pragma unroll
             for(int e = 0; e < 4; ++e)
@@ -393,9 +393,9 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
             m_run = m_new;
         }
         float rs = 0.0f;
-        uint32_t pk[4][2];
+        uint32_t pk[KB][2];
 #pragma unroll
-        for(int kb = 0; kb < 4; ++kb)
+        for(int kb = 0; kb < KB; ++kb)
         {
             const float p0 = fast_exp2(fmaf(s[kb][0], c, -mc));
             const float p1 = fast_exp2(fmaf(s[kb][1], c, -mc));
@@ -410,7 +410,7 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
 
         // ---- O^T += V^T P^T: 2 steps of 32 keys ----------------------------------
 #pragma unroll
-        for(int t = 0; t < 2; ++t)
+        for(int t = 0; t < KB / 2; ++t)
         {
             const u32x4 praw = {pk[2 * t][0], pk[2 * t][1], pk[2 * t + 1][0],
                 pk[2 * t + 1][1]};
@@ -490,10 +490,26 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
     const int64_t qb = nb + (int64_t)p.n_batch * (g + (int64_t)p.kv_group * hkv);
 
     const int64_t base = (int64_t)unit * p.n_splits * p.rows + rr;
+    const int last_split = p.n_splits - 1;
+    typedef __attribute__((ext_vector_type(2))) float f32x2;
+    // The loads of up to 8 splits are issued together (indices past the last
+    // split are clamped and get weight 0): the latency of the partials is
+    // paid once per 8 splits, not once per split.
     float top = neg_inf();
-    for(int s = 0; s < p.n_splits; ++s)
+    for(int s0 = 0; s0 < p.n_splits; s0 += 8)
     {
-        top = fmaxf(top, p.part_ml[2 * (base + (int64_t)s * p.rows)]);
+        float m[8];
+#pragma unroll
+        for(int j = 0; j < 8; ++j)
+        {
+            const int sidx = min(s0 + j, last_split);
+            m[j] = p.part_ml[2 * (base + (int64_t)sidx * p.rows)];
+        }
+#pragma unroll
+        for(int j = 0; j < 8; ++j)
+        {
+            top = fmaxf(top, m[j]);
+        }
     }
     const int64_t row = qb * p.q_seq + tok;
     uint16_t *Adst = static_cast<uint16_t *>(p.A) + row * HEAD + d4;
@@ -513,18 +529,26 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
     }
     float l = 0.0f;
     f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-    for(int s = 0; s < p.n_splits; ++s)
+    for(int s0 = 0; s0 < p.n_splits; s0 += 8)
     {
-        const int64_t prow = base + (int64_t)s * p.rows;
-        const float m = p.part_ml[2 * prow];
-        if(m == neg_inf())
+        f32x2 ml[8];
+        f32x4 v[8];
+#pragma unroll
+        for(int j = 0; j < 8; ++j)
         {
-            continue;
+            const int sidx = min(s0 + j, last_split);
+            const int64_t prow = base + (int64_t)sidx * p.rows;
+            ml[j] = *reinterpret_cast<const f32x2 *>(p.part_ml + 2 * prow);
+            v[j] = *reinterpret_cast<const f32x4 *>(p.part_o + prow * HEAD + d4);
         }
-        const float w = __expf(m - top);
-        l += w * p.part_ml[2 * prow + 1];
-        const f32x4 v = *reinterpret_cast<const f32x4 *>(p.part_o + prow * HEAD + d4);
-        acc += w * v;
+#pragma unroll
+        for(int j = 0; j < 8; ++j)
+        {
+            const bool live = (s0 + j <= last_split) && (ml[j][0] != neg_inf());
+            const float w = live ? __expf(ml[j][0] - top) : 0.0f;
+            l += w * ml[j][1];
+            acc += w * v[j];
+        }
     }
     const float lse_new = top + __logf(l);
     const float lse_old = p.overwrite ? neg_inf() : p.lse[row];

@@ -307,10 +307,90 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         }
     };
 
-    // Score units: in the analytic modes the raw dot product is kept and the
-    // scale is folded into the exponent; with an explicit mask the score is
-    // scaled first and the mask value added.
-    const float c = EXPLICIT ? kLog2e : p.scale * kLog2e;
+    // Score units: the raw dot product is kept and the scale is folded into
+    // the exponent; an additive mask value is divided by the scale before it
+    // is added, which is the same thing.
+    const float c = p.scale * kLog2e;
+    const float inv_scale = 1.0f / p.scale;
+
+    // ---- explicit mask tiles ----------------------------------------------------
+    // The lane's 32 mask values of a key step (query my_q, keys
+    // mb*32 + 8*rg + 4*half + 0..3) are 8 groups of 4 consecutive elements:
+    // one 8-byte (additive) or 4-byte (boolean) load per group, issued one
+    // step ahead.  At the top of a step the wavefront classifies its 32 x 64
+    // block from the raw bits: nothing hidden (the step runs as if there were
+    // no mask), everything hidden (the step is skipped), or mixed (the values
+    // are applied).  Ragged steps and masks that are not aligned for the wide
+    // loads take the element-wise path.
+    constexpr int MW = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 16 : 8;    // dwords per lane and step
+    enum { MASK_ZERO = 0, MASK_HIDDEN = 1, MASK_MIXED = 2, MASK_SLOW = 3 };
+    uint32_t mraw[MW];
+#pragma unroll
+    for(int i = 0; i < MW; ++i)
+    {
+        mraw[i] = 0;
+    }
+    const int64_t mask_row = (int64_t)(q_ok ? my_q : 0) * p.mask_ld;
+    const bool mask_wide = EXPLICIT && (p.mask_ld % 4 == 0)
+        && (reinterpret_cast<uintptr_t>(p.mask) % 8 == 0);
+    // loads of the mask values of key step kb (a full step) into mraw
+    auto mask_fetch = [&](int kb)
+    {
+        if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+        {
+            const uint16_t *mp = static_cast<const uint16_t *>(p.mask) + mask_row
+                + kb * kKeys + 4 * half;
+#pragma unroll
+            for(int i = 0; i < 8; ++i)
+            {
+                const u32x2 v = *reinterpret_cast<const u32x2 *>(
+                        mp + (i >> 2) * 32 + (i & 3) * 8);
+                mraw[2 * i] = v[0];
+                mraw[2 * i + 1] = v[1];
+            }
+        }
+        else if(MODE == NNTILE_HIP_MASK_BOOL)
+        {
+            const uint8_t *mp = static_cast<const uint8_t *>(p.mask) + mask_row
+                + kb * kKeys + 4 * half;
+#pragma unroll
+            for(int i = 0; i < 8; ++i)
+            {
+                mraw[i] = *reinterpret_cast<const uint32_t *>(
+                        mp + (i >> 2) * 32 + (i & 3) * 8);
+            }
+        }
+    };
+    auto mask_classify = [&]() -> int
+    {
+        uint32_t all_or = 0u, all_and = 0xffffffffu;
+#pragma unroll
+        for(int i = 0; i < MW; ++i)
+        {
+            all_or |= mraw[i];
+            all_and &= mraw[i];
+        }
+        bool lane_open, lane_hidden;
+        if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+        {
+            lane_open = (all_or == 0u);                 // every value is +0
+            lane_hidden = (all_or == T::kNegInfPair) && (all_and == T::kNegInfPair);
+        }
+        else
+        {
+            lane_open = (all_or == 0x01010101u) && (all_and == 0x01010101u);
+            lane_hidden = (all_or == 0u);
+        }
+        if(__builtin_amdgcn_ballot_w64(!lane_open) == 0)
+        {
+            return MASK_ZERO;
+        }
+        if(__builtin_amdgcn_ballot_w64(!lane_hidden) == 0)
+        {
+            return MASK_HIDDEN;
+        }
+        return MASK_MIXED;
+    };
 
     f32x16 o[DBLOCKS];
 #pragma unroll
@@ -334,6 +414,10 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     {
         fetch(nxt, lds_a);
         advance(nxt);
+        if(mask_wide && cur.rows_left >= kKeys)
+        {
+            mask_fetch(0);
+        }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -347,9 +431,16 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         const int k_row0 = cur.kb * kKeys;                   // within the tile
         const int kg0 = cur.kt * k_tile + k_row0;            // key row overall
         const int keys_here = min(kKeys, cur.rows_left);
+        // explicit mask: what this wavefront's block of the mask looks like
+        // (the values were loaded during the previous step)
+        int mask_class = MASK_SLOW;
+        if(EXPLICIT && mask_wide && keys_here == kKeys)
+        {
+            mask_class = mask_classify();
+        }
         // nothing of this step is visible to this wavefront
-        const bool idle = (MODE == NNTILE_HIP_MASK_CAUSAL)
-            && (kg0 > wave_rel_lo + 31);
+        const bool idle = EXPLICIT ? (mask_class == MASK_HIDDEN)
+            : ((MODE == NNTILE_HIP_MASK_CAUSAL) && (kg0 > wave_rel_lo + 31));
 
         // ---- loads of the next step into the other buffer ----------------------
         // (every wavefront passed the barrier that ended step g-1, so nobody
@@ -388,45 +479,70 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             // register r of block mb holds key  mb*32 + 8*(r/4) + 4*half + r%4
             if(EXPLICIT)
             {
-                const int64_t qrow = q_ok ? my_q : 0;
-#pragma unroll
-                for(int mb = 0; mb < 2; ++mb)
+                if(mask_class == MASK_MIXED)
                 {
 #pragma unroll
-                    for(int rg = 0; rg < 4; ++rg)
+                    for(int i = 0; i < 8; ++i)
                     {
-                        const int key0 = mb * 32 + 8 * rg + 4 * half;
-                        const int64_t krow = k_row0 + key0;
-                        float add[4];
+                        // group i: block i/4, registers 4*(i%4) .. +3
+                        const int mb = i >> 2, r0 = 4 * (i & 3);
                         if(MODE == NNTILE_HIP_MASK_ADDITIVE)
                         {
-                            const uint16_t *mp = static_cast<const uint16_t *>(
-                                    p.mask) + qrow * p.mask_ld + krow;
 #pragma unroll
                             for(int e = 0; e < 4; ++e)
                             {
-                                add[e] = (key0 + e < keys_here)
-                                    ? T::to_float(mp[e]) : neg_inf();
+                                const uint32_t w = mraw[2 * i + (e >> 1)];
+                                const float add = T::to_float((uint16_t)(
+                                            (e & 1) ? (w >> 16) : (w & 0xffffu)));
+                                s[mb][r0 + e] = fmaf(add, inv_scale, s[mb][r0 + e]);
                             }
                         }
                         else
                         {
-                            const uint8_t *mp = static_cast<const uint8_t *>(
-                                    p.mask) + qrow * p.mask_ld + krow;
 #pragma unroll
                             for(int e = 0; e < 4; ++e)
                             {
-                                add[e] = (key0 + e < keys_here && mp[e] != 0)
-                                    ? 0.0f : neg_inf();
+                                if(((mraw[i] >> (8 * e)) & 0xffu) == 0u)
+                                {
+                                    s[mb][r0 + e] = neg_inf();
+                                }
                             }
                         }
+                    }
+                }
+                else if(mask_class == MASK_SLOW)
+                {
 #pragma unroll
-                        for(int e = 0; e < 4; ++e)
+                    for(int mb = 0; mb < 2; ++mb)
+                    {
+#pragma unroll
+                        for(int rg = 0; rg < 4; ++rg)
                         {
-                            const float v = s[mb][4 * rg + e] * p.scale + add[e];
-                            // a hidden key stays hidden whatever the score is
-                            s[mb][4 * rg + e] = (add[e] == neg_inf())
-                                ? neg_inf() : v;
+                            const int key0 = mb * 32 + 8 * rg + 4 * half;
+                            const int64_t krow = k_row0 + key0;
+#pragma unroll
+                            for(int e = 0; e < 4; ++e)
+                            {
+                                // out-of-range keys of a ragged step are hidden
+                                // and their mask element is not touched
+                                float add = neg_inf();
+                                if(key0 + e < keys_here)
+                                {
+                                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                                    {
+                                        add = T::to_float(static_cast<const uint16_t *>(
+                                                    p.mask)[mask_row + krow + e]);
+                                    }
+                                    else
+                                    {
+                                        add = static_cast<const uint8_t *>(
+                                                p.mask)[mask_row + krow + e] != 0
+                                            ? 0.0f : neg_inf();
+                                    }
+                                }
+                                s[mb][4 * rg + e] = fmaf(add, inv_scale,
+                                        s[mb][4 * rg + e]);
+                            }
                         }
                     }
                 }
@@ -512,6 +628,12 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             }
             l_run += rs;
         }
+        // mask values of the next step (this step's have been consumed)
+        if(EXPLICIT && mask_wide && g + 1 < n_steps
+                && cur.rows_left - kKeys >= kKeys)
+        {
+            mask_fetch(cur.kb + 1);
+        }
         NNTILE_PHASE(2)
 
         // ---- O^T += V^T P^T ------------------------------------------------------
@@ -561,7 +683,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     {
         return;     // leave lse and A as they are
     }
-    const float to_ln = EXPLICIT ? 1.0f : p.scale;
+    const float to_ln = p.scale;
     const float lse_new = empty ? neg_inf() : m_run * to_ln + __logf(l_tot);
     float *lse_ptr = p.lse[qt] + (int64_t)b * q_len + my_q;
     const float lse_old = p.overwrite ? neg_inf() : *lse_ptr;
