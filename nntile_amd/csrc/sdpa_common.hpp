@@ -165,6 +165,23 @@ __device__ __forceinline__ float max_across_halves(float x)
     return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
+// (No inline assembly on values that an MFMA may have produced: the wait
+// states between an MFMA's write and a VALU read are only inserted for real
+// instructions, not for assembly text.)
+__device__ __forceinline__ float max3(float a, float b, float c)
+{
+    return fmaxf(fmaxf(a, b), c);
+}
+
+// max(m, x, value of x in lane ^ 32)
+__device__ __forceinline__ float max_with_other_half(float m, float x)
+{
+    typedef __attribute__((ext_vector_type(2))) uint32_t pair;
+    const uint32_t u = __float_as_uint(x);
+    const pair r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return max3(m, __uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 __device__ __forceinline__ float sum_across_halves(float x)
 {
     typedef __attribute__((ext_vector_type(2))) uint32_t pair;

@@ -73,16 +73,19 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     constexpr int LOADS = kKeys / ROWS_PER_LOAD;  // load instructions per K (or V) step
     constexpr int LOADS_PER_WAVE = LOADS / 4;
     constexpr int K_BYTES = kKeys * RB;
-    constexpr int BUF_BYTES = 2 * K_BYTES;  // K then V
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
-    static_assert(LOADS_PER_WAVE >= 1, "head size too small for this tiling");
+    static_assert(LOADS_PER_WAVE == 1 || LOADS_PER_WAVE == 2 || LOADS_PER_WAVE == 4,
+            "head size does not fit this tiling");
 
-    // Two separate arrays, not one: the compiler then knows that the loads
-    // streaming into one buffer cannot alias the reads of the other and does
-    // not make those reads wait for the loads.
-    __shared__ __attribute__((aligned(1024))) char lds_a[BUF_BYTES];
-    __shared__ __attribute__((aligned(1024))) char lds_b[BUF_BYTES];
+    // Separate arrays, not one: the compiler then knows that the loads
+    // streaming into one of them cannot alias the reads of the others and
+    // does not make those reads wait for the loads.  Key step g lives in
+    // lds_k[g % 2] and lds_v[g % 2].
+    __shared__ __attribute__((aligned(1024))) char lds_k0[K_BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_k1[K_BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_v0[K_BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_v1[K_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -184,18 +187,24 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // Load instruction `ld` fills rows [ld*ROWS_PER_LOAD, +ROWS_PER_LOAD): lane
     // L lands on row ld*ROWS_PER_LOAD + L/CPR, chunk position L%CPR, and so must
     // fetch the logical chunk that belongs there.
-    uint32_t k_goff[LOADS_PER_WAVE], v_goff[LOADS_PER_WAVE];
-    int ld_row[LOADS_PER_WAVE];
+    // (V: the swizzle repeats from one load instruction to the next, so its
+    // offsets are v_goff0 + i*1024 and go into the instructions' immediates,
+    // which advance the global and the LDS address alike)
+    uint32_t k_goff[LOADS_PER_WAVE], v_goff0 = 0;
+    int ld_row0 = 0;
     const int ld_cpos = lane % CPR;
 #pragma unroll
     for(int i = 0; i < LOADS_PER_WAVE; ++i)
     {
         const int ld = wave * LOADS_PER_WAVE + i;
         const int r = ld * ROWS_PER_LOAD + lane / CPR;
-        ld_row[i] = r;
         k_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ ((r / RPL) % CPR)) * 16);
-        v_goff[i] = (uint32_t)(r * RB
-                + (ld_cpos ^ (4 * ((r / RPL) % (CPR >= 4 ? CPR / 4 : 1)))) * 16);
+        if(i == 0)
+        {
+            ld_row0 = r;
+            v_goff0 = (uint32_t)(r * RB
+                    + (ld_cpos ^ (4 * ((r / RPL) % (CPR >= 4 ? CPR / 4 : 1)))) * 16);
+        }
     }
     // S operand: lane (col, half) reads row mb*32+col, logical chunk 2*ks+half.
     uint32_t k_raddr[2][KSTEPS];
@@ -227,7 +236,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         for(int db = 0; db < DBLOCKS; ++db)
         {
             const int c = 4 * db + 2 * dblk + (r4 >> 1);
-            v_raddr[db] = (uint32_t)(K_BYTES + r * RB + (c ^ swz) * 16
+            v_raddr[db] = (uint32_t)(r * RB + (c ^ swz) * 16
                     + 8 * (r4 & 1));
         }
     }
@@ -243,26 +252,23 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         return (int64_t)kvb * tile_rows(kt) * HEAD * 2;
     };
 
-    // Global -> LDS loads of one step into buffer `buf`.  Rows past the end of
-    // the tile are clamped to its last row: their scores are masked and their
-    // probabilities are exactly 0, so any finite stand-in value works.
-    auto fetch = [&](const StepCursor &cur, char *buf_base)
+    // Global -> LDS loads of the K (or V) rows of one step.  Rows past the end
+    // of the tile are clamped to its last row: their scores are masked and
+    // their probabilities are exactly 0, so any finite stand-in value works.
+    typedef const void __attribute__((address_space(1))) *gptr;
+    typedef void __attribute__((address_space(3))) *lptr;
+    auto fetch_k = [&](const StepCursor &cur, char *dst_base)
     {
         // (wave index made visibly uniform: the LDS target goes into M0)
-        char *kdst = buf_base
+        char *dst = dst_base
             + __builtin_amdgcn_readfirstlane(wave) * LOADS_PER_WAVE * 1024;
-        char *vdst = kdst + K_BYTES;
-        typedef const void __attribute__((address_space(1))) *gptr;
-        typedef void __attribute__((address_space(3))) *lptr;
         if(cur.rows_left >= kKeys)
         {
 #pragma unroll
             for(int i = 0; i < LOADS_PER_WAVE; ++i)
             {
                 __builtin_amdgcn_global_load_lds((gptr)(cur.Kp + k_goff[i]),
-                        (lptr)(kdst + i * 1024), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((gptr)(cur.Vp + v_goff[i]),
-                        (lptr)(vdst + i * 1024), 16, 0, 0);
+                        (lptr)(dst + i * 1024), 16, 0, 0);
             }
         }
         else
@@ -272,13 +278,42 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             for(int i = 0; i < LOADS_PER_WAVE; ++i)
             {
                 // same chunk, clamped row
-                const uint32_t back = (uint32_t)(max(ld_row[i] - last, 0) * RB);
+                const uint32_t back = (uint32_t)(
+                        max(ld_row0 + i * ROWS_PER_LOAD - last, 0) * RB);
+                __builtin_amdgcn_global_load_lds((gptr)(cur.Kp + (k_goff[i] - back)),
+                        (lptr)(dst + i * 1024), 16, 0, 0);
+            }
+        }
+    };
+    auto fetch_v = [&](const StepCursor &cur, char *dst_base)
+    {
+        char *dst = dst_base
+            + __builtin_amdgcn_readfirstlane(wave) * LOADS_PER_WAVE * 1024;
+        if(cur.rows_left >= kKeys)
+        {
+            const char *src = cur.Vp + v_goff0;
+            __builtin_amdgcn_global_load_lds((gptr)src, (lptr)dst, 16, 0, 0);
+            if(LOADS_PER_WAVE > 1)
+            {
+                __builtin_amdgcn_global_load_lds((gptr)src, (lptr)dst, 16, 1024, 0);
+            }
+            if(LOADS_PER_WAVE > 2)
+            {
+                __builtin_amdgcn_global_load_lds((gptr)src, (lptr)dst, 16, 2048, 0);
+                __builtin_amdgcn_global_load_lds((gptr)src, (lptr)dst, 16, 3072, 0);
+            }
+        }
+        else
+        {
+            const int last = cur.rows_left - 1;
+#pragma unroll
+            for(int i = 0; i < LOADS_PER_WAVE; ++i)
+            {
+                const uint32_t back = (uint32_t)(
+                        max(ld_row0 + i * ROWS_PER_LOAD - last, 0) * RB);
                 __builtin_amdgcn_global_load_lds(
-                        (gptr)(cur.Kp + (k_goff[i] - back)),
-                        (lptr)(kdst + i * 1024), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds(
-                        (gptr)(cur.Vp + (v_goff[i] - back)),
-                        (lptr)(vdst + i * 1024), 16, 0, 0);
+                        (gptr)(cur.Vp + (v_goff0 + i * 1024 - back)),
+                        (lptr)(dst + i * 1024), 16, 0, 0);
             }
         }
     };
@@ -410,10 +445,29 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         static_cast<const char *>(p.K[0]) + slab(0),
         static_cast<const char *>(p.V[0]) + slab(0)};     // step being computed
     StepCursor nxt = cur;                        // step being fetched
+    // Leading steps that are complete (64 keys) and visible to every query of
+    // the workgroup need no mask at all; they run in the pipelined loop below.
+    int n_fast = 0;
+    if(!EXPLICIT)
+    {
+        const int n_full = (p.n_kv_tiles == 1 || k_tile % kKeys == 0)
+            ? k_seq / kKeys : k_tile / kKeys;
+        n_fast = min(n_steps, n_full);
+        if(MODE == NNTILE_HIP_MASK_CAUSAL)
+        {
+            n_fast = min(n_fast, max(rel0 + 1, 0) / kKeys);
+        }
+        n_fast = n_fast >= 2 ? n_fast : 0;
+    }
     if(n_steps > 0)
     {
-        fetch(nxt, lds_a);
+        fetch_k(nxt, lds_k0);
+        fetch_v(nxt, lds_v0);
         advance(nxt);
+        if(n_fast > 0)
+        {
+            fetch_k(nxt, lds_k1);       // the pipelined loop keeps K two steps ahead
+        }
         if(mask_wide && cur.rows_left >= kKeys)
         {
             mask_fetch(0);
@@ -424,10 +478,11 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
 
     // One key step on LDS buffer BUF (a compile-time constant, so that every
     // LDS address is a fixed register plus an immediate).
-    auto step = [&](int g, auto buf_tag)
+    auto step = [&](int g, auto buf_tag) __attribute__((always_inline))
     {
         constexpr int BUF = decltype(buf_tag)::value;
-        const char *Ks = BUF ? lds_b : lds_a;
+        const char *Ks = BUF ? lds_k1 : lds_k0;
+        const char *Vs = BUF ? lds_v1 : lds_v0;
         const int k_row0 = cur.kb * kKeys;                   // within the tile
         const int kg0 = cur.kt * k_tile + k_row0;            // key row overall
         const int keys_here = min(kKeys, cur.rows_left);
@@ -448,7 +503,8 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         NNTILE_PHASE(0)
         if(g + 1 < n_steps)
         {
-            fetch(nxt, BUF ? lds_a : lds_b);
+            fetch_k(nxt, BUF ? lds_k0 : lds_k1);
+            fetch_v(nxt, BUF ? lds_v0 : lds_v1);
             advance(nxt);
         }
 
@@ -649,7 +705,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
 #pragma unroll
                 for(int db = 0; db < DBLOCKS; ++db)
                 {
-                    const char *src = Ks + v_raddr[db] + (16 * t) * RB;
+                    const char *src = Vs + v_raddr[db] + (16 * t) * RB;
                     const u32x2 lo = lds_read_tr16(src);
                     const u32x2 hi = lds_read_tr16(src + 8 * RB);
                     const u32x4 araw = {lo[0], lo[1], hi[0], hi[1]};
@@ -666,12 +722,292 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         NNTILE_PHASE(4)
     };
 
-    for(int g = 0; g < n_steps; g += 2)
+    // ---- pipelined loop over the unmasked steps ---------------------------------
+    // A step is two sub-blocks of 32 keys.  While the softmax of sub-block j
+    // runs on the vector ALU, the matrix unit computes the scores of sub-block
+    // j+1 and adds sub-block j-1 to the output: the three are independent, and
+    // a wavefront's MFMAs execute in the background of its own VALU work.  One
+    // MFMA and a slice of the softmax form a slot; scheduling barriers keep the
+    // compiler from regrouping the slots.  K is fetched two steps ahead and V
+    // one step ahead, with one workgroup barrier in the middle of each step.
+    int g_first = 0;        // first step of the general loop
+    if(n_fast > 0)
     {
-        step(g, std::integral_constant<int, 0>{});
-        if(g + 1 < n_steps)
+        constexpr int NSLOT = 2 * KSTEPS;       // KSTEPS score MFMAs + 2*DBLOCKS output MFMAs
+        constexpr int NITEM = 28;               // softmax work items of a sub-block
+        constexpr int AHEAD = 3;                // LDS operands are read this many slots early
+        f32x16 zero16;
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
         {
-            step(g + 1, std::integral_constant<int, 1>{});
+            zero16[r] = 0.0f;
+        }
+        f32x16 sa = zero16, sb = zero16;        // scores of the current / next sub-block
+        uint32_t pp[8];                         // probabilities (packed pairs) of a sub-block
+#pragma unroll
+        for(int i = 0; i < 8; ++i)
+        {
+            pp[i] = 0u;
+        }
+        float alpha_pending = 1.0f;             // rescale of O that the last softmax asked for
+        StepCursor c1 = nxt;                    // step g+1: its V is fetched during step g
+        StepCursor c2 = nxt;                    // step g+2: its K is fetched during step g
+        advance(c2);
+
+        // MFMA of slot sl.  Order: the output MFMAs of the first 16 keys, then
+        // those of the second 16 keys alternating with score MFMAs, then the
+        // remaining score MFMAs.  pp holds the probabilities of sub-block j-1
+        // on entry and is overwritten with those of sub-block j as the softmax
+        // proceeds; in this order every old value is consumed before its slot
+        // in pp is written, and the scores are complete a slot before the
+        // next body needs them.
+        //   kind 0: output MFMA number idx (16-key half idx / DBLOCKS, block idx % DBLOCKS)
+        //   kind 1: score MFMA number idx (head values 16*idx .. +15)
+        auto slot_kind = [](int sl) -> int
+        {
+            if(sl < DBLOCKS) { return 0; }
+            if(sl < 3 * DBLOCKS) { return (sl - DBLOCKS) & 1; }
+            return 1;
+        };
+        auto slot_idx = [](int sl) -> int
+        {
+            if(sl < DBLOCKS) { return sl; }
+            if(sl < 3 * DBLOCKS) { return ((sl - DBLOCKS) & 1) ? (sl - DBLOCKS) / 2
+                : DBLOCKS + (sl - DBLOCKS) / 2; }
+            return sl - 2 * DBLOCKS;
+        };
+
+        // One sub-block body.  s_cur: scores to turn into probabilities;
+        // s_nxt: scores to compute from the 32 keys of block kh of buffer Kb;
+        // the probabilities in pp multiply the keys 32*vh.. of buffer Vb.
+        auto body = [&](auto do_s_tag, auto do_pv_tag, auto do_sm_tag, const char *Kb, int kh,
+                const char *Vb, int vh, const f32x16 &s_cur, f32x16 &s_nxt)
+            __attribute__((always_inline))
+        {
+            constexpr bool DO_S = decltype(do_s_tag)::value;
+            constexpr bool DO_PV = decltype(do_pv_tag)::value;
+            constexpr bool DO_SM = decltype(do_sm_tag)::value;
+            // the rescale that the previous softmax decided on (rare after the
+            // first steps): O holds every sub-block up to j-2 at this point
+            if(__builtin_amdgcn_ballot_w64(alpha_pending != 1.0f) != 0)
+            {
+#pragma unroll
+                for(int db = 0; db < DBLOCKS; ++db)
+                {
+#pragma unroll
+                    for(int r = 0; r < 16; ++r)
+                    {
+                        o[db][r] *= alpha_pending;
+                    }
+                }
+            }
+            vec8 opnd[NSLOT];       // LDS operand of each slot's MFMA
+            auto read_operand = [&](int sl) __attribute__((always_inline))
+            {
+                if(sl >= NSLOT)
+                {
+                    return;
+                }
+                const int i = slot_idx(sl);
+                if(slot_kind(sl) == 1)
+                {
+                    if(DO_S)
+                    {
+                        opnd[sl] = *reinterpret_cast<const vec8 *>(Kb + k_raddr[0][i]
+                                + kh * 32 * RB);
+                    }
+                }
+                else if(DO_PV)
+                {
+                    const int t = 2 * vh + i / DBLOCKS, db = i % DBLOCKS;
+                    const char *src = Vb + v_raddr[db] + (16 * t) * RB;
+                    const u32x2 lo = lds_read_tr16(src);
+                    const u32x2 hi = lds_read_tr16(src + 8 * RB);
+                    const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
+                    opnd[sl] = __builtin_bit_cast(vec8, raw);
+                }
+            };
+            float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f, mx = 0.0f, mc = 0.0f;
+            float m_new = 0.0f, alpha = 1.0f, rs = 0.0f;
+            float pe[2] = {0.0f, 0.0f};
+            auto item = [&](int it) __attribute__((always_inline))
+            {
+                if(it == 0)
+                {
+                    t0 = max3(s_cur[0], s_cur[1], s_cur[2]);
+                    t1 = max3(s_cur[3], s_cur[4], s_cur[5]);
+                    t2 = max3(s_cur[6], s_cur[7], s_cur[8]);
+                    t3 = max3(s_cur[9], s_cur[10], s_cur[11]);
+                }
+                else if(it == 1)
+                {
+                    const float t4 = max3(s_cur[12], s_cur[13], s_cur[14]);
+                    t0 = max3(t0, t1, t2);
+                    t3 = max3(t3, t4, s_cur[15]);
+                }
+                else if(it == 2)
+                {
+                    mx = fmaxf(t0, t3);
+                    m_new = max_with_other_half(m_run, mx);
+                }
+                else if(it == 3)
+                {
+                    // every key of these steps is visible: m_new is finite
+                    alpha = fast_exp2((m_run - m_new) * c);
+                    mc = m_new * c;
+                    l_run *= alpha;
+                    m_run = m_new;
+                }
+                else
+                {
+                    const int q = it - 4, k = q / 3, r = q % 3;
+                    if(r < 2)
+                    {
+                        pe[r] = fast_exp2(fmaf(s_cur[2 * k + r], c, -mc));
+                    }
+                    else
+                    {
+                        pp[k] = T::pack2(pe[0], pe[1]);
+                        rs = T::add_pair(pp[k], rs);
+                    }
+                }
+            };
+#pragma unroll
+            for(int sl = 0; sl < AHEAD; ++sl)
+            {
+                read_operand(sl);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for(int sl = 0; sl < NSLOT; ++sl)
+            {
+                read_operand(sl + AHEAD);
+                const int i = slot_idx(sl);
+                if(slot_kind(sl) == 1)
+                {
+                    if(DO_S)
+                    {
+                        s_nxt = T::mfma(opnd[sl], qf[i], i == 0 ? zero16 : s_nxt);
+                    }
+                }
+                else if(DO_PV)
+                {
+                    const int t = i / DBLOCKS, db = i % DBLOCKS;
+                    const u32x4 praw = {pp[4 * t], pp[4 * t + 1], pp[4 * t + 2],
+                        pp[4 * t + 3]};
+                    o[db] = T::mfma(opnd[sl], __builtin_bit_cast(vec8, praw), o[db]);
+                }
+                // the softmax items are spread over the slots 1 .. NSLOT-1
+                if(DO_SM && sl >= 1)
+                {
+#pragma unroll
+                    for(int it = (sl - 1) * NITEM / (NSLOT - 1);
+                            it < sl * NITEM / (NSLOT - 1); ++it)
+                    {
+                        item(it);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            l_run += rs;
+            alpha_pending = alpha;
+            // Everything above belongs to this body: without this the compiler
+            // sinks the tail of the softmax, whose results are first used by
+            // the next body, behind that body's rescale branch and out of the
+            // shadow of the MFMAs.
+            asm volatile("" : "+v"(pp[0]), "+v"(pp[1]), "+v"(pp[2]), "+v"(pp[3]),
+                    "+v"(pp[4]), "+v"(pp[5]), "+v"(pp[6]), "+v"(pp[7]),
+                    "+v"(l_run), "+v"(alpha_pending), "+v"(m_run));
+            if(DO_S)
+            {
+                asm volatile("" : "+v"(s_nxt));
+            }
+        };
+        typedef std::integral_constant<bool, true> Yes;
+        typedef std::integral_constant<bool, false> No;
+
+        // scores of sub-block (0, 0)
+#pragma unroll
+        for(int ks = 0; ks < KSTEPS; ++ks)
+        {
+            const vec8 a = *reinterpret_cast<const vec8 *>(lds_k0 + k_raddr[0][ks]);
+            sa = T::mfma(a, qf[ks], ks == 0 ? zero16 : sa);
+        }
+
+        // The middle of step g on the buffers of parity BUF: K(g+1) and V(g)
+        // have landed for everyone (they were requested a step ago) and nobody
+        // reads K(g) or V(g-1) any more, so their buffers take K(g+2), V(g+1).
+        auto mid_step = [&](int g, auto buf_tag) __attribute__((always_inline))
+        {
+            constexpr int BUF = decltype(buf_tag)::value;
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if(g + 2 < n_steps)
+            {
+                fetch_k(c2, BUF ? lds_k1 : lds_k0);
+            }
+            if(g + 1 < n_steps)
+            {
+                fetch_v(c1, BUF ? lds_v0 : lds_v1);
+            }
+            c1 = c2;
+            advance(c2);
+        };
+        // One step on the buffers of parity BUF: sub-block (g, 0) with the
+        // scores of (g, 1) and the output of (g-1, 1), then sub-block (g, 1)
+        // with the scores of (g+1, 0) and the output of (g, 0).  (After the
+        // last pipelined step the scores computed ahead are not used.)
+        auto fast_step = [&](int g, auto buf_tag) __attribute__((always_inline))
+        {
+            constexpr int BUF = decltype(buf_tag)::value;
+            body(Yes{}, Yes{}, Yes{}, BUF ? lds_k1 : lds_k0, 1, BUF ? lds_v0 : lds_v1, 1, sa, sb);
+            mid_step(g, buf_tag);
+            body(Yes{}, Yes{}, Yes{}, BUF ? lds_k0 : lds_k1, 0, BUF ? lds_v1 : lds_v0, 0, sb, sa);
+            advance(cur);
+        };
+        // step 0: there is no output yet in its first half
+        body(Yes{}, No{}, Yes{}, lds_k0, 1, lds_v1, 1, sa, sb);
+        mid_step(0, std::integral_constant<int, 0>{});
+        body(Yes{}, Yes{}, Yes{}, lds_k1, 0, lds_v0, 0, sb, sa);
+        advance(cur);
+        for(int g = 1; g < n_fast; g += 2)
+        {
+            fast_step(g, std::integral_constant<int, 1>{});
+            if(g + 1 < n_fast)
+            {
+                fast_step(g + 1, std::integral_constant<int, 0>{});
+            }
+        }
+        // drain: the output of the last sub-block
+        if((n_fast - 1) & 1)
+        {
+            body(No{}, Yes{}, No{}, lds_k0, 0, lds_v1, 1, sb, sa);
+        }
+        else
+        {
+            body(No{}, Yes{}, No{}, lds_k0, 0, lds_v0, 1, sb, sa);
+        }
+        g_first = n_fast;
+        nxt = c1;
+        // the general loop expects step g_first complete in its buffers
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+
+    {
+        int g = g_first;
+        if(g < n_steps && (g & 1))
+        {
+            step(g, std::integral_constant<int, 1>{});
+            g += 1;
+        }
+        for(; g < n_steps; g += 2)
+        {
+            step(g, std::integral_constant<int, 0>{});
+            if(g + 1 < n_steps)
+            {
+                step(g + 1, std::integral_constant<int, 1>{});
+            }
         }
     }
     NNTILE_PHASE_DUMP()
