@@ -31,8 +31,8 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # WRITE_SIZE x 1.000, the factors a 1 GiB device copy calibrates); the runs
 # and their figures are in profiles/sdpa_*_kernel_cfg*.txt.  They are
 # properties of the kernel and the workload, not of one timing run.
-TRAFFIC_PREFILL_CFG3 = 177748615      # Q+K+V 96 MiB in, A+lse 32.5 MiB out, K/V re-read 1.6x
-TRAFFIC_DECODE_CFG4 = 312418907       # main kernel + merge kernel, incl. 16.25 MiB of partials
+TRAFFIC_PREFILL_CFG3 = 176170234      # Q+K+V 96 MiB in, A+lse 32.5 MiB out, K/V re-read 1.6x
+TRAFFIC_DECODE_CFG4 = 312419785       # main kernel + merge kernel, incl. 16.25 MiB of partials
 
 
 def time_steps(step, steps, warmup):
@@ -52,6 +52,10 @@ def time_steps(step, steps, warmup):
     for _ in range(steps):
         step()
     b.record()
+    # spin on the closing event first: a blocking synchronize alone adds its
+    # wake-up latency (of the order of a millisecond here) to the timed region
+    while not b.query():
+        pass
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
     dev = a.elapsed_time(b) / steps
@@ -194,8 +198,8 @@ def cpu_baseline(cfg, target_seconds=15.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
                     help="run only this leg: prefill | decode | per_task | extras | copy (for profiling)")
