@@ -297,3 +297,45 @@ def test_overwrite_flag_decode(oracle):
     torch.cuda.synchronize()
     assert H.rel_fro(H.to_np(A), want) < 1e-2
     assert H.rel_fro(H.to_np(lse), want_lse) < 1e-2
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("head", [32, 64, 128])
+@pytest.mark.parametrize("q_seq,k_seq,k_tile", [(192, 448, 448), (130, 397, 397), (256, 576, 192),
+                                                (96, 480, 160), (128, 128, 128)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_unmasked_steps_loop(oracle, dtype, head, q_seq, k_seq, k_tile, causal):
+    """Shapes chosen for the pipelined loop over complete, fully visible key
+    steps: odd and even numbers of such steps, a ragged last step, key tiles
+    that are and are not multiples of the step, every head size, GQA, and a
+    running pair that is merged into rather than overwritten."""
+    print("case", dtype, head, q_seq, k_seq, k_tile, causal, flush=True)
+    n_batch, group, n_kv = 2, 2, 2
+    batch = n_batch * group * n_kv
+    offset = k_seq - q_seq
+    (Q, K, V), f32 = H.make_qkv(23, batch, q_seq, k_seq, head, dtype, kv_batch=n_batch * n_kv)
+    mask = synth.causal_mask(q_seq, k_seq, offset) if causal else None
+    want, want_lse = _oracle(oracle, f32, mask, k_tile=k_tile, n_batch=n_batch, kv_repeat=group)
+    Kt = [K[:, s:s + k_tile].contiguous().cuda() for s in range(0, k_seq, k_tile)]
+    Vt = [V[:, s:s + k_tile].contiguous().cuda() for s in range(0, k_seq, k_tile)]
+    mode = hip_sdpa.MASK_CAUSAL if causal else hip_sdpa.MASK_NONE
+    lse, A = H.fresh_outputs(batch, q_seq, head, dtype)
+    hip_sdpa.sdpa_fwd_grid(Kt, [Q.cuda()], [lse], Vt, [A], q_seq, k_seq, q_seq, k_tile, mode,
+                           n_batch=n_batch, kv_group=group, causal_offset=offset)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+    # the same through per-tile calls that merge into the running pair, and twice
+    # in a row: bit-identical results (no dependence on timing)
+    runs = []
+    for _ in range(2):
+        lse2, A2 = H.fresh_outputs(batch, q_seq, head, dtype)
+        for i, (kt, vt) in enumerate(zip(Kt, Vt)):
+            hip_sdpa.sdpa_fwd_tile(kt, Q.cuda(), None, lse2, vt, A2, mode, n_batch=n_batch,
+                                   kv_group=group, k_pos0=i * k_tile, causal_offset=offset)
+        torch.cuda.synchronize()
+        runs.append((lse2, A2))
+    assert torch.equal(runs[0][0], runs[1][0])
+    assert torch.equal(runs[0][1].view(torch.int16), runs[1][1].view(torch.int16))
+    assert H.rel_fro(H.to_np(runs[0][1]), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(runs[0][0]), want_lse) < H.TOL[dtype]
