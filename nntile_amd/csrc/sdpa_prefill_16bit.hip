@@ -734,7 +734,8 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     if(n_fast > 0)
     {
         constexpr int NSLOT = 2 * KSTEPS;       // KSTEPS score MFMAs + 2*DBLOCKS output MFMAs
-        constexpr int NITEM = 28;               // softmax work items of a sub-block
+        constexpr int NITEM = 24;               // softmax work items of a sub-block
+        constexpr float kLazyLimit = 16384.0f;  // largest row sum of a sub-block taken without a new maximum
         constexpr int AHEAD = 3;                // LDS operands are read this many slots early
         f32x16 zero16;
 #pragma unroll
@@ -802,6 +803,14 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 }
             }
             vec8 opnd[NSLOT];       // LDS operand of each slot's MFMA
+            // the probabilities of sub-block j-1, as they are on entry: pp is
+            // rewritten with those of sub-block j while the output MFMAs run
+            uint32_t pin[8];
+#pragma unroll
+            for(int i = 0; i < 8; ++i)
+            {
+                pin[i] = pp[i];
+            }
             auto read_operand = [&](int sl) __attribute__((always_inline))
             {
                 if(sl >= NSLOT)
@@ -827,49 +836,27 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                     opnd[sl] = __builtin_bit_cast(vec8, raw);
                 }
             };
-            float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f, mx = 0.0f, mc = 0.0f;
-            float m_new = 0.0f, alpha = 1.0f, rs = 0.0f;
+            // Lazy maximum: the probabilities are taken relative to the running
+            // maximum as it stands, without looking at this sub-block's scores
+            // first (softmax does not depend on the reference point, only
+            // overflow does).  The row sums, which are needed anyway, tell
+            // afterwards whether that was safe; if not (first sub-block, or
+            // scores far above everything seen so far) the sub-block is redone
+            // with a new maximum at the end of the body.
+            const float mc = m_run * c;
+            float rs = 0.0f;
             float pe[2] = {0.0f, 0.0f};
             auto item = [&](int it) __attribute__((always_inline))
             {
-                if(it == 0)
+                const int k = it / 3, r = it % 3;
+                if(r < 2)
                 {
-                    t0 = max3(s_cur[0], s_cur[1], s_cur[2]);
-                    t1 = max3(s_cur[3], s_cur[4], s_cur[5]);
-                    t2 = max3(s_cur[6], s_cur[7], s_cur[8]);
-                    t3 = max3(s_cur[9], s_cur[10], s_cur[11]);
-                }
-                else if(it == 1)
-                {
-                    const float t4 = max3(s_cur[12], s_cur[13], s_cur[14]);
-                    t0 = max3(t0, t1, t2);
-                    t3 = max3(t3, t4, s_cur[15]);
-                }
-                else if(it == 2)
-                {
-                    mx = fmaxf(t0, t3);
-                    m_new = max_with_other_half(m_run, mx);
-                }
-                else if(it == 3)
-                {
-                    // every key of these steps is visible: m_new is finite
-                    alpha = fast_exp2((m_run - m_new) * c);
-                    mc = m_new * c;
-                    l_run *= alpha;
-                    m_run = m_new;
+                    pe[r] = fast_exp2(fmaf(s_cur[2 * k + r], c, -mc));
                 }
                 else
                 {
-                    const int q = it - 4, k = q / 3, r = q % 3;
-                    if(r < 2)
-                    {
-                        pe[r] = fast_exp2(fmaf(s_cur[2 * k + r], c, -mc));
-                    }
-                    else
-                    {
-                        pp[k] = T::pack2(pe[0], pe[1]);
-                        rs = T::add_pair(pp[k], rs);
-                    }
+                    pp[k] = T::pack2(pe[0], pe[1]);
+                    rs = T::add_pair(pp[k], rs);
                 }
             };
 #pragma unroll
@@ -893,8 +880,8 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 else if(DO_PV)
                 {
                     const int t = i / DBLOCKS, db = i % DBLOCKS;
-                    const u32x4 praw = {pp[4 * t], pp[4 * t + 1], pp[4 * t + 2],
-                        pp[4 * t + 3]};
+                    const u32x4 praw = {pin[4 * t], pin[4 * t + 1], pin[4 * t + 2],
+                        pin[4 * t + 3]};
                     o[db] = T::mfma(opnd[sl], __builtin_bit_cast(vec8, praw), o[db]);
                 }
                 // the softmax items are spread over the slots 1 .. NSLOT-1
@@ -909,8 +896,36 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            l_run += rs;
-            alpha_pending = alpha;
+            alpha_pending = 1.0f;
+            if(DO_SM)
+            {
+                if(__builtin_amdgcn_ballot_w64(!(rs <= kLazyLimit)) != 0)
+                {
+                    float mx = s_cur[0];
+#pragma unroll
+                    for(int r = 1; r < 16; ++r)
+                    {
+                        mx = fmaxf(mx, s_cur[r]);
+                    }
+                    // every key of these steps is visible: the new maximum is finite
+                    const float m_new = max_with_other_half(m_run, mx);
+                    const float alpha = fast_exp2((m_run - m_new) * c);
+                    const float mc_new = m_new * c;
+                    rs = 0.0f;
+#pragma unroll
+                    for(int k = 0; k < 8; ++k)
+                    {
+                        const float p0 = fast_exp2(fmaf(s_cur[2 * k], c, -mc_new));
+                        const float p1 = fast_exp2(fmaf(s_cur[2 * k + 1], c, -mc_new));
+                        pp[k] = T::pack2(p0, p1);
+                        rs = T::add_pair(pp[k], rs);
+                    }
+                    l_run *= alpha;
+                    m_run = m_new;
+                    alpha_pending = alpha;
+                }
+                l_run += rs;
+            }
             // Everything above belongs to this body: without this the compiler
             // sinks the tail of the softmax, whose results are first used by
             // the next body, behind that body's rescale branch and out of the
