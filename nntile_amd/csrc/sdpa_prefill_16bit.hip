@@ -755,27 +755,18 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         StepCursor c2 = nxt;                    // step g+2: its K is fetched during step g
         advance(c2);
 
-        // MFMA of slot sl.  Order: the output MFMAs of the first 16 keys, then
-        // those of the second 16 keys alternating with score MFMAs, then the
-        // remaining score MFMAs.  pp holds the probabilities of sub-block j-1
-        // on entry and is overwritten with those of sub-block j as the softmax
-        // proceeds; in this order every old value is consumed before its slot
-        // in pp is written, and the scores are complete a slot before the
-        // next body needs them.
+        // MFMA of slot sl.  Order: first the score MFMAs (one accumulator
+        // chain, which costs nothing extra), then the output MFMAs: the scores
+        // are complete half a body before the next body's softmax needs them.
         //   kind 0: output MFMA number idx (16-key half idx / DBLOCKS, block idx % DBLOCKS)
         //   kind 1: score MFMA number idx (head values 16*idx .. +15)
         auto slot_kind = [](int sl) -> int
         {
-            if(sl < DBLOCKS) { return 0; }
-            if(sl < 3 * DBLOCKS) { return (sl - DBLOCKS) & 1; }
-            return 1;
+            return sl < KSTEPS ? 1 : 0;
         };
         auto slot_idx = [](int sl) -> int
         {
-            if(sl < DBLOCKS) { return sl; }
-            if(sl < 3 * DBLOCKS) { return ((sl - DBLOCKS) & 1) ? (sl - DBLOCKS) / 2
-                : DBLOCKS + (sl - DBLOCKS) / 2; }
-            return sl - 2 * DBLOCKS;
+            return sl < KSTEPS ? sl : sl - KSTEPS;
         };
 
         // One sub-block body.  s_cur: scores to turn into probabilities;
