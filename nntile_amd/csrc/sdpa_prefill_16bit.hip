@@ -751,6 +751,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             pp[i] = 0u;
         }
         float alpha_pending = 1.0f;             // rescale of O that the last softmax asked for
+        bool rescale_pending = false;           // ... if it asked for one (the same for the whole wavefront)
         StepCursor c1 = nxt;                    // step g+1: its V is fetched during step g
         StepCursor c2 = nxt;                    // step g+2: its K is fetched during step g
         advance(c2);
@@ -781,7 +782,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             constexpr bool DO_SM = decltype(do_sm_tag)::value;
             // the rescale that the previous softmax decided on (rare after the
             // first steps): O holds every sub-block up to j-2 at this point
-            if(__builtin_amdgcn_ballot_w64(alpha_pending != 1.0f) != 0)
+            if(rescale_pending)
             {
 #pragma unroll
                 for(int db = 0; db < DBLOCKS; ++db)
@@ -887,7 +888,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            alpha_pending = 1.0f;
+            rescale_pending = false;
             if(DO_SM)
             {
                 if(__builtin_amdgcn_ballot_w64(!(rs <= kLazyLimit)) != 0)
@@ -914,6 +915,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                     l_run *= alpha;
                     m_run = m_new;
                     alpha_pending = alpha;
+                    rescale_pending = true;
                 }
                 l_run += rs;
             }
@@ -923,7 +925,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             // shadow of the MFMAs.
             asm volatile("" : "+v"(pp[0]), "+v"(pp[1]), "+v"(pp[2]), "+v"(pp[3]),
                     "+v"(pp[4]), "+v"(pp[5]), "+v"(pp[6]), "+v"(pp[7]),
-                    "+v"(l_run), "+v"(alpha_pending), "+v"(m_run));
+                    "+v"(l_run), "+v"(m_run));
             if(DO_S)
             {
                 asm volatile("" : "+v"(s_nxt));
