@@ -494,25 +494,78 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
     typedef __attribute__((ext_vector_type(2))) float f32x2;
     // The loads of up to 8 splits are issued together (indices past the last
     // split are clamped and get weight 0): the latency of the partials is
-    // paid once per 8 splits, not once per split.
+    // paid once per 8 splits, not once per split; with at most 8 splits the
+    // maxima and the values travel in the same round trip.
+    const int64_t row = qb * p.q_seq + tok;
+    uint16_t *Adst = static_cast<uint16_t *>(p.A) + row * HEAD + d4;
     float top = neg_inf();
-    for(int s0 = 0; s0 < p.n_splits; s0 += 8)
+    float l = 0.0f;
+    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto load8 = [&](int s0, f32x2 (&ml)[8], f32x4 (&v)[8])
     {
-        float m[8];
 #pragma unroll
         for(int j = 0; j < 8; ++j)
         {
             const int sidx = min(s0 + j, last_split);
-            m[j] = p.part_ml[2 * (base + (int64_t)sidx * p.rows)];
+            const int64_t prow = base + (int64_t)sidx * p.rows;
+            ml[j] = *reinterpret_cast<const f32x2 *>(p.part_ml + 2 * prow);
+            v[j] = *reinterpret_cast<const f32x4 *>(p.part_o + prow * HEAD + d4);
         }
+    };
+    auto add8 = [&](int s0, const f32x2 (&ml)[8], const f32x4 (&v)[8])
+    {
 #pragma unroll
         for(int j = 0; j < 8; ++j)
         {
-            top = fmaxf(top, m[j]);
+            const bool live = (s0 + j <= last_split) && (ml[j][0] != neg_inf());
+            const float w = live ? __expf(ml[j][0] - top) : 0.0f;
+            l += w * ml[j][1];
+            acc += w * v[j];
+        }
+    };
+    if(p.n_splits <= 8)
+    {
+        f32x2 ml[8];
+        f32x4 v[8];
+        load8(0, ml, v);
+#pragma unroll
+        for(int j = 0; j < 8; ++j)
+        {
+            top = fmaxf(top, ml[j][0]);
+        }
+        if(top != neg_inf())
+        {
+            add8(0, ml, v);
         }
     }
-    const int64_t row = qb * p.q_seq + tok;
-    uint16_t *Adst = static_cast<uint16_t *>(p.A) + row * HEAD + d4;
+    else
+    {
+        for(int s0 = 0; s0 < p.n_splits; s0 += 8)
+        {
+            float m[8];
+#pragma unroll
+            for(int j = 0; j < 8; ++j)
+            {
+                const int sidx = min(s0 + j, last_split);
+                m[j] = p.part_ml[2 * (base + (int64_t)sidx * p.rows)];
+            }
+#pragma unroll
+            for(int j = 0; j < 8; ++j)
+            {
+                top = fmaxf(top, m[j]);
+            }
+        }
+        if(top != neg_inf())
+        {
+            for(int s0 = 0; s0 < p.n_splits; s0 += 8)
+            {
+                f32x2 ml[8];
+                f32x4 v[8];
+                load8(s0, ml, v);
+                add8(s0, ml, v);
+            }
+        }
+    }
     if(top == neg_inf())
     {
         // no visible key at all: leave lse and A untouched, or write the
@@ -526,29 +579,6 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
             }
         }
         return;
-    }
-    float l = 0.0f;
-    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-    for(int s0 = 0; s0 < p.n_splits; s0 += 8)
-    {
-        f32x2 ml[8];
-        f32x4 v[8];
-#pragma unroll
-        for(int j = 0; j < 8; ++j)
-        {
-            const int sidx = min(s0 + j, last_split);
-            const int64_t prow = base + (int64_t)sidx * p.rows;
-            ml[j] = *reinterpret_cast<const f32x2 *>(p.part_ml + 2 * prow);
-            v[j] = *reinterpret_cast<const f32x4 *>(p.part_o + prow * HEAD + d4);
-        }
-#pragma unroll
-        for(int j = 0; j < 8; ++j)
-        {
-            const bool live = (s0 + j <= last_split) && (ml[j][0] != neg_inf());
-            const float w = live ? __expf(ml[j][0] - top) : 0.0f;
-            l += w * ml[j][1];
-            acc += w * v[j];
-        }
     }
     const float lse_new = top + __logf(l);
     const float lse_old = p.overwrite ? neg_inf() : p.lse[row];
