@@ -1023,27 +1023,69 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // ---- epilogue: normalise, merge into the running (lse, A) ----------------
     const float l_tot = sum_across_halves(l_run);
     const bool empty = !(l_tot > 0.0f);     // no visible key for this query
-    if(!q_ok || (empty && !p.overwrite))
-    {
-        return;     // leave lse and A as they are
-    }
+    // rows that are written; the others leave lse and A as they are
+    const bool live = q_ok && !(empty && !p.overwrite);
     const float to_ln = p.scale;
     const float lse_new = empty ? neg_inf() : m_run * to_ln + __logf(l_tot);
-    float *lse_ptr = p.lse[qt] + (int64_t)b * q_len + my_q;
-    const float lse_old = p.overwrite ? neg_inf() : *lse_ptr;
+    float *lse_ptr = p.lse[qt] + (int64_t)b * q_len + (q_ok ? my_q : 0);
+    const float lse_old = (p.overwrite || !live) ? neg_inf() : *lse_ptr;
     float w_old = 0.0f, w_new = 0.0f, lse_out = neg_inf();
-    if(!empty)
+    if(live && !empty)
     {
         merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
     }
-    if(half == 0)
+    if(live && half == 0)
     {
         *lse_ptr = lse_out;
     }
-    const float w_o = empty ? 0.0f : w_new / l_tot;
+    const float w_o = (empty || !live) ? 0.0f : w_new / l_tot;
+    // register r of block db holds head value  db*32 + 8*(r/4) + 4*half + r%4
+
+    if(__builtin_amdgcn_ballot_w64(live && w_old != 0.0f) == 0)
+    {
+        // Nothing of the old A is needed by this wavefront: its 32 rows go
+        // through LDS (its own quarter of the K buffers, which nobody reads
+        // any more after the last barrier) so that they leave as whole rows,
+        // 16 bytes per lane, instead of 8-byte pieces 2*HEAD bytes apart.
+        // 16-byte chunk c of row r sits at chunk position c ^ (r % CPR).
+        char *xch = (wave < 2 ? lds_k0 : lds_k1) + (wave & 1) * 32 * RB;
+#pragma unroll
+        for(int db = 0; db < DBLOCKS; ++db)
+        {
+#pragma unroll
+            for(int rg = 0; rg < 4; ++rg)
+            {
+                u32x2 out;
+                out[0] = T::pack2(o[db][4 * rg] * w_o, o[db][4 * rg + 1] * w_o);
+                out[1] = T::pack2(o[db][4 * rg + 2] * w_o, o[db][4 * rg + 3] * w_o);
+                const int cpos = (db * 4 + rg) ^ (col % CPR);
+                *reinterpret_cast<u32x2 *>(xch + col * RB + cpos * 16 + 8 * half) = out;
+            }
+        }
+        const uint64_t live_rows = __builtin_amdgcn_ballot_w64(live && half == 0);
+        constexpr int ROWS_PER_ST = 1024 / RB;      // rows one store instruction covers
+        char *Abase = static_cast<char *>(p.A[qt])
+            + ((int64_t)b * q_len + q_row0 + wave * 32) * RB;
+#pragma unroll
+        for(int i = 0; i < 32 / ROWS_PER_ST; ++i)
+        {
+            const int r = i * ROWS_PER_ST + lane / CPR;
+            const int c = lane % CPR;
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(
+                    xch + r * RB + (c ^ (r % CPR)) * 16);
+            if((live_rows >> r) & 1)
+            {
+                *reinterpret_cast<u32x4 *>(Abase + (int64_t)r * RB + c * 16) = v;
+            }
+        }
+        return;
+    }
+    if(!live)
+    {
+        return;
+    }
     uint16_t *Arow = static_cast<uint16_t *>(p.A[qt])
         + ((int64_t)b * q_len + my_q) * HEAD;
-    // register r of block db holds head value  db*32 + 8*(r/4) + 4*half + r%4
 #pragma unroll
     for(int db = 0; db < DBLOCKS; ++db)
     {
