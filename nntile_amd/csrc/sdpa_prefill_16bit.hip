@@ -39,6 +39,7 @@ namespace nntile_hip
 constexpr int kQRows = 128;     // queries per workgroup
 constexpr int kKeys = 64;       // keys per step
 constexpr int kThreads = 256;
+constexpr unsigned kCUsPerXCD = 32;   // MI355X: 256 CUs in 8 XCDs
 
 // Walks the key steps of all key tiles in order: tile kt, step kb within the
 // tile, rows left in the tile from this step on.
@@ -99,19 +100,35 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // K and V in that XCD's L2); in both layouts the query blocks are handed
     // out last-first, all batch entries of a block before the next block, so
     // that under a causal mask the longest workgroups start first.
+    //
+    // An XCD places its workgroups i = 0..31 on its 32 CUs and i = 32..63
+    // beside them, i+32 next to i.  With the plain longest-first order the CU
+    // that gets the longest workgroup also gets the longest of the second
+    // group, and the CUs end the first round with very different amounts of
+    // work done.  The second group is therefore dealt in reverse: the longest
+    // workgroup shares its CU with the shortest of the first 64.
     const int q_blocks = p.n_q_tiles * p.q_blocks_per_tile;
+    unsigned wg = blockIdx.x;
+    if(gridDim.x >= 8u * 2u * kCUsPerXCD)
+    {
+        const unsigned i = wg >> 3;
+        if(i >= kCUsPerXCD && i < 2u * kCUsPerXCD)
+        {
+            wg = ((3u * kCUsPerXCD - 1u - i) << 3) | (wg & 7u);
+        }
+    }
     int b, qblk;
     if(p.xcd_remap)
     {
         const int b_per_xcd = p.batch >> 3;
-        const int i = (int)(blockIdx.x >> 3);
-        b = (int)(blockIdx.x & 7) * b_per_xcd + i % b_per_xcd;
+        const int i = (int)(wg >> 3);
+        b = (int)(wg & 7) * b_per_xcd + i % b_per_xcd;
         qblk = q_blocks - 1 - i / b_per_xcd;
     }
     else
     {
-        b = (int)blockIdx.x % p.batch;
-        qblk = q_blocks - 1 - (int)blockIdx.x / p.batch;
+        b = (int)wg % p.batch;
+        qblk = q_blocks - 1 - (int)wg / p.batch;
     }
     const int qt = qblk / p.q_blocks_per_tile;
     const int qb = qblk % p.q_blocks_per_tile;
