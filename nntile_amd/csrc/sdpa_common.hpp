@@ -75,6 +75,55 @@ struct DecodeParams
     float scale;
 };
 
+// 16 bytes per lane from global memory straight into LDS: lane l reads
+// gaddr + OFF (its own address) and its bytes land at lds_dst + OFF + 16*l
+// (lds_dst is the same for the whole wavefront; it travels in M0).  Written
+// as assembly text on purpose: the compiler takes the builtin form for an
+// access that may touch both memories, and while one is in flight it turns
+// every wait for an LDS read into a wait for all LDS reads, which undoes
+// reading operands ahead of their use.  The caller waits (vmcnt) and
+// synchronises before anyone reads the target; nothing else here uses M0.
+template<int OFF, bool NT>
+__device__ __forceinline__ void load_to_lds16(const void *gaddr, char *lds_dst)
+{
+    typedef char __attribute__((address_space(3))) *lds_ptr;
+    const uint32_t base = (uint32_t)(uintptr_t)(lds_ptr)lds_dst;
+    if(NT)
+    {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "global_load_lds_dwordx4 %1, off offset:%2 nt"
+                :: "s"(base), "v"(gaddr), "n"(OFF) : "memory");
+    }
+    else
+    {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "global_load_lds_dwordx4 %1, off offset:%2"
+                :: "s"(base), "v"(gaddr), "n"(OFF) : "memory");
+    }
+}
+
+// The same with the address as a base common to the wavefront plus a 32-bit
+// offset per lane (no 64-bit address arithmetic on the vector unit).
+template<int OFF, bool NT>
+__device__ __forceinline__ void load_to_lds16(const void *gbase, uint32_t lane_off,
+        char *lds_dst)
+{
+    typedef char __attribute__((address_space(3))) *lds_ptr;
+    const uint32_t base = (uint32_t)(uintptr_t)(lds_ptr)lds_dst;
+    if(NT)
+    {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "global_load_lds_dwordx4 %1, %2 offset:%3 nt"
+                :: "s"(base), "v"(lane_off), "s"(gbase), "n"(OFF) : "memory");
+    }
+    else
+    {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "global_load_lds_dwordx4 %1, %2 offset:%3"
+                :: "s"(base), "v"(lane_off), "s"(gbase), "n"(OFF) : "memory");
+    }
+}
+
 __device__ __forceinline__ float fast_exp2(float x)
 {
     return __builtin_amdgcn_exp2f(x);

@@ -25,8 +25,8 @@ namespace nntile_hip
 {
 
 // Cache policy of the K/V stream: non-temporal (each byte is used once).
-#ifndef NNTILE_DMA_AUX
-#define NNTILE_DMA_AUX 2
+#ifndef NNTILE_DMA_NT
+#define NNTILE_DMA_NT true
 #endif
 
 constexpr int kDecThreads = 256;  // 4 wavefronts x 16 query rows
@@ -186,8 +186,6 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         }
     }
 
-    typedef const void __attribute__((address_space(1))) *gptr;
-    typedef void __attribute__((address_space(3))) *lptr;
 
     // Loads of key step `step` into ring slot `slot`; rows past the end of the
     // cache are clamped to its last row (their probabilities are exactly 0).
@@ -204,10 +202,8 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
 #pragma unroll
             for(int i = 0; i < LOADS_PER_WAVE; ++i)
             {
-                __builtin_amdgcn_global_load_lds((gptr)(Kp + k_goff[i]),
-                        (lptr)(kdst + i * 1024), 16, 0, NNTILE_DMA_AUX);
-                __builtin_amdgcn_global_load_lds((gptr)(Vp + v_goff[i]),
-                        (lptr)(vdst + i * 1024), 16, 0, NNTILE_DMA_AUX);
+                load_to_lds16<0, NNTILE_DMA_NT>(Kp + k_goff[i], kdst + i * 1024);
+                load_to_lds16<0, NNTILE_DMA_NT>(Vp + v_goff[i], vdst + i * 1024);
             }
         }
         else
@@ -217,10 +213,8 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
             for(int i = 0; i < LOADS_PER_WAVE; ++i)
             {
                 const uint32_t back = (uint32_t)(max(ld_row[i] - last, 0) * RB);
-                __builtin_amdgcn_global_load_lds((gptr)(Kp + (k_goff[i] - back)),
-                        (lptr)(kdst + i * 1024), 16, 0, NNTILE_DMA_AUX);
-                __builtin_amdgcn_global_load_lds((gptr)(Vp + (v_goff[i] - back)),
-                        (lptr)(vdst + i * 1024), 16, 0, NNTILE_DMA_AUX);
+                load_to_lds16<0, NNTILE_DMA_NT>(Kp + (k_goff[i] - back), kdst + i * 1024);
+                load_to_lds16<0, NNTILE_DMA_NT>(Vp + (v_goff[i] - back), vdst + i * 1024);
             }
         }
     };

@@ -33,6 +33,10 @@
 
 #include "sdpa_common.hpp"
 
+#ifndef NNTILE_PF_AHEAD
+#define NNTILE_PF_AHEAD 3
+#endif
+
 namespace nntile_hip
 {
 
@@ -272,8 +276,6 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // Global -> LDS loads of the K (or V) rows of one step.  Rows past the end
     // of the tile are clamped to its last row: their scores are masked and
     // their probabilities are exactly 0, so any finite stand-in value works.
-    typedef const void __attribute__((address_space(1))) *gptr;
-    typedef void __attribute__((address_space(3))) *lptr;
     auto fetch_k = [&](const StepCursor &cur, char *dst_base)
     {
         // (wave index made visibly uniform: the LDS target goes into M0)
@@ -284,8 +286,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
 #pragma unroll
             for(int i = 0; i < LOADS_PER_WAVE; ++i)
             {
-                __builtin_amdgcn_global_load_lds((gptr)(cur.Kp + k_goff[i]),
-                        (lptr)(dst + i * 1024), 16, 0, 0);
+                load_to_lds16<0, false>(cur.Kp + k_goff[i], dst + i * 1024);
             }
         }
         else
@@ -297,8 +298,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 // same chunk, clamped row
                 const uint32_t back = (uint32_t)(
                         max(ld_row0 + i * ROWS_PER_LOAD - last, 0) * RB);
-                __builtin_amdgcn_global_load_lds((gptr)(cur.Kp + (k_goff[i] - back)),
-                        (lptr)(dst + i * 1024), 16, 0, 0);
+                load_to_lds16<0, false>(cur.Kp + (k_goff[i] - back), dst + i * 1024);
             }
         }
     };
@@ -309,15 +309,15 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         if(cur.rows_left >= kKeys)
         {
             const char *src = cur.Vp + v_goff0;
-            __builtin_amdgcn_global_load_lds((gptr)src, (lptr)dst, 16, 0, 0);
+            load_to_lds16<0, false>(src, dst);
             if(LOADS_PER_WAVE > 1)
             {
-                __builtin_amdgcn_global_load_lds((gptr)src, (lptr)dst, 16, 1024, 0);
+                load_to_lds16<1024, false>(src, dst);
             }
             if(LOADS_PER_WAVE > 2)
             {
-                __builtin_amdgcn_global_load_lds((gptr)src, (lptr)dst, 16, 2048, 0);
-                __builtin_amdgcn_global_load_lds((gptr)src, (lptr)dst, 16, 3072, 0);
+                load_to_lds16<2048, false>(src, dst);
+                load_to_lds16<3072, false>(src, dst);
             }
         }
         else
@@ -328,9 +328,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             {
                 const uint32_t back = (uint32_t)(
                         max(ld_row0 + i * ROWS_PER_LOAD - last, 0) * RB);
-                __builtin_amdgcn_global_load_lds(
-                        (gptr)(cur.Vp + (v_goff0 + i * 1024 - back)),
-                        (lptr)(dst + i * 1024), 16, 0, 0);
+                load_to_lds16<0, false>(cur.Vp + (v_goff0 + i * 1024 - back), dst + i * 1024);
             }
         }
     };
@@ -465,11 +463,13 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // Leading steps that are complete (64 keys) and visible to every query of
     // the workgroup need no mask at all; they run in the pipelined loop below.
     int n_fast = 0;
+    int n_spread = 0;       // leading steps that exist and are complete
     if(!EXPLICIT)
     {
         const int n_full = (p.n_kv_tiles == 1 || k_tile % kKeys == 0)
             ? k_seq / kKeys : k_tile / kKeys;
         n_fast = min(n_steps, n_full);
+        n_spread = n_fast;
         if(MODE == NNTILE_HIP_MASK_CAUSAL)
         {
             n_fast = min(n_fast, max(rel0 + 1, 0) / kKeys);
@@ -753,7 +753,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         constexpr int NSLOT = 2 * KSTEPS;       // KSTEPS score MFMAs + 2*DBLOCKS output MFMAs
         constexpr int NITEM = 24;               // softmax work items of a sub-block
         constexpr float kLazyLimit = 16384.0f;  // largest row sum of a sub-block taken without a new maximum
-        constexpr int AHEAD = 3;                // LDS operands are read this many slots early
+        constexpr int AHEAD = NNTILE_PF_AHEAD;  // LDS operands are read this many slots early
         f32x16 zero16;
 #pragma unroll
         for(int r = 0; r < 16; ++r)
@@ -790,13 +790,38 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         // One sub-block body.  s_cur: scores to turn into probabilities;
         // s_nxt: scores to compute from the 32 keys of block kh of buffer Kb;
         // the probabilities in pp multiply the keys 32*vh.. of buffer Vb.
-        auto body = [&](auto do_s_tag, auto do_pv_tag, auto do_sm_tag, const char *Kb, int kh,
-                const char *Vb, int vh, const f32x16 &s_cur, f32x16 &s_nxt)
+        // With DO_FETCH the loads of K(c2) into kdst and V(c1) into vdst (both
+        // full steps) are issued one every second slot: issued together after
+        // the barrier they queue up behind each other - the loads of a step
+        // take the CU's memory path about 500 cycles - and the wavefront
+        // stands still until its last one is accepted.
+        auto body = [&](auto do_s_tag, auto do_pv_tag, auto do_sm_tag, auto do_fetch_tag,
+                const char *Kb, int kh, const char *Vb, int vh, const f32x16 &s_cur,
+                f32x16 &s_nxt, char *kdst, char *vdst)
             __attribute__((always_inline))
         {
             constexpr bool DO_S = decltype(do_s_tag)::value;
             constexpr bool DO_PV = decltype(do_pv_tag)::value;
             constexpr bool DO_SM = decltype(do_sm_tag)::value;
+            constexpr bool DO_FETCH = decltype(do_fetch_tag)::value;
+            static_assert(2 * LOADS_PER_WAVE <= NSLOT / 2, "one load every second slot");
+            auto fetch_piece = [&](int i) __attribute__((always_inline))
+            {
+                if(i < LOADS_PER_WAVE)
+                {
+                    load_to_lds16<0, false>(c2.Kp, k_goff[i], kdst + i * 1024);
+                }
+                else if(i < 2 * LOADS_PER_WAVE)
+                {
+                    switch(i - LOADS_PER_WAVE)
+                    {
+                        case 0: load_to_lds16<0, false>(c1.Vp, v_goff0, vdst); break;
+                        case 1: load_to_lds16<1024, false>(c1.Vp, v_goff0, vdst); break;
+                        case 2: load_to_lds16<2048, false>(c1.Vp, v_goff0, vdst); break;
+                        default: load_to_lds16<3072, false>(c1.Vp, v_goff0, vdst); break;
+                    }
+                }
+            };
             // the rescale that the previous softmax decided on (rare after the
             // first steps): O holds every sub-block up to j-2 at this point
             if(rescale_pending)
@@ -903,6 +928,10 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                         item(it);
                     }
                 }
+                if(DO_FETCH && (sl & 1))
+                {
+                    fetch_piece(sl >> 1);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
             rescale_pending = false;
@@ -978,39 +1007,66 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             c1 = c2;
             advance(c2);
         };
+        char *const no_dst = nullptr;
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
         // One step on the buffers of parity BUF: sub-block (g, 0) with the
         // scores of (g, 1) and the output of (g-1, 1), then sub-block (g, 1)
         // with the scores of (g+1, 0) and the output of (g, 0).  (After the
         // last pipelined step the scores computed ahead are not used.)
-        auto fast_step = [&](int g, auto buf_tag) __attribute__((always_inline))
+        // spread_tag: steps g+1 and g+2 exist and are complete, and their
+        // loads go into the slots of the second sub-block.
+        auto fast_step = [&](int g, auto buf_tag, auto spread_tag) __attribute__((always_inline))
         {
             constexpr int BUF = decltype(buf_tag)::value;
-            body(Yes{}, Yes{}, Yes{}, BUF ? lds_k1 : lds_k0, 1, BUF ? lds_v0 : lds_v1, 1, sa, sb);
-            mid_step(g, buf_tag);
-            body(Yes{}, Yes{}, Yes{}, BUF ? lds_k0 : lds_k1, 0, BUF ? lds_v1 : lds_v0, 0, sb, sa);
+            body(Yes{}, Yes{}, Yes{}, No{}, BUF ? lds_k1 : lds_k0, 1, BUF ? lds_v0 : lds_v1, 1,
+                    sa, sb, no_dst, no_dst);
+            if(decltype(spread_tag)::value)
+            {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                char *kdst = (BUF ? lds_k1 : lds_k0) + wave_u * LOADS_PER_WAVE * 1024;
+                char *vdst = (BUF ? lds_v0 : lds_v1) + wave_u * LOADS_PER_WAVE * 1024;
+                body(Yes{}, Yes{}, Yes{}, Yes{}, BUF ? lds_k0 : lds_k1, 0,
+                        BUF ? lds_v1 : lds_v0, 0, sb, sa, kdst, vdst);
+                c1 = c2;
+                advance(c2);
+            }
+            else
+            {
+                mid_step(g, buf_tag);
+                body(Yes{}, Yes{}, Yes{}, No{}, BUF ? lds_k0 : lds_k1, 0,
+                        BUF ? lds_v1 : lds_v0, 0, sb, sa, no_dst, no_dst);
+            }
             advance(cur);
         };
         // step 0: there is no output yet in its first half
-        body(Yes{}, No{}, Yes{}, lds_k0, 1, lds_v1, 1, sa, sb);
+        body(Yes{}, No{}, Yes{}, No{}, lds_k0, 1, lds_v1, 1, sa, sb, no_dst, no_dst);
         mid_step(0, std::integral_constant<int, 0>{});
-        body(Yes{}, Yes{}, Yes{}, lds_k1, 0, lds_v0, 0, sb, sa);
+        body(Yes{}, Yes{}, Yes{}, No{}, lds_k1, 0, lds_v0, 0, sb, sa, no_dst, no_dst);
         advance(cur);
-        for(int g = 1; g < n_fast; g += 2)
+        int g = 1;
+        for(; g + 1 < n_fast && g + 3 < n_spread; g += 2)
         {
-            fast_step(g, std::integral_constant<int, 1>{});
+            fast_step(g, std::integral_constant<int, 1>{}, Yes{});
+            fast_step(g + 1, std::integral_constant<int, 0>{}, Yes{});
+        }
+        // the last steps, whose successors may be incomplete or absent
+        for(; g < n_fast; g += 2)
+        {
+            fast_step(g, std::integral_constant<int, 1>{}, No{});
             if(g + 1 < n_fast)
             {
-                fast_step(g + 1, std::integral_constant<int, 0>{});
+                fast_step(g + 1, std::integral_constant<int, 0>{}, No{});
             }
         }
         // drain: the output of the last sub-block
         if((n_fast - 1) & 1)
         {
-            body(No{}, Yes{}, No{}, lds_k0, 0, lds_v1, 1, sb, sa);
+            body(No{}, Yes{}, No{}, No{}, lds_k0, 0, lds_v1, 1, sb, sa, no_dst, no_dst);
         }
         else
         {
-            body(No{}, Yes{}, No{}, lds_k0, 0, lds_v0, 1, sb, sa);
+            body(No{}, Yes{}, No{}, No{}, lds_k0, 0, lds_v0, 1, sb, sa, no_dst, no_dst);
         }
         g_first = n_fast;
         nxt = c1;

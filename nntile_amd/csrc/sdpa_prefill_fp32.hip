@@ -11,6 +11,12 @@
 //   O^T: the B operand is the S^T accumulator register itself (key
 //        8*(r/4) + 4h + r%4), the A operand is V[that key][d] read from LDS
 //        with the head axis across lanes - no transposition is needed.
+//
+// SPLIT variant, for launches with fewer workgroups than CUs: a workgroup is
+// 32 queries, and its four wavefronts take every fourth key step each (four
+// steps are staged per iteration), then merge their (max, sum, O) through LDS.
+// The chain of dependent steps a wavefront walks, which bounds such a launch,
+// is a quarter as long, and four times as many workgroups spread over the CUs.
 #include "sdpa_common.hpp"
 
 namespace nntile_hip
@@ -20,10 +26,12 @@ constexpr int kQRows32 = 128;
 constexpr int kKeys32 = 32;
 constexpr int kThreads32 = 256;
 
-template<int HEAD, int MODE>
-__global__ __launch_bounds__(kThreads32, 2)
+template<int HEAD, int MODE, bool SPLIT>
+__global__ __launch_bounds__(kThreads32, SPLIT ? 1 : 2)
 void sdpa_prefill_fp32_kernel(const PrefillParams p)
 {
+    constexpr int QROWS = SPLIT ? 32 : kQRows32;    // queries per workgroup
+    constexpr int NSUB = SPLIT ? 4 : 1;             // key steps staged per iteration
     constexpr int QSTEPS = HEAD / 8;        // 16-byte groups per lane half along head
     constexpr int DBLOCKS = HEAD / 32;
     constexpr int PAD = HEAD + 4;           // row stride in LDS (floats)
@@ -31,8 +39,8 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
 
-    __shared__ __attribute__((aligned(16))) float Ks[kKeys32 * PAD];
-    __shared__ __attribute__((aligned(16))) float Vs[kKeys32 * PAD];
+    __shared__ __attribute__((aligned(16))) float Ks[NSUB * kKeys32 * PAD];
+    __shared__ __attribute__((aligned(16))) float Vs[NSUB * kKeys32 * PAD];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -52,7 +60,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     const int qt = qblk / p.q_blocks_per_tile;
     const int qb = qblk % p.q_blocks_per_tile;
     const int64_t q_len = min(p.q_tile, p.q_seq - (int64_t)qt * p.q_tile);
-    const int64_t q_row0 = (int64_t)qb * kQRows32;
+    const int64_t q_row0 = (int64_t)qb * QROWS;
     if(q_row0 >= q_len)
     {
         return;
@@ -61,7 +69,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
 
     const float *Qt = static_cast<const float *>(p.Q[qt])
         + (int64_t)b * q_len * HEAD;
-    const int64_t my_q = q_row0 + wave * 32 + col;
+    const int64_t my_q = q_row0 + (SPLIT ? 0 : wave * 32) + col;
     const bool q_ok = my_q < q_len;
     const int64_t my_qpos = p.q_pos0 + (int64_t)qt * p.q_tile + my_q;
 
@@ -81,9 +89,9 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     int n_steps = (p.n_kv_tiles - 1) * p.k_blocks_per_tile
         + (int)((last_k_len + kKeys32 - 1) / kKeys32);
     const int64_t wg_qpos_hi = p.q_pos0 + (int64_t)qt * p.q_tile
-        + min(q_row0 + kQRows32, q_len) - 1;
+        + min(q_row0 + QROWS, q_len) - 1;
     const int64_t wave_qpos_lo = p.q_pos0 + (int64_t)qt * p.q_tile + q_row0
-        + wave * 32;
+        + (SPLIT ? 0 : wave * 32);
     const int64_t wave_qpos_hi = wave_qpos_lo + 31;
 
     // Cooperative loads: 32 rows x CHUNKS chunks for K and for V.
@@ -91,39 +99,51 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     constexpr int PASSES = kKeys32 / ROWS_PER_PASS;
     const int ld_chunk = tid % CHUNKS;
     const int ld_row = tid / CHUNKS;
-    f32x4 k_regs[PASSES], v_regs[PASSES];
+    f32x4 k_regs[NSUB][PASSES], v_regs[NSUB][PASSES];
 
-    auto fetch = [&](int g)
+    // loads of the key steps NSUB*G .. NSUB*G + NSUB-1 (zeros past the end)
+    auto fetch = [&](int G, int n_steps_all)
     {
-        const int kt = g / p.k_blocks_per_tile;
-        const int kb = g % p.k_blocks_per_tile;
-        const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
-        const int64_t row0 = (int64_t)kb * kKeys32;
-        const float *Kt = static_cast<const float *>(p.K[kt])
-            + ((int64_t)kvb * k_len) * HEAD;
-        const float *Vtile = static_cast<const float *>(p.V[kt])
-            + ((int64_t)kvb * k_len) * HEAD;
 #pragma unroll
-        for(int i = 0; i < PASSES; ++i)
+        for(int sub = 0; sub < NSUB; ++sub)
         {
-            const int64_t r = row0 + ld_row + i * ROWS_PER_PASS;
-            const bool ok = r < k_len;
-            const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-            k_regs[i] = ok ? *reinterpret_cast<const f32x4 *>(
-                    Kt + r * HEAD + ld_chunk * 4) : zero;
-            v_regs[i] = ok ? *reinterpret_cast<const f32x4 *>(
-                    Vtile + r * HEAD + ld_chunk * 4) : zero;
+            const int g = G * NSUB + sub;
+            const bool step_ok = g < n_steps_all;
+            const int kt = step_ok ? g / p.k_blocks_per_tile : 0;
+            const int kb = step_ok ? g % p.k_blocks_per_tile : 0;
+            const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
+            const int64_t row0 = (int64_t)kb * kKeys32;
+            const float *Kt = static_cast<const float *>(p.K[kt])
+                + ((int64_t)kvb * k_len) * HEAD;
+            const float *Vtile = static_cast<const float *>(p.V[kt])
+                + ((int64_t)kvb * k_len) * HEAD;
+#pragma unroll
+            for(int i = 0; i < PASSES; ++i)
+            {
+                const int64_t r = row0 + ld_row + i * ROWS_PER_PASS;
+                const bool ok = step_ok && r < k_len;
+                const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+                k_regs[sub][i] = ok ? *reinterpret_cast<const f32x4 *>(
+                        Kt + r * HEAD + ld_chunk * 4) : zero;
+                v_regs[sub][i] = ok ? *reinterpret_cast<const f32x4 *>(
+                        Vtile + r * HEAD + ld_chunk * 4) : zero;
+            }
         }
     };
 
     auto stage = [&]()
     {
 #pragma unroll
-        for(int i = 0; i < PASSES; ++i)
+        for(int sub = 0; sub < NSUB; ++sub)
         {
-            const int off = (ld_row + i * ROWS_PER_PASS) * PAD + ld_chunk * 4;
-            *reinterpret_cast<f32x4 *>(&Ks[off]) = k_regs[i];
-            *reinterpret_cast<f32x4 *>(&Vs[off]) = v_regs[i];
+#pragma unroll
+            for(int i = 0; i < PASSES; ++i)
+            {
+                const int off = (sub * kKeys32 + ld_row + i * ROWS_PER_PASS) * PAD
+                    + ld_chunk * 4;
+                *reinterpret_cast<f32x4 *>(&Ks[off]) = k_regs[sub][i];
+                *reinterpret_cast<f32x4 *>(&Vs[off]) = v_regs[sub][i];
+            }
         }
     };
 
@@ -163,18 +183,27 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     float m_run = neg_inf();
     float l_run = 0.0f;
 
-    if(n_steps > 0)
+    const int n_iter = (n_steps + NSUB - 1) / NSUB;
+    // this wavefront's part of the staged keys
+    const float *Kw = Ks + (SPLIT ? wave * kKeys32 * PAD : 0);
+    const float *Vw = Vs + (SPLIT ? wave * kKeys32 * PAD : 0);
+    if(n_iter > 0)
     {
-        fetch(0);
+        fetch(0, n_steps);
     }
-    for(int g = 0; g < n_steps; ++g)
+    for(int G = 0; G < n_iter; ++G)
     {
         __syncthreads();
         stage();
         __syncthreads();
-        if(g + 1 < n_steps)
+        if(G + 1 < n_iter)
         {
-            fetch(g + 1);
+            fetch(G + 1, n_steps);
+        }
+        const int g = SPLIT ? G * NSUB + wave : G;      // this wavefront's step
+        if(g >= n_steps)
+        {
+            continue;
         }
 
         const int kt = g / p.k_blocks_per_tile;
@@ -201,7 +230,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         for(int j = 0; j < QSTEPS; ++j)
         {
             const f32x4 a = *reinterpret_cast<const f32x4 *>(
-                    &Ks[col * PAD + j * 8 + half * 4]);
+                    &Kw[col * PAD + j * 8 + half * 4]);
 #pragma unroll
             for(int e = 0; e < 4; ++e)
             {
@@ -305,10 +334,61 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
 #pragma unroll
             for(int db = 0; db < DBLOCKS; ++db)
             {
-                const float a = Vs[key * PAD + db * 32 + col];
+                const float a = Vw[key * PAD + db * 32 + col];
                 o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s[r], o[db],
                         0, 0, 0);
             }
+        }
+    }
+
+    // ---- SPLIT: merge the four wavefronts' results into wavefront 0 ----------------
+    if constexpr(SPLIT)
+    {
+        // word w of lane l of wavefront v (v = 1..3) sits at ((v-1)*NW + w)*64 + l
+        constexpr int NW = 2 + 16 * DBLOCKS;
+        static_assert(3 * NW * 64 <= NSUB * kKeys32 * PAD, "exchange area does not fit");
+        float *xch = Ks;
+        __syncthreads();        // everyone is done with the staged keys
+        if(wave > 0)
+        {
+            float *dst = xch + (wave - 1) * NW * 64 + lane;
+            dst[0] = m_run;
+            dst[64] = l_run;
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+#pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    dst[(2 + 16 * db + r) * 64] = o[db][r];
+                }
+            }
+        }
+        __syncthreads();
+        if(wave > 0)
+        {
+            return;
+        }
+#pragma unroll
+        for(int v = 0; v < 3; ++v)
+        {
+            const float *src = xch + v * NW * 64 + lane;
+            const float m_other = src[0];
+            const float m_new = fmaxf(m_run, m_other);
+            const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+            const float a_mine = fast_exp2((m_run - m_use) * c);
+            const float a_other = fast_exp2((m_other - m_use) * c);
+            l_run = l_run * a_mine + src[64] * a_other;
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+#pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    o[db][r] = o[db][r] * a_mine + src[(2 + 16 * db + r) * 64] * a_other;
+                }
+            }
+            m_run = m_new;
         }
     }
 
@@ -362,7 +442,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     }
 }
 
-template<int HEAD>
+template<int HEAD, bool SPLIT>
 static int launch_mode32(hipStream_t stream, const PrefillParams &p, int mode,
         dim3 grid)
 {
@@ -370,22 +450,22 @@ static int launch_mode32(hipStream_t stream, const PrefillParams &p, int mode,
     {
         case NNTILE_HIP_MASK_ADDITIVE:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_ADDITIVE>), grid, dim3(kThreads32), 0,
+                        NNTILE_HIP_MASK_ADDITIVE, SPLIT>), grid, dim3(kThreads32), 0,
                     stream, p);
             break;
         case NNTILE_HIP_MASK_NONE:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_NONE>), grid, dim3(kThreads32), 0,
+                        NNTILE_HIP_MASK_NONE, SPLIT>), grid, dim3(kThreads32), 0,
                     stream, p);
             break;
         case NNTILE_HIP_MASK_CAUSAL:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_CAUSAL>), grid, dim3(kThreads32), 0,
+                        NNTILE_HIP_MASK_CAUSAL, SPLIT>), grid, dim3(kThreads32), 0,
                     stream, p);
             break;
         case NNTILE_HIP_MASK_BOOL:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_BOOL>), grid, dim3(kThreads32), 0,
+                        NNTILE_HIP_MASK_BOOL, SPLIT>), grid, dim3(kThreads32), 0,
                     stream, p);
             break;
         default:
@@ -396,8 +476,14 @@ static int launch_mode32(hipStream_t stream, const PrefillParams &p, int mode,
 
 int launch_prefill_fp32(hipStream_t stream, PrefillParams &p, int head, int mode)
 {
-    p.q_blocks_per_tile = (int)((p.q_tile + kQRows32 - 1) / kQRows32);
     p.k_blocks_per_tile = (int)((p.k_tile + kKeys32 - 1) / kKeys32);
+    // with fewer 128-query workgroups than CUs, 32-query workgroups whose
+    // wavefronts share the keys instead
+    const int64_t n_wide = (int64_t)p.batch * p.n_q_tiles
+        * ((p.q_tile + kQRows32 - 1) / kQRows32);
+    const bool split = n_wide < 256;
+    const int q_rows = split ? 32 : kQRows32;
+    p.q_blocks_per_tile = (int)((p.q_tile + q_rows - 1) / q_rows);
     const int64_t n_wg = (int64_t)p.batch * p.n_q_tiles * p.q_blocks_per_tile;
     if(n_wg <= 0 || n_wg > 0x7fffffff)
     {
@@ -408,11 +494,14 @@ int launch_prefill_fp32(hipStream_t stream, PrefillParams &p, int head, int mode
     switch(head)
     {
         case 32:
-            return launch_mode32<32>(stream, p, mode, grid);
+            return split ? launch_mode32<32, true>(stream, p, mode, grid)
+                : launch_mode32<32, false>(stream, p, mode, grid);
         case 64:
-            return launch_mode32<64>(stream, p, mode, grid);
+            return split ? launch_mode32<64, true>(stream, p, mode, grid)
+                : launch_mode32<64, false>(stream, p, mode, grid);
         case 128:
-            return launch_mode32<128>(stream, p, mode, grid);
+            return split ? launch_mode32<128, true>(stream, p, mode, grid)
+                : launch_mode32<128, false>(stream, p, mode, grid);
         default:
             return NNTILE_HIP_EUNSUPPORTED;
     }
