@@ -397,8 +397,9 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
             const float p3 = fast_exp2(fmaf(s[kb][3], c, -mc));
             pk[kb][0] = T::pack2(p0, p1);
             pk[kb][1] = T::pack2(p2, p3);
-            rs = T::add_pair(pk[kb][0], rs);
-            rs = T::add_pair(pk[kb][1], rs);
+            // (plain additions: the dot-product instruction that would sum a
+            // packed pair waits for the matrix unit)
+            rs += (p0 + p1) + (p2 + p3);
         }
         l_run += rs;
 

@@ -684,7 +684,9 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 m_run = m_new;
             }
 
-            float rs = 0.0f;
+            // row sums by plain additions (the dot-product instruction that
+            // would sum a packed pair waits for the matrix unit)
+            float rs0 = 0.0f, rs1 = 0.0f;
 #pragma unroll
             for(int mb = 0; mb < 2; ++mb)
             {
@@ -694,12 +696,11 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                     const float p0 = fast_exp2(fmaf(s[mb][r], c, -mc));
                     const float p1 = fast_exp2(fmaf(s[mb][r + 1], c, -mc));
                     pk[mb][r >> 1] = T::pack2(p0, p1);
-                    // the row sum runs over the ROUNDED probabilities, the
-                    // values the second product actually uses
-                    rs = T::add_pair(pk[mb][r >> 1], rs);
+                    rs0 += p0;
+                    rs1 += p1;
                 }
             }
-            l_run += rs;
+            l_run += rs0 + rs1;
         }
         // mask values of the next step (this step's have been consumed)
         if(EXPLICIT && mask_wide && g + 1 < n_steps
@@ -889,8 +890,13 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 }
                 else
                 {
+                    // (plain additions: the dot-product instruction that sums a
+                    // packed pair waits for the matrix unit, 15 cycles each)
+                    rs += pe[0];
+                    rs += pe[1];
                     pp[k] = T::pack2(pe[0], pe[1]);
-                    rs = T::add_pair(pp[k], rs);
+                    // (keeps the conversion in this slot)
+                    asm volatile("" : "+v"(pp[k]));
                 }
             };
 #pragma unroll
@@ -956,7 +962,8 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                         const float p0 = fast_exp2(fmaf(s_cur[2 * k], c, -mc_new));
                         const float p1 = fast_exp2(fmaf(s_cur[2 * k + 1], c, -mc_new));
                         pp[k] = T::pack2(p0, p1);
-                        rs = T::add_pair(pp[k], rs);
+                        rs += p0;
+                        rs += p1;
                     }
                     l_run *= alpha;
                     m_run = m_new;
