@@ -21,7 +21,10 @@ namespace nntile_hip
 {
 
 constexpr int kMaxTiles = NNTILE_HIP_SDPA_MAX_TILES;
-constexpr int kDecKeys = 64;    // keys per step of the decode kernel
+#ifndef NNTILE_DEC_KEYS
+#define NNTILE_DEC_KEYS 64
+#endif
+constexpr int kDecKeys = NNTILE_DEC_KEYS;    // keys per step of the decode kernel
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 

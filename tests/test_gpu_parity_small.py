@@ -339,3 +339,38 @@ def test_unmasked_steps_loop(oracle, dtype, head, q_seq, k_seq, k_tile, causal):
     assert torch.equal(runs[0][1].view(torch.int16), runs[1][1].view(torch.int16))
     assert H.rel_fro(H.to_np(runs[0][1]), want) < H.TOL[dtype]
     assert H.rel_fro(H.to_np(runs[0][0]), want_lse) < H.TOL[dtype]
+
+
+@pytest.mark.parametrize("head", [32, 64, 128])
+@pytest.mark.parametrize("batch,q_seq,k_seq,k_tile", [(3, 200, 333, 333), (2, 64, 1000, 250),
+                                                      (40, 1024, 320, 320), (70, 512, 200, 96)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_fp32_launch_forms(oracle, head, batch, q_seq, k_seq, k_tile, causal):
+    """The fp32 kernel has two launch forms: 128-query workgroups, and - for
+    launches with fewer of those than the GPU has CUs - 32-query workgroups
+    whose four wavefronts share the keys and merge at the end.  Small batches
+    take the second form, the large ones the first; both against the checker,
+    over one and several key tiles (ragged ones included), with key counts
+    that leave some wavefronts of the second form without a step."""
+    print("case fp32", head, batch, q_seq, k_seq, k_tile, causal, flush=True)
+    offset = max(k_seq - q_seq, 0)
+    (Q, K, V), f32 = H.make_qkv(31, batch, q_seq, k_seq, head, "fp32")
+    mask = synth.causal_mask(q_seq, k_seq, offset) if causal else None
+    want, want_lse = _oracle(oracle, f32, mask, k_tile=k_tile)
+    Kt = [K[:, s:s + k_tile].contiguous().cuda() for s in range(0, k_seq, k_tile)]
+    Vt = [V[:, s:s + k_tile].contiguous().cuda() for s in range(0, k_seq, k_tile)]
+    mode = hip_sdpa.MASK_CAUSAL if causal else hip_sdpa.MASK_NONE
+    lse, A = H.fresh_outputs(batch, q_seq, head, "fp32")
+    hip_sdpa.sdpa_fwd_grid(Kt, [Q.cuda()], [lse], Vt, [A], q_seq, k_seq, q_seq, k_tile, mode,
+                           causal_offset=offset)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < H.TOL["fp32"]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL["fp32"]
+    # per key tile, merged into the running pair
+    lse2, A2 = H.fresh_outputs(batch, q_seq, head, "fp32")
+    for i, (kt, vt) in enumerate(zip(Kt, Vt)):
+        hip_sdpa.sdpa_fwd_tile(kt, Q.cuda(), None, lse2, vt, A2, mode, k_pos0=i * k_tile,
+                               causal_offset=offset)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A2), want) < H.TOL["fp32"]
+    assert H.rel_fro(H.to_np(lse2), want_lse) < H.TOL["fp32"]
