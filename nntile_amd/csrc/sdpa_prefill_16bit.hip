@@ -197,6 +197,65 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                     + (hi - kt_hi * k_tile) / kKeys + 1);
         }
     }
+    if(EXPLICIT)
+    {
+        // A mask tile that hides every key from every query of the workgroup
+        // (the tile pairs above the diagonal when a causal mask arrives as
+        // values) is recognised before anything is fetched: the workgroup's
+        // mask rows are read 16 bytes per thread, 16 loads in flight, until
+        // some value is not "hidden".  Such a launch then costs a scan of its
+        // mask instead of a pass over K and V.
+        constexpr int ES = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 2 : 1;
+        const int64_t row_bytes = (int64_t)k_seq * ES;
+        if(n_steps > 0 && row_bytes % 16 == 0 && (p.mask_ld * ES) % 16 == 0
+                && reinterpret_cast<uintptr_t>(p.mask) % 16 == 0
+                && row_bytes * kQRows < (int64_t)(1 << 30))
+        {
+            const int n_chunks = (int)(row_bytes / 16);
+            const int total = min(kQRows, q_len - q_row0) * n_chunks;
+            const char *mbase = static_cast<const char *>(p.mask)
+                + (int64_t)q_row0 * p.mask_ld * ES;
+            int any = 0;
+            for(int base = 0; base < total && !any; base += 16 * kThreads)
+            {
+                // (indices past the end re-read the last chunk: no branches,
+                // so that the 16 loads are in flight together)
+                u32x4 v[16];
+#pragma unroll
+                for(int u = 0; u < 16; ++u)
+                {
+                    const int idx = min(base + u * kThreads + tid, total - 1);
+                    const int row = idx / n_chunks;
+                    const int c = idx - row * n_chunks;
+                    v[u] = *reinterpret_cast<const u32x4 *>(
+                            mbase + (int64_t)row * p.mask_ld * ES + c * 16);
+                }
+                bool seen = false;
+#pragma unroll
+                for(int u = 0; u < 16; ++u)
+                {
+                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                    {
+                        seen |= (v[u][0] != T::kNegInfPair) | (v[u][1] != T::kNegInfPair)
+                            | (v[u][2] != T::kNegInfPair) | (v[u][3] != T::kNegInfPair);
+                    }
+                    else
+                    {
+                        seen |= (v[u][0] | v[u][1] | v[u][2] | v[u][3]) != 0u;
+                    }
+                }
+                any = __syncthreads_or(seen ? 1 : 0);
+            }
+            if(!any)
+            {
+                if(!p.overwrite)
+                {
+                    return;
+                }
+                n_steps = 0;    // the epilogue writes empty rows
+            }
+        }
+    }
     const int wave_rel_lo = rel0 + wave * 32;       // first query of the wavefront
     const int my_rel = wave_rel_lo + col;
 
