@@ -197,56 +197,90 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                     + (hi - kt_hi * k_tile) / kKeys + 1);
         }
     }
+    // Explicit masks: number of leading key steps in which the mask changes
+    // nothing for any query of the workgroup (they run in the pipelined loop).
+    int n_open = 0;
     if(EXPLICIT)
     {
-        // A mask tile that hides every key from every query of the workgroup
-        // (the tile pairs above the diagonal when a causal mask arrives as
-        // values) is recognised before anything is fetched: the workgroup's
-        // mask rows are read 16 bytes per thread, 16 loads in flight, until
-        // some value is not "hidden".  Such a launch then costs a scan of its
-        // mask instead of a pass over K and V.
+        // The workgroup's rows of the mask are scanned once, 16 bytes per
+        // thread and load, 16 loads in flight, before anything is fetched.
+        // Per key step the scan records whether every value is "open" (+0 /
+        // true) and whether every value is "hidden" (-inf / false).  Hidden
+        // steps at the end are dropped - a tile pair above the diagonal of a
+        // causal mask given as values costs this scan instead of a pass over K
+        // and V - and the open steps at the start need no mask handling.
         constexpr int ES = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 2 : 1;
+        constexpr int CHUNKS_PER_STEP = kKeys * ES / 16;
+        constexpr uint32_t OPEN = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 0u : 0x01010101u;
+        constexpr uint32_t HIDDEN = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? T::kNegInfPair : 0u;
         const int64_t row_bytes = (int64_t)k_seq * ES;
         if(n_steps > 0 && row_bytes % 16 == 0 && (p.mask_ld * ES) % 16 == 0
                 && reinterpret_cast<uintptr_t>(p.mask) % 16 == 0
-                && row_bytes * kQRows < (int64_t)(1 << 30))
+                && p.mask_ld * ES * kQRows < (int64_t)(1 << 30))
         {
+            __shared__ unsigned long long scan_bits[2];
+            if(tid == 0)
+            {
+                scan_bits[0] = 0ull;
+                scan_bits[1] = 0ull;
+            }
+            __syncthreads();
             const int n_chunks = (int)(row_bytes / 16);
-            const int total = min(kQRows, q_len - q_row0) * n_chunks;
+            const int n_rows = min(kQRows, q_len - q_row0);
+            const int total = n_rows * n_chunks;
             const char *mbase = static_cast<const char *>(p.mask)
                 + (int64_t)q_row0 * p.mask_ld * ES;
-            int any = 0;
-            for(int base = 0; base < total && !any; base += 16 * kThreads)
+            // bit s: some value of step s (steps >= 63 share bit 63) is not open / not hidden
+            unsigned long long not_open = 0ull, not_hidden = 0ull;
+            // chunk tid, tid + 256, ... of the rows laid end to end: (row, c)
+            // advances by 256 chunks per load without a division
+            const int d_row = kThreads / n_chunks, d_c = kThreads % n_chunks;
+            const int ld_bytes = (int)(p.mask_ld * ES);     // fits: checked above
+            int row = tid / n_chunks, c = tid % n_chunks;
+            for(int base = 0; base < total; base += 16 * kThreads)
             {
-                // (indices past the end re-read the last chunk: no branches,
-                // so that the 16 loads are in flight together)
+                // (rows past the end re-read the last row: no branches, so
+                // that the 16 loads are in flight together)
                 u32x4 v[16];
+                int st[16];
 #pragma unroll
                 for(int u = 0; u < 16; ++u)
                 {
-                    const int idx = min(base + u * kThreads + tid, total - 1);
-                    const int row = idx / n_chunks;
-                    const int c = idx - row * n_chunks;
+                    const int r = min(row, n_rows - 1);
+                    st[u] = min(c / CHUNKS_PER_STEP, 63);
                     v[u] = *reinterpret_cast<const u32x4 *>(
-                            mbase + (int64_t)row * p.mask_ld * ES + c * 16);
+                            mbase + (uint32_t)(r * ld_bytes + c * 16));
+                    row += d_row;
+                    c += d_c;
+                    if(c >= n_chunks)
+                    {
+                        c -= n_chunks;
+                        row += 1;
+                    }
                 }
-                bool seen = false;
 #pragma unroll
                 for(int u = 0; u < 16; ++u)
                 {
-                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
-                    {
-                        seen |= (v[u][0] != T::kNegInfPair) | (v[u][1] != T::kNegInfPair)
-                            | (v[u][2] != T::kNegInfPair) | (v[u][3] != T::kNegInfPair);
-                    }
-                    else
-                    {
-                        seen |= (v[u][0] | v[u][1] | v[u][2] | v[u][3]) != 0u;
-                    }
+                    const uint32_t any1 = v[u][0] | v[u][1] | v[u][2] | v[u][3];
+                    const uint32_t all1 = v[u][0] & v[u][1] & v[u][2] & v[u][3];
+                    const bool open = (any1 == OPEN) & (all1 == OPEN);
+                    const bool hidden = (any1 == HIDDEN) & (all1 == HIDDEN);
+                    not_open |= (unsigned long long)(!open) << st[u];
+                    not_hidden |= (unsigned long long)(!hidden) << st[u];
                 }
-                any = __syncthreads_or(seen ? 1 : 0);
             }
-            if(!any)
+            if(not_open != 0ull)
+            {
+                atomicOr(&scan_bits[0], not_open);
+            }
+            if(not_hidden != 0ull)
+            {
+                atomicOr(&scan_bits[1], not_hidden);
+            }
+            __syncthreads();
+            not_open = scan_bits[0];
+            not_hidden = scan_bits[1];
+            if(not_hidden == 0ull)
             {
                 if(!p.overwrite)
                 {
@@ -254,6 +288,11 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 }
                 n_steps = 0;    // the epilogue writes empty rows
             }
+            else if((not_hidden >> 63) == 0ull)
+            {
+                n_steps = min(n_steps, 64 - __builtin_clzll(not_hidden));
+            }
+            n_open = not_open == 0ull ? 63 : min(__builtin_ctzll(not_open), 63);
         }
     }
     const int wave_rel_lo = rel0 + wave * 32;       // first query of the wavefront
@@ -523,7 +562,6 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // the workgroup need no mask at all; they run in the pipelined loop below.
     int n_fast = 0;
     int n_spread = 0;       // leading steps that exist and are complete
-    if(!EXPLICIT)
     {
         const int n_full = (p.n_kv_tiles == 1 || k_tile % kKeys == 0)
             ? k_seq / kKeys : k_tile / kKeys;
@@ -532,6 +570,10 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         if(MODE == NNTILE_HIP_MASK_CAUSAL)
         {
             n_fast = min(n_fast, max(rel0 + 1, 0) / kKeys);
+        }
+        if(EXPLICIT)
+        {
+            n_fast = min(n_fast, n_open);
         }
         n_fast = n_fast >= 2 ? n_fast : 0;
     }
@@ -544,7 +586,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         {
             fetch_k(nxt, lds_k1);       // the pipelined loop keeps K two steps ahead
         }
-        if(mask_wide && cur.rows_left >= kKeys)
+        if(mask_wide && n_fast == 0 && cur.rows_left >= kKeys)
         {
             mask_fetch(0);
         }
@@ -1136,6 +1178,10 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         }
         g_first = n_fast;
         nxt = c1;
+        if(EXPLICIT && mask_wide && g_first < n_steps && cur.rows_left >= kKeys)
+        {
+            mask_fetch(cur.kb);     // the general step finds its mask values loaded
+        }
         // the general loop expects step g_first complete in its buffers
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
