@@ -374,3 +374,51 @@ def test_fp32_launch_forms(oracle, head, batch, q_seq, k_seq, k_tile, causal):
     torch.cuda.synchronize()
     assert H.rel_fro(H.to_np(A2), want) < H.TOL["fp32"]
     assert H.rel_fro(H.to_np(lse2), want_lse) < H.TOL["fp32"]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("form", ["additive", "bool"])
+@pytest.mark.parametrize("q_seq,k_seq", [(256, 1024), (200, 712), (128, 520), (130, 333)])
+@pytest.mark.parametrize("pattern", ["band", "late_start", "holes", "all_hidden", "all_open"])
+def test_explicit_mask_scan_paths(oracle, dtype, form, q_seq, k_seq, pattern):
+    """Masks given as values are scanned once per workgroup: leading key steps
+    in which nothing is masked run in the unmasked pipelined loop, trailing
+    steps in which everything is hidden are dropped.  The patterns put the
+    boundaries of those runs at, before and after multiples of the 64-key
+    step, per 128-query block differently; 333 keys make rows that are not a
+    multiple of 16 bytes (no scan), 712 and 520 a ragged last step."""
+    print("case scan", dtype, form, q_seq, k_seq, pattern, flush=True)
+    batch, head = 3, 128
+    i = np.arange(q_seq)[:, None]
+    j = np.arange(k_seq)[None, :]
+    if pattern == "band":            # open prefix, mixed band, hidden suffix
+        mask = j <= (k_seq // 3 + 2 * i)
+    elif pattern == "late_start":    # first keys hidden for some rows, rest open
+        mask = j >= (i % 7) * 3
+    elif pattern == "holes":         # a hidden stretch in the middle, rows with nothing visible
+        mask = ((j < 100) | (j >= 300)) & (i % 50 != 49)
+    elif pattern == "all_hidden":
+        mask = np.zeros((q_seq, k_seq), bool)
+    else:
+        mask = np.ones((q_seq, k_seq), bool)
+    mask = np.ascontiguousarray(np.broadcast_to(mask, (q_seq, k_seq)))
+    (Q, K, V), f32 = H.make_qkv(77, batch, q_seq, k_seq, head, dtype)
+    want, want_lse = _oracle(oracle, f32, mask)
+    m = (H.additive_mask(mask, dtype) if form == "additive" else torch.from_numpy(mask.copy())).cuda()
+    mode = hip_sdpa.MASK_ADDITIVE if form == "additive" else hip_sdpa.MASK_BOOL
+    # merged into a running pair that starts empty ...
+    lse, A = H.fresh_outputs(batch, q_seq, head, dtype)
+    hip_sdpa.sdpa_fwd_tile(K.cuda(), Q.cuda(), m, lse, V.cuda(), A, mode)
+    torch.cuda.synchronize()
+    got, got_lse = H.to_np(A), H.to_np(lse)
+    vis = mask.any(axis=1)
+    assert np.all(np.isneginf(got_lse[:, ~vis]))
+    assert H.rel_fro(got[:, vis], want[:, vis]) < H.TOL[dtype] or not vis.any()
+    assert H.rel_fro(got_lse[:, vis], want_lse[:, vis]) < H.TOL[dtype] or not vis.any()
+    # ... and in overwrite mode, where rows without a visible key become 0 / -inf
+    lse2, A2 = H.fresh_outputs(batch, q_seq, head, dtype)
+    hip_sdpa.sdpa_fwd_tile(K.cuda(), Q.cuda(), m, lse2, V.cuda(), A2, mode, flags=hip_sdpa.OVERWRITE)
+    torch.cuda.synchronize()
+    got2, got2_lse = H.to_np(A2), H.to_np(lse2)
+    assert np.all(got2[:, ~vis] == 0) and np.all(np.isneginf(got2_lse[:, ~vis]))
+    assert np.array_equal(got2[:, vis], got[:, vis]) and np.array_equal(got2_lse[:, vis], got_lse[:, vis])
