@@ -1,0 +1,76 @@
+"""Checks on the generated GPU code that no run-time test would catch.
+
+The kernels move K and V from global memory into LDS with
+`global_load_lds_dwordx4`, issued from assembly text that writes M0 (the LDS
+target) without the compiler knowing.  That is safe only while the compiler
+itself never uses M0 in these kernels; this test compiles every kernel source
+to gfx950 assembly and looks.  It also checks that the packed-fp32
+instructions, which the build switches off, do not appear."""
+import os
+import re
+import subprocess
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
+
+import pytest
+
+from nntile_amd import build as B
+
+KERNEL_SOURCES = [s for s in B.SOURCES if s != "capi.hip"]
+
+
+def _assembly(name, outdir):
+    src = os.path.join(B.CSRC, name)
+    out = os.path.join(outdir, name + ".s")
+    flags = [f for f in B.FLAGS if f != "-fPIC"]
+    subprocess.run([B.HIPCC] + flags + ["-S", "--cuda-device-only", "-o", out, src],
+                   check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    with open(out) as f:
+        return f.read()
+
+
+@pytest.fixture(scope="module")
+def assemblies():
+    if not os.path.exists(B.HIPCC):
+        pytest.skip("hipcc not found")
+    with tempfile.TemporaryDirectory() as d:
+        with ThreadPoolExecutor(max_workers=4) as ex:
+            texts = list(ex.map(lambda n: _assembly(n, d), KERNEL_SOURCES))
+    return dict(zip(KERNEL_SOURCES, texts))
+
+
+def _instructions(text):
+    for line in text.splitlines():
+        line = line.split(";")[0].strip()
+        if line and not line.startswith(".") and not line.endswith(":"):
+            yield line
+
+
+def test_m0_is_written_only_by_the_lds_load_helper(assemblies):
+    uses = 0
+    for name, text in assemblies.items():
+        ins = list(_instructions(text))
+        for i, line in enumerate(ins):
+            if not re.search(r"\bm0\b", line):
+                continue
+            # the helper's three lines: s_mov_b32 m0, sN / s_nop 0 / global_load_lds_dwordx4
+            assert re.fullmatch(r"s_mov_b32 m0, s\d+", line), (name, line)
+            assert ins[i + 1] == "s_nop 0", (name, ins[i + 1])
+            assert ins[i + 2].startswith("global_load_lds_dwordx4 "), (name, ins[i + 2])
+            uses += 1
+    assert uses > 0     # the prefill and decode kernels do use the helper
+
+
+def test_every_lds_load_sets_m0_first(assemblies):
+    for name, text in assemblies.items():
+        ins = list(_instructions(text))
+        for i, line in enumerate(ins):
+            if line.startswith("global_load_lds_"):
+                assert i >= 2 and ins[i - 1] == "s_nop 0" \
+                    and re.fullmatch(r"s_mov_b32 m0, s\d+", ins[i - 2]), (name, line)
+
+
+def test_no_packed_fp32_instructions(assemblies):
+    for name, text in assemblies.items():
+        for line in _instructions(text):
+            assert not re.match(r"v_pk_(add|mul|fma)_f32\b", line), (name, line)
