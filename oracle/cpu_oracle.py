@@ -192,3 +192,99 @@ def sdpa_bruteforce_f64(K, Q, V, add_mask=None):
                                             _p(Q), _p(m), _p(V), _p(A),
                                             _p(lse))
     return A, lse
+
+
+# ---- backward (numpy; test infrastructure like everything above) -------------
+
+def sdpa_bwd_vanilla(K, Q, V, dY, mask=None):
+    """Gradients of the forward composition, step by step as the reference's
+    `Sdpa._backward_vanilla` (wrappers/python/nntile/layer/sdpa.py:595-698)
+    takes them, in fp32:
+
+        attn.grad  = V^T dY                                   (gemm, :606-618)
+        v.grad    += dY attn^T                                (gemm, :623-635)
+        s[q]       = sum_h y[h,q] dY[h,q]                     (sumprod_slice, :640-648)
+        attn.grad  = (attn.grad - s[q]) * attn                (add_slice_inplace, multiply_inplace, :649-653)
+        attn.grad  = 0 where the mask hides (k, q)            (mask_scalar, :656-660)
+        k.grad    += scale Q attn.grad^T                      (gemm, :667-679)
+        q.grad    += scale K attn.grad                        (gemm, :686-698)
+
+    with attn = softmax over keys of scale K^T Q (+ mask), y = V attn as the
+    forward pass left them.  K, Q, V, dY: [batch, seq, head] (C-order views of
+    the Fortran tiles), mask: bool [q_seq, k_seq] or None.  Returns
+    (dK, dQ, dV) as the increments that are added to the .grad tensors."""
+    K = _c(K, np.float32)
+    Q = _c(Q, np.float32)
+    V = _c(V, np.float32)
+    dY = _c(dY, np.float32)
+    head = Q.shape[2]
+    scale = np.float32(1.0) / np.sqrt(np.float32(head))
+    # forward quantities, as the forward composition produces them
+    scores = np.einsum("bkh,bqh->bkq", K, Q).astype(np.float32) * scale
+    if mask is not None:
+        scores = np.where(np.asarray(mask, bool).T[None], scores, np.float32(-np.inf))
+    mx = scores.max(axis=1, keepdims=True)
+    mx = np.where(np.isfinite(mx), mx, np.float32(0))
+    e = np.exp(scores - mx, dtype=np.float32)
+    sm = e.sum(axis=1, keepdims=True)
+    attn = np.where(sm > 0, e / np.where(sm > 0, sm, 1), 0).astype(np.float32)
+    y = np.einsum("bkh,bkq->bqh", V, attn).astype(np.float32)
+    # backward steps
+    dattn = np.einsum("bkh,bqh->bkq", V, dY).astype(np.float32)
+    dV = np.einsum("bqh,bkq->bkh", dY, attn).astype(np.float32)
+    s = np.einsum("bqh,bqh->bq", y, dY).astype(np.float32)
+    dattn = (dattn - s[:, None, :]) * attn
+    if mask is not None:
+        dattn = np.where(np.asarray(mask, bool).T[None], dattn, np.float32(0))
+    dK = scale * np.einsum("bqh,bkq->bkh", Q, dattn).astype(np.float32)
+    dQ = scale * np.einsum("bkh,bkq->bqh", K, dattn).astype(np.float32)
+    return dK.astype(np.float32), dQ.astype(np.float32), dV
+
+
+def sdpa_bwd_flash_f64(K, Q, V, A, dA, lse, add_mask=None, kv_repeat=1, n_batch=None):
+    """The flash form in fp64, with the forward output A and the logsumexp
+    taken as given (they need not belong to K, Q, V), as the reference's test
+    of its backward kernel computes it
+    (tests/kernel/flash_sdpa_bwd_cudnn.cc:174-262):
+
+        P[q,k]  = exp(scale q.k + mask[q,k] - lse[q])   (0 where the score is -inf)
+        dP[q,k] = dA[q,:] . V[k,:]
+        D[q]    = dA[q,:] . A[q,:]
+        dS      = P (dP - D)
+        dV[k,:] = sum_q P[q,k] dA[q,:];  dQ[q,:] = scale sum_k dS[q,k] K[k,:];
+        dK[k,:] = scale sum_q dS[q,k] Q[q,:]
+
+    add_mask: additive fp32 [q_seq, k_seq] or None.  With kv_repeat > 1 query
+    batch entry b = nb + n_batch*(g + kv_repeat*hkv) reads K/V entry
+    nb + n_batch*hkv and dK, dV sum over the group.  Returns (dK, dQ, dV)."""
+    K = np.asarray(K, np.float64)
+    Q = np.asarray(Q, np.float64)
+    V = np.asarray(V, np.float64)
+    A = np.asarray(A, np.float64)
+    dA = np.asarray(dA, np.float64)
+    lse = np.asarray(lse, np.float64)
+    batch, q_seq, head = Q.shape
+    kv_batch = K.shape[0]
+    if n_batch is None:
+        n_batch = batch if kv_repeat == 1 else None
+    assert n_batch is not None and kv_batch * kv_repeat == batch
+    scale = 1.0 / np.sqrt(float(head))
+    dK = np.zeros_like(K)
+    dV = np.zeros_like(V)
+    dQ = np.zeros_like(Q)
+    for b in range(batch):
+        nb = b % n_batch
+        hkv = (b // n_batch) // kv_repeat
+        kv = nb + n_batch * hkv
+        s = scale * (Q[b] @ K[kv].T)
+        if add_mask is not None:
+            s = s + np.asarray(add_mask, np.float64)
+        with np.errstate(over="ignore", invalid="ignore"):
+            p = np.where(np.isneginf(s), 0.0, np.exp(s - lse[b][:, None]))
+        dp = dA[b] @ V[kv].T
+        d = (dA[b] * A[b]).sum(axis=1)
+        ds = p * (dp - d[:, None])
+        dV[kv] += p.T @ dA[b]
+        dQ[b] = scale * (ds @ K[kv])
+        dK[kv] += scale * (ds.T @ Q[b])
+    return dK, dQ, dV
