@@ -113,6 +113,54 @@ int nntile_hip_sdpa_fwd_tile_bf16(void *stream, const nntile_hip_sdpa_tile_args 
 int nntile_hip_sdpa_fwd_tile_fp16(void *stream, const nntile_hip_sdpa_tile_args *args);
 int nntile_hip_sdpa_fwd_tile_fp32(void *stream, const nntile_hip_sdpa_tile_args *args);
 
+/* ---- 2b. backward of one (query tile, key tile) pair ------------------------
+ * Replaces kernel::flash_sdpa_bwd_cudnn::execute_graph<T>
+ * (include/nntile/kernel/flash_sdpa_bwd_cudnn/cuda.hh:44-68,
+ *  src/kernel/flash_sdpa_bwd_cudnn/cuda.cc:171-218): same argument order and
+ * meaning, the cuDNN handle/graph pair replaced by the stream and the cuDNN
+ * workspace dropped.  The forward output A and the logsumexp are inputs; the
+ * gradients of this tile pair are ADDED to dK, dQ, dV (the reference computes
+ * them into the scratch tiles and adds those, cuda.cc:213-217).  scratch_dK
+ * and scratch_dV are accepted for signature compatibility and never touched;
+ * the first seq*batch floats of scratch_dQ hold the row dots dA.A between the
+ * two kernels of the call (it must not be null).  The reference's pack is
+ * {bf16, fp16} (include/nntile/starpu/flash_sdpa_bwd_cudnn.hh). */
+int nntile_hip_flash_sdpa_bwd_bf16(void *stream, int64_t seq, int64_t head,
+        int64_t batch, const uint16_t *K, const uint16_t *Q, const uint16_t *V,
+        const uint16_t *A, const uint16_t *dA, const uint16_t *mask,
+        const float *lse, uint16_t *scratch_dK, uint16_t *scratch_dQ,
+        uint16_t *scratch_dV, uint16_t *dK, uint16_t *dQ, uint16_t *dV);
+int nntile_hip_flash_sdpa_bwd_fp16(void *stream, int64_t seq, int64_t head,
+        int64_t batch, const uint16_t *K, const uint16_t *Q, const uint16_t *V,
+        const uint16_t *A, const uint16_t *dA, const uint16_t *mask,
+        const float *lse, uint16_t *scratch_dK, uint16_t *scratch_dQ,
+        uint16_t *scratch_dV, uint16_t *dK, uint16_t *dQ, uint16_t *dV);
+
+/* General form, what tile::flash_sdpa_bwd_cudnn_async
+ * (src/tile/flash_sdpa_bwd_cudnn.cc) would submit if tiles need not be square
+ * and the mask need not be materialised: shapes, batch mapping, mask modes
+ * and positions as in nntile_hip_sdpa_tile_args; with kv_group > 1 the
+ * gradients of a key/value head sum over its query heads.  flags:
+ * NNTILE_HIP_SDPA_OVERWRITE writes the gradients instead of adding to them.
+ * workspace: q_seq*batch floats (nntile_hip_sdpa_bwd_workspace_bytes). */
+typedef struct nntile_hip_sdpa_bwd_args
+{
+    int64_t q_seq, k_seq, head;
+    int64_t batch, n_batch, kv_group;
+    int32_t mask_mode;
+    int32_t flags;
+    int64_t q_pos0, k_pos0, causal_offset;
+    const void *K, *Q, *V, *A, *dA, *mask;
+    const float *lse;
+    void *dK, *dQ, *dV;
+    void *workspace;
+    size_t workspace_bytes;
+} nntile_hip_sdpa_bwd_args;
+
+size_t nntile_hip_sdpa_bwd_workspace_bytes(int64_t q_seq, int64_t batch);
+int nntile_hip_sdpa_bwd_tile_bf16(void *stream, const nntile_hip_sdpa_bwd_args *args);
+int nntile_hip_sdpa_bwd_tile_fp16(void *stream, const nntile_hip_sdpa_bwd_args *args);
+
 /* ---- 3. a whole grid of tiles in one launch ---------------------------------
  * What tensor::flash_sdpa_fwd_cudnn_async (src/tensor/flash_sdpa_fwd_cudnn.cc:
  * 210-279) computes when every tile of one (batch, head) slab is resident on

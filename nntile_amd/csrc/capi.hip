@@ -14,6 +14,8 @@ int launch_prefill_fp32(hipStream_t stream, PrefillParams &p, int head, int mode
 template<typename T>
 int launch_decode_16bit(hipStream_t stream, DecodeParams &p, int head, int mode);
 int decode_choose_splits(int units, int n_steps);
+template<typename T>
+int launch_bwd_16bit(hipStream_t stream, const BwdParams &p, int head, int mode);
 size_t decode_workspace_bytes(int units, int n_splits, int rows, int head);
 
 struct F32Store;
@@ -99,6 +101,99 @@ static int tile_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a)
     p.A[0] = a->A;
     return dispatch_prefill(dt, static_cast<hipStream_t>(stream), p, a->head,
             a->mask_mode);
+}
+
+static int bwd_call(DType dt, void *stream, const nntile_hip_sdpa_bwd_args *a)
+{
+    if(a == nullptr || a->q_seq <= 0 || a->k_seq <= 0 || a->head <= 0
+            || a->batch <= 0 || a->n_batch <= 0 || a->kv_group <= 0
+            || !mode_ok(a->mask_mode) || a->K == nullptr || a->Q == nullptr
+            || a->V == nullptr || a->A == nullptr || a->dA == nullptr
+            || a->lse == nullptr || a->dK == nullptr || a->dQ == nullptr
+            || a->dV == nullptr
+            || a->batch % (a->n_batch * a->kv_group) != 0
+            || a->batch > 0x7fffffff || a->q_seq > 0x7fffffff
+            || a->k_seq > 0x7fffffff)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    const bool explicit_mask = a->mask_mode == NNTILE_HIP_MASK_ADDITIVE
+        || a->mask_mode == NNTILE_HIP_MASK_BOOL;
+    if(explicit_mask && a->mask == nullptr)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(!aligned16(a->K) || !aligned16(a->Q) || !aligned16(a->V) || !aligned16(a->A)
+            || !aligned16(a->dA) || !aligned16(a->dK) || !aligned16(a->dQ)
+            || !aligned16(a->dV))
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(a->head != 32 && a->head != 64 && a->head != 128)
+    {
+        return NNTILE_HIP_EUNSUPPORTED;
+    }
+    if(a->workspace == nullptr
+            || a->workspace_bytes < nntile_hip_sdpa_bwd_workspace_bytes(a->q_seq, a->batch)
+            || (reinterpret_cast<uintptr_t>(a->workspace) & 3u) != 0)
+    {
+        return NNTILE_HIP_EWORKSPACE;
+    }
+    BwdParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.q_seq = a->q_seq;
+    p.k_seq = a->k_seq;
+    p.q_pos0 = a->q_pos0;
+    p.k_pos0 = a->k_pos0;
+    p.causal_offset = a->causal_offset;
+    p.mask = a->mask;
+    p.mask_ld = a->k_seq;
+    p.K = a->K;
+    p.Q = a->Q;
+    p.V = a->V;
+    p.A = a->A;
+    p.dA = a->dA;
+    p.lse = a->lse;
+    p.D = static_cast<float *>(a->workspace);
+    p.dK = a->dK;
+    p.dQ = a->dQ;
+    p.dV = a->dV;
+    p.batch = (int32_t)a->batch;
+    p.n_batch = (int32_t)a->n_batch;
+    p.kv_group = (int32_t)a->kv_group;
+    p.overwrite = (a->flags & NNTILE_HIP_SDPA_OVERWRITE) ? 1 : 0;
+    p.scale = 1.0f / sqrtf(static_cast<float>(a->head));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dt == DType::bf16 ? launch_bwd_16bit<Bf16>(s, p, (int)a->head, a->mask_mode)
+        : launch_bwd_16bit<Fp16>(s, p, (int)a->head, a->mask_mode);
+}
+
+static int flash_bwd_call(DType dt, void *stream, int64_t seq, int64_t head,
+        int64_t batch, const void *K, const void *Q, const void *V, const void *A,
+        const void *dA, const void *mask, const float *lse, void *scratch_dQ,
+        void *dK, void *dQ, void *dV)
+{
+    nntile_hip_sdpa_bwd_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.q_seq = a.k_seq = seq;
+    a.head = head;
+    a.batch = a.n_batch = batch;
+    a.kv_group = 1;
+    a.mask_mode = NNTILE_HIP_MASK_ADDITIVE;
+    a.K = K;
+    a.Q = Q;
+    a.V = V;
+    a.A = A;
+    a.dA = dA;
+    a.mask = mask;
+    a.lse = lse;
+    a.dK = dK;
+    a.dQ = dQ;
+    a.dV = dV;
+    // the scratch tile of dQ (seq*head*batch 16-bit values) holds the row dots
+    a.workspace = scratch_dQ;
+    a.workspace_bytes = (size_t)seq * (size_t)head * (size_t)batch * 2;
+    return bwd_call(dt, stream, &a);
 }
 
 static int flash_call(DType dt, void *stream, int64_t seq, int64_t head,
@@ -446,6 +541,45 @@ void nntile_hip_flash_sdpa_fwd_codelet_fp16(void *buffers[], void *cl_args)
 void nntile_hip_flash_sdpa_fwd_codelet_fp32(void *buffers[], void *cl_args)
 {
     codelet_call(DType::fp32, "nntile_flash_sdpa_fwd_hip_fp32", buffers, cl_args);
+}
+
+size_t nntile_hip_sdpa_bwd_workspace_bytes(int64_t q_seq, int64_t batch)
+{
+    if(q_seq <= 0 || batch <= 0)
+    {
+        return 0;
+    }
+    return (size_t)q_seq * (size_t)batch * sizeof(float);
+}
+
+int nntile_hip_sdpa_bwd_tile_bf16(void *stream, const nntile_hip_sdpa_bwd_args *args)
+{
+    return bwd_call(DType::bf16, stream, args);
+}
+
+int nntile_hip_sdpa_bwd_tile_fp16(void *stream, const nntile_hip_sdpa_bwd_args *args)
+{
+    return bwd_call(DType::fp16, stream, args);
+}
+
+int nntile_hip_flash_sdpa_bwd_bf16(void *stream, int64_t seq, int64_t head,
+        int64_t batch, const uint16_t *K, const uint16_t *Q, const uint16_t *V,
+        const uint16_t *A, const uint16_t *dA, const uint16_t *mask,
+        const float *lse, uint16_t *, uint16_t *scratch_dQ, uint16_t *,
+        uint16_t *dK, uint16_t *dQ, uint16_t *dV)
+{
+    return flash_bwd_call(DType::bf16, stream, seq, head, batch, K, Q, V, A, dA, mask,
+            lse, scratch_dQ, dK, dQ, dV);
+}
+
+int nntile_hip_flash_sdpa_bwd_fp16(void *stream, int64_t seq, int64_t head,
+        int64_t batch, const uint16_t *K, const uint16_t *Q, const uint16_t *V,
+        const uint16_t *A, const uint16_t *dA, const uint16_t *mask,
+        const float *lse, uint16_t *, uint16_t *scratch_dQ, uint16_t *,
+        uint16_t *dK, uint16_t *dQ, uint16_t *dV)
+{
+    return flash_bwd_call(DType::fp16, stream, seq, head, batch, K, Q, V, A, dA, mask,
+            lse, scratch_dQ, dK, dQ, dV);
 }
 
 const char *nntile_hip_sdpa_version(void)

@@ -1,0 +1,756 @@
+// Scaled dot-product attention backward for 16-bit tiles on gfx950, in the
+// flash form: the forward output A and the logsumexp are inputs, the
+// probabilities are recomputed from them,
+//
+//   P[q,k]  = exp(scale q.k + mask[q,k] - lse[q])        D[q] = dA[q,:] . A[q,:]
+//   dP[q,k] = dA[q,:] . V[k,:]                           dS   = P (dP - D)
+//   dV[k,:] += sum_q P[q,k] dA[q,:]      dQ[q,:] += scale sum_k dS[q,k] K[k,:]
+//   dK[k,:] += scale sum_q dS[q,k] Q[q,:]
+//
+// (include/nntile/kernel/flash_sdpa_bwd_cudnn/cuda.hh:44-68 is the interface
+// this replaces; tests/kernel/flash_sdpa_bwd_cudnn.cc:174-262 the arithmetic).
+// Two kernels, no atomics, results independent of timing:
+//
+//  * sdpa_bwd_dq_kernel: a workgroup owns 128 queries (a wavefront 32, a lane
+//    one query) and walks the keys in steps of 64, as the forward kernel does:
+//    S^T = K Q^T and dP^T = V dA^T with Q and dA fragments in registers and K, V
+//    rows from LDS; dS^T packed to 16 bits is the B operand of
+//    dQ^T += K^T dS^T, whose A operand comes through the transposing LDS read.
+//    It also writes D for the second kernel.
+//  * sdpa_bwd_dkv_kernel: a workgroup owns 128 keys (a lane one key) and walks
+//    the queries of every head of its group in steps of 64: S = Q K^T and
+//    dP = dA V^T with K and V fragments in registers and Q, dA rows from LDS;
+//    dV^T += dA^T P and dK^T += Q^T dS through transposing reads of the same
+//    two LDS tiles.
+//
+// K, V, Q, dA steps go from global memory straight into LDS, double buffered;
+// 16-byte chunk c of row r of a step sits at chunk position
+// c ^ ((r / RPL) % CPR), which keeps the row reads free of bank conflicts and
+// the transposing reads nearly so.
+#include <type_traits>
+
+#include "sdpa_common.hpp"
+
+namespace nntile_hip
+{
+
+constexpr int kBwdRows = 128;       // queries (dQ kernel) / keys (dK,dV kernel) per workgroup
+constexpr int kBwdStep = 64;        // rows of the other axis per step
+constexpr int kBwdThreads = 256;
+
+__device__ __forceinline__ u32x2 bwd_lds_read_tr16(const char *lds_ptr)
+{
+    typedef __attribute__((ext_vector_type(4))) short s16x4;
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(lds_ptr));
+    return __builtin_bit_cast(u32x2, v);
+}
+
+// What the two kernels share: the geometry of a 64-row step in LDS.
+template<int HEAD>
+struct BwdTile
+{
+    static constexpr int KSTEPS = HEAD / 16;       // MFMA steps along head
+    static constexpr int DBLOCKS = HEAD / 32;      // 32-row blocks of a transposed gradient
+    static constexpr int RB = HEAD * 2;            // bytes per row
+    static constexpr int CPR = HEAD / 8;           // 16-byte chunks per row
+    static constexpr int RPL = 16 / CPR;           // rows per 256-byte line of LDS banks
+    static constexpr int ROWS_PER_LOAD = 1024 / RB;
+    static constexpr int LOADS = kBwdStep / ROWS_PER_LOAD;
+    static constexpr int LOADS_PER_WAVE = LOADS / 4;
+    static constexpr int BYTES = kBwdStep * RB;
+    static_assert(LOADS_PER_WAVE >= 1, "head size does not fit this tiling");
+
+    static __device__ __forceinline__ int swz(int r)
+    {
+        return (r / RPL) % CPR;
+    }
+};
+
+// The registers of a 32x32 accumulator tile of lane (col, half): register r is
+// row 8*(r/4) + 4*half + r%4 of the tile, column col.
+__device__ __forceinline__ int tile_row(int r, int half)
+{
+    return 8 * (r >> 2) + 4 * half + (r & 3);
+}
+
+// ---------------------------------------------------------------------------------
+template<typename T, int HEAD, int MODE>
+__global__ __launch_bounds__(kBwdThreads, 2)
+void sdpa_bwd_dq_kernel(const BwdParams p)
+{
+    typedef typename T::vec8 vec8;
+    typedef BwdTile<HEAD> G;
+    constexpr int KSTEPS = G::KSTEPS, DBLOCKS = G::DBLOCKS, RB = G::RB, CPR = G::CPR;
+    constexpr int LOADS_PER_WAVE = G::LOADS_PER_WAVE, ROWS_PER_LOAD = G::ROWS_PER_LOAD;
+    constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
+            || MODE == NNTILE_HIP_MASK_BOOL);
+
+    __shared__ __attribute__((aligned(1024))) char lds_k0[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_k1[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_v0[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_v1[G::BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int col = lane & 31;
+    const int half = lane >> 5;
+
+    const int q_blocks = (int)((p.q_seq + kBwdRows - 1) / kBwdRows);
+    const int b = blockIdx.x / q_blocks;
+    const int q_row0 = (blockIdx.x % q_blocks) * kBwdRows;
+    const int kvb = kv_entry(b, p.n_batch, p.kv_group);
+    const int q_seq = (int)p.q_seq, k_seq = (int)p.k_seq;
+    const int my_q = q_row0 + wave * 32 + col;
+    const bool q_ok = my_q < q_seq;
+    const int64_t q_off = ((int64_t)b * q_seq + (q_ok ? my_q : 0)) * HEAD;
+
+    // Q and dA fragments (B operands) and the row dot D = dA . A
+    vec8 qf[KSTEPS], gf[KSTEPS];
+    float d_row = 0.0f;
+    {
+        const uint16_t *qs = static_cast<const uint16_t *>(p.Q) + q_off + half * 8;
+        const uint16_t *gs = static_cast<const uint16_t *>(p.dA) + q_off + half * 8;
+        const uint16_t *as = static_cast<const uint16_t *>(p.A) + q_off + half * 8;
+#pragma unroll
+        for(int ks = 0; ks < KSTEPS; ++ks)
+        {
+            u32x4 q = *reinterpret_cast<const u32x4 *>(qs + ks * 16);
+            u32x4 g = *reinterpret_cast<const u32x4 *>(gs + ks * 16);
+            u32x4 a = *reinterpret_cast<const u32x4 *>(as + ks * 16);
+            if(!q_ok)
+            {
+                q = u32x4{0, 0, 0, 0};
+                g = u32x4{0, 0, 0, 0};
+                a = u32x4{0, 0, 0, 0};
+            }
+            qf[ks] = __builtin_bit_cast(vec8, q);
+            gf[ks] = __builtin_bit_cast(vec8, g);
+#pragma unroll
+            for(int e = 0; e < 4; ++e)
+            {
+                d_row += T::to_float((uint16_t)(g[e] & 0xffffu)) * T::to_float((uint16_t)(a[e] & 0xffffu));
+                d_row += T::to_float((uint16_t)(g[e] >> 16)) * T::to_float((uint16_t)(a[e] >> 16));
+            }
+        }
+    }
+    d_row = sum_across_halves(d_row);
+    const float lse_q = q_ok ? p.lse[(int64_t)b * q_seq + my_q] : neg_inf();
+    // exponent offset in log2 units; a row that saw nothing has P = 0
+    const float lse2 = (lse_q == neg_inf()) ? __builtin_huge_valf() : lse_q * kLog2e;
+    if(p.D != nullptr && q_ok && half == 0)
+    {
+        p.D[(int64_t)b * q_seq + my_q] = d_row;
+    }
+
+    // ---- which keys ---------------------------------------------------------------
+    // key row kg is visible to query row q iff kg <= rel + q (causal)
+    int64_t rel64 = p.q_pos0 + p.causal_offset - p.k_pos0;
+    rel64 = max((int64_t)-(1 << 30), min(rel64, (int64_t)(1 << 30)));
+    const int rel = (int)rel64;
+    int n_steps = (k_seq + kBwdStep - 1) / kBwdStep;
+    if(MODE == NNTILE_HIP_MASK_CAUSAL)
+    {
+        const int hi = min(rel + min(q_row0 + kBwdRows, q_seq) - 1, k_seq - 1);
+        n_steps = hi < 0 ? 0 : min(n_steps, hi / kBwdStep + 1);
+    }
+    const int my_lim = rel + my_q;          // last visible key of this lane's query
+
+    // ---- LDS addresses --------------------------------------------------------------
+    uint32_t ld_goff[LOADS_PER_WAVE];
+    int ld_row[LOADS_PER_WAVE];
+    const int ld_cpos = lane % CPR;
+#pragma unroll
+    for(int i = 0; i < LOADS_PER_WAVE; ++i)
+    {
+        const int r = (wave * LOADS_PER_WAVE + i) * ROWS_PER_LOAD + lane / CPR;
+        ld_row[i] = r;
+        ld_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ G::swz(r)) * 16);
+    }
+    // row operand: lane (col, half) reads row mb*32+col, logical chunk 2*ks+half
+    uint32_t row_raddr[2][KSTEPS];
+#pragma unroll
+    for(int mb = 0; mb < 2; ++mb)
+    {
+        const int r = mb * 32 + col;
+#pragma unroll
+        for(int ks = 0; ks < KSTEPS; ++ks)
+        {
+            row_raddr[mb][ks] = (uint32_t)(r * RB + ((2 * ks + half) ^ G::swz(r)) * 16);
+        }
+    }
+    // transposed operand: within a 16-lane block lane i addresses row j = i/4 and
+    // head values 4*(i%4)..+3 of the block's 16; lanes 16..31 take the upper 16
+    // head values of a 32-row block, the lane half the rows 4..7.  For the
+    // 16-row sub-step t the two reads cover rows 16t + 4*half + j and + 8; the
+    // swizzle of a row does not depend on t, so 16t goes into the immediate.
+    uint32_t tr_raddr[2][DBLOCKS];
+    {
+        const int i16 = lane & 15, dblk = (lane >> 4) & 1;
+        const int j = i16 >> 2, r4 = i16 & 3;
+#pragma unroll
+        for(int a = 0; a < 2; ++a)
+        {
+            const int r = 4 * half + j + 8 * a;
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+                const int c = 4 * db + 2 * dblk + (r4 >> 1);
+                tr_raddr[a][db] = (uint32_t)(r * RB + (c ^ G::swz(r)) * 16 + 8 * (r4 & 1));
+            }
+        }
+    }
+
+    const char *Kb = static_cast<const char *>(p.K) + (int64_t)kvb * k_seq * RB;
+    const char *Vb = static_cast<const char *>(p.V) + (int64_t)kvb * k_seq * RB;
+    // loads of key step g; rows past the end are clamped to the last row
+    // (their probabilities are exactly 0)
+    auto fetch = [&](int g, char *kdst_base, char *vdst_base)
+    {
+        const int row0 = g * kBwdStep;
+        const int last = min(kBwdStep, k_seq - row0) - 1;
+        char *kdst = kdst_base + wave_u * LOADS_PER_WAVE * 1024;
+        char *vdst = vdst_base + wave_u * LOADS_PER_WAVE * 1024;
+#pragma unroll
+        for(int i = 0; i < LOADS_PER_WAVE; ++i)
+        {
+            const uint32_t back = (uint32_t)(max(ld_row[i] - last, 0) * RB);
+            load_to_lds16<0, false>(Kb + (int64_t)row0 * RB, ld_goff[i] - back, kdst + i * 1024);
+            load_to_lds16<0, false>(Vb + (int64_t)row0 * RB, ld_goff[i] - back, vdst + i * 1024);
+        }
+    };
+
+    f32x16 acc[DBLOCKS];
+#pragma unroll
+    for(int db = 0; db < DBLOCKS; ++db)
+    {
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+        {
+            acc[db][r] = 0.0f;
+        }
+    }
+    const float c = p.scale * kLog2e;
+    const int64_t mask_row = (int64_t)(q_ok ? my_q : 0) * p.mask_ld;
+
+    if(n_steps > 0)
+    {
+        fetch(0, lds_k0, lds_v0);
+    }
+    auto step = [&](int g, auto buf_tag) __attribute__((always_inline))
+    {
+        constexpr int BUF = decltype(buf_tag)::value;
+        const char *Ks = BUF ? lds_k1 : lds_k0;
+        const char *Vs = BUF ? lds_v1 : lds_v0;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if(g + 1 < n_steps)
+        {
+            fetch(g + 1, BUF ? lds_k0 : lds_k1, BUF ? lds_v0 : lds_v1);
+        }
+        const int kg0 = g * kBwdStep;
+        const int keys_here = min(kBwdStep, k_seq - kg0);
+
+        // ---- S^T = K Q^T, dP^T = V dA^T -------------------------------------------------
+        // (one 32-key block at a time: half the accumulators live)
+        // ---- P^T, dS^T: register r of block mb is key mb*32 + tile_row(r, half) ------------
+        uint32_t ds_pk[2][8];
+        int lim = keys_here - 1;
+        if(MODE == NNTILE_HIP_MASK_CAUSAL)
+        {
+            lim = min(lim, my_lim - kg0);
+        }
+#pragma unroll
+        for(int mb = 0; mb < 2; ++mb)
+        {
+            f32x16 sv, dpv;
+#pragma unroll
+            for(int r = 0; r < 16; ++r)
+            {
+                sv[r] = 0.0f;
+                dpv[r] = 0.0f;
+            }
+#pragma unroll
+            for(int ks = 0; ks < KSTEPS; ++ks)
+            {
+                const vec8 ka = *reinterpret_cast<const vec8 *>(Ks + row_raddr[mb][ks]);
+                const vec8 va = *reinterpret_cast<const vec8 *>(Vs + row_raddr[mb][ks]);
+                sv = T::mfma(ka, qf[ks], sv);
+                dpv = T::mfma(va, gf[ks], dpv);
+            }
+            float dsv[16];
+#pragma unroll
+            for(int r = 0; r < 16; ++r)
+            {
+                const int key = mb * 32 + tile_row(r, half);
+                float e = fmaf(sv[r], c, -lse2);
+                bool visible = key <= lim;
+                if(EXPLICIT)
+                {
+                    const int64_t mi = mask_row + kg0 + min(key, keys_here - 1);
+                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                    {
+                        const float add = T::to_float(static_cast<const uint16_t *>(p.mask)[mi]);
+                        visible = visible && (add != neg_inf());
+                        e = fmaf(add, kLog2e, e);
+                    }
+                    else
+                    {
+                        visible = visible && (static_cast<const uint8_t *>(p.mask)[mi] != 0);
+                    }
+                }
+                const float pr = visible ? fast_exp2(e) : 0.0f;
+                dsv[r] = pr * (dpv[r] - d_row);
+            }
+#pragma unroll
+            for(int k = 0; k < 8; ++k)
+            {
+                ds_pk[mb][k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
+            }
+        }
+
+        // ---- dQ^T += K^T dS^T: four sub-steps of 16 keys --------------------------------
+#pragma unroll
+        for(int t = 0; t < 4; ++t)
+        {
+            const int mb = t >> 1, tt = t & 1;
+            const u32x4 braw = {ds_pk[mb][4 * tt], ds_pk[mb][4 * tt + 1],
+                ds_pk[mb][4 * tt + 2], ds_pk[mb][4 * tt + 3]};
+            const vec8 bop = __builtin_bit_cast(vec8, braw);
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+                const u32x2 lo = bwd_lds_read_tr16(Ks + tr_raddr[0][db] + (16 * t) * RB);
+                const u32x2 hi = bwd_lds_read_tr16(Ks + tr_raddr[1][db] + (16 * t) * RB);
+                const u32x4 araw = {lo[0], lo[1], hi[0], hi[1]};
+                acc[db] = T::mfma(__builtin_bit_cast(vec8, araw), bop, acc[db]);
+            }
+        }
+    };
+    for(int g = 0; g < n_steps; g += 2)
+    {
+        step(g, std::integral_constant<int, 0>{});
+        if(g + 1 < n_steps)
+        {
+            step(g + 1, std::integral_constant<int, 1>{});
+        }
+    }
+
+    // ---- dQ (+)= scale acc: register r of block db is head value
+    // db*32 + tile_row(r, half); four consecutive ones per 8-byte store ----------------
+    if(!q_ok)
+    {
+        return;
+    }
+    uint16_t *dst = static_cast<uint16_t *>(p.dQ) + q_off;
+#pragma unroll
+    for(int db = 0; db < DBLOCKS; ++db)
+    {
+#pragma unroll
+        for(int rg = 0; rg < 4; ++rg)
+        {
+            uint16_t *ptr = dst + db * 32 + 8 * rg + 4 * half;
+            float v[4];
+#pragma unroll
+            for(int e = 0; e < 4; ++e)
+            {
+                v[e] = acc[db][4 * rg + e] * p.scale;
+            }
+            if(!p.overwrite)
+            {
+                const u32x2 old = *reinterpret_cast<const u32x2 *>(ptr);
+                v[0] += T::to_float((uint16_t)(old[0] & 0xffffu));
+                v[1] += T::to_float((uint16_t)(old[0] >> 16));
+                v[2] += T::to_float((uint16_t)(old[1] & 0xffffu));
+                v[3] += T::to_float((uint16_t)(old[1] >> 16));
+            }
+            u32x2 out;
+            out[0] = T::pack2(v[0], v[1]);
+            out[1] = T::pack2(v[2], v[3]);
+            *reinterpret_cast<u32x2 *>(ptr) = out;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+template<typename T, int HEAD, int MODE>
+__global__ __launch_bounds__(kBwdThreads, 1)
+void sdpa_bwd_dkv_kernel(const BwdParams p)
+{
+    typedef typename T::vec8 vec8;
+    typedef BwdTile<HEAD> G;
+    constexpr int KSTEPS = G::KSTEPS, DBLOCKS = G::DBLOCKS, RB = G::RB, CPR = G::CPR;
+    constexpr int LOADS_PER_WAVE = G::LOADS_PER_WAVE, ROWS_PER_LOAD = G::ROWS_PER_LOAD;
+    constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
+            || MODE == NNTILE_HIP_MASK_BOOL);
+
+    __shared__ __attribute__((aligned(1024))) char lds_q0[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_q1[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_g0[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_g1[G::BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int col = lane & 31;
+    const int half = lane >> 5;
+
+    const int q_seq = (int)p.q_seq, k_seq = (int)p.k_seq;
+    const int k_blocks = (k_seq + kBwdRows - 1) / kBwdRows;
+    const int kvb = blockIdx.x / k_blocks;          // nb + n_batch*hkv
+    const int k_row0 = (blockIdx.x % k_blocks) * kBwdRows;
+    const int nb = kvb % p.n_batch, hkv = kvb / p.n_batch;
+    const int my_k = k_row0 + wave * 32 + col;
+    const bool k_ok = my_k < k_seq;
+    const int64_t k_off = ((int64_t)kvb * k_seq + (k_ok ? my_k : 0)) * HEAD;
+
+    // K and V fragments (B operands): lane (col, half) holds head values 16*ks + 8*half..+7
+    vec8 kf[KSTEPS], vf[KSTEPS];
+    {
+        const uint16_t *ks_ = static_cast<const uint16_t *>(p.K) + k_off + half * 8;
+        const uint16_t *vs_ = static_cast<const uint16_t *>(p.V) + k_off + half * 8;
+#pragma unroll
+        for(int ks = 0; ks < KSTEPS; ++ks)
+        {
+            u32x4 k = *reinterpret_cast<const u32x4 *>(ks_ + ks * 16);
+            u32x4 v = *reinterpret_cast<const u32x4 *>(vs_ + ks * 16);
+            if(!k_ok)
+            {
+                k = u32x4{0, 0, 0, 0};
+                v = u32x4{0, 0, 0, 0};
+            }
+            kf[ks] = __builtin_bit_cast(vec8, k);
+            vf[ks] = __builtin_bit_cast(vec8, v);
+        }
+    }
+
+    // key row kg is visible to query row q iff kg <= rel + q (causal)
+    int64_t rel64 = p.q_pos0 + p.causal_offset - p.k_pos0;
+    rel64 = max((int64_t)-(1 << 30), min(rel64, (int64_t)(1 << 30)));
+    const int rel = (int)rel64;
+    const int n_steps = (q_seq + kBwdStep - 1) / kBwdStep;
+    int first_step = 0;
+    if(MODE == NNTILE_HIP_MASK_CAUSAL)
+    {
+        // the first query that sees the workgroup's first key
+        const int q_lo = max(k_row0 - rel, 0);
+        first_step = min(q_lo / kBwdStep, n_steps);
+    }
+
+    uint32_t ld_goff[LOADS_PER_WAVE];
+    int ld_row[LOADS_PER_WAVE];
+    const int ld_cpos = lane % CPR;
+#pragma unroll
+    for(int i = 0; i < LOADS_PER_WAVE; ++i)
+    {
+        const int r = (wave * LOADS_PER_WAVE + i) * ROWS_PER_LOAD + lane / CPR;
+        ld_row[i] = r;
+        ld_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ G::swz(r)) * 16);
+    }
+    uint32_t row_raddr[2][KSTEPS];
+#pragma unroll
+    for(int mb = 0; mb < 2; ++mb)
+    {
+        const int r = mb * 32 + col;
+#pragma unroll
+        for(int ks = 0; ks < KSTEPS; ++ks)
+        {
+            row_raddr[mb][ks] = (uint32_t)(r * RB + ((2 * ks + half) ^ G::swz(r)) * 16);
+        }
+    }
+    uint32_t tr_raddr[2][DBLOCKS];
+    {
+        const int i16 = lane & 15, dblk = (lane >> 4) & 1;
+        const int j = i16 >> 2, r4 = i16 & 3;
+#pragma unroll
+        for(int a = 0; a < 2; ++a)
+        {
+            const int r = 4 * half + j + 8 * a;
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+                const int c = 4 * db + 2 * dblk + (r4 >> 1);
+                tr_raddr[a][db] = (uint32_t)(r * RB + (c ^ G::swz(r)) * 16 + 8 * (r4 & 1));
+            }
+        }
+    }
+
+    f32x16 dk[DBLOCKS], dv[DBLOCKS];
+#pragma unroll
+    for(int db = 0; db < DBLOCKS; ++db)
+    {
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+        {
+            dk[db][r] = 0.0f;
+            dv[db][r] = 0.0f;
+        }
+    }
+    const float c = p.scale * kLog2e;
+    const int n_local = n_steps - first_step;       // steps per head of the group
+    const int total = n_local * p.kv_group;         // steps of the whole walk
+
+    // walk position i -> (head g of the group, query step)
+    auto locate = [&](int i, int &bq, int &qs)
+    {
+        const int g = i / n_local;
+        qs = first_step + i % n_local;
+        bq = nb + p.n_batch * (g + p.kv_group * hkv);
+    };
+    auto fetch = [&](int i, char *qdst_base, char *gdst_base)
+    {
+        int bq, qs;
+        locate(i, bq, qs);
+        const int row0 = qs * kBwdStep;
+        const int last = min(kBwdStep, q_seq - row0) - 1;
+        const char *Qp = static_cast<const char *>(p.Q) + ((int64_t)bq * q_seq + row0) * RB;
+        const char *Gp = static_cast<const char *>(p.dA) + ((int64_t)bq * q_seq + row0) * RB;
+        char *qdst = qdst_base + wave_u * LOADS_PER_WAVE * 1024;
+        char *gdst = gdst_base + wave_u * LOADS_PER_WAVE * 1024;
+#pragma unroll
+        for(int j = 0; j < LOADS_PER_WAVE; ++j)
+        {
+            const uint32_t back = (uint32_t)(max(ld_row[j] - last, 0) * RB);
+            load_to_lds16<0, false>(Qp, ld_goff[j] - back, qdst + j * 1024);
+            load_to_lds16<0, false>(Gp, ld_goff[j] - back, gdst + j * 1024);
+        }
+    };
+
+    if(total > 0)
+    {
+        fetch(0, lds_q0, lds_g0);
+    }
+    auto step = [&](int i, auto buf_tag) __attribute__((always_inline))
+    {
+        constexpr int BUF = decltype(buf_tag)::value;
+        const char *Qs = BUF ? lds_q1 : lds_q0;
+        const char *Gs = BUF ? lds_g1 : lds_g0;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if(i + 1 < total)
+        {
+            fetch(i + 1, BUF ? lds_q0 : lds_q1, BUF ? lds_g0 : lds_g1);
+        }
+        int bq, qs;
+        locate(i, bq, qs);
+        const int q0 = qs * kBwdStep;
+        const int rows_here = min(kBwdStep, q_seq - q0);
+        const float *lse_p = p.lse + (int64_t)bq * q_seq + q0;
+        const float *d_p = p.D + (int64_t)bq * q_seq + q0;
+
+        // ---- S = Q K^T, dP = dA V^T: rows are queries, the lane's column its key ----------
+        // (one 32-query block at a time: half the accumulators live)
+        // ---- P, dS: register r of block mb is query q0 + mb*32 + tile_row(r, half) ----------
+        uint32_t p_pk[2][8], ds_pk[2][8];
+#pragma unroll
+        for(int mb = 0; mb < 2; ++mb)
+        {
+            f32x16 sv, dpv;
+#pragma unroll
+            for(int r = 0; r < 16; ++r)
+            {
+                sv[r] = 0.0f;
+                dpv[r] = 0.0f;
+            }
+#pragma unroll
+            for(int ks = 0; ks < KSTEPS; ++ks)
+            {
+                const vec8 qa = *reinterpret_cast<const vec8 *>(Qs + row_raddr[mb][ks]);
+                const vec8 ga = *reinterpret_cast<const vec8 *>(Gs + row_raddr[mb][ks]);
+                sv = T::mfma(qa, kf[ks], sv);
+                dpv = T::mfma(ga, vf[ks], dpv);
+            }
+            float pv[16], dsv[16];
+#pragma unroll
+            for(int rg = 0; rg < 4; ++rg)
+            {
+                // four consecutive queries: their lse and D in one load each
+                // (rows past the end are clamped and hidden below)
+                const int qr0 = mb * 32 + 8 * rg + 4 * half;
+                float lse4[4], d4[4];
+#pragma unroll
+                for(int e = 0; e < 4; ++e)
+                {
+                    const int qi = min(qr0 + e, rows_here - 1);
+                    lse4[e] = lse_p[qi];
+                    d4[e] = d_p[qi];
+                }
+#pragma unroll
+                for(int e = 0; e < 4; ++e)
+                {
+                    const int r = 4 * rg + e;
+                    const int qr = qr0 + e;                 // query row within the step
+                    const float lse2 = (lse4[e] == neg_inf()) ? __builtin_huge_valf()
+                        : lse4[e] * kLog2e;
+                    float ex = fmaf(sv[r], c, -lse2);
+                    bool visible = k_ok && qr < rows_here;
+                    if(MODE == NNTILE_HIP_MASK_CAUSAL)
+                    {
+                        visible = visible && (my_k <= rel + q0 + qr);
+                    }
+                    if(EXPLICIT)
+                    {
+                        const int64_t mi = (int64_t)(q0 + min(qr, rows_here - 1)) * p.mask_ld
+                            + (k_ok ? my_k : 0);
+                        if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                        {
+                            const float add = T::to_float(
+                                    static_cast<const uint16_t *>(p.mask)[mi]);
+                            visible = visible && (add != neg_inf());
+                            ex = fmaf(add, kLog2e, ex);
+                        }
+                        else
+                        {
+                            visible = visible
+                                && (static_cast<const uint8_t *>(p.mask)[mi] != 0);
+                        }
+                    }
+                    pv[r] = visible ? fast_exp2(ex) : 0.0f;
+                    dsv[r] = pv[r] * (dpv[r] - d4[e]);
+                }
+            }
+#pragma unroll
+            for(int k = 0; k < 8; ++k)
+            {
+                p_pk[mb][k] = T::pack2(pv[2 * k], pv[2 * k + 1]);
+                ds_pk[mb][k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
+            }
+        }
+
+        // ---- dV^T += dA^T P, dK^T += Q^T dS: four sub-steps of 16 queries -------------------
+#pragma unroll
+        for(int t = 0; t < 4; ++t)
+        {
+            const int mb = t >> 1, tt = t & 1;
+            const u32x4 praw = {p_pk[mb][4 * tt], p_pk[mb][4 * tt + 1],
+                p_pk[mb][4 * tt + 2], p_pk[mb][4 * tt + 3]};
+            const u32x4 sraw = {ds_pk[mb][4 * tt], ds_pk[mb][4 * tt + 1],
+                ds_pk[mb][4 * tt + 2], ds_pk[mb][4 * tt + 3]};
+            const vec8 pb = __builtin_bit_cast(vec8, praw);
+            const vec8 sb = __builtin_bit_cast(vec8, sraw);
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+                const u32x2 glo = bwd_lds_read_tr16(Gs + tr_raddr[0][db] + (16 * t) * RB);
+                const u32x2 ghi = bwd_lds_read_tr16(Gs + tr_raddr[1][db] + (16 * t) * RB);
+                const u32x4 graw = {glo[0], glo[1], ghi[0], ghi[1]};
+                dv[db] = T::mfma(__builtin_bit_cast(vec8, graw), pb, dv[db]);
+                const u32x2 qlo = bwd_lds_read_tr16(Qs + tr_raddr[0][db] + (16 * t) * RB);
+                const u32x2 qhi = bwd_lds_read_tr16(Qs + tr_raddr[1][db] + (16 * t) * RB);
+                const u32x4 qraw = {qlo[0], qlo[1], qhi[0], qhi[1]};
+                dk[db] = T::mfma(__builtin_bit_cast(vec8, qraw), sb, dk[db]);
+            }
+        }
+    };
+    for(int i = 0; i < total; i += 2)
+    {
+        step(i, std::integral_constant<int, 0>{});
+        if(i + 1 < total)
+        {
+            step(i + 1, std::integral_constant<int, 1>{});
+        }
+    }
+
+    // ---- dK (+)= scale dk, dV (+)= dv -------------------------------------------------
+    if(!k_ok)
+    {
+        return;
+    }
+    auto store = [&](void *base, const f32x16 (&acc)[DBLOCKS], float factor)
+    {
+        uint16_t *dst = static_cast<uint16_t *>(base) + k_off;
+#pragma unroll
+        for(int db = 0; db < DBLOCKS; ++db)
+        {
+#pragma unroll
+            for(int rg = 0; rg < 4; ++rg)
+            {
+                uint16_t *ptr = dst + db * 32 + 8 * rg + 4 * half;
+                float v[4];
+#pragma unroll
+                for(int e = 0; e < 4; ++e)
+                {
+                    v[e] = acc[db][4 * rg + e] * factor;
+                }
+                if(!p.overwrite)
+                {
+                    const u32x2 old = *reinterpret_cast<const u32x2 *>(ptr);
+                    v[0] += T::to_float((uint16_t)(old[0] & 0xffffu));
+                    v[1] += T::to_float((uint16_t)(old[0] >> 16));
+                    v[2] += T::to_float((uint16_t)(old[1] & 0xffffu));
+                    v[3] += T::to_float((uint16_t)(old[1] >> 16));
+                }
+                u32x2 out;
+                out[0] = T::pack2(v[0], v[1]);
+                out[1] = T::pack2(v[2], v[3]);
+                *reinterpret_cast<u32x2 *>(ptr) = out;
+            }
+        }
+    };
+    store(p.dK, dk, p.scale);
+    store(p.dV, dv, 1.0f);
+}
+
+template<typename T, int HEAD, int MODE>
+static int launch_bwd_mode(hipStream_t stream, const BwdParams &p)
+{
+    const int64_t q_blocks = (p.q_seq + kBwdRows - 1) / kBwdRows;
+    const int64_t k_blocks = (p.k_seq + kBwdRows - 1) / kBwdRows;
+    const int64_t kv_batch = p.batch / p.kv_group;
+    const int64_t n_dq = (int64_t)p.batch * q_blocks, n_dkv = kv_batch * k_blocks;
+    if(n_dq <= 0 || n_dkv <= 0 || n_dq > 0x7fffffff || n_dkv > 0x7fffffff)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, HEAD, MODE>), dim3((unsigned)n_dq),
+            dim3(kBwdThreads), 0, stream, p);
+    if(hipGetLastError() != hipSuccess)
+    {
+        return NNTILE_HIP_ELAUNCH;
+    }
+    hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, HEAD, MODE>), dim3((unsigned)n_dkv),
+            dim3(kBwdThreads), 0, stream, p);
+    return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
+}
+
+template<typename T, int HEAD>
+static int launch_bwd_head(hipStream_t stream, const BwdParams &p, int mode)
+{
+    switch(mode)
+    {
+        case NNTILE_HIP_MASK_ADDITIVE:
+            return launch_bwd_mode<T, HEAD, NNTILE_HIP_MASK_ADDITIVE>(stream, p);
+        case NNTILE_HIP_MASK_NONE:
+            return launch_bwd_mode<T, HEAD, NNTILE_HIP_MASK_NONE>(stream, p);
+        case NNTILE_HIP_MASK_CAUSAL:
+            return launch_bwd_mode<T, HEAD, NNTILE_HIP_MASK_CAUSAL>(stream, p);
+        case NNTILE_HIP_MASK_BOOL:
+            return launch_bwd_mode<T, HEAD, NNTILE_HIP_MASK_BOOL>(stream, p);
+        default:
+            return NNTILE_HIP_EINVAL;
+    }
+}
+
+template<typename T>
+int launch_bwd_16bit(hipStream_t stream, const BwdParams &p, int head, int mode)
+{
+    switch(head)
+    {
+        case 32:
+            return launch_bwd_head<T, 32>(stream, p, mode);
+        case 64:
+            return launch_bwd_head<T, 64>(stream, p, mode);
+        case 128:
+            return launch_bwd_head<T, 128>(stream, p, mode);
+        default:
+            return NNTILE_HIP_EUNSUPPORTED;
+    }
+}
+
+template int launch_bwd_16bit<Bf16>(hipStream_t, const BwdParams &, int, int);
+template int launch_bwd_16bit<Fp16>(hipStream_t, const BwdParams &, int, int);
+
+} // namespace nntile_hip

@@ -78,6 +78,24 @@ struct DecodeParams
     float scale;
 };
 
+// Kernel arguments of the backward kernels.  K, V, dK, dV: [head, k_seq,
+// n_batch, n_head_kv]; Q, A, dA, dQ: [head, q_seq, n_batch, kv_group,
+// n_head_kv]; lse and the row dots D = sum_h dA*A: [q_seq, batch] fp32.
+struct BwdParams
+{
+    int64_t q_seq, k_seq;
+    int64_t q_pos0, k_pos0, causal_offset;
+    int64_t mask_ld;
+    const void *mask;
+    const void *K, *Q, *V, *A, *dA;
+    const float *lse;
+    float *D;               // workspace: written by the dQ kernel, read by the dK/dV kernel
+    void *dK, *dQ, *dV;
+    int32_t batch, n_batch, kv_group;
+    int32_t overwrite;      // 1: write the gradients, 0: add to what is there
+    float scale;
+};
+
 // 16 bytes per lane from global memory straight into LDS: lane l reads
 // gaddr + OFF (its own address) and its bytes land at lds_dst + OFF + 16*l
 // (lds_dst is the same for the whole wavefront; it travels in M0).  Written

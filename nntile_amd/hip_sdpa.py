@@ -49,6 +49,17 @@ class GridArgs(ctypes.Structure):
                 ("A", _vp * MAX_TILES)]
 
 
+class BwdArgs(ctypes.Structure):
+    _fields_ = [("q_seq", _i64), ("k_seq", _i64), ("head", _i64),
+                ("batch", _i64), ("n_batch", _i64), ("kv_group", _i64),
+                ("mask_mode", ctypes.c_int32), ("flags", ctypes.c_int32),
+                ("q_pos0", _i64), ("k_pos0", _i64), ("causal_offset", _i64),
+                ("K", _vp), ("Q", _vp), ("V", _vp), ("A", _vp), ("dA", _vp),
+                ("mask", _vp), ("lse", _vp), ("dK", _vp), ("dQ", _vp),
+                ("dV", _vp), ("workspace", _vp),
+                ("workspace_bytes", ctypes.c_size_t)]
+
+
 class VariableInterface(ctypes.Structure):
     _fields_ = [("id", ctypes.c_int), ("ptr", ctypes.c_size_t),
                 ("dev_handle", ctypes.c_size_t), ("offset", ctypes.c_size_t),
@@ -67,6 +78,9 @@ EXPORTS = (
     + ["nntile_hip_sdpa_fwd_grid_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_fwd_decode_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_sdpa_fwd_decode_workspace_bytes"]
+    + ["nntile_hip_flash_sdpa_bwd_" + t for t in ("bf16", "fp16")]
+    + ["nntile_hip_sdpa_bwd_tile_" + t for t in ("bf16", "fp16")]
+    + ["nntile_hip_sdpa_bwd_workspace_bytes"]
     + ["nntile_hip_accumulate_attn_output_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_flash_sdpa_fwd_codelet_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_set_stream_provider", "nntile_hip_sdpa_version"])
@@ -102,6 +116,14 @@ def lib():
             f = getattr(L, "nntile_hip_sdpa_fwd_decode_" + t)
             f.argtypes = [_vp, ctypes.POINTER(TileArgs), _vp, ctypes.c_size_t]
             f.restype = ctypes.c_int
+            f = getattr(L, "nntile_hip_flash_sdpa_bwd_" + t)
+            f.argtypes = [_vp, _i64, _i64, _i64] + [_vp] * 13
+            f.restype = ctypes.c_int
+            f = getattr(L, "nntile_hip_sdpa_bwd_tile_" + t)
+            f.argtypes = [_vp, ctypes.POINTER(BwdArgs)]
+            f.restype = ctypes.c_int
+        L.nntile_hip_sdpa_bwd_workspace_bytes.argtypes = [_i64, _i64]
+        L.nntile_hip_sdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.argtypes = [ctypes.POINTER(TileArgs)]
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.restype = ctypes.c_size_t
         L.nntile_hip_set_stream_provider.argtypes = [_vp]
@@ -182,6 +204,46 @@ def sdpa_fwd_tile(K, Q, mask, lse, V, A, mask_mode, n_batch=None, kv_group=1,
                    k_pos0, causal_offset, flags)
     fn = getattr(lib(), "nntile_hip_sdpa_fwd_tile_" + dtype_name(Q))
     _check(fn(_stream(stream), ctypes.byref(a)), "sdpa_fwd_tile")
+
+
+def flash_sdpa_bwd(K, Q, V, A, dA, mask, lse, scratch_dQ, dK, dQ, dV, stream=None):
+    """One square tile with an additive mask: the reference's backward kernel
+    call (execute_graph) with its argument order; the gradients are added to
+    dK, dQ, dV.  scratch_dQ is the reference's scratch tile for dQ."""
+    _dev(K, Q, V, A, dA, mask, lse, scratch_dQ, dK, dQ, dV)
+    batch, seq, head = Q.shape
+    fn = getattr(lib(), "nntile_hip_flash_sdpa_bwd_" + dtype_name(Q))
+    _check(fn(_stream(stream), seq, head, batch, _ptr(K), _ptr(Q), _ptr(V), _ptr(A),
+              _ptr(dA), _ptr(mask), _ptr(lse), None, _ptr(scratch_dQ), None,
+              _ptr(dK), _ptr(dQ), _ptr(dV)), "flash_sdpa_bwd")
+
+
+def sdpa_bwd_tile(K, Q, V, A, dA, mask, lse, dK, dQ, dV, mask_mode, n_batch=None,
+                  kv_group=1, q_pos0=0, k_pos0=0, causal_offset=0, flags=0,
+                  workspace=None, stream=None):
+    """Backward of one (query tile, key tile) pair; the gradients are added to
+    dK, dQ, dV (written with flags=OVERWRITE)."""
+    _dev(K, Q, V, A, dA, mask, lse, dK, dQ, dV, workspace)
+    batch, q_seq, head = Q.shape
+    k_seq = K.shape[1]
+    need = lib().nntile_hip_sdpa_bwd_workspace_bytes(q_seq, batch)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
+    a = BwdArgs()
+    a.q_seq, a.k_seq, a.head, a.batch = q_seq, k_seq, head, batch
+    a.n_batch = batch if n_batch is None else n_batch
+    a.kv_group = kv_group
+    a.mask_mode = mask_mode
+    a.flags = flags
+    a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
+    a.K, a.Q, a.V, a.A, a.dA = (t.data_ptr() for t in (K, Q, V, A, dA))
+    a.mask = None if mask is None else mask.data_ptr()
+    a.lse = lse.data_ptr()
+    a.dK, a.dQ, a.dV = dK.data_ptr(), dQ.data_ptr(), dV.data_ptr()
+    a.workspace = workspace.data_ptr()
+    a.workspace_bytes = workspace.numel() * workspace.element_size()
+    fn = getattr(lib(), "nntile_hip_sdpa_bwd_tile_" + dtype_name(Q))
+    _check(fn(_stream(stream), ctypes.byref(a)), "sdpa_bwd_tile")
 
 
 def sdpa_fwd_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq,

@@ -1,0 +1,184 @@
+"""GPU parity of the backward kernels against the fp64 flash-form checker,
+through the C ABI.  Tolerances are the reference's own for its backward
+kernel (tests/kernel/flash_sdpa_bwd_cudnn.cc:312-327): relative Frobenius
+error 1e-2 for bf16 and 2e-3 for fp16."""
+import numpy as np
+import pytest
+import torch
+
+from nntile_amd import hip_sdpa, synth
+from . import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+BWD_TOL = {"bf16": 1e-2, "fp16": 2e-3}
+
+
+def _rounded(x, dtype):
+    return H.rounded(np.ascontiguousarray(x, dtype=np.float32), dtype)
+
+
+def _check(got, want, dtype, what):
+    err = H.rel_fro(H.to_np(got), want)
+    assert err < BWD_TOL[dtype], (what, err)
+
+
+def _reference_case(strategy, seq, head, batch, dtype):
+    """Inputs of the reference's backward test: PRESET by its formulas
+    (tests/kernel/flash_sdpa_bwd_cudnn.cc:112-127); RANDOM with its
+    distributions (:130-150: inputs uniform in (-0.5, 0.5), dA = K / 2, lse
+    uniform in (-1, 1)) from numpy's generator, since a C++ mt19937 stream is
+    not reproduced here.  A and lse do not belong to K, Q, V in either."""
+    total = batch * seq * head
+    shape = (batch, seq, head)
+    if strategy == "preset":
+        i = np.arange(total)
+        base = ((i % 23 - 11) * 0.04).astype(np.float32)
+        k, q, v, a = base, base * np.float32(0.7), base * np.float32(1.1), base * np.float32(-0.3)
+        g = (0.02 * ((i % 17) - 8)).astype(np.float32)
+        lse = ((np.arange(batch * seq) % 13 - 6) * 0.01).astype(np.float32)
+    else:
+        rng = np.random.default_rng(2024)
+        k, q, v, a = (rng.uniform(-0.5, 0.5, total).astype(np.float32) for _ in range(4))
+        g = k * np.float32(0.5)
+        lse = rng.uniform(-1, 1, batch * seq).astype(np.float32)
+    tiles = [_rounded(x.reshape(shape), dtype) for x in (k, q, v, a, g)]
+    return tiles, lse.reshape(batch, seq)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("mask_kind", ["causal", "full"])
+@pytest.mark.parametrize("strategy,seq,head,batch", [
+    ("preset", 64, 32, 1), ("preset", 64, 32, 4), ("random", 64, 32, 1), ("random", 64, 32, 4),
+    ("random", 128, 64, 4), ("random", 128, 128, 8), ("random", 1024, 128, 4)])
+def test_reference_kernel_test_cases(oracle, dtype, mask_kind, strategy, seq, head, batch):
+    """The reference's test of its backward kernel, through the entry point
+    with the reference's signature: its shapes where a kernel exists here
+    (seq 64, head 32, batch 1 and 4; head 8 has none) and some of its
+    benchmark shapes (:578-580), causal and full additive masks (:155-171),
+    gradients added to tiles that start at zero, its tolerances."""
+    print("case bwd reference", dtype, mask_kind, strategy, seq, head, batch, flush=True)
+    ((K, kf), (Q, qf), (V, vf), (A, af), (G, gf)), lse = _reference_case(
+        strategy, seq, head, batch, dtype)
+    shape = (batch, seq, head)
+    mask = synth.causal_mask(seq, seq) if mask_kind == "causal" else np.ones((seq, seq), bool)
+    add = np.where(mask, 0, -np.inf).astype(np.float32)
+    want = oracle.sdpa_bwd_flash_f64(kf, qf, vf, af, gf, lse, add)
+    dK, dQ, dV = (torch.zeros(shape, dtype=H.TORCH_DT[dtype], device="cuda") for _ in range(3))
+    scratch = torch.empty(shape, dtype=H.TORCH_DT[dtype], device="cuda")
+    hip_sdpa.flash_sdpa_bwd(K.cuda(), Q.cuda(), V.cuda(), A.cuda(), G.cuda(),
+                            H.additive_mask(mask, dtype).cuda(),
+                            torch.from_numpy(lse).cuda(), scratch, dK, dQ, dV)
+    torch.cuda.synchronize()
+    for got, w, name in ((dK, want[0], "dK"), (dQ, want[1], "dQ"), (dV, want[2], "dV")):
+        _check(got, w, dtype, name)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("head", [32, 64, 128])
+@pytest.mark.parametrize("q_seq,k_seq", [(128, 128), (200, 333), (64, 520), (257, 100)])
+@pytest.mark.parametrize("mode", ["causal", "none", "additive", "bool"])
+def test_modes_and_shapes(oracle, dtype, head, q_seq, k_seq, mode):
+    """Every mask mode on rectangular and ragged shapes, with A and lse from a
+    forward pass of the same inputs, gradients accumulated onto non-zero
+    tiles and, second, written in overwrite mode."""
+    print("case bwd", dtype, head, q_seq, k_seq, mode, flush=True)
+    batch = 2
+    offset = max(k_seq - q_seq, 0)
+    (Q, K, V), (qf, kf, vf) = H.make_qkv(91, batch, q_seq, k_seq, head, dtype)
+    G, gf = _rounded(synth.randn(92, 0, batch * q_seq * head).reshape(batch, q_seq, head), dtype)
+    if mode == "none":
+        mask = np.ones((q_seq, k_seq), bool)
+    elif mode == "causal":
+        mask = synth.causal_mask(q_seq, k_seq, offset)
+    else:   # a band: some rows of the last queries see little, none sees nothing
+        i = np.arange(q_seq)[:, None]
+        j = np.arange(k_seq)[None, :]
+        mask = (j <= i + offset) & (j + 40 >= i)
+        mask[:, 0] = True
+    add = np.where(mask, 0, -np.inf).astype(np.float32)
+    A64, lse64 = oracle.sdpa_bruteforce_f64(kf, qf, vf, add)
+    A, af = _rounded(A64, dtype)
+    lse = lse64.astype(np.float32)
+    want = oracle.sdpa_bwd_flash_f64(kf, qf, vf, af, gf, lse, add)
+    m = None
+    if mode == "additive":
+        m = H.additive_mask(mask, dtype).cuda()
+    elif mode == "bool":
+        m = torch.from_numpy(mask.copy()).cuda()
+    mm = {"causal": hip_sdpa.MASK_CAUSAL, "none": hip_sdpa.MASK_NONE,
+          "additive": hip_sdpa.MASK_ADDITIVE, "bool": hip_sdpa.MASK_BOOL}[mode]
+    dt = H.TORCH_DT[dtype]
+    init = [_rounded(0.25 * synth.randn(93, i, t.numel()).reshape(t.shape), dtype)
+            for i, t in enumerate((K, Q, V))]
+    dK, dQ, dV = (x[0].clone().cuda() for x in init)
+    args = (K.cuda(), Q.cuda(), V.cuda(), A.cuda(), G.cuda(), m, torch.from_numpy(lse).cuda())
+    hip_sdpa.sdpa_bwd_tile(*args, dK, dQ, dV, mm, causal_offset=offset)
+    torch.cuda.synchronize()
+    for got, w, x0, name in ((dK, want[0], init[0][1], "dK"), (dQ, want[1], init[1][1], "dQ"),
+                             (dV, want[2], init[2][1], "dV")):
+        err = np.linalg.norm(H.to_np(got).astype(np.float64) - (w + x0)) / np.linalg.norm(w + x0)
+        assert err < BWD_TOL[dtype], (name, err)
+    dK2, dQ2, dV2 = (torch.full_like(x, float("nan")) for x in (dK, dQ, dV))
+    hip_sdpa.sdpa_bwd_tile(*args, dK2, dQ2, dV2, mm, causal_offset=offset,
+                           flags=hip_sdpa.OVERWRITE)
+    torch.cuda.synchronize()
+    for got, w, name in ((dK2, want[0], "dK"), (dQ2, want[1], "dQ"), (dV2, want[2], "dV")):
+        _check(got, w, dtype, name + " overwrite")
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+def test_grouped_queries_and_key_tiles(oracle, dtype):
+    """Query heads that share a key/value head (their dK, dV sum over the
+    group), and a key axis cut into tiles whose gradients accumulate into dQ
+    tile by tile, as the tensor-level loop of the reference does."""
+    n_batch, group, n_kv, q_seq, k_seq, head, k_tile = 2, 2, 2, 160, 320, 64, 128
+    batch = n_batch * group * n_kv
+    (Q, K, V), (qf, kf, vf) = H.make_qkv(95, batch, q_seq, k_seq, head, dtype,
+                                          kv_batch=n_batch * n_kv)
+    G, gf = _rounded(synth.randn(96, 0, batch * q_seq * head).reshape(batch, q_seq, head), dtype)
+    offset = k_seq - q_seq
+    mask = synth.causal_mask(q_seq, k_seq, offset)
+    add = np.where(mask, 0, -np.inf).astype(np.float32)
+    kv_of = [(b % n_batch) + n_batch * ((b // n_batch) // group) for b in range(batch)]
+    A64, lse64 = oracle.sdpa_bruteforce_f64(kf[kv_of], qf, vf[kv_of], add)
+    A, af = _rounded(A64, dtype)
+    lse = lse64.astype(np.float32)
+    want = oracle.sdpa_bwd_flash_f64(kf, qf, vf, af, gf, lse, add, kv_repeat=group,
+                                     n_batch=n_batch)
+    dt = H.TORCH_DT[dtype]
+    dQ = torch.zeros_like(Q, device="cuda")
+    dK = torch.zeros_like(K, device="cuda")
+    dV = torch.zeros_like(V, device="cuda")
+    Qc, Ac, Gc, lc = Q.cuda(), A.cuda(), G.cuda(), torch.from_numpy(lse).cuda()
+    for s in range(0, k_seq, k_tile):
+        Kt, Vt = K[:, s:s + k_tile].contiguous().cuda(), V[:, s:s + k_tile].contiguous().cuda()
+        dKt = torch.zeros_like(Kt)
+        dVt = torch.zeros_like(Vt)
+        hip_sdpa.sdpa_bwd_tile(Kt, Qc, Vt, Ac, Gc, None, lc, dKt, dQ, dVt, hip_sdpa.MASK_CAUSAL,
+                               n_batch=n_batch, kv_group=group, k_pos0=s, causal_offset=offset)
+        dK[:, s:s + k_tile] = dKt
+        dV[:, s:s + k_tile] = dVt
+    torch.cuda.synchronize()
+    for got, w, name in ((dK, want[0], "dK"), (dQ, want[1], "dQ"), (dV, want[2], "dV")):
+        _check(got, w, dtype, name)
+
+
+def test_inputs_unchanged_and_errors():
+    batch, seq, head = 2, 64, 64
+    (Q, K, V), _ = H.make_qkv(97, batch, seq, seq, head, "bf16")
+    ins = [t.cuda() for t in (K, Q, V, Q, K)]
+    keep = [t.clone() for t in ins]
+    lse = torch.zeros(batch, seq, device="cuda")
+    outs = [torch.zeros_like(t) for t in ins[:3]]
+    hip_sdpa.sdpa_bwd_tile(*ins, None, lse, *outs, hip_sdpa.MASK_CAUSAL)
+    torch.cuda.synchronize()
+    for a, b in zip(ins, keep):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    small = torch.empty(8, dtype=torch.uint8, device="cuda")
+    with pytest.raises(hip_sdpa.SdpaError) as e:
+        hip_sdpa.sdpa_bwd_tile(*ins, None, lse, *outs, hip_sdpa.MASK_CAUSAL, workspace=small)
+    assert e.value.code == hip_sdpa.EWORKSPACE
+    with pytest.raises(hip_sdpa.SdpaError) as e:
+        hip_sdpa.sdpa_bwd_tile(*ins, None, lse, *outs, hip_sdpa.MASK_ADDITIVE)
+    assert e.value.code == hip_sdpa.EINVAL

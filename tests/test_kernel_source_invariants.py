@@ -17,6 +17,9 @@ import pytest
 from nntile_amd import build as B
 
 KERNEL_SOURCES = [s for s in B.SOURCES if s != "capi.hip"]
+# the helper's first line: the LDS target from a scalar register (which may be
+# one half of VCC when the kernel is short of SGPRs)
+M0_WRITE = r"s_mov_b32 m0, (s\d+|vcc_lo|vcc_hi)"
 
 
 def _assembly(name, outdir):
@@ -54,7 +57,7 @@ def test_m0_is_written_only_by_the_lds_load_helper(assemblies):
             if not re.search(r"\bm0\b", line):
                 continue
             # the helper's three lines: s_mov_b32 m0, sN / s_nop 0 / global_load_lds_dwordx4
-            assert re.fullmatch(r"s_mov_b32 m0, s\d+", line), (name, line)
+            assert re.fullmatch(M0_WRITE, line), (name, line)
             assert ins[i + 1] == "s_nop 0", (name, ins[i + 1])
             assert ins[i + 2].startswith("global_load_lds_dwordx4 "), (name, ins[i + 2])
             uses += 1
@@ -67,7 +70,7 @@ def test_every_lds_load_sets_m0_first(assemblies):
         for i, line in enumerate(ins):
             if line.startswith("global_load_lds_"):
                 assert i >= 2 and ins[i - 1] == "s_nop 0" \
-                    and re.fullmatch(r"s_mov_b32 m0, s\d+", ins[i - 2]), (name, line)
+                    and re.fullmatch(M0_WRITE, ins[i - 2]), (name, line)
 
 
 def test_no_packed_fp32_instructions(assemblies):
