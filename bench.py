@@ -164,6 +164,36 @@ def bench_decode(cfg, steps, warmup):
             "tflops": cfg.flops() / (wall * 1e-3) / 1e12}
 
 
+def bench_backward(cfg, steps, warmup):
+    """Backward of the same attention (dQ, dK, dV from dA, A and lse) as one
+    call over the whole sequence with the analytic causal mask: two launches.
+    FLOPs counted as 2.5 x the forward's (five products where the forward has
+    two); the two kernels execute seven, recomputing the scores in each."""
+    import torch
+    from nntile_amd import hip_sdpa as h
+    dt = {"bf16": torch.bfloat16, "fp16": torch.float16}[cfg.dtype]
+    shape = (cfg.batch_flat, cfg.q_seq, cfg.head)
+    Q, K, V, G = (_randn(shape, dt, cfg.seed * 1000 + 700 + i) for i in range(4))
+    A = torch.zeros_like(Q)
+    lse = torch.full((cfg.batch_flat, cfg.q_seq), float("-inf"), device="cuda")
+    h.sdpa_fwd_tile(K, Q, None, lse, V, A, h.MASK_CAUSAL, flags=h.OVERWRITE)
+    dK, dQ, dV = (torch.zeros_like(Q) for _ in range(3))
+    ws = torch.empty(h.lib().nntile_hip_sdpa_bwd_workspace_bytes(cfg.q_seq, cfg.batch_flat),
+                     dtype=torch.uint8, device="cuda")
+
+    def step():
+        h.sdpa_bwd_tile(K, Q, V, A, G, None, lse, dK, dQ, dV, h.MASK_CAUSAL,
+                        flags=h.OVERWRITE, workspace=ws)
+
+    wall, dev = time_steps(step, steps, warmup)
+    fl = 2.5 * cfg.flops()
+    return {"ms_per_step": round(wall, 4), "device_ms_per_step": round(dev, 4),
+            "tflops": round(fl / (dev * 1e-3) / 1e12, 1), "flops_per_step": fl,
+            "frac_of_peak": round(fl / (dev * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+            "what": "backward of %s in one call (dQ kernel + dK/dV kernel), analytic causal "
+                    "mask, gradients written" % cfg.name}
+
+
 def cpu_baseline(cfg, target_seconds=15.0):
     """The CPU checker (port of the reference's gemm -> mask_scalar ->
     maxsumexp -> softmax_inplace -> gemm composition) on a bounded sample of
@@ -202,7 +232,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run only this leg: prefill | decode | per_task | extras | copy (for profiling)")
+                    help="run only this leg: prefill | decode | per_task | backward | extras | copy (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
@@ -239,6 +269,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         return
+    if only == "backward":
+        print(json.dumps(bench_backward(cfg3, args.steps, args.warmup)))
+        return
     if only == "extras":
         for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):
             bench_prefill(BY_NAME[name], args.steps, args.warmup)
@@ -257,6 +290,7 @@ def main():
                         "frac_of_peak": round(r["kernel_tflops"] / peak, 4),
                         "peak_tflops": peak, "flops_causal_exact": c.flops(),
                         "launches_per_step": r["launches_per_step"]}
+    backward = bench_backward(cfg3, max(5, args.steps // 10), 2)
     # The headline leg runs last: the first timed loop of a process measures
     # 5 % slower than the same loop a second later (clocks still settling),
     # whatever the warmup count.
@@ -302,6 +336,7 @@ def main():
                           "ms_per_step": round(per_task["ms_per_step"], 4),
                           "tflops": round(per_task["tflops"], 2)},
         "other_configs": extras,
+        "backward": backward,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg3)

@@ -17,7 +17,7 @@
 //    rows from LDS; dS^T packed to 16 bits is the B operand of
 //    dQ^T += K^T dS^T, whose A operand comes through the transposing LDS read.
 //    It also writes D for the second kernel.
-//  * sdpa_bwd_dkv_kernel: a workgroup owns 128 keys (a lane one key) and walks
+//  * sdpa_bwd_dkv_kernel: a workgroup owns 256 keys (a lane one key) and walks
 //    the queries of every head of its group in steps of 64: S = Q K^T and
 //    dP = dA V^T with K and V fragments in registers and Q, dA rows from LDS;
 //    dV^T += dA^T P and dK^T += Q^T dS through transposing reads of the same
@@ -375,14 +375,24 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
 }
 
 // ---------------------------------------------------------------------------------
+// 8 wavefronts x 32 keys: K and V fragments plus the two accumulators take
+// 192 registers of a lane at head 128, so a CU holds one wavefront of this
+// kernel per SIMD at 4 wavefronts per workgroup; with 8 the Q and dA steps in
+// LDS serve twice the keys and every SIMD has two wavefronts to alternate.
+constexpr int kDkvWaves = 8;
+constexpr int kDkvThreads = kDkvWaves * 64;
+constexpr int kDkvRows = kDkvWaves * 32;        // keys per workgroup
+
 template<typename T, int HEAD, int MODE>
-__global__ __launch_bounds__(kBwdThreads, 1)
+__global__ __launch_bounds__(kDkvThreads, 1)
 void sdpa_bwd_dkv_kernel(const BwdParams p)
 {
     typedef typename T::vec8 vec8;
     typedef BwdTile<HEAD> G;
     constexpr int KSTEPS = G::KSTEPS, DBLOCKS = G::DBLOCKS, RB = G::RB, CPR = G::CPR;
-    constexpr int LOADS_PER_WAVE = G::LOADS_PER_WAVE, ROWS_PER_LOAD = G::ROWS_PER_LOAD;
+    constexpr int ROWS_PER_LOAD = G::ROWS_PER_LOAD;
+    constexpr int LPW = G::LOADS >= kDkvWaves ? G::LOADS / kDkvWaves : 1;   // loads per loading wavefront
+    constexpr int LOADERS = G::LOADS / LPW;                                  // wavefronts that load
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
 
@@ -390,6 +400,9 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
     __shared__ __attribute__((aligned(1024))) char lds_q1[G::BYTES];
     __shared__ __attribute__((aligned(1024))) char lds_g0[G::BYTES];
     __shared__ __attribute__((aligned(1024))) char lds_g1[G::BYTES];
+    // per query of a step: logsumexp in log2 units (+inf for a row that saw
+    // nothing) and the row dot D; rows past the end hold +inf / 0
+    __shared__ __attribute__((aligned(16))) float lds_stat[2][2][kBwdStep];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -399,9 +412,9 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
     const int half = lane >> 5;
 
     const int q_seq = (int)p.q_seq, k_seq = (int)p.k_seq;
-    const int k_blocks = (k_seq + kBwdRows - 1) / kBwdRows;
+    const int k_blocks = (k_seq + kDkvRows - 1) / kDkvRows;
     const int kvb = blockIdx.x / k_blocks;          // nb + n_batch*hkv
-    const int k_row0 = (blockIdx.x % k_blocks) * kBwdRows;
+    const int k_row0 = (blockIdx.x % k_blocks) * kDkvRows;
     const int nb = kvb % p.n_batch, hkv = kvb / p.n_batch;
     const int my_k = k_row0 + wave * 32 + col;
     const bool k_ok = my_k < k_seq;
@@ -440,26 +453,23 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
         first_step = min(q_lo / kBwdStep, n_steps);
     }
 
-    uint32_t ld_goff[LOADS_PER_WAVE];
-    int ld_row[LOADS_PER_WAVE];
+    uint32_t ld_goff[LPW];
+    int ld_row[LPW];
     const int ld_cpos = lane % CPR;
 #pragma unroll
-    for(int i = 0; i < LOADS_PER_WAVE; ++i)
+    for(int i = 0; i < LPW; ++i)
     {
-        const int r = (wave * LOADS_PER_WAVE + i) * ROWS_PER_LOAD + lane / CPR;
+        const int r = ((wave % LOADERS) * LPW + i) * ROWS_PER_LOAD + lane / CPR;
         ld_row[i] = r;
         ld_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ G::swz(r)) * 16);
     }
-    uint32_t row_raddr[2][KSTEPS];
+    // row operand: lane (col, half) reads row mb*32+col, logical chunk 2*ks+half;
+    // 32 rows further on the swizzle is the same, so mb goes into the immediate
+    uint32_t row_raddr[KSTEPS];
 #pragma unroll
-    for(int mb = 0; mb < 2; ++mb)
+    for(int ks = 0; ks < KSTEPS; ++ks)
     {
-        const int r = mb * 32 + col;
-#pragma unroll
-        for(int ks = 0; ks < KSTEPS; ++ks)
-        {
-            row_raddr[mb][ks] = (uint32_t)(r * RB + ((2 * ks + half) ^ G::swz(r)) * 16);
-        }
+        row_raddr[ks] = (uint32_t)(col * RB + ((2 * ks + half) ^ G::swz(col)) * 16);
     }
     uint32_t tr_raddr[2][DBLOCKS];
     {
@@ -500,54 +510,74 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
         qs = first_step + i % n_local;
         bq = nb + p.n_batch * (g + p.kv_group * hkv);
     };
-    auto fetch = [&](int i, char *qdst_base, char *gdst_base)
+    // loads of walk position i: the Q and dA rows straight into LDS, the
+    // logsumexp and D of its queries through registers (threads 0..127)
+    auto fetch = [&](int i, char *qdst_base, char *gdst_base, float (*stat)[kBwdStep])
     {
         int bq, qs;
         locate(i, bq, qs);
         const int row0 = qs * kBwdStep;
         const int last = min(kBwdStep, q_seq - row0) - 1;
-        const char *Qp = static_cast<const char *>(p.Q) + ((int64_t)bq * q_seq + row0) * RB;
-        const char *Gp = static_cast<const char *>(p.dA) + ((int64_t)bq * q_seq + row0) * RB;
-        char *qdst = qdst_base + wave_u * LOADS_PER_WAVE * 1024;
-        char *gdst = gdst_base + wave_u * LOADS_PER_WAVE * 1024;
-#pragma unroll
-        for(int j = 0; j < LOADS_PER_WAVE; ++j)
+        if(wave_u < LOADERS)
         {
-            const uint32_t back = (uint32_t)(max(ld_row[j] - last, 0) * RB);
-            load_to_lds16<0, false>(Qp, ld_goff[j] - back, qdst + j * 1024);
-            load_to_lds16<0, false>(Gp, ld_goff[j] - back, gdst + j * 1024);
+            const char *Qp = static_cast<const char *>(p.Q) + ((int64_t)bq * q_seq + row0) * RB;
+            const char *Gp = static_cast<const char *>(p.dA) + ((int64_t)bq * q_seq + row0) * RB;
+            char *qdst = qdst_base + wave_u * LPW * 1024;
+            char *gdst = gdst_base + wave_u * LPW * 1024;
+#pragma unroll
+            for(int j = 0; j < LPW; ++j)
+            {
+                const uint32_t back = (uint32_t)(max(ld_row[j] - last, 0) * RB);
+                load_to_lds16<0, false>(Qp, ld_goff[j] - back, qdst + j * 1024);
+                load_to_lds16<0, false>(Gp, ld_goff[j] - back, gdst + j * 1024);
+            }
+        }
+        if(tid < 2 * kBwdStep)
+        {
+            const int which = tid / kBwdStep, r = tid % kBwdStep;
+            const int64_t src = (int64_t)bq * q_seq + row0 + min(r, last);
+            float v;
+            if(which == 0)
+            {
+                const float l = p.lse[src];
+                v = (r > last || l == neg_inf()) ? __builtin_huge_valf() : l * kLog2e;
+            }
+            else
+            {
+                v = r > last ? 0.0f : p.D[src];
+            }
+            stat[which][r] = v;
         }
     };
 
     if(total > 0)
     {
-        fetch(0, lds_q0, lds_g0);
+        fetch(0, lds_q0, lds_g0, lds_stat[0]);
     }
     auto step = [&](int i, auto buf_tag) __attribute__((always_inline))
     {
         constexpr int BUF = decltype(buf_tag)::value;
         const char *Qs = BUF ? lds_q1 : lds_q0;
         const char *Gs = BUF ? lds_g1 : lds_g0;
+        const float (*stat)[kBwdStep] = lds_stat[BUF];
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if(i + 1 < total)
         {
-            fetch(i + 1, BUF ? lds_q0 : lds_q1, BUF ? lds_g0 : lds_g1);
+            fetch(i + 1, BUF ? lds_q0 : lds_q1, BUF ? lds_g0 : lds_g1, lds_stat[BUF ^ 1]);
         }
         int bq, qs;
         locate(i, bq, qs);
         const int q0 = qs * kBwdStep;
         const int rows_here = min(kBwdStep, q_seq - q0);
-        const float *lse_p = p.lse + (int64_t)bq * q_seq + q0;
-        const float *d_p = p.D + (int64_t)bq * q_seq + q0;
 
-        // ---- S = Q K^T, dP = dA V^T: rows are queries, the lane's column its key ----------
         // (one 32-query block at a time: half the accumulators live)
-        // ---- P, dS: register r of block mb is query q0 + mb*32 + tile_row(r, half) ----------
-        uint32_t p_pk[2][8], ds_pk[2][8];
+        // ---- S = Q K^T, dP = dA V^T: rows are queries, the lane's column its key;
+        // P, dS: register r of block mb is query q0 + mb*32 + tile_row(r, half) --------------
 #pragma unroll
         for(int mb = 0; mb < 2; ++mb)
         {
+            uint32_t p_pk[8], ds_pk[8];
             f32x16 sv, dpv;
 #pragma unroll
             for(int r = 0; r < 16; ++r)
@@ -558,8 +588,8 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
 #pragma unroll
             for(int ks = 0; ks < KSTEPS; ++ks)
             {
-                const vec8 qa = *reinterpret_cast<const vec8 *>(Qs + row_raddr[mb][ks]);
-                const vec8 ga = *reinterpret_cast<const vec8 *>(Gs + row_raddr[mb][ks]);
+                const vec8 qa = *reinterpret_cast<const vec8 *>(Qs + row_raddr[ks] + mb * 32 * RB);
+                const vec8 ga = *reinterpret_cast<const vec8 *>(Gs + row_raddr[ks] + mb * 32 * RB);
                 sv = T::mfma(qa, kf[ks], sv);
                 dpv = T::mfma(ga, vf[ks], dpv);
             }
@@ -567,26 +597,17 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
 #pragma unroll
             for(int rg = 0; rg < 4; ++rg)
             {
-                // four consecutive queries: their lse and D in one load each
-                // (rows past the end are clamped and hidden below)
+                // four consecutive queries: their statistics in one LDS read each
                 const int qr0 = mb * 32 + 8 * rg + 4 * half;
-                float lse4[4], d4[4];
-#pragma unroll
-                for(int e = 0; e < 4; ++e)
-                {
-                    const int qi = min(qr0 + e, rows_here - 1);
-                    lse4[e] = lse_p[qi];
-                    d4[e] = d_p[qi];
-                }
+                const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(&stat[0][qr0]);
+                const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&stat[1][qr0]);
 #pragma unroll
                 for(int e = 0; e < 4; ++e)
                 {
                     const int r = 4 * rg + e;
                     const int qr = qr0 + e;                 // query row within the step
-                    const float lse2 = (lse4[e] == neg_inf()) ? __builtin_huge_valf()
-                        : lse4[e] * kLog2e;
-                    float ex = fmaf(sv[r], c, -lse2);
-                    bool visible = k_ok && qr < rows_here;
+                    float ex = fmaf(sv[r], c, -lse4[e]);    // -inf for rows past the end
+                    bool visible = k_ok;
                     if(MODE == NNTILE_HIP_MASK_CAUSAL)
                     {
                         visible = visible && (my_k <= rel + q0 + qr);
@@ -615,33 +636,32 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
 #pragma unroll
             for(int k = 0; k < 8; ++k)
             {
-                p_pk[mb][k] = T::pack2(pv[2 * k], pv[2 * k + 1]);
-                ds_pk[mb][k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
+                p_pk[k] = T::pack2(pv[2 * k], pv[2 * k + 1]);
+                ds_pk[k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
             }
-        }
-
-        // ---- dV^T += dA^T P, dK^T += Q^T dS: four sub-steps of 16 queries -------------------
+            // ---- dV^T += dA^T P, dK^T += Q^T dS: the block's two sub-steps of 16 queries ----
 #pragma unroll
-        for(int t = 0; t < 4; ++t)
-        {
-            const int mb = t >> 1, tt = t & 1;
-            const u32x4 praw = {p_pk[mb][4 * tt], p_pk[mb][4 * tt + 1],
-                p_pk[mb][4 * tt + 2], p_pk[mb][4 * tt + 3]};
-            const u32x4 sraw = {ds_pk[mb][4 * tt], ds_pk[mb][4 * tt + 1],
-                ds_pk[mb][4 * tt + 2], ds_pk[mb][4 * tt + 3]};
-            const vec8 pb = __builtin_bit_cast(vec8, praw);
-            const vec8 sb = __builtin_bit_cast(vec8, sraw);
-#pragma unroll
-            for(int db = 0; db < DBLOCKS; ++db)
+            for(int tt = 0; tt < 2; ++tt)
             {
-                const u32x2 glo = bwd_lds_read_tr16(Gs + tr_raddr[0][db] + (16 * t) * RB);
-                const u32x2 ghi = bwd_lds_read_tr16(Gs + tr_raddr[1][db] + (16 * t) * RB);
-                const u32x4 graw = {glo[0], glo[1], ghi[0], ghi[1]};
-                dv[db] = T::mfma(__builtin_bit_cast(vec8, graw), pb, dv[db]);
-                const u32x2 qlo = bwd_lds_read_tr16(Qs + tr_raddr[0][db] + (16 * t) * RB);
-                const u32x2 qhi = bwd_lds_read_tr16(Qs + tr_raddr[1][db] + (16 * t) * RB);
-                const u32x4 qraw = {qlo[0], qlo[1], qhi[0], qhi[1]};
-                dk[db] = T::mfma(__builtin_bit_cast(vec8, qraw), sb, dk[db]);
+                const int t = 2 * mb + tt;
+                const u32x4 praw = {p_pk[4 * tt], p_pk[4 * tt + 1], p_pk[4 * tt + 2],
+                    p_pk[4 * tt + 3]};
+                const u32x4 sraw = {ds_pk[4 * tt], ds_pk[4 * tt + 1], ds_pk[4 * tt + 2],
+                    ds_pk[4 * tt + 3]};
+                const vec8 pb = __builtin_bit_cast(vec8, praw);
+                const vec8 sb = __builtin_bit_cast(vec8, sraw);
+#pragma unroll
+                for(int db = 0; db < DBLOCKS; ++db)
+                {
+                    const u32x2 glo = bwd_lds_read_tr16(Gs + tr_raddr[0][db] + (16 * t) * RB);
+                    const u32x2 ghi = bwd_lds_read_tr16(Gs + tr_raddr[1][db] + (16 * t) * RB);
+                    const u32x4 graw = {glo[0], glo[1], ghi[0], ghi[1]};
+                    dv[db] = T::mfma(__builtin_bit_cast(vec8, graw), pb, dv[db]);
+                    const u32x2 qlo = bwd_lds_read_tr16(Qs + tr_raddr[0][db] + (16 * t) * RB);
+                    const u32x2 qhi = bwd_lds_read_tr16(Qs + tr_raddr[1][db] + (16 * t) * RB);
+                    const u32x4 qraw = {qlo[0], qlo[1], qhi[0], qhi[1]};
+                    dk[db] = T::mfma(__builtin_bit_cast(vec8, qraw), sb, dk[db]);
+                }
             }
         }
     };
@@ -698,7 +718,7 @@ template<typename T, int HEAD, int MODE>
 static int launch_bwd_mode(hipStream_t stream, const BwdParams &p)
 {
     const int64_t q_blocks = (p.q_seq + kBwdRows - 1) / kBwdRows;
-    const int64_t k_blocks = (p.k_seq + kBwdRows - 1) / kBwdRows;
+    const int64_t k_blocks = (p.k_seq + kDkvRows - 1) / kDkvRows;
     const int64_t kv_batch = p.batch / p.kv_group;
     const int64_t n_dq = (int64_t)p.batch * q_blocks, n_dkv = kv_batch * k_blocks;
     if(n_dq <= 0 || n_dkv <= 0 || n_dq > 0x7fffffff || n_dkv > 0x7fffffff)
@@ -712,7 +732,7 @@ static int launch_bwd_mode(hipStream_t stream, const BwdParams &p)
         return NNTILE_HIP_ELAUNCH;
     }
     hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, HEAD, MODE>), dim3((unsigned)n_dkv),
-            dim3(kBwdThreads), 0, stream, p);
+            dim3(kDkvThreads), 0, stream, p);
     return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
 }
 

@@ -126,11 +126,19 @@ __device__ __forceinline__ void load_to_lds16(const void *gaddr, char *lds_dst)
 // The same with the address as a base common to the wavefront plus a 32-bit
 // offset per lane (no 64-bit address arithmetic on the vector unit).
 template<int OFF, bool NT>
-__device__ __forceinline__ void load_to_lds16(const void *gbase, uint32_t lane_off,
+__device__ __forceinline__ void load_to_lds16(const void *gbase_in, uint32_t lane_off,
         char *lds_dst)
 {
     typedef char __attribute__((address_space(3))) *lds_ptr;
     const uint32_t base = (uint32_t)(uintptr_t)(lds_ptr)lds_dst;
+    // (the base is the same in every lane; this makes the compiler see it)
+    const uint64_t g64 = reinterpret_cast<uint64_t>(gbase_in);
+    // (the builtin returns a signed int: widen it as unsigned, or a set bit 31
+    // of the low half would fill the high half)
+    const uint32_t g_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)g64);
+    const uint32_t g_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(g64 >> 32));
+    const uint64_t g_uni = (uint64_t)g_lo | ((uint64_t)g_hi << 32);
+    const void *gbase = reinterpret_cast<const void *>(g_uni);
     if(NT)
     {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
