@@ -254,6 +254,13 @@ void nntile_hip_set_stream_provider(nntile_hip_stream_provider fn);
 void nntile_hip_flash_sdpa_fwd_codelet_bf16(void *buffers[], void *cl_args);
 void nntile_hip_flash_sdpa_fwd_codelet_fp16(void *buffers[], void *cl_args);
 void nntile_hip_flash_sdpa_fwd_codelet_fp32(void *buffers[], void *cl_args);
+/* Backward twin: the body of starpu::FlashSdpaBwdCudnn<T>::cuda
+ * (src/starpu/flash_sdpa_bwd_cudnn.cc:51-157), 13 buffers in the reference's
+ * order K Q V A dA mask logsumexp dK dQ dV scratch_dK scratch_dQ scratch_dV
+ * (:103-115) and the same args_t prefix {owner, seq, head, batch}
+ * (include/nntile/starpu/flash_sdpa_bwd_cudnn.hh:48-57). */
+void nntile_hip_flash_sdpa_bwd_codelet_bf16(void *buffers[], void *cl_args);
+void nntile_hip_flash_sdpa_bwd_codelet_fp16(void *buffers[], void *cl_args);
 
 /* Library version and the ISA it was built for ("gfx950"). */
 const char *nntile_hip_sdpa_version(void);

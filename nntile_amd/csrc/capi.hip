@@ -416,6 +416,43 @@ static void codelet_call(DType dt, const char *name, void *buffers[],
     }
 }
 
+static void bwd_codelet_call(DType dt, const char *name, void *buffers[],
+        void *cl_args)
+{
+    // Buffer order of the reference body (src/starpu/flash_sdpa_bwd_cudnn.cc:
+    // 103-115, modes :175-187): K Q V A dA mask logsumexp (R), dK dQ dV (RW),
+    // scratch_dK scratch_dQ scratch_dV (SCRATCH); same error behaviour.
+    if(buffers == nullptr || cl_args == nullptr)
+    {
+        std::fprintf(stderr, "HIP Worker: %s: null buffers or arguments, "
+                "skipping task\n", name);
+        return;
+    }
+    const auto *args = static_cast<const nntile_hip_flash_sdpa_cl_args *>(cl_args);
+    auto **ifs = reinterpret_cast<nntile_hip_variable_interface **>(buffers);
+    for(int i = 0; i < 12; ++i)
+    {
+        if(i != 10 && ifs[i] == nullptr)
+        {
+            std::fprintf(stderr, "HIP Worker: %s: buffer %d is null, skipping "
+                    "task\n", name, i);
+            return;
+        }
+    }
+    void *stream = g_stream_provider ? g_stream_provider() : nullptr;
+    auto ptr = [&](int i) { return reinterpret_cast<void *>(ifs[i]->ptr); };
+    const int rc = flash_bwd_call(dt, stream, args->seq, args->head, args->batch,
+            ptr(0), ptr(1), ptr(2), ptr(3), ptr(4), ptr(5),
+            reinterpret_cast<const float *>(ifs[6]->ptr), ptr(11), ptr(7), ptr(8), ptr(9));
+    if(rc != NNTILE_HIP_OK)
+    {
+        std::fprintf(stderr, "HIP Worker: %s: launch failed with code %d "
+                "(seq=%lld head=%lld batch=%lld), skipping task\n", name, rc,
+                (long long)args->seq, (long long)args->head,
+                (long long)args->batch);
+    }
+}
+
 } // namespace nntile_hip
 
 using namespace nntile_hip;
@@ -580,6 +617,16 @@ int nntile_hip_flash_sdpa_bwd_fp16(void *stream, int64_t seq, int64_t head,
 {
     return flash_bwd_call(DType::fp16, stream, seq, head, batch, K, Q, V, A, dA, mask,
             lse, scratch_dQ, dK, dQ, dV);
+}
+
+void nntile_hip_flash_sdpa_bwd_codelet_bf16(void *buffers[], void *cl_args)
+{
+    bwd_codelet_call(DType::bf16, "nntile_flash_sdpa_bwd_hip_bf16", buffers, cl_args);
+}
+
+void nntile_hip_flash_sdpa_bwd_codelet_fp16(void *buffers[], void *cl_args)
+{
+    bwd_codelet_call(DType::fp16, "nntile_flash_sdpa_bwd_hip_fp16", buffers, cl_args);
 }
 
 const char *nntile_hip_sdpa_version(void)

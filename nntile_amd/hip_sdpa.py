@@ -81,6 +81,7 @@ EXPORTS = (
     + ["nntile_hip_flash_sdpa_bwd_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_sdpa_bwd_tile_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_sdpa_bwd_workspace_bytes"]
+    + ["nntile_hip_flash_sdpa_bwd_codelet_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_accumulate_attn_output_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_flash_sdpa_fwd_codelet_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_set_stream_provider", "nntile_hip_sdpa_version"])
@@ -119,6 +120,9 @@ def lib():
             f = getattr(L, "nntile_hip_flash_sdpa_bwd_" + t)
             f.argtypes = [_vp, _i64, _i64, _i64] + [_vp] * 13
             f.restype = ctypes.c_int
+            f = getattr(L, "nntile_hip_flash_sdpa_bwd_codelet_" + t)
+            f.argtypes = [ctypes.POINTER(_vp), _vp]
+            f.restype = None
             f = getattr(L, "nntile_hip_sdpa_bwd_tile_" + t)
             f.argtypes = [_vp, ctypes.POINTER(BwdArgs)]
             f.restype = ctypes.c_int
@@ -381,4 +385,25 @@ def flash_sdpa_fwd_codelet(K, Q, mask, lse, V, A, scratch_lse=None, scratch_A=No
     args = FlashClArgs(None, s if seq is None else seq, h if head is None else head,
                        b if batch is None else batch)
     fn = getattr(lib(), "nntile_hip_flash_sdpa_fwd_codelet_" + dtype_name(Q))
+    fn(bufs, ctypes.addressof(args))
+
+
+def flash_sdpa_bwd_codelet(K, Q, V, A, dA, mask, lse, dK, dQ, dV, scratch_dK=None,
+                           scratch_dQ=None, scratch_dV=None):
+    """Calls the StarPU-shaped backward codelet body with look-alike variable
+    interfaces (13 buffers in the reference's order)."""
+    tensors = [K, Q, V, A, dA, mask, lse, dK, dQ, dV, scratch_dK, scratch_dQ, scratch_dV]
+    ifs = []
+    for t in tensors:
+        v = VariableInterface()
+        v.id = 2
+        v.ptr = 0 if t is None else t.data_ptr()
+        v.dev_handle = v.ptr
+        v.offset = 0
+        v.elemsize = 0 if t is None else t.numel() * t.element_size()
+        ifs.append(v)
+    bufs = (_vp * 13)(*[ctypes.addressof(v) for v in ifs])
+    b, s, h = Q.shape
+    args = FlashClArgs(None, s, h, b)
+    fn = getattr(lib(), "nntile_hip_flash_sdpa_bwd_codelet_" + dtype_name(Q))
     fn(bufs, ctypes.addressof(args))

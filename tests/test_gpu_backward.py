@@ -182,3 +182,23 @@ def test_inputs_unchanged_and_errors():
     with pytest.raises(hip_sdpa.SdpaError) as e:
         hip_sdpa.sdpa_bwd_tile(*ins, None, lse, *outs, hip_sdpa.MASK_ADDITIVE)
     assert e.value.code == hip_sdpa.EINVAL
+
+
+def test_codelet_body(oracle):
+    """The StarPU-shaped body: 13 variable interfaces in the reference's buffer
+    order, gradients added to the RW tiles."""
+    batch, seq, head, dtype = 3, 128, 64, "bf16"
+    ((K, kf), (Q, qf), (V, vf), (A, af), (G, gf)), lse = _reference_case(
+        "random", seq, head, batch, dtype)
+    mask = synth.causal_mask(seq, seq)
+    add = np.where(mask, 0, -np.inf).astype(np.float32)
+    want = oracle.sdpa_bwd_flash_f64(kf, qf, vf, af, gf, lse, add)
+    shape = (batch, seq, head)
+    dK, dQ, dV = (torch.zeros(shape, dtype=torch.bfloat16, device="cuda") for _ in range(3))
+    scr = [torch.empty(shape, dtype=torch.bfloat16, device="cuda") for _ in range(3)]
+    hip_sdpa.flash_sdpa_bwd_codelet(K.cuda(), Q.cuda(), V.cuda(), A.cuda(), G.cuda(),
+                                    H.additive_mask(mask, dtype).cuda(),
+                                    torch.from_numpy(lse).cuda(), dK, dQ, dV, *scr)
+    torch.cuda.synchronize()
+    for got, w, name in ((dK, want[0], "dK"), (dQ, want[1], "dQ"), (dV, want[2], "dV")):
+        _check(got, w, dtype, name)
