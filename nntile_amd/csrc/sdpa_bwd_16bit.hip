@@ -9,7 +9,8 @@
 //
 // (include/nntile/kernel/flash_sdpa_bwd_cudnn/cuda.hh:44-68 is the interface
 // this replaces; tests/kernel/flash_sdpa_bwd_cudnn.cc:174-262 the arithmetic).
-// Two kernels, no atomics, results independent of timing:
+// Two kernels (the second launched once per gradient), no atomics, results
+// independent of timing:
 //
 //  * sdpa_bwd_dq_kernel: a workgroup owns 128 queries (a wavefront 32, a lane
 //    one query) and walks the keys in steps of 64, as the forward kernel does:
@@ -17,7 +18,7 @@
 //    rows from LDS; dS^T packed to 16 bits is the B operand of
 //    dQ^T += K^T dS^T, whose A operand comes through the transposing LDS read.
 //    It also writes D for the second kernel.
-//  * sdpa_bwd_dkv_kernel: a workgroup owns 256 keys (a lane one key) and walks
+//  * sdpa_bwd_dkv_kernel: a workgroup owns 128 keys (a lane one key) and walks
 //    the queries of every head of its group in steps of 64: S = Q K^T and
 //    dP = dA V^T with K and V fragments in registers and Q, dA rows from LDS;
 //    dV^T += dA^T P and dK^T += Q^T dS through transposing reads of the same
@@ -375,18 +376,21 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
 }
 
 // ---------------------------------------------------------------------------------
-// 8 wavefronts x 32 keys: K and V fragments plus the two accumulators take
-// 192 registers of a lane at head 128, so a CU holds one wavefront of this
-// kernel per SIMD at 4 wavefronts per workgroup; with 8 the Q and dA steps in
-// LDS serve twice the keys and every SIMD has two wavefronts to alternate.
-constexpr int kDkvWaves = 8;
+// PART says which gradient: K and V fragments plus both accumulators take 192
+// registers of a lane at head 128, which leaves too few for two wavefronts
+// per SIMD to run without spilling and without room to read operands ahead.
+// One launch per gradient (dK: S, dP, dK^T; dV: S, dV^T - the scores are
+// computed once more) fits two workgroups of 4 wavefronts on a CU each.
+enum { BWD_PART_DK = 1, BWD_PART_DV = 2 };
+constexpr int kDkvWaves = 4;
 constexpr int kDkvThreads = kDkvWaves * 64;
 constexpr int kDkvRows = kDkvWaves * 32;        // keys per workgroup
 
-template<typename T, int HEAD, int MODE>
-__global__ __launch_bounds__(kDkvThreads, 1)
+template<typename T, int HEAD, int MODE, int PART>
+__global__ __launch_bounds__(kDkvThreads, 2)
 void sdpa_bwd_dkv_kernel(const BwdParams p)
 {
+    constexpr bool DO_DK = PART == BWD_PART_DK, DO_DV = PART == BWD_PART_DV;
     typedef typename T::vec8 vec8;
     typedef BwdTile<HEAD> G;
     constexpr int KSTEPS = G::KSTEPS, DBLOCKS = G::DBLOCKS, RB = G::RB, CPR = G::CPR;
@@ -436,7 +440,7 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
                 v = u32x4{0, 0, 0, 0};
             }
             kf[ks] = __builtin_bit_cast(vec8, k);
-            vf[ks] = __builtin_bit_cast(vec8, v);
+            vf[ks] = __builtin_bit_cast(vec8, DO_DK ? v : u32x4{0, 0, 0, 0});
         }
     }
 
@@ -589,9 +593,13 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
             for(int ks = 0; ks < KSTEPS; ++ks)
             {
                 const vec8 qa = *reinterpret_cast<const vec8 *>(Qs + row_raddr[ks] + mb * 32 * RB);
-                const vec8 ga = *reinterpret_cast<const vec8 *>(Gs + row_raddr[ks] + mb * 32 * RB);
                 sv = T::mfma(qa, kf[ks], sv);
-                dpv = T::mfma(ga, vf[ks], dpv);
+                if(DO_DK)
+                {
+                    const vec8 ga = *reinterpret_cast<const vec8 *>(Gs + row_raddr[ks]
+                            + mb * 32 * RB);
+                    dpv = T::mfma(ga, vf[ks], dpv);
+                }
             }
             float pv[16], dsv[16];
 #pragma unroll
@@ -653,14 +661,20 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
 #pragma unroll
                 for(int db = 0; db < DBLOCKS; ++db)
                 {
-                    const u32x2 glo = bwd_lds_read_tr16(Gs + tr_raddr[0][db] + (16 * t) * RB);
-                    const u32x2 ghi = bwd_lds_read_tr16(Gs + tr_raddr[1][db] + (16 * t) * RB);
-                    const u32x4 graw = {glo[0], glo[1], ghi[0], ghi[1]};
-                    dv[db] = T::mfma(__builtin_bit_cast(vec8, graw), pb, dv[db]);
-                    const u32x2 qlo = bwd_lds_read_tr16(Qs + tr_raddr[0][db] + (16 * t) * RB);
-                    const u32x2 qhi = bwd_lds_read_tr16(Qs + tr_raddr[1][db] + (16 * t) * RB);
-                    const u32x4 qraw = {qlo[0], qlo[1], qhi[0], qhi[1]};
-                    dk[db] = T::mfma(__builtin_bit_cast(vec8, qraw), sb, dk[db]);
+                    if(DO_DV)
+                    {
+                        const u32x2 glo = bwd_lds_read_tr16(Gs + tr_raddr[0][db] + (16 * t) * RB);
+                        const u32x2 ghi = bwd_lds_read_tr16(Gs + tr_raddr[1][db] + (16 * t) * RB);
+                        const u32x4 graw = {glo[0], glo[1], ghi[0], ghi[1]};
+                        dv[db] = T::mfma(__builtin_bit_cast(vec8, graw), pb, dv[db]);
+                    }
+                    if(DO_DK)
+                    {
+                        const u32x2 qlo = bwd_lds_read_tr16(Qs + tr_raddr[0][db] + (16 * t) * RB);
+                        const u32x2 qhi = bwd_lds_read_tr16(Qs + tr_raddr[1][db] + (16 * t) * RB);
+                        const u32x4 qraw = {qlo[0], qlo[1], qhi[0], qhi[1]};
+                        dk[db] = T::mfma(__builtin_bit_cast(vec8, qraw), sb, dk[db]);
+                    }
                 }
             }
         }
@@ -710,8 +724,14 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
             }
         }
     };
-    store(p.dK, dk, p.scale);
-    store(p.dV, dv, 1.0f);
+    if(DO_DK)
+    {
+        store(p.dK, dk, p.scale);
+    }
+    if(DO_DV)
+    {
+        store(p.dV, dv, 1.0f);
+    }
 }
 
 template<typename T, int HEAD, int MODE>
@@ -731,8 +751,14 @@ static int launch_bwd_mode(hipStream_t stream, const BwdParams &p)
     {
         return NNTILE_HIP_ELAUNCH;
     }
-    hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, HEAD, MODE>), dim3((unsigned)n_dkv),
-            dim3(kDkvThreads), 0, stream, p);
+    hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, HEAD, MODE, BWD_PART_DV>),
+            dim3((unsigned)n_dkv), dim3(kDkvThreads), 0, stream, p);
+    if(hipGetLastError() != hipSuccess)
+    {
+        return NNTILE_HIP_ELAUNCH;
+    }
+    hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, HEAD, MODE, BWD_PART_DK>),
+            dim3((unsigned)n_dkv), dim3(kDkvThreads), 0, stream, p);
     return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
 }
 
