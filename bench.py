@@ -178,7 +178,7 @@ def bench_backward(cfg, steps, warmup):
     lse = torch.full((cfg.batch_flat, cfg.q_seq), float("-inf"), device="cuda")
     h.sdpa_fwd_tile(K, Q, None, lse, V, A, h.MASK_CAUSAL, flags=h.OVERWRITE)
     dK, dQ, dV = (torch.zeros_like(Q) for _ in range(3))
-    ws = torch.empty(h.lib().nntile_hip_sdpa_bwd_workspace_bytes(cfg.q_seq, cfg.batch_flat),
+    ws = torch.empty(h.sdpa_bwd_workspace_bytes(cfg.q_seq, cfg.q_seq, cfg.batch_flat, h.MASK_CAUSAL),
                      dtype=torch.uint8, device="cuda")
 
     def step():

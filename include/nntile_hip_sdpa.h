@@ -142,7 +142,14 @@ int nntile_hip_flash_sdpa_bwd_fp16(void *stream, int64_t seq, int64_t head,
  * and positions as in nntile_hip_sdpa_tile_args; with kv_group > 1 the
  * gradients of a key/value head sum over its query heads.  flags:
  * NNTILE_HIP_SDPA_OVERWRITE writes the gradients instead of adding to them.
- * workspace: q_seq*batch floats (nntile_hip_sdpa_bwd_workspace_bytes). */
+ * workspace: device memory of nntile_hip_sdpa_bwd_workspace_bytes(args)
+ * bytes, 4-byte aligned, private to the call until it has completed:
+ * q_seq*batch floats (the row dots dA.A), then, for the two modes that pass
+ * the mask as values, one byte per 64 x 64 block of the mask (whether the
+ * block hides everything, nothing, or some).  A workspace that only holds the
+ * floats is accepted: the kernels then read every value of the mask instead
+ * of skipping by block.  A mask passed as values may have at most 2^24 keys
+ * per row (NNTILE_HIP_EUNSUPPORTED beyond). */
 typedef struct nntile_hip_sdpa_bwd_args
 {
     int64_t q_seq, k_seq, head;
@@ -157,7 +164,7 @@ typedef struct nntile_hip_sdpa_bwd_args
     size_t workspace_bytes;
 } nntile_hip_sdpa_bwd_args;
 
-size_t nntile_hip_sdpa_bwd_workspace_bytes(int64_t q_seq, int64_t batch);
+size_t nntile_hip_sdpa_bwd_workspace_bytes(const nntile_hip_sdpa_bwd_args *args);
 int nntile_hip_sdpa_bwd_tile_bf16(void *stream, const nntile_hip_sdpa_bwd_args *args);
 int nntile_hip_sdpa_bwd_tile_fp16(void *stream, const nntile_hip_sdpa_bwd_args *args);
 

@@ -133,12 +133,21 @@ static int bwd_call(DType dt, void *stream, const nntile_hip_sdpa_bwd_args *a)
     {
         return NNTILE_HIP_EUNSUPPORTED;
     }
-    if(a->workspace == nullptr
-            || a->workspace_bytes < nntile_hip_sdpa_bwd_workspace_bytes(a->q_seq, a->batch)
+    // the kernels address 128 rows of a mask given as values with 32 bits
+    if(explicit_mask && a->k_seq > (1 << 24))
+    {
+        return NNTILE_HIP_EUNSUPPORTED;
+    }
+    // workspace: q_seq*batch floats (the row dots), then, if there is room
+    // and the mask is given as values, one byte per 64 x 64 block of the mask
+    const size_t d_bytes = (size_t)a->q_seq * (size_t)a->batch * sizeof(float);
+    if(a->workspace == nullptr || a->workspace_bytes < d_bytes
             || (reinterpret_cast<uintptr_t>(a->workspace) & 3u) != 0)
     {
         return NNTILE_HIP_EWORKSPACE;
     }
+    const int64_t q_blocks64 = (a->q_seq + 63) / 64, k_blocks64 = (a->k_seq + 63) / 64;
+    const size_t cls_bytes = (size_t)q_blocks64 * (size_t)k_blocks64;
     BwdParams p;
     std::memset(&p, 0, sizeof(p));
     p.q_seq = a->q_seq;
@@ -155,6 +164,11 @@ static int bwd_call(DType dt, void *stream, const nntile_hip_sdpa_bwd_args *a)
     p.dA = a->dA;
     p.lse = a->lse;
     p.D = static_cast<float *>(a->workspace);
+    if(explicit_mask && a->workspace_bytes >= d_bytes + cls_bytes && k_blocks64 <= 0x7fffffff)
+    {
+        p.mask_class = static_cast<const uint8_t *>(a->workspace) + d_bytes;
+        p.class_ld = (int32_t)k_blocks64;
+    }
     p.dK = a->dK;
     p.dQ = a->dQ;
     p.dV = a->dV;
@@ -580,13 +594,20 @@ void nntile_hip_flash_sdpa_fwd_codelet_fp32(void *buffers[], void *cl_args)
     codelet_call(DType::fp32, "nntile_flash_sdpa_fwd_hip_fp32", buffers, cl_args);
 }
 
-size_t nntile_hip_sdpa_bwd_workspace_bytes(int64_t q_seq, int64_t batch)
+size_t nntile_hip_sdpa_bwd_workspace_bytes(const nntile_hip_sdpa_bwd_args *a)
 {
-    if(q_seq <= 0 || batch <= 0)
+    if(a == nullptr || a->q_seq <= 0 || a->k_seq <= 0 || a->batch <= 0)
     {
         return 0;
     }
-    return (size_t)q_seq * (size_t)batch * sizeof(float);
+    // the row dots, then the classes of the 64 x 64 blocks of a mask given
+    // as values
+    size_t bytes = (size_t)a->q_seq * (size_t)a->batch * sizeof(float);
+    if(a->mask_mode == NNTILE_HIP_MASK_ADDITIVE || a->mask_mode == NNTILE_HIP_MASK_BOOL)
+    {
+        bytes += (size_t)((a->q_seq + 63) / 64) * (size_t)((a->k_seq + 63) / 64);
+    }
+    return bytes;
 }
 
 int nntile_hip_sdpa_bwd_tile_bf16(void *stream, const nntile_hip_sdpa_bwd_args *args)

@@ -76,6 +76,141 @@ __device__ __forceinline__ int tile_row(int r, int half)
 }
 
 // ---------------------------------------------------------------------------------
+// Masks given as values: one pass writes the class of every 64 x 64 block of
+// the mask (the reference hands the kernel a materialised tile even where it is
+// causal, src/tile/flash_sdpa_bwd_cudnn.cc), so that the three kernels below skip
+// the steps whose blocks hide everything - without fetching them - and read no
+// mask values in the steps whose blocks mask nothing.
+constexpr int kMaskMixed = 0, kMaskOpen = 1, kMaskHidden = 2;
+
+template<typename T, int MODE>
+__global__ __launch_bounds__(256)
+void sdpa_bwd_mask_classes_kernel(const void *mask, int64_t mask_ld, int q_seq, int k_seq,
+        uint8_t *table, int class_ld)
+{
+    const int qb = blockIdx.x / class_ld, kb = blockIdx.x % class_ld;
+    const int row = qb * kBwdStep + (int)threadIdx.x / 4;
+    const int col0 = kb * kBwdStep + ((int)threadIdx.x % 4) * 16;
+    bool any_visible = false, any_masked = false;
+    constexpr int ES = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 2 : 1;
+    const bool wide = (mask_ld * ES) % 16 == 0 && reinterpret_cast<uintptr_t>(mask) % 16 == 0;
+    if(row < q_seq && col0 < k_seq)
+    {
+        const char *src = static_cast<const char *>(mask) + ((int64_t)row * mask_ld + col0) * ES;
+        if(wide && col0 + 16 <= k_seq)
+        {
+            // the thread's 16 values as 16-byte loads
+#pragma unroll
+            for(int i = 0; i < ES; ++i)
+            {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(src + 16 * i);
+#pragma unroll
+                for(int w = 0; w < 4; ++w)
+                {
+                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                    {
+                        any_masked |= v[w] != 0u;
+                        any_visible |= v[w] != T::kNegInfPair;
+                    }
+                    else
+                    {
+                        any_masked |= v[w] != 0x01010101u;
+                        any_visible |= v[w] != 0u;
+                    }
+                }
+            }
+        }
+        else
+        {
+            for(int e = 0; e < 16 && col0 + e < k_seq; ++e)
+            {
+                if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                {
+                    const uint16_t v = reinterpret_cast<const uint16_t *>(src)[e];
+                    any_visible |= (T::to_float(v) != neg_inf());
+                    any_masked |= (v != 0);         // anything but +0 changes the score
+                }
+                else
+                {
+                    const bool vis = reinterpret_cast<const uint8_t *>(src)[e] != 0;
+                    any_visible |= vis;
+                    any_masked |= !vis;
+                }
+            }
+        }
+    }
+    const int vis = __syncthreads_or(any_visible ? 1 : 0);
+    const int msk = __syncthreads_or(any_masked ? 1 : 0);
+    if(threadIdx.x == 0)
+    {
+        table[blockIdx.x] = (uint8_t)(!msk ? kMaskOpen : (!vis ? kMaskHidden : kMaskMixed));
+    }
+}
+
+// The steps a workgroup takes, as a bit set (up to 64 of them; longer walks
+// take every step), and the subset in which nothing is masked.
+struct StepSet
+{
+    unsigned long long active, open;
+    bool use_bits;
+    int first, last;        // [first, last): the walk without the table
+
+    __device__ __forceinline__ int begin() const
+    {
+        if(!use_bits)
+        {
+            return first < last ? first : -1;
+        }
+        return active != 0ull ? __builtin_ctzll(active) : -1;
+    }
+    __device__ __forceinline__ int next(int g) const
+    {
+        if(!use_bits)
+        {
+            return g + 1 < last ? g + 1 : -1;
+        }
+        const unsigned long long rest = g >= 63 ? 0ull : (active >> (g + 1)) << (g + 1);
+        return rest != 0ull ? __builtin_ctzll(rest) : -1;
+    }
+    __device__ __forceinline__ bool is_open(int g) const
+    {
+        return use_bits && ((open >> g) & 1ull) != 0ull;
+    }
+};
+
+// Step set of a workgroup that owns the blocks [own0, own0 + n_own) of one axis
+// and walks the blocks [first, last) of the other.  by_row: the owned blocks
+// are query blocks (rows of the table).
+__device__ __forceinline__ StepSet make_step_set(const BwdParams &p, bool explicit_mask,
+        int own0, int n_own, int first, int last, bool by_row)
+{
+    StepSet s;
+    s.first = first;
+    s.last = last;
+    s.use_bits = explicit_mask && p.mask_class != nullptr && last <= 64;
+    s.active = 0ull;
+    s.open = 0ull;
+    if(s.use_bits)
+    {
+        // lane g looks at step g; the ballots make the two sets (every
+        // wavefront computes the same)
+        const int g = (int)(threadIdx.x & 63);
+        const bool in_walk = g >= first && g < last;
+        bool hidden = true, open = true;
+        for(int o = 0; o < n_own; ++o)
+        {
+            const int idx = by_row ? (own0 + o) * p.class_ld + g : g * p.class_ld + own0 + o;
+            const int c = in_walk ? p.mask_class[idx] : kMaskHidden;
+            hidden = hidden && (c == kMaskHidden);
+            open = open && (c == kMaskOpen);
+        }
+        s.active = __builtin_amdgcn_ballot_w64(in_walk && !hidden);
+        s.open = __builtin_amdgcn_ballot_w64(in_walk && open);
+    }
+    return s;
+}
+
+// ---------------------------------------------------------------------------------
 template<typename T, int HEAD, int MODE>
 __global__ __launch_bounds__(kBwdThreads, 2)
 void sdpa_bwd_dq_kernel(const BwdParams p)
@@ -234,25 +369,42 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
         }
     }
     const float c = p.scale * kLog2e;
-    const int64_t mask_row = (int64_t)(q_ok ? my_q : 0) * p.mask_ld;
+    // mask values: the workgroup's first row of the mask, and the byte offset
+    // of the lane's row from there (the launcher keeps 128 rows of the mask
+    // within 32 bits); mask_off is that of the lane's first key in a step
+    constexpr uint32_t MASK_ES = MODE == NNTILE_HIP_MASK_ADDITIVE ? 2u : 1u;
+    const char *mask_wg = static_cast<const char *>(p.mask)
+        + (int64_t)q_row0 * p.mask_ld * (int64_t)MASK_ES;
+    const uint32_t mask_row_off = (uint32_t)(q_ok ? my_q - q_row0 : 0) * (uint32_t)p.mask_ld * MASK_ES;
+    const uint32_t mask_off = mask_row_off + (uint32_t)(4 * half) * MASK_ES;
 
-    if(n_steps > 0)
+    // the workgroup's two query blocks of 64 against the key blocks 0 .. n_steps-1
+    const StepSet steps = make_step_set(p, EXPLICIT, q_row0 / kBwdStep,
+            min(2, (q_seq - q_row0 + kBwdStep - 1) / kBwdStep), 0, n_steps, true);
+    int g_cur = steps.begin();
+    if(g_cur >= 0)
     {
-        fetch(0, lds_k0, lds_v0);
+        fetch(g_cur, lds_k0, lds_v0);
     }
-    auto step = [&](int g, auto buf_tag) __attribute__((always_inline))
+    // masked_tag: the step reads mask values (as a compile-time choice, so
+    // that the reads of a step stay one batch of loads)
+    auto step = [&](int g, int g_next, auto buf_tag, auto masked_tag)
+        __attribute__((always_inline))
     {
         constexpr int BUF = decltype(buf_tag)::value;
         const char *Ks = BUF ? lds_k1 : lds_k0;
         const char *Vs = BUF ? lds_v1 : lds_v0;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if(g + 1 < n_steps)
+        if(g_next >= 0)
         {
-            fetch(g + 1, BUF ? lds_k0 : lds_k1, BUF ? lds_v0 : lds_v1);
+            fetch(g_next, BUF ? lds_k0 : lds_k1, BUF ? lds_v0 : lds_v1);
         }
+        constexpr bool use_mask = EXPLICIT && decltype(masked_tag)::value;
         const int kg0 = g * kBwdStep;
         const int keys_here = min(kBwdStep, k_seq - kg0);
+        const char *mask_step = mask_wg + (int64_t)kg0 * MASK_ES;
+        const uint32_t mask_off_last = mask_row_off + (uint32_t)(keys_here - 1) * MASK_ES;
 
         // ---- S^T = K Q^T, dP^T = V dA^T -------------------------------------------------
         // (one 32-key block at a time: half the accumulators live)
@@ -288,18 +440,23 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
                 const int key = mb * 32 + tile_row(r, half);
                 float e = fmaf(sv[r], c, -lse2);
                 bool visible = key <= lim;
-                if(EXPLICIT)
+                if(use_mask)
                 {
-                    const int64_t mi = mask_row + kg0 + min(key, keys_here - 1);
+                    // wave-common address of the step's first key in the
+                    // workgroup's first row + the lane's 32-bit offset;
+                    // keys past the end read the last key, and are hidden
+                    const uint32_t key_off = (uint32_t)(mb * 32 + tile_row(r, 0)) * MASK_ES;
+                    const char *mp = mask_step + min(mask_off + key_off, mask_off_last);
                     if(MODE == NNTILE_HIP_MASK_ADDITIVE)
                     {
-                        const float add = T::to_float(static_cast<const uint16_t *>(p.mask)[mi]);
+                        const float add = T::to_float(*reinterpret_cast<const uint16_t *>(mp));
                         visible = visible && (add != neg_inf());
                         e = fmaf(add, kLog2e, e);
                     }
                     else
                     {
-                        visible = visible && (static_cast<const uint8_t *>(p.mask)[mi] != 0);
+                        const uint8_t shown = *reinterpret_cast<const uint8_t *>(mp);
+                        visible = visible && (shown != 0);
                     }
                 }
                 const float pr = visible ? fast_exp2(e) : 0.0f;
@@ -330,13 +487,29 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
             }
         }
     };
-    for(int g = 0; g < n_steps; g += 2)
+    auto run = [&](int g, int g_next, auto buf_tag) __attribute__((always_inline))
     {
-        step(g, std::integral_constant<int, 0>{});
-        if(g + 1 < n_steps)
+        if(EXPLICIT && !steps.is_open(g))
         {
-            step(g + 1, std::integral_constant<int, 1>{});
+            step(g, g_next, buf_tag, std::true_type{});
         }
+        else
+        {
+            step(g, g_next, buf_tag, std::false_type{});
+        }
+    };
+    while(g_cur >= 0)
+    {
+        int g_next = steps.next(g_cur);
+        run(g_cur, g_next, std::integral_constant<int, 0>{});
+        g_cur = g_next;
+        if(g_cur < 0)
+        {
+            break;
+        }
+        g_next = steps.next(g_cur);
+        run(g_cur, g_next, std::integral_constant<int, 1>{});
+        g_cur = g_next;
     }
 
     // ---- dQ (+)= scale acc: register r of block db is head value
@@ -504,15 +677,40 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
         }
     }
     const float c = p.scale * kLog2e;
-    const int n_local = n_steps - first_step;       // steps per head of the group
-    const int total = n_local * p.kv_group;         // steps of the whole walk
-
-    // walk position i -> (head g of the group, query step)
+    // mask values: byte offsets of the lane's key within a row of the mask,
+    // for the rows of the lower and of the upper half of the wave (the
+    // launcher keeps 64 rows of the mask within 32 bits)
+    constexpr uint32_t MASK_ES = MODE == NNTILE_HIP_MASK_ADDITIVE ? 2u : 1u;
+    const uint32_t mask_row_bytes = (uint32_t)p.mask_ld * MASK_ES;
+    const uint32_t mask_off_lo = (uint32_t)(k_ok ? my_k : 0) * MASK_ES;
+    const uint32_t mask_off_hi = mask_off_lo + (uint32_t)(4 * half) * mask_row_bytes;
+    // the workgroup's key blocks of 64 against the query blocks
+    // first_step .. n_steps-1, once per head of the group: walk position
+    // i = head * 64K + query step
+    const StepSet steps = make_step_set(p, EXPLICIT, k_row0 / kBwdStep,
+            min(kDkvRows / kBwdStep, (k_seq - k_row0 + kBwdStep - 1) / kBwdStep),
+            first_step, n_steps, false);
+    constexpr int kHeadStride = 1 << 16;
     auto locate = [&](int i, int &bq, int &qs)
     {
-        const int g = i / n_local;
-        qs = first_step + i % n_local;
+        const int g = i / kHeadStride;
+        qs = i % kHeadStride;
         bq = nb + p.n_batch * (g + p.kv_group * hkv);
+    };
+    auto walk_begin = [&]() -> int
+    {
+        return steps.begin();       // head 0
+    };
+    auto walk_next = [&](int i) -> int
+    {
+        const int g = i / kHeadStride;
+        const int nxt = steps.next(i % kHeadStride);
+        if(nxt >= 0)
+        {
+            return g * kHeadStride + nxt;
+        }
+        const int b0 = steps.begin();
+        return (g + 1 < p.kv_group && b0 >= 0) ? (g + 1) * kHeadStride + b0 : -1;
     };
     // loads of walk position i: the Q and dA rows straight into LDS, the
     // logsumexp and D of its queries through registers (threads 0..127)
@@ -554,11 +752,13 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
         }
     };
 
-    if(total > 0)
+    int i_cur = walk_begin();
+    if(i_cur >= 0)
     {
-        fetch(0, lds_q0, lds_g0, lds_stat[0]);
+        fetch(i_cur, lds_q0, lds_g0, lds_stat[0]);
     }
-    auto step = [&](int i, auto buf_tag) __attribute__((always_inline))
+    auto step = [&](int i, int i_next, auto buf_tag, auto masked_tag)
+        __attribute__((always_inline))
     {
         constexpr int BUF = decltype(buf_tag)::value;
         const char *Qs = BUF ? lds_q1 : lds_q0;
@@ -566,14 +766,18 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
         const float (*stat)[kBwdStep] = lds_stat[BUF];
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if(i + 1 < total)
+        if(i_next >= 0)
         {
-            fetch(i + 1, BUF ? lds_q0 : lds_q1, BUF ? lds_g0 : lds_g1, lds_stat[BUF ^ 1]);
+            fetch(i_next, BUF ? lds_q0 : lds_q1, BUF ? lds_g0 : lds_g1, lds_stat[BUF ^ 1]);
         }
         int bq, qs;
         locate(i, bq, qs);
+        constexpr bool use_mask = EXPLICIT && decltype(masked_tag)::value;
         const int q0 = qs * kBwdStep;
         const int rows_here = min(kBwdStep, q_seq - q0);
+        const char *mask_step = static_cast<const char *>(p.mask)
+            + (int64_t)q0 * (int64_t)mask_row_bytes;
+        const uint32_t mask_last_row = (uint32_t)(rows_here - 1) * mask_row_bytes;
 
         // (one 32-query block at a time: half the accumulators live)
         // ---- S = Q K^T, dP = dA V^T: rows are queries, the lane's column its key;
@@ -620,21 +824,28 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
                     {
                         visible = visible && (my_k <= rel + q0 + qr);
                     }
-                    if(EXPLICIT)
+                    if(use_mask)
                     {
-                        const int64_t mi = (int64_t)(q0 + min(qr, rows_here - 1)) * p.mask_ld
-                            + (k_ok ? my_k : 0);
+                        // the row is the same for the lanes of one half: its
+                        // address is wave-common, the lane adds its key (and
+                        // four rows in the upper half, while those exist;
+                        // rows past the end read a row that exists and are
+                        // dropped by their logsumexp of +inf)
+                        const int rb = mb * 32 + 8 * rg + e;
+                        const char *mrow = mask_step
+                            + min((uint32_t)rb * mask_row_bytes, mask_last_row);
+                        const char *mp = mrow + (rb + 4 < rows_here ? mask_off_hi : mask_off_lo);
                         if(MODE == NNTILE_HIP_MASK_ADDITIVE)
                         {
                             const float add = T::to_float(
-                                    static_cast<const uint16_t *>(p.mask)[mi]);
+                                    *reinterpret_cast<const uint16_t *>(mp));
                             visible = visible && (add != neg_inf());
                             ex = fmaf(add, kLog2e, ex);
                         }
                         else
                         {
-                            visible = visible
-                                && (static_cast<const uint8_t *>(p.mask)[mi] != 0);
+                            const uint8_t shown = *reinterpret_cast<const uint8_t *>(mp);
+                        visible = visible && (shown != 0);
                         }
                     }
                     pv[r] = visible ? fast_exp2(ex) : 0.0f;
@@ -679,13 +890,29 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
             }
         }
     };
-    for(int i = 0; i < total; i += 2)
+    auto run = [&](int i, int i_next, auto buf_tag) __attribute__((always_inline))
     {
-        step(i, std::integral_constant<int, 0>{});
-        if(i + 1 < total)
+        if(EXPLICIT && !steps.is_open(i % kHeadStride))
         {
-            step(i + 1, std::integral_constant<int, 1>{});
+            step(i, i_next, buf_tag, std::true_type{});
         }
+        else
+        {
+            step(i, i_next, buf_tag, std::false_type{});
+        }
+    };
+    while(i_cur >= 0)
+    {
+        int i_next = walk_next(i_cur);
+        run(i_cur, i_next, std::integral_constant<int, 0>{});
+        i_cur = i_next;
+        if(i_cur < 0)
+        {
+            break;
+        }
+        i_next = walk_next(i_cur);
+        run(i_cur, i_next, std::integral_constant<int, 1>{});
+        i_cur = i_next;
     }
 
     // ---- dK (+)= scale dk, dV (+)= dv -------------------------------------------------
@@ -744,6 +971,18 @@ static int launch_bwd_mode(hipStream_t stream, const BwdParams &p)
     if(n_dq <= 0 || n_dkv <= 0 || n_dq > 0x7fffffff || n_dkv > 0x7fffffff)
     {
         return NNTILE_HIP_EINVAL;
+    }
+    if((MODE == NNTILE_HIP_MASK_ADDITIVE || MODE == NNTILE_HIP_MASK_BOOL)
+            && p.mask_class != nullptr)
+    {
+        const int64_t n_cls = ((p.q_seq + kBwdStep - 1) / kBwdStep) * p.class_ld;
+        hipLaunchKernelGGL((sdpa_bwd_mask_classes_kernel<T, MODE>), dim3((unsigned)n_cls),
+                dim3(256), 0, stream, p.mask, p.mask_ld, (int)p.q_seq, (int)p.k_seq,
+                const_cast<uint8_t *>(p.mask_class), p.class_ld);
+        if(hipGetLastError() != hipSuccess)
+        {
+            return NNTILE_HIP_ELAUNCH;
+        }
     }
     hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, HEAD, MODE>), dim3((unsigned)n_dq),
             dim3(kBwdThreads), 0, stream, p);

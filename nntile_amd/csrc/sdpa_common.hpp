@@ -90,6 +90,11 @@ struct BwdParams
     const void *K, *Q, *V, *A, *dA;
     const float *lse;
     float *D;               // workspace: written by the dQ kernel, read by the dK/dV kernel
+    // explicit masks: class of every 64 x 64 block of the mask, row = query
+    // block, class_ld entries per row (0 mixed, 1 nothing masked, 2 all
+    // hidden); null when the workspace has no room for it
+    const uint8_t *mask_class;
+    int32_t class_ld;
     void *dK, *dQ, *dV;
     int32_t batch, n_batch, kv_group;
     int32_t overwrite;      // 1: write the gradients, 0: add to what is there

@@ -126,7 +126,7 @@ def lib():
             f = getattr(L, "nntile_hip_sdpa_bwd_tile_" + t)
             f.argtypes = [_vp, ctypes.POINTER(BwdArgs)]
             f.restype = ctypes.c_int
-        L.nntile_hip_sdpa_bwd_workspace_bytes.argtypes = [_i64, _i64]
+        L.nntile_hip_sdpa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
         L.nntile_hip_sdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.argtypes = [ctypes.POINTER(TileArgs)]
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.restype = ctypes.c_size_t
@@ -222,6 +222,13 @@ def flash_sdpa_bwd(K, Q, V, A, dA, mask, lse, scratch_dQ, dK, dQ, dV, stream=Non
               _ptr(dK), _ptr(dQ), _ptr(dV)), "flash_sdpa_bwd")
 
 
+def sdpa_bwd_workspace_bytes(q_seq, k_seq, batch, mask_mode):
+    """Bytes of workspace sdpa_bwd_tile wants for these shapes."""
+    a = BwdArgs()
+    a.q_seq, a.k_seq, a.batch, a.mask_mode = q_seq, k_seq, batch, mask_mode
+    return lib().nntile_hip_sdpa_bwd_workspace_bytes(ctypes.byref(a))
+
+
 def sdpa_bwd_tile(K, Q, V, A, dA, mask, lse, dK, dQ, dV, mask_mode, n_batch=None,
                   kv_group=1, q_pos0=0, k_pos0=0, causal_offset=0, flags=0,
                   workspace=None, stream=None):
@@ -230,14 +237,14 @@ def sdpa_bwd_tile(K, Q, V, A, dA, mask, lse, dK, dQ, dV, mask_mode, n_batch=None
     _dev(K, Q, V, A, dA, mask, lse, dK, dQ, dV, workspace)
     batch, q_seq, head = Q.shape
     k_seq = K.shape[1]
-    need = lib().nntile_hip_sdpa_bwd_workspace_bytes(q_seq, batch)
-    if workspace is None:
-        workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
     a = BwdArgs()
     a.q_seq, a.k_seq, a.head, a.batch = q_seq, k_seq, head, batch
     a.n_batch = batch if n_batch is None else n_batch
     a.kv_group = kv_group
     a.mask_mode = mask_mode
+    if workspace is None:
+        need = lib().nntile_hip_sdpa_bwd_workspace_bytes(ctypes.byref(a))
+        workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
     a.flags = flags
     a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
     a.K, a.Q, a.V, a.A, a.dA = (t.data_ptr() for t in (K, Q, V, A, dA))

@@ -2,6 +2,8 @@
 through the C ABI.  Tolerances are the reference's own for its backward
 kernel (tests/kernel/flash_sdpa_bwd_cudnn.cc:312-327): relative Frobenius
 error 1e-2 for bf16 and 2e-3 for fp16."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -182,6 +184,18 @@ def test_inputs_unchanged_and_errors():
     with pytest.raises(hip_sdpa.SdpaError) as e:
         hip_sdpa.sdpa_bwd_tile(*ins, None, lse, *outs, hip_sdpa.MASK_ADDITIVE)
     assert e.value.code == hip_sdpa.EINVAL
+    # a mask given as values with rows of more than 2^24 keys is refused
+    # before anything is read (the sizes below are not those of the tensors)
+    a = hip_sdpa.BwdArgs()
+    a.q_seq, a.k_seq, a.head, a.batch, a.n_batch, a.kv_group = seq, (1 << 24) + 1, head, batch, batch, 1
+    a.mask_mode = hip_sdpa.MASK_BOOL
+    a.K, a.Q, a.V, a.A, a.dA = (t.data_ptr() for t in ins)
+    a.mask = ins[0].data_ptr()
+    a.lse = lse.data_ptr()
+    a.dK, a.dQ, a.dV = (t.data_ptr() for t in outs)
+    a.workspace, a.workspace_bytes = small.data_ptr(), 8
+    fn = hip_sdpa.lib().nntile_hip_sdpa_bwd_tile_bf16
+    assert fn(None, ctypes.byref(a)) == hip_sdpa.EUNSUPPORTED
 
 
 def test_codelet_body(oracle):
@@ -202,3 +216,61 @@ def test_codelet_body(oracle):
     torch.cuda.synchronize()
     for got, w, name in ((dK, want[0], "dK"), (dQ, want[1], "dQ"), (dV, want[2], "dV")):
         _check(got, w, dtype, name)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("form", ["additive", "bool"])
+@pytest.mark.parametrize("q_seq,k_seq", [(256, 1024), (200, 712), (130, 333), (320, 192)])
+@pytest.mark.parametrize("pattern", ["band", "late_start", "holes", "all_hidden", "all_open"])
+@pytest.mark.parametrize("room", [True, False])
+def test_mask_block_classes(oracle, dtype, form, q_seq, k_seq, pattern, room):
+    """Masks given as values are classified in 64 x 64 blocks first: steps
+    whose blocks hide everything are skipped, steps whose blocks mask nothing
+    read no mask values.  The patterns put the borders of those runs at,
+    before and after multiples of 64 on both axes; without room for the
+    classes in the workspace the kernels read every mask value instead.
+    Rows with no visible key have lse = -inf and contribute nothing."""
+    print("case bwd classes", dtype, form, q_seq, k_seq, pattern, room, flush=True)
+    batch, head = 2, 64
+    i = np.arange(q_seq)[:, None]
+    j = np.arange(k_seq)[None, :]
+    if pattern == "band":
+        mask = (j <= (k_seq // 3 + 2 * i)) & (j + 300 >= i)
+    elif pattern == "late_start":
+        mask = j >= (i % 7) * 3
+    elif pattern == "holes":
+        mask = ((j < 100) | (j >= 300)) & (i % 50 != 49)
+    elif pattern == "all_hidden":
+        mask = np.zeros((q_seq, k_seq), bool)
+    else:
+        mask = np.ones((q_seq, k_seq), bool)
+    mask = np.ascontiguousarray(np.broadcast_to(mask, (q_seq, k_seq)))
+    add = np.where(mask, 0, -np.inf).astype(np.float32)
+    (Q, K, V), (qf, kf, vf) = H.make_qkv(98, batch, q_seq, k_seq, head, dtype)
+    G, gf = _rounded(synth.randn(99, 0, batch * q_seq * head).reshape(batch, q_seq, head), dtype)
+    vis = mask.any(axis=1)
+    with np.errstate(all="ignore"):
+        A64, lse64 = oracle.sdpa_bruteforce_f64(kf, qf, vf, add)
+    A64 = np.where(vis[None, :, None], A64, 0.0)
+    lse64 = np.where(vis[None, :], lse64, -np.inf)
+    A, af = _rounded(A64, dtype)
+    lse = lse64.astype(np.float32)
+    with np.errstate(all="ignore"):
+        want = oracle.sdpa_bwd_flash_f64(kf, qf, vf, af, gf, np.where(vis[None, :], lse, 0.0),
+                                         np.where(vis[:, None], add, -np.inf))
+    m = (H.additive_mask(mask, dtype) if form == "additive" else torch.from_numpy(mask.copy())).cuda()
+    mm = hip_sdpa.MASK_ADDITIVE if form == "additive" else hip_sdpa.MASK_BOOL
+    ws = None if room else torch.empty(4 * q_seq * batch, dtype=torch.uint8, device="cuda")
+    dK, dQ, dV = (torch.full(t.shape, float("nan"), dtype=H.TORCH_DT[dtype], device="cuda")
+                  for t in (K, Q, V))
+    hip_sdpa.sdpa_bwd_tile(K.cuda(), Q.cuda(), V.cuda(), A.cuda(), G.cuda(), m,
+                           torch.from_numpy(lse).cuda(), dK, dQ, dV, mm, flags=hip_sdpa.OVERWRITE,
+                           workspace=ws)
+    torch.cuda.synchronize()
+    for got, w, name in ((dK, want[0], "dK"), (dQ, want[1], "dQ"), (dV, want[2], "dV")):
+        g = H.to_np(got).astype(np.float64)
+        assert np.all(np.isfinite(g)), name
+        if np.linalg.norm(w) == 0:
+            assert np.all(g == 0), name
+        else:
+            assert np.linalg.norm(g - w) / np.linalg.norm(w) < BWD_TOL[dtype], name
