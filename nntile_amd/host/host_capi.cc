@@ -66,6 +66,29 @@ void run_op(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *mask, AnyTensor *lse,
     }
 }
 
+template<typename T>
+void run_bwd(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *V, AnyTensor *A,
+        AnyTensor *dA, AnyTensor *mask, AnyTensor *lse, AnyTensor *dK,
+        AnyTensor *dQ, AnyTensor *dV)
+{
+    switch(op)
+    {
+        case 0:     // tensor-level, per-tile tasks, blocking
+            tensor::flash_sdpa_bwd_cudnn<T>(get<T>(K), get<T>(Q), get<T>(V),
+                    get<T>(A), get<T>(dA), get<T>(mask), get<fp32_t>(lse),
+                    get<T>(dK), get<T>(dQ), get<T>(dV));
+            break;
+        case 1:     // tile-level on single-tile tensors, blocking
+            tile::flash_sdpa_bwd_cudnn<T>(get<T>(K).get_tile(0), get<T>(Q).get_tile(0),
+                    get<T>(V).get_tile(0), get<T>(A).get_tile(0), get<T>(dA).get_tile(0),
+                    get<T>(mask).get_tile(0), get<fp32_t>(lse).get_tile(0),
+                    get<T>(dK).get_tile(0), get<T>(dQ).get_tile(0), get<T>(dV).get_tile(0));
+            break;
+        default:
+            throw std::runtime_error("unknown operation");
+    }
+}
+
 } // namespace
 
 extern "C"
@@ -175,6 +198,77 @@ int nntile_host_check_shapes(int level, const int64_t *desc, char *err, int errl
         return 0;
     }
     catch(const std::exception &e) { return fail(err, errlen, e); }
+}
+
+// op: 0 tensor::flash_sdpa_bwd_cudnn, 1 tile::flash_sdpa_bwd_cudnn (single-tile
+// tensors); dtype bf16 or fp16, as the reference's pack
+int nntile_host_flash_sdpa_bwd(int op, int dtype, void *K, void *Q, void *V,
+        void *A, void *dA, void *mask, void *lse, void *dK, void *dQ, void *dV,
+        char *err, int errlen)
+{
+    try
+    {
+        AnyTensor *t[10] = {static_cast<AnyTensor *>(K), static_cast<AnyTensor *>(Q),
+            static_cast<AnyTensor *>(V), static_cast<AnyTensor *>(A),
+            static_cast<AnyTensor *>(dA), static_cast<AnyTensor *>(mask),
+            static_cast<AnyTensor *>(lse), static_cast<AnyTensor *>(dK),
+            static_cast<AnyTensor *>(dQ), static_cast<AnyTensor *>(dV)};
+        if(dtype == DT_BF16) run_bwd<bf16_t>(op, t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7], t[8], t[9]);
+        else if(dtype == DT_FP16) run_bwd<fp16_t>(op, t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7], t[8], t[9]);
+        else throw std::runtime_error("flash_sdpa_bwd_cudnn: no fp32 instance");
+        return 0;
+    }
+    catch(const std::exception &e) { return fail(err, errlen, e); }
+}
+
+// Shape rules of the backward only: level 0 = tile, 1 = tensor; 10 blocks
+// (ndim, dims..., basetile dims...) in the order K, Q, V, A, dA, mask,
+// logsumexp, dK, dQ, dV.
+int nntile_host_check_shapes_bwd(int level, const int64_t *desc, char *err, int errlen)
+{
+    try
+    {
+        std::vector<tensor::TensorTraits> tt;
+        const int64_t *p = desc;
+        for(int i = 0; i < 10; ++i)
+        {
+            const int nd = static_cast<int>(*p++);
+            auto shape = vec(p, nd); p += nd;
+            auto base = vec(p, nd); p += nd;
+            tt.emplace_back(shape, base);
+        }
+        if(level == 0)
+        {
+            tile::flash_sdpa_bwd_cudnn_check(tt[0], tt[1], tt[2], tt[3], tt[4], tt[5],
+                    tt[6], tt[7], tt[8], tt[9]);
+        }
+        else
+        {
+            tensor::flash_sdpa_bwd_cudnn_check(tt[0], tt[1], tt[2], tt[3], tt[4], tt[5],
+                    tt[6], tt[7], tt[8], tt[9]);
+        }
+        return 0;
+    }
+    catch(const std::exception &e) { return fail(err, errlen, e); }
+}
+
+uint32_t nntile_host_footprint_bwd(int64_t seq, int64_t head, int64_t batch)
+{
+    return starpu::FlashSdpaBwdCudnn<std::tuple<bf16_t>>::hash_parameters(seq, head, batch);
+}
+
+int64_t nntile_host_tasks_submitted_bwd(int dtype)
+{
+    if(dtype == DT_BF16) return starpu::flash_sdpa_bwd_cudnn<bf16_t>().submitted;
+    if(dtype == DT_FP16) return starpu::flash_sdpa_bwd_cudnn<fp16_t>().submitted;
+    return -1;
+}
+
+const char *nntile_host_codelet_name_bwd(int dtype)
+{
+    if(dtype == DT_BF16) return starpu::flash_sdpa_bwd_cudnn<bf16_t>().name.c_str();
+    if(dtype == DT_FP16) return starpu::flash_sdpa_bwd_cudnn<fp16_t>().name.c_str();
+    return "";
 }
 
 uint32_t nntile_host_footprint(int64_t seq, int64_t head, int64_t batch)

@@ -247,6 +247,83 @@ template FlashSdpaFwdCudnn<std::tuple<bf16_t>> &flash_sdpa_fwd_cudnn<bf16_t>();
 template FlashSdpaFwdCudnn<std::tuple<fp16_t>> &flash_sdpa_fwd_cudnn<fp16_t>();
 template FlashSdpaFwdCudnn<std::tuple<fp32_t>> &flash_sdpa_fwd_cudnn<fp32_t>();
 
+// ---- backward codelet: src/starpu/flash_sdpa_bwd_cudnn.cc:31-196 ----------
+
+template<typename T>
+FlashSdpaBwdCudnn<std::tuple<T>>::FlashSdpaBwdCudnn():
+    name(std::string("nntile_flash_sdpa_bwd_cudnn_") + T::short_name)
+{
+}
+
+template<typename T>
+std::uint32_t FlashSdpaBwdCudnn<std::tuple<T>>::hash_parameters(Index seq,
+        Index head, Index batch)
+{
+    std::uint32_t hash = 0;
+    hash = crc32c_be_n(&seq, sizeof(seq), hash);
+    hash = crc32c_be_n(&head, sizeof(head), hash);
+    hash = crc32c_be_n(&batch, sizeof(batch), hash);
+    return hash;
+}
+
+template<> void FlashSdpaBwdCudnn<std::tuple<bf16_t>>::hip(void *buffers[], void *cl_args) noexcept
+{
+    nntile_hip_flash_sdpa_bwd_codelet_bf16(buffers, cl_args);
+}
+
+template<> void FlashSdpaBwdCudnn<std::tuple<fp16_t>>::hip(void *buffers[], void *cl_args) noexcept
+{
+    nntile_hip_flash_sdpa_bwd_codelet_fp16(buffers, cl_args);
+}
+
+template<typename T>
+void FlashSdpaBwdCudnn<std::tuple<T>>::submit(Index seq, Index head, Index batch,
+        Handle K, Handle Q, Handle V, Handle A, Handle dA, Handle mask,
+        Handle logsumexp, Handle dK, Handle dQ, Handle dV, Handle scratch_dK,
+        Handle scratch_dQ, Handle scratch_dV)
+{
+    auto *args = static_cast<args_t *>(std::malloc(sizeof(args_t)));
+    if(args == nullptr)
+    {
+        throw std::runtime_error("Error in flash_sdpa_bwd_cudnn task submission");
+    }
+    args->owner = this;
+    args->seq = seq;
+    args->head = head;
+    args->batch = batch;
+    // Buffer order and access modes of the reference
+    // (src/starpu/flash_sdpa_bwd_cudnn.cc:175-187):
+    //   K Q V A dA mask logsumexp (R), dK dQ dV (RW), three scratch buffers
+    const Handle *handles[13] = {&K, &Q, &V, &A, &dA, &mask, &logsumexp, &dK,
+        &dQ, &dV, &scratch_dK, &scratch_dQ, &scratch_dV};
+    nntile_hip_variable_interface ifs[13];
+    void *buffers[13];
+    for(int i = 0; i < 13; ++i)
+    {
+        ifs[i].id = 2;      // STARPU_VARIABLE_INTERFACE_ID
+        ifs[i].ptr = reinterpret_cast<std::uintptr_t>(handles[i]->get_ptr());
+        ifs[i].dev_handle = ifs[i].ptr;
+        ifs[i].offset = 0;
+        ifs[i].elemsize = handles[i]->size();
+        buffers[i] = &ifs[i];
+    }
+    (void)get_local_stream();
+    hip(buffers, args);
+    std::free(args);
+    ++submitted;
+}
+
+template<typename T> FlashSdpaBwdCudnn<std::tuple<T>> &flash_sdpa_bwd_cudnn()
+{
+    static FlashSdpaBwdCudnn<std::tuple<T>> codelet;
+    return codelet;
+}
+
+template class FlashSdpaBwdCudnn<std::tuple<bf16_t>>;
+template class FlashSdpaBwdCudnn<std::tuple<fp16_t>>;
+template FlashSdpaBwdCudnn<std::tuple<bf16_t>> &flash_sdpa_bwd_cudnn<bf16_t>();
+template FlashSdpaBwdCudnn<std::tuple<fp16_t>> &flash_sdpa_bwd_cudnn<fp16_t>();
+
 } // namespace starpu
 
 // ---------------------------------------------------------------------------
@@ -337,6 +414,93 @@ void flash_sdpa_fwd_cudnn(const Tile<T> &K, const Tile<T> &Q,
 NNTILE_HOST_INSTANTIATE_TILE(bf16_t)
 NNTILE_HOST_INSTANTIATE_TILE(fp16_t)
 NNTILE_HOST_INSTANTIATE_TILE(fp32_t)
+
+// ---- backward: src/tile/flash_sdpa_bwd_cudnn.cc:24-151 ---------------------
+
+// The ten traits share the rules below at both levels (tile and tensor).
+template<typename Traits>
+static void bwd_common_check(const Traits &K, const Traits &Q, const Traits &V,
+        const Traits &A, const Traits &dA, const Traits &mask,
+        const Traits &logsumexp, const Traits &dK, const Traits &dQ,
+        const Traits &dV)
+{
+    const Traits *five[8] = {&K, &Q, &V, &A, &dA, &dK, &dQ, &dV};
+    static const char *const names[8] = {"K", "Q", "V", "A", "dA", "dK", "dQ", "dV"};
+    for(int i = 0; i < 8; ++i)
+    {
+        if(five[i]->ndim != 5)
+        {
+            throw std::runtime_error(std::string(names[i]) + ".ndim != 5");
+        }
+    }
+    require(mask.ndim == 2, "mask.ndim != 2");
+    require(logsumexp.ndim == 4, "logsumexp.ndim != 4");
+    // every 5-D operand has the shape of K (square tile pairs only)
+    for(int i = 1; i < 8; ++i)
+    {
+        if(K.shape != five[i]->shape)
+        {
+            throw std::runtime_error(std::string("K.shape != ") + names[i] + ".shape");
+        }
+    }
+    require(K.shape[1] == mask.shape[0] && K.shape[1] == mask.shape[1],
+            "Mask shape mismatch");
+    require(K.shape[1] == logsumexp.shape[0], "logsumexp axis 0 must match sequence length");
+    require(K.shape[2] == logsumexp.shape[1], "logsumexp axis 1 must match batch");
+    require(K.shape[3] == logsumexp.shape[2], "logsumexp axis 2 must match kv_group_size");
+    require(K.shape[4] == logsumexp.shape[3], "logsumexp axis 3 must match n_head_kv");
+}
+
+void flash_sdpa_bwd_cudnn_check(const TileTraits &K, const TileTraits &Q,
+        const TileTraits &V, const TileTraits &A, const TileTraits &dA,
+        const TileTraits &mask, const TileTraits &logsumexp,
+        const TileTraits &dK, const TileTraits &dQ, const TileTraits &dV)
+{
+    bwd_common_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
+}
+
+template<typename T>
+void flash_sdpa_bwd_cudnn_async(const Tile<T> &K, const Tile<T> &Q,
+        const Tile<T> &V, const Tile<T> &A, const Tile<T> &dA,
+        const Tile<T> &mask, const Tile<fp32_t> &logsumexp, const Tile<T> &dK,
+        const Tile<T> &dQ, const Tile<T> &dV)
+{
+    flash_sdpa_bwd_cudnn_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
+    const Index seq = K.shape[1];
+    const Index head = K.shape[0];
+    const Index batch = K.shape[2] * K.shape[3] * K.shape[4];
+    // The reference registers three scratch handles of the size of the
+    // gradients.  The HIP body adds into dK, dQ, dV directly and only uses
+    // scratch_dQ (for the row dots dA.A and the classes of the mask blocks);
+    // the other two stay empty and keep the submit signature.
+    starpu::VariableHandle scratch_dK, scratch_dV;
+    starpu::VariableHandle scratch_dQ(sizeof(typename T::storage_t) * dQ.nelems);
+    starpu::flash_sdpa_bwd_cudnn<T>().submit(seq, head, batch, K, Q, V, A, dA,
+            mask, logsumexp, dK, dQ, dV, scratch_dK, scratch_dQ, scratch_dV);
+    scratch_dK.unregister_submit();
+    scratch_dQ.unregister_submit();
+    scratch_dV.unregister_submit();
+}
+
+template<typename T>
+void flash_sdpa_bwd_cudnn(const Tile<T> &K, const Tile<T> &Q,
+        const Tile<T> &V, const Tile<T> &A, const Tile<T> &dA,
+        const Tile<T> &mask, const Tile<fp32_t> &logsumexp, const Tile<T> &dK,
+        const Tile<T> &dQ, const Tile<T> &dV)
+{
+    flash_sdpa_bwd_cudnn_async<T>(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
+    starpu::task_wait_for_all();
+}
+
+#define NNTILE_HOST_INSTANTIATE_TILE_BWD(T) \
+    template void flash_sdpa_bwd_cudnn_async<T>(const Tile<T> &, const Tile<T> &, \
+            const Tile<T> &, const Tile<T> &, const Tile<T> &, const Tile<T> &, \
+            const Tile<fp32_t> &, const Tile<T> &, const Tile<T> &, const Tile<T> &); \
+    template void flash_sdpa_bwd_cudnn<T>(const Tile<T> &, const Tile<T> &, \
+            const Tile<T> &, const Tile<T> &, const Tile<T> &, const Tile<T> &, \
+            const Tile<fp32_t> &, const Tile<T> &, const Tile<T> &, const Tile<T> &);
+NNTILE_HOST_INSTANTIATE_TILE_BWD(bf16_t)
+NNTILE_HOST_INSTANTIATE_TILE_BWD(fp16_t)
 
 } // namespace tile
 
@@ -648,6 +812,99 @@ void flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
         }
     }
 }
+
+// ---- backward: src/tensor/flash_sdpa_bwd_cudnn.cc:22-261 -------------------
+
+void flash_sdpa_bwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
+        const TensorTraits &V, const TensorTraits &A, const TensorTraits &dA,
+        const TensorTraits &mask, const TensorTraits &logsumexp,
+        const TensorTraits &dK, const TensorTraits &dQ, const TensorTraits &dV)
+{
+    tile::bwd_common_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
+    // basetile compatibility for multi-tile execution
+    const auto &Kb = K.basetile_shape, &Qb = Q.basetile_shape,
+          &Vb = V.basetile_shape, &Ab = A.basetile_shape,
+          &dAb = dA.basetile_shape, &dKb = dK.basetile_shape,
+          &dQb = dQ.basetile_shape, &dVb = dV.basetile_shape,
+          &Mb = mask.basetile_shape, &Lb = logsumexp.basetile_shape;
+    require(Qb == dQb && Qb == Ab && Qb == dAb, "Q, dQ, A, dA basetile shapes must match");
+    for(Index d : {Index(0), Index(2), Index(3), Index(4)})
+    {
+        require(Kb[d] == Qb[d], "K and Q basetile shapes mismatch");
+        require(Vb[d] == Qb[d], "V and Q basetile shapes mismatch");
+        require(dKb[d] == Qb[d], "dK and Q basetile shapes mismatch");
+        require(dVb[d] == Qb[d], "dV and Q basetile shapes mismatch");
+    }
+    require(Mb[0] == Kb[1], "mask basetile axis 0 must match K basetile sequence dimension");
+    require(Mb[1] == Qb[1], "mask basetile axis 1 must match Q basetile sequence dimension");
+    require(Lb[0] == Qb[1] && Lb[1] == Qb[2] && Lb[2] == Qb[3] && Lb[3] == Qb[4],
+            "logsumexp basetile shape must match Q basetile shape (excluding head dimension)");
+    require(Kb[0] == K.shape[0] && Qb[0] == Q.shape[0] && Vb[0] == V.shape[0]
+            && Ab[0] == A.shape[0] && dAb[0] == dA.shape[0] && dKb[0] == dK.shape[0]
+            && dQb[0] == dQ.shape[0] && dVb[0] == dV.shape[0],
+            "head dimension must not be tiled");
+}
+
+template<typename T>
+void flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV)
+{
+    flash_sdpa_bwd_cudnn_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
+    const Index num_k_seq_tiles = K.grid.shape[1];
+    // dQ tiles define the Q, A, dA and logsumexp tiles; each gets the
+    // contribution of every key tile along the sequence axis, and each key
+    // tile's dK, dV collect over the dQ tiles of their slab
+    // (src/tensor/flash_sdpa_bwd_cudnn.cc:172-247)
+    for(Index dq_linear = 0; dq_linear < dQ.grid.nelems; ++dq_linear)
+    {
+        const auto dq_index = dQ.grid.linear_to_index(dq_linear);
+        const auto &Q_tile = Q.get_tile(dq_linear);
+        const auto &A_tile = A.get_tile(dq_linear);
+        const auto &dA_tile = dA.get_tile(dq_linear);
+        const auto &dQ_tile = dQ.get_tile(dq_linear);
+        const auto &lse_tile = logsumexp.get_tile(
+                {dq_index[1], dq_index[2], dq_index[3], dq_index[4]});
+        const Index seq = dQ_tile.shape[1];
+        for(Index k_idx = 0; k_idx < num_k_seq_tiles; ++k_idx)
+        {
+            auto kv_index = dq_index;
+            kv_index[1] = k_idx;
+            const auto &K_tile = K.get_tile(kv_index);
+            const auto &V_tile = V.get_tile(kv_index);
+            const auto &dK_tile = dK.get_tile(kv_index);
+            const auto &dV_tile = dV.get_tile(kv_index);
+            const auto &mask_tile = mask.get_tile({k_idx, dq_index[1]});
+            require(K_tile.shape[1] == seq, "K tile sequence length mismatches dQ tile");
+            require(mask_tile.shape[0] == K_tile.shape[1] && mask_tile.shape[1] == seq,
+                    "Mask tile shape mismatches dQ/K tiles");
+            require(lse_tile.shape[0] == seq, "logsumexp tile shape mismatches dQ tile");
+            tile::flash_sdpa_bwd_cudnn_async<T>(K_tile, Q_tile, V_tile, A_tile,
+                    dA_tile, mask_tile, lse_tile, dK_tile, dQ_tile, dV_tile);
+        }
+    }
+}
+
+template<typename T>
+void flash_sdpa_bwd_cudnn(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV)
+{
+    flash_sdpa_bwd_cudnn_async<T>(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
+    starpu::task_wait_for_all();
+}
+
+#define NNTILE_HOST_INSTANTIATE_TENSOR_BWD(T) \
+    template void flash_sdpa_bwd_cudnn_async<T>(const Tensor<T> &, const Tensor<T> &, \
+            const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, \
+            const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &); \
+    template void flash_sdpa_bwd_cudnn<T>(const Tensor<T> &, const Tensor<T> &, \
+            const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, \
+            const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &);
+NNTILE_HOST_INSTANTIATE_TENSOR_BWD(bf16_t)
+NNTILE_HOST_INSTANTIATE_TENSOR_BWD(fp16_t)
 
 #define NNTILE_HOST_INSTANTIATE_TENSOR(T) \
     template class Tensor<T>; \

@@ -8,6 +8,10 @@
 //                                 src/starpu/flash_sdpa_fwd_cudnn.cc:37-296
 //   tile::flash_sdpa_fwd_cudnn*   src/tile/flash_sdpa_fwd_cudnn.cc:25-213
 //   tensor::flash_sdpa_fwd_cudnn* src/tensor/flash_sdpa_fwd_cudnn.cc:23-297
+//   starpu::FlashSdpaBwdCudnn     include/nntile/starpu/flash_sdpa_bwd_cudnn.hh:44-187,
+//                                 src/starpu/flash_sdpa_bwd_cudnn.cc:31-196
+//   tile::flash_sdpa_bwd_cudnn*   src/tile/flash_sdpa_bwd_cudnn.cc:24-151
+//   tensor::flash_sdpa_bwd_cudnn* src/tensor/flash_sdpa_bwd_cudnn.cc:22-261
 // What differs, on purpose: the codelet carries a HIP body (the C-ABI entry
 // point nntile_hip_flash_sdpa_fwd_codelet_<T>) next to the empty CPU list, the
 // pack gains fp32, and tensor:: gains flash_sdpa_fwd_hip_async, which merges
@@ -119,6 +123,36 @@ public:
 //! One codelet object per value type, looked up by type
 template<typename T> FlashSdpaFwdCudnn<std::tuple<T>> &flash_sdpa_fwd_cudnn();
 
+//! Wrapper of the backward codelet for one value type (bf16, fp16)
+template<typename T> class FlashSdpaBwdCudnn;
+
+template<typename T>
+class FlashSdpaBwdCudnn<std::tuple<T>>
+{
+public:
+    std::string name;       // "nntile_flash_sdpa_bwd_cudnn_<type>"
+    struct args_t
+    {
+        FlashSdpaBwdCudnn<std::tuple<T>> *owner;
+        Index seq;
+        Index head;
+        Index batch;
+    };
+    FlashSdpaBwdCudnn();
+    static std::uint32_t hash_parameters(Index seq, Index head, Index batch);
+    static constexpr std::array<void (*)(void **, void *), 1> cpu_funcs = {nullptr};
+    static void hip(void *buffers[], void *cl_args) noexcept;
+    //! Handles in the reference's order; dK, dQ, dV are read-write (the
+    //! gradients of the tile pair are added), the last three are scratch
+    void submit(Index seq, Index head, Index batch, Handle K, Handle Q,
+            Handle V, Handle A, Handle dA, Handle mask, Handle logsumexp,
+            Handle dK, Handle dQ, Handle dV, Handle scratch_dK,
+            Handle scratch_dQ, Handle scratch_dV);
+    Index submitted = 0;
+};
+
+template<typename T> FlashSdpaBwdCudnn<std::tuple<T>> &flash_sdpa_bwd_cudnn();
+
 } // namespace starpu
 
 namespace tile
@@ -154,6 +188,25 @@ template<typename T>
 void flash_sdpa_fwd_cudnn(const Tile<T> &K, const Tile<T> &Q,
         const Tile<T> &mask, const Tile<fp32_t> &logsumexp, const Tile<T> &V,
         const Tile<T> &A);
+
+//! Shape rules of one backward tile task; throws std::runtime_error
+void flash_sdpa_bwd_cudnn_check(const TileTraits &K, const TileTraits &Q,
+        const TileTraits &V, const TileTraits &A, const TileTraits &dA,
+        const TileTraits &mask, const TileTraits &logsumexp,
+        const TileTraits &dK, const TileTraits &dQ, const TileTraits &dV);
+
+//! dK, dQ, dV += gradients of one (query tile, key tile) pair
+template<typename T>
+void flash_sdpa_bwd_cudnn_async(const Tile<T> &K, const Tile<T> &Q,
+        const Tile<T> &V, const Tile<T> &A, const Tile<T> &dA,
+        const Tile<T> &mask, const Tile<fp32_t> &logsumexp, const Tile<T> &dK,
+        const Tile<T> &dQ, const Tile<T> &dV);
+
+template<typename T>
+void flash_sdpa_bwd_cudnn(const Tile<T> &K, const Tile<T> &Q,
+        const Tile<T> &V, const Tile<T> &A, const Tile<T> &dA,
+        const Tile<T> &mask, const Tile<fp32_t> &logsumexp, const Tile<T> &dK,
+        const Tile<T> &dQ, const Tile<T> &dV);
 
 } // namespace tile
 
@@ -211,6 +264,25 @@ template<typename T>
 void flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
         int mask_mode, Index causal_offset, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &V, const Tensor<T> &A, bool overwrite);
+
+//! Shape and tiling rules of the tensor-level backward; throws
+void flash_sdpa_bwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
+        const TensorTraits &V, const TensorTraits &A, const TensorTraits &dA,
+        const TensorTraits &mask, const TensorTraits &logsumexp,
+        const TensorTraits &dK, const TensorTraits &dQ, const TensorTraits &dV);
+
+//! One tile task per (dQ tile, key tile) pair, in the reference's order
+template<typename T>
+void flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV);
+
+template<typename T>
+void flash_sdpa_bwd_cudnn(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV);
 
 } // namespace tensor
 

@@ -37,6 +37,16 @@ def lib():
                                                  ctypes.c_int]
         L.nntile_host_check_shapes.argtypes = [ctypes.c_int, ctypes.POINTER(i64), ctypes.c_char_p,
                                                ctypes.c_int]
+        L.nntile_host_flash_sdpa_bwd.argtypes = [ctypes.c_int, ctypes.c_int] + [vp] * 10 + [
+            ctypes.c_char_p, ctypes.c_int]
+        L.nntile_host_check_shapes_bwd.argtypes = [ctypes.c_int, ctypes.POINTER(i64), ctypes.c_char_p,
+                                                   ctypes.c_int]
+        L.nntile_host_footprint_bwd.argtypes = [i64, i64, i64]
+        L.nntile_host_footprint_bwd.restype = ctypes.c_uint32
+        L.nntile_host_tasks_submitted_bwd.argtypes = [ctypes.c_int]
+        L.nntile_host_tasks_submitted_bwd.restype = i64
+        L.nntile_host_codelet_name_bwd.argtypes = [ctypes.c_int]
+        L.nntile_host_codelet_name_bwd.restype = ctypes.c_char_p
         L.nntile_host_footprint.argtypes = [i64, i64, i64]
         L.nntile_host_footprint.restype = ctypes.c_uint32
         L.nntile_host_tasks_submitted.argtypes = [ctypes.c_int]
@@ -97,6 +107,22 @@ def flash_sdpa_fwd(op, K, Q, mask, lse, V, A, mask_mode=0, offset=0, overwrite=F
           None if mask is None else mask.h, lse.h, V.h, A.h, mask_mode, offset, int(overwrite))
 
 
+def flash_sdpa_bwd(op, K, Q, V, A, dA, mask, lse, dK, dQ, dV):
+    """tensor::flash_sdpa_bwd_cudnn (op 0) or tile::flash_sdpa_bwd_cudnn (op 1):
+    the gradients are added to dK, dQ, dV."""
+    _call(lib().nntile_host_flash_sdpa_bwd, op, DTYPES[Q.dtype],
+          *(t.h for t in (K, Q, V, A, dA, mask, lse, dK, dQ, dV)))
+
+
+def check_shapes_bwd(level, specs):
+    """specs: ten (shape, basetile) pairs in the order K, Q, V, A, dA, mask,
+    logsumexp, dK, dQ, dV."""
+    flat = []
+    for shape, base in specs:
+        flat += [len(shape)] + list(shape) + list(base)
+    _call(lib().nntile_host_check_shapes_bwd, level, _arr(flat))
+
+
 def check_shapes(level, specs):
     """specs: six (shape, basetile) pairs in the order K, Q, mask, logsumexp, V, A."""
     flat = []
@@ -107,6 +133,18 @@ def check_shapes(level, specs):
 
 def footprint(seq, head, batch):
     return int(lib().nntile_host_footprint(seq, head, batch))
+
+
+def footprint_bwd(seq, head, batch):
+    return int(lib().nntile_host_footprint_bwd(seq, head, batch))
+
+
+def tasks_submitted_bwd(dtype):
+    return int(lib().nntile_host_tasks_submitted_bwd(DTYPES[dtype]))
+
+
+def codelet_name_bwd(dtype):
+    return lib().nntile_host_codelet_name_bwd(DTYPES[dtype]).decode()
 
 
 def tasks_submitted(dtype):
