@@ -70,6 +70,29 @@ struct BwdTile
 
 // The registers of a 32x32 accumulator tile of lane (col, half): register r is
 // row 8*(r/4) + 4*half + r%4 of the tile, column col.
+// Workgroup number -> (batch entry, block along the sequence).  Workgroups
+// go to the 8 XCDs round robin: the entries of the batch are dealt so that
+// all blocks of one entry run on one XCD and share its L2, and the blocks are
+// taken in the order longest first (`last_first`: from the last block down).
+__device__ __forceinline__ void map_workgroup(unsigned wg, int entries, int blocks,
+        bool last_first, int &entry, int &block)
+{
+    int i;
+    if((entries & 7) == 0)
+    {
+        const int per_xcd = entries >> 3;
+        i = (int)(wg >> 3);
+        entry = (int)(wg & 7u) * per_xcd + i % per_xcd;
+        i /= per_xcd;
+    }
+    else
+    {
+        entry = (int)(wg % (unsigned)entries);
+        i = (int)(wg / (unsigned)entries);
+    }
+    block = last_first ? blocks - 1 - i : i;
+}
+
 __device__ __forceinline__ int tile_row(int r, int half)
 {
     return 8 * (r >> 2) + 4 * half + (r & 3);
@@ -235,8 +258,10 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
     const int half = lane >> 5;
 
     const int q_blocks = (int)((p.q_seq + kBwdRows - 1) / kBwdRows);
-    const int b = blockIdx.x / q_blocks;
-    const int q_row0 = (blockIdx.x % q_blocks) * kBwdRows;
+    // the last query blocks see the most keys under a causal mask: first
+    int b, q_block;
+    map_workgroup(blockIdx.x, p.batch, q_blocks, true, b, q_block);
+    const int q_row0 = q_block * kBwdRows;
     const int kvb = kv_entry(b, p.n_batch, p.kv_group);
     const int q_seq = (int)p.q_seq, k_seq = (int)p.k_seq;
     const int my_q = q_row0 + wave * 32 + col;
@@ -590,8 +615,10 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
 
     const int q_seq = (int)p.q_seq, k_seq = (int)p.k_seq;
     const int k_blocks = (k_seq + kDkvRows - 1) / kDkvRows;
-    const int kvb = blockIdx.x / k_blocks;          // nb + n_batch*hkv
-    const int k_row0 = (blockIdx.x % k_blocks) * kDkvRows;
+    // the first key blocks are seen by the most queries under a causal mask
+    int kvb, k_block;                               // kvb = nb + n_batch*hkv
+    map_workgroup(blockIdx.x, p.batch / p.kv_group, k_blocks, false, kvb, k_block);
+    const int k_row0 = k_block * kDkvRows;
     const int nb = kvb % p.n_batch, hkv = kvb / p.n_batch;
     const int my_k = k_row0 + wave * 32 + col;
     const bool k_ok = my_k < k_seq;
