@@ -35,6 +35,11 @@
 namespace nntile_hip
 {
 
+// Where the tile loads of the next step are issued: 0 = all at the start of
+// the step, 1 = between the MFMAs of the step's first half, 2 = of the whole
+#ifndef NNTILE_BWD_SPREAD
+#define NNTILE_BWD_SPREAD 2
+#endif
 constexpr int kBwdRows = 128;       // queries (dQ kernel) / keys (dK,dV kernel) per workgroup
 constexpr int kBwdStep = 64;        // rows of the other axis per step
 constexpr int kBwdThreads = 256;
@@ -368,20 +373,31 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
     const char *Vb = static_cast<const char *>(p.V) + (int64_t)kvb * k_seq * RB;
     // loads of key step g; rows past the end are clamped to the last row
     // (their probabilities are exactly 0)
-    auto fetch = [&](int g, char *kdst_base, char *vdst_base)
+    // (a wave gets one such load accepted every ~64 cycles and stands still
+    // until then: inside the loop the loads go between the MFMAs, one K and
+    // one V load at a time)
+    auto fetch_piece = [&](int g, char *kdst_base, char *vdst_base, int i)
+        __attribute__((always_inline))
     {
         const int row0 = g * kBwdStep;
         const int last = min(kBwdStep, k_seq - row0) - 1;
         char *kdst = kdst_base + wave_u * LOADS_PER_WAVE * 1024;
         char *vdst = vdst_base + wave_u * LOADS_PER_WAVE * 1024;
+        const uint32_t back = (uint32_t)(max(ld_row[i] - last, 0) * RB);
+        load_to_lds16<0, false>(Kb + (int64_t)row0 * RB, ld_goff[i] - back, kdst + i * 1024);
+        load_to_lds16<0, false>(Vb + (int64_t)row0 * RB, ld_goff[i] - back, vdst + i * 1024);
+    };
+    auto fetch = [&](int g, char *kdst_base, char *vdst_base)
+    {
 #pragma unroll
         for(int i = 0; i < LOADS_PER_WAVE; ++i)
         {
-            const uint32_t back = (uint32_t)(max(ld_row[i] - last, 0) * RB);
-            load_to_lds16<0, false>(Kb + (int64_t)row0 * RB, ld_goff[i] - back, kdst + i * 1024);
-            load_to_lds16<0, false>(Vb + (int64_t)row0 * RB, ld_goff[i] - back, vdst + i * 1024);
+            fetch_piece(g, kdst_base, vdst_base, i);
         }
     };
+    constexpr int FETCH_STRIDE = (NNTILE_BWD_SPREAD == 2 ? 2 : 1) * KSTEPS / LOADS_PER_WAVE;
+    static_assert(FETCH_STRIDE >= 1 && 1 + (LOADS_PER_WAVE - 1) * FETCH_STRIDE < 2 * KSTEPS,
+            "the pieces of a fetch must fit between the MFMAs of a step");
 
     f32x16 acc[DBLOCKS];
 #pragma unroll
@@ -421,7 +437,9 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
         const char *Vs = BUF ? lds_v1 : lds_v0;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if(g_next >= 0)
+        // the last step loads its own tile once more, rather than branch
+        const int g_fetch = g_next >= 0 ? g_next : g;
+        if(NNTILE_BWD_SPREAD == 0 && g_next >= 0)
         {
             fetch(g_next, BUF ? lds_k0 : lds_k1, BUF ? lds_v0 : lds_v1);
         }
@@ -457,6 +475,14 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
                 const vec8 va = *reinterpret_cast<const vec8 *>(Vs + row_raddr[mb][ks]);
                 sv = T::mfma(ka, qf[ks], sv);
                 dpv = T::mfma(va, gf[ks], dpv);
+#pragma unroll
+                for(int j = 0; j < LOADS_PER_WAVE; ++j)
+                {
+                    if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
+                    {
+                        fetch_piece(g_fetch, BUF ? lds_k0 : lds_k1, BUF ? lds_v0 : lds_v1, j);
+                    }
+                }
             }
             float dsv[16];
 #pragma unroll
@@ -536,6 +562,9 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
         run(g_cur, g_next, std::integral_constant<int, 1>{});
         g_cur = g_next;
     }
+    // (the last step's spare loads into LDS must have landed before the
+    // workgroup's LDS can be given away)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // ---- dQ (+)= scale acc: register r of block db is head value
     // db*32 + tile_row(r, half); four consecutive ones per 8-byte store ----------------
@@ -741,26 +770,21 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
     };
     // loads of walk position i: the Q and dA rows straight into LDS, the
     // logsumexp and D of its queries through registers (threads 0..127)
-    auto fetch = [&](int i, char *qdst_base, char *gdst_base, float (*stat)[kBwdStep])
+    // (inside the loop the tile loads go between the MFMAs, one Q and one dA
+    // load at a time: a wave stands still ~64 cycles per load)
+    auto fetch_piece = [&](int bq, int row0, int last, char *qdst_base, char *gdst_base, int j)
+        __attribute__((always_inline))
     {
-        int bq, qs;
-        locate(i, bq, qs);
-        const int row0 = qs * kBwdStep;
-        const int last = min(kBwdStep, q_seq - row0) - 1;
-        if(wave_u < LOADERS)
-        {
-            const char *Qp = static_cast<const char *>(p.Q) + ((int64_t)bq * q_seq + row0) * RB;
-            const char *Gp = static_cast<const char *>(p.dA) + ((int64_t)bq * q_seq + row0) * RB;
-            char *qdst = qdst_base + wave_u * LPW * 1024;
-            char *gdst = gdst_base + wave_u * LPW * 1024;
-#pragma unroll
-            for(int j = 0; j < LPW; ++j)
-            {
-                const uint32_t back = (uint32_t)(max(ld_row[j] - last, 0) * RB);
-                load_to_lds16<0, false>(Qp, ld_goff[j] - back, qdst + j * 1024);
-                load_to_lds16<0, false>(Gp, ld_goff[j] - back, gdst + j * 1024);
-            }
-        }
+        const char *Qp = static_cast<const char *>(p.Q) + ((int64_t)bq * q_seq + row0) * RB;
+        const char *Gp = static_cast<const char *>(p.dA) + ((int64_t)bq * q_seq + row0) * RB;
+        char *qdst = qdst_base + wave_u * LPW * 1024;
+        char *gdst = gdst_base + wave_u * LPW * 1024;
+        const uint32_t back = (uint32_t)(max(ld_row[j] - last, 0) * RB);
+        load_to_lds16<0, false>(Qp, ld_goff[j] - back, qdst + j * 1024);
+        load_to_lds16<0, false>(Gp, ld_goff[j] - back, gdst + j * 1024);
+    };
+    auto fetch_stat = [&](int bq, int row0, int last, float (*stat)[kBwdStep])
+    {
         if(tid < 2 * kBwdStep)
         {
             const int which = tid / kBwdStep, r = tid % kBwdStep;
@@ -778,6 +802,25 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
             stat[which][r] = v;
         }
     };
+    constexpr int FETCH_STRIDE = (NNTILE_BWD_SPREAD == 2 ? 2 : 1) * KSTEPS / LPW;
+    static_assert(FETCH_STRIDE >= 1 && 1 + (LPW - 1) * FETCH_STRIDE < 2 * KSTEPS,
+            "the pieces of a fetch must fit between the MFMAs of a step");
+    auto fetch = [&](int i, char *qdst_base, char *gdst_base, float (*stat)[kBwdStep])
+    {
+        int bq, qs;
+        locate(i, bq, qs);
+        const int row0 = qs * kBwdStep;
+        const int last = min(kBwdStep, q_seq - row0) - 1;
+        if(wave_u < LOADERS)
+        {
+#pragma unroll
+            for(int j = 0; j < LPW; ++j)
+            {
+                fetch_piece(bq, row0, last, qdst_base, gdst_base, j);
+            }
+        }
+        fetch_stat(bq, row0, last, stat);
+    };
 
     int i_cur = walk_begin();
     if(i_cur >= 0)
@@ -793,9 +836,25 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
         const float (*stat)[kBwdStep] = lds_stat[BUF];
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+        // the statistics of the next step now, its tiles between the MFMAs
+        // below (the last step loads its own tiles once more, rather than
+        // branch)
+        int bq_f, qs_f;
+        locate(i_next >= 0 ? i_next : i, bq_f, qs_f);
+        const int row0_f = qs_f * kBwdStep;
+        const int last_f = min(kBwdStep, q_seq - row0_f) - 1;
         if(i_next >= 0)
         {
-            fetch(i_next, BUF ? lds_q0 : lds_q1, BUF ? lds_g0 : lds_g1, lds_stat[BUF ^ 1]);
+            fetch_stat(bq_f, row0_f, last_f, lds_stat[BUF ^ 1]);
+            if(NNTILE_BWD_SPREAD == 0 && wave_u < LOADERS)
+            {
+#pragma unroll
+                for(int j = 0; j < LPW; ++j)
+                {
+                    fetch_piece(bq_f, row0_f, last_f, BUF ? lds_q0 : lds_q1,
+                            BUF ? lds_g0 : lds_g1, j);
+                }
+            }
         }
         int bq, qs;
         locate(i, bq, qs);
@@ -830,6 +889,18 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
                     const vec8 ga = *reinterpret_cast<const vec8 *>(Gs + row_raddr[ks]
                             + mb * 32 * RB);
                     dpv = T::mfma(ga, vf[ks], dpv);
+                }
+                if(wave_u < LOADERS)
+                {
+#pragma unroll
+                    for(int j = 0; j < LPW; ++j)
+                    {
+                        if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
+                        {
+                            fetch_piece(bq_f, row0_f, last_f, BUF ? lds_q0 : lds_q1,
+                                    BUF ? lds_g0 : lds_g1, j);
+                        }
+                    }
                 }
             }
             float pv[16], dsv[16];
@@ -941,6 +1012,9 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
         run(i_cur, i_next, std::integral_constant<int, 1>{});
         i_cur = i_next;
     }
+    // (the last step's spare loads into LDS must have landed before the
+    // workgroup's LDS can be given away)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // ---- dK (+)= scale dk, dV (+)= dv -------------------------------------------------
     if(!k_ok)
