@@ -190,7 +190,7 @@ def bench_backward(cfg, steps, warmup):
     return {"ms_per_step": round(wall, 4), "device_ms_per_step": round(dev, 4),
             "tflops": round(fl / (dev * 1e-3) / 1e12, 1), "flops_per_step": fl,
             "frac_of_peak": round(fl / (dev * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
-            "what": "backward of %s in one call (dQ kernel + dK/dV kernel), analytic causal "
+            "what": "backward of %s in one call (row dots + one launch for dQ, dK, dV), analytic causal "
                     "mask, gradients written" % cfg.name}
 
 

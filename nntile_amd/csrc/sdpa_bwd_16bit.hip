@@ -9,20 +9,19 @@
 //
 // (include/nntile/kernel/flash_sdpa_bwd_cudnn/cuda.hh:44-68 is the interface
 // this replaces; tests/kernel/flash_sdpa_bwd_cudnn.cc:174-262 the arithmetic).
-// Two kernels (the second launched once per gradient), no atomics, results
-// independent of timing:
+// A small kernel writes D; then ONE launch computes the three gradients, each
+// by its own workgroups (no atomics, results independent of timing):
 //
-//  * sdpa_bwd_dq_kernel: a workgroup owns 128 queries (a wavefront 32, a lane
+//  * sdpa_bwd_dq_body: a workgroup owns 128 queries (a wavefront 32, a lane
 //    one query) and walks the keys in steps of 64, as the forward kernel does:
 //    S^T = K Q^T and dP^T = V dA^T with Q and dA fragments in registers and K, V
 //    rows from LDS; dS^T packed to 16 bits is the B operand of
 //    dQ^T += K^T dS^T, whose A operand comes through the transposing LDS read.
-//    It also writes D for the second kernel.
-//  * sdpa_bwd_dkv_kernel: a workgroup owns 128 keys (a lane one key) and walks
-//    the queries of every head of its group in steps of 64: S = Q K^T and
-//    dP = dA V^T with K and V fragments in registers and Q, dA rows from LDS;
-//    dV^T += dA^T P and dK^T += Q^T dS through transposing reads of the same
-//    two LDS tiles.
+//  * sdpa_bwd_dkv_body<PART>: a workgroup owns 128 keys (a lane one key) and
+//    walks the queries of every head of its group in steps of 64: S = Q K^T
+//    and dP = dA V^T with K and V fragments in registers and Q, dA rows from
+//    LDS; dV^T += dA^T P or dK^T += Q^T dS (PART) through transposing reads of
+//    the same two LDS tiles.
 //
 // K, V, Q, dA steps go from global memory straight into LDS, double buffered;
 // 16-byte chunk c of row r of a step sits at chunk position
@@ -239,9 +238,43 @@ __device__ __forceinline__ StepSet make_step_set(const BwdParams &p, bool explic
 }
 
 // ---------------------------------------------------------------------------------
+// D[b][q] = dA[b][q][:] . A[b][q][:] in fp32, for the workgroups below: 16-byte
+// loads, HEAD/8 lanes a row, summed across those lanes.
+template<typename T, int HEAD>
+__global__ __launch_bounds__(256)
+void sdpa_bwd_rowdot_kernel(const void *dA, const void *A, float *D, int64_t rows)
+{
+    constexpr int LANES = HEAD / 8;             // lanes per row: 16, 8 or 4
+    const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LANES;
+    const int part = (int)(threadIdx.x % LANES);
+    float d = 0.0f;
+    if(row < rows)
+    {
+        const u32x4 g = *reinterpret_cast<const u32x4 *>(
+                static_cast<const uint16_t *>(dA) + row * HEAD + part * 8);
+        const u32x4 a = *reinterpret_cast<const u32x4 *>(
+                static_cast<const uint16_t *>(A) + row * HEAD + part * 8);
+#pragma unroll
+        for(int e = 0; e < 4; ++e)
+        {
+            d += T::to_float((uint16_t)(g[e] & 0xffffu)) * T::to_float((uint16_t)(a[e] & 0xffffu));
+            d += T::to_float((uint16_t)(g[e] >> 16)) * T::to_float((uint16_t)(a[e] >> 16));
+        }
+    }
+#pragma unroll
+    for(int o = LANES / 2; o >= 1; o >>= 1)
+    {
+        d += __shfl_xor(d, o, 64);
+    }
+    if(row < rows && part == 0)
+    {
+        D[row] = d;
+    }
+}
+
 template<typename T, int HEAD, int MODE>
-__global__ __launch_bounds__(kBwdThreads, 2)
-void sdpa_bwd_dq_kernel(const BwdParams p)
+__device__ __forceinline__ void sdpa_bwd_dq_body(const BwdParams &p, unsigned wg,
+        char *lds_k0, char *lds_k1, char *lds_v0, char *lds_v1)
 {
     typedef typename T::vec8 vec8;
     typedef BwdTile<HEAD> G;
@@ -249,11 +282,6 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
     constexpr int LOADS_PER_WAVE = G::LOADS_PER_WAVE, ROWS_PER_LOAD = G::ROWS_PER_LOAD;
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
-
-    __shared__ __attribute__((aligned(1024))) char lds_k0[G::BYTES];
-    __shared__ __attribute__((aligned(1024))) char lds_k1[G::BYTES];
-    __shared__ __attribute__((aligned(1024))) char lds_v0[G::BYTES];
-    __shared__ __attribute__((aligned(1024))) char lds_v1[G::BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -265,7 +293,7 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
     const int q_blocks = (int)((p.q_seq + kBwdRows - 1) / kBwdRows);
     // the last query blocks see the most keys under a causal mask: first
     int b, q_block;
-    map_workgroup(blockIdx.x, p.batch, q_blocks, true, b, q_block);
+    map_workgroup(wg, p.batch, q_blocks, true, b, q_block);
     const int q_row0 = q_block * kBwdRows;
     const int kvb = kv_entry(b, p.n_batch, p.kv_group);
     const int q_seq = (int)p.q_seq, k_seq = (int)p.k_seq;
@@ -273,43 +301,29 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
     const bool q_ok = my_q < q_seq;
     const int64_t q_off = ((int64_t)b * q_seq + (q_ok ? my_q : 0)) * HEAD;
 
-    // Q and dA fragments (B operands) and the row dot D = dA . A
+    // Q and dA fragments (B operands); the row dot D = dA . A of the query
     vec8 qf[KSTEPS], gf[KSTEPS];
-    float d_row = 0.0f;
     {
         const uint16_t *qs = static_cast<const uint16_t *>(p.Q) + q_off + half * 8;
         const uint16_t *gs = static_cast<const uint16_t *>(p.dA) + q_off + half * 8;
-        const uint16_t *as = static_cast<const uint16_t *>(p.A) + q_off + half * 8;
 #pragma unroll
         for(int ks = 0; ks < KSTEPS; ++ks)
         {
             u32x4 q = *reinterpret_cast<const u32x4 *>(qs + ks * 16);
             u32x4 g = *reinterpret_cast<const u32x4 *>(gs + ks * 16);
-            u32x4 a = *reinterpret_cast<const u32x4 *>(as + ks * 16);
             if(!q_ok)
             {
                 q = u32x4{0, 0, 0, 0};
                 g = u32x4{0, 0, 0, 0};
-                a = u32x4{0, 0, 0, 0};
             }
             qf[ks] = __builtin_bit_cast(vec8, q);
             gf[ks] = __builtin_bit_cast(vec8, g);
-#pragma unroll
-            for(int e = 0; e < 4; ++e)
-            {
-                d_row += T::to_float((uint16_t)(g[e] & 0xffffu)) * T::to_float((uint16_t)(a[e] & 0xffffu));
-                d_row += T::to_float((uint16_t)(g[e] >> 16)) * T::to_float((uint16_t)(a[e] >> 16));
-            }
         }
     }
-    d_row = sum_across_halves(d_row);
+    const float d_row = q_ok ? p.D[(int64_t)b * q_seq + my_q] : 0.0f;
     const float lse_q = q_ok ? p.lse[(int64_t)b * q_seq + my_q] : neg_inf();
     // exponent offset in log2 units; a row that saw nothing has P = 0
     const float lse2 = (lse_q == neg_inf()) ? __builtin_huge_valf() : lse_q * kLog2e;
-    if(p.D != nullptr && q_ok && half == 0)
-    {
-        p.D[(int64_t)b * q_seq + my_q] = d_row;
-    }
 
     // ---- which keys ---------------------------------------------------------------
     // key row kg is visible to query row q iff kg <= rel + q (causal)
@@ -326,26 +340,21 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
 
     // ---- LDS addresses --------------------------------------------------------------
     uint32_t ld_goff[LOADS_PER_WAVE];
-    int ld_row[LOADS_PER_WAVE];
     const int ld_cpos = lane % CPR;
+    const int ld_row0 = wave * LOADS_PER_WAVE * ROWS_PER_LOAD + lane / CPR;   // + i * ROWS_PER_LOAD
 #pragma unroll
     for(int i = 0; i < LOADS_PER_WAVE; ++i)
     {
-        const int r = (wave * LOADS_PER_WAVE + i) * ROWS_PER_LOAD + lane / CPR;
-        ld_row[i] = r;
+        const int r = ld_row0 + i * ROWS_PER_LOAD;
         ld_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ G::swz(r)) * 16);
     }
-    // row operand: lane (col, half) reads row mb*32+col, logical chunk 2*ks+half
-    uint32_t row_raddr[2][KSTEPS];
+    // row operand: lane (col, half) reads row mb*32+col, logical chunk 2*ks+half;
+    // 32 rows further on the swizzle is the same, so mb goes into the immediate
+    uint32_t row_raddr[KSTEPS];
 #pragma unroll
-    for(int mb = 0; mb < 2; ++mb)
+    for(int ks = 0; ks < KSTEPS; ++ks)
     {
-        const int r = mb * 32 + col;
-#pragma unroll
-        for(int ks = 0; ks < KSTEPS; ++ks)
-        {
-            row_raddr[mb][ks] = (uint32_t)(r * RB + ((2 * ks + half) ^ G::swz(r)) * 16);
-        }
+        row_raddr[ks] = (uint32_t)(col * RB + ((2 * ks + half) ^ G::swz(col)) * 16);
     }
     // transposed operand: within a 16-lane block lane i addresses row j = i/4 and
     // head values 4*(i%4)..+3 of the block's 16; lanes 16..31 take the upper 16
@@ -383,7 +392,7 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
         const int last = min(kBwdStep, k_seq - row0) - 1;
         char *kdst = kdst_base + wave_u * LOADS_PER_WAVE * 1024;
         char *vdst = vdst_base + wave_u * LOADS_PER_WAVE * 1024;
-        const uint32_t back = (uint32_t)(max(ld_row[i] - last, 0) * RB);
+        const uint32_t back = (uint32_t)(max(ld_row0 + i * ROWS_PER_LOAD - last, 0) * RB);
         load_to_lds16<0, false>(Kb + (int64_t)row0 * RB, ld_goff[i] - back, kdst + i * 1024);
         load_to_lds16<0, false>(Vb + (int64_t)row0 * RB, ld_goff[i] - back, vdst + i * 1024);
     };
@@ -452,7 +461,6 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
         // ---- S^T = K Q^T, dP^T = V dA^T -------------------------------------------------
         // (one 32-key block at a time: half the accumulators live)
         // ---- P^T, dS^T: register r of block mb is key mb*32 + tile_row(r, half) ------------
-        uint32_t ds_pk[2][8];
         int lim = keys_here - 1;
         if(MODE == NNTILE_HIP_MASK_CAUSAL)
         {
@@ -471,8 +479,8 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
 #pragma unroll
             for(int ks = 0; ks < KSTEPS; ++ks)
             {
-                const vec8 ka = *reinterpret_cast<const vec8 *>(Ks + row_raddr[mb][ks]);
-                const vec8 va = *reinterpret_cast<const vec8 *>(Vs + row_raddr[mb][ks]);
+                const vec8 ka = *reinterpret_cast<const vec8 *>(Ks + row_raddr[ks] + mb * 32 * RB);
+                const vec8 va = *reinterpret_cast<const vec8 *>(Vs + row_raddr[ks] + mb * 32 * RB);
                 sv = T::mfma(ka, qf[ks], sv);
                 dpv = T::mfma(va, gf[ks], dpv);
 #pragma unroll
@@ -513,28 +521,28 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
                 const float pr = visible ? fast_exp2(e) : 0.0f;
                 dsv[r] = pr * (dpv[r] - d_row);
             }
+            uint32_t ds_pk[8];
 #pragma unroll
             for(int k = 0; k < 8; ++k)
             {
-                ds_pk[mb][k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
+                ds_pk[k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
             }
-        }
-
-        // ---- dQ^T += K^T dS^T: four sub-steps of 16 keys --------------------------------
+            // ---- dQ^T += K^T dS^T: the block's two sub-steps of 16 keys ------------------
 #pragma unroll
-        for(int t = 0; t < 4; ++t)
-        {
-            const int mb = t >> 1, tt = t & 1;
-            const u32x4 braw = {ds_pk[mb][4 * tt], ds_pk[mb][4 * tt + 1],
-                ds_pk[mb][4 * tt + 2], ds_pk[mb][4 * tt + 3]};
-            const vec8 bop = __builtin_bit_cast(vec8, braw);
-#pragma unroll
-            for(int db = 0; db < DBLOCKS; ++db)
+            for(int tt = 0; tt < 2; ++tt)
             {
-                const u32x2 lo = bwd_lds_read_tr16(Ks + tr_raddr[0][db] + (16 * t) * RB);
-                const u32x2 hi = bwd_lds_read_tr16(Ks + tr_raddr[1][db] + (16 * t) * RB);
-                const u32x4 araw = {lo[0], lo[1], hi[0], hi[1]};
-                acc[db] = T::mfma(__builtin_bit_cast(vec8, araw), bop, acc[db]);
+                const int t = 2 * mb + tt;
+                const u32x4 braw = {ds_pk[4 * tt], ds_pk[4 * tt + 1], ds_pk[4 * tt + 2],
+                    ds_pk[4 * tt + 3]};
+                const vec8 bop = __builtin_bit_cast(vec8, braw);
+#pragma unroll
+                for(int db = 0; db < DBLOCKS; ++db)
+                {
+                    const u32x2 lo = bwd_lds_read_tr16(Ks + tr_raddr[0][db] + (16 * t) * RB);
+                    const u32x2 hi = bwd_lds_read_tr16(Ks + tr_raddr[1][db] + (16 * t) * RB);
+                    const u32x4 araw = {lo[0], lo[1], hi[0], hi[1]};
+                    acc[db] = T::mfma(__builtin_bit_cast(vec8, araw), bop, acc[db]);
+                }
             }
         }
     };
@@ -606,16 +614,17 @@ void sdpa_bwd_dq_kernel(const BwdParams p)
 // PART says which gradient: K and V fragments plus both accumulators take 192
 // registers of a lane at head 128, which leaves too few for two wavefronts
 // per SIMD to run without spilling and without room to read operands ahead.
-// One launch per gradient (dK: S, dP, dK^T; dV: S, dV^T - the scores are
-// computed once more) fits two workgroups of 4 wavefronts on a CU each.
+// One set of workgroups per gradient (dK: S, dP, dK^T; dV: S, dV^T - the
+// scores are computed once more) fits two workgroups of 4 wavefronts on a CU.
 enum { BWD_PART_DK = 1, BWD_PART_DV = 2 };
 constexpr int kDkvWaves = 4;
 constexpr int kDkvThreads = kDkvWaves * 64;
 constexpr int kDkvRows = kDkvWaves * 32;        // keys per workgroup
 
 template<typename T, int HEAD, int MODE, int PART>
-__global__ __launch_bounds__(kDkvThreads, 2)
-void sdpa_bwd_dkv_kernel(const BwdParams p)
+__device__ __forceinline__ void sdpa_bwd_dkv_body(const BwdParams &p, unsigned wg,
+        char *lds_q0, char *lds_q1, char *lds_g0, char *lds_g1,
+        float (*lds_stat)[2][kBwdStep])
 {
     constexpr bool DO_DK = PART == BWD_PART_DK, DO_DV = PART == BWD_PART_DV;
     typedef typename T::vec8 vec8;
@@ -626,14 +635,6 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
     constexpr int LOADERS = G::LOADS / LPW;                                  // wavefronts that load
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
-
-    __shared__ __attribute__((aligned(1024))) char lds_q0[G::BYTES];
-    __shared__ __attribute__((aligned(1024))) char lds_q1[G::BYTES];
-    __shared__ __attribute__((aligned(1024))) char lds_g0[G::BYTES];
-    __shared__ __attribute__((aligned(1024))) char lds_g1[G::BYTES];
-    // per query of a step: logsumexp in log2 units (+inf for a row that saw
-    // nothing) and the row dot D; rows past the end hold +inf / 0
-    __shared__ __attribute__((aligned(16))) float lds_stat[2][2][kBwdStep];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -646,7 +647,7 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
     const int k_blocks = (k_seq + kDkvRows - 1) / kDkvRows;
     // the first key blocks are seen by the most queries under a causal mask
     int kvb, k_block;                               // kvb = nb + n_batch*hkv
-    map_workgroup(blockIdx.x, p.batch / p.kv_group, k_blocks, false, kvb, k_block);
+    map_workgroup(wg, p.batch / p.kv_group, k_blocks, false, kvb, k_block);
     const int k_row0 = k_block * kDkvRows;
     const int nb = kvb % p.n_batch, hkv = kvb / p.n_batch;
     const int my_k = k_row0 + wave * 32 + col;
@@ -811,7 +812,7 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
         locate(i, bq, qs);
         const int row0 = qs * kBwdStep;
         const int last = min(kBwdStep, q_seq - row0) - 1;
-        if(wave_u < LOADERS)
+        if(LOADERS == kDkvWaves || wave_u < LOADERS)
         {
 #pragma unroll
             for(int j = 0; j < LPW; ++j)
@@ -846,7 +847,7 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
         if(i_next >= 0)
         {
             fetch_stat(bq_f, row0_f, last_f, lds_stat[BUF ^ 1]);
-            if(NNTILE_BWD_SPREAD == 0 && wave_u < LOADERS)
+            if(NNTILE_BWD_SPREAD == 0 && (LOADERS == kDkvWaves || wave_u < LOADERS))
             {
 #pragma unroll
                 for(int j = 0; j < LPW; ++j)
@@ -890,7 +891,7 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
                             + mb * 32 * RB);
                     dpv = T::mfma(ga, vf[ks], dpv);
                 }
-                if(wave_u < LOADERS)
+                if(LOADERS == kDkvWaves || wave_u < LOADERS)
                 {
 #pragma unroll
                     for(int j = 0; j < LPW; ++j)
@@ -1062,6 +1063,40 @@ void sdpa_bwd_dkv_kernel(const BwdParams p)
     }
 }
 
+// One launch for the three gradients: workgroups [0, n_dkv) compute dK,
+// the next n_dq dQ (three products a step each, the longer workgroups), the
+// last n_dkv dV.  A tile-pair call has fewer workgroups per gradient than the
+// chip has places (two a CU); together they fill it, and a long call loses
+// the ends of two launches.
+template<typename T, int HEAD, int MODE>
+__global__ __launch_bounds__(kDkvThreads, 2)
+void sdpa_bwd_kernel(const BwdParams p, unsigned n_dkv, unsigned n_dq)
+{
+    typedef BwdTile<HEAD> G;
+    static_assert(kDkvThreads == kBwdThreads, "one block size for the three parts");
+    __shared__ __attribute__((aligned(1024))) char lds_0[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_1[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_2[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_3[G::BYTES];
+    // dK, dV parts, per query of a step: logsumexp in log2 units (+inf for a
+    // row that saw nothing) and the row dot D; rows past the end hold +inf / 0
+    __shared__ __attribute__((aligned(16))) float lds_stat[2][2][kBwdStep];
+    if(blockIdx.x < n_dkv)
+    {
+        sdpa_bwd_dkv_body<T, HEAD, MODE, BWD_PART_DK>(p, blockIdx.x, lds_0, lds_1, lds_2,
+                lds_3, lds_stat);
+    }
+    else if(blockIdx.x < n_dkv + n_dq)
+    {
+        sdpa_bwd_dq_body<T, HEAD, MODE>(p, blockIdx.x - n_dkv, lds_0, lds_1, lds_2, lds_3);
+    }
+    else
+    {
+        sdpa_bwd_dkv_body<T, HEAD, MODE, BWD_PART_DV>(p, blockIdx.x - n_dkv - n_dq, lds_0,
+                lds_1, lds_2, lds_3, lds_stat);
+    }
+}
+
 template<typename T, int HEAD, int MODE>
 static int launch_bwd_mode(hipStream_t stream, const BwdParams &p)
 {
@@ -1069,7 +1104,8 @@ static int launch_bwd_mode(hipStream_t stream, const BwdParams &p)
     const int64_t k_blocks = (p.k_seq + kDkvRows - 1) / kDkvRows;
     const int64_t kv_batch = p.batch / p.kv_group;
     const int64_t n_dq = (int64_t)p.batch * q_blocks, n_dkv = kv_batch * k_blocks;
-    if(n_dq <= 0 || n_dkv <= 0 || n_dq > 0x7fffffff || n_dkv > 0x7fffffff)
+    if(n_dq <= 0 || n_dkv <= 0 || n_dq > 0x3fffffff || n_dkv > 0x3fffffff
+            || (int64_t)p.batch * p.q_seq * (HEAD / 8) / 256 > 0x7ffffffe)
     {
         return NNTILE_HIP_EINVAL;
     }
@@ -1085,20 +1121,17 @@ static int launch_bwd_mode(hipStream_t stream, const BwdParams &p)
             return NNTILE_HIP_ELAUNCH;
         }
     }
-    hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, HEAD, MODE>), dim3((unsigned)n_dq),
-            dim3(kBwdThreads), 0, stream, p);
+    const int64_t rows = (int64_t)p.batch * p.q_seq;
+    hipLaunchKernelGGL((sdpa_bwd_rowdot_kernel<T, HEAD>),
+            dim3((unsigned)((rows * (HEAD / 8) + 255) / 256)), dim3(256), 0, stream, p.dA, p.A,
+            p.D, rows);
     if(hipGetLastError() != hipSuccess)
     {
         return NNTILE_HIP_ELAUNCH;
     }
-    hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, HEAD, MODE, BWD_PART_DV>),
-            dim3((unsigned)n_dkv), dim3(kDkvThreads), 0, stream, p);
-    if(hipGetLastError() != hipSuccess)
-    {
-        return NNTILE_HIP_ELAUNCH;
-    }
-    hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, HEAD, MODE, BWD_PART_DK>),
-            dim3((unsigned)n_dkv), dim3(kDkvThreads), 0, stream, p);
+    hipLaunchKernelGGL((sdpa_bwd_kernel<T, HEAD, MODE>),
+            dim3((unsigned)(2 * n_dkv + n_dq)), dim3(kDkvThreads), 0, stream, p,
+            (unsigned)n_dkv, (unsigned)n_dq);
     return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
 }
 
