@@ -194,6 +194,38 @@ def bench_backward(cfg, steps, warmup):
                     "mask, gradients written" % cfg.name}
 
 
+def bench_rope(cfg, steps, warmup):
+    """Rotary embedding of the Q tensor of the workload (the step before the
+    attention kernel): sin, cos of shape [head/2, seq], src and dst
+    [head, seq, heads].  HBM-bound: reads src, writes dst; sin and cos are
+    re-read from cache.  Eight buffer pairs rotate so that the 256 MiB
+    last-level cache cannot serve a pass."""
+    import torch
+    from nntile_amd import hip_sdpa as h
+    dt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg.dtype]
+    half = cfg.head // 2
+    ang = torch.rand(cfg.q_seq, half, device="cuda") * 6.28
+    sin, cos = torch.sin(ang).to(dt).contiguous(), torch.cos(ang).to(dt).contiguous()
+    nrot = 8
+    src = [_randn((cfg.batch_flat, cfg.q_seq, cfg.head), dt, cfg.seed * 1000 + 800 + i) for i in range(nrot)]
+    dst = [torch.empty_like(x) for x in src]
+    i = [0]
+
+    def step():
+        j = i[0] % nrot
+        h.rope(sin, cos, src[j], dst[j])
+        i[0] += 1
+
+    wall, dev = time_steps(step, steps, warmup)
+    nbytes = 2 * src[0].numel() * src[0].element_size() + 2 * sin.numel() * sin.element_size()
+    return {"what": "rotary embedding of the Q tensor of %s (%d MiB in, %d MiB out)"
+                    % (cfg.name, src[0].numel() * src[0].element_size() >> 20,
+                       src[0].numel() * src[0].element_size() >> 20),
+            "device_ms_per_step": round(dev, 4), "algorithmic_bytes": nbytes,
+            "gbs": round(nbytes / (dev * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(nbytes / (dev * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+
+
 def cpu_baseline(cfg, target_seconds=15.0):
     """The CPU checker (port of the reference's gemm -> mask_scalar ->
     maxsumexp -> softmax_inplace -> gemm composition) on a bounded sample of
@@ -232,7 +264,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run only this leg: prefill | decode | per_task | backward | extras | copy (for profiling)")
+                    help="run only this leg: prefill | decode | per_task | backward | rope | extras | copy (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
@@ -272,6 +304,9 @@ def main():
     if only == "backward":
         print(json.dumps(bench_backward(cfg3, args.steps, args.warmup)))
         return
+    if only == "rope":
+        print(json.dumps(bench_rope(cfg3, args.steps, args.warmup)))
+        return
     if only == "extras":
         for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):
             bench_prefill(BY_NAME[name], args.steps, args.warmup)
@@ -291,6 +326,7 @@ def main():
                         "peak_tflops": peak, "flops_causal_exact": c.flops(),
                         "launches_per_step": r["launches_per_step"]}
     backward = bench_backward(cfg3, max(5, args.steps // 10), 2)
+    rope = bench_rope(cfg3, max(5, args.steps // 5), 5)
     # The headline leg runs last: the first timed loop of a process measures
     # 5 % slower than the same loop a second later (clocks still settling),
     # whatever the warmup count.
@@ -337,6 +373,7 @@ def main():
                           "tflops": round(per_task["tflops"], 2)},
         "other_configs": extras,
         "backward": backward,
+        "rope": rope,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg3)

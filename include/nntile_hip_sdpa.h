@@ -269,6 +269,30 @@ void nntile_hip_flash_sdpa_fwd_codelet_fp32(void *buffers[], void *cl_args);
 void nntile_hip_flash_sdpa_bwd_codelet_bf16(void *buffers[], void *cl_args);
 void nntile_hip_flash_sdpa_bwd_codelet_fp16(void *buffers[], void *cl_args);
 
+/* ---- 7. The step before the attention kernel: rotary position embedding ----
+ * Replace kernel::rope::cuda<T> (include/nntile/kernel/rope/cuda.hh:24-27,
+ * src/kernel/rope/cuda.cu:22-55) and kernel::rope_backward::cuda<T>
+ * (include/nntile/kernel/rope_backward/cuda.hh:24-27,
+ * src/kernel/rope_backward/cuda.cu): same argument order and meaning.  src
+ * and dst are (2, m, n) in memory order, sin and cos hold m values each:
+ *   dst[2i,j]   = cos[i] src[2i,j] - sin[i] src[2i+1,j]
+ *   dst[2i+1,j] = sin[i] src[2i,j] + cos[i] src[2i+1,j]
+ * and the backward is the transposed rotation, written (not added) to dx.
+ * Arithmetic in fp32, one rounding to the tile type.  m == 0 or n == 0 is a
+ * no-op; src and dst may be the same buffer. */
+int nntile_hip_rope_bf16(void *stream, int64_t m, int64_t n, const uint16_t *sin,
+        const uint16_t *cos, const uint16_t *src, uint16_t *dst);
+int nntile_hip_rope_fp16(void *stream, int64_t m, int64_t n, const uint16_t *sin,
+        const uint16_t *cos, const uint16_t *src, uint16_t *dst);
+int nntile_hip_rope_fp32(void *stream, int64_t m, int64_t n, const float *sin,
+        const float *cos, const float *src, float *dst);
+int nntile_hip_rope_backward_bf16(void *stream, int64_t m, int64_t n, const uint16_t *sin,
+        const uint16_t *cos, const uint16_t *dy, uint16_t *dx);
+int nntile_hip_rope_backward_fp16(void *stream, int64_t m, int64_t n, const uint16_t *sin,
+        const uint16_t *cos, const uint16_t *dy, uint16_t *dx);
+int nntile_hip_rope_backward_fp32(void *stream, int64_t m, int64_t n, const float *sin,
+        const float *cos, const float *dy, float *dx);
+
 /* Library version and the ISA it was built for ("gfx950"). */
 const char *nntile_hip_sdpa_version(void);
 

@@ -26,6 +26,9 @@ int launch_accumulate(hipStream_t stream, int64_t head, int64_t seq,
         int64_t batch, const float *src_lse, const void *src_attn,
         float *dst_lse, void *dst_attn);
 
+int launch_rope(hipStream_t stream, int dtype, bool backward, int64_t m, int64_t n,
+        const void *sin, const void *cos, const void *src, void *dst);
+
 enum class DType { bf16, fp16, fp32 };
 
 static bool aligned16(const void *p)
@@ -389,6 +392,27 @@ static int accumulate_call(void *stream, int64_t head, int64_t seq,
             batch, src_lse, src_attn, dst_lse, dst_attn);
 }
 
+static int rope_call(DType dt, bool backward, void *stream, int64_t m, int64_t n,
+        const void *sin, const void *cos, const void *src, void *dst)
+{
+    if(m < 0 || n < 0)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(m == 0 || n == 0)
+    {
+        return NNTILE_HIP_OK;   // nothing to rotate (the reference launches an empty grid)
+    }
+    if(sin == nullptr || cos == nullptr || src == nullptr || dst == nullptr
+            || m > (int64_t)0x3fffffffffffffff / n)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    const int code = dt == DType::bf16 ? 0 : (dt == DType::fp16 ? 1 : 2);
+    return launch_rope(static_cast<hipStream_t>(stream), code, backward, m, n, sin, cos, src,
+            dst);
+}
+
 static nntile_hip_stream_provider g_stream_provider = nullptr;
 
 static void codelet_call(DType dt, const char *name, void *buffers[],
@@ -649,6 +673,22 @@ void nntile_hip_flash_sdpa_bwd_codelet_fp16(void *buffers[], void *cl_args)
 {
     bwd_codelet_call(DType::fp16, "nntile_flash_sdpa_bwd_hip_fp16", buffers, cl_args);
 }
+
+#define NNTILE_HIP_ROPE_ENTRY(suffix, dt, ctype) \
+    int nntile_hip_rope_##suffix(void *stream, int64_t m, int64_t n, const ctype *sin, \
+            const ctype *cos, const ctype *src, ctype *dst) \
+    { \
+        return rope_call(dt, false, stream, m, n, sin, cos, src, dst); \
+    } \
+    int nntile_hip_rope_backward_##suffix(void *stream, int64_t m, int64_t n, const ctype *sin, \
+            const ctype *cos, const ctype *dy, ctype *dx) \
+    { \
+        return rope_call(dt, true, stream, m, n, sin, cos, dy, dx); \
+    }
+NNTILE_HIP_ROPE_ENTRY(bf16, DType::bf16, uint16_t)
+NNTILE_HIP_ROPE_ENTRY(fp16, DType::fp16, uint16_t)
+NNTILE_HIP_ROPE_ENTRY(fp32, DType::fp32, float)
+#undef NNTILE_HIP_ROPE_ENTRY
 
 const char *nntile_hip_sdpa_version(void)
 {

@@ -84,6 +84,8 @@ EXPORTS = (
     + ["nntile_hip_flash_sdpa_bwd_codelet_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_accumulate_attn_output_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_flash_sdpa_fwd_codelet_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_rope_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_rope_backward_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_set_stream_provider", "nntile_hip_sdpa_version"])
 
 _lib = None
@@ -126,6 +128,11 @@ def lib():
             f = getattr(L, "nntile_hip_sdpa_bwd_tile_" + t)
             f.argtypes = [_vp, ctypes.POINTER(BwdArgs)]
             f.restype = ctypes.c_int
+        for t in ("bf16", "fp16", "fp32"):
+            for name in ("nntile_hip_rope_", "nntile_hip_rope_backward_"):
+                f = getattr(L, name + t)
+                f.argtypes = [_vp, _i64, _i64, _vp, _vp, _vp, _vp]
+                f.restype = ctypes.c_int
         L.nntile_hip_sdpa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
         L.nntile_hip_sdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.argtypes = [ctypes.POINTER(TileArgs)]
@@ -370,6 +377,19 @@ def accumulate_attn_output(src_lse, src_attn, dst_lse, dst_attn, stream=None):
     fn = getattr(lib(), "nntile_hip_accumulate_attn_output_" + dtype_name(dst_attn))
     _check(fn(_stream(stream), head, seq, batch, _ptr(src_lse), _ptr(src_attn),
               _ptr(dst_lse), _ptr(dst_attn)), "accumulate_attn_output")
+
+
+def rope(sin, cos, src, dst, backward=False, stream=None):
+    """Rotary embedding of src (memory order (2, m, n), m = sin.numel()) into
+    dst; backward=True applies the transposed rotation (dy -> dx)."""
+    _dev(sin, cos, src, dst)
+    m = sin.numel()
+    if cos.numel() != m or src.numel() != dst.numel() or (m and src.numel() % (2 * m)):
+        raise SdpaError(EINVAL, "rope")
+    n = src.numel() // (2 * m) if m else 0
+    name = "nntile_hip_rope_backward_" if backward else "nntile_hip_rope_"
+    fn = getattr(lib(), name + dtype_name(src))
+    _check(fn(_stream(stream), m, n, _ptr(sin), _ptr(cos), _ptr(src), _ptr(dst)), "rope")
 
 
 def flash_sdpa_fwd_codelet(K, Q, mask, lse, V, A, scratch_lse=None, scratch_A=None,

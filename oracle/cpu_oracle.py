@@ -288,3 +288,32 @@ def sdpa_bwd_flash_f64(K, Q, V, A, dA, lse, add_mask=None, kv_repeat=1, n_batch=
         dQ[b] = scale * (ds @ K[kv])
         dK[kv] += scale * (ds.T @ Q[b])
     return dK, dQ, dV
+
+
+def rope(sin, cos, src, backward=False):
+    """Rotary embedding of a (2, m, n) tensor (memory order: the pair fastest,
+    then the m positions of sin / cos, then n), in fp32 as the reference's
+    repr_t (src/kernel/rope/cpu.cc:22-52):
+
+        dst[2i,j]   = cos[i] src[2i,j] - sin[i] src[2i+1,j]
+        dst[2i+1,j] = sin[i] src[2i,j] + cos[i] src[2i+1,j]
+
+    backward=True is src/kernel/rope_backward/cpu.cc:22-53 (dy -> dx, written,
+    not added): dx[2i] = c dy[2i] + s dy[2i+1], dx[2i+1] = c dy[2i+1] - s dy[2i].
+    Returns a float32 array of src's shape (not yet rounded to the tile type)."""
+    s = np.asarray(sin, np.float32).ravel()
+    c = np.asarray(cos, np.float32).ravel()
+    x = np.asarray(src, np.float32)
+    m = s.size
+    if m == 0 or x.size == 0:
+        return np.zeros(x.shape, np.float32)
+    v = x.reshape(-1, m, 2)
+    a, b = v[..., 0], v[..., 1]
+    out = np.empty_like(v)
+    if backward:
+        out[..., 0] = c * a + s * b
+        out[..., 1] = c * b - s * a
+    else:
+        out[..., 0] = c * a - s * b
+        out[..., 1] = s * a + c * b
+    return out.reshape(x.shape)
