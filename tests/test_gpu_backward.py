@@ -274,3 +274,55 @@ def test_mask_block_classes(oracle, dtype, form, q_seq, k_seq, pattern, room):
             assert np.all(g == 0), name
         else:
             assert np.linalg.norm(g - w) / np.linalg.norm(w) < BWD_TOL[dtype], name
+
+
+def test_full_size_llama_prefill_shape(oracle):
+    """The backward at the benchmark's shape (head 128, 32 heads, seq 4096,
+    causal, bf16) in one call.  Three heads against the fp64 checker; every
+    head through two properties that hold exactly in floating point: twice
+    the incoming gradient gives twice every gradient bit for bit (a power of
+    two scales D, dP and dS exactly), and the sequence cut into four key
+    tiles whose dQ accumulate in fp32-rounded-to-bf16 steps stays within the
+    tolerance of the one-call result."""
+    print("case bwd full size", flush=True)
+    batch, seq, head, dtype = 32, 4096, 128, "bf16"
+    dt = torch.bfloat16
+    g = torch.Generator(device="cuda").manual_seed(1234)
+    Q, K, V, G = (torch.randn((batch, seq, head), generator=g, device="cuda", dtype=torch.float32).to(dt)
+                  for _ in range(4))
+    A = torch.zeros_like(Q)
+    lse = torch.full((batch, seq), float("-inf"), device="cuda")
+    hip_sdpa.sdpa_fwd_tile(K, Q, None, lse, V, A, hip_sdpa.MASK_CAUSAL, flags=hip_sdpa.OVERWRITE)
+    grads = [torch.full_like(Q, float("nan")) for _ in range(3)]
+    hip_sdpa.sdpa_bwd_tile(K, Q, V, A, G, None, lse, *grads, hip_sdpa.MASK_CAUSAL,
+                           flags=hip_sdpa.OVERWRITE)
+    torch.cuda.synchronize()
+    for t in grads:
+        assert bool(torch.isfinite(t.float()).all())
+    mask = synth.causal_mask(seq, seq)
+    add = np.where(mask, 0, -np.inf).astype(np.float32)
+    for b in (0, 17, 31):
+        sl = slice(b, b + 1)
+        want = oracle.sdpa_bwd_flash_f64(H.to_np(K[sl]), H.to_np(Q[sl]), H.to_np(V[sl]),
+                                         H.to_np(A[sl]), H.to_np(G[sl]), H.to_np(lse[sl]), add)
+        for got, w, name in zip(grads, want, ("dK", "dQ", "dV")):
+            _check(got[sl], w, dtype, "%s head %d" % (name, b))
+    twice = [torch.full_like(Q, float("nan")) for _ in range(3)]
+    hip_sdpa.sdpa_bwd_tile(K, Q, V, A, (G.float() * 2).to(dt), None, lse, *twice,
+                           hip_sdpa.MASK_CAUSAL, flags=hip_sdpa.OVERWRITE)
+    torch.cuda.synchronize()
+    for one, two, name in zip(grads, twice, ("dK", "dQ", "dV")):
+        assert torch.equal((one.float() * 2).to(dt).view(torch.int16), two.view(torch.int16)), name
+    tiled = [torch.zeros_like(Q) for _ in range(3)]
+    tile = 1024
+    for s in range(0, seq, tile):
+        Kt, Vt = K[:, s:s + tile].contiguous(), V[:, s:s + tile].contiguous()
+        dKt, dVt = torch.zeros_like(Kt), torch.zeros_like(Vt)
+        hip_sdpa.sdpa_bwd_tile(Kt, Q, Vt, A, G, None, lse, dKt, tiled[1], dVt, hip_sdpa.MASK_CAUSAL,
+                               k_pos0=s)
+        tiled[0][:, s:s + tile] = dKt
+        tiled[2][:, s:s + tile] = dVt
+    torch.cuda.synchronize()
+    for one, t, name in zip(grads, tiled, ("dK", "dQ", "dV")):
+        a, b = one.float(), t.float()
+        assert float((a - b).norm() / a.norm()) < BWD_TOL[dtype], name
