@@ -17,6 +17,7 @@ int decode_choose_splits(int units, int n_steps);
 template<typename T>
 int launch_bwd_16bit(hipStream_t stream, const BwdParams &p, int head, int mode);
 size_t decode_workspace_bytes(int units, int n_splits, int rows, int head);
+size_t decode_partial_o_bytes(int units, int n_splits, int rows, int head);
 
 struct F32Store;
 struct Bf16Store;
@@ -359,7 +360,8 @@ static int decode_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *
     p.lse = a->lse;
     p.A = a->A;
     p.part_o = static_cast<float *>(workspace);
-    p.part_ml = p.part_o + (size_t)units * splits * rows * a->head;
+    p.part_ml = reinterpret_cast<float *>(static_cast<char *>(workspace)
+            + decode_partial_o_bytes(units, splits, rows, (int)a->head));
     p.n_batch = (int32_t)a->n_batch;
     p.kv_group = (int32_t)a->kv_group;
     p.n_head_kv = (int32_t)(units / a->n_batch);

@@ -69,7 +69,7 @@ struct DecodeParams
     const void *K, *V, *Q;
     float *lse;
     void *A;
-    float *part_o;      // [unit][split][rows][HEAD]
+    float *part_o;      // [unit][split][rows][HEAD], fp32 or (normalised) in the tile type
     float *part_ml;     // [unit][split][rows][2]
     int32_t n_batch, kv_group, n_head_kv;
     int32_t rows;       // kv_group * q_seq

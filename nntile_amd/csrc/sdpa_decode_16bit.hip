@@ -32,6 +32,11 @@ namespace nntile_hip
 constexpr int kDecThreads = 256;  // 4 wavefronts x 16 query rows
 constexpr int kDecodeCUs = 256;   // MI355X
 
+// Partial outputs of the key splits: 1 = normalised and in the tile type,
+// 0 = unnormalised fp32
+#ifndef NNTILE_DEC_PART16
+#define NNTILE_DEC_PART16 1
+#endif
 typedef __attribute__((ext_vector_type(4))) float acc4;
 
 template<typename T> struct Mfma16;
@@ -453,12 +458,27 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         p.part_ml[2 * prow + 1] = l_tot;
     }
     // o[db][r] is head value 16*db + 4*quad + r of row rr
+#if NNTILE_DEC_PART16
+    // the partial output, normalised, in the tile type: half the bytes of
+    // fp32 partials (one more rounding, as the reference's scratch tile has)
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    uint16_t *dst = reinterpret_cast<uint16_t *>(p.part_o) + prow * HEAD + 4 * quad;
+#pragma unroll
+    for(int db = 0; db < DBLOCKS; ++db)
+    {
+        u32x2 w;
+        w[0] = T::pack2(o[db][0] * inv, o[db][1] * inv);
+        w[1] = T::pack2(o[db][2] * inv, o[db][3] * inv);
+        *reinterpret_cast<u32x2 *>(dst + 16 * db) = w;
+    }
+#else
     float *dst = p.part_o + prow * HEAD + 4 * quad;
 #pragma unroll
     for(int db = 0; db < DBLOCKS; ++db)
     {
         *reinterpret_cast<acc4 *>(dst + 16 * db) = o[db];
     }
+#endif
 }
 
 // Merge the split partials of each row and fold the result into (lse, A).
@@ -504,7 +524,14 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
             const int sidx = min(s0 + j, last_split);
             const int64_t prow = base + (int64_t)sidx * p.rows;
             ml[j] = *reinterpret_cast<const f32x2 *>(p.part_ml + 2 * prow);
+#if NNTILE_DEC_PART16
+            const u32x2 raw = *reinterpret_cast<const u32x2 *>(
+                    reinterpret_cast<const uint16_t *>(p.part_o) + prow * HEAD + d4);
+            v[j] = f32x4{T::to_float((uint16_t)(raw[0] & 0xffffu)), T::to_float((uint16_t)(raw[0] >> 16)),
+                T::to_float((uint16_t)(raw[1] & 0xffffu)), T::to_float((uint16_t)(raw[1] >> 16))};
+#else
             v[j] = *reinterpret_cast<const f32x4 *>(p.part_o + prow * HEAD + d4);
+#endif
         }
     };
     auto add8 = [&](int s0, const f32x2 (&ml)[8], const f32x4 (&v)[8])
@@ -513,8 +540,13 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
         for(int j = 0; j < 8; ++j)
         {
             const bool live = (s0 + j <= last_split) && (ml[j][0] != neg_inf());
+#if NNTILE_DEC_PART16
+            const float w = live ? __expf(ml[j][0] - top) * ml[j][1] : 0.0f;
+            l += w;
+#else
             const float w = live ? __expf(ml[j][0] - top) : 0.0f;
             l += w * ml[j][1];
+#endif
             acc += w * v[j];
         }
     };
@@ -664,9 +696,17 @@ int decode_choose_splits(int units, int n_steps)
     return splits;
 }
 
+// The workspace: the partial outputs [unit][split][rows][head], then the
+// (max, sum) pairs [unit][split][rows][2] in fp32
+size_t decode_partial_o_bytes(int units, int n_splits, int rows, int head)
+{
+    return (size_t)units * n_splits * rows * head * (NNTILE_DEC_PART16 ? 2 : sizeof(float));
+}
+
 size_t decode_workspace_bytes(int units, int n_splits, int rows, int head)
 {
-    return (size_t)units * n_splits * rows * (head + 2) * sizeof(float);
+    return decode_partial_o_bytes(units, n_splits, rows, head)
+        + (size_t)units * n_splits * rows * 2 * sizeof(float);
 }
 
 template<typename T>
