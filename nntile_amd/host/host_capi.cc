@@ -67,12 +67,20 @@ void run_op(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *mask, AnyTensor *lse,
 }
 
 template<typename T>
-void run_bwd(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *V, AnyTensor *A,
+int64_t run_bwd(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *V, AnyTensor *A,
         AnyTensor *dA, AnyTensor *mask, AnyTensor *lse, AnyTensor *dK,
-        AnyTensor *dQ, AnyTensor *dV)
+        AnyTensor *dQ, AnyTensor *dV, int mask_mode, int64_t offset)
 {
     switch(op)
     {
+        case 2:     // tensor-level, analytic mask, hidden tile pairs skipped
+        {
+            const Index n = tensor::flash_sdpa_bwd_hip_async<T>(get<T>(K), get<T>(Q), get<T>(V),
+                    get<T>(A), get<T>(dA), mask_mode, offset, get<fp32_t>(lse),
+                    get<T>(dK), get<T>(dQ), get<T>(dV));
+            starpu::task_wait_for_all();
+            return n;
+        }
         case 0:     // tensor-level, per-tile tasks, blocking
             tensor::flash_sdpa_bwd_cudnn<T>(get<T>(K), get<T>(Q), get<T>(V),
                     get<T>(A), get<T>(dA), get<T>(mask), get<fp32_t>(lse),
@@ -87,6 +95,7 @@ void run_bwd(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *V, AnyTensor *A,
         default:
             throw std::runtime_error("unknown operation");
     }
+    return 0;
 }
 
 } // namespace
@@ -201,10 +210,11 @@ int nntile_host_check_shapes(int level, const int64_t *desc, char *err, int errl
 }
 
 // op: 0 tensor::flash_sdpa_bwd_cudnn, 1 tile::flash_sdpa_bwd_cudnn (single-tile
-// tensors); dtype bf16 or fp16, as the reference's pack
+// tensors), 2 tensor::flash_sdpa_bwd_hip_async + wait (mask may be null;
+// *submitted = tile pairs launched); dtype bf16 or fp16, as the reference's pack
 int nntile_host_flash_sdpa_bwd(int op, int dtype, void *K, void *Q, void *V,
         void *A, void *dA, void *mask, void *lse, void *dK, void *dQ, void *dV,
-        char *err, int errlen)
+        int mask_mode, int64_t offset, int64_t *submitted, char *err, int errlen)
 {
     try
     {
@@ -213,9 +223,11 @@ int nntile_host_flash_sdpa_bwd(int op, int dtype, void *K, void *Q, void *V,
             static_cast<AnyTensor *>(dA), static_cast<AnyTensor *>(mask),
             static_cast<AnyTensor *>(lse), static_cast<AnyTensor *>(dK),
             static_cast<AnyTensor *>(dQ), static_cast<AnyTensor *>(dV)};
-        if(dtype == DT_BF16) run_bwd<bf16_t>(op, t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7], t[8], t[9]);
-        else if(dtype == DT_FP16) run_bwd<fp16_t>(op, t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7], t[8], t[9]);
+        int64_t n = 0;
+        if(dtype == DT_BF16) n = run_bwd<bf16_t>(op, t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7], t[8], t[9], mask_mode, offset);
+        else if(dtype == DT_FP16) n = run_bwd<fp16_t>(op, t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7], t[8], t[9], mask_mode, offset);
         else throw std::runtime_error("flash_sdpa_bwd_cudnn: no fp32 instance");
+        if(submitted != nullptr) *submitted = n;
         return 0;
     }
     catch(const std::exception &e) { return fail(err, errlen, e); }

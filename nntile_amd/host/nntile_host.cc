@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstring>
 #include <iostream>
 #include <mutex>
@@ -896,7 +897,102 @@ void flash_sdpa_bwd_cudnn(const Tensor<T> &K, const Tensor<T> &Q,
     starpu::task_wait_for_all();
 }
 
+template<typename T> struct BwdTileCall;
+template<> struct BwdTileCall<bf16_t>
+{
+    static int run(void *s, const nntile_hip_sdpa_bwd_args *a) { return nntile_hip_sdpa_bwd_tile_bf16(s, a); }
+};
+template<> struct BwdTileCall<fp16_t>
+{
+    static int run(void *s, const nntile_hip_sdpa_bwd_args *a) { return nntile_hip_sdpa_bwd_tile_fp16(s, a); }
+};
+
+template<typename T>
+Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        int mask_mode, Index causal_offset, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV)
+{
+    // Same shape rules as the reference operation, with a stand-in for the
+    // mask that is no longer materialised.
+    const TensorTraits mask({K.shape[1], Q.shape[1]},
+            {K.basetile_shape[1], Q.basetile_shape[1]});
+    flash_sdpa_bwd_cudnn_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
+    require(mask_mode == NNTILE_HIP_MASK_NONE || mask_mode == NNTILE_HIP_MASK_CAUSAL,
+            "flash_sdpa_bwd_hip: mask_mode must be NONE or CAUSAL");
+    const Index num_k_seq_tiles = K.grid.shape[1];
+    const Index q_tile = Q.basetile_shape[1], k_tile = K.basetile_shape[1];
+    // One workspace for all calls: they run in order on one stream, and each
+    // call writes what it reads there.
+    std::size_t ws_bytes = 0;
+    for(Index i = 0; i < dQ.grid.nelems; ++i)
+    {
+        const auto &t = dQ.get_tile(i);
+        ws_bytes = std::max(ws_bytes, static_cast<std::size_t>(
+                    t.shape[1] * t.shape[2] * t.shape[3] * t.shape[4]) * sizeof(float));
+    }
+    starpu::VariableHandle workspace(ws_bytes);
+    Index submitted = 0;
+    for(Index dq_linear = 0; dq_linear < dQ.grid.nelems; ++dq_linear)
+    {
+        const auto dq_index = dQ.grid.linear_to_index(dq_linear);
+        const auto &Q_tile = Q.get_tile(dq_linear);
+        const auto &lse_tile = logsumexp.get_tile(
+                {dq_index[1], dq_index[2], dq_index[3], dq_index[4]});
+        const Index q_pos0 = dq_index[1] * q_tile;
+        const Index q_len = Q_tile.shape[1];
+        for(Index k_idx = 0; k_idx < num_k_seq_tiles; ++k_idx)
+        {
+            const Index k_pos0 = k_idx * k_tile;
+            // the last query of the tile sees keys up to its position + offset
+            if(mask_mode == NNTILE_HIP_MASK_CAUSAL
+                    && k_pos0 > q_pos0 + q_len - 1 + causal_offset)
+            {
+                continue;
+            }
+            auto kv_index = dq_index;
+            kv_index[1] = k_idx;
+            const auto &K_tile = K.get_tile(kv_index);
+            nntile_hip_sdpa_bwd_args a;
+            std::memset(&a, 0, sizeof(a));
+            a.q_seq = q_len;
+            a.k_seq = K_tile.shape[1];
+            a.head = Q_tile.shape[0];
+            a.batch = Q_tile.shape[2] * Q_tile.shape[3] * Q_tile.shape[4];
+            a.n_batch = a.batch;
+            a.kv_group = 1;
+            a.mask_mode = mask_mode;
+            a.q_pos0 = q_pos0;
+            a.k_pos0 = k_pos0;
+            a.causal_offset = causal_offset;
+            a.K = K_tile.get_ptr();
+            a.Q = Q_tile.get_ptr();
+            a.V = V.get_tile(kv_index).get_ptr();
+            a.A = A.get_tile(dq_linear).get_ptr();
+            a.dA = dA.get_tile(dq_linear).get_ptr();
+            a.lse = static_cast<const float *>(lse_tile.get_ptr());
+            a.dK = dK.get_tile(kv_index).get_ptr();
+            a.dQ = dQ.get_tile(dq_linear).get_ptr();
+            a.dV = dV.get_tile(kv_index).get_ptr();
+            a.workspace = workspace.get_ptr();
+            a.workspace_bytes = ws_bytes;
+            const int rc = BwdTileCall<T>::run(starpu::get_local_stream(), &a);
+            if(rc != NNTILE_HIP_OK)
+            {
+                throw std::runtime_error("Error in flash_sdpa_bwd_hip launch (code "
+                        + std::to_string(rc) + ")");
+            }
+            ++submitted;
+        }
+    }
+    workspace.unregister_submit();
+    return submitted;
+}
+
 #define NNTILE_HOST_INSTANTIATE_TENSOR_BWD(T) \
+    template Index flash_sdpa_bwd_hip_async<T>(const Tensor<T> &, const Tensor<T> &, \
+            const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, int, Index, \
+            const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &); \
     template void flash_sdpa_bwd_cudnn_async<T>(const Tensor<T> &, const Tensor<T> &, \
             const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, \
             const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &); \

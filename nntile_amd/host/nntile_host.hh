@@ -284,6 +284,17 @@ void flash_sdpa_bwd_cudnn(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV);
 
+//! Same gradients with an analytic mask (NNTILE_HIP_MASK_NONE, or
+//! NNTILE_HIP_MASK_CAUSAL with `causal_offset`): no mask tensor, one call per
+//! (dQ tile, key tile) pair with the pair's positions, and pairs that a
+//! causal mask hides completely are not submitted.  Gradients are added.
+//! Returns the number of tile pairs submitted.
+template<typename T>
+Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        int mask_mode, Index causal_offset, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV);
+
 } // namespace tensor
 
 } // namespace nntile

@@ -38,7 +38,7 @@ def lib():
         L.nntile_host_check_shapes.argtypes = [ctypes.c_int, ctypes.POINTER(i64), ctypes.c_char_p,
                                                ctypes.c_int]
         L.nntile_host_flash_sdpa_bwd.argtypes = [ctypes.c_int, ctypes.c_int] + [vp] * 10 + [
-            ctypes.c_char_p, ctypes.c_int]
+            ctypes.c_int, i64, ctypes.POINTER(i64), ctypes.c_char_p, ctypes.c_int]
         L.nntile_host_check_shapes_bwd.argtypes = [ctypes.c_int, ctypes.POINTER(i64), ctypes.c_char_p,
                                                    ctypes.c_int]
         L.nntile_host_footprint_bwd.argtypes = [i64, i64, i64]
@@ -107,11 +107,15 @@ def flash_sdpa_fwd(op, K, Q, mask, lse, V, A, mask_mode=0, offset=0, overwrite=F
           None if mask is None else mask.h, lse.h, V.h, A.h, mask_mode, offset, int(overwrite))
 
 
-def flash_sdpa_bwd(op, K, Q, V, A, dA, mask, lse, dK, dQ, dV):
-    """tensor::flash_sdpa_bwd_cudnn (op 0) or tile::flash_sdpa_bwd_cudnn (op 1):
-    the gradients are added to dK, dQ, dV."""
+def flash_sdpa_bwd(op, K, Q, V, A, dA, mask, lse, dK, dQ, dV, mask_mode=0, offset=0):
+    """tensor::flash_sdpa_bwd_cudnn (op 0), tile::flash_sdpa_bwd_cudnn (op 1) or
+    tensor::flash_sdpa_bwd_hip_async (op 2: analytic mask, mask=None): the
+    gradients are added to dK, dQ, dV.  Returns the tile pairs op 2 launched."""
+    n = ctypes.c_int64(0)
     _call(lib().nntile_host_flash_sdpa_bwd, op, DTYPES[Q.dtype],
-          *(t.h for t in (K, Q, V, A, dA, mask, lse, dK, dQ, dV)))
+          *(None if t is None else t.h for t in (K, Q, V, A, dA, mask, lse, dK, dQ, dV)),
+          mask_mode, offset, ctypes.byref(n))
+    return n.value
 
 
 def check_shapes_bwd(level, specs):

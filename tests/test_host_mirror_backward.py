@@ -114,7 +114,7 @@ def _flat(x, head, seq):
     return np.ascontiguousarray(x.transpose(4, 3, 2, 1, 0)).reshape(-1, seq, head)
 
 
-def _run(op, dtype, data, lse, add_mask, shape5, base5, grads0=None):
+def _run(op, dtype, data, lse, add_mask, shape5, base5, grads0=None, mask_mode=0, offset=0):
     """data: fp32 C-ordered [batch_flat, seq, head] arrays of tile-dtype values
     for K, Q, V, A, dA.  Returns (dK, dQ, dV) the same way, and the task count."""
     head, seq, nb, grp, nkv = shape5
@@ -132,9 +132,14 @@ def _run(op, dtype, data, lse, add_mask, shape5, base5, grads0=None):
     M = hm.Tensor(dtype, [seq, seq], [base5[1], base5[1]]).from_array(
         np.asfortranarray(_bits(m).T))                      # Fortran [k, q]
     before = hm.tasks_submitted_bwd(dtype)
-    hm.flash_sdpa_bwd(op, T["K"], T["Q"], T["V"], T["A"], T["dA"], M, L, T["dK"], T["dQ"], T["dV"])
+    if op == hm.OP_HIP:
+        pairs = hm.flash_sdpa_bwd(op, T["K"], T["Q"], T["V"], T["A"], T["dA"], None, L, T["dK"], T["dQ"],
+                                  T["dV"], mask_mode=mask_mode, offset=offset)
+    else:
+        hm.flash_sdpa_bwd(op, T["K"], T["Q"], T["V"], T["A"], T["dA"], M, L, T["dK"], T["dQ"], T["dV"])
+        pairs = hm.tasks_submitted_bwd(dtype) - before
     out = [_flat(_values(T[n].to_array(), dtype), head, seq) for n in ("dK", "dQ", "dV")]
-    return out, hm.tasks_submitted_bwd(dtype) - before, T["dQ"].ntiles
+    return out, pairs, T["dQ"].ntiles
 
 
 def _reference_data(n, dtype):
@@ -207,3 +212,42 @@ def test_tile_level_adds_to_the_gradients_and_reads_the_mask_as_key_by_query(ora
     f32 = hm.Tensor("fp32", shape5, shape5)
     with pytest.raises(hm.HostError, match="no fp32 instance"):
         hm.flash_sdpa_bwd(hm.OP_TILE, f32, f32, f32, f32, f32, f32, L, f32, f32, f32)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("mode,offset", [("causal", 0), ("causal", -70), ("none", 0)])
+def test_analytic_mask_form_skips_hidden_tile_pairs(oracle, dtype, mode, offset):
+    """tensor::flash_sdpa_bwd_hip_async: no mask tensor, the tile pairs a
+    causal mask hides are not launched, gradients as the checker's with the
+    same mask written out."""
+    head, seq, tile, nb, grp, nkv = 64, 320, 64, 2, 1, 2
+    batch = nb * grp * nkv
+    shape5, base5 = [head, seq, nb, grp, nkv], [head, tile, 1, 1, 2]
+    (Q, K, V), (qf, kf, vf) = H.make_qkv(51, batch, seq, seq, head, dtype)
+    _, gf = H.rounded(synth.randn(52, 0, batch * seq * head).reshape(batch, seq, head), dtype)
+    i = np.arange(seq)
+    mask = (i[None, :] <= i[:, None] + offset) if mode == "causal" else np.ones((seq, seq), bool)
+    add = np.where(mask, 0.0, -np.inf).astype(np.float32)
+    vis = mask.any(axis=1)
+    with np.errstate(all="ignore"):
+        A64, lse64 = oracle.sdpa_bruteforce_f64(kf, qf, vf, add)
+    A64 = np.where(vis[None, :, None], A64, 0.0)
+    lse = np.where(vis[None, :], lse64, -np.inf).astype(np.float32)
+    _, af = H.rounded(A64, dtype)
+    data = {"K": kf, "Q": qf, "V": vf, "A": af, "dA": gf}
+    got, pairs, ntiles = _run(hm.OP_HIP, dtype, data, lse, add, shape5, base5,
+                              mask_mode=2 if mode == "causal" else 1, offset=offset)
+    nt = seq // tile
+    slabs = ntiles // nt
+    if mode == "none":
+        assert pairs == slabs * nt * nt
+    else:
+        visible_pairs = sum(1 for q in range(nt) for k in range(nt)
+                            if k * tile <= q * tile + tile - 1 + offset)
+        assert pairs == slabs * visible_pairs and visible_pairs < nt * nt
+    with np.errstate(all="ignore"):
+        want = oracle.sdpa_bwd_flash_f64(kf, qf, vf, af, gf, np.where(vis[None, :], lse, 0.0),
+                                         np.where(vis[:, None], add, -np.inf))
+    for g, w, n in zip(got, want, ("dK", "dQ", "dV")):
+        assert H.rel_fro(g, w) < (1e-2 if dtype == "bf16" else 2e-3), n
