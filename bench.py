@@ -226,6 +226,34 @@ def bench_rope(cfg, steps, warmup):
             "frac_of_hbm_peak": round(nbytes / (dev * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
 
 
+def bench_transpose(cfg, steps, warmup):
+    """The transpose that follows the attention kernel (attention output
+    [head, seq, heads] -> [heads, head, seq], llama_attention.py:622-625):
+    m = head * seq, n = heads as one m x n matrix.  HBM-bound: reads and
+    writes the tensor once; eight buffer pairs rotate."""
+    import torch
+    from nntile_amd import hip_sdpa as h
+    dt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg.dtype]
+    m, n = cfg.head * cfg.q_seq, cfg.batch_flat
+    nrot = 8
+    src = [_randn((n, m), dt, cfg.seed * 1000 + 900 + i) for i in range(nrot)]
+    dst = [torch.empty_like(x) for x in src]
+    i = [0]
+
+    def step():
+        j = i[0] % nrot
+        h.transpose(1.0, src[j], dst[j], m, n)
+        i[0] += 1
+
+    wall, dev = time_steps(step, steps, warmup)
+    nbytes = 2 * src[0].numel() * src[0].element_size()
+    return {"what": "transpose of the attention output of %s (%d x %d, %d MiB)"
+                    % (cfg.name, m, n, src[0].numel() * src[0].element_size() >> 20),
+            "device_ms_per_step": round(dev, 4), "algorithmic_bytes": nbytes,
+            "gbs": round(nbytes / (dev * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(nbytes / (dev * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+
+
 def cpu_baseline(cfg, target_seconds=15.0):
     """The CPU checker (port of the reference's gemm -> mask_scalar ->
     maxsumexp -> softmax_inplace -> gemm composition) on a bounded sample of
@@ -264,7 +292,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run only this leg: prefill | decode | per_task | backward | rope | extras | copy (for profiling)")
+                    help="run only this leg: prefill | decode | per_task | backward | rope | transpose | extras | copy (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
@@ -304,6 +332,9 @@ def main():
     if only == "backward":
         print(json.dumps(bench_backward(cfg3, args.steps, args.warmup)))
         return
+    if only == "transpose":
+        print(json.dumps(bench_transpose(cfg3, args.steps, args.warmup)))
+        return
     if only == "rope":
         print(json.dumps(bench_rope(cfg3, args.steps, args.warmup)))
         return
@@ -327,6 +358,7 @@ def main():
                         "launches_per_step": r["launches_per_step"]}
     backward = bench_backward(cfg3, max(5, args.steps // 10), 2)
     rope = bench_rope(cfg3, max(5, args.steps // 5), 5)
+    transpose = bench_transpose(cfg3, max(5, args.steps // 5), 5)
     # The headline leg runs last: the first timed loop of a process measures
     # 5 % slower than the same loop a second later (clocks still settling),
     # whatever the warmup count.
@@ -374,6 +406,7 @@ def main():
         "other_configs": extras,
         "backward": backward,
         "rope": rope,
+        "transpose": transpose,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg3)

@@ -293,6 +293,18 @@ int nntile_hip_rope_backward_fp16(void *stream, int64_t m, int64_t n, const uint
 int nntile_hip_rope_backward_fp32(void *stream, int64_t m, int64_t n, const float *sin,
         const float *cos, const float *dy, float *dx);
 
+/* ---- 8. The transposes either side of the attention block -------------------
+ * Replace kernel::transpose::cuda<T> (include/nntile/kernel/transpose/cuda.hh:25,
+ * arithmetic src/kernel/transpose/cpu.cc:21-43): dst = alpha * src^T for an
+ * m x n matrix in Fortran order (src(i,j) at i + j*m, dst(j,i) at j + i*n).
+ * The reference's Scalar alpha is a float.  src and dst must not overlap. */
+int nntile_hip_transpose_bf16(void *stream, int64_t m, int64_t n, float alpha,
+        const uint16_t *src, uint16_t *dst);
+int nntile_hip_transpose_fp16(void *stream, int64_t m, int64_t n, float alpha,
+        const uint16_t *src, uint16_t *dst);
+int nntile_hip_transpose_fp32(void *stream, int64_t m, int64_t n, float alpha,
+        const float *src, float *dst);
+
 /* Library version and the ISA it was built for ("gfx950"). */
 const char *nntile_hip_sdpa_version(void);
 

@@ -30,6 +30,9 @@ int launch_accumulate(hipStream_t stream, int64_t head, int64_t seq,
 int launch_rope(hipStream_t stream, int dtype, bool backward, int64_t m, int64_t n,
         const void *sin, const void *cos, const void *src, void *dst);
 
+int launch_transpose(hipStream_t stream, int dtype, int64_t m, int64_t n, float alpha,
+        const void *src, void *dst);
+
 enum class DType { bf16, fp16, fp32 };
 
 static bool aligned16(const void *p)
@@ -415,6 +418,26 @@ static int rope_call(DType dt, bool backward, void *stream, int64_t m, int64_t n
             dst);
 }
 
+static int transpose_call(DType dt, void *stream, int64_t m, int64_t n, float alpha,
+        const void *src, void *dst)
+{
+    if(m < 0 || n < 0)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(m == 0 || n == 0)
+    {
+        return NNTILE_HIP_OK;
+    }
+    if(src == nullptr || dst == nullptr || src == dst
+            || m > (int64_t)0x3fffffffffffffff / n)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    const int code = dt == DType::bf16 ? 0 : (dt == DType::fp16 ? 1 : 2);
+    return launch_transpose(static_cast<hipStream_t>(stream), code, m, n, alpha, src, dst);
+}
+
 static nntile_hip_stream_provider g_stream_provider = nullptr;
 
 static void codelet_call(DType dt, const char *name, void *buffers[],
@@ -691,6 +714,24 @@ NNTILE_HIP_ROPE_ENTRY(bf16, DType::bf16, uint16_t)
 NNTILE_HIP_ROPE_ENTRY(fp16, DType::fp16, uint16_t)
 NNTILE_HIP_ROPE_ENTRY(fp32, DType::fp32, float)
 #undef NNTILE_HIP_ROPE_ENTRY
+
+int nntile_hip_transpose_bf16(void *stream, int64_t m, int64_t n, float alpha,
+        const uint16_t *src, uint16_t *dst)
+{
+    return transpose_call(DType::bf16, stream, m, n, alpha, src, dst);
+}
+
+int nntile_hip_transpose_fp16(void *stream, int64_t m, int64_t n, float alpha,
+        const uint16_t *src, uint16_t *dst)
+{
+    return transpose_call(DType::fp16, stream, m, n, alpha, src, dst);
+}
+
+int nntile_hip_transpose_fp32(void *stream, int64_t m, int64_t n, float alpha,
+        const float *src, float *dst)
+{
+    return transpose_call(DType::fp32, stream, m, n, alpha, src, dst);
+}
 
 const char *nntile_hip_sdpa_version(void)
 {

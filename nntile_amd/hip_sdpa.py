@@ -86,6 +86,7 @@ EXPORTS = (
     + ["nntile_hip_flash_sdpa_fwd_codelet_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_rope_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_rope_backward_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_transpose_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_set_stream_provider", "nntile_hip_sdpa_version"])
 
 _lib = None
@@ -133,6 +134,10 @@ def lib():
                 f = getattr(L, name + t)
                 f.argtypes = [_vp, _i64, _i64, _vp, _vp, _vp, _vp]
                 f.restype = ctypes.c_int
+        for t in ("bf16", "fp16", "fp32"):
+            f = getattr(L, "nntile_hip_transpose_" + t)
+            f.argtypes = [_vp, _i64, _i64, ctypes.c_float, _vp, _vp]
+            f.restype = ctypes.c_int
         L.nntile_hip_sdpa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
         L.nntile_hip_sdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.argtypes = [ctypes.POINTER(TileArgs)]
@@ -390,6 +395,16 @@ def rope(sin, cos, src, dst, backward=False, stream=None):
     name = "nntile_hip_rope_backward_" if backward else "nntile_hip_rope_"
     fn = getattr(lib(), name + dtype_name(src))
     _check(fn(_stream(stream), m, n, _ptr(sin), _ptr(cos), _ptr(src), _ptr(dst)), "rope")
+
+
+def transpose(alpha, src, dst, m, n, stream=None):
+    """dst = alpha * src^T; src is m x n in Fortran order (memory order of a
+    C-ordered [n, m] tensor), dst n x m in Fortran order."""
+    _dev(src, dst)
+    if src.numel() != m * n or dst.numel() != m * n:
+        raise SdpaError(EINVAL, "transpose")
+    fn = getattr(lib(), "nntile_hip_transpose_" + dtype_name(src))
+    _check(fn(_stream(stream), m, n, float(alpha), _ptr(src), _ptr(dst)), "transpose")
 
 
 def flash_sdpa_fwd_codelet(K, Q, mask, lse, V, A, scratch_lse=None, scratch_A=None,

@@ -317,3 +317,11 @@ def rope(sin, cos, src, backward=False):
         out[..., 0] = c * a - s * b
         out[..., 1] = s * a + c * b
     return out.reshape(x.shape)
+
+
+def transpose(m, n, alpha, src):
+    """dst[i*n + j] = alpha * src[i + j*m] (src/kernel/transpose/cpu.cc:21-43):
+    src is an m x n matrix in Fortran order, dst its transpose in Fortran
+    order, the product in fp32.  Returns the flat float32 dst."""
+    x = np.asarray(src, np.float32).reshape(n, m)      # x[j, i] = src(i, j)
+    return (np.float32(alpha) * np.ascontiguousarray(x.T)).reshape(-1)
