@@ -166,9 +166,11 @@ def bench_decode(cfg, steps, warmup):
 
 def bench_backward(cfg, steps, warmup):
     """Backward of the same attention (dQ, dK, dV from dA, A and lse) as one
-    call over the whole sequence with the analytic causal mask: two launches.
+    call over the whole sequence with the analytic causal mask: the row dots,
+    then one launch for the three gradients.
     FLOPs counted as 2.5 x the forward's (five products where the forward has
-    two); the two kernels execute seven, recomputing the scores in each."""
+    two); the workgroups execute eight, recomputing the scores for each
+    gradient."""
     import torch
     from nntile_amd import hip_sdpa as h
     dt = {"bf16": torch.bfloat16, "fp16": torch.float16}[cfg.dtype]

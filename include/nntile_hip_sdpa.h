@@ -122,8 +122,9 @@ int nntile_hip_sdpa_fwd_tile_fp32(void *stream, const nntile_hip_sdpa_tile_args 
  * gradients of this tile pair are ADDED to dK, dQ, dV (the reference computes
  * them into the scratch tiles and adds those, cuda.cc:213-217).  scratch_dK
  * and scratch_dV are accepted for signature compatibility and never touched;
- * the first seq*batch floats of scratch_dQ hold the row dots dA.A between the
- * two kernels of the call (it must not be null).  The reference's pack is
+ * scratch_dQ is the call's workspace (it must not be null): its first
+ * seq*batch floats hold the row dots dA.A, the bytes behind them one class
+ * per 64 x 64 block of the mask.  The reference's pack is
  * {bf16, fp16} (include/nntile/starpu/flash_sdpa_bwd_cudnn.hh). */
 int nntile_hip_flash_sdpa_bwd_bf16(void *stream, int64_t seq, int64_t head,
         int64_t batch, const uint16_t *K, const uint16_t *Q, const uint16_t *V,

@@ -39,7 +39,7 @@ namespace nntile_hip
 #ifndef NNTILE_BWD_SPREAD
 #define NNTILE_BWD_SPREAD 2
 #endif
-constexpr int kBwdRows = 128;       // queries (dQ kernel) / keys (dK,dV kernel) per workgroup
+constexpr int kBwdRows = 128;       // queries (dQ workgroups) / keys (dK, dV workgroups) per workgroup
 constexpr int kBwdStep = 64;        // rows of the other axis per step
 constexpr int kBwdThreads = 256;
 
@@ -51,7 +51,7 @@ __device__ __forceinline__ u32x2 bwd_lds_read_tr16(const char *lds_ptr)
     return __builtin_bit_cast(u32x2, v);
 }
 
-// What the two kernels share: the geometry of a 64-row step in LDS.
+// What the three kinds of workgroup share: the geometry of a 64-row step in LDS.
 template<int HEAD>
 struct BwdTile
 {

@@ -89,7 +89,7 @@ struct BwdParams
     const void *mask;
     const void *K, *Q, *V, *A, *dA;
     const float *lse;
-    float *D;               // workspace: written by the dQ kernel, read by the dK/dV kernel
+    float *D;               // workspace: the row dots dA . A, written before the gradient launch
     // explicit masks: class of every 64 x 64 block of the mask, row = query
     // block, class_ld entries per row (0 mixed, 1 nothing masked, 2 all
     // hidden); null when the workspace has no room for it
