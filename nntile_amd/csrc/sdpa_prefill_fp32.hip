@@ -22,6 +22,10 @@
 namespace nntile_hip
 {
 
+// 16-byte K operand reads issued ahead of the MFMAs that use them
+#ifndef NNTILE_F32_AHEAD
+#define NNTILE_F32_AHEAD 2
+#endif
 constexpr int kQRows32 = 128;
 constexpr int kKeys32 = 32;
 constexpr int kThreads32 = 256;
@@ -101,32 +105,76 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     const int ld_row = tid / CHUNKS;
     f32x4 k_regs[NSUB][PASSES], v_regs[NSUB][PASSES];
 
-    // loads of the key steps NSUB*G .. NSUB*G + NSUB-1 (zeros past the end)
-    auto fetch = [&](int G, int n_steps_all)
+    // Where the rows of a key step come from.  One key tile (every tile-pair
+    // call): the tile's addresses are computed once, a step needs no division
+    // and no look-up in the tile table.
+    struct StepSource
+    {
+        const float *K, *V;
+        int row0, last_row;
+    };
+    const int64_t k_len0 = min(p.k_tile, p.k_seq);
+    const bool one_tile = p.n_kv_tiles == 1;
+    const float *K0 = static_cast<const float *>(p.K[0]) + ((int64_t)kvb * k_len0) * HEAD;
+    const float *V0 = static_cast<const float *>(p.V[0]) + ((int64_t)kvb * k_len0) * HEAD;
+    auto locate = [&](int g, int n_steps_all) -> StepSource
+    {
+        // steps past the last re-read the last one (nobody uses them)
+        g = min(g, max(n_steps_all - 1, 0));
+        StepSource src;
+        if(one_tile)
+        {
+            src.K = K0;
+            src.V = V0;
+            src.row0 = g * kKeys32;
+            src.last_row = (int)k_len0 - 1;
+        }
+        else
+        {
+            const int kt = g / p.k_blocks_per_tile;
+            const int kb = g % p.k_blocks_per_tile;
+            const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
+            src.K = static_cast<const float *>(p.K[kt]) + ((int64_t)kvb * k_len) * HEAD;
+            src.V = static_cast<const float *>(p.V[kt]) + ((int64_t)kvb * k_len) * HEAD;
+            src.row0 = kb * kKeys32;
+            src.last_row = (int)k_len - 1;
+        }
+        return src;
+    };
+    // The loads of the staged steps, one 16-byte load per thread and piece:
+    // piece k is step k / (2 PASSES), pass (k / 2) % PASSES, K for even k and V
+    // for odd k.  Rows past the end of the tile re-read its last row: their
+    // keys are masked out of the scores, so their probabilities are exactly
+    // 0, and a load that is never conditional does not make the wave wait.
+    // (the launcher keeps a tile's rows x HEAD within 31 bits)
+    constexpr int PIECES = NSUB * PASSES * 2;
+    StepSource src[NSUB];
+    auto fetch_piece = [&](int k) __attribute__((always_inline))
+    {
+        const int sub = k / (2 * PASSES), i = (k / 2) % PASSES;
+        const uint32_t off = (uint32_t)min(src[sub].row0 + ld_row + i * ROWS_PER_PASS,
+                src[sub].last_row) * HEAD + ld_chunk * 4;
+        if(k % 2 == 0)
+        {
+            k_regs[sub][i] = *reinterpret_cast<const f32x4 *>(src[sub].K + off);
+        }
+        else
+        {
+            v_regs[sub][i] = *reinterpret_cast<const f32x4 *>(src[sub].V + off);
+        }
+    };
+    // A wave gets one load accepted every ~70 cycles and stands still until
+    // then; inside the loop the pieces therefore go between the MFMAs, which
+    // run meanwhile: slot t of SLOTS takes the pieces k with k*SLOTS/PIECES == t.
+    constexpr int SLOTS = QSTEPS + 16;
+    auto fetch_slot = [&](int t) __attribute__((always_inline))
     {
 #pragma unroll
-        for(int sub = 0; sub < NSUB; ++sub)
+        for(int k = 0; k < PIECES; ++k)
         {
-            const int g = G * NSUB + sub;
-            const bool step_ok = g < n_steps_all;
-            const int kt = step_ok ? g / p.k_blocks_per_tile : 0;
-            const int kb = step_ok ? g % p.k_blocks_per_tile : 0;
-            const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
-            const int64_t row0 = (int64_t)kb * kKeys32;
-            const float *Kt = static_cast<const float *>(p.K[kt])
-                + ((int64_t)kvb * k_len) * HEAD;
-            const float *Vtile = static_cast<const float *>(p.V[kt])
-                + ((int64_t)kvb * k_len) * HEAD;
-#pragma unroll
-            for(int i = 0; i < PASSES; ++i)
+            if(k * SLOTS / PIECES == t)
             {
-                const int64_t r = row0 + ld_row + i * ROWS_PER_PASS;
-                const bool ok = step_ok && r < k_len;
-                const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-                k_regs[sub][i] = ok ? *reinterpret_cast<const f32x4 *>(
-                        Kt + r * HEAD + ld_chunk * 4) : zero;
-                v_regs[sub][i] = ok ? *reinterpret_cast<const f32x4 *>(
-                        Vtile + r * HEAD + ld_chunk * 4) : zero;
+                fetch_piece(k);
             }
         }
     };
@@ -189,20 +237,36 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     const float *Vw = Vs + (SPLIT ? wave * kKeys32 * PAD : 0);
     if(n_iter > 0)
     {
-        fetch(0, n_steps);
+#pragma unroll
+        for(int sub = 0; sub < NSUB; ++sub)
+        {
+            src[sub] = locate(sub, n_steps);
+        }
+#pragma unroll
+        for(int k = 0; k < PIECES; ++k)
+        {
+            fetch_piece(k);
+        }
     }
     for(int G = 0; G < n_iter; ++G)
     {
         __syncthreads();
         stage();
         __syncthreads();
-        if(G + 1 < n_iter)
+        // the next iteration's steps: located now, loaded between the MFMAs
+#pragma unroll
+        for(int sub = 0; sub < NSUB; ++sub)
         {
-            fetch(G + 1, n_steps);
+            src[sub] = locate((G + 1) * NSUB + sub, n_steps);
         }
         const int g = SPLIT ? G * NSUB + wave : G;      // this wavefront's step
         if(g >= n_steps)
         {
+#pragma unroll
+            for(int k = 0; k < PIECES; ++k)
+            {
+                fetch_piece(k);
+            }
             continue;
         }
 
@@ -216,6 +280,12 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         if(MODE == NNTILE_HIP_MASK_CAUSAL
                 && k_pos_base > wave_qpos_hi + p.causal_offset)
         {
+            // (nothing visible for this wavefront; its share of the loads remains)
+#pragma unroll
+            for(int k = 0; k < PIECES; ++k)
+            {
+                fetch_piece(k);
+            }
             continue;
         }
 
@@ -226,16 +296,37 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         {
             s[r] = 0.0f;
         }
-#pragma unroll
-        for(int j = 0; j < QSTEPS; ++j)
+        // (the K operands of the step are read ahead of the chain of
+        // dependent MFMAs: a read issued behind four of them would only start
+        // once they have all been issued, i.e. when the last one runs)
         {
-            const f32x4 a = *reinterpret_cast<const f32x4 *>(
-                    &Kw[col * PAD + j * 8 + half * 4]);
+            constexpr int AHEAD = NNTILE_F32_AHEAD < QSTEPS ? NNTILE_F32_AHEAD : QSTEPS;
+            f32x4 ka[QSTEPS];
 #pragma unroll
-            for(int e = 0; e < 4; ++e)
+            for(int j = 0; j < AHEAD; ++j)
             {
-                s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], qf[j][e], s,
-                        0, 0, 0);
+                ka[j] = *reinterpret_cast<const f32x4 *>(&Kw[col * PAD + j * 8 + half * 4]);
+            }
+#pragma unroll
+            for(int j = 0; j < QSTEPS; ++j)
+            {
+                if(j + AHEAD < QSTEPS)
+                {
+                    ka[j + AHEAD] = *reinterpret_cast<const f32x4 *>(
+                            &Kw[col * PAD + (j + AHEAD) * 8 + half * 4]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for(int e = 0; e < 4; ++e)
+                {
+                    s = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[j][e], qf[j][e], s,
+                            0, 0, 0);
+                    if(e == 0)
+                    {
+                        fetch_slot(j);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
             }
         }
 
@@ -327,16 +418,48 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         }
 
         // ---- O^T += V^T P^T ----------------------------------------------------
-#pragma unroll
-        for(int r = 0; r < 16; ++r)
+        // (V operands four keys at a time, one group ahead of its MFMAs)
         {
-            const int key = 8 * (r >> 2) + 4 * half + (r & 3);
-#pragma unroll
-            for(int db = 0; db < DBLOCKS; ++db)
+            float va[16][DBLOCKS];
+            auto read_group = [&](int g4)
             {
-                const float a = Vw[key * PAD + db * 32 + col];
-                o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s[r], o[db],
-                        0, 0, 0);
+#pragma unroll
+                for(int x = 0; x < 4; ++x)
+                {
+                    const int r = 4 * g4 + x;
+                    const int key = 8 * (r >> 2) + 4 * half + (r & 3);
+#pragma unroll
+                    for(int db = 0; db < DBLOCKS; ++db)
+                    {
+                        va[r][db] = Vw[key * PAD + db * 32 + col];
+                    }
+                }
+            };
+            read_group(0);
+#pragma unroll
+            for(int g4 = 0; g4 < 4; ++g4)
+            {
+                if(g4 + 1 < 4)
+                {
+                    read_group(g4 + 1);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for(int x = 0; x < 4; ++x)
+                {
+                    const int r = 4 * g4 + x;
+#pragma unroll
+                    for(int db = 0; db < DBLOCKS; ++db)
+                    {
+                        o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[r][db], s[r], o[db],
+                                0, 0, 0);
+                        if(db == 0)
+                        {
+                            fetch_slot(QSTEPS + r);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                }
             }
         }
     }
@@ -477,6 +600,11 @@ static int launch_mode32(hipStream_t stream, const PrefillParams &p, int mode,
 int launch_prefill_fp32(hipStream_t stream, PrefillParams &p, int head, int mode)
 {
     p.k_blocks_per_tile = (int)((p.k_tile + kKeys32 - 1) / kKeys32);
+    // the kernel addresses the rows of a key tile with 32-bit element offsets
+    if(p.k_tile * head >= ((int64_t)1 << 31))
+    {
+        return NNTILE_HIP_EUNSUPPORTED;
+    }
     // with fewer 128-query workgroups than CUs, 32-query workgroups whose
     // wavefronts share the keys instead
     const int64_t n_wide = (int64_t)p.batch * p.n_q_tiles
