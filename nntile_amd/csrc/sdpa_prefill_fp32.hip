@@ -28,14 +28,24 @@ namespace nntile_hip
 #endif
 constexpr int kQRows32 = 128;
 constexpr int kKeys32 = 32;
-constexpr int kThreads32 = 256;
+constexpr int kThreads32 = 256;          // first form: 4 wavefronts
+#ifndef NNTILE_F32_SPLIT_WAVES
+#define NNTILE_F32_SPLIT_WAVES 4
+#endif
+// second form: wavefronts sharing the keys.  Head 64 stages 8 steps (139 KiB
+// of LDS); head 128 has room for 4, head 32 has 256 16-byte chunks a step.
+__host__ __device__ constexpr int split_waves32(int head)
+{
+    return head == 64 ? NNTILE_F32_SPLIT_WAVES : 4;
+}
 
 template<int HEAD, int MODE, bool SPLIT>
-__global__ __launch_bounds__(kThreads32, SPLIT ? 1 : 2)
+__global__ __launch_bounds__(SPLIT ? split_waves32(HEAD) * 64 : kThreads32, SPLIT ? 1 : 2)
 void sdpa_prefill_fp32_kernel(const PrefillParams p)
 {
     constexpr int QROWS = SPLIT ? 32 : kQRows32;    // queries per workgroup
-    constexpr int NSUB = SPLIT ? 4 : 1;             // key steps staged per iteration
+    constexpr int THREADS = SPLIT ? split_waves32(HEAD) * 64 : kThreads32;
+    constexpr int NSUB = SPLIT ? split_waves32(HEAD) : 1;   // key steps staged per iteration
     constexpr int QSTEPS = HEAD / 8;        // 16-byte groups per lane half along head
     constexpr int DBLOCKS = HEAD / 32;
     constexpr int PAD = HEAD + 4;           // row stride in LDS (floats)
@@ -99,7 +109,8 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     const int64_t wave_qpos_hi = wave_qpos_lo + 31;
 
     // Cooperative loads: 32 rows x CHUNKS chunks for K and for V.
-    constexpr int ROWS_PER_PASS = kThreads32 / CHUNKS;
+    constexpr int ROWS_PER_PASS = THREADS / CHUNKS;
+    static_assert(THREADS <= kKeys32 * CHUNKS, "more threads than 16-byte chunks of a step");
     constexpr int PASSES = kKeys32 / ROWS_PER_PASS;
     const int ld_chunk = tid % CHUNKS;
     const int ld_row = tid / CHUNKS;
@@ -469,7 +480,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     {
         // word w of lane l of wavefront v (v = 1..3) sits at ((v-1)*NW + w)*64 + l
         constexpr int NW = 2 + 16 * DBLOCKS;
-        static_assert(3 * NW * 64 <= NSUB * kKeys32 * PAD, "exchange area does not fit");
+        static_assert((NSUB - 1) * NW * 64 <= NSUB * kKeys32 * PAD, "exchange area does not fit");
         float *xch = Ks;
         __syncthreads();        // everyone is done with the staged keys
         if(wave > 0)
@@ -493,7 +504,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
             return;
         }
 #pragma unroll
-        for(int v = 0; v < 3; ++v)
+        for(int v = 0; v < NSUB - 1; ++v)
         {
             const float *src = xch + v * NW * 64 + lane;
             const float m_other = src[0];
@@ -573,22 +584,22 @@ static int launch_mode32(hipStream_t stream, const PrefillParams &p, int mode,
     {
         case NNTILE_HIP_MASK_ADDITIVE:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_ADDITIVE, SPLIT>), grid, dim3(kThreads32), 0,
+                        NNTILE_HIP_MASK_ADDITIVE, SPLIT>), grid, dim3(SPLIT ? split_waves32(HEAD) * 64 : kThreads32), 0,
                     stream, p);
             break;
         case NNTILE_HIP_MASK_NONE:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_NONE, SPLIT>), grid, dim3(kThreads32), 0,
+                        NNTILE_HIP_MASK_NONE, SPLIT>), grid, dim3(SPLIT ? split_waves32(HEAD) * 64 : kThreads32), 0,
                     stream, p);
             break;
         case NNTILE_HIP_MASK_CAUSAL:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_CAUSAL, SPLIT>), grid, dim3(kThreads32), 0,
+                        NNTILE_HIP_MASK_CAUSAL, SPLIT>), grid, dim3(SPLIT ? split_waves32(HEAD) * 64 : kThreads32), 0,
                     stream, p);
             break;
         case NNTILE_HIP_MASK_BOOL:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_BOOL, SPLIT>), grid, dim3(kThreads32), 0,
+                        NNTILE_HIP_MASK_BOOL, SPLIT>), grid, dim3(SPLIT ? split_waves32(HEAD) * 64 : kThreads32), 0,
                     stream, p);
             break;
         default:
