@@ -24,9 +24,9 @@
 //    the same two LDS tiles.
 //
 // K, V, Q, dA steps go from global memory straight into LDS, double buffered;
-// 16-byte chunk c of row r of a step sits at chunk position
-// c ^ ((r / RPL) % CPR), which keeps the row reads free of bank conflicts and
-// the transposing reads nearly so.
+// 16-byte chunk c of row r of a step sits at chunk position c ^ swz(r)
+// (BwdTile::swz), which keeps both the row reads and the transposing reads
+// free of bank conflicts.
 #include <type_traits>
 
 #include "sdpa_common.hpp"
@@ -38,6 +38,9 @@ namespace nntile_hip
 // the step, 1 = between the MFMAs of the step's first half, 2 = of the whole
 #ifndef NNTILE_BWD_SPREAD
 #define NNTILE_BWD_SPREAD 2
+#endif
+#ifndef NNTILE_BWD_SWIZZLE_ROTATED
+#define NNTILE_BWD_SWIZZLE_ROTATED 1
 #endif
 constexpr int kBwdRows = 128;       // queries (dQ workgroups) / keys (dK, dV workgroups) per workgroup
 constexpr int kBwdStep = 64;        // rows of the other axis per step
@@ -66,9 +69,23 @@ struct BwdTile
     static constexpr int BYTES = kBwdStep * RB;
     static_assert(LOADS_PER_WAVE >= 1, "head size does not fit this tiling");
 
+    // Chunk c of row r sits at chunk position c ^ swz(r).  Every tile is read
+    // both ways: 16 lanes read the same chunk of 16 consecutive rows (they
+    // need 16 different positions: swz must be one-to-one on 16 rows), and 32
+    // lanes of a transposing read take 4 neighbouring chunks of 4 consecutive
+    // rows (the 4 rows need different groups of 4 positions: the low bits of
+    // the line number must land in the top bits).  Both hold for the line
+    // number (r / RPL) % CPR rotated right by log2(CPR) - 2 bits.
     static __device__ __forceinline__ int swz(int r)
     {
-        return (r / RPL) % CPR;
+        constexpr int ROT = CPR == 16 ? 2 : (CPR == 8 ? 1 : 0);
+        constexpr int BITS = CPR == 16 ? 4 : (CPR == 8 ? 3 : 2);
+        const int line = (r / RPL) % CPR;
+#if NNTILE_BWD_SWIZZLE_ROTATED
+        return ((line >> ROT) | (line << (BITS - ROT))) & (CPR - 1);
+#else
+        return line;
+#endif
     }
 };
 
