@@ -220,7 +220,8 @@ def test_codelet_body(oracle):
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16"])
 @pytest.mark.parametrize("form", ["additive", "bool"])
-@pytest.mark.parametrize("q_seq,k_seq", [(256, 1024), (200, 712), (130, 333), (320, 192)])
+@pytest.mark.parametrize("q_seq,k_seq", [(256, 1024), (200, 712), (130, 333), (320, 192),
+                                         (70, 4200), (4200, 70)])     # more than 64 steps on one axis
 @pytest.mark.parametrize("pattern", ["band", "late_start", "holes", "all_hidden", "all_open"])
 @pytest.mark.parametrize("room", [True, False])
 def test_mask_block_classes(oracle, dtype, form, q_seq, k_seq, pattern, room):
