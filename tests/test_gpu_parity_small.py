@@ -378,7 +378,8 @@ def test_fp32_launch_forms(oracle, head, batch, q_seq, k_seq, k_tile, causal):
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16"])
 @pytest.mark.parametrize("form", ["additive", "bool"])
-@pytest.mark.parametrize("q_seq,k_seq", [(256, 1024), (200, 712), (128, 520), (130, 333)])
+@pytest.mark.parametrize("q_seq,k_seq", [(256, 1024), (200, 712), (128, 520), (130, 333),
+                                         (130, 4232)])      # more than 64 key steps: the last bit is shared
 @pytest.mark.parametrize("pattern", ["band", "late_start", "holes", "all_hidden", "all_open"])
 def test_explicit_mask_scan_paths(oracle, dtype, form, q_seq, k_seq, pattern):
     """Masks given as values are scanned once per workgroup: leading key steps
