@@ -31,6 +31,13 @@ namespace nntile_hip
 
 constexpr int kDecThreads = 256;  // 4 wavefronts x 16 query rows
 constexpr int kDecodeCUs = 256;   // MI355X
+// Ring stages and workgroups per CU the kernel is built for
+#ifndef NNTILE_DEC_STAGES
+#define NNTILE_DEC_STAGES 2
+#endif
+#ifndef NNTILE_DEC_WGS_PER_CU
+#define NNTILE_DEC_WGS_PER_CU 2
+#endif
 
 // Partial outputs of the key splits: 1 = normalised and in the tile type,
 // 0 = unnormalised fp32
@@ -72,7 +79,7 @@ template<int N> __device__ __forceinline__ void wait_vmcnt()
 }
 
 template<typename T, int HEAD, int MODE, int STAGES>
-__global__ __launch_bounds__(kDecThreads, 2)
+__global__ __launch_bounds__(kDecThreads, NNTILE_DEC_WGS_PER_CU)
 void sdpa_decode_16bit_kernel(const DecodeParams p)
 {
     typedef typename T::vec8 vec8;
@@ -681,7 +688,7 @@ static int launch_decode_stages(hipStream_t stream, const DecodeParams &p, int m
 template<typename T, int HEAD>
 static int launch_decode_head(hipStream_t stream, const DecodeParams &p, int mode)
 {
-    return launch_decode_stages<T, HEAD, 2>(stream, p, mode);
+    return launch_decode_stages<T, HEAD, NNTILE_DEC_STAGES>(stream, p, mode);
 }
 
 // Number of key splits per unit: two workgroups per CU when the units allow
@@ -689,7 +696,7 @@ static int launch_decode_head(hipStream_t stream, const DecodeParams &p, int mod
 // partials to write and merge.
 int decode_choose_splits(int units, int n_steps)
 {
-    int splits = (2 * kDecodeCUs + units - 1) / units;
+    int splits = (NNTILE_DEC_WGS_PER_CU * kDecodeCUs + units - 1) / units;
     splits = splits < 1 ? 1 : splits;
     splits = splits > n_steps ? n_steps : splits;
     splits = splits > 64 ? 64 : splits;
