@@ -483,6 +483,10 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(const BwdParams &p, unsigned wg
         {
             lim = min(lim, my_lim - kg0);
         }
+        // (wave-common: the last key of the step against the last key that
+        // exists and the last key the workgroup's first query sees)
+        const bool bounds = keys_here < kBwdStep
+            || (MODE == NNTILE_HIP_MASK_CAUSAL && kg0 + kBwdStep - 1 > rel + q_row0);
 #pragma unroll
         for(int mb = 0; mb < 2; ++mb)
         {
@@ -509,13 +513,24 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(const BwdParams &p, unsigned wg
                     }
                 }
             }
+            // Keys past the end and keys the causal mask hides: their scores
+            // become -inf in a pass of their own, which only the steps at the
+            // end of the keys and on the diagonal run (a wave-common branch).
+            if(bounds)
+            {
+#pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    const int key = mb * 32 + tile_row(r, half);
+                    sv[r] = key <= lim ? sv[r] : neg_inf();
+                }
+            }
             float dsv[16];
 #pragma unroll
             for(int r = 0; r < 16; ++r)
             {
-                const int key = mb * 32 + tile_row(r, half);
-                float e = fmaf(sv[r], c, -lse2);
-                bool visible = key <= lim;
+                float e = fmaf(sv[r], c, -lse2);        // -inf: hidden, or a row that saw nothing
+                bool visible = true;
                 if(use_mask)
                 {
                     // wave-common address of the step's first key in the
@@ -535,7 +550,7 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(const BwdParams &p, unsigned wg
                         visible = visible && (shown != 0);
                     }
                 }
-                const float pr = visible ? fast_exp2(e) : 0.0f;
+                const float pr = use_mask ? (visible ? fast_exp2(e) : 0.0f) : fast_exp2(e);
                 dsv[r] = pr * (dpv[r] - d_row);
             }
             uint32_t ds_pk[8];
@@ -879,6 +894,10 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(const BwdParams &p, unsigned w
         constexpr bool use_mask = EXPLICIT && decltype(masked_tag)::value;
         const int q0 = qs * kBwdStep;
         const int rows_here = min(kBwdStep, q_seq - q0);
+        // (wave-common: the workgroup's last key against the last key that
+        // exists and the last key the step's first query sees)
+        const bool bounds = k_row0 + kDkvRows > k_seq
+            || (MODE == NNTILE_HIP_MASK_CAUSAL && k_row0 + kDkvRows - 1 > rel + q0);
         const char *mask_step = static_cast<const char *>(p.mask)
             + (int64_t)q0 * (int64_t)mask_row_bytes;
         const uint32_t mask_last_row = (uint32_t)(rows_here - 1) * mask_row_bytes;
@@ -921,6 +940,24 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(const BwdParams &p, unsigned w
                     }
                 }
             }
+            // Keys past the end and pairs the causal mask hides: their scores
+            // become -inf in a pass of their own, which only the workgroups at
+            // the end of the keys and the steps on the diagonal run (a
+            // wave-common branch).
+            if(bounds)
+            {
+#pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    const int qr = mb * 32 + tile_row(r, half);
+                    bool vis = k_ok;
+                    if(MODE == NNTILE_HIP_MASK_CAUSAL)
+                    {
+                        vis = vis && (my_k <= rel + q0 + qr);
+                    }
+                    sv[r] = vis ? sv[r] : neg_inf();
+                }
+            }
             float pv[16], dsv[16];
 #pragma unroll
             for(int rg = 0; rg < 4; ++rg)
@@ -933,13 +970,8 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(const BwdParams &p, unsigned w
                 for(int e = 0; e < 4; ++e)
                 {
                     const int r = 4 * rg + e;
-                    const int qr = qr0 + e;                 // query row within the step
-                    float ex = fmaf(sv[r], c, -lse4[e]);    // -inf for rows past the end
-                    bool visible = k_ok;
-                    if(MODE == NNTILE_HIP_MASK_CAUSAL)
-                    {
-                        visible = visible && (my_k <= rel + q0 + qr);
-                    }
+                    float ex = fmaf(sv[r], c, -lse4[e]);    // -inf: hidden, or a row past the end
+                    bool visible = true;
                     if(use_mask)
                     {
                         // the row is the same for the lanes of one half: its
@@ -964,7 +996,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(const BwdParams &p, unsigned w
                         visible = visible && (shown != 0);
                         }
                     }
-                    pv[r] = visible ? fast_exp2(ex) : 0.0f;
+                    pv[r] = use_mask ? (visible ? fast_exp2(ex) : 0.0f) : fast_exp2(ex);
                     dsv[r] = pv[r] * (dpv[r] - d4[e]);
                 }
             }
