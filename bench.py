@@ -256,6 +256,56 @@ def bench_transpose(cfg, steps, warmup):
             "frac_of_hbm_peak": round(nbytes / (dev * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
 
 
+def bench_kv_cache(cfg, steps, warmup):
+    """One decode step through a preallocated key/value cache: the keys and
+    values of the q_seq new tokens are appended (one launch for both), then
+    the decode kernel reads the filled rows of the caches where they lie.  The
+    caches hold twice the filled rows (capacity 2 x k_seq); four cache pairs
+    rotate, as in the decode leg.  The reference's step copies the filled part
+    of both caches out first (cache_utils.py:177-215): twice the bytes of the
+    attention itself, which this path does not move."""
+    import torch
+    from nntile_amd import hip_sdpa as h
+    kvb = cfg.n_batch * cfg.n_head_kv
+    cap, nrot = 2 * cfg.k_seq, 4
+    Ks = [_randn((kvb, cap, cfg.head), torch.bfloat16, cfg.seed * 1000 + 300 + i) for i in range(nrot)]
+    Vs = [_randn((kvb, cap, cfg.head), torch.bfloat16, cfg.seed * 1000 + 350 + i) for i in range(nrot)]
+    k_new = _randn((kvb, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed * 1000 + 398)
+    v_new = _randn((kvb, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed * 1000 + 399)
+    Q = _randn((cfg.batch_flat, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed * 1000 + 99)
+    A = torch.zeros_like(Q)
+    lse = torch.full((cfg.batch_flat, cfg.q_seq), float("-inf"), device="cuda")
+    ws = torch.empty(h.decode_cache_workspace_bytes(cfg.k_seq, Q, cfg.n_batch, cfg.kv_group),
+                     dtype=torch.uint8, device="cuda")
+    plans = [h.plan_decode_cache(Ks[j], Vs[j], cfg.k_seq, Q, None, lse, A, h.MASK_CAUSAL,
+                                 cfg.n_batch, cfg.kv_group, ws, causal_offset=cfg.causal_offset,
+                                 flags=h.OVERWRITE) for j in range(nrot)]
+    filled = cfg.k_seq - cfg.q_seq
+    i = [0]
+
+    def step():
+        j = i[0] % nrot
+        h.kv_cache_append(k_new, v_new, Ks[j], Vs[j], filled)
+        plans[j].launch()
+        i[0] += 1
+
+    def append_only():
+        h.kv_cache_append(k_new, v_new, Ks[i[0] % nrot], Vs[i[0] % nrot], filled)
+        i[0] += 1
+
+    wall, dev = time_steps(step, steps, warmup)
+    _, dev_append = time_steps(append_only, steps, 2)
+    append_bytes = 2 * 2 * k_new.numel() * k_new.element_size()
+    nbytes = cfg.algorithmic_bytes() + append_bytes
+    return {"what": "append %d new tokens + decode over %d cached rows of %s, cache capacity %d"
+                    % (cfg.q_seq, cfg.k_seq, cfg.name, cap),
+            "ms_per_step": round(wall, 4), "device_ms_per_step": round(dev, 4),
+            "append_device_ms": round(dev_append, 4), "algorithmic_bytes": nbytes,
+            "gbs": round(nbytes / (dev * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(nbytes / (dev * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+            "reference_copy_out_bytes_not_moved": 2 * 2 * kvb * cfg.k_seq * cfg.head * 2}
+
+
 def cpu_baseline(cfg, target_seconds=15.0):
     """The CPU checker (port of the reference's gemm -> mask_scalar ->
     maxsumexp -> softmax_inplace -> gemm composition) on a bounded sample of
@@ -294,7 +344,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run only this leg: prefill | decode | per_task | backward | rope | transpose | extras | copy (for profiling)")
+                    help="run only this leg: prefill | decode | per_task | backward | rope | transpose | kv_cache | extras | copy (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
@@ -340,6 +390,9 @@ def main():
     if only == "rope":
         print(json.dumps(bench_rope(cfg3, args.steps, args.warmup)))
         return
+    if only == "kv_cache":
+        print(json.dumps(bench_kv_cache(cfg4, args.steps, args.warmup)))
+        return
     if only == "extras":
         for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):
             bench_prefill(BY_NAME[name], args.steps, args.warmup)
@@ -361,6 +414,7 @@ def main():
     backward = bench_backward(cfg3, max(5, args.steps // 10), 2)
     rope = bench_rope(cfg3, max(5, args.steps // 5), 5)
     transpose = bench_transpose(cfg3, max(5, args.steps // 5), 5)
+    kv_cache = bench_kv_cache(cfg4, max(5, args.steps // 5), 5)
     # The headline leg runs last: the first timed loop of a process measures
     # 5 % slower than the same loop a second later (clocks still settling),
     # whatever the warmup count.
@@ -409,6 +463,7 @@ def main():
         "backward": backward,
         "rope": rope,
         "transpose": transpose,
+        "kv_cache": kv_cache,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg3)

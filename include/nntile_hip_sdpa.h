@@ -306,6 +306,41 @@ int nntile_hip_transpose_fp16(void *stream, int64_t m, int64_t n, float alpha,
 int nntile_hip_transpose_fp32(void *stream, int64_t m, int64_t n, float alpha,
         const float *src, float *dst);
 
+/* ---- 9. key/value cache of the decode path -----------------------------------
+ * Replaces KVCache.append (wrappers/python/nntile/layer/cache_utils.py:
+ * 146-175: two copy_intersection_async calls into tensors preallocated with
+ * max_cache_size rows on the sequence axis) for caches of shape
+ * [head, capacity, n_batch, n_head_kv]: the rows of k_new and v_new
+ * ([head, rows, n_batch, n_head_kv], entries = n_batch*n_head_kv) are written
+ * behind the `filled` rows that each entry of k_cache / v_cache already
+ * holds, both tensors in one launch.  rows > capacity - filled is
+ * NNTILE_HIP_EINVAL, the condition on which LlamaAttention._append_to_kv_cache
+ * raises (wrappers/python/nntile/model/llama_attention.py:524-529); nothing
+ * is written then.  rows == 0 is a no-op. */
+int nntile_hip_kv_cache_append_bf16(void *stream, int64_t head, int64_t rows, int64_t entries,
+        int64_t capacity, int64_t filled, const uint16_t *k_new, const uint16_t *v_new,
+        uint16_t *k_cache, uint16_t *v_cache);
+int nntile_hip_kv_cache_append_fp16(void *stream, int64_t head, int64_t rows, int64_t entries,
+        int64_t capacity, int64_t filled, const uint16_t *k_new, const uint16_t *v_new,
+        uint16_t *k_cache, uint16_t *v_cache);
+int nntile_hip_kv_cache_append_fp32(void *stream, int64_t head, int64_t rows, int64_t entries,
+        int64_t capacity, int64_t filled, const float *k_new, const float *v_new,
+        float *k_cache, float *v_cache);
+
+/* nntile_hip_sdpa_fwd_decode_* reading such a cache where it lies: args->K and
+ * args->V point at the caches, args->k_seq is the number of filled rows and
+ * `capacity` (>= k_seq) the rows between two entries.  This stands for the
+ * k_partial / v_partial copies of the filled part that the reference makes
+ * before every attention call (cache_utils.py:177-215) and, with
+ * NNTILE_HIP_MASK_CAUSAL and causal_offset = k_seq - q_seq, for the bool mask
+ * that Sdpa._prepare_mask_for_kv_cache materialises
+ * (wrappers/python/nntile/layer/sdpa.py:489-531).  Workspace as for
+ * nntile_hip_sdpa_fwd_decode_* (its size does not depend on capacity). */
+int nntile_hip_sdpa_fwd_decode_cache_bf16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity, void *workspace, size_t workspace_bytes);
+int nntile_hip_sdpa_fwd_decode_cache_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity, void *workspace, size_t workspace_bytes);
+
 /* Library version and the ISA it was built for ("gfx950"). */
 const char *nntile_hip_sdpa_version(void);
 

@@ -33,6 +33,10 @@ int launch_rope(hipStream_t stream, int dtype, bool backward, int64_t m, int64_t
 int launch_transpose(hipStream_t stream, int dtype, int64_t m, int64_t n, float alpha,
         const void *src, void *dst);
 
+int launch_kv_cache_append(hipStream_t stream, int elem, int64_t head, int64_t rows,
+        int64_t entries, int64_t capacity, int64_t filled, const void *k_new,
+        const void *v_new, void *k_cache, void *v_cache);
+
 enum class DType { bf16, fp16, fp32 };
 
 static bool aligned16(const void *p)
@@ -322,9 +326,9 @@ static void decode_geometry(const nntile_hip_sdpa_tile_args *a, int &units,
 }
 
 static int decode_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a,
-        void *workspace, size_t workspace_bytes)
+        int64_t kv_rows, void *workspace, size_t workspace_bytes)
 {
-    if(!decode_args_ok(a) || !mode_ok(a->mask_mode) || a->K == nullptr
+    if(!decode_args_ok(a) || kv_rows < a->k_seq || !mode_ok(a->mask_mode) || a->K == nullptr
             || a->Q == nullptr || a->V == nullptr || a->lse == nullptr
             || a->A == nullptr || !aligned16(a->K) || !aligned16(a->Q)
             || !aligned16(a->V) || !aligned16(a->A))
@@ -352,6 +356,7 @@ static int decode_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *
     std::memset(&p, 0, sizeof(p));
     p.q_seq = a->q_seq;
     p.k_seq = a->k_seq;
+    p.kv_rows = kv_rows;
     p.q_pos0 = a->q_pos0;
     p.k_pos0 = a->k_pos0;
     p.causal_offset = a->causal_offset;
@@ -436,6 +441,33 @@ static int transpose_call(DType dt, void *stream, int64_t m, int64_t n, float al
     }
     const int code = dt == DType::bf16 ? 0 : (dt == DType::fp16 ? 1 : 2);
     return launch_transpose(static_cast<hipStream_t>(stream), code, m, n, alpha, src, dst);
+}
+
+static int kv_append_call(int elem, void *stream, int64_t head, int64_t rows, int64_t entries,
+        int64_t capacity, int64_t filled, const void *k_new, const void *v_new, void *k_cache,
+        void *v_cache)
+{
+    if(head <= 0 || rows < 0 || entries < 0 || capacity <= 0 || filled < 0)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(rows > capacity - filled)
+    {
+        // LlamaAttention._append_to_kv_cache raises here
+        // (wrappers/python/nntile/model/llama_attention.py:524-529)
+        return NNTILE_HIP_EINVAL;
+    }
+    if(rows == 0 || entries == 0)
+    {
+        return NNTILE_HIP_OK;
+    }
+    if(k_new == nullptr || v_new == nullptr || k_cache == nullptr || v_cache == nullptr
+            || entries > (int64_t)0x0fffffffffffffff / (capacity * head))
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    return launch_kv_cache_append(static_cast<hipStream_t>(stream), elem, head, rows, entries,
+            capacity, filled, k_new, v_new, k_cache, v_cache);
 }
 
 static nntile_hip_stream_provider g_stream_provider = nullptr;
@@ -590,13 +622,15 @@ size_t nntile_hip_sdpa_fwd_decode_workspace_bytes(const nntile_hip_sdpa_tile_arg
 int nntile_hip_sdpa_fwd_decode_bf16(void *stream, const nntile_hip_sdpa_tile_args *args,
         void *workspace, size_t workspace_bytes)
 {
-    return decode_call(DType::bf16, stream, args, workspace, workspace_bytes);
+    return decode_call(DType::bf16, stream, args, args ? args->k_seq : 0, workspace,
+            workspace_bytes);
 }
 
 int nntile_hip_sdpa_fwd_decode_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
         void *workspace, size_t workspace_bytes)
 {
-    return decode_call(DType::fp16, stream, args, workspace, workspace_bytes);
+    return decode_call(DType::fp16, stream, args, args ? args->k_seq : 0, workspace,
+            workspace_bytes);
 }
 
 int nntile_hip_accumulate_attn_output_bf16(void *stream, int64_t head, int64_t seq,
@@ -731,6 +765,42 @@ int nntile_hip_transpose_fp32(void *stream, int64_t m, int64_t n, float alpha,
         const float *src, float *dst)
 {
     return transpose_call(DType::fp32, stream, m, n, alpha, src, dst);
+}
+
+int nntile_hip_kv_cache_append_bf16(void *stream, int64_t head, int64_t rows, int64_t entries,
+        int64_t capacity, int64_t filled, const uint16_t *k_new, const uint16_t *v_new,
+        uint16_t *k_cache, uint16_t *v_cache)
+{
+    return kv_append_call(2, stream, head, rows, entries, capacity, filled, k_new, v_new,
+            k_cache, v_cache);
+}
+
+int nntile_hip_kv_cache_append_fp16(void *stream, int64_t head, int64_t rows, int64_t entries,
+        int64_t capacity, int64_t filled, const uint16_t *k_new, const uint16_t *v_new,
+        uint16_t *k_cache, uint16_t *v_cache)
+{
+    return kv_append_call(2, stream, head, rows, entries, capacity, filled, k_new, v_new,
+            k_cache, v_cache);
+}
+
+int nntile_hip_kv_cache_append_fp32(void *stream, int64_t head, int64_t rows, int64_t entries,
+        int64_t capacity, int64_t filled, const float *k_new, const float *v_new,
+        float *k_cache, float *v_cache)
+{
+    return kv_append_call(4, stream, head, rows, entries, capacity, filled, k_new, v_new,
+            k_cache, v_cache);
+}
+
+int nntile_hip_sdpa_fwd_decode_cache_bf16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity, void *workspace, size_t workspace_bytes)
+{
+    return decode_call(DType::bf16, stream, args, capacity, workspace, workspace_bytes);
+}
+
+int nntile_hip_sdpa_fwd_decode_cache_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity, void *workspace, size_t workspace_bytes)
+{
+    return decode_call(DType::fp16, stream, args, capacity, workspace, workspace_bytes);
 }
 
 const char *nntile_hip_sdpa_version(void)

@@ -63,6 +63,7 @@ struct PrefillParams
 struct DecodeParams
 {
     int64_t q_seq, k_seq;
+    int64_t kv_rows;    // rows between two entries of K and V (k_seq, or a cache's capacity)
     int64_t q_pos0, k_pos0, causal_offset;
     int64_t mask_ld;
     const void *mask;

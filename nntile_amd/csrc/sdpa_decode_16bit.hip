@@ -150,8 +150,8 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         }
     }
 
-    const char *Kb = static_cast<const char *>(p.K) + (int64_t)unit * p.k_seq * RB;
-    const char *Vb = static_cast<const char *>(p.V) + (int64_t)unit * p.k_seq * RB;
+    const char *Kb = static_cast<const char *>(p.K) + (int64_t)unit * p.kv_rows * RB;
+    const char *Vb = static_cast<const char *>(p.V) + (int64_t)unit * p.kv_rows * RB;
 
     // ---- LDS layout and the lane's fixed addresses ---------------------------
     // chunk c of row r sits at chunk position

@@ -87,6 +87,8 @@ EXPORTS = (
     + ["nntile_hip_rope_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_rope_backward_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_transpose_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_kv_cache_append_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_sdpa_fwd_decode_cache_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_set_stream_provider", "nntile_hip_sdpa_version"])
 
 _lib = None
@@ -120,6 +122,9 @@ def lib():
             f = getattr(L, "nntile_hip_sdpa_fwd_decode_" + t)
             f.argtypes = [_vp, ctypes.POINTER(TileArgs), _vp, ctypes.c_size_t]
             f.restype = ctypes.c_int
+            f = getattr(L, "nntile_hip_sdpa_fwd_decode_cache_" + t)
+            f.argtypes = [_vp, ctypes.POINTER(TileArgs), _i64, _vp, ctypes.c_size_t]
+            f.restype = ctypes.c_int
             f = getattr(L, "nntile_hip_flash_sdpa_bwd_" + t)
             f.argtypes = [_vp, _i64, _i64, _i64] + [_vp] * 13
             f.restype = ctypes.c_int
@@ -137,6 +142,9 @@ def lib():
         for t in ("bf16", "fp16", "fp32"):
             f = getattr(L, "nntile_hip_transpose_" + t)
             f.argtypes = [_vp, _i64, _i64, ctypes.c_float, _vp, _vp]
+            f.restype = ctypes.c_int
+            f = getattr(L, "nntile_hip_kv_cache_append_" + t)
+            f.argtypes = [_vp] + [_i64] * 5 + [_vp] * 4
             f.restype = ctypes.c_int
         L.nntile_hip_sdpa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
         L.nntile_hip_sdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
@@ -373,6 +381,62 @@ def sdpa_fwd_decode(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group,
     nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _check(fn(_stream(stream), ctypes.byref(a), _ptr(workspace), nbytes),
            "sdpa_fwd_decode")
+
+
+def kv_cache_append(k_new, v_new, k_cache, v_cache, filled, stream=None):
+    """Write k_new, v_new ([entries, rows, head]) behind the `filled` rows of
+    k_cache, v_cache ([entries, capacity, head])."""
+    _dev(k_new, v_new, k_cache, v_cache)
+    entries, rows, head = k_new.shape
+    if (tuple(v_new.shape) != (entries, rows, head) or k_cache.shape != v_cache.shape
+            or k_cache.shape[0] != entries or k_cache.shape[2] != head):
+        raise SdpaError(EINVAL, "kv_cache_append")
+    fn = getattr(lib(), "nntile_hip_kv_cache_append_" + dtype_name(k_cache))
+    _check(fn(_stream(stream), head, rows, entries, k_cache.shape[1], filled, _ptr(k_new),
+              _ptr(v_new), _ptr(k_cache), _ptr(v_cache)), "kv_cache_append")
+
+
+def _cache_args(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch, kv_group, q_pos0,
+                k_pos0, causal_offset, flags):
+    a = _tile_args(K_cache, Q, mask, lse, V_cache, A, mask_mode, n_batch, kv_group, q_pos0,
+                   k_pos0, causal_offset, flags)
+    a.k_seq = k_seq
+    return a
+
+
+def sdpa_fwd_decode_cache(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch,
+                          kv_group, workspace, q_pos0=0, k_pos0=0, causal_offset=0, flags=0,
+                          stream=None):
+    """sdpa_fwd_decode over the first k_seq rows of every entry of the caches
+    ([n_head_kv*n_batch, capacity, head]), read where they lie."""
+    _dev(K_cache, V_cache, Q, mask, lse, A, workspace)
+    if K_cache.shape != V_cache.shape:
+        raise SdpaError(EINVAL, "sdpa_fwd_decode_cache")
+    a = _cache_args(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch, kv_group,
+                    q_pos0, k_pos0, causal_offset, flags)
+    fn = getattr(lib(), "nntile_hip_sdpa_fwd_decode_cache_" + dtype_name(Q))
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _check(fn(_stream(stream), ctypes.byref(a), K_cache.shape[1], _ptr(workspace), nbytes),
+           "sdpa_fwd_decode_cache")
+
+
+def plan_decode_cache(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch, kv_group,
+                      workspace, q_pos0=0, k_pos0=0, causal_offset=0, flags=0):
+    _dev(K_cache, V_cache, Q, mask, lse, A, workspace)
+    a = _cache_args(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch, kv_group,
+                    q_pos0, k_pos0, causal_offset, flags)
+    fn = getattr(lib(), "nntile_hip_sdpa_fwd_decode_cache_" + dtype_name(Q))
+    nbytes = workspace.numel() * workspace.element_size()
+    return Plan(fn, a, "sdpa_fwd_decode_cache",
+                extra=(K_cache.shape[1], _ptr(workspace), nbytes),
+                keep=(K_cache, V_cache, Q, mask, lse, A, workspace))
+
+
+def decode_cache_workspace_bytes(k_seq, Q, n_batch, kv_group):
+    a = TileArgs()
+    a.batch, a.q_seq, a.head = Q.shape
+    a.k_seq, a.n_batch, a.kv_group = k_seq, n_batch, kv_group
+    return int(lib().nntile_hip_sdpa_fwd_decode_workspace_bytes(ctypes.byref(a)))
 
 
 def accumulate_attn_output(src_lse, src_attn, dst_lse, dst_attn, stream=None):

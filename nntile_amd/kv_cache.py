@@ -1,0 +1,93 @@
+"""Key/value cache of the decode path, on the HIP entry points.
+
+Mirror of `KVCache` (wrappers/python/nntile/layer/cache_utils.py:117-225) and
+of the way `LlamaAttention.forward_dynamic` uses it
+(wrappers/python/nntile/model/llama_attention.py:518-531, 643-731): tensors
+preallocated with `max_cache_size` rows on the sequence axis, `append` writes
+the new rows behind the filled ones, `len()` is the number of filled rows.
+
+What differs, on purpose: the reference copies the filled part of both caches
+into fresh dense tensors before every attention call (`k_partial`,
+`v_partial`) and materialises a bool mask slice for the new queries; here
+`attend` hands the caches to the decode kernel with their capacity and the
+visibility rule `key <= query + (len - q_seq)`, so a decode step reads the
+filled rows once and writes only the new ones.
+
+Tensors are C-ordered torch device tensors: K, V `[entries, seq, head]`
+(entries = n_batch * n_head_kv, NNTile's `[head, seq, n_batch, n_head_kv]`),
+Q, A `[entries * kv_group, q_seq, head]`.
+"""
+import torch
+
+from . import hip_sdpa
+
+
+class KVCache:
+    def __init__(self, max_cache_size, seq_size_dim=1):
+        if seq_size_dim != 1:
+            # [head, seq, ...] is the only layout the attention path uses
+            raise ValueError("the sequence axis of an attention tile is axis 1")
+        self.max_cache_size = int(max_cache_size)
+        self.seq_size_dim = seq_size_dim
+        self.k = None
+        self.v = None
+        self.k_cache_size = 0
+        self.v_cache_size = 0
+        self._workspace = None
+
+    def __len__(self):
+        return self.k_cache_size
+
+    def _init_from_tensor(self, t):
+        entries, _, head = t.shape
+        return torch.zeros((entries, self.max_cache_size, head), dtype=t.dtype, device=t.device)
+
+    def append(self, k_partial, v_partial, stream=None):
+        """Write the new rows behind the filled ones.  More rows than the cache
+        has left raise (the reference raises in
+        LlamaAttention._append_to_kv_cache); nothing is written then."""
+        if k_partial.shape[1] != v_partial.shape[1]:
+            raise ValueError("k and v must bring the same number of tokens")
+        if self.k is None:
+            self.k = self._init_from_tensor(k_partial)
+            self.v = self._init_from_tensor(v_partial)
+        rows = k_partial.shape[1]
+        if rows + self.k_cache_size > self.max_cache_size:
+            raise hip_sdpa.SdpaError(
+                hip_sdpa.EINVAL,
+                "kv_cache_append: overload internal state: try add %d to %d, max: %d"
+                % (rows, self.k_cache_size, self.max_cache_size))
+        hip_sdpa.kv_cache_append(k_partial, v_partial, self.k, self.v, self.k_cache_size,
+                                 stream=stream)
+        self.k_cache_size += rows
+        self.v_cache_size += rows
+
+    @property
+    def k_partial(self):
+        """The filled rows, as a view (the reference returns a copy)."""
+        return self.k[:, :self.k_cache_size]
+
+    @property
+    def v_partial(self):
+        return self.v[:, :self.v_cache_size]
+
+    def clear(self):
+        self.k = None
+        self.v = None
+        self.k_cache_size = 0
+        self.v_cache_size = 0
+        self._workspace = None
+
+    def attend(self, Q, lse, A, n_batch, kv_group, causal=True, stream=None):
+        """A = attention of Q over the filled rows; the q_seq queries are the
+        last q_seq tokens of the cache (append first).  lse and A are
+        overwritten."""
+        k_seq = len(self)
+        q_seq = Q.shape[1]
+        need = hip_sdpa.decode_cache_workspace_bytes(k_seq, Q, n_batch, kv_group)
+        if self._workspace is None or self._workspace.numel() < need:
+            self._workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
+        mode = hip_sdpa.MASK_CAUSAL if causal else hip_sdpa.MASK_NONE
+        hip_sdpa.sdpa_fwd_decode_cache(
+            self.k, self.v, k_seq, Q, None, lse, A, mode, n_batch, kv_group, self._workspace,
+            causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)

@@ -325,3 +325,91 @@ def transpose(m, n, alpha, src):
     order, the product in fp32.  Returns the flat float32 dst."""
     x = np.asarray(src, np.float32).reshape(n, m)      # x[j, i] = src(i, j)
     return (np.float32(alpha) * np.ascontiguousarray(x.T)).reshape(-1)
+
+
+# ---- key/value cache of the decode path --------------------------------------
+
+def copy_intersection(src, src_offset, dst, dst_offset):
+    """dst <- src where the two overlap, both placed in one global index space
+    at their offsets (src/tensor/copy_intersection.cc:84-112; the tile loop
+    behind it only distributes the same copy).  Arrays are indexed in the
+    reference's axis order (numpy arrays whose axis i is the reference's axis
+    i).  dst is changed in place and returned."""
+    sl_s, sl_d = [], []
+    for n_s, o_s, n_d, o_d in zip(src.shape, src_offset, dst.shape, dst_offset):
+        if o_s + n_s <= o_d or o_d + n_d <= o_s:
+            return dst
+        if o_s < o_d:
+            s0, d0 = o_d - o_s, 0
+            n = min(n_s - s0, n_d)
+        else:
+            s0, d0 = 0, o_s - o_d
+            n = min(n_d - d0, n_s)
+        sl_s.append(slice(s0, s0 + n))
+        sl_d.append(slice(d0, d0 + n))
+    dst[tuple(sl_d)] = src[tuple(sl_s)]
+    return dst
+
+
+class KVCache:
+    """KVCache of wrappers/python/nntile/layer/cache_utils.py:117-225 on numpy
+    arrays in the reference's axis order ([head, seq, ...]): zeros of
+    max_cache_size rows on the sequence axis, append at the filled size,
+    k_partial / v_partial copy the filled part out."""
+
+    def __init__(self, max_cache_size, seq_size_dim):
+        self.max_cache_size, self.seq_size_dim = max_cache_size, seq_size_dim
+        self.k = self.v = None
+        self.k_cache_size = self.v_cache_size = 0
+
+    def __len__(self):
+        return self.k_cache_size
+
+    def _zeros_like_cache(self, t):
+        shape = list(t.shape)
+        shape[self.seq_size_dim] = self.max_cache_size
+        return np.zeros(shape, t.dtype)
+
+    def append(self, k_partial, v_partial):
+        assert k_partial.shape[self.seq_size_dim] == v_partial.shape[self.seq_size_dim]
+        if self.k is None:
+            self.k = self._zeros_like_cache(k_partial)
+        off = [0] * k_partial.ndim
+        off[self.seq_size_dim] = self.k_cache_size
+        copy_intersection(k_partial, off, self.k, [0] * self.k.ndim)
+        self.k_cache_size += k_partial.shape[self.seq_size_dim]
+        if self.v is None:
+            self.v = self._zeros_like_cache(v_partial)
+        off = [0] * v_partial.ndim
+        off[self.seq_size_dim] = self.v_cache_size
+        copy_intersection(v_partial, off, self.v, [0] * self.v.ndim)
+        self.v_cache_size += v_partial.shape[self.seq_size_dim]
+
+    def _partial(self, full, size):
+        shape = list(full.shape)
+        shape[self.seq_size_dim] = size
+        out = np.empty(shape, full.dtype)
+        return copy_intersection(full, [0] * full.ndim, out, [0] * out.ndim)
+
+    @property
+    def k_partial(self):
+        return self._partial(self.k, self.k_cache_size)
+
+    @property
+    def v_partial(self):
+        return self._partial(self.v, self.v_cache_size)
+
+
+def prepare_mask_for_kv_cache(mask, k_seq, q_seq):
+    """The bool mask slice that goes with cached keys
+    (wrappers/python/nntile/layer/sdpa.py:489-531).  mask: bool in the
+    reference's axis order [keys, queries] (True = visible).  A mask that
+    already has shape (k_seq, q_seq) is used as it is; otherwise ones of that
+    shape, overwritten by the mask placed at [0, 0] against a destination
+    placed at [0, k_seq - q_seq]: query column j takes the mask column of the
+    token at position j + k_seq - q_seq."""
+    mask = np.asarray(mask, bool)
+    if mask.shape == (k_seq, q_seq):
+        return mask
+    out = np.ones((k_seq, q_seq), bool)
+    return copy_intersection(mask, [0, 0], out, [0, k_seq - q_seq])
