@@ -69,11 +69,15 @@ def _randn(shape, dtype, seed):
     return torch.randn(shape, generator=g, device="cuda", dtype=torch.float32).to(dtype)
 
 
-def bench_prefill(cfg, steps, warmup, per_task=False):
+def bench_prefill(cfg, steps, warmup, per_task=False, classified=False):
     """Fused: one launch for the whole tile grid (analytic causal mask, tile
     skipping).  per_task: the reference's task structure - one launch per
     (query tile, key tile) pair with a materialised additive mask tile, no
-    skipping, (lse, A) handed over in memory between launches."""
+    skipping, (lse, A) handed over in memory between launches.
+    classified (with per_task): the mask tiles are classified once, outside the
+    timed region, as a layer would when it builds its mask; pairs whose tile
+    hides everything are not launched, open and causal ones run without
+    reading the mask."""
     import torch
     from nntile_amd import hip_sdpa as h, synth
     dt = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[cfg.dtype]
@@ -102,12 +106,25 @@ def bench_prefill(cfg, steps, warmup, per_task=False):
 
     # Calls are prepared once (tile addresses do not change between steps).
     plans = []
+    classes = None
+    if per_task and classified:
+        t = cfg.seq_tile
+        classes = [[h.mask_tile_class(masks[qi][ki], (qi - ki) * t) for ki in range(nt)]
+                   for qi in range(nt)]
     for Q, K, V, A, lse in calls:
         if per_task:
             for qi in range(nt):
                 for ki in range(nt):
-                    plans.append(h.plan_tile(K[ki], Q[qi], masks[qi][ki], lse[qi], V[ki], A[qi],
-                                             h.MASK_ADDITIVE))
+                    cls = h.TILE_MIXED if classes is None else classes[qi][ki]
+                    if cls == h.TILE_HIDDEN:
+                        continue
+                    if cls == h.TILE_MIXED:
+                        plans.append(h.plan_tile(K[ki], Q[qi], masks[qi][ki], lse[qi], V[ki],
+                                                 A[qi], h.MASK_ADDITIVE))
+                    else:
+                        mode = h.MASK_NONE if cls == h.TILE_OPEN else h.MASK_CAUSAL
+                        plans.append(h.plan_tile(K[ki], Q[qi], None, lse[qi], V[ki], A[qi], mode,
+                                                 q_pos0=qi * cfg.seq_tile, k_pos0=ki * cfg.seq_tile))
         else:
             plans.append(h.plan_grid(K, Q, lse, V, A, cfg.q_seq, cfg.k_seq, cfg.seq_tile,
                                      cfg.seq_tile, h.MASK_CAUSAL, flags=h.OVERWRITE))
@@ -127,7 +144,7 @@ def bench_prefill(cfg, steps, warmup, per_task=False):
     wall, dev = time_steps(step, steps, warmup)
     reset()
     _, kdev = time_steps(kernels_only, steps, 2)
-    launches = cfg.calls * (nt * nt if per_task else 1)
+    launches = len(plans)
     return {"ms_per_step": wall, "device_ms_per_step": dev, "kernel_ms_per_step": kdev,
             "launches_per_step": launches,
             "tflops": cfg.flops() / (wall * 1e-3) / 1e12,
@@ -366,6 +383,10 @@ def main():
     if only == "prefill":
         bench_prefill(cfg3, args.steps, args.warmup)
         return
+    if only == "per_task_classified":
+        r = bench_prefill(cfg3, args.steps, args.warmup, per_task=True, classified=True)
+        print(json.dumps({k: round(v, 4) for k, v in r.items()}))
+        return
     if only == "per_task":
         bench_prefill(cfg3, args.steps, args.warmup, per_task=True)
         return
@@ -400,6 +421,7 @@ def main():
 
     dec = bench_decode(cfg4, args.steps, args.warmup)
     per_task = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True)
+    per_task_cls = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True, classified=True)
     extras = {}
     for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):
         c = BY_NAME[name]
@@ -459,6 +481,12 @@ def main():
                                   "tiles, no skipping, (lse, A) handed over in bf16",
                           "ms_per_step": round(per_task["ms_per_step"], 4),
                           "tflops": round(per_task["tflops"], 2)},
+        "per_task_classified": {"what": "the same 16 tile pairs with the mask tiles classified once: "
+                                        "hidden pairs not launched, open and causal ones without "
+                                        "reading the mask",
+                                "launches_per_step": per_task_cls["launches_per_step"],
+                                "ms_per_step": round(per_task_cls["ms_per_step"], 4),
+                                "tflops": round(per_task_cls["tflops"], 2)},
         "other_configs": extras,
         "backward": backward,
         "rope": rope,

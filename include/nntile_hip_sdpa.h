@@ -341,6 +341,35 @@ int nntile_hip_sdpa_fwd_decode_cache_bf16(void *stream, const nntile_hip_sdpa_ti
 int nntile_hip_sdpa_fwd_decode_cache_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
         int64_t capacity, void *workspace, size_t workspace_bytes);
 
+/* ---- 10. class of a mask tile -------------------------------------------------
+ * For the layer that submits one task per (query tile, key tile) pair with
+ * the pair's mask tile (src/tensor/flash_sdpa_fwd_cudnn.cc:246-274, which
+ * submits every pair): reads one tile of a materialised mask - [k_rows,
+ * q_cols] in Fortran order, additive in the tile type (0 visible, -inf
+ * hidden) or bool (nonzero visible) - and tells whether the pair needs a task
+ * and whether that task needs the mask:
+ *   HIDDEN  every element hidden: the pair leaves (lse, A) as they are
+ *   OPEN    every element visible: NNTILE_HIP_MASK_NONE gives the same result
+ *   CAUSAL  visible exactly where k <= q + offset (k, q counted inside the
+ *           tile): NNTILE_HIP_MASK_CAUSAL with causal_offset = offset does
+ *   MIXED   anything else, additive values other than 0 and -inf included:
+ *           the mask must be passed
+ * Blocking: synchronises the stream and writes *class_out on the host.  A
+ * mask is classified once and the classes kept with it; workspace is one
+ * 4-byte aligned device word, private to the call. */
+#define NNTILE_HIP_MASK_TILE_MIXED 0
+#define NNTILE_HIP_MASK_TILE_OPEN 1
+#define NNTILE_HIP_MASK_TILE_HIDDEN 2
+#define NNTILE_HIP_MASK_TILE_CAUSAL 3
+int nntile_hip_mask_tile_class_bf16(void *stream, int64_t k_rows, int64_t q_cols,
+        const uint16_t *mask, int64_t offset, int32_t *workspace, int32_t *class_out);
+int nntile_hip_mask_tile_class_fp16(void *stream, int64_t k_rows, int64_t q_cols,
+        const uint16_t *mask, int64_t offset, int32_t *workspace, int32_t *class_out);
+int nntile_hip_mask_tile_class_fp32(void *stream, int64_t k_rows, int64_t q_cols,
+        const float *mask, int64_t offset, int32_t *workspace, int32_t *class_out);
+int nntile_hip_mask_tile_class_bool(void *stream, int64_t k_rows, int64_t q_cols,
+        const uint8_t *mask, int64_t offset, int32_t *workspace, int32_t *class_out);
+
 /* Library version and the ISA it was built for ("gfx950"). */
 const char *nntile_hip_sdpa_version(void);
 

@@ -37,6 +37,9 @@ int launch_kv_cache_append(hipStream_t stream, int elem, int64_t head, int64_t r
         int64_t entries, int64_t capacity, int64_t filled, const void *k_new,
         const void *v_new, void *k_cache, void *v_cache);
 
+int launch_mask_classify(hipStream_t stream, int dtype, int64_t k_rows, int64_t q_cols,
+        int64_t offset, const void *mask, uint32_t *flags);
+
 enum class DType { bf16, fp16, fp32 };
 
 static bool aligned16(const void *p)
@@ -470,6 +473,49 @@ static int kv_append_call(int elem, void *stream, int64_t head, int64_t rows, in
             capacity, filled, k_new, v_new, k_cache, v_cache);
 }
 
+// Blocking: the class comes back to the host.
+static int mask_class_call(int dtype, void *stream, int64_t k_rows, int64_t q_cols,
+        const void *mask, int64_t offset, int32_t *workspace, int32_t *class_out)
+{
+    if(k_rows <= 0 || q_cols <= 0 || mask == nullptr || workspace == nullptr
+            || class_out == nullptr || k_rows > (int64_t)0x3fffffffffffffff / q_cols
+            || (reinterpret_cast<uintptr_t>(workspace) & 3u) != 0)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int rc = launch_mask_classify(s, dtype, k_rows, q_cols, offset, mask,
+            reinterpret_cast<uint32_t *>(workspace));
+    if(rc != NNTILE_HIP_OK)
+    {
+        return rc;
+    }
+    uint32_t seen = 0;
+    if(hipMemcpyAsync(&seen, workspace, sizeof(seen), hipMemcpyDeviceToHost, s) != hipSuccess
+            || hipStreamSynchronize(s) != hipSuccess)
+    {
+        return NNTILE_HIP_ELAUNCH;
+    }
+    const bool visible = seen & 1u, hidden = seen & 2u, other = seen & 4u, off_rule = seen & 8u;
+    if(other)
+    {
+        *class_out = NNTILE_HIP_MASK_TILE_MIXED;
+    }
+    else if(!hidden)
+    {
+        *class_out = NNTILE_HIP_MASK_TILE_OPEN;
+    }
+    else if(!visible)
+    {
+        *class_out = NNTILE_HIP_MASK_TILE_HIDDEN;
+    }
+    else
+    {
+        *class_out = off_rule ? NNTILE_HIP_MASK_TILE_MIXED : NNTILE_HIP_MASK_TILE_CAUSAL;
+    }
+    return NNTILE_HIP_OK;
+}
+
 static nntile_hip_stream_provider g_stream_provider = nullptr;
 
 static void codelet_call(DType dt, const char *name, void *buffers[],
@@ -801,6 +847,30 @@ int nntile_hip_sdpa_fwd_decode_cache_fp16(void *stream, const nntile_hip_sdpa_ti
         int64_t capacity, void *workspace, size_t workspace_bytes)
 {
     return decode_call(DType::fp16, stream, args, capacity, workspace, workspace_bytes);
+}
+
+int nntile_hip_mask_tile_class_bf16(void *stream, int64_t k_rows, int64_t q_cols,
+        const uint16_t *mask, int64_t offset, int32_t *workspace, int32_t *class_out)
+{
+    return mask_class_call(0, stream, k_rows, q_cols, mask, offset, workspace, class_out);
+}
+
+int nntile_hip_mask_tile_class_fp16(void *stream, int64_t k_rows, int64_t q_cols,
+        const uint16_t *mask, int64_t offset, int32_t *workspace, int32_t *class_out)
+{
+    return mask_class_call(1, stream, k_rows, q_cols, mask, offset, workspace, class_out);
+}
+
+int nntile_hip_mask_tile_class_fp32(void *stream, int64_t k_rows, int64_t q_cols,
+        const float *mask, int64_t offset, int32_t *workspace, int32_t *class_out)
+{
+    return mask_class_call(2, stream, k_rows, q_cols, mask, offset, workspace, class_out);
+}
+
+int nntile_hip_mask_tile_class_bool(void *stream, int64_t k_rows, int64_t q_cols,
+        const uint8_t *mask, int64_t offset, int32_t *workspace, int32_t *class_out)
+{
+    return mask_class_call(3, stream, k_rows, q_cols, mask, offset, workspace, class_out);
 }
 
 const char *nntile_hip_sdpa_version(void)

@@ -21,6 +21,7 @@ MAX_TILES = 64
 OVERWRITE = 1
 
 OK, EINVAL, EUNSUPPORTED, ELAUNCH, EWORKSPACE = 0, -1, -2, -3, -4
+TILE_MIXED, TILE_OPEN, TILE_HIDDEN, TILE_CAUSAL = 0, 1, 2, 3
 _ERR = {EINVAL: "invalid argument", EUNSUPPORTED: "unsupported configuration",
         ELAUNCH: "HIP launch failed", EWORKSPACE: "workspace missing or too small"}
 
@@ -89,6 +90,7 @@ EXPORTS = (
     + ["nntile_hip_transpose_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_kv_cache_append_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_fwd_decode_cache_" + t for t in ("bf16", "fp16")]
+    + ["nntile_hip_mask_tile_class_" + t for t in ("bf16", "fp16", "fp32", "bool")]
     + ["nntile_hip_set_stream_provider", "nntile_hip_sdpa_version"])
 
 _lib = None
@@ -145,6 +147,10 @@ def lib():
             f.restype = ctypes.c_int
             f = getattr(L, "nntile_hip_kv_cache_append_" + t)
             f.argtypes = [_vp] + [_i64] * 5 + [_vp] * 4
+            f.restype = ctypes.c_int
+        for t in ("bf16", "fp16", "fp32", "bool"):
+            f = getattr(L, "nntile_hip_mask_tile_class_" + t)
+            f.argtypes = [_vp, _i64, _i64, _vp, _i64, _vp, ctypes.POINTER(ctypes.c_int32)]
             f.restype = ctypes.c_int
         L.nntile_hip_sdpa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
         L.nntile_hip_sdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
@@ -437,6 +443,24 @@ def decode_cache_workspace_bytes(k_seq, Q, n_batch, kv_group):
     a.batch, a.q_seq, a.head = Q.shape
     a.k_seq, a.n_batch, a.kv_group = k_seq, n_batch, kv_group
     return int(lib().nntile_hip_sdpa_fwd_decode_workspace_bytes(ctypes.byref(a)))
+
+
+def mask_tile_class(mask, offset=0, workspace=None, stream=None):
+    """Class (TILE_*) of one mask tile: a [q_cols, k_rows] C-ordered device
+    tensor (NNTile's [k_rows, q_cols]), additive in a tile type or bool,
+    against the rule `key <= query + offset`.  Blocking."""
+    _dev(mask, workspace)
+    if mask.dim() != 2 or not mask.is_contiguous():
+        raise SdpaError(EINVAL, "mask_tile_class")
+    if workspace is None:
+        workspace = torch.empty(1, dtype=torch.int32, device=mask.device)
+    q_cols, k_rows = mask.shape
+    name = "bool" if mask.dtype in (torch.bool, torch.uint8) else dtype_name(mask)
+    out = ctypes.c_int32(-1)
+    fn = getattr(lib(), "nntile_hip_mask_tile_class_" + name)
+    _check(fn(_stream(stream), k_rows, q_cols, _ptr(mask), offset, _ptr(workspace),
+              ctypes.byref(out)), "mask_tile_class")
+    return out.value
 
 
 def accumulate_attn_output(src_lse, src_attn, dst_lse, dst_attn, stream=None):

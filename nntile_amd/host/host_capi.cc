@@ -180,6 +180,55 @@ int nntile_host_flash_sdpa_fwd(int op, int dtype, void *K, void *Q, void *mask,
     catch(const std::exception &e) { return fail(err, errlen, e); }
 }
 
+} // extern "C"
+
+namespace
+{
+
+template<typename T>
+int64_t run_classified(AnyTensor *K, AnyTensor *Q, AnyTensor *mask, AnyTensor *lse,
+        AnyTensor *V, AnyTensor *A, int64_t offset, int32_t *classes, int64_t n_classes)
+{
+    const auto cls = tensor::flash_sdpa_mask_classes<T>(get<T>(mask), offset);
+    for(int64_t i = 0; classes != nullptr && i < n_classes
+            && i < static_cast<int64_t>(cls.size()); ++i)
+    {
+        classes[i] = cls[i];
+    }
+    const Index n = tensor::flash_sdpa_fwd_cudnn_async<T>(get<T>(K), get<T>(Q), get<T>(mask),
+            cls, offset, get<fp32_t>(lse), get<T>(V), get<T>(A));
+    starpu::task_wait_for_all();
+    return n;
+}
+
+} // namespace
+
+extern "C"
+{
+
+// tensor::flash_sdpa_mask_classes, then tensor::flash_sdpa_fwd_cudnn_async
+// with those classes + wait.  classes (may be null): room for n_classes
+// values, one per mask tile in the linear order of the mask's grid;
+// *submitted = tile pairs launched.
+int nntile_host_flash_sdpa_fwd_classified(int dtype, void *K, void *Q, void *mask,
+        void *lse, void *V, void *A, int64_t offset, int32_t *classes, int64_t n_classes,
+        int64_t *submitted, char *err, int errlen)
+{
+    try
+    {
+        auto k = static_cast<AnyTensor *>(K), q = static_cast<AnyTensor *>(Q),
+             m = static_cast<AnyTensor *>(mask), l = static_cast<AnyTensor *>(lse),
+             v = static_cast<AnyTensor *>(V), a = static_cast<AnyTensor *>(A);
+        int64_t n;
+        if(dtype == DT_BF16) n = run_classified<bf16_t>(k, q, m, l, v, a, offset, classes, n_classes);
+        else if(dtype == DT_FP16) n = run_classified<fp16_t>(k, q, m, l, v, a, offset, classes, n_classes);
+        else n = run_classified<fp32_t>(k, q, m, l, v, a, offset, classes, n_classes);
+        if(submitted != nullptr) *submitted = n;
+        return 0;
+    }
+    catch(const std::exception &e) { return fail(err, errlen, e); }
+}
+
 // Shape rules only (no device memory): level 0 = tile, 1 = tensor.  Shapes are
 // given as 6 x (ndim, dims..., basetile dims...) blocks in the order
 // K, Q, mask, logsumexp, V, A.

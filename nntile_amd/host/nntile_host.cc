@@ -814,6 +814,127 @@ void flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
     }
 }
 
+template<typename T> struct TileCall;
+template<> struct TileCall<bf16_t>
+{
+    static int run(void *s, const nntile_hip_sdpa_tile_args *a) { return nntile_hip_sdpa_fwd_tile_bf16(s, a); }
+    static int classify(void *s, Index k, Index q, const void *m, Index off, int32_t *ws, int32_t *out)
+    {
+        return nntile_hip_mask_tile_class_bf16(s, k, q, static_cast<const uint16_t *>(m), off, ws, out);
+    }
+};
+template<> struct TileCall<fp16_t>
+{
+    static int run(void *s, const nntile_hip_sdpa_tile_args *a) { return nntile_hip_sdpa_fwd_tile_fp16(s, a); }
+    static int classify(void *s, Index k, Index q, const void *m, Index off, int32_t *ws, int32_t *out)
+    {
+        return nntile_hip_mask_tile_class_fp16(s, k, q, static_cast<const uint16_t *>(m), off, ws, out);
+    }
+};
+template<> struct TileCall<fp32_t>
+{
+    static int run(void *s, const nntile_hip_sdpa_tile_args *a) { return nntile_hip_sdpa_fwd_tile_fp32(s, a); }
+    static int classify(void *s, Index k, Index q, const void *m, Index off, int32_t *ws, int32_t *out)
+    {
+        return nntile_hip_mask_tile_class_fp32(s, k, q, static_cast<const float *>(m), off, ws, out);
+    }
+};
+
+template<typename T>
+std::vector<int> flash_sdpa_mask_classes(const Tensor<T> &mask, Index causal_offset)
+{
+    require(mask.ndim == 2, "mask must be 2-dimensional");
+    std::vector<int> classes(mask.grid.nelems, NNTILE_HIP_MASK_TILE_MIXED);
+    starpu::VariableHandle word(sizeof(int32_t));
+    for(Index i = 0; i < mask.grid.nelems; ++i)
+    {
+        const auto index = mask.grid.linear_to_index(i);
+        const auto &tile = mask.get_tile(i);
+        // positions inside the tile: key k0 + k, query q0 + q
+        const Index k0 = index[0] * mask.basetile_shape[0];
+        const Index q0 = index[1] * mask.basetile_shape[1];
+        int32_t cls = NNTILE_HIP_MASK_TILE_MIXED;
+        const int rc = TileCall<T>::classify(starpu::get_local_stream(), tile.shape[0],
+                tile.shape[1], tile.get_ptr(), q0 - k0 + causal_offset,
+                static_cast<int32_t *>(word.get_ptr()), &cls);
+        if(rc != NNTILE_HIP_OK)
+        {
+            throw std::runtime_error("Error in mask_tile_class launch (code "
+                    + std::to_string(rc) + ")");
+        }
+        classes[i] = cls;
+    }
+    word.unregister_submit();
+    return classes;
+}
+
+template<typename T>
+Index flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &mask, const std::vector<int> &mask_classes,
+        Index causal_offset, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &V, const Tensor<T> &A)
+{
+    flash_sdpa_fwd_cudnn_check(K, Q, mask, logsumexp, V, A);
+    require(static_cast<Index>(mask_classes.size()) == mask.grid.nelems,
+            "one class per mask tile is required");
+    const Index num_k_seq_tiles = K.grid.shape[1];
+    const Index q_tile = Q.basetile_shape[1], k_tile = K.basetile_shape[1];
+    Index submitted = 0;
+    for(Index a_linear = 0; a_linear < A.grid.nelems; ++a_linear)
+    {
+        const auto a_index = A.grid.linear_to_index(a_linear);
+        const auto &Q_tile = Q.get_tile(a_linear);
+        const auto &A_tile = A.get_tile(a_linear);
+        const auto &lse_tile = logsumexp.get_tile(
+                {a_index[1], a_index[2], a_index[3], a_index[4]});
+        for(Index k_idx = 0; k_idx < num_k_seq_tiles; ++k_idx)
+        {
+            const Index m_linear = mask.grid.index_to_linear({k_idx, a_index[1]});
+            const int cls = mask_classes[m_linear];
+            if(cls == NNTILE_HIP_MASK_TILE_HIDDEN)
+            {
+                continue;       // the pair would leave (lse, A) as they are
+            }
+            auto kv_index = a_index;
+            kv_index[1] = k_idx;
+            const auto &K_tile = K.get_tile(kv_index);
+            const auto &V_tile = V.get_tile(kv_index);
+            ++submitted;
+            if(cls == NNTILE_HIP_MASK_TILE_MIXED)
+            {
+                tile::flash_sdpa_fwd_cudnn_async<T>(K_tile, Q_tile, mask.get_tile(m_linear),
+                        lse_tile, V_tile, A_tile);
+                continue;
+            }
+            nntile_hip_sdpa_tile_args a;
+            std::memset(&a, 0, sizeof(a));
+            a.q_seq = Q_tile.shape[1];
+            a.k_seq = K_tile.shape[1];
+            a.head = Q_tile.shape[0];
+            a.batch = Q_tile.shape[2] * Q_tile.shape[3] * Q_tile.shape[4];
+            a.n_batch = a.batch;
+            a.kv_group = 1;
+            a.mask_mode = cls == NNTILE_HIP_MASK_TILE_OPEN ? NNTILE_HIP_MASK_NONE
+                : NNTILE_HIP_MASK_CAUSAL;
+            a.q_pos0 = a_index[1] * q_tile;
+            a.k_pos0 = k_idx * k_tile;
+            a.causal_offset = causal_offset;
+            a.K = K_tile.get_ptr();
+            a.Q = Q_tile.get_ptr();
+            a.V = V_tile.get_ptr();
+            a.lse = static_cast<float *>(lse_tile.get_ptr());
+            a.A = A_tile.get_ptr();
+            const int rc = TileCall<T>::run(starpu::get_local_stream(), &a);
+            if(rc != NNTILE_HIP_OK)
+            {
+                throw std::runtime_error("Error in flash_sdpa_fwd tile launch (code "
+                        + std::to_string(rc) + ")");
+            }
+        }
+    }
+    return submitted;
+}
+
 // ---- backward: src/tensor/flash_sdpa_bwd_cudnn.cc:22-261 -------------------
 
 void flash_sdpa_bwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
@@ -1009,7 +1130,11 @@ NNTILE_HOST_INSTANTIATE_TENSOR_BWD(fp16_t)
     template void flash_sdpa_fwd_cudnn<T>(const Tensor<T> &, const Tensor<T> &, \
             const Tensor<T> &, const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &); \
     template void flash_sdpa_fwd_hip_async<T>(const Tensor<T> &, const Tensor<T> &, int, \
-            Index, const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, bool);
+            Index, const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, bool); \
+    template std::vector<int> flash_sdpa_mask_classes<T>(const Tensor<T> &, Index); \
+    template Index flash_sdpa_fwd_cudnn_async<T>(const Tensor<T> &, const Tensor<T> &, \
+            const Tensor<T> &, const std::vector<int> &, Index, const Tensor<fp32_t> &, \
+            const Tensor<T> &, const Tensor<T> &);
 NNTILE_HOST_INSTANTIATE_TENSOR(bf16_t)
 NNTILE_HOST_INSTANTIATE_TENSOR(fp16_t)
 NNTILE_HOST_INSTANTIATE_TENSOR(fp32_t)

@@ -265,6 +265,24 @@ void flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
         int mask_mode, Index causal_offset, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &V, const Tensor<T> &A, bool overwrite);
 
+//! Class (NNTILE_HIP_MASK_TILE_*) of every tile of a materialised mask, in
+//! the linear order of mask.grid, against the rule key <= query +
+//! causal_offset on global positions.  Blocking; a layer does this once per
+//! mask and keeps the result with it.
+template<typename T>
+std::vector<int> flash_sdpa_mask_classes(const Tensor<T> &mask, Index causal_offset);
+
+//! flash_sdpa_fwd_cudnn_async that uses those classes: a pair whose mask tile
+//! hides everything is not submitted, a pair whose mask tile hides nothing
+//! runs without a mask, a pair on the causal rule runs with the analytic
+//! mask, the rest as in the reference.  Returns the number of tile pairs
+//! submitted.
+template<typename T>
+Index flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &mask, const std::vector<int> &mask_classes,
+        Index causal_offset, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &V, const Tensor<T> &A);
+
 //! Shape and tiling rules of the tensor-level backward; throws
 void flash_sdpa_bwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
         const TensorTraits &V, const TensorTraits &A, const TensorTraits &dA,

@@ -35,6 +35,9 @@ def lib():
         L.nntile_host_flash_sdpa_fwd.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp,
                                                  ctypes.c_int, i64, ctypes.c_int, ctypes.c_char_p,
                                                  ctypes.c_int]
+        L.nntile_host_flash_sdpa_fwd_classified.argtypes = [
+            ctypes.c_int, vp, vp, vp, vp, vp, vp, i64, ctypes.POINTER(ctypes.c_int32), i64,
+            ctypes.POINTER(i64), ctypes.c_char_p, ctypes.c_int]
         L.nntile_host_check_shapes.argtypes = [ctypes.c_int, ctypes.POINTER(i64), ctypes.c_char_p,
                                                ctypes.c_int]
         L.nntile_host_flash_sdpa_bwd.argtypes = [ctypes.c_int, ctypes.c_int] + [vp] * 10 + [
@@ -105,6 +108,19 @@ class Tensor:
 def flash_sdpa_fwd(op, K, Q, mask, lse, V, A, mask_mode=0, offset=0, overwrite=False):
     _call(lib().nntile_host_flash_sdpa_fwd, op, DTYPES[Q.dtype], K.h, Q.h,
           None if mask is None else mask.h, lse.h, V.h, A.h, mask_mode, offset, int(overwrite))
+
+
+def flash_sdpa_fwd_classified(K, Q, mask, lse, V, A, offset=0):
+    """tensor::flash_sdpa_mask_classes + the tensor::flash_sdpa_fwd_cudnn_async
+    overload that takes them: pairs whose mask tile hides everything are not
+    submitted, open and causal ones run without reading the mask.  Returns
+    (classes per mask tile in the mask grid's linear order, pairs submitted)."""
+    n_tiles = mask.ntiles
+    classes = (ctypes.c_int32 * n_tiles)()
+    n = ctypes.c_int64(0)
+    _call(lib().nntile_host_flash_sdpa_fwd_classified, DTYPES[Q.dtype], K.h, Q.h, mask.h, lse.h,
+          V.h, A.h, offset, classes, n_tiles, ctypes.byref(n))
+    return list(classes), n.value
 
 
 def flash_sdpa_bwd(op, K, Q, V, A, dA, mask, lse, dK, dQ, dV, mask_mode=0, offset=0):

@@ -413,3 +413,35 @@ def prepare_mask_for_kv_cache(mask, k_seq, q_seq):
         return mask
     out = np.ones((k_seq, q_seq), bool)
     return copy_intersection(mask, [0, 0], out, [0, k_seq - q_seq])
+
+
+# ---- class of a mask tile ------------------------------------------------------
+
+TILE_MIXED, TILE_OPEN, TILE_HIDDEN, TILE_CAUSAL = 0, 1, 2, 3
+
+
+def mask_tile_class(mask, offset=0):
+    """What one (query tile, key tile) task needs from its mask tile.  mask:
+    [k_rows, q_cols] in the reference's axis order (the mask argument of
+    src/tile/flash_sdpa_fwd_cudnn.cc:161-196), additive float (0 visible, -inf
+    hidden) or bool (True visible).  HIDDEN: nothing visible (the task would
+    change nothing); OPEN: everything visible; CAUSAL: visible exactly where
+    k <= q + offset; MIXED: anything else, additive values other than 0 and
+    -inf included.  No counterpart in the reference, which submits every
+    pair; the definition is the specification."""
+    m = np.asarray(mask)
+    if m.dtype == bool:
+        visible, other = m, np.zeros(m.shape, bool)
+    else:
+        m = m.astype(np.float32)
+        visible = m == 0
+        other = ~visible & ~np.isneginf(m)
+    if other.any():
+        return TILE_MIXED
+    if visible.all():
+        return TILE_OPEN
+    if not visible.any():
+        return TILE_HIDDEN
+    k = np.arange(m.shape[0])[:, None]
+    q = np.arange(m.shape[1])[None, :]
+    return TILE_CAUSAL if np.array_equal(visible, k <= q + offset) else TILE_MIXED
