@@ -81,6 +81,15 @@ int64_t run_bwd(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *V, AnyTensor *A,
             starpu::task_wait_for_all();
             return n;
         }
+        case 3:     // tensor-level, mask tiles classified first
+        {
+            const auto cls = tensor::flash_sdpa_mask_classes<T>(get<T>(mask), offset);
+            const Index n = tensor::flash_sdpa_bwd_cudnn_async<T>(get<T>(K), get<T>(Q), get<T>(V),
+                    get<T>(A), get<T>(dA), get<T>(mask), cls, offset, get<fp32_t>(lse),
+                    get<T>(dK), get<T>(dQ), get<T>(dV));
+            starpu::task_wait_for_all();
+            return n;
+        }
         case 0:     // tensor-level, per-tile tasks, blocking
             tensor::flash_sdpa_bwd_cudnn<T>(get<T>(K), get<T>(Q), get<T>(V),
                     get<T>(A), get<T>(dA), get<T>(mask), get<fp32_t>(lse),
@@ -259,8 +268,9 @@ int nntile_host_check_shapes(int level, const int64_t *desc, char *err, int errl
 }
 
 // op: 0 tensor::flash_sdpa_bwd_cudnn, 1 tile::flash_sdpa_bwd_cudnn (single-tile
-// tensors), 2 tensor::flash_sdpa_bwd_hip_async + wait (mask may be null;
-// *submitted = tile pairs launched); dtype bf16 or fp16, as the reference's pack
+// tensors), 2 tensor::flash_sdpa_bwd_hip_async + wait (mask may be null), 3
+// tensor::flash_sdpa_mask_classes + the overload that takes the classes + wait
+// (ops 2 and 3: *submitted = tile pairs launched); dtype bf16 or fp16, as the reference's pack
 int nntile_host_flash_sdpa_bwd(int op, int dtype, void *K, void *Q, void *V,
         void *A, void *dA, void *mask, void *lse, void *dK, void *dQ, void *dV,
         int mask_mode, int64_t offset, int64_t *submitted, char *err, int errlen)

@@ -1028,19 +1028,17 @@ template<> struct BwdTileCall<fp16_t>
     static int run(void *s, const nntile_hip_sdpa_bwd_args *a) { return nntile_hip_sdpa_bwd_tile_fp16(s, a); }
 };
 
+// Per (dQ tile, key tile) pair: analytic calls with the pair's positions.
+// With `mask` and its classes, the pair's class picks the mode (hidden: no
+// call; mixed: the reference's tile operation with the mask tile); without,
+// every pair runs in `mask_mode` and pairs a causal mask hides are skipped.
 template<typename T>
-Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
+static Index bwd_pairs(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        const Tensor<T> *mask, const std::vector<int> *mask_classes,
         int mask_mode, Index causal_offset, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV)
 {
-    // Same shape rules as the reference operation, with a stand-in for the
-    // mask that is no longer materialised.
-    const TensorTraits mask({K.shape[1], Q.shape[1]},
-            {K.basetile_shape[1], Q.basetile_shape[1]});
-    flash_sdpa_bwd_cudnn_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
-    require(mask_mode == NNTILE_HIP_MASK_NONE || mask_mode == NNTILE_HIP_MASK_CAUSAL,
-            "flash_sdpa_bwd_hip: mask_mode must be NONE or CAUSAL");
     const Index num_k_seq_tiles = K.grid.shape[1];
     const Index q_tile = Q.basetile_shape[1], k_tile = K.basetile_shape[1];
     // One workspace for all calls: they run in order on one stream, and each
@@ -1065,15 +1063,36 @@ Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
         for(Index k_idx = 0; k_idx < num_k_seq_tiles; ++k_idx)
         {
             const Index k_pos0 = k_idx * k_tile;
+            auto kv_index = dq_index;
+            kv_index[1] = k_idx;
+            const auto &K_tile = K.get_tile(kv_index);
+            int pair_mode = mask_mode;
+            if(mask != nullptr)
+            {
+                const Index m_linear = mask->grid.index_to_linear({k_idx, dq_index[1]});
+                const int cls = (*mask_classes)[m_linear];
+                if(cls == NNTILE_HIP_MASK_TILE_HIDDEN)
+                {
+                    continue;       // no gradient flows through this pair
+                }
+                if(cls == NNTILE_HIP_MASK_TILE_MIXED)
+                {
+                    tile::flash_sdpa_bwd_cudnn_async<T>(K_tile, Q_tile, V.get_tile(kv_index),
+                            A.get_tile(dq_linear), dA.get_tile(dq_linear),
+                            mask->get_tile(m_linear), lse_tile, dK.get_tile(kv_index),
+                            dQ.get_tile(dq_linear), dV.get_tile(kv_index));
+                    ++submitted;
+                    continue;
+                }
+                pair_mode = cls == NNTILE_HIP_MASK_TILE_OPEN ? NNTILE_HIP_MASK_NONE
+                    : NNTILE_HIP_MASK_CAUSAL;
+            }
             // the last query of the tile sees keys up to its position + offset
-            if(mask_mode == NNTILE_HIP_MASK_CAUSAL
+            else if(mask_mode == NNTILE_HIP_MASK_CAUSAL
                     && k_pos0 > q_pos0 + q_len - 1 + causal_offset)
             {
                 continue;
             }
-            auto kv_index = dq_index;
-            kv_index[1] = k_idx;
-            const auto &K_tile = K.get_tile(kv_index);
             nntile_hip_sdpa_bwd_args a;
             std::memset(&a, 0, sizeof(a));
             a.q_seq = q_len;
@@ -1082,7 +1101,7 @@ Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
             a.batch = Q_tile.shape[2] * Q_tile.shape[3] * Q_tile.shape[4];
             a.n_batch = a.batch;
             a.kv_group = 1;
-            a.mask_mode = mask_mode;
+            a.mask_mode = pair_mode;
             a.q_pos0 = q_pos0;
             a.k_pos0 = k_pos0;
             a.causal_offset = causal_offset;
@@ -1110,7 +1129,42 @@ Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
     return submitted;
 }
 
+template<typename T>
+Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        int mask_mode, Index causal_offset, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV)
+{
+    // Same shape rules as the reference operation, with a stand-in for the
+    // mask that is no longer materialised.
+    const TensorTraits mask({K.shape[1], Q.shape[1]},
+            {K.basetile_shape[1], Q.basetile_shape[1]});
+    flash_sdpa_bwd_cudnn_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
+    require(mask_mode == NNTILE_HIP_MASK_NONE || mask_mode == NNTILE_HIP_MASK_CAUSAL,
+            "flash_sdpa_bwd_hip: mask_mode must be NONE or CAUSAL");
+    return bwd_pairs<T>(K, Q, V, A, dA, nullptr, nullptr, mask_mode, causal_offset,
+            logsumexp, dK, dQ, dV);
+}
+
+template<typename T>
+Index flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        const Tensor<T> &mask, const std::vector<int> &mask_classes,
+        Index causal_offset, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV)
+{
+    flash_sdpa_bwd_cudnn_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
+    require(static_cast<Index>(mask_classes.size()) == mask.grid.nelems,
+            "one class per mask tile is required");
+    return bwd_pairs<T>(K, Q, V, A, dA, &mask, &mask_classes, NNTILE_HIP_MASK_CAUSAL,
+            causal_offset, logsumexp, dK, dQ, dV);
+}
+
 #define NNTILE_HOST_INSTANTIATE_TENSOR_BWD(T) \
+    template Index flash_sdpa_bwd_cudnn_async<T>(const Tensor<T> &, const Tensor<T> &, \
+            const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, \
+            const std::vector<int> &, Index, const Tensor<fp32_t> &, const Tensor<T> &, \
+            const Tensor<T> &, const Tensor<T> &); \
     template Index flash_sdpa_bwd_hip_async<T>(const Tensor<T> &, const Tensor<T> &, \
             const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, int, Index, \
             const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &); \

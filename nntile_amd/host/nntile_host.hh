@@ -313,6 +313,17 @@ Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
         int mask_mode, Index causal_offset, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV);
 
+//! flash_sdpa_bwd_cudnn_async that uses the classes of the mask's tiles
+//! (flash_sdpa_mask_classes): no call for a pair whose mask tile hides
+//! everything, analytic masks for open and causal ones, the reference's tile
+//! operation for the rest.  Gradients are added.  Returns the pairs submitted.
+template<typename T>
+Index flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        const Tensor<T> &mask, const std::vector<int> &mask_classes,
+        Index causal_offset, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV);
+
 } // namespace tensor
 
 } // namespace nntile

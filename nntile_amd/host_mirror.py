@@ -9,7 +9,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "host", "libnntile_host.so")
 DTYPES = {"bf16": 0, "fp16": 1, "fp32": 2}
-OP_TENSOR, OP_TILE, OP_HIP = 0, 1, 2
+OP_TENSOR, OP_TILE, OP_HIP, OP_CLASSIFIED = 0, 1, 2, 3
 _lib = None
 
 
@@ -125,8 +125,10 @@ def flash_sdpa_fwd_classified(K, Q, mask, lse, V, A, offset=0):
 
 def flash_sdpa_bwd(op, K, Q, V, A, dA, mask, lse, dK, dQ, dV, mask_mode=0, offset=0):
     """tensor::flash_sdpa_bwd_cudnn (op 0), tile::flash_sdpa_bwd_cudnn (op 1) or
-    tensor::flash_sdpa_bwd_hip_async (op 2: analytic mask, mask=None): the
-    gradients are added to dK, dQ, dV.  Returns the tile pairs op 2 launched."""
+    tensor::flash_sdpa_bwd_hip_async (op 2: analytic mask, mask=None) or the
+    tensor-level overload that classifies the mask's tiles first (op 3; offset
+    = the causal rule the tiles are compared with): the gradients are added
+    to dK, dQ, dV.  Returns the tile pairs ops 2 and 3 launched."""
     n = ctypes.c_int64(0)
     _call(lib().nntile_host_flash_sdpa_bwd, op, DTYPES[Q.dtype],
           *(None if t is None else t.h for t in (K, Q, V, A, dA, mask, lse, dK, dQ, dV)),

@@ -135,6 +135,9 @@ def _run(op, dtype, data, lse, add_mask, shape5, base5, grads0=None, mask_mode=0
     if op == hm.OP_HIP:
         pairs = hm.flash_sdpa_bwd(op, T["K"], T["Q"], T["V"], T["A"], T["dA"], None, L, T["dK"], T["dQ"],
                                   T["dV"], mask_mode=mask_mode, offset=offset)
+    elif op == hm.OP_CLASSIFIED:
+        pairs = hm.flash_sdpa_bwd(op, T["K"], T["Q"], T["V"], T["A"], T["dA"], M, L, T["dK"], T["dQ"],
+                                  T["dV"], offset=offset)
     else:
         hm.flash_sdpa_bwd(op, T["K"], T["Q"], T["V"], T["A"], T["dA"], M, L, T["dK"], T["dQ"], T["dV"])
         pairs = hm.tasks_submitted_bwd(dtype) - before
@@ -251,3 +254,44 @@ def test_analytic_mask_form_skips_hidden_tile_pairs(oracle, dtype, mode, offset)
                                          np.where(vis[:, None], add, -np.inf))
     for g, w, n in zip(got, want, ("dK", "dQ", "dV")):
         assert H.rel_fro(g, w) < (1e-2 if dtype == "bf16" else 2e-3), n
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("kind,offset", [("causal", 0), ("causal", -70), ("window", 0), ("full", 0)])
+def test_classified_submission_skips_hidden_tile_pairs(oracle, dtype, kind, offset):
+    """The tensor-level overload that takes the classes of the mask's tiles:
+    the gradients of the reference submission (every pair with its mask tile)
+    and of the checker, with no call for pairs whose mask tile hides
+    everything."""
+    head, seq, tile, nb, grp, nkv = 64, 320, 64, 2, 1, 2
+    batch = nb * grp * nkv
+    shape5, base5 = [head, seq, nb, grp, nkv], [head, tile, 1, 1, 2]
+    (Q, K, V), (qf, kf, vf) = H.make_qkv(61, batch, seq, seq, head, dtype)
+    _, gf = H.rounded(synth.randn(62, 0, batch * seq * head).reshape(batch, seq, head), dtype)
+    i = np.arange(seq)
+    mask = {"causal": i[None, :] <= i[:, None] + offset, "window": np.abs(i[None, :] - i[:, None]) <= 90,
+            "full": np.ones((seq, seq), bool)}[kind]
+    add = np.where(mask, 0.0, -np.inf).astype(np.float32)
+    vis = mask.any(axis=1)
+    with np.errstate(all="ignore"):
+        A64, lse64 = oracle.sdpa_bruteforce_f64(kf, qf, vf, add)
+    A64 = np.where(vis[None, :, None], A64, 0.0)
+    lse = np.where(vis[None, :], lse64, -np.inf).astype(np.float32)
+    _, af = H.rounded(A64, dtype)
+    data = {"K": kf, "Q": qf, "V": vf, "A": af, "dA": gf}
+    got, pairs, ntiles = _run(hm.OP_CLASSIFIED, dtype, data, lse, add, shape5, base5, offset=offset)
+    ref, all_pairs, _ = _run(hm.OP_TENSOR, dtype, data, lse, add, shape5, base5)
+    nt = seq // tile
+    slabs = ntiles // nt
+    live = sum(1 for q in range(nt) for k in range(nt)
+               if mask[q * tile:(q + 1) * tile, k * tile:(k + 1) * tile].any())
+    assert all_pairs == slabs * nt * nt and pairs == slabs * live
+    assert (live < nt * nt) == (kind != "full")
+    with np.errstate(all="ignore"):
+        want = oracle.sdpa_bwd_flash_f64(kf, qf, vf, af, gf, np.where(vis[None, :], lse, 0.0),
+                                         np.where(vis[:, None], add, -np.inf))
+    tol = 1e-2 if dtype == "bf16" else 2e-3
+    for g, r, w, n in zip(got, ref, want, ("dK", "dQ", "dV")):
+        assert H.rel_fro(g, w) < tol, n
+        assert H.rel_fro(g, r) < tol, n
