@@ -55,7 +55,7 @@ struct MaskBool
 
 // One workgroup per CHUNK elements of the flattened tile; a thread walks its
 // elements with stride 256 so that a wave reads neighbouring addresses.
-constexpr int kClassifyChunk = 16384;
+constexpr int kClassifyChunk = 4096;
 
 template<typename M>
 __global__ __launch_bounds__(256)
@@ -96,7 +96,10 @@ void mask_classify_kernel(int64_t k_rows, int64_t total, int64_t offset,
             seen |= bit;
         }
     }
-    if((threadIdx.x & 63) == 0 && seen != 0)
+    // Bits are only ever set, so a wave whose bits are all in the word already
+    // has nothing to add: after the first few waves the atomics stop.
+    if((threadIdx.x & 63) == 0
+            && (seen & ~__atomic_load_n(flags, __ATOMIC_RELAXED)) != 0)
     {
         atomicOr(flags, seen);
     }
