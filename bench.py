@@ -294,20 +294,22 @@ def bench_kv_cache(cfg, steps, warmup):
     lse = torch.full((cfg.batch_flat, cfg.q_seq), float("-inf"), device="cuda")
     ws = torch.empty(h.decode_cache_workspace_bytes(cfg.k_seq, Q, cfg.n_batch, cfg.kv_group),
                      dtype=torch.uint8, device="cuda")
+    filled = cfg.k_seq - cfg.q_seq
     plans = [h.plan_decode_cache(Ks[j], Vs[j], cfg.k_seq, Q, None, lse, A, h.MASK_CAUSAL,
                                  cfg.n_batch, cfg.kv_group, ws, causal_offset=cfg.causal_offset,
                                  flags=h.OVERWRITE) for j in range(nrot)]
-    filled = cfg.k_seq - cfg.q_seq
     i = [0]
+
+    appends = [h.plan_kv_cache_append(k_new, v_new, Ks[j], Vs[j], filled) for j in range(nrot)]
 
     def step():
         j = i[0] % nrot
-        h.kv_cache_append(k_new, v_new, Ks[j], Vs[j], filled)
+        appends[j].launch()
         plans[j].launch()
         i[0] += 1
 
     def append_only():
-        h.kv_cache_append(k_new, v_new, Ks[i[0] % nrot], Vs[i[0] % nrot], filled)
+        appends[i[0] % nrot].launch()
         i[0] += 1
 
     wall, dev = time_steps(step, steps, warmup)

@@ -402,6 +402,27 @@ def kv_cache_append(k_new, v_new, k_cache, v_cache, filled, stream=None):
               _ptr(v_new), _ptr(k_cache), _ptr(v_cache)), "kv_cache_append")
 
 
+def plan_kv_cache_append(k_new, v_new, k_cache, v_cache, filled):
+    """kv_cache_append prepared once for a fixed position (a benchmark's or a
+    graph's step); `launch(stream)` costs one foreign call."""
+    _dev(k_new, v_new, k_cache, v_cache)
+    entries, rows, head = k_new.shape
+    if (tuple(v_new.shape) != (entries, rows, head) or k_cache.shape != v_cache.shape
+            or k_cache.shape[0] != entries or k_cache.shape[2] != head):
+        raise SdpaError(EINVAL, "kv_cache_append")
+    fn = getattr(lib(), "nntile_hip_kv_cache_append_" + dtype_name(k_cache))
+    args = (head, rows, entries, k_cache.shape[1], filled, _ptr(k_new), _ptr(v_new),
+            _ptr(k_cache), _ptr(v_cache))
+
+    class _Append:
+        def launch(self, stream=None):
+            _check(fn(_stream(stream), *args), "kv_cache_append")
+
+    plan = _Append()
+    plan._keep = (k_new, v_new, k_cache, v_cache)
+    return plan
+
+
 def _cache_args(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch, kv_group, q_pos0,
                 k_pos0, causal_offset, flags):
     a = _tile_args(K_cache, Q, mask, lse, V_cache, A, mask_mode, n_batch, kv_group, q_pos0,

@@ -81,13 +81,26 @@ class KVCache:
     def attend(self, Q, lse, A, n_batch, kv_group, causal=True, stream=None):
         """A = attention of Q over the filled rows; the q_seq queries are the
         last q_seq tokens of the cache (append first).  lse and A are
-        overwritten."""
+        overwritten.  The decode entry point takes at most 64 // kv_group
+        query rows per call: longer chunks go through it piece by piece (each
+        piece with its position among the queries), through dense copies of
+        its rows."""
         k_seq = len(self)
         q_seq = Q.shape[1]
-        need = hip_sdpa.decode_cache_workspace_bytes(k_seq, Q, n_batch, kv_group)
-        if self._workspace is None or self._workspace.numel() < need:
-            self._workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
+        step = max(1, 64 // kv_group)
         mode = hip_sdpa.MASK_CAUSAL if causal else hip_sdpa.MASK_NONE
-        hip_sdpa.sdpa_fwd_decode_cache(
-            self.k, self.v, k_seq, Q, None, lse, A, mode, n_batch, kv_group, self._workspace,
-            causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)
+        for j0 in range(0, q_seq, step):
+            n = min(step, q_seq - j0)
+            whole = n == q_seq
+            Qs = Q if whole else Q[:, j0:j0 + n].contiguous()
+            ls = lse if whole else torch.empty((Q.shape[0], n), dtype=lse.dtype, device=Q.device)
+            As = A if whole else torch.empty_like(Qs)
+            need = hip_sdpa.decode_cache_workspace_bytes(k_seq, Qs, n_batch, kv_group)
+            if self._workspace is None or self._workspace.numel() < need:
+                self._workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
+            hip_sdpa.sdpa_fwd_decode_cache(
+                self.k, self.v, k_seq, Qs, None, ls, As, mode, n_batch, kv_group, self._workspace,
+                q_pos0=j0, causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)
+            if not whole:
+                lse[:, j0:j0 + n] = ls
+                A[:, j0:j0 + n] = As

@@ -104,16 +104,16 @@ def test_decode_from_cache(oracle, dtype, q_seq, k_seq, cap, n_batch, group, n_k
 @pytest.mark.parametrize("head,group", [(128, 4), (64, 1)])
 def test_prefill_then_decode_chunks_equal_the_full_pass(oracle, dtype, head, group):
     """Prefill with the causal tile entry, keys and values appended to the
-    cache; then chunks of 1, 1, 5 and 16 new tokens through the cache."""
+    cache; then chunks of 1, 1, 5, 16 and 40 new tokens through the cache."""
     n_batch, n_kv, prefill = 2, 2, 150
-    chunks = (1, 1, 5, 16)
+    chunks = (1, 1, 5, 16, 40)          # 40 > 64 // group rows: attend splits the chunk
     total = prefill + sum(chunks)
     batch, kvb = n_batch * group * n_kv, n_batch * n_kv
     (Q, K, V), (qf, kf, vf) = H.make_qkv(29, batch, total, total, head, dtype, kv_batch=kvb)
     want, want_lse = oracle.sdpa_vanilla(kf, qf, vf, synth.causal_mask(total, total),
                                          n_batch=n_batch, kv_repeat=group)
     Qd, Kd, Vd = Q.cuda(), K.cuda(), V.cuda()
-    cache = KVCache(max_cache_size=256)
+    cache = KVCache(max_cache_size=total + 7)
     got, got_lse = [], []
     # prefill: the dense causal pass, then the cache takes its keys and values
     Qp, Kp, Vp = (t[:, :prefill].contiguous() for t in (Qd, Kd, Vd))
