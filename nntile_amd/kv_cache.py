@@ -78,28 +78,53 @@ class KVCache:
         self.v_cache_size = 0
         self._workspace = None
 
-    def attend(self, Q, lse, A, n_batch, kv_group, causal=True, stream=None):
+    def mask_slice(self, mask, q_seq):
+        """The mask rows that go with the last q_seq tokens of the cache
+        (Sdpa._prepare_mask_for_kv_cache, wrappers/python/nntile/layer/sdpa.py:
+        489-531).  mask: bool device tensor [queries, keys] in C order (the
+        reference's [keys, queries]), True = visible.  A mask that already is
+        [q_seq, len] is used as it is; otherwise everything is visible except
+        where the mask, read at query position len - q_seq + j, says
+        otherwise."""
+        k_seq = len(self)
+        if tuple(mask.shape) == (q_seq, k_seq):
+            return mask.contiguous()
+        out = torch.ones((q_seq, k_seq), dtype=torch.bool, device=mask.device)
+        first = k_seq - q_seq
+        rows = max(0, min(q_seq, mask.shape[0] - first))
+        cols = min(k_seq, mask.shape[1])
+        if rows > 0 and cols > 0 and first >= 0:
+            out[:rows, :cols] = mask[first:first + rows, :cols]
+        return out
+
+    def attend(self, Q, lse, A, n_batch, kv_group, causal=True, mask=None, stream=None):
         """A = attention of Q over the filled rows; the q_seq queries are the
         last q_seq tokens of the cache (append first).  lse and A are
-        overwritten.  The decode entry point takes at most 64 // kv_group
-        query rows per call: longer chunks go through it piece by piece (each
-        piece with its position among the queries), through dense copies of
-        its rows."""
+        overwritten.  mask: None (the causal rule when `causal`, else nothing
+        hidden) or a bool mask as for `mask_slice`, whose slice is then passed
+        as values.  The decode entry point takes at most 64 // kv_group query
+        rows per call: longer chunks go through it piece by piece (each piece
+        with its position among the queries), through dense copies of its
+        rows."""
         k_seq = len(self)
         q_seq = Q.shape[1]
         step = max(1, 64 // kv_group)
         mode = hip_sdpa.MASK_CAUSAL if causal else hip_sdpa.MASK_NONE
+        sliced = None
+        if mask is not None:
+            sliced, mode = self.mask_slice(mask, q_seq), hip_sdpa.MASK_BOOL
         for j0 in range(0, q_seq, step):
             n = min(step, q_seq - j0)
             whole = n == q_seq
             Qs = Q if whole else Q[:, j0:j0 + n].contiguous()
             ls = lse if whole else torch.empty((Q.shape[0], n), dtype=lse.dtype, device=Q.device)
             As = A if whole else torch.empty_like(Qs)
+            ms = None if sliced is None else (sliced if whole else sliced[j0:j0 + n].contiguous())
             need = hip_sdpa.decode_cache_workspace_bytes(k_seq, Qs, n_batch, kv_group)
             if self._workspace is None or self._workspace.numel() < need:
                 self._workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
             hip_sdpa.sdpa_fwd_decode_cache(
-                self.k, self.v, k_seq, Qs, None, ls, As, mode, n_batch, kv_group, self._workspace,
+                self.k, self.v, k_seq, Qs, ms, ls, As, mode, n_batch, kv_group, self._workspace,
                 q_pos0=j0, causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)
             if not whole:
                 lse[:, j0:j0 + n] = ls

@@ -163,3 +163,47 @@ def test_full_size_decode_step_through_the_cache():
     assert torch.equal(A.view(torch.int16), A2.view(torch.int16))
     assert torch.equal(lse, lse2)
     assert bool(torch.isfinite(lse).all())
+
+
+@pytest.mark.parametrize("q_full,k_full", [(64, 64), (40, 64), (64, 40), (30, 30)])
+def test_mask_slice_equals_the_checker(oracle, q_full, k_full):
+    """KVCache.mask_slice == Sdpa._prepare_mask_for_kv_cache as the checker
+    restates it, also when the mask is smaller than the cache on either axis."""
+    rng = np.random.default_rng(q_full * 100 + k_full)
+    mask = rng.random((q_full, k_full)) < 0.6                      # [queries, keys]
+    cache = KVCache(64)
+    z = torch.zeros((2, 1, 64), dtype=torch.bfloat16, device="cuda")
+    for filled, q_seq in ((1, 1), (17, 16), (18, 1), (48, 30), (64, 16)):
+        while len(cache) < filled:
+            cache.append(z, z)
+        got = cache.mask_slice(torch.from_numpy(mask).cuda(), q_seq).cpu().numpy()
+        want = oracle.prepare_mask_for_kv_cache(mask.T, filled, q_seq).T
+        assert np.array_equal(got, want), (filled, q_seq)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+def test_attend_with_a_mask_given_as_values(oracle, dtype):
+    """A bool mask that is not causal (a window plus the first key), sliced
+    for the cached keys, chunks of 3 and 37 tokens."""
+    head, n_batch, n_kv, group, prefill = 128, 2, 2, 4, 60
+    chunks = (3, 37)
+    total = prefill + sum(chunks)
+    batch, kvb = n_batch * group * n_kv, n_batch * n_kv
+    (Q, K, V), (qf, kf, vf) = H.make_qkv(37, batch, total, total, head, dtype, kv_batch=kvb)
+    i = np.arange(total)
+    full = (np.abs(i[:, None] - i[None, :]) <= 20) & (i[None, :] <= i[:, None])
+    full[:, 0] = True                                              # [queries, keys]
+    want, want_lse = oracle.sdpa_vanilla(kf, qf, vf, full, n_batch=n_batch, kv_repeat=group)
+    Qd, Kd, Vd = Q.cuda(), K.cuda(), V.cuda()
+    mask_d = torch.from_numpy(full).cuda()
+    cache = KVCache(total)
+    cache.append(Kd[:, :prefill].contiguous(), Vd[:, :prefill].contiguous())
+    pos = prefill
+    for rows in chunks:
+        cache.append(Kd[:, pos:pos + rows].contiguous(), Vd[:, pos:pos + rows].contiguous())
+        lse, A = H.fresh_outputs(batch, rows, head, dtype)
+        cache.attend(Qd[:, pos:pos + rows].contiguous(), lse, A, n_batch, group, mask=mask_d)
+        torch.cuda.synchronize()
+        assert H.rel_fro(H.to_np(A), want[:, pos:pos + rows]) < H.TOL[dtype]
+        assert H.rel_fro(H.to_np(lse), want_lse[:, pos:pos + rows]) < H.TOL[dtype]
+        pos += rows
