@@ -341,6 +341,17 @@ int nntile_hip_sdpa_fwd_decode_cache_bf16(void *stream, const nntile_hip_sdpa_ti
 int nntile_hip_sdpa_fwd_decode_cache_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
         int64_t capacity, void *workspace, size_t workspace_bytes);
 
+/* nntile_hip_sdpa_fwd_tile_* reading the cache the same way, for what the
+ * decode form does not take: fp32 caches (the reference runs forward_dynamic
+ * in fp32 too, wrappers/python/tests/model/test_llama_attention.py:296-345),
+ * head 32, and chunks of more than 64 / kv_group new tokens.  No workspace. */
+int nntile_hip_sdpa_fwd_tile_cache_bf16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity);
+int nntile_hip_sdpa_fwd_tile_cache_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity);
+int nntile_hip_sdpa_fwd_tile_cache_fp32(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity);
+
 /* ---- 10. class of a mask tile -------------------------------------------------
  * For the layer that submits one task per (query tile, key tile) pair with
  * the pair's mask tile (src/tensor/flash_sdpa_fwd_cudnn.cc:246-274, which

@@ -71,7 +71,8 @@ static int dispatch_prefill(DType dt, hipStream_t stream, PrefillParams &p,
     }
 }
 
-static int tile_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a)
+static int tile_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a,
+        int64_t kv_rows = 0)
 {
     if(a == nullptr || a->q_seq <= 0 || a->k_seq <= 0 || a->head <= 0
             || a->batch <= 0 || a->n_batch <= 0 || a->kv_group <= 0
@@ -103,6 +104,7 @@ static int tile_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a)
     p.causal_offset = a->causal_offset;
     p.mask = a->mask;
     p.mask_ld = a->k_seq;
+    p.kv_rows = kv_rows;
     p.n_q_tiles = p.n_kv_tiles = 1;
     p.batch = (int32_t)a->batch;
     p.n_batch = (int32_t)a->n_batch;
@@ -835,6 +837,27 @@ int nntile_hip_kv_cache_append_fp32(void *stream, int64_t head, int64_t rows, in
 {
     return kv_append_call(4, stream, head, rows, entries, capacity, filled, k_new, v_new,
             k_cache, v_cache);
+}
+
+int nntile_hip_sdpa_fwd_tile_cache_bf16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity)
+{
+    return args != nullptr && capacity < args->k_seq ? NNTILE_HIP_EINVAL
+        : tile_call(DType::bf16, stream, args, capacity);
+}
+
+int nntile_hip_sdpa_fwd_tile_cache_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity)
+{
+    return args != nullptr && capacity < args->k_seq ? NNTILE_HIP_EINVAL
+        : tile_call(DType::fp16, stream, args, capacity);
+}
+
+int nntile_hip_sdpa_fwd_tile_cache_fp32(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity)
+{
+    return args != nullptr && capacity < args->k_seq ? NNTILE_HIP_EINVAL
+        : tile_call(DType::fp32, stream, args, capacity);
 }
 
 int nntile_hip_sdpa_fwd_decode_cache_bf16(void *stream, const nntile_hip_sdpa_tile_args *args,

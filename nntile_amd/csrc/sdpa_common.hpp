@@ -43,6 +43,8 @@ struct PrefillParams
     int64_t q_seq, k_seq, q_tile, k_tile;
     int64_t q_pos0, k_pos0, causal_offset;
     int64_t mask_ld;              // = k_seq of the single key tile (explicit masks)
+    int64_t kv_rows;              // rows between two entries of K and V; 0: the tile's own rows
+                                  // (a cache's capacity, single key tile only)
     const void *mask;
     int32_t n_q_tiles, n_kv_tiles;
     int32_t batch, n_batch, kv_group;

@@ -368,7 +368,8 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // Byte offset of batch entry kvb's slab inside key tile kt.
     auto slab = [&](int kt) -> int64_t
     {
-        return (int64_t)kvb * tile_rows(kt) * HEAD * 2;
+        const int64_t rows = p.kv_rows > 0 ? p.kv_rows : (int64_t)tile_rows(kt);
+        return (int64_t)kvb * rows * HEAD * 2;
     };
 
     // Global -> LDS loads of the K (or V) rows of one step.  Rows past the end

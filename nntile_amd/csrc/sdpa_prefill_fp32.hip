@@ -126,8 +126,9 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     };
     const int64_t k_len0 = min(p.k_tile, p.k_seq);
     const bool one_tile = p.n_kv_tiles == 1;
-    const float *K0 = static_cast<const float *>(p.K[0]) + ((int64_t)kvb * k_len0) * HEAD;
-    const float *V0 = static_cast<const float *>(p.V[0]) + ((int64_t)kvb * k_len0) * HEAD;
+    const int64_t entry_rows0 = p.kv_rows > 0 ? p.kv_rows : k_len0;
+    const float *K0 = static_cast<const float *>(p.K[0]) + ((int64_t)kvb * entry_rows0) * HEAD;
+    const float *V0 = static_cast<const float *>(p.V[0]) + ((int64_t)kvb * entry_rows0) * HEAD;
     auto locate = [&](int g, int n_steps_all) -> StepSource
     {
         // steps past the last re-read the last one (nobody uses them)

@@ -90,6 +90,7 @@ EXPORTS = (
     + ["nntile_hip_transpose_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_kv_cache_append_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_fwd_decode_cache_" + t for t in ("bf16", "fp16")]
+    + ["nntile_hip_sdpa_fwd_tile_cache_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_mask_tile_class_" + t for t in ("bf16", "fp16", "fp32", "bool")]
     + ["nntile_hip_set_stream_provider", "nntile_hip_sdpa_version"])
 
@@ -144,6 +145,9 @@ def lib():
         for t in ("bf16", "fp16", "fp32"):
             f = getattr(L, "nntile_hip_transpose_" + t)
             f.argtypes = [_vp, _i64, _i64, ctypes.c_float, _vp, _vp]
+            f.restype = ctypes.c_int
+            f = getattr(L, "nntile_hip_sdpa_fwd_tile_cache_" + t)
+            f.argtypes = [_vp, ctypes.POINTER(TileArgs), _i64]
             f.restype = ctypes.c_int
             f = getattr(L, "nntile_hip_kv_cache_append_" + t)
             f.argtypes = [_vp] + [_i64] * 5 + [_vp] * 4
@@ -445,6 +449,20 @@ def sdpa_fwd_decode_cache(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n
     nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _check(fn(_stream(stream), ctypes.byref(a), K_cache.shape[1], _ptr(workspace), nbytes),
            "sdpa_fwd_decode_cache")
+
+
+def sdpa_fwd_tile_cache(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch=None,
+                        kv_group=1, q_pos0=0, k_pos0=0, causal_offset=0, flags=0, stream=None):
+    """sdpa_fwd_tile over the first k_seq rows of every entry of the caches
+    ([entries, capacity, head]), read where they lie; any chunk length, fp32
+    included."""
+    _dev(K_cache, V_cache, Q, mask, lse, A)
+    if K_cache.shape != V_cache.shape:
+        raise SdpaError(EINVAL, "sdpa_fwd_tile_cache")
+    a = _cache_args(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch, kv_group,
+                    q_pos0, k_pos0, causal_offset, flags)
+    fn = getattr(lib(), "nntile_hip_sdpa_fwd_tile_cache_" + dtype_name(Q))
+    _check(fn(_stream(stream), ctypes.byref(a), K_cache.shape[1]), "sdpa_fwd_tile_cache")
 
 
 def plan_decode_cache(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch, kv_group,

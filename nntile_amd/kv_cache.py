@@ -102,30 +102,26 @@ class KVCache:
         last q_seq tokens of the cache (append first).  lse and A are
         overwritten.  mask: None (the causal rule when `causal`, else nothing
         hidden) or a bool mask as for `mask_slice`, whose slice is then passed
-        as values.  The decode entry point takes at most 64 // kv_group query
-        rows per call: longer chunks go through it piece by piece (each piece
-        with its position among the queries), through dense copies of its
-        rows."""
+        as values.  Few rows of a 16-bit type (kv_group * q_seq <= 64, head 64
+        or 128) take the split-key decode kernel, everything else - longer
+        chunks, fp32, head 32 - the tile kernel; both read the caches in
+        place."""
         k_seq = len(self)
         q_seq = Q.shape[1]
-        step = max(1, 64 // kv_group)
         mode = hip_sdpa.MASK_CAUSAL if causal else hip_sdpa.MASK_NONE
         sliced = None
         if mask is not None:
             sliced, mode = self.mask_slice(mask, q_seq), hip_sdpa.MASK_BOOL
-        for j0 in range(0, q_seq, step):
-            n = min(step, q_seq - j0)
-            whole = n == q_seq
-            Qs = Q if whole else Q[:, j0:j0 + n].contiguous()
-            ls = lse if whole else torch.empty((Q.shape[0], n), dtype=lse.dtype, device=Q.device)
-            As = A if whole else torch.empty_like(Qs)
-            ms = None if sliced is None else (sliced if whole else sliced[j0:j0 + n].contiguous())
-            need = hip_sdpa.decode_cache_workspace_bytes(k_seq, Qs, n_batch, kv_group)
-            if self._workspace is None or self._workspace.numel() < need:
-                self._workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
-            hip_sdpa.sdpa_fwd_decode_cache(
-                self.k, self.v, k_seq, Qs, ms, ls, As, mode, n_batch, kv_group, self._workspace,
-                q_pos0=j0, causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)
-            if not whole:
-                lse[:, j0:j0 + n] = ls
-                A[:, j0:j0 + n] = As
+        decode = (Q.dtype != torch.float32 and kv_group * q_seq <= 64
+                  and Q.shape[2] in (64, 128))
+        if not decode:
+            hip_sdpa.sdpa_fwd_tile_cache(
+                self.k, self.v, k_seq, Q, sliced, lse, A, mode, n_batch, kv_group,
+                causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)
+            return
+        need = hip_sdpa.decode_cache_workspace_bytes(k_seq, Q, n_batch, kv_group)
+        if self._workspace is None or self._workspace.numel() < need:
+            self._workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
+        hip_sdpa.sdpa_fwd_decode_cache(
+            self.k, self.v, k_seq, Q, sliced, lse, A, mode, n_batch, kv_group, self._workspace,
+            causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)

@@ -100,13 +100,13 @@ def test_decode_from_cache(oracle, dtype, q_seq, k_seq, cap, n_batch, group, n_k
     assert np.array_equal(_bits(lse), _bits(lse2))
 
 
-@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
-@pytest.mark.parametrize("head,group", [(128, 4), (64, 1)])
+@pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("head,group", [(128, 4), (64, 1), (32, 2)])
 def test_prefill_then_decode_chunks_equal_the_full_pass(oracle, dtype, head, group):
     """Prefill with the causal tile entry, keys and values appended to the
     cache; then chunks of 1, 1, 5, 16 and 40 new tokens through the cache."""
     n_batch, n_kv, prefill = 2, 2, 150
-    chunks = (1, 1, 5, 16, 40)          # 40 > 64 // group rows: attend splits the chunk
+    chunks = (1, 1, 5, 16, 40)          # short 16-bit chunks: decode kernel; the rest: tile kernel
     total = prefill + sum(chunks)
     batch, kvb = n_batch * group * n_kv, n_batch * n_kv
     (Q, K, V), (qf, kf, vf) = H.make_qkv(29, batch, total, total, head, dtype, kv_batch=kvb)
@@ -207,3 +207,38 @@ def test_attend_with_a_mask_given_as_values(oracle, dtype):
         assert H.rel_fro(H.to_np(A), want[:, pos:pos + rows]) < H.TOL[dtype]
         assert H.rel_fro(H.to_np(lse), want_lse[:, pos:pos + rows]) < H.TOL[dtype]
         pos += rows
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("q_seq,k_seq,cap,n_batch,group,n_kv,head,mode", [
+    (100, 300, 512, 2, 4, 2, 128, "causal"), (1, 77, 80, 3, 2, 2, 64, "causal"),
+    (130, 130, 131, 1, 1, 3, 32, "causal"), (70, 200, 333, 2, 2, 1, 64, "bool"),
+    (33, 1000, 1000, 1, 8, 1, 128, "none")])
+def test_tile_entry_reading_the_cache(oracle, dtype, q_seq, k_seq, cap, n_batch, group, n_kv, head, mode):
+    """The tile kernel over a cache whose unfilled rows hold NaN == the checker
+    within the tolerance and == the same call over dense copies bit for bit."""
+    print("case", dtype, q_seq, k_seq, cap, n_batch, group, n_kv, head, mode, flush=True)
+    batch, kvb = n_batch * group * n_kv, n_batch * n_kv
+    (Q, K, V), (qf, kf, vf) = H.make_qkv(41, batch, q_seq, k_seq, head, dtype, kv_batch=kvb)
+    offset = k_seq - q_seq
+    mask = None if mode == "none" else synth.causal_mask(q_seq, k_seq, offset)
+    want, want_lse = oracle.sdpa_vanilla(kf, qf, vf, mask, n_batch=n_batch, kv_repeat=group)
+    Qd = Q.cuda()
+    Kc = torch.full((kvb, cap, head), float("nan"), dtype=H.TORCH_DT[dtype], device="cuda")
+    Vc = torch.full_like(Kc, float("nan"))
+    Kc[:, :k_seq] = K.cuda()
+    Vc[:, :k_seq] = V.cuda()
+    m, mm = {"causal": (None, hip_sdpa.MASK_CAUSAL), "none": (None, hip_sdpa.MASK_NONE),
+             "bool": (None if mask is None else torch.from_numpy(mask).cuda(), hip_sdpa.MASK_BOOL)}[mode]
+    lse, A = H.fresh_outputs(batch, q_seq, head, dtype)
+    hip_sdpa.sdpa_fwd_tile_cache(Kc, Vc, k_seq, Qd, m, lse, A, mm, n_batch, group,
+                                 causal_offset=offset)
+    lse2, A2 = H.fresh_outputs(batch, q_seq, head, dtype)
+    hip_sdpa.sdpa_fwd_tile(K.cuda(), Qd, m, lse2, V.cuda(), A2, mm, n_batch=n_batch, kv_group=group,
+                           causal_offset=offset)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+    assert torch.equal(A.view(torch.int32 if dtype == "fp32" else torch.int16),
+                       A2.view(torch.int32 if dtype == "fp32" else torch.int16))
+    assert torch.equal(lse, lse2)

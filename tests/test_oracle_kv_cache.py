@@ -131,3 +131,10 @@ def test_append_and_cache_decode_argument_checks():
     assert dec(None, ctypes.byref(a), 511, 4096, 1 << 30) == h.EINVAL            # capacity < k_seq
     assert dec(None, ctypes.byref(a), 1024, None, 0) == h.EWORKSPACE
     assert dec(None, None, 1024, 4096, 1 << 30) == h.EINVAL
+    for t in ("bf16", "fp16", "fp32"):
+        tile = getattr(L, "nntile_hip_sdpa_fwd_tile_cache_" + t)
+        assert tile(None, ctypes.byref(a), 511) == h.EINVAL                      # capacity < k_seq
+        assert tile(None, None, 1024) == h.EINVAL
+        a.head = 48
+        assert tile(None, ctypes.byref(a), 1024) == h.EUNSUPPORTED
+        a.head = 128
