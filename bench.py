@@ -314,12 +314,27 @@ def bench_kv_cache(cfg, steps, warmup):
 
     wall, dev = time_steps(step, steps, warmup)
     _, dev_append = time_steps(append_only, steps, 2)
+    # the same step as a HIP graph (one per cache pair), replayed
+    graphs = []
+    for j in range(nrot):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            appends[j].launch()
+            plans[j].launch()
+        graphs.append(g)
+
+    def replay():
+        graphs[i[0] % nrot].replay()
+        i[0] += 1
+
+    _, dev_graph = time_steps(replay, steps, 5)
     append_bytes = 2 * 2 * k_new.numel() * k_new.element_size()
     nbytes = cfg.algorithmic_bytes() + append_bytes
     return {"what": "append %d new tokens + decode over %d cached rows of %s, cache capacity %d"
                     % (cfg.q_seq, cfg.k_seq, cfg.name, cap),
             "ms_per_step": round(wall, 4), "device_ms_per_step": round(dev, 4),
-            "append_device_ms": round(dev_append, 4), "algorithmic_bytes": nbytes,
+            "append_device_ms": round(dev_append, 4),
+            "graph_replay_device_ms_per_step": round(dev_graph, 4), "algorithmic_bytes": nbytes,
             "gbs": round(nbytes / (dev * 1e-3) / 1e9, 1),
             "frac_of_hbm_peak": round(nbytes / (dev * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
             "reference_copy_out_bytes_not_moved": 2 * 2 * kvb * cfg.k_seq * cfg.head * 2}

@@ -1,0 +1,115 @@
+"""The entry points enqueue kernels and nothing else (no allocation, no
+synchronisation, no memset nodes), so a caller can capture them in a HIP
+graph.  Each graph is replayed several times with eager work and
+synchronisations in between, and every replay is compared with the eager
+result."""
+import pytest
+import torch
+
+from nntile_amd import hip_sdpa
+from . import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _randn(shape, dtype, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return torch.randn(shape, generator=g, device="cuda").to(dtype)
+
+
+def _replays(graph, check, disturb):
+    for _ in range(3):
+        disturb()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        check()
+
+
+def test_decode_step_through_the_cache_in_a_graph():
+    n_batch, n_kv, group, head, cap, old, new = 2, 2, 4, 128, 1024, 600, 16
+    kvb, batch = n_batch * n_kv, n_batch * n_kv * group
+    dt = torch.bfloat16
+    Kc, Vc = _randn((kvb, cap, head), dt, 1), _randn((kvb, cap, head), dt, 2)
+    k_new, v_new = _randn((kvb, new, head), dt, 3), _randn((kvb, new, head), dt, 4)
+    Q = _randn((batch, new, head), dt, 5)
+    k_seq = old + new
+    ws = torch.empty(hip_sdpa.decode_cache_workspace_bytes(k_seq, Q, n_batch, group),
+                     dtype=torch.uint8, device="cuda")
+
+    def step(lse, A):
+        hip_sdpa.kv_cache_append(k_new, v_new, Kc, Vc, old)
+        hip_sdpa.sdpa_fwd_decode_cache(Kc, Vc, k_seq, Q, None, lse, A, hip_sdpa.MASK_CAUSAL, n_batch,
+                                       group, ws, causal_offset=old, flags=hip_sdpa.OVERWRITE)
+
+    lse0, A0 = H.fresh_outputs(batch, new, head, "bf16")
+    step(lse0, A0)
+    torch.cuda.synchronize()
+    lse, A = H.fresh_outputs(batch, new, head, "bf16")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(lse, A)
+
+    def disturb():      # what a replay must restore: the appended rows, the outputs, the workspace
+        Kc[:, old:k_seq].zero_()
+        Vc[:, old:k_seq].zero_()
+        A.fill_(float("nan"))
+        lse.fill_(float("nan"))
+        ws.random_(0, 255)
+
+    def check():
+        assert torch.equal(A.view(torch.int16), A0.view(torch.int16)) and torch.equal(lse, lse0)
+        assert torch.equal(Kc[:, old:k_seq], k_new) and torch.equal(Vc[:, old:k_seq], v_new)
+
+    _replays(graph, check, disturb)
+
+
+def test_prefill_and_backward_in_a_graph():
+    batch, seq, head, tile = 4, 512, 128, 256
+    dt = torch.bfloat16
+    Q, K, V, G = (_randn((batch, seq, head), dt, 10 + i) for i in range(4))
+    split = lambda t: [t[:, s:s + tile].contiguous() for s in range(0, seq, tile)]
+    Qt, Kt, Vt = split(Q), split(K), split(V)
+    nbytes = hip_sdpa.sdpa_bwd_workspace_bytes(seq, seq, batch, hip_sdpa.MASK_CAUSAL)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+
+    def step(lse_t, A_t, A, lse, dK, dQ, dV):
+        hip_sdpa.sdpa_fwd_grid(Kt, Qt, lse_t, Vt, A_t, seq, seq, tile, tile, hip_sdpa.MASK_CAUSAL,
+                               flags=hip_sdpa.OVERWRITE)
+        hip_sdpa.sdpa_fwd_tile(K, Q, None, lse, V, A, hip_sdpa.MASK_CAUSAL, flags=hip_sdpa.OVERWRITE)
+        hip_sdpa.sdpa_bwd_tile(K, Q, V, A, G, None, lse, dK, dQ, dV, hip_sdpa.MASK_CAUSAL,
+                               workspace=ws, flags=hip_sdpa.OVERWRITE)
+
+    def buffers():
+        lse_t = [torch.full((batch, tile), float("nan"), device="cuda") for _ in Qt]
+        A_t = [torch.full_like(q, float("nan")) for q in Qt]
+        A = torch.full_like(Q, float("nan"))
+        lse = torch.full((batch, seq), float("nan"), device="cuda")
+        return lse_t, A_t, A, lse, torch.full_like(Q, float("nan")), torch.full_like(Q, float("nan")), \
+            torch.full_like(Q, float("nan"))
+
+    want = buffers()
+    step(*want)
+    torch.cuda.synchronize()
+    got = buffers()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(*got)
+
+    def flat(b):
+        return list(b[0]) + list(b[1]) + list(b[2:])
+
+    def disturb():
+        for t in flat(got):
+            t.fill_(float("nan"))
+        ws.random_(0, 255)
+
+    def check():
+        for g, w in zip(flat(got), flat(want)):
+            gi = g.view(torch.int16) if g.dtype == dt else g.view(torch.int32)
+            wi = w.view(torch.int16) if w.dtype == dt else w.view(torch.int32)
+            assert torch.equal(gi, wi)
+        # the grid launch and the single-tile launch agree on the forward
+        assert torch.allclose(torch.cat(got[1], dim=1).float(), got[2].float(), rtol=2e-2, atol=2e-2)
+
+    _replays(graph, check, disturb)
