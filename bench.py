@@ -69,7 +69,7 @@ def _randn(shape, dtype, seed):
     return torch.randn(shape, generator=g, device="cuda", dtype=torch.float32).to(dtype)
 
 
-def bench_prefill(cfg, steps, warmup, per_task=False, classified=False):
+def bench_prefill(cfg, steps, warmup, per_task=False, classified=False, streams=1):
     """Fused: one launch for the whole tile grid (analytic causal mask, tile
     skipping).  per_task: the reference's task structure - one launch per
     (query tile, key tile) pair with a materialised additive mask tile, no
@@ -77,7 +77,11 @@ def bench_prefill(cfg, steps, warmup, per_task=False, classified=False):
     classified (with per_task): the mask tiles are classified once, outside the
     timed region, as a layer would when it builds its mask; pairs whose tile
     hides everything are not launched, open and causal ones run without
-    reading the mask."""
+    reading the mask.
+    streams > 1 (with per_task): the tasks of query tile i go to stream
+    i % streams, as StarPU workers with their own streams would run them; tasks
+    that share an (lse, A) tile stay ordered on one stream.  The timed region
+    ends when the launch stream has waited for all of them."""
     import torch
     from nntile_amd import hip_sdpa as h, synth
     dt = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[cfg.dtype]
@@ -106,6 +110,8 @@ def bench_prefill(cfg, steps, warmup, per_task=False, classified=False):
 
     # Calls are prepared once (tile addresses do not change between steps).
     plans = []
+    plan_stream = []
+    side = [torch.cuda.Stream() for _ in range(streams)] if streams > 1 else []
     classes = None
     if per_task and classified:
         t = cfg.seq_tile
@@ -118,6 +124,7 @@ def bench_prefill(cfg, steps, warmup, per_task=False, classified=False):
                     cls = h.TILE_MIXED if classes is None else classes[qi][ki]
                     if cls == h.TILE_HIDDEN:
                         continue
+                    plan_stream.append(qi % streams)
                     if cls == h.TILE_MIXED:
                         plans.append(h.plan_tile(K[ki], Q[qi], masks[qi][ki], lse[qi], V[ki],
                                                  A[qi], h.MASK_ADDITIVE))
@@ -130,8 +137,17 @@ def bench_prefill(cfg, steps, warmup, per_task=False, classified=False):
                                      cfg.seq_tile, h.MASK_CAUSAL, flags=h.OVERWRITE))
 
     def kernels_only():
-        for pl in plans:
-            pl.launch()
+        if not side:
+            for pl in plans:
+                pl.launch()
+            return
+        main = torch.cuda.current_stream()
+        for st in side:
+            st.wait_stream(main)
+        for pl, si in zip(plans, plan_stream):
+            pl.launch(side[si])
+        for st in side:
+            main.wait_stream(st)
 
     def step():
         # per_task: lse must start at -inf each pass; that fill is part of the
@@ -400,6 +416,12 @@ def main():
     if only == "prefill":
         bench_prefill(cfg3, args.steps, args.warmup)
         return
+    if only == "per_task_streams":
+        r = bench_prefill(cfg3, args.steps, args.warmup, per_task=True, classified=True, streams=4)
+        print(json.dumps({k: round(v, 4) for k, v in r.items()}))
+        r = bench_prefill(cfg3, args.steps, args.warmup, per_task=True, streams=4)
+        print(json.dumps({k: round(v, 4) for k, v in r.items()}))
+        return
     if only == "per_task_classified":
         r = bench_prefill(cfg3, args.steps, args.warmup, per_task=True, classified=True)
         print(json.dumps({k: round(v, 4) for k, v in r.items()}))
@@ -439,6 +461,8 @@ def main():
     dec = bench_decode(cfg4, args.steps, args.warmup)
     per_task = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True)
     per_task_cls = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True, classified=True)
+    per_task_cls4 = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True, classified=True,
+                                  streams=4)
     extras = {}
     for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):
         c = BY_NAME[name]
@@ -503,7 +527,10 @@ def main():
                                         "reading the mask",
                                 "launches_per_step": per_task_cls["launches_per_step"],
                                 "ms_per_step": round(per_task_cls["ms_per_step"], 4),
-                                "tflops": round(per_task_cls["tflops"], 2)},
+                                "tflops": round(per_task_cls["tflops"], 2),
+                                "on_4_streams": {"what": "the tasks of query tile i on stream i % 4",
+                                                 "ms_per_step": round(per_task_cls4["ms_per_step"], 4),
+                                                 "tflops": round(per_task_cls4["tflops"], 2)}},
         "other_configs": extras,
         "backward": backward,
         "rope": rope,
