@@ -289,6 +289,36 @@ def bench_transpose(cfg, steps, warmup):
             "frac_of_hbm_peak": round(nbytes / (dev * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
 
 
+def bench_accumulate(cfg, steps, warmup):
+    """The running-pair merge on its own (accumulate_attn_output) on one
+    attention tile of cfg: [head, seq_tile, heads] in the tile type plus the
+    fp32 logsumexp rows.  HBM-bound: reads the two attention tiles and the two
+    lse rows, writes one of each.  Eight buffer sets rotate."""
+    import torch
+    from nntile_amd import hip_sdpa as h
+    dt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg.dtype]
+    nrot = 8
+    shape = (cfg.batch_flat, cfg.seq_tile, cfg.head)
+    src = [_randn(shape, dt, cfg.seed * 1000 + 600 + i) for i in range(nrot)]
+    dst = [_randn(shape, dt, cfg.seed * 1000 + 620 + i) for i in range(nrot)]
+    src_lse = [_randn(shape[:2], torch.float32, cfg.seed * 1000 + 640 + i) for i in range(nrot)]
+    dst_lse = [_randn(shape[:2], torch.float32, cfg.seed * 1000 + 660 + i) for i in range(nrot)]
+    i = [0]
+
+    def step():
+        j = i[0] % nrot
+        h.accumulate_attn_output(src_lse[j], src[j], dst_lse[j], dst[j])
+        i[0] += 1
+
+    wall, dev = time_steps(step, steps, warmup)
+    nbytes = 3 * src[0].numel() * src[0].element_size() + 3 * src_lse[0].numel() * 4
+    return {"what": "accumulate_attn_output on one %d x %d x %d tile of %s"
+                    % (cfg.head, cfg.seq_tile, cfg.batch_flat, cfg.name),
+            "device_ms_per_step": round(dev, 4), "algorithmic_bytes": nbytes,
+            "gbs": round(nbytes / (dev * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(nbytes / (dev * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+
+
 def bench_kv_cache(cfg, steps, warmup):
     """One decode step through a preallocated key/value cache: the keys and
     values of the q_seq new tokens are appended (one launch for both), then
@@ -394,7 +424,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run only this leg: prefill | decode | per_task | backward | rope | transpose | kv_cache | extras | copy (for profiling)")
+                    help="run only this leg: prefill | decode | per_task | backward | rope | transpose | accumulate | kv_cache | extras | copy (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
@@ -450,6 +480,9 @@ def main():
     if only == "rope":
         print(json.dumps(bench_rope(cfg3, args.steps, args.warmup)))
         return
+    if only == "accumulate":
+        print(json.dumps(bench_accumulate(cfg3, args.steps, args.warmup)))
+        return
     if only == "kv_cache":
         print(json.dumps(bench_kv_cache(cfg4, args.steps, args.warmup)))
         return
@@ -478,6 +511,7 @@ def main():
     rope = bench_rope(cfg3, max(5, args.steps // 5), 5)
     transpose = bench_transpose(cfg3, max(5, args.steps // 5), 5)
     kv_cache = bench_kv_cache(cfg4, max(5, args.steps // 5), 5)
+    accumulate = bench_accumulate(cfg3, max(5, args.steps // 5), 5)
     # The headline leg runs last: the first timed loop of a process measures
     # 5 % slower than the same loop a second later (clocks still settling),
     # whatever the warmup count.
@@ -536,6 +570,7 @@ def main():
         "rope": rope,
         "transpose": transpose,
         "kv_cache": kv_cache,
+        "accumulate_attn_output": accumulate,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg3)
