@@ -117,8 +117,22 @@ def bench_prefill(cfg, steps, warmup, per_task=False, classified=False, streams=
         t = cfg.seq_tile
         classes = [[h.mask_tile_class(masks[qi][ki], (qi - ki) * t) for ki in range(nt)]
                    for qi in range(nt)]
+    whole = None
+    if classes is not None:
+        # what tensor::flash_sdpa_mask_rule decides from the classes: a mask
+        # that is the causal rule itself needs no tasks per pair
+        t = cfg.seq_tile
+        expect = [[h.TILE_OPEN if (ki + 1) * t - 1 <= qi * t else
+                   (h.TILE_HIDDEN if ki * t > (qi + 1) * t - 1 else h.TILE_CAUSAL)
+                   for ki in range(nt)] for qi in range(nt)]
+        if classes == expect:
+            whole = h.MASK_CAUSAL
     for Q, K, V, A, lse in calls:
-        if per_task:
+        if whole is not None:
+            plan_stream.append(0)
+            plans.append(h.plan_grid(K, Q, lse, V, A, cfg.q_seq, cfg.k_seq, cfg.seq_tile,
+                                     cfg.seq_tile, whole))
+        elif per_task:
             for qi in range(nt):
                 for ki in range(nt):
                     cls = h.TILE_MIXED if classes is None else classes[qi][ki]
@@ -447,8 +461,6 @@ def main():
         bench_prefill(cfg3, args.steps, args.warmup)
         return
     if only == "per_task_streams":
-        r = bench_prefill(cfg3, args.steps, args.warmup, per_task=True, classified=True, streams=4)
-        print(json.dumps({k: round(v, 4) for k, v in r.items()}))
         r = bench_prefill(cfg3, args.steps, args.warmup, per_task=True, streams=4)
         print(json.dumps({k: round(v, 4) for k, v in r.items()}))
         return
@@ -494,8 +506,7 @@ def main():
     dec = bench_decode(cfg4, args.steps, args.warmup)
     per_task = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True)
     per_task_cls = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True, classified=True)
-    per_task_cls4 = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True, classified=True,
-                                  streams=4)
+    per_task4 = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True, streams=4)
     extras = {}
     for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):
         c = BY_NAME[name]
@@ -555,16 +566,17 @@ def main():
         "per_task_path": {"what": "cfg3 as the reference submits it: 16 launches, additive mask "
                                   "tiles, no skipping, (lse, A) handed over in bf16",
                           "ms_per_step": round(per_task["ms_per_step"], 4),
-                          "tflops": round(per_task["tflops"], 2)},
-        "per_task_classified": {"what": "the same 16 tile pairs with the mask tiles classified once: "
-                                        "hidden pairs not launched, open and causal ones without "
-                                        "reading the mask",
+                          "tflops": round(per_task["tflops"], 2),
+                          "on_4_streams": {"what": "the tasks of query tile i on stream i % 4",
+                                           "ms_per_step": round(per_task4["ms_per_step"], 4),
+                                           "tflops": round(per_task4["tflops"], 2)}},
+        "per_task_classified": {"what": "the same tensors and materialised mask with the mask tiles "
+                                        "classified once: the classes say the mask is the causal "
+                                        "rule itself, so one launch merges all key tiles into all "
+                                        "query tiles (lse filled with -inf first, as for the tasks)",
                                 "launches_per_step": per_task_cls["launches_per_step"],
                                 "ms_per_step": round(per_task_cls["ms_per_step"], 4),
-                                "tflops": round(per_task_cls["tflops"], 2),
-                                "on_4_streams": {"what": "the tasks of query tile i on stream i % 4",
-                                                 "ms_per_step": round(per_task_cls4["ms_per_step"], 4),
-                                                 "tflops": round(per_task_cls4["tflops"], 2)}},
+                                "tflops": round(per_task_cls["tflops"], 2)},
         "other_configs": extras,
         "backward": backward,
         "rope": rope,

@@ -868,6 +868,33 @@ std::vector<int> flash_sdpa_mask_classes(const Tensor<T> &mask, Index causal_off
     return classes;
 }
 
+// What the classes say about the mask as a whole: NNTILE_HIP_MASK_NONE when
+// every tile is open, NNTILE_HIP_MASK_CAUSAL when every tile is what the rule
+// key <= query + causal_offset makes of it (open below the diagonal band,
+// hidden above, exactly on the rule where the band crosses), -1 otherwise.
+// Classes are exact statements about every element, so the answer is too.
+int flash_sdpa_mask_rule(const TensorTraits &mask, const std::vector<int> &mask_classes,
+        Index causal_offset)
+{
+    bool all_open = true, on_rule = true;
+    for(Index i = 0; i < mask.grid.nelems; ++i)
+    {
+        const auto index = mask.grid.linear_to_index(i);
+        const Index k0 = index[0] * mask.basetile_shape[0];
+        const Index q0 = index[1] * mask.basetile_shape[1];
+        const Index k_len = std::min(mask.basetile_shape[0], mask.shape[0] - k0);
+        const Index q_len = std::min(mask.basetile_shape[1], mask.shape[1] - q0);
+        // the rule inside the tile: visible <=> k0 + k <= q0 + q + causal_offset
+        const bool rule_all_visible = k0 + k_len - 1 <= q0 + causal_offset;
+        const bool rule_all_hidden = k0 > q0 + q_len - 1 + causal_offset;
+        const int expected = rule_all_visible ? NNTILE_HIP_MASK_TILE_OPEN
+            : (rule_all_hidden ? NNTILE_HIP_MASK_TILE_HIDDEN : NNTILE_HIP_MASK_TILE_CAUSAL);
+        all_open = all_open && mask_classes[i] == NNTILE_HIP_MASK_TILE_OPEN;
+        on_rule = on_rule && mask_classes[i] == expected;
+    }
+    return all_open ? NNTILE_HIP_MASK_NONE : (on_rule ? NNTILE_HIP_MASK_CAUSAL : -1);
+}
+
 template<typename T>
 Index flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &mask, const std::vector<int> &mask_classes,
@@ -879,6 +906,16 @@ Index flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
             "one class per mask tile is required");
     const Index num_k_seq_tiles = K.grid.shape[1];
     const Index q_tile = Q.basetile_shape[1], k_tile = K.basetile_shape[1];
+    // A mask that is the causal rule itself, or hides nothing, needs no tasks
+    // per pair: one launch per slab of the batch grid merges all key tiles
+    // into all query tiles.
+    const int whole = flash_sdpa_mask_rule(mask, mask_classes, causal_offset);
+    if(whole >= 0 && Q.grid.shape[1] <= NNTILE_HIP_SDPA_MAX_TILES
+            && num_k_seq_tiles <= NNTILE_HIP_SDPA_MAX_TILES)
+    {
+        flash_sdpa_fwd_hip_async<T>(K, Q, whole, causal_offset, logsumexp, V, A, false);
+        return Q.grid.shape[2] * Q.grid.shape[3] * Q.grid.shape[4];
+    }
     Index submitted = 0;
     for(Index a_linear = 0; a_linear < A.grid.nelems; ++a_linear)
     {

@@ -272,11 +272,18 @@ void flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
 template<typename T>
 std::vector<int> flash_sdpa_mask_classes(const Tensor<T> &mask, Index causal_offset);
 
-//! flash_sdpa_fwd_cudnn_async that uses those classes: a pair whose mask tile
-//! hides everything is not submitted, a pair whose mask tile hides nothing
-//! runs without a mask, a pair on the causal rule runs with the analytic
-//! mask, the rest as in the reference.  Returns the number of tile pairs
-//! submitted.
+//! NNTILE_HIP_MASK_NONE if the classes say the mask hides nothing,
+//! NNTILE_HIP_MASK_CAUSAL if they say it is exactly the rule key <= query +
+//! causal_offset, -1 otherwise
+int flash_sdpa_mask_rule(const TensorTraits &mask, const std::vector<int> &mask_classes,
+        Index causal_offset);
+
+//! flash_sdpa_fwd_cudnn_async that uses those classes.  A mask that is the
+//! causal rule itself (or hides nothing) runs as flash_sdpa_fwd_hip_async:
+//! one launch per slab of the batch grid.  Otherwise, per pair: a mask tile
+//! that hides everything - nothing submitted; one that hides nothing - no
+//! mask; one on the causal rule - the analytic mask; the rest as in the
+//! reference.  Returns the number of launches.
 template<typename T>
 Index flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &mask, const std::vector<int> &mask_classes,

@@ -80,13 +80,17 @@ def _read(dtype, A, lse, head, seq):
 @pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
 @pytest.mark.parametrize("kind,want_classes", [
     ("causal", {"hidden": 6, "open": 6, "causal": 4, "mixed": 0}),
-    ("window", None), ("full", {"hidden": 0, "open": 16, "causal": 0, "mixed": 0})])
+    ("window", None), ("full", {"hidden": 0, "open": 16, "causal": 0, "mixed": 0}),
+    ("causal_dent", {"hidden": 6, "open": 5, "causal": 4, "mixed": 1})])
 def test_classified_submission_equals_the_reference_submission(oracle, dtype, kind, want_classes):
     head, seq, nb, grp, nkv, tile = 64, 512, 2, 1, 2, 128
     arrs, (qf, kf, vf) = _case(dtype, head, seq, nb, grp, nkv, seed=11)
     k, q = np.arange(seq)[None, :], np.arange(seq)[:, None]
     mask = {"causal": synth.causal_mask(seq, seq), "window": np.abs(k - q) <= 100,
-            "full": np.ones((seq, seq), bool)}[kind]                           # [q, k]
+            "full": np.ones((seq, seq), bool), "causal_dent": synth.causal_mask(seq, seq)}[kind]  # [q, k]
+    if kind == "causal_dent":
+        mask = mask.copy()
+        mask[400, 3] = False            # one key hidden far below the diagonal
     want, want_lse = oracle.sdpa_vanilla(kf, qf, vf, mask, k_tile=tile)
     # the reference's submission: every pair with its mask tile
     T, A0, lse0, M = _tensors(dtype, arrs, mask, head, seq, nb, grp, nkv, tile)
@@ -112,7 +116,11 @@ def test_classified_submission_equals_the_reference_submission(oracle, dtype, ki
     else:
         assert count["hidden"] > 0 and count["mixed"] > 0
     slabs = A1.ntiles // n_t
-    assert submitted == slabs * (n_t * n_t - count["hidden"])
+    if kind in ("causal", "full"):
+        # the mask is the causal rule itself / hides nothing: one launch per slab
+        assert submitted == slabs
+    else:
+        assert submitted == slabs * (n_t * n_t - count["hidden"])
     assert H.rel_fro(got_a, want) < H.TOL[dtype] and H.rel_fro(got_lse, want_lse) < H.TOL[dtype]
     assert H.rel_fro(got_a, ref_a) < H.TOL[dtype] and H.rel_fro(got_lse, ref_lse) < H.TOL[dtype]
 
