@@ -31,8 +31,8 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # WRITE_SIZE x 1.000, the factors a 1 GiB device copy calibrates); the runs
 # and their figures are in profiles/sdpa_*_kernel_cfg*.txt.  They are
 # properties of the kernel and the workload, not of one timing run.
-TRAFFIC_PREFILL_CFG3 = 175215798
-TRAFFIC_DECODE_CFG4 = 295683173
+TRAFFIC_PREFILL_CFG3 = 175220098
+TRAFFIC_DECODE_CFG4 = 295683470
 
 
 def time_steps(step, steps, warmup):
