@@ -215,6 +215,26 @@ int64_t run_classified(AnyTensor *K, AnyTensor *Q, AnyTensor *mask, AnyTensor *l
 extern "C"
 {
 
+// tensor::flash_sdpa_mask_rule on a [k_seq, q_seq] mask tiled [k_tile, q_tile]
+// (no device memory): *rule = NNTILE_HIP_MASK_NONE, NNTILE_HIP_MASK_CAUSAL or -1
+int nntile_host_mask_rule(int64_t k_seq, int64_t q_seq, int64_t k_tile, int64_t q_tile,
+        const int32_t *classes, int64_t n_classes, int64_t offset, int32_t *rule,
+        char *err, int errlen)
+{
+    try
+    {
+        const tensor::TensorTraits mask({k_seq, q_seq}, {k_tile, q_tile});
+        if(n_classes != mask.grid.nelems)
+        {
+            throw std::runtime_error("one class per mask tile is required");
+        }
+        const std::vector<int> cls(classes, classes + n_classes);
+        *rule = tensor::flash_sdpa_mask_rule(mask, cls, offset);
+        return 0;
+    }
+    catch(const std::exception &e) { return fail(err, errlen, e); }
+}
+
 // tensor::flash_sdpa_mask_classes, then tensor::flash_sdpa_fwd_cudnn_async
 // with those classes + wait.  classes (may be null): room for n_classes
 // values, one per mask tile in the linear order of the mask's grid;

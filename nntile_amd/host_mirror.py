@@ -38,6 +38,9 @@ def lib():
         L.nntile_host_flash_sdpa_fwd_classified.argtypes = [
             ctypes.c_int, vp, vp, vp, vp, vp, vp, i64, ctypes.POINTER(ctypes.c_int32), i64,
             ctypes.POINTER(i64), ctypes.c_char_p, ctypes.c_int]
+        L.nntile_host_mask_rule.argtypes = [i64, i64, i64, i64, ctypes.POINTER(ctypes.c_int32), i64,
+                                            i64, ctypes.POINTER(ctypes.c_int32), ctypes.c_char_p,
+                                            ctypes.c_int]
         L.nntile_host_check_shapes.argtypes = [ctypes.c_int, ctypes.POINTER(i64), ctypes.c_char_p,
                                                ctypes.c_int]
         L.nntile_host_flash_sdpa_bwd.argtypes = [ctypes.c_int, ctypes.c_int] + [vp] * 10 + [
@@ -108,6 +111,17 @@ class Tensor:
 def flash_sdpa_fwd(op, K, Q, mask, lse, V, A, mask_mode=0, offset=0, overwrite=False):
     _call(lib().nntile_host_flash_sdpa_fwd, op, DTYPES[Q.dtype], K.h, Q.h,
           None if mask is None else mask.h, lse.h, V.h, A.h, mask_mode, offset, int(overwrite))
+
+
+def mask_rule(k_seq, q_seq, k_tile, q_tile, classes, offset=0):
+    """tensor::flash_sdpa_mask_rule: what the classes of a [k_seq, q_seq] mask's
+    tiles (linear order of its grid, key tile fastest) say about the whole
+    mask: 1 (MASK_NONE), 2 (MASK_CAUSAL with `offset`) or -1."""
+    arr = (ctypes.c_int32 * len(classes))(*classes)
+    out = ctypes.c_int32(-9)
+    _call(lib().nntile_host_mask_rule, k_seq, q_seq, k_tile, q_tile, arr, len(classes), offset,
+          ctypes.byref(out))
+    return out.value
 
 
 def flash_sdpa_fwd_classified(K, Q, mask, lse, V, A, offset=0):

@@ -102,3 +102,44 @@ def test_argument_checks_before_any_launch():
         assert f(None, 4, 4, 4096, 0, 4098, ctypes.byref(out)) == h.EINVAL        # misaligned word
         assert f(None, 4, 4, 4096, 0, 4096, None) == h.EINVAL
     assert out.value == -7
+
+
+def _classes(oracle, mask_kq, k_tile, q_tile, offset):
+    """Classes of the tiles of a [k, q] mask in the grid's linear order (key
+    tile fastest), each against the rule moved into the tile."""
+    k_seq, q_seq = mask_kq.shape
+    out = []
+    for q0 in range(0, q_seq, q_tile):
+        for k0 in range(0, k_seq, k_tile):
+            out.append(oracle.mask_tile_class(mask_kq[k0:k0 + k_tile, q0:q0 + q_tile],
+                                              q0 - k0 + offset))
+    return out
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_whole_mask_rule_from_the_classes(oracle, seed):
+    """tensor::flash_sdpa_mask_rule (host library, no GPU): the classes of a
+    mask that is the causal rule say so on any tiling, ragged last tiles
+    included; one element off the rule anywhere and they do not."""
+    from nntile_amd import host_mirror as hm
+    rng = np.random.default_rng(seed)
+    k_seq, q_seq = int(rng.integers(3, 40)), int(rng.integers(3, 40))
+    k_tile, q_tile = int(rng.integers(1, k_seq + 1)), int(rng.integers(1, q_seq + 1))
+    offset = int(rng.integers(-q_seq, k_seq))
+    k, q = np.arange(k_seq)[:, None], np.arange(q_seq)[None, :]
+    rule = k <= q + offset
+    cls = _classes(oracle, rule, k_tile, q_tile, offset)
+    want = 1
+    if not rule.all():
+        want = 2
+    assert hm.mask_rule(k_seq, q_seq, k_tile, q_tile, cls, offset) == want
+    if rule.any() and not rule.all():
+        dent = rule.copy()
+        dent[rng.integers(k_seq), rng.integers(q_seq)] ^= True
+        cls = _classes(oracle, dent, k_tile, q_tile, offset)
+        got = hm.mask_rule(k_seq, q_seq, k_tile, q_tile, cls, offset)
+        assert got == (1 if dent.all() else -1)
+    open_cls = _classes(oracle, np.ones((k_seq, q_seq), bool), k_tile, q_tile, offset)
+    assert hm.mask_rule(k_seq, q_seq, k_tile, q_tile, open_cls, offset) == 1
+    with pytest.raises(hm.HostError):
+        hm.mask_rule(k_seq, q_seq, k_tile, q_tile, open_cls + [1], offset)
