@@ -78,7 +78,9 @@ template<int N> __device__ __forceinline__ void wait_vmcnt()
     asm volatile("" ::: "memory");
 }
 
-template<typename T, int HEAD, int MODE, int STAGES>
+// DIRECT: the unit has one key split, so the partial is the result and is
+// folded into (lse, A) here; no partials are written and no merge kernel runs.
+template<typename T, int HEAD, int MODE, int STAGES, bool DIRECT = false>
 __global__ __launch_bounds__(kDecThreads, NNTILE_DEC_WGS_PER_CU)
 void sdpa_decode_16bit_kernel(const DecodeParams p)
 {
@@ -456,6 +458,61 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
     {
         return;
     }
+    if constexpr(DIRECT)
+    {
+        const int g = rr / (int)p.q_seq, tok = rr % (int)p.q_seq;
+        const int64_t qb = nb + (int64_t)p.n_batch * (g + (int64_t)p.kv_group * hkv);
+        const int64_t row = qb * p.q_seq + tok;
+        uint16_t *Adst = static_cast<uint16_t *>(p.A) + row * HEAD + 4 * quad;
+        if(m_run == neg_inf() || !(l_tot > 0.0f))
+        {
+            // no visible key at all: leave lse and A untouched, or write the
+            // empty row when the running pair is being overwritten
+            if(p.overwrite)
+            {
+#pragma unroll
+                for(int db = 0; db < DBLOCKS; ++db)
+                {
+                    *reinterpret_cast<u32x2 *>(Adst + 16 * db) = u32x2{0, 0};
+                }
+                if(quad == 0)
+                {
+                    p.lse[row] = neg_inf();
+                }
+            }
+            return;
+        }
+        const float to_ln = EXPLICIT ? 1.0f : p.scale;
+        const float lse_new = m_run * to_ln + __logf(l_tot);
+        const float lse_old = p.overwrite ? neg_inf() : p.lse[row];
+        float w_old, w_new, lse_out;
+        merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
+        const float sc = w_new / l_tot;
+#pragma unroll
+        for(int db = 0; db < DBLOCKS; ++db)
+        {
+            float v[4] = {o[db][0] * sc, o[db][1] * sc, o[db][2] * sc, o[db][3] * sc};
+            if(w_old != 0.0f)
+            {
+                const u32x2 old = *reinterpret_cast<const u32x2 *>(Adst + 16 * db);
+                v[0] += w_old * T::to_float((uint16_t)(old[0] & 0xffffu));
+                v[1] += w_old * T::to_float((uint16_t)(old[0] >> 16));
+                v[2] += w_old * T::to_float((uint16_t)(old[1] & 0xffffu));
+                v[3] += w_old * T::to_float((uint16_t)(old[1] >> 16));
+            }
+            u32x2 w;
+            w[0] = T::pack2(v[0], v[1]);
+            w[1] = T::pack2(v[2], v[3]);
+            *reinterpret_cast<u32x2 *>(Adst + 16 * db) = w;
+        }
+        // The four lanes of a row sit in one wavefront and run in lock step:
+        // all of them have read lse_old by now.
+        if(quad == 0)
+        {
+            p.lse[row] = lse_out;
+        }
+        return;
+    }
     const int64_t prow = ((int64_t)unit * p.n_splits + split) * p.rows + rr;
     if(quad == 0)
     {
@@ -643,6 +700,12 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
 template<typename T, int HEAD, int MODE, int STAGES>
 static void launch_decode_main(hipStream_t stream, const DecodeParams &p, dim3 grid)
 {
+    if(p.n_splits == 1)
+    {
+        auto kernel = sdpa_decode_16bit_kernel<T, HEAD, MODE, STAGES, true>;
+        hipLaunchKernelGGL(kernel, grid, dim3(kDecThreads), 0, stream, p);
+        return;
+    }
     auto kernel = sdpa_decode_16bit_kernel<T, HEAD, MODE, STAGES>;
     hipLaunchKernelGGL(kernel, grid, dim3(kDecThreads), 0, stream, p);
 }
@@ -673,6 +736,7 @@ static int launch_decode_stages(hipStream_t stream, const DecodeParams &p, int m
     {
         return NNTILE_HIP_ELAUNCH;
     }
+    if(p.n_splits > 1)
     {
         constexpr int rows_per_wg = 256 / (HEAD / 4);
         const int64_t total_rows = (int64_t)units * p.rows;

@@ -423,3 +423,30 @@ def test_explicit_mask_scan_paths(oracle, dtype, form, q_seq, k_seq, pattern):
     got2, got2_lse = H.to_np(A2), H.to_np(lse2)
     assert np.all(got2[:, ~vis] == 0) and np.all(np.isneginf(got2_lse[:, ~vis]))
     assert np.array_equal(got2[:, vis], got[:, vis]) and np.array_equal(got2_lse[:, vis], got_lse[:, vis])
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("overwrite", [True, False])
+def test_decode_with_one_key_split_per_unit(oracle, dtype, overwrite):
+    """512 (batch, kv head) units: every unit gets one key split and the main
+    kernel writes (lse, A) itself.  Both forms: overwrite, and two calls over
+    two halves of the keys merged into the running pair."""
+    q_seq, k_seq, n_batch, group, n_kv, head = 3, 200, 64, 2, 8, 64
+    batch = n_batch * group * n_kv
+    (Q, K, V), f32 = H.make_qkv(23, batch, q_seq, k_seq, head, dtype, kv_batch=n_batch * n_kv)
+    offset = k_seq - q_seq
+    want, want_lse = _oracle(oracle, f32, synth.causal_mask(q_seq, k_seq, offset),
+                             n_batch=n_batch, kv_repeat=group)
+    Qd = Q.cuda()
+    lse, A = H.fresh_outputs(batch, q_seq, head, dtype)
+    pieces = [(0, k_seq)] if overwrite else [(96, k_seq), (0, 96)]
+    for lo, hi in pieces:
+        Kd, Vd = K[:, lo:hi].contiguous().cuda(), V[:, lo:hi].contiguous().cuda()
+        ws = torch.empty(hip_sdpa.decode_workspace_bytes(Kd, Qd, n_batch, group),
+                         dtype=torch.uint8, device="cuda")
+        hip_sdpa.sdpa_fwd_decode(Kd, Qd, None, lse, Vd, A, hip_sdpa.MASK_CAUSAL, n_batch, group, ws,
+                                 k_pos0=lo, causal_offset=offset,
+                                 flags=hip_sdpa.OVERWRITE if overwrite else 0)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
