@@ -438,7 +438,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run only this leg: prefill | decode | per_task | backward | rope | transpose | accumulate | kv_cache | extras | copy (for profiling)")
+                    help="run only this leg: prefill | decode | decode_wide | per_task | backward | rope | transpose | accumulate | kv_cache | extras | copy (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
@@ -492,6 +492,13 @@ def main():
     if only == "rope":
         print(json.dumps(bench_rope(cfg3, args.steps, args.warmup)))
         return
+    if only == "decode_wide":
+        from nntile_amd.configs import Workload
+        wide = Workload("cfg4_bytes_as_64_sequences_of_1024_keys", "bf16", 128, 16, 1024, 64, 4, 8,
+                        1024, 1, 45, decode=True)
+        r = bench_decode(wide, args.steps, args.warmup)
+        print(json.dumps({k: round(v, 4) for k, v in r.items()}))
+        return
     if only == "accumulate":
         print(json.dumps(bench_accumulate(cfg3, args.steps, args.warmup)))
         return
@@ -504,6 +511,12 @@ def main():
         return
 
     dec = bench_decode(cfg4, args.steps, args.warmup)
+    # the same bytes as 64 sequences of 1024 cached keys: 512 (sequence, kv
+    # head) units, one key split each, (lse, A) written by the main kernel
+    from nntile_amd.configs import Workload
+    cfg4_wide = Workload("cfg4_bytes_as_64_sequences_of_1024_keys", "bf16", 128, 16, 1024, 64, 4, 8,
+                         1024, 1, 45, decode=True)
+    dec_wide = bench_decode(cfg4_wide, max(5, args.steps // 5), 5)
     per_task = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True)
     per_task_cls = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True, classified=True)
     per_task4 = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True, streams=4)
@@ -563,6 +576,14 @@ def main():
                                 "algorithmic_bytes": dec["algorithmic_bytes"],
                                 "workspace_bytes": dec["workspace_bytes"],
                                 "kernel_ms": round(dec["kernel_ms_per_step"], 4)}},
+        "decode_many_sequences": {"workload": cfg4_wide.name,
+                                  "what": "for information: cfg4's bytes as 64 sequences x 8 kv heads x "
+                                          "1024 keys, 16 new tokens each; one key split per unit, no "
+                                          "merge launch",
+                                  "kernel_ms": round(dec_wide["kernel_ms_per_step"], 4),
+                                  "algorithmic_bytes": dec_wide["algorithmic_bytes"],
+                                  "gbs": round(dec_wide["kernel_gbs"], 1),
+                                  "frac_of_hbm_peak": round(dec_wide["kernel_gbs"] / PEAK_HBM_GBS, 4)},
         "per_task_path": {"what": "cfg3 as the reference submits it: 16 launches, additive mask "
                                   "tiles, no skipping, (lse, A) handed over in bf16",
                           "ms_per_step": round(per_task["ms_per_step"], 4),
