@@ -2,8 +2,11 @@
  *
  * One shared library, libnntile_hip_sdpa.so, plain pointers and sizes only.
  * Every entry point only ENQUEUES work on the HIP stream it is given: it never
- * synchronises, never allocates and never frees.  Return value: 0 on success,
- * a negative NNTILE_HIP_E* code otherwise (nothing is enqueued on error).
+ * allocates, never frees and - with one exception, the mask classification
+ * nntile_hip_mask_tile_class_* of section 10, which hands a value back to the
+ * host and therefore waits for the stream - never synchronises.  Return
+ * value: 0 on success, a negative NNTILE_HIP_E* code otherwise (nothing is
+ * enqueued on error).
  *
  * Data layout (NNTile tiles are Fortran-ordered):
  *   K, V       [head, k_seq, kv_batch]   element (h, s, b) at h + head*(s + k_seq*b)
@@ -116,9 +119,11 @@ int nntile_hip_sdpa_fwd_tile_fp32(void *stream, const nntile_hip_sdpa_tile_args 
 /* ---- 2b. backward of one (query tile, key tile) pair ------------------------
  * Replaces kernel::flash_sdpa_bwd_cudnn::execute_graph<T>
  * (include/nntile/kernel/flash_sdpa_bwd_cudnn/cuda.hh:44-68,
- *  src/kernel/flash_sdpa_bwd_cudnn/cuda.cc:171-218): same argument order and
- * meaning, the cuDNN handle/graph pair replaced by the stream and the cuDNN
- * workspace dropped.  The forward output A and the logsumexp are inputs; the
+ *  src/kernel/flash_sdpa_bwd_cudnn/cuda.cc:171-218): the reference's argument
+ * order and meaning MINUS ITS LAST ARGUMENT - the cuDNN handle/graph pair is
+ * replaced by the stream, and the trailing `void *workspace` (cuDNN's own
+ * scratch, cuda.hh:58) has no counterpart and is dropped: seq, head, batch
+ * and the 13 tile pointers are the reference's, in its order.  The forward output A and the logsumexp are inputs; the
  * gradients of this tile pair are ADDED to dK, dQ, dV (the reference computes
  * them into the scratch tiles and adds those, cuda.cc:213-217).  scratch_dK
  * and scratch_dV are accepted for signature compatibility and never touched;
@@ -213,6 +218,27 @@ int nntile_hip_sdpa_fwd_decode_bf16(void *stream, const nntile_hip_sdpa_tile_arg
         void *workspace, size_t workspace_bytes);
 int nntile_hip_sdpa_fwd_decode_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
         void *workspace, size_t workspace_bytes);
+
+/* ---- 4b. decode for callers that cannot allocate -------------------------------
+ * No counterpart in the reference.  For callers that cannot call hipMalloc
+ * and have no scratch buffer to pass: work under HIP graph capture, tight
+ * serving loops, harnesses that forbid allocation.  Same computation and
+ * result as nntile_hip_sdpa_fwd_decode_{bf16,fp16} (dtype picks the tile
+ * type), with the split partials in a device array that is part of the
+ * library's code object: NNTILE_HIP_DECODE_STATIC_SCRATCH_BYTES per GPU,
+ * held from the library's load until the process ends.  The call allocates
+ * and frees nothing.  A shape whose partials need more
+ * (nntile_hip_sdpa_fwd_decode_workspace_bytes(args) tells) is refused with
+ * NNTILE_HIP_EWORKSPACE and a line on stderr.  The array's address on the
+ * current device is looked up on the first call made with that device current
+ * (make that call outside a capture); the stream must belong to the current
+ * device.  All calls on one GPU share the array: two of them in flight at the
+ * same time (different streams) race, calls on one stream do not. */
+#define NNTILE_HIP_DECODE_STATIC_SCRATCH_BYTES (16u << 20)
+#define NNTILE_HIP_DTYPE_BF16 0
+#define NNTILE_HIP_DTYPE_FP16 1
+int nntile_hip_sdpa_fwd_decode_static(void *stream, int32_t dtype,
+        const nntile_hip_sdpa_tile_args *args);
 
 /* ---- 5. the running-statistics hand-off on its own ---------------------------
  * Replaces kernel::accumulate_attn_output::cuda<T>

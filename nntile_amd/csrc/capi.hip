@@ -1,6 +1,8 @@
 // C ABI of libnntile_hip_sdpa.so: argument checks and dispatch to the kernels.
+#include <atomic>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "sdpa_common.hpp"
 
@@ -389,6 +391,85 @@ static int decode_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *
         : launch_decode_16bit<Fp16>(s, p, (int)a->head, a->mask_mode);
 }
 
+// ---- decode with the split partials in memory the library owns ---------------
+// For callers that may not allocate (a stream under graph capture, a serving
+// loop that forbids it): the workspace of decode_call is this file-scope
+// device array instead of a caller's buffer.  Every GPU holds its own copy at
+// its own address; in host code the array's name is only a handle for
+// hipGetSymbolAddress, never an address to pass on.  The decode kernels write
+// every partial they later read, so nothing has to be cleared between calls;
+// calls that overlap on one GPU share the array and race.
+static __device__ __align__(256) unsigned char scratch[NNTILE_HIP_DECODE_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void *> scratch_ptr[kMaxDevices];
+static std::mutex scratch_mutex;
+
+// Device address of `scratch` on the current device, resolved on the first
+// call per device.
+static int static_scratch(void **out)
+{
+    int dev = -1;
+    if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    {
+        return NNTILE_HIP_ELAUNCH;
+    }
+    void *ptr = scratch_ptr[dev].load(std::memory_order_acquire);
+    if(ptr == nullptr)
+    {
+        std::lock_guard<std::mutex> guard(scratch_mutex);
+        ptr = scratch_ptr[dev].load(std::memory_order_acquire);
+        if(ptr == nullptr)
+        {
+            if(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess
+                    || ptr == nullptr)
+            {
+                (void)hipGetLastError();
+                return NNTILE_HIP_ELAUNCH;
+            }
+            scratch_ptr[dev].store(ptr, std::memory_order_release);
+        }
+    }
+    *out = ptr;
+    return NNTILE_HIP_OK;
+}
+
+static int decode_static_call(void *stream, int32_t dtype,
+        const nntile_hip_sdpa_tile_args *a)
+{
+    if(dtype != NNTILE_HIP_DTYPE_BF16 && dtype != NNTILE_HIP_DTYPE_FP16)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(!decode_args_ok(a))
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(a->head != 64 && a->head != 128)
+    {
+        return NNTILE_HIP_EUNSUPPORTED;
+    }
+    int units, n_steps, splits, rows;
+    decode_geometry(a, units, n_steps, splits, rows);
+    const size_t need = decode_workspace_bytes(units, splits, rows, (int)a->head);
+    if(need > (size_t)NNTILE_HIP_DECODE_STATIC_SCRATCH_BYTES)
+    {
+        std::fprintf(stderr, "nntile_hip_sdpa_fwd_decode_static: the split partials of this "
+                "shape need %zu bytes, the library's own buffer holds %zu; use "
+                "nntile_hip_sdpa_fwd_decode_* with a workspace\n", need,
+                (size_t)NNTILE_HIP_DECODE_STATIC_SCRATCH_BYTES);
+        return NNTILE_HIP_EWORKSPACE;
+    }
+    void *ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if(rc != NNTILE_HIP_OK)
+    {
+        return rc;
+    }
+    return decode_call(dtype == NNTILE_HIP_DTYPE_BF16 ? DType::bf16 : DType::fp16, stream, a,
+            a->k_seq, ws, (size_t)NNTILE_HIP_DECODE_STATIC_SCRATCH_BYTES);
+}
+
 template<typename S>
 static int accumulate_call(void *stream, int64_t head, int64_t seq,
         int64_t batch, const float *src_lse, const void *src_attn,
@@ -679,6 +760,12 @@ int nntile_hip_sdpa_fwd_decode_fp16(void *stream, const nntile_hip_sdpa_tile_arg
 {
     return decode_call(DType::fp16, stream, args, args ? args->k_seq : 0, workspace,
             workspace_bytes);
+}
+
+int nntile_hip_sdpa_fwd_decode_static(void *stream, int32_t dtype,
+        const nntile_hip_sdpa_tile_args *args)
+{
+    return decode_static_call(stream, dtype, args);
 }
 
 int nntile_hip_accumulate_attn_output_bf16(void *stream, int64_t head, int64_t seq,

@@ -78,7 +78,7 @@ EXPORTS = (
     + ["nntile_hip_sdpa_fwd_tile_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_fwd_grid_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_fwd_decode_" + t for t in ("bf16", "fp16")]
-    + ["nntile_hip_sdpa_fwd_decode_workspace_bytes"]
+    + ["nntile_hip_sdpa_fwd_decode_workspace_bytes", "nntile_hip_sdpa_fwd_decode_static"]
     + ["nntile_hip_flash_sdpa_bwd_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_sdpa_bwd_tile_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_sdpa_bwd_workspace_bytes"]
@@ -160,6 +160,9 @@ def lib():
         L.nntile_hip_sdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.argtypes = [ctypes.POINTER(TileArgs)]
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.restype = ctypes.c_size_t
+        L.nntile_hip_sdpa_fwd_decode_static.argtypes = [_vp, ctypes.c_int32,
+                                                        ctypes.POINTER(TileArgs)]
+        L.nntile_hip_sdpa_fwd_decode_static.restype = ctypes.c_int
         L.nntile_hip_set_stream_provider.argtypes = [_vp]
         L.nntile_hip_set_stream_provider.restype = None
         L.nntile_hip_sdpa_version.restype = ctypes.c_char_p
@@ -391,6 +394,21 @@ def sdpa_fwd_decode(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group,
     nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _check(fn(_stream(stream), ctypes.byref(a), _ptr(workspace), nbytes),
            "sdpa_fwd_decode")
+
+
+DECODE_STATIC_SCRATCH_BYTES = 16 << 20
+
+
+def sdpa_fwd_decode_static(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0=0,
+                           k_pos0=0, causal_offset=0, flags=0, stream=None):
+    """sdpa_fwd_decode with the split partials in the library's own device
+    array (at most DECODE_STATIC_SCRATCH_BYTES): no workspace, no allocation."""
+    _dev(K, Q, mask, lse, V, A)
+    a = _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0,
+                   k_pos0, causal_offset, flags)
+    code = {"bf16": 0, "fp16": 1}.get(dtype_name(Q), -1)
+    _check(lib().nntile_hip_sdpa_fwd_decode_static(_stream(stream), code, ctypes.byref(a)),
+           "sdpa_fwd_decode_static")
 
 
 def kv_cache_append(k_new, v_new, k_cache, v_cache, filled, stream=None):

@@ -1,0 +1,82 @@
+"""The decode entry point that allocates nothing
+(nntile_hip_sdpa_fwd_decode_static: split partials in a device array the
+library owns) against nntile_hip_sdpa_fwd_decode_* with a caller's workspace,
+through the C ABI: same kernels, so the results must agree bit for bit, on two
+calls in a row, the second on a smaller input (the array keeps the first
+call's partials), and against the checker within the tolerance.  A shape
+whose partials exceed the array is refused before anything is enqueued."""
+import pytest
+import torch
+
+from nntile_amd import hip_sdpa, synth
+from . import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle(oracle, f32, mask, n_batch, group):
+    qf, kf, vf = f32
+    return oracle.sdpa_vanilla(kf, qf, vf, mask, n_batch=n_batch, kv_repeat=group)
+
+
+def _both(oracle, dtype, q_seq, k_seq, n_batch, group, n_kv, head, seed, overwrite):
+    print("case", dtype, q_seq, k_seq, n_batch, group, n_kv, head, seed, overwrite, flush=True)
+    batch = n_batch * group * n_kv
+    (Q, K, V), f32 = H.make_qkv(seed, batch, q_seq, k_seq, head, dtype, kv_batch=n_batch * n_kv)
+    offset = k_seq - q_seq
+    want, want_lse = _oracle(oracle, f32, synth.causal_mask(q_seq, k_seq, offset), n_batch, group)
+    Kd, Qd, Vd = K.cuda(), Q.cuda(), V.cuda()
+    need = hip_sdpa.decode_workspace_bytes(Kd, Qd, n_batch, group)
+    assert 0 < need <= hip_sdpa.DECODE_STATIC_SCRATCH_BYTES
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    flags = hip_sdpa.OVERWRITE if overwrite else 0
+    lse0, A0 = H.fresh_outputs(batch, q_seq, head, dtype)
+    lse1, A1 = H.fresh_outputs(batch, q_seq, head, dtype)
+    hip_sdpa.sdpa_fwd_decode(Kd, Qd, None, lse0, Vd, A0, hip_sdpa.MASK_CAUSAL, n_batch, group, ws,
+                             causal_offset=offset, flags=flags)
+    hip_sdpa.sdpa_fwd_decode_static(Kd, Qd, None, lse1, Vd, A1, hip_sdpa.MASK_CAUSAL, n_batch,
+                                    group, causal_offset=offset, flags=flags)
+    torch.cuda.synchronize()
+    assert torch.equal(lse0, lse1)
+    assert torch.equal(A0.view(torch.int16), A1.view(torch.int16))
+    assert H.rel_fro(H.to_np(A1), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse1), want_lse) < H.TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+def test_static_scratch_decode_twice_second_smaller(oracle, dtype):
+    # several key splits per unit (partials go through the array), then a
+    # smaller input whose partials cover only the start of what the first left
+    _both(oracle, dtype, 16, 2048, 2, 4, 2, 128, 51, False)
+    _both(oracle, dtype, 5, 700, 1, 4, 2, 128, 52, True)
+    # and the larger one again: nothing of the small call's leftovers shows
+    _both(oracle, dtype, 16, 2048, 2, 4, 2, 128, 53, True)
+
+
+def test_static_scratch_decode_head64_and_merge(oracle):
+    _both(oracle, "bf16", 16, 1000, 1, 4, 1, 64, 54, False)
+    _both(oracle, "bf16", 1, 300, 3, 4, 2, 64, 55, False)
+
+
+def test_static_scratch_refuses_what_does_not_fit():
+    # 64 rows x 4096 units x 1 split of bf16 partials alone are 64 MiB
+    n_batch, group, n_kv, head, q_seq, k_seq = 1024, 4, 4, 128, 16, 8192
+    batch = n_batch * group * n_kv
+    a = hip_sdpa.TileArgs()
+    a.q_seq, a.k_seq, a.head, a.batch = q_seq, k_seq, head, batch
+    a.n_batch, a.kv_group, a.mask_mode = n_batch, group, hip_sdpa.MASK_CAUSAL
+    import ctypes
+    need = int(hip_sdpa.lib().nntile_hip_sdpa_fwd_decode_workspace_bytes(ctypes.byref(a)))
+    if need <= hip_sdpa.DECODE_STATIC_SCRATCH_BYTES:
+        pytest.skip("this shape's partials fit the array")
+    # the pointers are never touched: the size check comes first
+    dummy = torch.zeros(16, dtype=torch.bfloat16, device="cuda")
+    a.K = a.Q = a.V = a.A = dummy.data_ptr()
+    a.lse = dummy.data_ptr()
+    code = hip_sdpa.lib().nntile_hip_sdpa_fwd_decode_static(
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), 0, ctypes.byref(a))
+    assert code == hip_sdpa.EWORKSPACE
+    # an unknown dtype code is an argument error
+    code = hip_sdpa.lib().nntile_hip_sdpa_fwd_decode_static(
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), 7, ctypes.byref(a))
+    assert code == hip_sdpa.EINVAL
