@@ -181,6 +181,42 @@ def bench_prefill(cfg, steps, warmup, per_task=False, classified=False, streams=
             "kernel_tflops": cfg.flops() / (kdev * 1e-3) / 1e12}
 
 
+def bench_reference_api(cfg, steps, warmup):
+    """cfg as an unchanged caller runs it: tensors tiled as the config says,
+    a materialised additive causal mask [k_seq, q_seq], and per pass what
+    Sdpa._forward_flash does (layer/sdpa.py:533-557) - logsumexp filled with
+    -inf, then tensor::flash_sdpa_fwd_cudnn_async(K, Q, mask, logsumexp, V, A)
+    with the reference's six arguments - through the C++ host mirror.  Timed
+    with HIP events on the mirror's stream.  Twice: the default overload
+    (mask tiles classified on first sight, classes kept with the mask), and
+    the reference's submission literally (one task per tile pair)."""
+    import numpy as np
+    from nntile_amd import host_mirror as hm, synth
+    assert cfg.dtype == "bf16" and cfg.kv_group == 1
+    s5 = [cfg.head, cfg.q_seq, cfg.n_batch, 1, cfg.n_head_kv]
+    b5 = [cfg.head, cfg.seq_tile, cfg.n_batch, 1, cfg.n_head_kv]
+    n = int(np.prod(s5))
+    T = {}
+    for i, name in enumerate(("Q", "K", "V")):
+        bits = synth.round_bf16(synth.randn(cfg.seed, i, n))[0]
+        T[name] = hm.Tensor("bf16", s5, b5).from_array(bits.reshape(s5, order="F"))
+    A = hm.Tensor("bf16", s5, b5).from_array(np.zeros(s5, np.uint16))
+    lse = hm.Tensor("fp32", s5[1:], b5[1:]).from_array(np.full(s5[1:], -np.inf, np.float32))
+    vis = synth.causal_mask(cfg.q_seq, cfg.k_seq)                # [q, k]
+    add = synth.round_bf16(np.where(vis, 0.0, -np.inf).astype(np.float32).T)[0]   # [k, q]
+    M = hm.Tensor("bf16", [cfg.k_seq, cfg.q_seq], [cfg.seq_tile, cfg.seq_tile]).from_array(
+        np.asfortranarray(add))
+    out = {}
+    for key, op in (("default_overload", hm.OP_TENSOR), ("every_pair", hm.OP_PAIRS)):
+        h0, m0 = hm.mask_cache_stats()
+        ms, launches = hm.time_flash_sdpa_fwd(op, T["K"], T["Q"], M, lse, T["V"], A, steps, warmup)
+        h1, m1 = hm.mask_cache_stats()
+        out[key] = {"ms_per_step": round(ms, 4), "launches_per_step": launches,
+                    "tflops": round(cfg.flops() / (ms * 1e-3) / 1e12, 2),
+                    "mask_classifications": m1 - m0, "mask_cache_hits": h1 - h0}
+    return out
+
+
 def bench_decode(cfg, steps, warmup):
     import torch
     from nntile_amd import hip_sdpa as h
@@ -473,6 +509,9 @@ def main():
         return
     if only == "decode":
         bench_decode(cfg4, args.steps, args.warmup)
+        return
+    if only == "reference_api":
+        print(json.dumps(bench_reference_api(cfg3, args.steps, args.warmup)))
         return
     if only == "copy":
         # calibration leg for the HBM traffic counters: a plain device copy

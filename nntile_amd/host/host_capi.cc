@@ -2,6 +2,7 @@
 // are created from shapes and Fortran-ordered host arrays, the operations are
 // the mirror's tile::/tensor:: functions, exceptions come back as messages.
 #include <cstring>
+#include <functional>
 #include <string>
 
 #include "nntile_host.hh"
@@ -47,7 +48,7 @@ void run_op(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *mask, AnyTensor *lse,
 {
     switch(op)
     {
-        case 0:     // tensor-level, per-tile tasks, blocking
+        case 0:     // tensor-level, the reference's signature, blocking
             tensor::flash_sdpa_fwd_cudnn<T>(get<T>(K), get<T>(Q), get<T>(mask),
                     get<fp32_t>(lse), get<T>(V), get<T>(A));
             break;
@@ -61,8 +62,33 @@ void run_op(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *mask, AnyTensor *lse,
                     offset, get<fp32_t>(lse), get<T>(V), get<T>(A), overwrite != 0);
             starpu::task_wait_for_all();
             break;
+        case 3:     // tensor-level, the reference's submission literally: every pair, blocking
+            tensor::flash_sdpa_fwd_cudnn_pairs_async<T>(get<T>(K), get<T>(Q), get<T>(mask),
+                    get<fp32_t>(lse), get<T>(V), get<T>(A));
+            starpu::task_wait_for_all();
+            break;
         default:
             throw std::runtime_error("unknown operation");
+    }
+}
+
+template<typename T>
+void run_async(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *mask, AnyTensor *lse,
+        AnyTensor *V, AnyTensor *A)
+{
+    if(op == 0)
+    {
+        tensor::flash_sdpa_fwd_cudnn_async<T>(get<T>(K), get<T>(Q), get<T>(mask),
+                get<fp32_t>(lse), get<T>(V), get<T>(A));
+    }
+    else if(op == 3)
+    {
+        tensor::flash_sdpa_fwd_cudnn_pairs_async<T>(get<T>(K), get<T>(Q), get<T>(mask),
+                get<fp32_t>(lse), get<T>(V), get<T>(A));
+    }
+    else
+    {
+        throw std::runtime_error("unknown operation");
     }
 }
 
@@ -90,10 +116,16 @@ int64_t run_bwd(int op, AnyTensor *K, AnyTensor *Q, AnyTensor *V, AnyTensor *A,
             starpu::task_wait_for_all();
             return n;
         }
-        case 0:     // tensor-level, per-tile tasks, blocking
+        case 0:     // tensor-level, the reference's signature, blocking
             tensor::flash_sdpa_bwd_cudnn<T>(get<T>(K), get<T>(Q), get<T>(V),
                     get<T>(A), get<T>(dA), get<T>(mask), get<fp32_t>(lse),
                     get<T>(dK), get<T>(dQ), get<T>(dV));
+            break;
+        case 4:     // tensor-level, the reference's submission literally: every pair
+            tensor::flash_sdpa_bwd_cudnn_pairs_async<T>(get<T>(K), get<T>(Q), get<T>(V),
+                    get<T>(A), get<T>(dA), get<T>(mask), get<fp32_t>(lse),
+                    get<T>(dK), get<T>(dQ), get<T>(dV));
+            starpu::task_wait_for_all();
             break;
         case 1:     // tile-level on single-tile tensors, blocking
             tile::flash_sdpa_bwd_cudnn<T>(get<T>(K).get_tile(0), get<T>(Q).get_tile(0),
@@ -171,7 +203,8 @@ int64_t nntile_host_tensor_ntiles(void *t_)
 }
 
 // op: 0 tensor::flash_sdpa_fwd_cudnn, 1 tile::flash_sdpa_fwd_cudnn (single-tile
-// tensors), 2 tensor::flash_sdpa_fwd_hip_async + wait (mask may be null)
+// tensors), 2 tensor::flash_sdpa_fwd_hip_async + wait (mask may be null),
+// 3 tensor::flash_sdpa_fwd_cudnn_pairs_async + wait
 int nntile_host_flash_sdpa_fwd(int op, int dtype, void *K, void *Q, void *mask,
         void *lse, void *V, void *A, int mask_mode, int64_t offset, int overwrite,
         char *err, int errlen)
@@ -290,7 +323,9 @@ int nntile_host_check_shapes(int level, const int64_t *desc, char *err, int errl
 // op: 0 tensor::flash_sdpa_bwd_cudnn, 1 tile::flash_sdpa_bwd_cudnn (single-tile
 // tensors), 2 tensor::flash_sdpa_bwd_hip_async + wait (mask may be null), 3
 // tensor::flash_sdpa_mask_classes + the overload that takes the classes + wait
-// (ops 2 and 3: *submitted = tile pairs launched); dtype bf16 or fp16, as the reference's pack
+// (ops 2 and 3: *submitted = tile pairs launched), 4
+// tensor::flash_sdpa_bwd_cudnn_pairs_async + wait; dtype bf16 or fp16, as the
+// reference's pack
 int nntile_host_flash_sdpa_bwd(int op, int dtype, void *K, void *Q, void *V,
         void *A, void *dA, void *mask, void *lse, void *dK, void *dQ, void *dV,
         int mask_mode, int64_t offset, int64_t *submitted, char *err, int errlen)
@@ -379,6 +414,81 @@ const char *nntile_host_codelet_name(int dtype)
     if(dtype == DT_BF16) return starpu::flash_sdpa_fwd_cudnn<bf16_t>().name.c_str();
     if(dtype == DT_FP16) return starpu::flash_sdpa_fwd_cudnn<fp16_t>().name.c_str();
     return starpu::flash_sdpa_fwd_cudnn<fp32_t>().name.c_str();
+}
+
+// Counters of the mask-class cache behind the reference-signature tensor
+// operations, a reset of the cache, and a "some writer got this tensor" mark
+// on every tile of a tensor.
+void nntile_host_mask_cache_stats(uint64_t *hits, uint64_t *misses)
+{
+    const auto st = tensor::flash_sdpa_mask_cache_stats();
+    *hits = st.hits;
+    *misses = st.misses;
+}
+
+void nntile_host_mask_cache_clear(void)
+{
+    tensor::flash_sdpa_mask_cache_clear();
+}
+
+void nntile_host_tensor_mark_written(void *t_)
+{
+    auto *t = static_cast<AnyTensor *>(t_);
+    const int64_t n = nntile_host_tensor_ntiles(t_);
+    for(int64_t i = 0; i < n; ++i)
+    {
+        if(t->dtype == DT_BF16) t->bf16->get_tile(i).mark_written();
+        else if(t->dtype == DT_FP16) t->fp16->get_tile(i).mark_written();
+        else t->fp32->get_tile(i).mark_written();
+    }
+}
+
+// Times `steps` passes (after `warmup` untimed ones) of what a layer does per
+// forward through the reference's interface (Sdpa._forward_flash,
+// wrappers/python/nntile/layer/sdpa.py:533-557): logsumexp filled with -inf,
+// then tensor::flash_sdpa_fwd_cudnn_async (op 0) or
+// tensor::flash_sdpa_fwd_cudnn_pairs_async (op 3), with HIP events on the
+// mirror's stream.  *ms = milliseconds per pass, *launches = attention
+// launches per pass (tile tasks + direct launches).
+int nntile_host_time_flash_sdpa_fwd(int op, int dtype, void *K, void *Q, void *mask,
+        void *lse, void *V, void *A, int steps, int warmup, double *ms, int64_t *launches,
+        char *err, int errlen)
+{
+    try
+    {
+        auto k = static_cast<AnyTensor *>(K), q = static_cast<AnyTensor *>(Q),
+             m = static_cast<AnyTensor *>(mask), l = static_cast<AnyTensor *>(lse),
+             v = static_cast<AnyTensor *>(V), a = static_cast<AnyTensor *>(A);
+        const int64_t before = nntile_host_tasks_submitted(dtype)
+            + starpu::direct_launches();
+        double total = 0.0;
+        auto pass = [&]()
+        {
+            tensor::fill_async(-__builtin_huge_valf(), get<fp32_t>(l));
+            if(dtype == DT_BF16) run_async<bf16_t>(op, k, q, m, l, v, a);
+            else if(dtype == DT_FP16) run_async<fp16_t>(op, k, q, m, l, v, a);
+            else run_async<fp32_t>(op, k, q, m, l, v, a);
+        };
+        for(int i = 0; i < warmup; ++i)
+        {
+            pass();
+        }
+        starpu::task_wait_for_all();
+        const int64_t mid = nntile_host_tasks_submitted(dtype) + starpu::direct_launches();
+        total = starpu::time_on_stream_ms([&]()
+        {
+            for(int i = 0; i < steps; ++i)
+            {
+                pass();
+            }
+        });
+        const int64_t after = nntile_host_tasks_submitted(dtype) + starpu::direct_launches();
+        (void)before;
+        *ms = total / (steps > 0 ? steps : 1);
+        *launches = steps > 0 ? (after - mid) / steps : 0;
+        return 0;
+    }
+    catch(const std::exception &e) { return fail(err, errlen, e); }
 }
 
 } // extern "C"

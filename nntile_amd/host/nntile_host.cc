@@ -125,16 +125,61 @@ void task_wait_for_all()
             "hipStreamSynchronize");
 }
 
+static std::uint64_t next_stamp()
+{
+    static std::atomic<std::uint64_t> counter{0};
+    return ++counter;
+}
+
+static std::atomic<std::int64_t> direct_launch_counter{0};
+
+std::int64_t direct_launches()
+{
+    return direct_launch_counter.load();
+}
+
+void count_direct_launch()
+{
+    ++direct_launch_counter;
+}
+
+double time_on_stream_ms(const std::function<void()> &enqueue)
+{
+    hipStream_t stream = static_cast<hipStream_t>(get_local_stream());
+    hipEvent_t e0, e1;
+    hip_check(hipEventCreate(&e0), "hipEventCreate");
+    hip_check(hipEventCreate(&e1), "hipEventCreate");
+    hip_check(hipEventRecord(e0, stream), "hipEventRecord");
+    enqueue();
+    hip_check(hipEventRecord(e1, stream), "hipEventRecord");
+    hip_check(hipEventSynchronize(e1), "hipEventSynchronize");
+    float ms = 0.0f;
+    hip_check(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return ms;
+}
+
 Handle::Handle(std::size_t size): nbytes(size)
 {
     void *ptr = nullptr;
     hip_check(hipMalloc(&ptr, size > 0 ? size : 1), "hipMalloc");
     mem = std::shared_ptr<void>(ptr, [](void *p) { (void)hipFree(p); });
+    stamp = std::make_shared<std::atomic<std::uint64_t>>(next_stamp());
+}
+
+void Handle::mark_written() const
+{
+    if(stamp)
+    {
+        stamp->store(next_stamp());
+    }
 }
 
 void Handle::from_host(const void *src) const
 {
     task_wait_for_all();
+    mark_written();
     hip_check(hipMemcpy(mem.get(), src, nbytes, hipMemcpyHostToDevice), "hipMemcpy");
 }
 
@@ -228,6 +273,8 @@ void FlashSdpaFwdCudnn<std::tuple<T>>::submit(Index seq, Index head, Index batch
         buffers[i] = &ifs[i];
     }
     (void)get_local_stream();       // makes sure the provider is registered
+    logsumexp.mark_written();       // the RW buffers
+    A.mark_written();
     // "Task execution": the body only enqueues on the stream; the stream's
     // order is the order of submission.
     hip(buffers, args);
@@ -309,6 +356,9 @@ void FlashSdpaBwdCudnn<std::tuple<T>>::submit(Index seq, Index head, Index batch
         buffers[i] = &ifs[i];
     }
     (void)get_local_stream();
+    dK.mark_written();              // the RW buffers
+    dQ.mark_written();
+    dV.mark_written();
     hip(buffers, args);
     std::free(args);
     ++submitted;
@@ -643,6 +693,23 @@ static void require(bool ok, const char *message)
     }
 }
 
+void fill_async(float val, const Tensor<fp32_t> &dst)
+{
+    std::uint32_t bits;
+    std::memcpy(&bits, &val, sizeof(bits));
+    for(Index i = 0; i < dst.grid.nelems; ++i)
+    {
+        const auto &tile = dst.get_tile(i);
+        tile.mark_written();
+        if(hipMemsetD32Async(reinterpret_cast<hipDeviceptr_t>(tile.get_ptr()),
+                    static_cast<int>(bits), static_cast<std::size_t>(tile.nelems),
+                    static_cast<hipStream_t>(starpu::get_local_stream())) != hipSuccess)
+        {
+            throw std::runtime_error("Error in fill_async");
+        }
+    }
+}
+
 void flash_sdpa_fwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
         const TensorTraits &mask, const TensorTraits &logsumexp,
         const TensorTraits &V, const TensorTraits &A)
@@ -696,7 +763,7 @@ void flash_sdpa_fwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
 }
 
 template<typename T>
-void flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+void flash_sdpa_fwd_cudnn_pairs_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &V, const Tensor<T> &A)
 {
@@ -737,6 +804,43 @@ void flash_sdpa_fwd_cudnn(const Tensor<T> &K, const Tensor<T> &Q,
 {
     flash_sdpa_fwd_cudnn_async<T>(K, Q, mask, logsumexp, V, A);
     starpu::task_wait_for_all();
+}
+
+// ---- what is known about a mask, kept with its handles ----------------------
+// A layer builds its mask once and passes the same tensor to every call
+// (wrappers/python/nntile/model/gpt2_attention.py:72-87), so the classes of
+// its tiles are worth one blocking pass on first sight.  An entry is valid as
+// long as every tile of the mask is the allocation it was and has not been
+// given to a writer since (Handle::write_stamp); the key is the first tile's
+// address.
+namespace
+{
+
+struct MaskCacheEntry
+{
+    std::vector<std::pair<const void *, std::uint64_t>> tiles;  // (address, stamp)
+    Index causal_offset;
+    std::vector<Index> shape, basetile;
+    std::vector<int> classes;
+};
+
+std::mutex mask_cache_mutex;
+std::vector<MaskCacheEntry> mask_cache;         // few masks per process: linear search
+std::uint64_t mask_cache_hits = 0, mask_cache_misses = 0;
+constexpr std::size_t kMaskCacheEntries = 64;
+
+} // namespace
+
+MaskCacheStats flash_sdpa_mask_cache_stats()
+{
+    std::lock_guard<std::mutex> guard(mask_cache_mutex);
+    return MaskCacheStats{mask_cache_hits, mask_cache_misses};
+}
+
+void flash_sdpa_mask_cache_clear()
+{
+    std::lock_guard<std::mutex> guard(mask_cache_mutex);
+    mask_cache.clear();
 }
 
 template<typename T> struct GridCall;
@@ -803,6 +907,12 @@ void flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
                     a.lse[t] = static_cast<float *>(
                             logsumexp.get_tile({t, g2, g3, g4}).get_ptr());
                 }
+                for(Index t = 0; t < n_q; ++t)
+                {
+                    A.get_tile({0, t, g2, g3, g4}).mark_written();
+                    logsumexp.get_tile({t, g2, g3, g4}).mark_written();
+                }
+                starpu::count_direct_launch();
                 const int rc = GridCall<T>::run(starpu::get_local_stream(), &a);
                 if(rc != NNTILE_HIP_OK)
                 {
@@ -865,6 +975,61 @@ std::vector<int> flash_sdpa_mask_classes(const Tensor<T> &mask, Index causal_off
         classes[i] = cls;
     }
     word.unregister_submit();
+    return classes;
+}
+
+template<typename T>
+std::vector<int> flash_sdpa_cached_mask_classes(const Tensor<T> &mask, Index causal_offset)
+{
+    require(mask.ndim == 2, "mask must be 2-dimensional");
+    std::vector<std::pair<const void *, std::uint64_t>> ident(mask.grid.nelems);
+    for(Index i = 0; i < mask.grid.nelems; ++i)
+    {
+        const auto &tile = mask.get_tile(i);
+        ident[i] = {tile.get_ptr(), tile.write_stamp()};
+    }
+    {
+        std::lock_guard<std::mutex> guard(mask_cache_mutex);
+        for(std::size_t e = 0; e < mask_cache.size(); )
+        {
+            auto &entry = mask_cache[e];
+            if(entry.tiles.empty() || ident.empty() || entry.tiles[0].first != ident[0].first)
+            {
+                ++e;
+                continue;
+            }
+            if(entry.tiles == ident && entry.causal_offset == causal_offset
+                    && entry.shape == mask.shape && entry.basetile == mask.basetile_shape)
+            {
+                ++mask_cache_hits;
+                return entry.classes;
+            }
+            if(entry.tiles[0].second != ident[0].second)
+            {
+                // the memory at this address was written or reallocated
+                mask_cache.erase(mask_cache.begin() + static_cast<std::ptrdiff_t>(e));
+                continue;
+            }
+            ++e;
+        }
+        ++mask_cache_misses;
+    }
+    // (outside the lock: this blocks on the device)
+    MaskCacheEntry fresh;
+    fresh.classes = flash_sdpa_mask_classes<T>(mask, causal_offset);
+    fresh.tiles = std::move(ident);
+    fresh.causal_offset = causal_offset;
+    fresh.shape = mask.shape;
+    fresh.basetile = mask.basetile_shape;
+    std::vector<int> classes = fresh.classes;
+    {
+        std::lock_guard<std::mutex> guard(mask_cache_mutex);
+        if(mask_cache.size() >= kMaskCacheEntries)
+        {
+            mask_cache.erase(mask_cache.begin());
+        }
+        mask_cache.push_back(std::move(fresh));
+    }
     return classes;
 }
 
@@ -961,6 +1126,9 @@ Index flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
             a.V = V_tile.get_ptr();
             a.lse = static_cast<float *>(lse_tile.get_ptr());
             a.A = A_tile.get_ptr();
+            lse_tile.mark_written();
+            A_tile.mark_written();
+            starpu::count_direct_launch();
             const int rc = TileCall<T>::run(starpu::get_local_stream(), &a);
             if(rc != NNTILE_HIP_OK)
             {
@@ -970,6 +1138,19 @@ Index flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
         }
     }
     return submitted;
+}
+
+template<typename T>
+void flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &V, const Tensor<T> &A)
+{
+    flash_sdpa_fwd_cudnn_check(K, Q, mask, logsumexp, V, A);
+    // The reference's signature carries no offset: its masks are square
+    // (K.shape[1] == Q.shape[1] is one of its checks), the rule to look for is
+    // key <= query.
+    const std::vector<int> classes = flash_sdpa_cached_mask_classes<T>(mask, 0);
+    (void)flash_sdpa_fwd_cudnn_async<T>(K, Q, mask, classes, 0, logsumexp, V, A);
 }
 
 // ---- backward: src/tensor/flash_sdpa_bwd_cudnn.cc:22-261 -------------------
@@ -1005,7 +1186,7 @@ void flash_sdpa_bwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
 }
 
 template<typename T>
-void flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+void flash_sdpa_bwd_cudnn_pairs_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
         const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV)
@@ -1153,6 +1334,10 @@ static Index bwd_pairs(const Tensor<T> &K, const Tensor<T> &Q,
             a.dV = dV.get_tile(kv_index).get_ptr();
             a.workspace = workspace.get_ptr();
             a.workspace_bytes = ws_bytes;
+            dK.get_tile(kv_index).mark_written();
+            dQ.get_tile(dq_linear).mark_written();
+            dV.get_tile(kv_index).mark_written();
+            starpu::count_direct_launch();
             const int rc = BwdTileCall<T>::run(starpu::get_local_stream(), &a);
             if(rc != NNTILE_HIP_OK)
             {
@@ -1197,6 +1382,18 @@ Index flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
             causal_offset, logsumexp, dK, dQ, dV);
 }
 
+template<typename T>
+void flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV)
+{
+    flash_sdpa_bwd_cudnn_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
+    const std::vector<int> classes = flash_sdpa_cached_mask_classes<T>(mask, 0);
+    (void)flash_sdpa_bwd_cudnn_async<T>(K, Q, V, A, dA, mask, classes, 0, logsumexp,
+            dK, dQ, dV);
+}
+
 #define NNTILE_HOST_INSTANTIATE_TENSOR_BWD(T) \
     template Index flash_sdpa_bwd_cudnn_async<T>(const Tensor<T> &, const Tensor<T> &, \
             const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, \
@@ -1209,6 +1406,9 @@ Index flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
             const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, \
             const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &); \
     template void flash_sdpa_bwd_cudnn<T>(const Tensor<T> &, const Tensor<T> &, \
+            const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, \
+            const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &); \
+    template void flash_sdpa_bwd_cudnn_pairs_async<T>(const Tensor<T> &, const Tensor<T> &, \
             const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &, \
             const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, const Tensor<T> &);
 NNTILE_HOST_INSTANTIATE_TENSOR_BWD(bf16_t)
@@ -1223,6 +1423,9 @@ NNTILE_HOST_INSTANTIATE_TENSOR_BWD(fp16_t)
     template void flash_sdpa_fwd_hip_async<T>(const Tensor<T> &, const Tensor<T> &, int, \
             Index, const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, bool); \
     template std::vector<int> flash_sdpa_mask_classes<T>(const Tensor<T> &, Index); \
+    template std::vector<int> flash_sdpa_cached_mask_classes<T>(const Tensor<T> &, Index); \
+    template void flash_sdpa_fwd_cudnn_pairs_async<T>(const Tensor<T> &, const Tensor<T> &, \
+            const Tensor<T> &, const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &); \
     template Index flash_sdpa_fwd_cudnn_async<T>(const Tensor<T> &, const Tensor<T> &, \
             const Tensor<T> &, const std::vector<int> &, Index, const Tensor<fp32_t> &, \
             const Tensor<T> &, const Tensor<T> &);

@@ -23,8 +23,10 @@
 #pragma once
 
 #include <array>
+#include <atomic>
 #include <cstdint>
 #include <cstdlib>
+#include <functional>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -72,6 +74,11 @@ class Handle
 {
     std::shared_ptr<void> mem;
     std::size_t nbytes = 0;
+    //! Shared by all copies of the handle: a process-wide unique number taken
+    //! when the memory is allocated and again at every write access.  Two
+    //! equal stamps of one address mean "same allocation, not written in
+    //! between" - what a cache of facts about the contents is keyed on.
+    std::shared_ptr<std::atomic<std::uint64_t>> stamp;
 public:
     Handle() = default;
     explicit Handle(std::size_t size);      // allocates device memory
@@ -80,6 +87,10 @@ public:
     //! Blocking copies (the analogue of acquire/release on the host)
     void from_host(const void *src) const;
     void to_host(void *dst) const;
+    //! To be called by whoever gives a writer access to the memory (under
+    //! StarPU: every acquire or task access in a W or RW mode)
+    void mark_written() const;
+    std::uint64_t write_stamp() const { return stamp ? stamp->load() : 0; }
     //! The reference's scratch handles are unregistered right after the
     //! submission (src/tile/flash_sdpa_fwd_cudnn.cc:194-195)
     void unregister_submit() { mem.reset(); nbytes = 0; }
@@ -90,6 +101,13 @@ using VariableHandle = Handle;
 //! Stream every codelet body of this process enqueues on
 void *get_local_stream();
 void task_wait_for_all();
+//! Launches that tensor-level functions made through the C ABI directly
+//! (not as codelet tasks) since the start of the process
+std::int64_t direct_launches();
+void count_direct_launch();
+//! Milliseconds the stream needs for what `enqueue` puts on it (HIP events
+//! around it; blocks until done)
+double time_on_stream_ms(const std::function<void()> &enqueue);
 
 //! Wrapper of the attention codelet for one value type
 template<typename T> class FlashSdpaFwdCudnn;
@@ -240,16 +258,50 @@ public:
     void to_array(typename T::storage_t *dst) const;
 };
 
+//! Every element of every tile set to val (fill_async of the reference,
+//! src/tensor/fill.cc; what the layer does to logsumexp before the forward)
+void fill_async(float val, const Tensor<fp32_t> &dst);
+
 //! Shape and tiling rules of the tensor-level operation; throws
 void flash_sdpa_fwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
         const TensorTraits &mask, const TensorTraits &logsumexp,
         const TensorTraits &V, const TensorTraits &A);
 
-//! One tile task per (output tile, key tile) pair, in the reference's order
+//! The reference's operation with the reference's arguments
+//! (src/tensor/flash_sdpa_fwd_cudnn.cc:210-279).  What it computes is the
+//! reference's result; how it is submitted depends on what the mask holds.
+//! The first call that sees a mask classifies its tiles (blocking, once:
+//! flash_sdpa_mask_classes against the rule key <= query) and keeps the
+//! classes keyed on the mask tiles' handles; later calls with the same,
+//! unwritten mask find them.  Then, as the overload that takes the classes
+//! does: a mask that is the causal rule or hides nothing - one launch per slab
+//! of the batch grid; otherwise per pair, hidden pairs not submitted, open and
+//! causal pairs without mask memory, the rest (a mask with bias values: every
+//! pair) exactly as flash_sdpa_fwd_cudnn_pairs_async.
 template<typename T>
 void flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &V, const Tensor<T> &A);
+
+//! One tile task per (output tile, key tile) pair with the pair's mask tile,
+//! in the reference's order, none skipped: the reference's submission
+//! literally (src/tensor/flash_sdpa_fwd_cudnn.cc:221-274)
+template<typename T>
+void flash_sdpa_fwd_cudnn_pairs_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &V, const Tensor<T> &A);
+
+//! The classes of flash_sdpa_mask_classes(mask, causal_offset), computed on
+//! first sight of the mask and kept until one of its tiles is written or
+//! freed (Handle::write_stamp).  Blocking on a miss.
+template<typename T>
+std::vector<int> flash_sdpa_cached_mask_classes(const Tensor<T> &mask, Index causal_offset);
+
+//! Counters of that cache since the start of the process, and a reset of the
+//! cache (not of the counters)
+struct MaskCacheStats { std::uint64_t hits, misses; };
+MaskCacheStats flash_sdpa_mask_cache_stats();
+void flash_sdpa_mask_cache_clear();
 
 template<typename T>
 void flash_sdpa_fwd_cudnn(const Tensor<T> &K, const Tensor<T> &Q,
@@ -296,9 +348,20 @@ void flash_sdpa_bwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
         const TensorTraits &mask, const TensorTraits &logsumexp,
         const TensorTraits &dK, const TensorTraits &dQ, const TensorTraits &dV);
 
-//! One tile task per (dQ tile, key tile) pair, in the reference's order
+//! The reference's operation with the reference's arguments
+//! (src/tensor/flash_sdpa_bwd_cudnn.cc:172-247); submitted through the cached
+//! classes of the mask's tiles like the forward (hidden pairs not submitted,
+//! open and causal pairs without mask memory, the rest as the reference does)
 template<typename T>
 void flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV);
+
+//! One tile task per (dQ tile, key tile) pair, in the reference's order, none
+//! skipped: the reference's submission literally
+template<typename T>
+void flash_sdpa_bwd_cudnn_pairs_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
         const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV);

@@ -10,6 +10,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "host", "libnntile_host.so")
 DTYPES = {"bf16": 0, "fp16": 1, "fp32": 2}
 OP_TENSOR, OP_TILE, OP_HIP, OP_CLASSIFIED = 0, 1, 2, 3
+# the reference's submission literally, one task per tile pair (forward / backward op codes)
+OP_PAIRS, OP_PAIRS_BWD = 3, 4
 _lib = None
 
 
@@ -59,6 +61,15 @@ def lib():
         L.nntile_host_tasks_submitted.restype = i64
         L.nntile_host_codelet_name.argtypes = [ctypes.c_int]
         L.nntile_host_codelet_name.restype = ctypes.c_char_p
+        L.nntile_host_mask_cache_stats.argtypes = [ctypes.POINTER(ctypes.c_uint64)] * 2
+        L.nntile_host_mask_cache_stats.restype = None
+        L.nntile_host_mask_cache_clear.argtypes = []
+        L.nntile_host_mask_cache_clear.restype = None
+        L.nntile_host_tensor_mark_written.argtypes = [vp]
+        L.nntile_host_tensor_mark_written.restype = None
+        L.nntile_host_time_flash_sdpa_fwd.argtypes = [
+            ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp, ctypes.c_int, ctypes.c_int,
+            ctypes.POINTER(ctypes.c_double), ctypes.POINTER(i64), ctypes.c_char_p, ctypes.c_int]
         _lib = L
     return _lib
 
@@ -107,10 +118,38 @@ class Tensor:
         _call(lib().nntile_host_tensor_to_array, self.h, out.ctypes.data_as(ctypes.c_void_p))
         return out
 
+    def mark_written(self):
+        """What the runtime does when it hands the tiles to a writer: facts
+        cached about their contents (the classes of a mask) are dropped."""
+        lib().nntile_host_tensor_mark_written(self.h)
+
 
 def flash_sdpa_fwd(op, K, Q, mask, lse, V, A, mask_mode=0, offset=0, overwrite=False):
     _call(lib().nntile_host_flash_sdpa_fwd, op, DTYPES[Q.dtype], K.h, Q.h,
           None if mask is None else mask.h, lse.h, V.h, A.h, mask_mode, offset, int(overwrite))
+
+
+def mask_cache_stats():
+    """(hits, misses) of the mask-class cache behind the reference-signature
+    tensor operations (OP_TENSOR), since the start of the process."""
+    hits, misses = ctypes.c_uint64(0), ctypes.c_uint64(0)
+    lib().nntile_host_mask_cache_stats(ctypes.byref(hits), ctypes.byref(misses))
+    return hits.value, misses.value
+
+
+def mask_cache_clear():
+    lib().nntile_host_mask_cache_clear()
+
+
+def time_flash_sdpa_fwd(op, K, Q, mask, lse, V, A, steps, warmup):
+    """Milliseconds per pass and attention launches per pass of: logsumexp
+    filled with -inf, then tensor::flash_sdpa_fwd_cudnn_async (OP_TENSOR) or
+    tensor::flash_sdpa_fwd_cudnn_pairs_async (OP_PAIRS); HIP events on the
+    mirror's stream."""
+    ms, launches = ctypes.c_double(0.0), ctypes.c_int64(0)
+    _call(lib().nntile_host_time_flash_sdpa_fwd, op, DTYPES[Q.dtype], K.h, Q.h, mask.h, lse.h,
+          V.h, A.h, steps, warmup, ctypes.byref(ms), ctypes.byref(launches))
+    return ms.value, launches.value
 
 
 def mask_rule(k_seq, q_seq, k_tile, q_tile, classes, offset=0):

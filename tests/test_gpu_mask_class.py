@@ -95,7 +95,7 @@ def test_classified_submission_equals_the_reference_submission(oracle, dtype, ki
     # the reference's submission: every pair with its mask tile
     T, A0, lse0, M = _tensors(dtype, arrs, mask, head, seq, nb, grp, nkv, tile)
     before = hm.tasks_submitted(dtype)
-    hm.flash_sdpa_fwd(hm.OP_TENSOR, T["K"], T["Q"], M, lse0, T["V"], A0)
+    hm.flash_sdpa_fwd(hm.OP_PAIRS, T["K"], T["Q"], M, lse0, T["V"], A0)
     all_pairs = hm.tasks_submitted(dtype) - before
     ref_a, ref_lse = _read(dtype, A0, lse0, head, seq)
     # the classified submission
@@ -145,6 +145,6 @@ def test_a_bias_mask_is_submitted_as_the_reference_does(oracle):
             classes, submitted = hm.flash_sdpa_fwd_classified(T["K"], T["Q"], M, lse, T["V"], A)
             assert classes == [hip_sdpa.TILE_MIXED] * 4 and submitted == A.ntiles * 2
         else:
-            hm.flash_sdpa_fwd(hm.OP_TENSOR, T["K"], T["Q"], M, lse, T["V"], A)
+            hm.flash_sdpa_fwd(hm.OP_PAIRS, T["K"], T["Q"], M, lse, T["V"], A)
         outs.append((A.to_array().copy(), lse.to_array().copy()))
     assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])

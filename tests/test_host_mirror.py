@@ -105,7 +105,7 @@ def _run(dtype, arrs, mask_bool, head, seq, nb, grp, nkv, tile, op, **kw):
     A = hm.Tensor(dtype, s5, b5).from_array(np.zeros(s5, np.float32 if dtype == "fp32" else np.uint16))
     lse = hm.Tensor("fp32", s5[1:], b5[1:]).from_array(np.full(s5[1:], -np.inf, np.float32))
     mask = None
-    if op != hm.OP_HIP:
+    if op != hm.OP_HIP:     # (OP_TENSOR, OP_PAIRS: a materialised additive mask)
         add = np.where(mask_bool, 0.0, -np.inf).astype(np.float32).T       # [k_seq, q_seq] Fortran
         m_t, _ = H.rounded(add, dtype)
         m_np = m_t.numpy() if dtype == "fp32" else m_t.view(__import__("torch").int16).numpy().view(np.uint16)
@@ -129,9 +129,14 @@ def test_tensor_level_tiles_match_oracle(oracle, dtype, head, seq, nb, grp, nkv,
     mask = synth.causal_mask(seq, seq)
     want, want_lse = oracle.sdpa_vanilla(kf, qf, vf, mask, k_tile=tile)
     if seq % tile == 0:
-        got, got_lse, tasks, ntiles = _run(dtype, arrs, mask, head, seq, nb, grp, nkv, tile, hm.OP_TENSOR)
+        got, got_lse, tasks, ntiles = _run(dtype, arrs, mask, head, seq, nb, grp, nkv, tile, hm.OP_PAIRS)
         # one task per (output tile, key tile), none skipped (src/tensor/...:221-274)
         assert tasks == ntiles * (seq // tile)
+        assert H.rel_fro(got, want) < H.TOL[dtype] and H.rel_fro(got_lse, want_lse) < H.TOL[dtype]
+        # the reference's signature: the mask's tiles are classified on first
+        # sight, a causal mask then needs no tile tasks at all
+        got, got_lse, tasks, ntiles = _run(dtype, arrs, mask, head, seq, nb, grp, nkv, tile, hm.OP_TENSOR)
+        assert tasks == 0
         assert H.rel_fro(got, want) < H.TOL[dtype] and H.rel_fro(got_lse, want_lse) < H.TOL[dtype]
     # the single-launch path on the same tiling, ragged last tile included
     got, got_lse, tasks, _ = _run(dtype, arrs, mask, head, seq, nb, grp, nkv, tile, hm.OP_HIP,
@@ -161,3 +166,111 @@ def test_tile_level_entry_and_its_errors(oracle):
     bad = hm.Tensor("bf16", [head, seq // 2, nb, grp, nkv], [head, seq // 2, nb, grp, nkv])
     with pytest.raises(hm.HostError, match=r"K.shape\[1\] != Q.shape\[1\]"):
         hm.flash_sdpa_fwd(hm.OP_TILE, T["K"], bad, M, lse, T["V"], A)
+
+
+# ---- the reference's signature and what it learns about its mask ---------------
+
+def _mask_tensor(dtype, mask_bool, tile, values=None):
+    import torch
+    seq = mask_bool.shape[0]
+    add = np.where(mask_bool, 0.0, -np.inf).astype(np.float32) if values is None else values
+    m_t, _ = H.rounded(add.T, dtype)                        # [k_seq, q_seq]
+    m_np = m_t.numpy() if dtype == "fp32" else m_t.view(torch.int16).numpy().view(np.uint16)
+    return np.asfortranarray(m_np), hm.Tensor(dtype, [seq, seq], [tile, tile])
+
+
+def _outputs(dtype, s5, b5):
+    A = hm.Tensor(dtype, s5, b5).from_array(np.zeros(s5, np.float32 if dtype == "fp32" else np.uint16))
+    lse = hm.Tensor("fp32", s5[1:], b5[1:]).from_array(np.full(s5[1:], -np.inf, np.float32))
+    return A, lse
+
+
+def _read_out(dtype, A, lse, head, seq):
+    import torch
+    a = A.to_array()
+    if dtype != "fp32":
+        a = H.to_np(torch.from_numpy(a.view(np.int16).copy()).view(H.TORCH_DT[dtype]))
+    got = np.ascontiguousarray(a.transpose(4, 3, 2, 1, 0)).reshape(-1, seq, head)
+    got_lse = np.ascontiguousarray(lse.to_array().transpose(3, 2, 1, 0)).reshape(-1, seq)
+    return got, got_lse
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bf16", "fp32"])
+def test_reference_signature_caches_the_mask_classes_and_drops_them_on_a_write(oracle, dtype):
+    head, seq, nb, grp, nkv, tile = 64, 256, 2, 1, 2, 64
+    arrs, (qf, kf, vf) = _case(dtype, head, seq, nb, grp, nkv, seed=21)
+    s5, b5 = [head, seq, nb, grp, nkv], [head, tile, 1, 1, 1]
+    T = {n: hm.Tensor(dtype, s5, b5).from_array(arrs[n]) for n in ("K", "Q", "V")}
+    causal = synth.causal_mask(seq, seq)
+    i = np.arange(seq)
+    window = np.abs(i[None, :] - i[:, None]) <= 40
+    n_t = seq // tile
+    slabs = nb * grp * nkv
+
+    def run(M, mask_bool):
+        A, lse = _outputs(dtype, s5, b5)
+        tasks0, (h0, m0) = hm.tasks_submitted(dtype), hm.mask_cache_stats()
+        hm.flash_sdpa_fwd(hm.OP_TENSOR, T["K"], T["Q"], M, lse, T["V"], A)
+        (h1, m1) = hm.mask_cache_stats()
+        got, got_lse = _read_out(dtype, A, lse, head, seq)
+        want, want_lse = oracle.sdpa_vanilla(kf, qf, vf, mask_bool, k_tile=tile)
+        assert H.rel_fro(got, want) < H.TOL[dtype] and H.rel_fro(got_lse, want_lse) < H.TOL[dtype]
+        return hm.tasks_submitted(dtype) - tasks0, h1 - h0, m1 - m0
+
+    arr, M = _mask_tensor(dtype, causal, tile)
+    M.from_array(arr)
+    # first sight: classified (a miss); the causal rule: no tile tasks
+    assert run(M, causal) == (0, 0, 1)
+    # the same mask again: found, nothing re-read
+    assert run(M, causal) == (0, 1, 0)
+    assert run(M, causal) == (0, 1, 0)
+    # the mask is rewritten with a window: the classes are dropped, the result
+    # follows the new contents, pairs the window hides are not submitted and
+    # the others take the tile path (their tiles are MIXED) or the open path
+    arr_w, _ = _mask_tensor(dtype, window, tile)
+    M.from_array(arr_w)
+    tasks, hits, misses = run(M, window)
+    assert (hits, misses) == (0, 1)
+    live = sum(1 for q in range(n_t) for k in range(n_t)
+               if window[q * tile:(q + 1) * tile, k * tile:(k + 1) * tile].any())
+    mixed = sum(1 for q in range(n_t) for k in range(n_t)
+                if window[q * tile:(q + 1) * tile, k * tile:(k + 1) * tile].any()
+                and not window[q * tile:(q + 1) * tile, k * tile:(k + 1) * tile].all())
+    assert live < n_t * n_t and 0 < tasks <= slabs * mixed
+    assert run(M, window)[1:] == (1, 0)
+    # a writer got the tiles (same contents): classified again, same answer
+    M.mark_written()
+    assert run(M, window)[1:] == (0, 1)
+    # back to the causal contents
+    M.from_array(arr)
+    assert run(M, causal) == (0, 0, 1)
+    # another tensor, freed and re-created in between (its memory may be
+    # the one the freed tensor had): never served from the old entry
+    for mask_bool in (window, causal, window):
+        arr2, M2 = _mask_tensor(dtype, mask_bool, tile)
+        M2.from_array(arr2)
+        assert run(M2, mask_bool)[1:] == (0, 1)
+        del M2
+
+
+@pytest.mark.gpu
+def test_reference_signature_with_a_bias_mask_is_the_reference_submission_bit_for_bit():
+    dtype, head, seq, nb, grp, nkv, tile = "bf16", 64, 256, 2, 1, 2, 128
+    arrs, _ = _case(dtype, head, seq, nb, grp, nkv, seed=22)
+    s5, b5 = [head, seq, nb, grp, nkv], [head, tile, 1, 1, 1]
+    i = np.arange(seq)
+    bias = (-0.25 * np.abs(i[:, None] - i[None, :]) - 0.25).astype(np.float32)
+    outs = []
+    for op in (hm.OP_PAIRS, hm.OP_TENSOR, hm.OP_TENSOR):
+        T = {n: hm.Tensor(dtype, s5, b5).from_array(arrs[n]) for n in ("K", "Q", "V")}
+        arr, M = _mask_tensor(dtype, np.ones((seq, seq), bool), tile, values=bias)
+        M.from_array(arr)
+        A, lse = _outputs(dtype, s5, b5)
+        before = hm.tasks_submitted(dtype)
+        hm.flash_sdpa_fwd(op, T["K"], T["Q"], M, lse, T["V"], A)
+        # every pair is a tile task with its mask tile, in both forms
+        assert hm.tasks_submitted(dtype) - before == A.ntiles * (seq // tile)
+        outs.append((A.to_array().copy(), lse.to_array().copy()))
+    for a, l in outs[1:]:
+        assert np.array_equal(outs[0][0], a) and np.array_equal(outs[0][1], l)

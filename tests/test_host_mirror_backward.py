@@ -167,9 +167,9 @@ def test_reference_tensor_test_multi_tile_equals_single_tile(oracle, dtype, case
     lse = (0.1 * (np.arange(batch * seq) % 10 - 5)).astype(np.float32).reshape(batch, seq)
     i = np.arange(seq)
     add = np.where(np.abs(i[:, None] - i[None, :]) <= 32, 0.0, -np.inf).astype(np.float32)
-    single, tasks1, _ = _run(hm.OP_TENSOR, dtype, data, lse, add, shape5, shape5)
+    single, tasks1, _ = _run(hm.OP_PAIRS_BWD, dtype, data, lse, add, shape5, shape5)
     assert tasks1 == 1
-    multi, tasks, ntiles = _run(hm.OP_TENSOR, dtype, data, lse, add, shape5,
+    multi, tasks, ntiles = _run(hm.OP_PAIRS_BWD, dtype, data, lse, add, shape5,
                                 [head, seq_tile, nb_tile, grp_tile, nkv_tile])
     # one task per (dQ tile, key tile), none skipped (src/tensor/...:172-247)
     assert tasks == ntiles * (seq // seq_tile)
@@ -281,7 +281,7 @@ def test_classified_submission_skips_hidden_tile_pairs(oracle, dtype, kind, offs
     _, af = H.rounded(A64, dtype)
     data = {"K": kf, "Q": qf, "V": vf, "A": af, "dA": gf}
     got, pairs, ntiles = _run(hm.OP_CLASSIFIED, dtype, data, lse, add, shape5, base5, offset=offset)
-    ref, all_pairs, _ = _run(hm.OP_TENSOR, dtype, data, lse, add, shape5, base5)
+    ref, all_pairs, _ = _run(hm.OP_PAIRS_BWD, dtype, data, lse, add, shape5, base5)
     nt = seq // tile
     slabs = ntiles // nt
     live = sum(1 for q in range(nt) for k in range(nt)
@@ -295,3 +295,14 @@ def test_classified_submission_skips_hidden_tile_pairs(oracle, dtype, kind, offs
     for g, r, w, n in zip(got, ref, want, ("dK", "dQ", "dV")):
         assert H.rel_fro(g, w) < tol, n
         assert H.rel_fro(g, r) < tol, n
+    if offset == 0:
+        # the reference's signature classifies the mask itself (rule key <= query)
+        # and submits the same calls: same bits, and only MIXED pairs as tile tasks
+        dflt, tile_tasks, _ = _run(hm.OP_TENSOR, dtype, data, lse, add, shape5, base5)
+        for g, d, n in zip(got, dflt, ("dK", "dQ", "dV")):
+            assert np.array_equal(g, d), n
+        mixed = sum(1 for q in range(nt) for k in range(nt)
+                    if mask[q * tile:(q + 1) * tile, k * tile:(k + 1) * tile].any()
+                    and not mask[q * tile:(q + 1) * tile, k * tile:(k + 1) * tile].all()
+                    and not (kind == "causal" and q == k))
+        assert tile_tasks == slabs * mixed
