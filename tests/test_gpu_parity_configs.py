@@ -40,6 +40,7 @@ def test_cfg1_single_head_fp32(oracle):
     torch.cuda.synchronize()
     assert H.rel_fro(H.to_np(A), want) < 1e-4
     assert H.rel_fro(H.to_np(lse), want_lse) < 1e-4
+    H.check_rows(H.to_np(A), want, H.to_np(lse), want_lse, "fp32", "cfg1")
 
 
 def test_cfg2_gpt2_small_fp32(oracle):
@@ -61,6 +62,7 @@ def test_cfg2_gpt2_small_fp32(oracle):
         A_all[:, nb], lse_all[:, nb] = H.to_np(A), H.to_np(lse)
     assert H.rel_fro(A_all.reshape(want.shape), want) < 1e-4
     assert H.rel_fro(lse_all.reshape(want_lse.shape), want_lse) < 1e-4
+    H.check_rows(A_all.reshape(want.shape), want, lse_all.reshape(want_lse.shape), want_lse, "fp32", "cfg2")
 
 
 def _split(t, tile):
@@ -84,6 +86,7 @@ def test_cfg3_llama_prefill_bf16(oracle):
     lse = np.concatenate([H.to_np(o[0]) for o in outs], axis=1)
     assert H.rel_fro(A, want) < 1e-2
     assert H.rel_fro(lse, want_lse) < 1e-2
+    H.check_rows(A, want, lse, want_lse, "bf16", "cfg3 one launch")
     # (b) the reference's task structure: 16 calls, additive mask tiles, the
     # running (lse, A) carried through memory across the 4 key tiles
     outs2 = [H.fresh_outputs(cfg.batch_flat, t, cfg.head, "bf16") for _ in range(nt)]
@@ -96,6 +99,7 @@ def test_cfg3_llama_prefill_bf16(oracle):
     lse2 = np.concatenate([H.to_np(o[0]) for o in outs2], axis=1)
     assert H.rel_fro(A2, want) < 1e-2
     assert H.rel_fro(lse2, want_lse) < 1e-2
+    H.check_rows(A2, want, lse2, want_lse, "bf16", "cfg3 sixteen tasks")
 
 
 def test_cfg4_gqa_decode_bf16(oracle):
@@ -112,6 +116,7 @@ def test_cfg4_gqa_decode_bf16(oracle):
     torch.cuda.synchronize()
     assert H.rel_fro(H.to_np(A), want) < 1e-2
     assert H.rel_fro(H.to_np(lse), want_lse) < 1e-2
+    H.check_rows(H.to_np(A), want, H.to_np(lse), want_lse, "bf16", "cfg4 decode")
     # the same answer from the prefill tile kernel with the GQA index map
     lse2, A2 = H.fresh_outputs(cfg.batch_flat, cfg.q_seq, cfg.head, "bf16")
     hip_sdpa.sdpa_fwd_tile(Kd, Qd, None, lse2, Vd, A2, hip_sdpa.MASK_CAUSAL, n_batch=cfg.n_batch,
@@ -119,6 +124,7 @@ def test_cfg4_gqa_decode_bf16(oracle):
     torch.cuda.synchronize()
     assert H.rel_fro(H.to_np(A2), want) < 1e-2
     assert H.rel_fro(H.to_np(lse2), want_lse) < 1e-2
+    H.check_rows(H.to_np(A2), want, H.to_np(lse2), want_lse, "bf16", "cfg4 tile kernel")
 
 
 def test_cfg5_long_sequence_bf16(oracle):
@@ -144,6 +150,8 @@ def test_cfg5_long_sequence_bf16(oracle):
                                              np.ascontiguousarray(mask[rows]), k_tile=t)
         assert H.rel_fro(H.to_np(outs[qi][1]), want) < 1e-2
         assert H.rel_fro(H.to_np(outs[qi][0]), want_lse) < 1e-2
+        H.check_rows(H.to_np(outs[qi][1]), want, H.to_np(outs[qi][0]), want_lse, "bf16",
+                     "cfg5 query tile %d" % qi)
     # exact property over the whole output: doubling V doubles A bit for bit
     # and leaves lse unchanged (a power-of-two scale commutes with rounding)
     V2 = [v * 2 for v in Vt]
@@ -170,3 +178,4 @@ def test_cfg5_long_sequence_bf16(oracle):
     torch.cuda.synchronize()
     assert H.rel_fro(H.to_np(A_pt), want) < 1e-2
     assert H.rel_fro(H.to_np(lse_pt), want_lse) < 1e-2
+    H.check_rows(H.to_np(A_pt), want, H.to_np(lse_pt), want_lse, "bf16", "cfg5 sixteen hand-offs")
