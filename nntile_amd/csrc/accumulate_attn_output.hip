@@ -35,7 +35,10 @@ struct Fp16Store
 __device__ __forceinline__ bool row_weights(float have, float inc, float &w_have,
         float &w_inc, float &merged)
 {
-    if(inc == neg_inf())
+    // A source row whose logsumexp is not finite (-inf: no key seen; NaN or
+    // +inf: a broken partial) leaves the destination as it is, the rule of the
+    // reference's GPU kernel (src/kernel/accumulate_attn_output/cuda.cu:43-50).
+    if(!__builtin_isfinite(inc))
     {
         return false;
     }

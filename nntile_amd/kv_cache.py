@@ -112,6 +112,17 @@ class KVCache:
         sliced = None
         if mask is not None:
             sliced, mode = self.mask_slice(mask, q_seq), hip_sdpa.MASK_BOOL
+
+        def keep(t):
+            # The kernels are enqueued through ctypes; torch's allocator does
+            # not know they read t.  On a stream other than the current one the
+            # allocator is told; in every case the tensor stays referenced
+            # here until the next call.
+            if stream is not None and t is not None:
+                t.record_stream(stream)
+            return t
+
+        self._mask_in_use = keep(sliced)
         decode = (Q.dtype != torch.float32 and kv_group * q_seq <= 64
                   and Q.shape[2] in (64, 128))
         if not decode:
@@ -121,7 +132,11 @@ class KVCache:
             return
         need = hip_sdpa.decode_cache_workspace_bytes(k_seq, Q, n_batch, kv_group)
         if self._workspace is None or self._workspace.numel() < need:
+            # (a launch of an earlier call may still read the old workspace:
+            # it is kept until the one after next replaces it)
+            self._retired_workspace = self._workspace
             self._workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
+        keep(self._workspace)
         hip_sdpa.sdpa_fwd_decode_cache(
             self.k, self.v, k_seq, Q, sliced, lse, A, mode, n_batch, kv_group, self._workspace,
             causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)

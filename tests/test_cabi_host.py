@@ -103,3 +103,42 @@ def test_accumulate_zero_sizes_return_silently():
     L = h.lib()
     assert L.nntile_hip_accumulate_attn_output_fp32(None, 0, 4, 4, None, None, None, None) == h.OK
     assert L.nntile_hip_accumulate_attn_output_fp32(None, 8, 4, 4, None, None, None, None) == h.EINVAL
+
+
+def test_starpu_registration_unit_compiles_to_stubs_here():
+    """StarPU is not installed in this image: the registration unit reduces
+    to two stubs that say so."""
+    from nntile_amd import host_mirror as hm
+    L = hm.lib()
+    assert L.nntile_hip_starpu_available() == 0
+    assert L.nntile_hip_starpu_register(None, None, 0) == -1
+
+
+def test_starpu_registration_unit_is_valid_against_the_api_it_names(tmp_path):
+    """Syntax check of the StarPU branch of the registration unit against a
+    declaration-only rendering of the StarPU API it uses (starpu_codelet's
+    hip_funcs / hip_flags / where, STARPU_HIP, STARPU_HIP_ASYNC,
+    starpu_hip_get_local_stream, struct starpu_variable_interface as published
+    in starpu_data_interfaces.h).  Nothing is linked or run: this only keeps the
+    guarded code from rotting where StarPU is absent.  The struct layout is
+    asserted again, against the real header, wherever StarPU is installed."""
+    import shutil
+    import subprocess
+    gxx = shutil.which("g++")
+    if gxx is None:
+        pytest.skip("g++ not found")
+    (tmp_path / "starpu.h").write_text(
+        "#pragma once\n#include <stddef.h>\n#include <stdint.h>\n"
+        "#define STARPU_MAXIMPLEMENTATIONS 4\n#define STARPU_HIP (1 << 7)\n"
+        "#define STARPU_HIP_ASYNC 1\n"
+        "struct starpu_codelet { uint32_t where; void (*hip_funcs[STARPU_MAXIMPLEMENTATIONS])(void **, void *);"
+        " char hip_flags[STARPU_MAXIMPLEMENTATIONS]; };\n"
+        "struct starpu_variable_interface { int id; uintptr_t ptr; uintptr_t dev_handle; size_t offset;"
+        " size_t elemsize; };\n")
+    (tmp_path / "starpu_hip.h").write_text(
+        "#pragma once\ntypedef struct ihipStream_t *hipStream_t;\n"
+        "extern \"C\" hipStream_t starpu_hip_get_local_stream(void);\n")
+    unit = os.path.join(ROOT, "nntile_amd", "host", "starpu_hip_registration.cc")
+    r = subprocess.run([gxx, "-std=c++17", "-fsyntax-only", "-Wall", "-Werror", "-I", str(tmp_path), unit],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr

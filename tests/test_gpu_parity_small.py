@@ -221,6 +221,43 @@ def test_accumulate_attn_output_preset(oracle, dtype, head, seq, batch):
     assert np.max(np.abs(got_lse[fin] - want_lse[fin])) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("head", [128, 6])      # the 16-byte path and the element path
+def test_accumulate_attn_output_skips_rows_whose_source_logsumexp_is_not_finite(dtype, head):
+    """src/kernel/accumulate_attn_output/cuda.cu:43-50: a source row with a
+    non-finite logsumexp (-inf, NaN, +inf) has no influence; its destination
+    row - values and logsumexp, even a -inf one with NaN values behind it - stays
+    bit for bit.  (The reference's CPU statement only knows -inf, cpu.cc:73-97;
+    the GPU kernel is what this entry point replaces.)"""
+    seq, batch = 9, 2
+    rows = seq * batch
+    src_lse = np.linspace(-1.0, 1.0, rows).astype(np.float32)
+    bad = {1: np.nan, 4: np.inf, 7: -np.inf, 10: np.nan, 13: -np.inf}
+    for r, v in bad.items():
+        src_lse[r] = v
+    dst_lse = np.linspace(0.5, -0.5, rows).astype(np.float32)
+    dst_lse[10] = -np.inf
+    dt = H.TORCH_DT[dtype]
+    g = torch.Generator().manual_seed(5)
+    src = torch.randn(batch, seq, head, generator=g).to(dt)
+    dst = torch.randn(batch, seq, head, generator=g).to(dt)
+    dst.view(rows, head)[10] = float("nan")        # never read: its logsumexp is -inf
+    Dd, dl = dst.clone().cuda(), torch.from_numpy(dst_lse.reshape(batch, seq)).cuda()
+    hip_sdpa.accumulate_attn_output(torch.from_numpy(src_lse.reshape(batch, seq)).cuda(), src.cuda(), dl, Dd)
+    torch.cuda.synchronize()
+    bits = lambda t: t.cpu().contiguous().view(torch.int32 if t.element_size() == 4 else torch.int16)
+    got, got_lse = Dd.cpu().view(rows, head), dl.cpu().view(rows)
+    for r in range(rows):
+        if r in bad:
+            assert torch.equal(bits(got[r]), bits(dst.view(rows, head)[r])), r
+            assert np.array_equal(got_lse[r:r + 1].numpy().view(np.int32),
+                                  dst_lse[r:r + 1].view(np.int32)), r
+        else:
+            want_lse = np.logaddexp(np.float64(dst_lse[r]), np.float64(src_lse[r]))
+            assert abs(float(got_lse[r]) - want_lse) < 1e-5, r
+            assert torch.isfinite(got[r].float()).all(), r
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])
 def test_codelet_body(oracle, dtype):
     """The StarPU-shaped body with the reference's buffer order, run twice on

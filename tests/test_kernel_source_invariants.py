@@ -64,6 +64,23 @@ def test_m0_is_written_only_by_the_lds_load_helper(assemblies):
     assert uses > 0     # the prefill and decode kernels do use the helper
 
 
+# Instructions that read or write M0 without naming it: relative register
+# addressing, the GPR index mode, messages, global wave sync, LDS parameter
+# and direct loads, and LDS instructions in the add-TID form.  (An "m0"
+# clobber on the helper's assembly text is not an alternative: M0 is a
+# reserved register for the compiler, which warns that such a clobber is not
+# honoured.)
+IMPLICIT_M0 = (r"^(s_movrel[sd]_|v_movrel[sd]|v_movrelsd|s_set_gpr_idx_|s_sendmsg|s_sendmsghalt|"
+               r"ds_gws_|v_interp_|lds_param_load|lds_direct_load|ds_\w+_addtid_|s_ttracedata|"
+               r"v_readlane_b32 \S+ \S+ m0|v_writelane_b32 \S+ \S+ m0)")
+
+
+def test_no_instruction_uses_m0_implicitly(assemblies):
+    for name, text in assemblies.items():
+        for line in _instructions(text):
+            assert not re.match(IMPLICIT_M0, line), (name, line)
+
+
 def test_every_lds_load_sets_m0_first(assemblies):
     for name, text in assemblies.items():
         ins = list(_instructions(text))
