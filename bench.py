@@ -28,11 +28,28 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 
 
 # HBM bytes per launch from the hardware counters (FETCH_SIZE x 2.000 +
-# WRITE_SIZE x 1.000, the factors a 1 GiB device copy calibrates); the runs
-# and their figures are in profiles/sdpa_*_kernel_cfg*.txt.  They are
-# properties of the kernel and the workload, not of one timing run.
-TRAFFIC_PREFILL_CFG3 = 175220098
-TRAFFIC_DECODE_CFG4 = 295683470
+# WRITE_SIZE x 1.000, the factors a 1 GiB device copy calibrates).  They are
+# properties of the kernel and the workload, not of one timing run; each names
+# the committed rocprofv3 summary it was read from.
+TRAFFIC = {
+    "cfg3_llama_prefill_bf16": (175220098, "profiles/sdpa_prefill_16bit_kernel_cfg3_llama_prefill_bf16.txt"),
+    "cfg4_gqa_decode_bf16": (295683470, "profiles/sdpa_decode_16bit_kernel_cfg4_gqa_decode_bf16.txt"),
+}
+
+
+def roofline(bound, kernel, work, ms, peak, unit, traffic=None, extra=None):
+    """The roofline object of one leg: work (FLOPs or bytes) per step over the
+    device time per step, against the published peak."""
+    scale = 1e12 if bound == "mfma" else 1e9
+    achieved = work / (ms * 1e-3) / scale
+    r = {"bound": bound, "kernel": kernel, "achieved": round(achieved, 2), "peak": peak,
+         "unit": unit, "frac": round(achieved / peak, 4), "kernel_ms": round(ms, 4),
+         "traffic": None, "traffic_source": None}
+    if traffic is not None:
+        r["traffic"], r["traffic_source"] = traffic
+    if extra:
+        r.update(extra)
+    return r
 
 
 def time_steps(step, steps, warmup):
@@ -58,127 +75,129 @@ def time_steps(step, steps, warmup):
         pass
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
-    dev = a.elapsed_time(b) / steps
+    # the events sit inside the two host time stamps
+    dev = min(a.elapsed_time(b) / steps, wall)
     return wall, dev
 
 
-def _randn(shape, dtype, seed):
-    import torch
-    g = torch.Generator(device="cuda")
-    g.manual_seed(seed)
-    return torch.randn(shape, generator=g, device="cuda", dtype=torch.float32).to(dtype)
+def _randn(shape, dtype, seed, stream=0):
+    """i.i.d. N(0,1) values of stream (seed, stream) of the counter-based
+    generator the parity tests use (nntile_amd/synth.py), evaluated on the
+    GPU, in C order of `shape` (= Fortran order of the NNTile tile), rounded
+    to the tile type."""
+    import numpy as np
+    from nntile_amd import synth
+    n = int(np.prod(shape))
+    return synth.randn_torch(seed, stream, n, "cuda").view(shape).to(dtype)
 
 
-def bench_prefill(cfg, steps, warmup, per_task=False, classified=False, streams=1):
-    """Fused: one launch for the whole tile grid (analytic causal mask, tile
-    skipping).  per_task: the reference's task structure - one launch per
-    (query tile, key tile) pair with a materialised additive mask tile, no
-    skipping, (lse, A) handed over in memory between launches.
-    classified (with per_task): the mask tiles are classified once, outside the
-    timed region, as a layer would when it builds its mask; pairs whose tile
-    hides everything are not launched, open and causal ones run without
-    reading the mask.
-    streams > 1 (with per_task): the tasks of query tile i go to stream
-    i % streams, as StarPU workers with their own streams would run them; tasks
-    that share an (lse, A) tile stay ordered on one stream.  The timed region
-    ends when the launch stream has waited for all of them."""
+DATA = ("synthetic: i.i.d. N(0,1) from the counter-based generator of the parity tests "
+        "(nntile_amd/synth.py: splitmix64 -> Box-Muller) evaluated on the GPU, seed 42 + config "
+        "index, streams Q, K, V in that order, each tensor drawn in Fortran element order and "
+        "rounded to the tile type; legs that rotate buffer sets draw the further sets from "
+        "further streams")
+
+
+def _outliers(cfg, q):
+    """cfg5: the query positions (first floor(frac * seq) of a seeded
+    permutation) scaled across all heads, as in the parity test."""
+    if cfg.outlier_frac > 0:
+        import torch
+        from nntile_amd import synth
+        rows = synth.permutation(cfg.seed, 7, cfg.q_seq)[:int(cfg.outlier_frac * cfg.q_seq)]
+        q[:, torch.from_numpy(rows.copy()).cuda(), :] *= cfg.outlier_scale
+    return q
+
+
+def bench_prefill(cfg, steps, warmup):
+    """One fused launch per independent slab of cfg over its whole tile grid
+    (analytic causal mask, hidden tile pairs skipped, overwrite mode).  Tiles
+    are separate allocations, as NNTile tensors are."""
     import torch
-    from nntile_amd import hip_sdpa as h, synth
+    from nntile_amd import hip_sdpa as h
     dt = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[cfg.dtype]
     per_call = cfg.batch_flat // cfg.calls
     nt = cfg.q_seq // cfg.seq_tile
-    calls = []
+    shape = (cfg.batch_flat, cfg.q_seq, cfg.head)
+    q_all = _outliers(cfg, _randn(shape, torch.float32, cfg.seed, 0)).to(dt)
+    k_all, v_all = _randn(shape, dt, cfg.seed, 1), _randn(shape, dt, cfg.seed, 2)
+    plans = []
+    keep = []
     for c in range(cfg.calls):
-        mk = lambda o: [_randn((per_call, cfg.seq_tile, cfg.head), dt,
-                               cfg.seed * 1000 + c * 100 + o * 10 + i) for i in range(nt)]
-        Q, K, V = mk(0), mk(1), mk(2)
+        sl = slice(c * per_call, (c + 1) * per_call)
+        tiles = lambda x: [x[sl, i * cfg.seq_tile:(i + 1) * cfg.seq_tile].contiguous() for i in range(nt)]
+        Q, K, V = tiles(q_all), tiles(k_all), tiles(v_all)
         A = [torch.zeros_like(q) for q in Q]
         lse = [torch.full((per_call, cfg.seq_tile), float("-inf"), device="cuda") for _ in range(nt)]
-        calls.append((Q, K, V, A, lse))
-    masks = None
-    if per_task:
-        full = synth.causal_mask(cfg.q_seq, cfg.k_seq)
-        t = cfg.seq_tile
-        masks = [[torch.from_numpy(full[qi * t:(qi + 1) * t, ki * t:(ki + 1) * t].copy()).cuda()
-                  for ki in range(nt)] for qi in range(nt)]
-        masks = [[torch.where(m, 0.0, float("-inf")).to(dt) for m in row] for row in masks]
-
-    def reset():
-        for _, _, _, _, lse in calls:
-            for l in lse:
-                l.fill_(float("-inf"))
-
-    # Calls are prepared once (tile addresses do not change between steps).
-    plans = []
-    plan_stream = []
-    side = [torch.cuda.Stream() for _ in range(streams)] if streams > 1 else []
-    classes = None
-    if per_task and classified:
-        t = cfg.seq_tile
-        classes = [[h.mask_tile_class(masks[qi][ki], (qi - ki) * t) for ki in range(nt)]
-                   for qi in range(nt)]
-    whole = None
-    if classes is not None:
-        # what tensor::flash_sdpa_mask_rule decides from the classes: a mask
-        # that is the causal rule itself needs no tasks per pair
-        t = cfg.seq_tile
-        expect = [[h.TILE_OPEN if (ki + 1) * t - 1 <= qi * t else
-                   (h.TILE_HIDDEN if ki * t > (qi + 1) * t - 1 else h.TILE_CAUSAL)
-                   for ki in range(nt)] for qi in range(nt)]
-        if classes == expect:
-            whole = h.MASK_CAUSAL
-    for Q, K, V, A, lse in calls:
-        if whole is not None:
-            plan_stream.append(0)
-            plans.append(h.plan_grid(K, Q, lse, V, A, cfg.q_seq, cfg.k_seq, cfg.seq_tile,
-                                     cfg.seq_tile, whole))
-        elif per_task:
-            for qi in range(nt):
-                for ki in range(nt):
-                    cls = h.TILE_MIXED if classes is None else classes[qi][ki]
-                    if cls == h.TILE_HIDDEN:
-                        continue
-                    plan_stream.append(qi % streams)
-                    if cls == h.TILE_MIXED:
-                        plans.append(h.plan_tile(K[ki], Q[qi], masks[qi][ki], lse[qi], V[ki],
-                                                 A[qi], h.MASK_ADDITIVE))
-                    else:
-                        mode = h.MASK_NONE if cls == h.TILE_OPEN else h.MASK_CAUSAL
-                        plans.append(h.plan_tile(K[ki], Q[qi], None, lse[qi], V[ki], A[qi], mode,
-                                                 q_pos0=qi * cfg.seq_tile, k_pos0=ki * cfg.seq_tile))
-        else:
-            plans.append(h.plan_grid(K, Q, lse, V, A, cfg.q_seq, cfg.k_seq, cfg.seq_tile,
-                                     cfg.seq_tile, h.MASK_CAUSAL, flags=h.OVERWRITE))
-
-    def kernels_only():
-        if not side:
-            for pl in plans:
-                pl.launch()
-            return
-        main = torch.cuda.current_stream()
-        for st in side:
-            st.wait_stream(main)
-        for pl, si in zip(plans, plan_stream):
-            pl.launch(side[si])
-        for st in side:
-            main.wait_stream(st)
+        keep.append((Q, K, V, A, lse))
+        plans.append(h.plan_grid(K, Q, lse, V, A, cfg.q_seq, cfg.k_seq, cfg.seq_tile,
+                                 cfg.seq_tile, h.MASK_CAUSAL, flags=h.OVERWRITE))
+    del q_all, k_all, v_all
 
     def step():
-        # per_task: lse must start at -inf each pass; that fill is part of the
-        # op's contract (layer/sdpa.py:538) and is timed with it.  The fused
-        # launch runs in OVERWRITE mode, which needs no fill.
-        if per_task:
-            reset()
-        kernels_only()
+        for pl in plans:
+            pl.launch()
 
     wall, dev = time_steps(step, steps, warmup)
-    reset()
-    _, kdev = time_steps(kernels_only, steps, 2)
-    launches = len(plans)
-    return {"ms_per_step": wall, "device_ms_per_step": dev, "kernel_ms_per_step": kdev,
-            "launches_per_step": launches,
-            "tflops": cfg.flops() / (wall * 1e-3) / 1e12,
-            "kernel_tflops": cfg.flops() / (kdev * 1e-3) / 1e12}
+    return {"ms_per_step": wall, "device_ms_per_step": dev, "launches_per_step": len(plans),
+            "tflops": cfg.flops() / (wall * 1e-3) / 1e12}
+
+
+def bench_reference_grid(steps, warmup):
+    """The reference's own benchmark grid for this kernel
+    (tests/kernel/flash_sdpa_fwd_cudnn.cc:591-613): seq in {128, 1024, 4096} x
+    head in {64, 128} x batch in {4, 8} x {causal, full} x {bf16, fp16}, one
+    square tile, random data.  Each case twice: through
+    nntile_hip_flash_sdpa_fwd_* with the additive mask tile the reference
+    passes (merge into an lse of -inf, as its test does), and through the tile
+    entry point with the same mask given analytically (overwrite mode).
+    FLOPs: 4 * head * visible pairs * batch (causal-exact for the causal mask)."""
+    import numpy as np
+    import torch
+    from nntile_amd import hip_sdpa as h, synth
+    rows = []
+    for dtype, dt in (("bf16", torch.bfloat16), ("fp16", torch.float16)):
+        for seq in (128, 1024, 4096):
+            vis = synth.causal_mask(seq, seq)
+            masks = {"causal": torch.from_numpy(np.where(vis, 0.0, -np.inf).astype(np.float32)).to(dt).cuda(),
+                     "full": torch.zeros((seq, seq), dtype=dt, device="cuda")}
+            for head in (64, 128):
+                for batch in (4, 8):
+                    shape = (batch, seq, head)
+                    Q, K, V = (_randn(shape, dt, 42, i) for i in range(3))
+                    A = torch.zeros_like(Q)
+                    lse = torch.empty((batch, seq), dtype=torch.float32, device="cuda")
+                    for mask_type in ("causal", "full"):
+                        pairs = seq * (seq + 1) // 2 if mask_type == "causal" else seq * seq
+                        flops = 4.0 * head * pairs * batch
+                        m = masks[mask_type]
+                        additive = h.plan_tile(K, Q, m, lse, V, A, h.MASK_ADDITIVE)
+
+                        def with_mask():
+                            lse.fill_(float("-inf"))
+                            additive.launch()
+
+                        analytic = h.plan_tile(K, Q, None, lse, V, A,
+                                               h.MASK_CAUSAL if mask_type == "causal" else h.MASK_NONE,
+                                               flags=h.OVERWRITE)
+                        _, dev_mask = time_steps(with_mask, steps, warmup)
+                        _, dev_an = time_steps(analytic.launch, steps, warmup)
+                        tf_mask = flops / (dev_mask * 1e-3) / 1e12
+                        tf_an = flops / (dev_an * 1e-3) / 1e12
+                        rows.append({"dtype": dtype, "seq": seq, "head": head, "batch": batch,
+                                     "mask": mask_type,
+                                     "additive_mask_ms": round(dev_mask, 4),
+                                     "additive_mask_tflops": round(tf_mask, 1),
+                                     "additive_mask_frac": round(tf_mask / PEAK_BF16_TFLOPS, 4),
+                                     "analytic_ms": round(dev_an, 4),
+                                     "analytic_tflops": round(tf_an, 1),
+                                     "analytic_frac": round(tf_an / PEAK_BF16_TFLOPS, 4)})
+    return {"what": "the reference's benchmark grid (tests/kernel/flash_sdpa_fwd_cudnn.cc:591-613), one "
+                    "square tile per case: additive_mask = nntile_hip_flash_sdpa_fwd_* with the "
+                    "materialised mask (plus the -inf fill of lse), analytic = the same mask as a rule "
+                    "(overwrite mode); device ms per call, TFLOP/s on causal-exact / dense FLOPs, "
+                    "fraction of the 2.5 PFLOP/s bf16/fp16 MFMA peak",
+            "cases": rows}
 
 
 def bench_reference_api(cfg, steps, warmup):
@@ -197,8 +216,10 @@ def bench_reference_api(cfg, steps, warmup):
     b5 = [cfg.head, cfg.seq_tile, cfg.n_batch, 1, cfg.n_head_kv]
     n = int(np.prod(s5))
     T = {}
+    import torch
     for i, name in enumerate(("Q", "K", "V")):
-        bits = synth.round_bf16(synth.randn(cfg.seed, i, n))[0]
+        bits = synth.randn_torch(cfg.seed, i, n, "cuda").to(torch.bfloat16).view(torch.int16) \
+            .cpu().numpy().view(np.uint16)
         T[name] = hm.Tensor("bf16", s5, b5).from_array(bits.reshape(s5, order="F"))
     A = hm.Tensor("bf16", s5, b5).from_array(np.zeros(s5, np.uint16))
     lse = hm.Tensor("fp32", s5[1:], b5[1:]).from_array(np.full(s5[1:], -np.inf, np.float32))
@@ -218,13 +239,16 @@ def bench_reference_api(cfg, steps, warmup):
 
 
 def bench_decode(cfg, steps, warmup):
+    """The GQA decode shape: main kernel + merge of the key splits per step.
+    Four (K, V) sets rotate (4 x 256 MiB at cfg4: the 256 MiB last-level cache
+    cannot serve a pass)."""
     import torch
     from nntile_amd import hip_sdpa as h
     kvb = cfg.n_batch * cfg.n_head_kv
-    nrot = 4      # 4 x 256 MiB of K+V: the 256 MiB last-level cache cannot serve a pass
-    Ks = [_randn((kvb, cfg.k_seq, cfg.head), torch.bfloat16, cfg.seed * 1000 + i) for i in range(nrot)]
-    Vs = [_randn((kvb, cfg.k_seq, cfg.head), torch.bfloat16, cfg.seed * 1000 + 50 + i) for i in range(nrot)]
-    Q = _randn((cfg.batch_flat, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed * 1000 + 99)
+    nrot = 4
+    Ks = [_randn((kvb, cfg.k_seq, cfg.head), torch.bfloat16, cfg.seed, 1 + 10 * j) for j in range(nrot)]
+    Vs = [_randn((kvb, cfg.k_seq, cfg.head), torch.bfloat16, cfg.seed, 2 + 10 * j) for j in range(nrot)]
+    Q = _randn((cfg.batch_flat, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed, 0)
     A = torch.zeros_like(Q)
     lse = torch.full((cfg.batch_flat, cfg.q_seq), float("-inf"), device="cuda")
     ws = torch.empty(h.decode_workspace_bytes(Ks[0], Q, cfg.n_batch, cfg.kv_group),
@@ -239,26 +263,23 @@ def bench_decode(cfg, steps, warmup):
         i[0] += 1
 
     wall, dev = time_steps(step, steps, warmup)
-    _, kdev = time_steps(step, steps, 2)
     nbytes = cfg.algorithmic_bytes()
-    return {"ms_per_step": wall, "device_ms_per_step": dev, "kernel_ms_per_step": kdev,
-            "gbs": nbytes / (wall * 1e-3) / 1e9, "kernel_gbs": nbytes / (kdev * 1e-3) / 1e9,
-            "algorithmic_bytes": nbytes, "workspace_bytes": ws.numel(),
-            "tflops": cfg.flops() / (wall * 1e-3) / 1e12}
+    return {"ms_per_step": wall, "device_ms_per_step": dev,
+            "gbs": nbytes / (wall * 1e-3) / 1e9, "algorithmic_bytes": nbytes,
+            "workspace_bytes": ws.numel(), "tflops": cfg.flops() / (wall * 1e-3) / 1e12}
 
 
 def bench_backward(cfg, steps, warmup):
     """Backward of the same attention (dQ, dK, dV from dA, A and lse) as one
     call over the whole sequence with the analytic causal mask: the row dots,
-    then one launch for the three gradients.
-    FLOPs counted as 2.5 x the forward's (five products where the forward has
-    two); the workgroups execute eight, recomputing the scores for each
-    gradient."""
+    then one launch for the three gradients.  FLOPs counted as 2.5 x the
+    forward's (five products where the forward has two); the workgroups
+    execute eight, recomputing the scores for each gradient."""
     import torch
     from nntile_amd import hip_sdpa as h
     dt = {"bf16": torch.bfloat16, "fp16": torch.float16}[cfg.dtype]
     shape = (cfg.batch_flat, cfg.q_seq, cfg.head)
-    Q, K, V, G = (_randn(shape, dt, cfg.seed * 1000 + 700 + i) for i in range(4))
+    Q, K, V, G = (_randn(shape, dt, cfg.seed, i) for i in range(4))
     A = torch.zeros_like(Q)
     lse = torch.full((cfg.batch_flat, cfg.q_seq), float("-inf"), device="cuda")
     h.sdpa_fwd_tile(K, Q, None, lse, V, A, h.MASK_CAUSAL, flags=h.OVERWRITE)
@@ -272,11 +293,11 @@ def bench_backward(cfg, steps, warmup):
 
     wall, dev = time_steps(step, steps, warmup)
     fl = 2.5 * cfg.flops()
-    return {"ms_per_step": round(wall, 4), "device_ms_per_step": round(dev, 4),
-            "tflops": round(fl / (dev * 1e-3) / 1e12, 1), "flops_per_step": fl,
-            "frac_of_peak": round(fl / (dev * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
-            "what": "backward of %s in one call (row dots + one launch for dQ, dK, dV), analytic causal "
-                    "mask, gradients written" % cfg.name}
+    return {"workload": cfg.name, "ms_per_step": round(wall, 4), "flops_per_step": fl,
+            "what": "backward of %s in one call (row dots + one launch for dQ, dK, dV), analytic "
+                    "causal mask, gradients written; 2.5 x the forward's causal-exact FLOPs" % cfg.name,
+            "roofline": roofline("mfma", "sdpa_bwd_rowdot_kernel + sdpa_bwd_kernel<bf16,128,causal>",
+                                 fl, dev, PEAK_BF16_TFLOPS, "TFLOP/s")}
 
 
 def bench_rope(cfg, steps, warmup):
@@ -289,10 +310,12 @@ def bench_rope(cfg, steps, warmup):
     from nntile_amd import hip_sdpa as h
     dt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg.dtype]
     half = cfg.head // 2
-    ang = torch.rand(cfg.q_seq, half, device="cuda") * 6.28
+    # the angles of rotary embedding: position x 10000^(-2i/head)
+    freq = 10000.0 ** (-torch.arange(half, device="cuda", dtype=torch.float64) * 2.0 / cfg.head)
+    ang = (torch.arange(cfg.q_seq, device="cuda", dtype=torch.float64)[:, None] * freq[None, :]).float()
     sin, cos = torch.sin(ang).to(dt).contiguous(), torch.cos(ang).to(dt).contiguous()
     nrot = 8
-    src = [_randn((cfg.batch_flat, cfg.q_seq, cfg.head), dt, cfg.seed * 1000 + 800 + i) for i in range(nrot)]
+    src = [_randn((cfg.batch_flat, cfg.q_seq, cfg.head), dt, cfg.seed, 10 * i) for i in range(nrot)]
     dst = [torch.empty_like(x) for x in src]
     i = [0]
 
@@ -321,7 +344,7 @@ def bench_transpose(cfg, steps, warmup):
     dt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg.dtype]
     m, n = cfg.head * cfg.q_seq, cfg.batch_flat
     nrot = 8
-    src = [_randn((n, m), dt, cfg.seed * 1000 + 900 + i) for i in range(nrot)]
+    src = [_randn((n, m), dt, cfg.seed, 10 * i + 5) for i in range(nrot)]
     dst = [torch.empty_like(x) for x in src]
     i = [0]
 
@@ -349,10 +372,10 @@ def bench_accumulate(cfg, steps, warmup):
     dt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[cfg.dtype]
     nrot = 8
     shape = (cfg.batch_flat, cfg.seq_tile, cfg.head)
-    src = [_randn(shape, dt, cfg.seed * 1000 + 600 + i) for i in range(nrot)]
-    dst = [_randn(shape, dt, cfg.seed * 1000 + 620 + i) for i in range(nrot)]
-    src_lse = [_randn(shape[:2], torch.float32, cfg.seed * 1000 + 640 + i) for i in range(nrot)]
-    dst_lse = [_randn(shape[:2], torch.float32, cfg.seed * 1000 + 660 + i) for i in range(nrot)]
+    src = [_randn(shape, dt, cfg.seed, 10 * i + 6) for i in range(nrot)]
+    dst = [_randn(shape, dt, cfg.seed, 10 * i + 7) for i in range(nrot)]
+    src_lse = [_randn(shape[:2], torch.float32, cfg.seed, 10 * i + 8) for i in range(nrot)]
+    dst_lse = [_randn(shape[:2], torch.float32, cfg.seed, 10 * i + 9) for i in range(nrot)]
     i = [0]
 
     def step():
@@ -381,11 +404,11 @@ def bench_kv_cache(cfg, steps, warmup):
     from nntile_amd import hip_sdpa as h
     kvb = cfg.n_batch * cfg.n_head_kv
     cap, nrot = 2 * cfg.k_seq, 4
-    Ks = [_randn((kvb, cap, cfg.head), torch.bfloat16, cfg.seed * 1000 + 300 + i) for i in range(nrot)]
-    Vs = [_randn((kvb, cap, cfg.head), torch.bfloat16, cfg.seed * 1000 + 350 + i) for i in range(nrot)]
-    k_new = _randn((kvb, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed * 1000 + 398)
-    v_new = _randn((kvb, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed * 1000 + 399)
-    Q = _randn((cfg.batch_flat, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed * 1000 + 99)
+    Ks = [_randn((kvb, cap, cfg.head), torch.bfloat16, cfg.seed, 1 + 10 * i) for i in range(nrot)]
+    Vs = [_randn((kvb, cap, cfg.head), torch.bfloat16, cfg.seed, 2 + 10 * i) for i in range(nrot)]
+    k_new = _randn((kvb, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed, 3)
+    v_new = _randn((kvb, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed, 4)
+    Q = _randn((cfg.batch_flat, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed, 0)
     A = torch.zeros_like(Q)
     lse = torch.full((cfg.batch_flat, cfg.q_seq), float("-inf"), device="cuda")
     ws = torch.empty(h.decode_cache_workspace_bytes(cfg.k_seq, Q, cfg.n_batch, cfg.kv_group),
@@ -461,6 +484,7 @@ def cpu_baseline(cfg, target_seconds=15.0):
     per_slab = dt / (reps * slabs)
     fl = cfg.flops() / cfg.batch_flat
     return {"value": fl / per_slab / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sgemm": "builtin (the checker's own blocked kernel; no CBLAS headers in the image)",
             "sample": "%d of %d (batch,head) slabs of %s x %d passes, all %d queries, key tiles of %d; "
                       "FLOPs counted causal-exact as for the GPU (the CPU path computes the dense "
                       "score matrix)" % (slabs, cfg.batch_flat, cfg.name, reps, cfg.q_seq, cfg.seq_tile),
@@ -474,7 +498,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run only this leg: prefill | decode | decode_wide | per_task | backward | rope | transpose | accumulate | kv_cache | extras | copy (for profiling)")
+                    help="run only this leg (for profiling): prefill | cfg5 | cfg2 | decode | decode_wide | "
+                         "reference_api | reference_grid | backward | rope | transpose | accumulate | "
+                         "kv_cache | copy")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
@@ -484,35 +510,31 @@ def main():
 
     import torch
     from nntile_amd import hip_sdpa as h
-    from nntile_amd.configs import BY_NAME
+    from nntile_amd.configs import BY_NAME, Workload
     h.lib()      # fails loudly if the HIP library is not built
     torch.cuda.set_device(0)
 
     cfg3 = BY_NAME["cfg3_llama_prefill_bf16"]
     cfg4 = BY_NAME["cfg4_gqa_decode_bf16"]
-    out = {}
+    # cfg4's bytes as 64 sequences of 1024 cached keys: 512 (sequence, kv head)
+    # units, one key split each, (lse, A) written by the main kernel
+    cfg4_wide = Workload("cfg4_bytes_as_64_sequences_of_1024_keys", "bf16", 128, 16, 1024, 64, 4, 8,
+                         1024, 1, 45, decode=True)
     only = args.only
-
-    if only == "prefill":
-        bench_prefill(cfg3, args.steps, args.warmup)
-        return
-    if only == "per_task_streams":
-        r = bench_prefill(cfg3, args.steps, args.warmup, per_task=True, streams=4)
-        print(json.dumps({k: round(v, 4) for k, v in r.items()}))
-        return
-    if only == "per_task_classified":
-        r = bench_prefill(cfg3, args.steps, args.warmup, per_task=True, classified=True)
-        print(json.dumps({k: round(v, 4) for k, v in r.items()}))
-        return
-    if only == "per_task":
-        bench_prefill(cfg3, args.steps, args.warmup, per_task=True)
-        return
-    if only == "decode":
-        bench_decode(cfg4, args.steps, args.warmup)
-        return
-    if only == "reference_api":
-        print(json.dumps(bench_reference_api(cfg3, args.steps, args.warmup)))
-        return
+    show = lambda r: print(json.dumps({k: (round(v, 4) if isinstance(v, float) else v)
+                                       for k, v in r.items()}))
+    legs = {"prefill": lambda: bench_prefill(cfg3, args.steps, args.warmup),
+            "cfg5": lambda: bench_prefill(BY_NAME["cfg5_long_seq_bf16"], args.steps, args.warmup),
+            "cfg2": lambda: bench_prefill(BY_NAME["cfg2_gpt2_small_fp32"], args.steps, args.warmup),
+            "decode": lambda: bench_decode(cfg4, args.steps, args.warmup),
+            "decode_wide": lambda: bench_decode(cfg4_wide, args.steps, args.warmup),
+            "reference_api": lambda: bench_reference_api(cfg3, args.steps, args.warmup),
+            "reference_grid": lambda: bench_reference_grid(args.steps, args.warmup),
+            "backward": lambda: bench_backward(cfg3, args.steps, args.warmup),
+            "rope": lambda: bench_rope(cfg3, args.steps, args.warmup),
+            "transpose": lambda: bench_transpose(cfg3, args.steps, args.warmup),
+            "accumulate": lambda: bench_accumulate(cfg3, args.steps, args.warmup),
+            "kv_cache": lambda: bench_kv_cache(cfg4, args.steps, args.warmup)}
     if only == "copy":
         # calibration leg for the HBM traffic counters: a plain device copy
         # of 1 GiB (reads 2^30 bytes, writes 2^30 bytes per launch)
@@ -522,59 +544,35 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         return
-    if only == "backward":
-        print(json.dumps(bench_backward(cfg3, args.steps, args.warmup)))
-        return
-    if only == "transpose":
-        print(json.dumps(bench_transpose(cfg3, args.steps, args.warmup)))
-        return
-    if only == "rope":
-        print(json.dumps(bench_rope(cfg3, args.steps, args.warmup)))
-        return
-    if only == "decode_wide":
-        from nntile_amd.configs import Workload
-        wide = Workload("cfg4_bytes_as_64_sequences_of_1024_keys", "bf16", 128, 16, 1024, 64, 4, 8,
-                        1024, 1, 45, decode=True)
-        r = bench_decode(wide, args.steps, args.warmup)
-        print(json.dumps({k: round(v, 4) for k, v in r.items()}))
-        return
-    if only == "accumulate":
-        print(json.dumps(bench_accumulate(cfg3, args.steps, args.warmup)))
-        return
-    if only == "kv_cache":
-        print(json.dumps(bench_kv_cache(cfg4, args.steps, args.warmup)))
-        return
-    if only == "extras":
-        for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):
-            bench_prefill(BY_NAME[name], args.steps, args.warmup)
+    if only is not None:
+        if only not in legs:
+            sys.stderr.write("bench.py: unknown leg %r\n" % only)
+            sys.exit(2)
+        show(legs[only]())
         return
 
+    few = max(5, args.steps // 5)
     dec = bench_decode(cfg4, args.steps, args.warmup)
-    # the same bytes as 64 sequences of 1024 cached keys: 512 (sequence, kv
-    # head) units, one key split each, (lse, A) written by the main kernel
-    from nntile_amd.configs import Workload
-    cfg4_wide = Workload("cfg4_bytes_as_64_sequences_of_1024_keys", "bf16", 128, 16, 1024, 64, 4, 8,
-                         1024, 1, 45, decode=True)
-    dec_wide = bench_decode(cfg4_wide, max(5, args.steps // 5), 5)
-    per_task = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True)
-    per_task_cls = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True, classified=True)
-    per_task4 = bench_prefill(cfg3, max(5, args.steps // 5), 2, per_task=True, streams=4)
+    dec_wide = bench_decode(cfg4_wide, few, 5)
+    ref_api = bench_reference_api(cfg3, few, 5)
+    ref_grid = bench_reference_grid(max(5, args.steps // 25), 3)
     extras = {}
     for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):
         c = BY_NAME[name]
-        r = bench_prefill(c, max(5, args.steps // 5), 2)
-        peak = PEAK_FP32_TFLOPS if c.dtype == "fp32" else PEAK_BF16_TFLOPS
-        extras[name] = {"ms_per_step": round(r["ms_per_step"], 4),
-                        "tflops": round(r["tflops"], 2),
-                        "kernel_tflops": round(r["kernel_tflops"], 2),
-                        "frac_of_peak": round(r["kernel_tflops"] / peak, 4),
-                        "peak_tflops": peak, "flops_causal_exact": c.flops(),
-                        "launches_per_step": r["launches_per_step"]}
-    backward = bench_backward(cfg3, max(5, args.steps // 10), 2)
-    rope = bench_rope(cfg3, max(5, args.steps // 5), 5)
-    transpose = bench_transpose(cfg3, max(5, args.steps // 5), 5)
-    kv_cache = bench_kv_cache(cfg4, max(5, args.steps // 5), 5)
-    accumulate = bench_accumulate(cfg3, max(5, args.steps // 5), 5)
+        r = bench_prefill(c, few, 3)
+        fp32 = c.dtype == "fp32"
+        extras[name] = {
+            "ms_per_step": round(r["ms_per_step"], 4), "tflops": round(r["tflops"], 2),
+            "flops_causal_exact": c.flops(), "launches_per_step": r["launches_per_step"],
+            "roofline": roofline("mfma", "sdpa_prefill_fp32_kernel<%d,causal>" % c.head if fp32
+                                 else "sdpa_prefill_16bit_kernel<bf16,%d,causal>" % c.head,
+                                 c.flops(), r["device_ms_per_step"],
+                                 PEAK_FP32_TFLOPS if fp32 else PEAK_BF16_TFLOPS, "TFLOP/s")}
+    backward = bench_backward(cfg3, max(5, args.steps // 10), 3)
+    rope = bench_rope(cfg3, few, 5)
+    transpose = bench_transpose(cfg3, few, 5)
+    kv_cache = bench_kv_cache(cfg4, few, 5)
+    accumulate = bench_accumulate(cfg3, few, 5)
     # The headline leg runs last: the first timed loop of a process measures
     # 5 % slower than the same loop a second later (clocks still settling),
     # whatever the warmup count.
@@ -592,51 +590,52 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic: i.i.d. N(0,1) rounded to bf16, torch generator seeded per tile",
+        "data": DATA,
         "config": {"workload": cfg3.name, "head_size": cfg3.head, "n_head": cfg3.n_head_kv,
                    "seq_len": cfg3.q_seq, "batch": cfg3.n_batch, "seq_tile": cfg3.seq_tile,
                    "mask": "causal", "flops_per_step_causal_exact": cfg3.flops(),
                    "flops_per_step_dense": cfg3.flops(False),
                    "launches_per_step": main_leg["launches_per_step"],
-                   "timed": "one fused launch over the 4x4 tile grid in overwrite mode (6 fully "
-                            "hidden tile pairs skipped, no lse fill needed)"},
-        "roofline": {"bound": "mfma", "kernel": "sdpa_prefill_16bit_kernel<bf16,128,causal>",
-                     "achieved": round(main_leg["kernel_tflops"], 2), "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(main_leg["kernel_tflops"] / PEAK_BF16_TFLOPS, 4),
-                     "traffic": TRAFFIC_PREFILL_CFG3,
-                     "kernel_ms": round(main_leg["kernel_ms_per_step"], 4)},
+                   "timed": "one fused launch over the 4x4 grid of separately allocated tiles, "
+                            "analytic causal mask (6 fully hidden tile pairs skipped), overwrite mode: "
+                            "the launch defines (lse, A), which replaces the caller's fills of lse "
+                            "with -inf and of A with 0 (layer/sdpa.py:538-539); value = causal-exact "
+                            "FLOPs / wall time per step; roofline.kernel_ms = HIP-event time per "
+                            "step of the same loop"},
+        "roofline": roofline("mfma", "sdpa_prefill_16bit_kernel<bf16,128,causal>", cfg3.flops(),
+                             main_leg["device_ms_per_step"], PEAK_BF16_TFLOPS, "TFLOP/s",
+                             TRAFFIC[cfg3.name]),
         "decode": {"workload": cfg4.name, "ms_per_step": round(dec["ms_per_step"], 4),
                    "value": round(dec["gbs"], 1), "unit": "GB/s",
                    "tflops": round(dec["tflops"], 2),
-                   "roofline": {"bound": "hbm", "kernel": "sdpa_decode_16bit_kernel + reduce",
-                                "achieved": round(dec["kernel_gbs"], 1), "peak": PEAK_HBM_GBS,
-                                "unit": "GB/s", "frac": round(dec["kernel_gbs"] / PEAK_HBM_GBS, 4),
-                                "traffic": TRAFFIC_DECODE_CFG4,
-                                "algorithmic_bytes": dec["algorithmic_bytes"],
-                                "workspace_bytes": dec["workspace_bytes"],
-                                "kernel_ms": round(dec["kernel_ms_per_step"], 4)}},
-        "decode_many_sequences": {"workload": cfg4_wide.name,
-                                  "what": "for information: cfg4's bytes as 64 sequences x 8 kv heads x "
-                                          "1024 keys, 16 new tokens each; one key split per unit, no "
-                                          "merge launch",
-                                  "kernel_ms": round(dec_wide["kernel_ms_per_step"], 4),
-                                  "algorithmic_bytes": dec_wide["algorithmic_bytes"],
-                                  "gbs": round(dec_wide["kernel_gbs"], 1),
-                                  "frac_of_hbm_peak": round(dec_wide["kernel_gbs"] / PEAK_HBM_GBS, 4)},
-        "per_task_path": {"what": "cfg3 as the reference submits it: 16 launches, additive mask "
-                                  "tiles, no skipping, (lse, A) handed over in bf16",
-                          "ms_per_step": round(per_task["ms_per_step"], 4),
-                          "tflops": round(per_task["tflops"], 2),
-                          "on_4_streams": {"what": "the tasks of query tile i on stream i % 4",
-                                           "ms_per_step": round(per_task4["ms_per_step"], 4),
-                                           "tflops": round(per_task4["tflops"], 2)}},
-        "per_task_classified": {"what": "the same tensors and materialised mask with the mask tiles "
-                                        "classified once: the classes say the mask is the causal "
-                                        "rule itself, so one launch merges all key tiles into all "
-                                        "query tiles (lse filled with -inf first, as for the tasks)",
-                                "launches_per_step": per_task_cls["launches_per_step"],
-                                "ms_per_step": round(per_task_cls["ms_per_step"], 4),
-                                "tflops": round(per_task_cls["tflops"], 2)},
+                   "roofline": roofline("hbm", "sdpa_decode_16bit_kernel + sdpa_decode_reduce_kernel",
+                                        dec["algorithmic_bytes"], dec["device_ms_per_step"],
+                                        PEAK_HBM_GBS, "GB/s", TRAFFIC[cfg4.name],
+                                        {"algorithmic_bytes": dec["algorithmic_bytes"],
+                                         "workspace_bytes": dec["workspace_bytes"]})},
+        "decode_many_sequences": {
+            "workload": cfg4_wide.name,
+            "what": "for information: cfg4's bytes as 64 sequences x 8 kv heads x 1024 keys, 16 new "
+                    "tokens each; one key split per unit, no merge launch",
+            "roofline": roofline("hbm", "sdpa_decode_16bit_kernel (single split)",
+                                 dec_wide["algorithmic_bytes"], dec_wide["device_ms_per_step"],
+                                 PEAK_HBM_GBS, "GB/s")},
+        "per_task_path": {
+            "what": "cfg3 as an unchanged caller runs it, through the C++ mirror of the reference's "
+                    "tensor layer: tiled tensors, a materialised additive causal mask, per pass the "
+                    "-inf fill of logsumexp and tensor::flash_sdpa_fwd_cudnn_async(K, Q, mask, "
+                    "logsumexp, V, A) with the reference's six arguments.  The mask's tiles are "
+                    "classified the first time the mask is seen and the classes kept with its "
+                    "handles: the causal rule -> one launch in merge mode",
+            "ms_per_step": ref_api["default_overload"]["ms_per_step"],
+            "tflops": ref_api["default_overload"]["tflops"],
+            "launches_per_step": ref_api["default_overload"]["launches_per_step"],
+            "mask_classifications": ref_api["default_overload"]["mask_classifications"],
+            "every_pair": dict(ref_api["every_pair"],
+                               what="the reference's submission literally "
+                                    "(tensor::flash_sdpa_fwd_cudnn_pairs_async): 16 tile tasks with "
+                                    "their additive mask tiles, (lse, A) handed over in bf16")},
+        "reference_bench_grid": ref_grid,
         "other_configs": extras,
         "backward": backward,
         "rope": rope,

@@ -39,6 +39,44 @@ def randn(seed, stream, n, offset=0, chunk=1 << 22):
     return out
 
 
+def _signed(u):
+    """A 64-bit pattern as the int64 with the same bits."""
+    u = int(u)
+    return u - (1 << 64) if u >= (1 << 63) else u
+
+
+def randn_torch(seed, stream, n, device="cuda", offset=0, chunk=1 << 24):
+    """`randn` evaluated with torch on `device` (int64 arithmetic wraps like
+    uint64; the logical right shifts are masked arithmetic ones): the same
+    stream of values, produced where they are needed.  The uniform variates
+    are bit-identical to the numpy version's; log, sqrt and cos are the
+    device's, so a value may differ from numpy's in its last bit."""
+    import torch
+    key = _signed(_splitmix64(np.uint64(seed) * np.uint64(0x100000001B3) + np.uint64(stream)))
+    golden, m1, m2 = _signed(_GOLDEN), _signed(_M1), _signed(_M2)
+
+    def lsr(z, k):
+        return (z >> k) & ((1 << (64 - k)) - 1)
+
+    def mix(x):
+        z = x + golden
+        z = (z ^ lsr(z, 30)) * m1
+        z = (z ^ lsr(z, 27)) * m2
+        return z ^ lsr(z, 31)
+
+    out = torch.empty(n, dtype=torch.float32, device=device)
+    for start in range(0, n, chunk):
+        m = min(chunk, n - start)
+        ctr = torch.arange(offset + start, offset + start + m, dtype=torch.int64, device=device)
+        a = mix((ctr * 2) ^ key)
+        b = mix((ctr * 2 + 1) ^ key)
+        u1 = (lsr(a, 11).to(torch.float64) + 1.0) * (2.0 ** -53)
+        u2 = lsr(b, 11).to(torch.float64) * (2.0 ** -53)
+        out[start:start + m] = (torch.sqrt(-2.0 * torch.log(u1))
+                                * torch.cos(2.0 * np.pi * u2)).to(torch.float32)
+    return out
+
+
 def permutation(seed, stream, n):
     """A seeded permutation of range(n) (argsort of a hashed counter)."""
     with np.errstate(over="ignore"):
