@@ -1,22 +1,34 @@
 // Prefill attention forward for fp32 tiles on gfx950.
 //
-// Same decomposition as the 16-bit kernel (one workgroup = 4 wavefronts = 128
-// queries, S^T = K Q^T and O^T += V^T P^T with a lane owning one query), but
-// on v_mfma_f32_32x32x2_f32: operands and products are true fp32, which the
-// 1e-4 tolerance of the fp32 configurations needs.  Keys are walked in steps
-// of 32.  With a 2-deep contraction per MFMA the lane half h supplies the
-// operand element k = h, so:
+// Same decomposition as the 16-bit kernel (S^T = K Q^T and O^T += V^T P^T with
+// a lane owning one query), but on v_mfma_f32_32x32x2_f32: operands and
+// products are true fp32, which the 1e-4 tolerance of the fp32 configurations
+// needs.  Keys are walked in steps of 32.  With a 2-deep contraction per MFMA
+// the lane half h supplies the operand element k = h, so:
 //   S^T: 4 consecutive MFMAs consume one 16-byte read K[key][8j+4h .. +3]
 //        against the matching 4 query values held in registers;
 //   O^T: the B operand is the S^T accumulator register itself (key
 //        8*(r/4) + 4h + r%4), the A operand is V[that key][d] read from LDS
 //        with the head axis across lanes - no transposition is needed.
+// K and V steps go from global memory straight into LDS (global_load_lds, 16
+// bytes per lane, 1 KB per instruction, no registers in between); rows are
+// unpadded and their 16-byte chunks XOR-swizzled by row against bank
+// conflicts, as in the 16-bit kernel.
 //
-// SPLIT variant, for launches with fewer workgroups than CUs: a workgroup is
-// 32 queries, and its four wavefronts take every fourth key step each (four
-// steps are staged per iteration), then merge their (max, sum, O) through LDS.
-// The chain of dependent steps a wavefront walks, which bounds such a launch,
-// is a quarter as long, and four times as many workgroups spread over the CUs.
+// Two forms:
+//   * 128 queries per workgroup, four wavefronts of 32 queries sharing every
+//     key step: two LDS buffers per operand, the loads of step g+1 issued at
+//     the top of step g, one barrier per step;
+//   * SPLIT, for launches with fewer such workgroups than CUs: a workgroup is
+//     32 queries and its four wavefronts take every fourth key step each, each
+//     through its own LDS buffer - K of the next step is requested when the
+//     scores of this one are done, V when its output products are, and there
+//     is no barrier in the loop; at the end the four merge their (max, sum, O)
+//     through LDS.  The chain of dependent steps a wavefront walks, which
+//     bounds such a launch, is a quarter as long, and four times as many
+//     workgroups spread over the CUs.
+#include <type_traits>
+
 #include "sdpa_common.hpp"
 
 namespace nntile_hip
@@ -28,33 +40,45 @@ namespace nntile_hip
 #endif
 constexpr int kQRows32 = 128;
 constexpr int kKeys32 = 32;
-constexpr int kThreads32 = 256;          // first form: 4 wavefronts
-#ifndef NNTILE_F32_SPLIT_WAVES
-#define NNTILE_F32_SPLIT_WAVES 4
-#endif
-// second form: wavefronts sharing the keys.  Head 64 stages 8 steps (139 KiB
-// of LDS); head 128 has room for 4, head 32 has 256 16-byte chunks a step.
-__host__ __device__ constexpr int split_waves32(int head)
+constexpr int kThreads32 = 256;          // 4 wavefronts in both forms
+
+template<int N> __device__ __forceinline__ void f32_wait_vmcnt()
 {
-    return head == 64 ? NNTILE_F32_SPLIT_WAVES : 4;
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    // s_waitcnt simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14]
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+    asm volatile("" ::: "memory");
 }
 
 template<int HEAD, int MODE, bool SPLIT>
-__global__ __launch_bounds__(SPLIT ? split_waves32(HEAD) * 64 : kThreads32, SPLIT ? 1 : 2)
+__global__ __launch_bounds__(kThreads32, (SPLIT && HEAD == 128) ? 1 : 2)
 void sdpa_prefill_fp32_kernel(const PrefillParams p)
 {
     constexpr int QROWS = SPLIT ? 32 : kQRows32;    // queries per workgroup
-    constexpr int THREADS = SPLIT ? split_waves32(HEAD) * 64 : kThreads32;
-    constexpr int NSUB = SPLIT ? split_waves32(HEAD) : 1;   // key steps staged per iteration
+    constexpr int NSUB = SPLIT ? 4 : 1;     // key steps in flight side by side (one per wavefront)
     constexpr int QSTEPS = HEAD / 8;        // 16-byte groups per lane half along head
     constexpr int DBLOCKS = HEAD / 32;
-    constexpr int PAD = HEAD + 4;           // row stride in LDS (floats)
-    constexpr int CHUNKS = HEAD / 4;        // 16-byte chunks per row
+    constexpr int RB = HEAD * 4;            // bytes per K/V row
+    constexpr int CPR = HEAD / 4;           // 16-byte chunks per row
+    constexpr int RPL = CPR >= 16 ? 1 : 16 / CPR;   // rows per 256-byte line of LDS banks
+    constexpr int KSW = CPR >= 16 ? 16 : CPR;       // K: chunk c of row r at c ^ ((r / RPL) % KSW)
+    constexpr int ROWS_PER_LOAD = 1024 / RB;        // rows one load instruction fills
+    constexpr int LOADS = kKeys32 / ROWS_PER_LOAD;  // load instructions per K (or V) step
+    constexpr int LPW = SPLIT ? LOADS : LOADS / 4;  // ... of them issued by one wavefront
+    constexpr int BLOCK_BYTES = kKeys32 * RB;
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
+    static_assert(LPW >= 1, "head size does not fit this tiling");
 
-    __shared__ __attribute__((aligned(16))) float Ks[NSUB * kKeys32 * PAD];
-    __shared__ __attribute__((aligned(16))) float Vs[NSUB * kKeys32 * PAD];
+    // SPLIT: lds_k0 / lds_v0 hold one step per wavefront (wavefront w owns
+    // bytes [w * BLOCK_BYTES, +BLOCK_BYTES)); lds_k1 / lds_v1 are not used.
+    // Otherwise step g of the workgroup lives in lds_k[g % 2], lds_v[g % 2].
+    // (Separate arrays: the compiler then knows that what streams into one
+    // cannot alias the reads of another.)
+    __shared__ __attribute__((aligned(1024))) char lds_k0[NSUB * BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_v0[NSUB * BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_k1[SPLIT ? 16 : BLOCK_BYTES];
+    __shared__ __attribute__((aligned(1024))) char lds_v1[SPLIT ? 16 : BLOCK_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -64,13 +88,36 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
 
     const int q_blocks = p.n_q_tiles * p.q_blocks_per_tile;
     int wg = blockIdx.x;
-    if(p.xcd_remap)
+    int b, qblk;
+    if(SPLIT)
     {
-        const int per_xcd = gridDim.x >> 3;
-        wg = (wg & 7) * per_xcd + (wg >> 3);
+        // A launch of this form fits the GPU at once, so where a workgroup
+        // lands decides how evenly the CUs are loaded.  Workgroups are dealt
+        // round-robin to the 8 XCDs; each XCD puts its first 32 on its 32 CUs
+        // and the next ones beside them, i + 32 next to i.  Query blocks go out
+        // longest first (all batch entries of a block before the next block),
+        // and the workgroups beyond the first 32 of an XCD in reverse: the CU
+        // with the longest workgroup gets the shortest as its second.
+        const int per_xcd = (int)((gridDim.x + 7u - (unsigned)(wg & 7)) >> 3);
+        int i = wg >> 3;
+        if(i >= 32 && per_xcd <= 64)
+        {
+            i = 32 + (per_xcd - 1 - i);
+        }
+        const int k = (i << 3) | (wg & 7);
+        b = k % p.batch;
+        qblk = q_blocks - 1 - k / p.batch;
     }
-    const int b = wg / q_blocks;
-    const int qblk = q_blocks - 1 - (wg % q_blocks);
+    else
+    {
+        if(p.xcd_remap)
+        {
+            const int per_xcd = gridDim.x >> 3;
+            wg = (wg & 7) * per_xcd + (wg >> 3);
+        }
+        b = wg / q_blocks;
+        qblk = q_blocks - 1 - (wg % q_blocks);
+    }
     const int qt = qblk / p.q_blocks_per_tile;
     const int qb = qblk % p.q_blocks_per_tile;
     const int64_t q_len = min(p.q_tile, p.q_seq - (int64_t)qt * p.q_tile);
@@ -108,101 +155,101 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         + (SPLIT ? 0 : wave * 32);
     const int64_t wave_qpos_hi = wave_qpos_lo + 31;
 
-    // Cooperative loads: 32 rows x CHUNKS chunks for K and for V.
-    constexpr int ROWS_PER_PASS = THREADS / CHUNKS;
-    static_assert(THREADS <= kKeys32 * CHUNKS, "more threads than 16-byte chunks of a step");
-    constexpr int PASSES = kKeys32 / ROWS_PER_PASS;
-    const int ld_chunk = tid % CHUNKS;
-    const int ld_row = tid / CHUNKS;
-    f32x4 k_regs[NSUB][PASSES], v_regs[NSUB][PASSES];
+    // ---- LDS layout and the lane's fixed addresses ---------------------------
+    // A step's K (and V) block is 32 rows of RB bytes, unpadded.  The 16-byte
+    // chunk c of row r is stored at chunk position
+    //   K:  c ^ ((r / RPL) % KSW)      consecutive rows, same c -> different bank groups
+    //   V:  c ^ (8 * ((r / 4) % 2))    (rows of 256 bytes and more) the two lane
+    //                                  halves read rows 4 apart: different halves of the banks
+    // Load instruction `ld` fills rows [ld*ROWS_PER_LOAD, +ROWS_PER_LOAD): lane L
+    // lands on row ld*ROWS_PER_LOAD + L/CPR, chunk position L % CPR, and fetches
+    // the chunk that belongs there.
+    constexpr int VSW = CPR >= 16 ? 8 : 0;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    uint32_t k_goff[LPW], v_goff[LPW];
+    int ld_row[LPW];
+    const int ld_cpos = lane % CPR;
+#pragma unroll
+    for(int i = 0; i < LPW; ++i)
+    {
+        const int ld = SPLIT ? i : wave * LPW + i;
+        const int r = ld * ROWS_PER_LOAD + lane / CPR;
+        ld_row[i] = r;
+        k_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ ((r / RPL) % KSW)) * 16);
+        v_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ (VSW * ((r >> 2) & 1))) * 16);
+    }
+    // S operand: lane (col, half) reads row col, logical chunk 2*j + half.
+    uint32_t k_raddr[QSTEPS];
+#pragma unroll
+    for(int j = 0; j < QSTEPS; ++j)
+    {
+        k_raddr[j] = (uint32_t)(col * RB + ((2 * j + half) ^ ((col / RPL) % KSW)) * 16);
+    }
+    // PV operand: register r of the scores is key 8*(r/4) + 4*half + r%4, whose
+    // swizzle only depends on the lane half; lane (col, half) reads head value
+    // 32*db + col of that row.  8*(r/4) + r%4 goes into the immediate offset.
+    uint32_t v_raddr[DBLOCKS];
+#pragma unroll
+    for(int db = 0; db < DBLOCKS; ++db)
+    {
+        v_raddr[db] = (uint32_t)(4 * half * RB
+                + (((db * 8 + col / 4) ^ (VSW * half)) * 4 + col % 4) * 4);
+    }
 
-    // Where the rows of a key step come from.  One key tile (every tile-pair
-    // call): the tile's addresses are computed once, a step needs no division
-    // and no look-up in the tile table.
+    // Where the rows of a key step come from.
     struct StepSource
     {
-        const float *K, *V;
-        int row0, last_row;
+        const char *K, *V;      // first row of the step
+        int rows_left;          // rows of the tile from this step on
     };
     const int64_t k_len0 = min(p.k_tile, p.k_seq);
     const bool one_tile = p.n_kv_tiles == 1;
     const int64_t entry_rows0 = p.kv_rows > 0 ? p.kv_rows : k_len0;
-    const float *K0 = static_cast<const float *>(p.K[0]) + ((int64_t)kvb * entry_rows0) * HEAD;
-    const float *V0 = static_cast<const float *>(p.V[0]) + ((int64_t)kvb * entry_rows0) * HEAD;
-    auto locate = [&](int g, int n_steps_all) -> StepSource
+    const char *K0 = static_cast<const char *>(p.K[0]) + ((int64_t)kvb * entry_rows0) * RB;
+    const char *V0 = static_cast<const char *>(p.V[0]) + ((int64_t)kvb * entry_rows0) * RB;
+    auto locate = [&](int g) -> StepSource
     {
-        // steps past the last re-read the last one (nobody uses them)
-        g = min(g, max(n_steps_all - 1, 0));
         StepSource src;
         if(one_tile)
         {
-            src.K = K0;
-            src.V = V0;
-            src.row0 = g * kKeys32;
-            src.last_row = (int)k_len0 - 1;
+            src.K = K0 + (int64_t)g * kKeys32 * RB;
+            src.V = V0 + (int64_t)g * kKeys32 * RB;
+            src.rows_left = (int)k_len0 - g * kKeys32;
         }
         else
         {
             const int kt = g / p.k_blocks_per_tile;
             const int kb = g % p.k_blocks_per_tile;
             const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
-            src.K = static_cast<const float *>(p.K[kt]) + ((int64_t)kvb * k_len) * HEAD;
-            src.V = static_cast<const float *>(p.V[kt]) + ((int64_t)kvb * k_len) * HEAD;
-            src.row0 = kb * kKeys32;
-            src.last_row = (int)k_len - 1;
+            const int64_t off = ((int64_t)kvb * k_len + (int64_t)kb * kKeys32) * RB;
+            src.K = static_cast<const char *>(p.K[kt]) + off;
+            src.V = static_cast<const char *>(p.V[kt]) + off;
+            src.rows_left = (int)k_len - kb * kKeys32;
         }
         return src;
     };
-    // The loads of the staged steps, one 16-byte load per thread and piece:
-    // piece k is step k / (2 PASSES), pass (k / 2) % PASSES, K for even k and V
-    // for odd k.  Rows past the end of the tile re-read its last row: their
-    // keys are masked out of the scores, so their probabilities are exactly
-    // 0, and a load that is never conditional does not make the wave wait.
-    // (the launcher keeps a tile's rows x HEAD within 31 bits)
-    constexpr int PIECES = NSUB * PASSES * 2;
-    StepSource src[NSUB];
-    auto fetch_piece = [&](int k) __attribute__((always_inline))
+    // Global -> LDS loads of this wavefront's share of the K (or V) rows of a
+    // step.  Rows past the end of the tile are clamped to its last row: their
+    // keys are masked out of the scores, so their probabilities are exactly 0.
+    auto fetch = [&](const char *src, int rows_left, const uint32_t (&goff)[LPW], char *dst_base)
     {
-        const int sub = k / (2 * PASSES), i = (k / 2) % PASSES;
-        const uint32_t off = (uint32_t)min(src[sub].row0 + ld_row + i * ROWS_PER_PASS,
-                src[sub].last_row) * HEAD + ld_chunk * 4;
-        if(k % 2 == 0)
+        char *dst = dst_base + wave_u * (SPLIT ? BLOCK_BYTES : LPW * 1024);
+        if(rows_left >= kKeys32)
         {
-            k_regs[sub][i] = *reinterpret_cast<const f32x4 *>(src[sub].K + off);
+#pragma unroll
+            for(int i = 0; i < LPW; ++i)
+            {
+                load_to_lds16<0, false>(src, goff[i], dst + i * 1024);
+            }
         }
         else
         {
-            v_regs[sub][i] = *reinterpret_cast<const f32x4 *>(src[sub].V + off);
-        }
-    };
-    // A wave gets one load accepted every ~70 cycles and stands still until
-    // then; inside the loop the pieces therefore go between the MFMAs, which
-    // run meanwhile: slot t of SLOTS takes the pieces k with k*SLOTS/PIECES == t.
-    constexpr int SLOTS = QSTEPS + 16;
-    auto fetch_slot = [&](int t) __attribute__((always_inline))
-    {
+            const int last = rows_left - 1;
 #pragma unroll
-        for(int k = 0; k < PIECES; ++k)
-        {
-            if(k * SLOTS / PIECES == t)
+            for(int i = 0; i < LPW; ++i)
             {
-                fetch_piece(k);
-            }
-        }
-    };
-
-    auto stage = [&]()
-    {
-#pragma unroll
-        for(int sub = 0; sub < NSUB; ++sub)
-        {
-#pragma unroll
-            for(int i = 0; i < PASSES; ++i)
-            {
-                const int off = (sub * kKeys32 + ld_row + i * ROWS_PER_PASS) * PAD
-                    + ld_chunk * 4;
-                *reinterpret_cast<f32x4 *>(&Ks[off]) = k_regs[sub][i];
-                *reinterpret_cast<f32x4 *>(&Vs[off]) = v_regs[sub][i];
+                const uint32_t back = (uint32_t)(max(ld_row[i] - last, 0) * RB);
+                load_to_lds16<0, false>(src, goff[i] - back, dst + i * 1024);
             }
         }
     };
@@ -243,103 +290,70 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     float m_run = neg_inf();
     float l_run = 0.0f;
 
-    const int n_iter = (n_steps + NSUB - 1) / NSUB;
-    // this wavefront's part of the staged keys
-    const float *Kw = Ks + (SPLIT ? wave * kKeys32 * PAD : 0);
-    const float *Vw = Vs + (SPLIT ? wave * kKeys32 * PAD : 0);
-    if(n_iter > 0)
+    // Scores of key step g from the K block at Kw: S^T = K Q^T, mask.
+    // `between(t)` is called after the first MFMA of group t (QSTEPS groups):
+    // the place where a load instruction costs nothing, the matrix unit being
+    // busy with the group anyway.
+    auto scores = [&](int g, const char *Kw, f32x16 &s, auto between) __attribute__((always_inline))
     {
-#pragma unroll
-        for(int sub = 0; sub < NSUB; ++sub)
-        {
-            src[sub] = locate(sub, n_steps);
-        }
-#pragma unroll
-        for(int k = 0; k < PIECES; ++k)
-        {
-            fetch_piece(k);
-        }
-    }
-    for(int G = 0; G < n_iter; ++G)
-    {
-        __syncthreads();
-        stage();
-        __syncthreads();
-        // the next iteration's steps: located now, loaded between the MFMAs
-#pragma unroll
-        for(int sub = 0; sub < NSUB; ++sub)
-        {
-            src[sub] = locate((G + 1) * NSUB + sub, n_steps);
-        }
-        const int g = SPLIT ? G * NSUB + wave : G;      // this wavefront's step
-        if(g >= n_steps)
-        {
-#pragma unroll
-            for(int k = 0; k < PIECES; ++k)
-            {
-                fetch_piece(k);
-            }
-            continue;
-        }
-
         const int kt = g / p.k_blocks_per_tile;
         const int kb = g % p.k_blocks_per_tile;
         const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
         const int64_t k_row0 = (int64_t)kb * kKeys32;
         const int64_t k_pos_base = p.k_pos0 + (int64_t)kt * p.k_tile + k_row0;
         const int keys_here = (int)min((int64_t)kKeys32, k_len - k_row0);
-
-        if(MODE == NNTILE_HIP_MASK_CAUSAL
-                && k_pos_base > wave_qpos_hi + p.causal_offset)
-        {
-            // (nothing visible for this wavefront; its share of the loads remains)
-#pragma unroll
-            for(int k = 0; k < PIECES; ++k)
-            {
-                fetch_piece(k);
-            }
-            continue;
-        }
-
-        // ---- S^T = K Q^T ---------------------------------------------------
-        f32x16 s;
+        // Two accumulators take the MFMAs in turn: each of them would
+        // otherwise wait for the one before it (64 cycles in the pipe, 84 from
+        // issue to issue when dependent).
+        f32x16 s2;
 #pragma unroll
         for(int r = 0; r < 16; ++r)
         {
             s[r] = 0.0f;
+            s2[r] = 0.0f;
         }
-        // (the K operands of the step are read ahead of the chain of
-        // dependent MFMAs: a read issued behind four of them would only start
-        // once they have all been issued, i.e. when the last one runs)
+        // (the K operands of the step are read ahead of the chain of MFMAs: a
+        // read issued behind four of them would only start once they have all
+        // been issued)
         {
             constexpr int AHEAD = NNTILE_F32_AHEAD < QSTEPS ? NNTILE_F32_AHEAD : QSTEPS;
             f32x4 ka[QSTEPS];
 #pragma unroll
             for(int j = 0; j < AHEAD; ++j)
             {
-                ka[j] = *reinterpret_cast<const f32x4 *>(&Kw[col * PAD + j * 8 + half * 4]);
+                ka[j] = *reinterpret_cast<const f32x4 *>(Kw + k_raddr[j]);
             }
 #pragma unroll
             for(int j = 0; j < QSTEPS; ++j)
             {
                 if(j + AHEAD < QSTEPS)
                 {
-                    ka[j + AHEAD] = *reinterpret_cast<const f32x4 *>(
-                            &Kw[col * PAD + (j + AHEAD) * 8 + half * 4]);
+                    ka[j + AHEAD] = *reinterpret_cast<const f32x4 *>(Kw + k_raddr[j + AHEAD]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for(int e = 0; e < 4; ++e)
                 {
-                    s = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[j][e], qf[j][e], s,
-                            0, 0, 0);
+                    if(e & 1)
+                    {
+                        s2 = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[j][e], qf[j][e], s2, 0, 0, 0);
+                    }
+                    else
+                    {
+                        s = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[j][e], qf[j][e], s, 0, 0, 0);
+                    }
                     if(e == 0)
                     {
-                        fetch_slot(j);
+                        between(j);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
             }
+        }
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+        {
+            s[r] += s2[r];
         }
 
         // ---- mask: register r holds key 8*(r/4) + 4*half + r%4 ---------------
@@ -397,20 +411,38 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
                 }
             }
         }
+    };
 
-        // ---- online softmax ---------------------------------------------------
+    // Online softmax of the scores (they become the probabilities) and the
+    // rescale of what has been accumulated.
+    auto softmax = [&](f32x16 &s) __attribute__((always_inline))
+    {
         float mx = neg_inf();
 #pragma unroll
         for(int r = 0; r < 16; ++r)
         {
             mx = fmaxf(mx, s[r]);
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        mx = max_across_halves(mx);
         const float m_new = fmaxf(m_run, mx);
         const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
-        const float alpha = fast_exp2((m_run - m_use) * c);
         const float mc = m_use * c;
-        m_run = m_new;
+        // the running maximum rarely moves after the first steps
+        if(__builtin_amdgcn_ballot_w64(m_new != m_run) != 0)
+        {
+            const float alpha = fast_exp2((m_run - m_use) * c);
+            l_run *= alpha;
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+#pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    o[db][r] *= alpha;
+                }
+            }
+            m_run = m_new;
+        }
         float rs = 0.0f;
 #pragma unroll
         for(int r = 0; r < 16; ++r)
@@ -418,60 +450,214 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
             s[r] = fast_exp2(fmaf(s[r], c, -mc));
             rs += s[r];
         }
-        l_run = l_run * alpha + rs;
-#pragma unroll
-        for(int db = 0; db < DBLOCKS; ++db)
+        l_run += rs;
+    };
+
+    // O^T += V^T P^T from the V block at Vw (V operands four keys at a time,
+    // one group ahead of its MFMAs).
+    // `between(t)` is called after the first MFMA of key t (16 keys).
+    auto output = [&](const char *Vw, const f32x16 &s, auto between) __attribute__((always_inline))
+    {
+        float va[16][DBLOCKS];
+        auto read_group = [&](int g4)
         {
 #pragma unroll
-            for(int r = 0; r < 16; ++r)
+            for(int x = 0; x < 4; ++x)
             {
-                o[db][r] *= alpha;
+                const int r = 4 * g4 + x;
+#pragma unroll
+                for(int db = 0; db < DBLOCKS; ++db)
+                {
+                    va[r][db] = *reinterpret_cast<const float *>(
+                            Vw + v_raddr[db] + (8 * (r >> 2) + (r & 3)) * RB);
+                }
+            }
+        };
+        read_group(0);
+#pragma unroll
+        for(int g4 = 0; g4 < 4; ++g4)
+        {
+            if(g4 + 1 < 4)
+            {
+                read_group(g4 + 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for(int x = 0; x < 4; ++x)
+            {
+                const int r = 4 * g4 + x;
+#pragma unroll
+                for(int db = 0; db < DBLOCKS; ++db)
+                {
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[r][db], s[r], o[db],
+                            0, 0, 0);
+                    if(db == 0)
+                    {
+                        between(r);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
             }
         }
+    };
+    auto nothing = [](int) {};
+    // one load instruction of a step's K (or V) share: piece i of LPW
+    auto fetch_piece = [&](const char *src, int rows_left, const uint32_t (&goff)[LPW],
+            char *dst_base, int i) __attribute__((always_inline))
+    {
+        char *dst = dst_base + wave_u * (SPLIT ? BLOCK_BYTES : LPW * 1024);
+        const int last = rows_left - 1;
+        const uint32_t back = (uint32_t)(max(ld_row[i] - last, 0) * RB);
+        load_to_lds16<0, false>(src, goff[i] - back, dst + i * 1024);
+    };
 
-        // ---- O^T += V^T P^T ----------------------------------------------------
-        // (V operands four keys at a time, one group ahead of its MFMAs)
+    // nothing of key step g is visible to this wavefront
+    auto hidden = [&](int g) -> bool
+    {
+        if(MODE != NNTILE_HIP_MASK_CAUSAL)
         {
-            float va[16][DBLOCKS];
-            auto read_group = [&](int g4)
+            return false;
+        }
+        const int kt = g / p.k_blocks_per_tile;
+        const int kb = g % p.k_blocks_per_tile;
+        const int64_t k_pos_base = p.k_pos0 + (int64_t)kt * p.k_tile + (int64_t)kb * kKeys32;
+        return k_pos_base > wave_qpos_hi + p.causal_offset;
+    };
+
+    if constexpr(SPLIT)
+    {
+        // ---- every wavefront walks its own key steps wave, wave + 4, ... ---------
+        // through its own K and V buffer.  Loads complete in the order they
+        // were issued: K(i) V(i) K(i+1) V(i+1) ...
+        char *Kw = lds_k0 + wave_u * BLOCK_BYTES;
+        char *Vw = lds_v0 + wave_u * BLOCK_BYTES;
+        const int n_my = wave_u < n_steps ? (n_steps - wave_u + 3) / 4 : 0;
+        if(n_my > 0)
+        {
+            const StepSource src = locate(wave_u);
+            fetch(src.K, src.rows_left, k_goff, lds_k0);
+            fetch(src.V, src.rows_left, v_goff, lds_v0);
+        }
+        // The Q values (ordinary loads) have arrived - said with an instruction
+        // the compiler's own wait insertion sees: otherwise it waits for them
+        // at their first use inside the loop, on every pass, with vmcnt(0).
+        f32_wait_vmcnt<0>();
+        // K of the next step is requested between the output MFMAs of this one
+        // (its buffer is free once the scores are done), V between the score
+        // MFMAs of the next (its buffer is free once the output products are):
+        // a load instruction issued behind an MFMA costs the wavefront nothing.
+        constexpr int K_EVERY = 16 / (LPW < 16 ? LPW : 16);     // one K piece every so many keys
+        constexpr int V_EVERY = QSTEPS >= LPW ? QSTEPS / LPW : 1;
+        constexpr int V_PER = QSTEPS >= LPW ? 1 : LPW / QSTEPS;
+        StepSource cur = {nullptr, nullptr, 0};
+        bool v_pending = false;     // V of step i is still to be requested (inside its score MFMAs)
+        for(int i = 0; i < n_my; ++i)
+        {
+            const int g = wave_u + 4 * i;
+            const bool more = i + 1 < n_my;
+            StepSource nxt = {nullptr, nullptr, 0};
+            if(more)
             {
-#pragma unroll
-                for(int x = 0; x < 4; ++x)
-                {
-                    const int r = 4 * g4 + x;
-                    const int key = 8 * (r >> 2) + 4 * half + (r & 3);
-#pragma unroll
-                    for(int db = 0; db < DBLOCKS; ++db)
-                    {
-                        va[r][db] = Vw[key * PAD + db * 32 + col];
-                    }
-                }
-            };
-            read_group(0);
-#pragma unroll
-            for(int g4 = 0; g4 < 4; ++g4)
+                nxt = locate(g + 4);
+            }
+            const bool skip = hidden(g);
+            f32x16 s;
+            if(v_pending)
             {
-                if(g4 + 1 < 4)
+                // K(i) has landed (everything has); V(i) goes out now
+                f32_wait_vmcnt<0>();
+                if(!skip)
                 {
-                    read_group(g4 + 1);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for(int x = 0; x < 4; ++x)
-                {
-                    const int r = 4 * g4 + x;
-#pragma unroll
-                    for(int db = 0; db < DBLOCKS; ++db)
+                    scores(g, Kw, s, [&](int t)
                     {
-                        o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[r][db], s[r], o[db],
-                                0, 0, 0);
-                        if(db == 0)
+                        if(t % V_EVERY == 0 && t / V_EVERY * V_PER < LPW)
                         {
-                            fetch_slot(QSTEPS + r);
-                            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                            for(int x = 0; x < V_PER; ++x)
+                            {
+                                fetch_piece(cur.V, cur.rows_left, v_goff, lds_v0, t / V_EVERY * V_PER + x);
+                            }
                         }
-                    }
+                    });
                 }
+                else
+                {
+                    fetch(cur.V, cur.rows_left, v_goff, lds_v0);
+                }
+            }
+            else
+            {
+                // first step: K(0) has landed, V(0) is on its way behind it
+                f32_wait_vmcnt<LPW>();
+                if(!skip)
+                {
+                    scores(g, Kw, s, nothing);
+                }
+            }
+            if(!skip)
+            {
+                softmax(s);
+            }
+            // V(i) has landed
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            f32_wait_vmcnt<0>();
+            if(!skip)
+            {
+                output(Vw, s, [&](int t)
+                {
+                    if(more && t % K_EVERY == 0 && t / K_EVERY < LPW)
+                    {
+                        fetch_piece(nxt.K, nxt.rows_left, k_goff, lds_k0, t / K_EVERY);
+                    }
+                });
+            }
+            else if(more)
+            {
+                fetch(nxt.K, nxt.rows_left, k_goff, lds_k0);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            cur = nxt;
+            v_pending = more;
+        }
+    }
+    else
+    {
+        // ---- the four wavefronts share every key step ------------------------------
+        if(n_steps > 0)
+        {
+            const StepSource src = locate(0);
+            fetch(src.K, src.rows_left, k_goff, lds_k0);
+            fetch(src.V, src.rows_left, v_goff, lds_v0);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        auto step = [&](int g, auto buf_tag) __attribute__((always_inline))
+        {
+            constexpr int BUF = decltype(buf_tag)::value;
+            // loads of the next step into the other buffers (every wavefront
+            // passed the barrier that ended step g-1: nobody reads them)
+            if(g + 1 < n_steps)
+            {
+                const StepSource nxt = locate(g + 1);
+                fetch(nxt.K, nxt.rows_left, k_goff, BUF ? lds_k0 : lds_k1);
+                fetch(nxt.V, nxt.rows_left, v_goff, BUF ? lds_v0 : lds_v1);
+            }
+            if(!hidden(g))
+            {
+                f32x16 s;
+                scores(g, BUF ? lds_k1 : lds_k0, s, nothing);
+                softmax(s);
+                output(BUF ? lds_v1 : lds_v0, s, nothing);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        };
+        for(int g = 0; g < n_steps; g += 2)
+        {
+            step(g, std::integral_constant<int, 0>{});
+            if(g + 1 < n_steps)
+            {
+                step(g + 1, std::integral_constant<int, 1>{});
             }
         }
     }
@@ -481,9 +667,10 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     {
         // word w of lane l of wavefront v (v = 1..3) sits at ((v-1)*NW + w)*64 + l
         constexpr int NW = 2 + 16 * DBLOCKS;
-        static_assert((NSUB - 1) * NW * 64 <= NSUB * kKeys32 * PAD, "exchange area does not fit");
-        float *xch = Ks;
-        __syncthreads();        // everyone is done with the staged keys
+        static_assert((NSUB - 1) * NW * 64 * 4 <= NSUB * BLOCK_BYTES, "exchange area does not fit");
+        float *xch = reinterpret_cast<float *>(lds_k0);
+        f32_wait_vmcnt<0>();
+        __syncthreads();        // everyone is done with the key buffers
         if(wave > 0)
         {
             float *dst = xch + (wave - 1) * NW * 64 + lane;
@@ -585,22 +772,22 @@ static int launch_mode32(hipStream_t stream, const PrefillParams &p, int mode,
     {
         case NNTILE_HIP_MASK_ADDITIVE:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_ADDITIVE, SPLIT>), grid, dim3(SPLIT ? split_waves32(HEAD) * 64 : kThreads32), 0,
+                        NNTILE_HIP_MASK_ADDITIVE, SPLIT>), grid, dim3(kThreads32), 0,
                     stream, p);
             break;
         case NNTILE_HIP_MASK_NONE:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_NONE, SPLIT>), grid, dim3(SPLIT ? split_waves32(HEAD) * 64 : kThreads32), 0,
+                        NNTILE_HIP_MASK_NONE, SPLIT>), grid, dim3(kThreads32), 0,
                     stream, p);
             break;
         case NNTILE_HIP_MASK_CAUSAL:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_CAUSAL, SPLIT>), grid, dim3(SPLIT ? split_waves32(HEAD) * 64 : kThreads32), 0,
+                        NNTILE_HIP_MASK_CAUSAL, SPLIT>), grid, dim3(kThreads32), 0,
                     stream, p);
             break;
         case NNTILE_HIP_MASK_BOOL:
             hipLaunchKernelGGL((sdpa_prefill_fp32_kernel<HEAD,
-                        NNTILE_HIP_MASK_BOOL, SPLIT>), grid, dim3(SPLIT ? split_waves32(HEAD) * 64 : kThreads32), 0,
+                        NNTILE_HIP_MASK_BOOL, SPLIT>), grid, dim3(kThreads32), 0,
                     stream, p);
             break;
         default:
