@@ -32,8 +32,10 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # properties of the kernel and the workload, not of one timing run; each names
 # the committed rocprofv3 summary it was read from.
 TRAFFIC = {
-    "cfg3_llama_prefill_bf16": (175220098, "profiles/sdpa_prefill_16bit_kernel_cfg3_llama_prefill_bf16.txt"),
-    "cfg4_gqa_decode_bf16": (295683470, "profiles/sdpa_decode_16bit_kernel_cfg4_gqa_decode_bf16.txt"),
+    "cfg3_llama_prefill_bf16": (175127911, "profiles/sdpa_prefill_16bit_kernel_cfg3_llama_prefill_bf16.txt"),
+    "cfg4_gqa_decode_bf16": (295681626, "profiles/sdpa_decode_16bit_kernel_cfg4_gqa_decode_bf16.txt"),
+    # per step = four launches
+    "cfg2_gpt2_small_fp32": (75828302, "profiles/sdpa_prefill_fp32_kernel_cfg2_gpt2_small_fp32.txt"),
 }
 
 
@@ -143,7 +145,7 @@ def bench_prefill(cfg, steps, warmup):
             "tflops": cfg.flops() / (wall * 1e-3) / 1e12}
 
 
-def bench_reference_grid(steps, warmup):
+def bench_reference_grid(steps, warmup, case=None):
     """The reference's own benchmark grid for this kernel
     (tests/kernel/flash_sdpa_fwd_cudnn.cc:591-613): seq in {128, 1024, 4096} x
     head in {64, 128} x batch in {4, 8} x {causal, full} x {bf16, fp16}, one
@@ -151,23 +153,35 @@ def bench_reference_grid(steps, warmup):
     nntile_hip_flash_sdpa_fwd_* with the additive mask tile the reference
     passes (merge into an lse of -inf, as its test does), and through the tile
     entry point with the same mask given analytically (overwrite mode).
-    FLOPs: 4 * head * visible pairs * batch (causal-exact for the causal mask)."""
+    FLOPs: 4 * head * visible pairs * batch (causal-exact for the causal mask).
+    `case` = "dtype,seq,head,batch,mask" restricts the run to that one case
+    (for a profiler)."""
     import numpy as np
     import torch
     from nntile_amd import hip_sdpa as h, synth
     rows = []
+    want = case.split(",") if case else None
+    take = lambda i, v: want is None or i >= len(want) or want[i] in ("", "*", str(v))
     for dtype, dt in (("bf16", torch.bfloat16), ("fp16", torch.float16)):
+        if not take(0, dtype):
+            continue
         for seq in (128, 1024, 4096):
+            if not take(1, seq):
+                continue
             vis = synth.causal_mask(seq, seq)
             masks = {"causal": torch.from_numpy(np.where(vis, 0.0, -np.inf).astype(np.float32)).to(dt).cuda(),
                      "full": torch.zeros((seq, seq), dtype=dt, device="cuda")}
             for head in (64, 128):
                 for batch in (4, 8):
+                    if not (take(2, head) and take(3, batch)):
+                        continue
                     shape = (batch, seq, head)
                     Q, K, V = (_randn(shape, dt, 42, i) for i in range(3))
                     A = torch.zeros_like(Q)
                     lse = torch.empty((batch, seq), dtype=torch.float32, device="cuda")
                     for mask_type in ("causal", "full"):
+                        if not take(4, mask_type):
+                            continue
                         pairs = seq * (seq + 1) // 2 if mask_type == "causal" else seq * seq
                         flops = 4.0 * head * pairs * batch
                         m = masks[mask_type]
@@ -497,6 +511,9 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--case", default=None,
+                    help="with --only reference_grid: one case, as dtype,seq,head,batch,mask "
+                         "(e.g. bf16,4096,64,8,causal)")
     ap.add_argument("--only", default=None,
                     help="run only this leg (for profiling): prefill | cfg5 | cfg2 | decode | decode_wide | "
                          "reference_api | reference_grid | backward | rope | transpose | accumulate | "
@@ -529,7 +546,7 @@ def main():
             "decode": lambda: bench_decode(cfg4, args.steps, args.warmup),
             "decode_wide": lambda: bench_decode(cfg4_wide, args.steps, args.warmup),
             "reference_api": lambda: bench_reference_api(cfg3, args.steps, args.warmup),
-            "reference_grid": lambda: bench_reference_grid(args.steps, args.warmup),
+            "reference_grid": lambda: bench_reference_grid(args.steps, args.warmup, args.case),
             "backward": lambda: bench_backward(cfg3, args.steps, args.warmup),
             "rope": lambda: bench_rope(cfg3, args.steps, args.warmup),
             "transpose": lambda: bench_transpose(cfg3, args.steps, args.warmup),
@@ -567,7 +584,8 @@ def main():
             "roofline": roofline("mfma", "sdpa_prefill_fp32_kernel<%d,causal>" % c.head if fp32
                                  else "sdpa_prefill_16bit_kernel<bf16,%d,causal>" % c.head,
                                  c.flops(), r["device_ms_per_step"],
-                                 PEAK_FP32_TFLOPS if fp32 else PEAK_BF16_TFLOPS, "TFLOP/s")}
+                                 PEAK_FP32_TFLOPS if fp32 else PEAK_BF16_TFLOPS, "TFLOP/s",
+                                 TRAFFIC.get(name))}
     backward = bench_backward(cfg3, max(5, args.steps // 10), 3)
     rope = bench_rope(cfg3, few, 5)
     transpose = bench_transpose(cfg3, few, 5)
