@@ -111,10 +111,49 @@ def _outliers(cfg, q):
     return q
 
 
-def bench_prefill(cfg, steps, warmup):
+class PowerSampler:
+    """Board power in W from the amdgpu hwmon file, sampled every 50 ms by a
+    thread while a loop runs; None where the file cannot be read."""
+
+    def __init__(self):
+        import glob
+        files = glob.glob("/sys/class/drm/card*/device/hwmon/*/power1_input")
+        self.path = files[0] if files else None
+        self.samples = []
+
+    def __enter__(self):
+        import threading
+        self.stop = threading.Event()
+
+        def loop():
+            while not self.stop.is_set():
+                try:
+                    with open(self.path) as f:
+                        self.samples.append(int(f.read()) / 1e6)
+                except (OSError, ValueError, TypeError):
+                    pass
+                time.sleep(0.05)
+        self.thread = threading.Thread(target=loop)
+        if self.path:
+            self.thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self.stop.set()
+        if self.path:
+            self.thread.join()
+
+    def watts(self):
+        # the first quarter of the samples is the ramp
+        tail = self.samples[len(self.samples) // 4:]
+        return round(sum(tail) / len(tail), 0) if tail else None
+
+
+def bench_prefill(cfg, steps, warmup, zeros=False):
     """One fused launch per independent slab of cfg over its whole tile grid
     (analytic causal mask, hidden tile pairs skipped, overwrite mode).  Tiles
-    are separate allocations, as NNTile tensors are."""
+    are separate allocations, as NNTile tensors are.  zeros=True replaces the
+    inputs by zeros (for the power comparison only)."""
     import torch
     from nntile_amd import hip_sdpa as h
     dt = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[cfg.dtype]
@@ -123,6 +162,8 @@ def bench_prefill(cfg, steps, warmup):
     shape = (cfg.batch_flat, cfg.q_seq, cfg.head)
     q_all = _outliers(cfg, _randn(shape, torch.float32, cfg.seed, 0)).to(dt)
     k_all, v_all = _randn(shape, dt, cfg.seed, 1), _randn(shape, dt, cfg.seed, 2)
+    if zeros:
+        q_all.zero_(), k_all.zero_(), v_all.zero_()
     plans = []
     keep = []
     for c in range(cfg.calls):
@@ -143,6 +184,36 @@ def bench_prefill(cfg, steps, warmup):
     wall, dev = time_steps(step, steps, warmup)
     return {"ms_per_step": wall, "device_ms_per_step": dev, "launches_per_step": len(plans),
             "tflops": cfg.flops() / (wall * 1e-3) / 1e12}
+
+
+def bench_power_context(cfg, seconds=1.5):
+    """What the chip sustains under its power cap, for context: the cfg3
+    prefill launch and a plain library GEMM (torch.matmul, 8192^3 bf16), each
+    on N(0,1) data and on zeros, in loops of about `seconds`, with the board
+    power read beside them.  The matrix units' power depends on the data: on
+    zeros both run at the full clock, on random data both are held at the
+    power cap.  Not a roofline - the published peak stays the yardstick - but
+    it says how much of the distance to it any kernel can cover on such data."""
+    import torch
+    out = {"what": "loops of ~%.1f s; TFLOP/s and board power (W, amdgpu hwmon); the GEMM is the "
+                   "library's (torch.matmul 8192^3 bf16), shown only as the sustained matrix rate "
+                   "of this GPU on the same kind of data" % seconds}
+    for key, zeros in (("prefill_cfg3_randn", False), ("prefill_cfg3_zeros", True)):
+        with PowerSampler() as ps:
+            r = bench_prefill(cfg, int(seconds / 130e-6), 50, zeros=zeros)
+        out[key] = {"tflops": round(cfg.flops() / (r["device_ms_per_step"] * 1e-3) / 1e12, 1),
+                    "kernel_ms": round(r["device_ms_per_step"], 4), "watts": ps.watts()}
+    n = 8192
+    for key, zeros in (("library_gemm_randn", False), ("library_gemm_zeros", True)):
+        a = torch.zeros(n, n, dtype=torch.bfloat16, device="cuda") if zeros else \
+            _randn((n, n), torch.bfloat16, 7, 0)
+        b = torch.zeros_like(a) if zeros else _randn((n, n), torch.bfloat16, 7, 1)
+        c = torch.empty_like(a)
+        with PowerSampler() as ps:
+            _, dev = time_steps(lambda: torch.matmul(a, b.t(), out=c), int(seconds / 0.6e-3), 20)
+        out[key] = {"tflops": round(2.0 * n ** 3 / (dev * 1e-3) / 1e12, 1), "kernel_ms": round(dev, 4),
+                    "watts": ps.watts()}
+    return out
 
 
 def bench_reference_grid(steps, warmup, case=None):
@@ -516,7 +587,7 @@ def main():
                          "(e.g. bf16,4096,64,8,causal)")
     ap.add_argument("--only", default=None,
                     help="run only this leg (for profiling): prefill | cfg5 | cfg2 | decode | decode_wide | "
-                         "reference_api | reference_grid | backward | rope | transpose | accumulate | "
+                         "reference_api | reference_grid | power_context | backward | rope | transpose | accumulate | "
                          "kv_cache | copy")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -547,6 +618,7 @@ def main():
             "decode_wide": lambda: bench_decode(cfg4_wide, args.steps, args.warmup),
             "reference_api": lambda: bench_reference_api(cfg3, args.steps, args.warmup),
             "reference_grid": lambda: bench_reference_grid(args.steps, args.warmup, args.case),
+            "power_context": lambda: bench_power_context(cfg3),
             "backward": lambda: bench_backward(cfg3, args.steps, args.warmup),
             "rope": lambda: bench_rope(cfg3, args.steps, args.warmup),
             "transpose": lambda: bench_transpose(cfg3, args.steps, args.warmup),
@@ -591,6 +663,7 @@ def main():
     transpose = bench_transpose(cfg3, few, 5)
     kv_cache = bench_kv_cache(cfg4, few, 5)
     accumulate = bench_accumulate(cfg3, few, 5)
+    power = bench_power_context(cfg3)
     # The headline leg runs last: the first timed loop of a process measures
     # 5 % slower than the same loop a second later (clocks still settling),
     # whatever the warmup count.
@@ -660,6 +733,7 @@ def main():
         "transpose": transpose,
         "kv_cache": kv_cache,
         "accumulate_attn_output": accumulate,
+        "power_context": power,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg3)
