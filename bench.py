@@ -216,6 +216,30 @@ def bench_power_context(cfg, seconds=1.5):
     return out
 
 
+def bench_copy_context(steps, warmup):
+    """The runtime's plain device-to-device copy (torch's copy_) of 32 MiB and
+    128 MiB, buffers rotating: what a read-once / write-once stream of the size
+    of the rotary-embedding and transpose workloads reaches on this GPU."""
+    import torch
+    out = {"what": "hipMemcpy-class device copy, read + written bytes over device time; the "
+                   "HBM-bound helper kernels (rope, transpose, accumulate) move the same kind "
+                   "of stream"}
+    for mib, nrot in ((32, 8), (128, 4)):
+        srcs = [torch.empty(mib << 20, dtype=torch.uint8, device="cuda").fill_(j + 1) for j in range(nrot)]
+        dsts = [torch.empty_like(x) for x in srcs]
+        i = [0]
+
+        def step():
+            j = i[0] % nrot
+            dsts[j].copy_(srcs[j])
+            i[0] += 1
+        _, dev = time_steps(step, steps, warmup)
+        gbs = 2.0 * (mib << 20) / (dev * 1e-3) / 1e9
+        out["%d_MiB" % mib] = {"device_ms": round(dev, 4), "gbs": round(gbs, 1),
+                               "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)}
+    return out
+
+
 def bench_reference_grid(steps, warmup, case=None):
     """The reference's own benchmark grid for this kernel
     (tests/kernel/flash_sdpa_fwd_cudnn.cc:591-613): seq in {128, 1024, 4096} x
@@ -587,7 +611,7 @@ def main():
                          "(e.g. bf16,4096,64,8,causal)")
     ap.add_argument("--only", default=None,
                     help="run only this leg (for profiling): prefill | cfg5 | cfg2 | decode | decode_wide | "
-                         "reference_api | reference_grid | power_context | backward | rope | transpose | accumulate | "
+                         "reference_api | reference_grid | power_context | copy_context | backward | rope | transpose | accumulate | "
                          "kv_cache | copy")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -619,6 +643,7 @@ def main():
             "reference_api": lambda: bench_reference_api(cfg3, args.steps, args.warmup),
             "reference_grid": lambda: bench_reference_grid(args.steps, args.warmup, args.case),
             "power_context": lambda: bench_power_context(cfg3),
+            "copy_context": lambda: bench_copy_context(args.steps, args.warmup),
             "backward": lambda: bench_backward(cfg3, args.steps, args.warmup),
             "rope": lambda: bench_rope(cfg3, args.steps, args.warmup),
             "transpose": lambda: bench_transpose(cfg3, args.steps, args.warmup),
@@ -664,6 +689,7 @@ def main():
     kv_cache = bench_kv_cache(cfg4, few, 5)
     accumulate = bench_accumulate(cfg3, few, 5)
     power = bench_power_context(cfg3)
+    copy_ctx = bench_copy_context(few, 5)
     # The headline leg runs last: the first timed loop of a process measures
     # 5 % slower than the same loop a second later (clocks still settling),
     # whatever the warmup count.
@@ -734,6 +760,7 @@ def main():
         "kv_cache": kv_cache,
         "accumulate_attn_output": accumulate,
         "power_context": power,
+        "copy_context": copy_ctx,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg3)
