@@ -38,6 +38,21 @@ namespace nntile_hip
 #ifndef NNTILE_F32_AHEAD
 #define NNTILE_F32_AHEAD 2
 #endif
+// Developer builds can turn F32_STAMP into time stamps of one wavefront
+#ifndef F32_STAMP
+#define F32_STAMP(i)
+#define F32_STAMP_DECL
+#define F32_STAMP_DUMP
+#endif
+// SPLIT form: how early in a phase the loads of the next block go out
+#ifndef NNTILE_F32_FRONT
+#define NNTILE_F32_FRONT 1
+#endif
+// SPLIT form: the softmax of the previous step behind every score MFMA (1) or
+// behind the first of each group of four (0)
+#ifndef NNTILE_F32_FINE
+#define NNTILE_F32_FINE 0
+#endif
 constexpr int kQRows32 = 128;
 constexpr int kKeys32 = 32;
 constexpr int kThreads32 = 256;          // 4 wavefronts in both forms
@@ -85,6 +100,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     const int wave = tid >> 6;
     const int col = lane & 31;
     const int half = lane >> 5;
+    F32_STAMP_DECL
 
     const int q_blocks = p.n_q_tiles * p.q_blocks_per_tile;
     int wg = blockIdx.x;
@@ -291,9 +307,10 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     float l_run = 0.0f;
 
     // Scores of key step g from the K block at Kw: S^T = K Q^T, mask.
-    // `between(t)` is called after the first MFMA of group t (QSTEPS groups):
-    // the place where a load instruction costs nothing, the matrix unit being
-    // busy with the group anyway.
+    // `between(t)` is called after MFMA t of the 4 * QSTEPS: whatever it issues
+    // (a load instruction, a few VALU instructions) runs while the matrix unit
+    // is busy with that MFMA - as long as it is short: work bunched up behind
+    // one MFMA leaves the unit idle for the rest of it.
     auto scores = [&](int g, const char *Kw, f32x16 &s, auto between) __attribute__((always_inline))
     {
         const int kt = g / p.k_blocks_per_tile;
@@ -302,21 +319,20 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         const int64_t k_row0 = (int64_t)kb * kKeys32;
         const int64_t k_pos_base = p.k_pos0 + (int64_t)kt * p.k_tile + k_row0;
         const int keys_here = (int)min((int64_t)kKeys32, k_len - k_row0);
-        // Two accumulators take the MFMAs in turn: each of them would
-        // otherwise wait for the one before it (64 cycles in the pipe, 84 from
-        // issue to issue when dependent).
-        f32x16 s2;
-#pragma unroll
-        for(int r = 0; r < 16; ++r)
-        {
-            s[r] = 0.0f;
-            s2[r] = 0.0f;
-        }
+        // One accumulator chain: a dependent MFMA of this shape issues right
+        // behind its predecessor (64 cycles apart, measured), and the first one
+        // takes a constant zero, so nothing is cleared or added up afterwards.
         // (the K operands of the step are read ahead of the chain of MFMAs: a
         // read issued behind four of them would only start once they have all
         // been issued)
         {
             constexpr int AHEAD = NNTILE_F32_AHEAD < QSTEPS ? NNTILE_F32_AHEAD : QSTEPS;
+            f32x16 zero16;
+#pragma unroll
+            for(int r = 0; r < 16; ++r)
+            {
+                zero16[r] = 0.0f;
+            }
             f32x4 ka[QSTEPS];
 #pragma unroll
             for(int j = 0; j < AHEAD; ++j)
@@ -334,26 +350,12 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
 #pragma unroll
                 for(int e = 0; e < 4; ++e)
                 {
-                    if(e & 1)
-                    {
-                        s2 = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[j][e], qf[j][e], s2, 0, 0, 0);
-                    }
-                    else
-                    {
-                        s = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[j][e], qf[j][e], s, 0, 0, 0);
-                    }
-                    if(e == 0)
-                    {
-                        between(j);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
+                    s = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[j][e], qf[j][e],
+                            (j == 0 && e == 0) ? zero16 : s, 0, 0, 0);
+                    between(4 * j + e);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
-        }
-#pragma unroll
-        for(int r = 0; r < 16; ++r)
-        {
-            s[r] += s2[r];
         }
 
         // ---- mask: register r holds key 8*(r/4) + 4*half + r%4 ---------------
@@ -453,51 +455,37 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         l_run += rs;
     };
 
-    // O^T += V^T P^T from the V block at Vw (V operands four keys at a time,
-    // one group ahead of its MFMAs).
-    // `between(t)` is called after the first MFMA of key t (16 keys).
+    // O^T += V^T P^T from the V block at Vw: MFMA n of the 16 * DBLOCKS takes
+    // key n / DBLOCKS and output block n % DBLOCKS; its V operand is read from
+    // LDS eight MFMAs ahead.  `between(n)` is called after MFMA n.
     auto output = [&](const char *Vw, const f32x16 &s, auto between) __attribute__((always_inline))
     {
-        float va[16][DBLOCKS];
-        auto read_group = [&](int g4)
+        constexpr int NM = 16 * DBLOCKS;
+        constexpr int AH = 8;
+        float va[NM];
+        auto read_operand = [&](int n) __attribute__((always_inline))
         {
-#pragma unroll
-            for(int x = 0; x < 4; ++x)
-            {
-                const int r = 4 * g4 + x;
-#pragma unroll
-                for(int db = 0; db < DBLOCKS; ++db)
-                {
-                    va[r][db] = *reinterpret_cast<const float *>(
-                            Vw + v_raddr[db] + (8 * (r >> 2) + (r & 3)) * RB);
-                }
-            }
+            const int r = n / DBLOCKS, db = n % DBLOCKS;
+            va[n] = *reinterpret_cast<const float *>(
+                    Vw + v_raddr[db] + (8 * (r >> 2) + (r & 3)) * RB);
         };
-        read_group(0);
 #pragma unroll
-        for(int g4 = 0; g4 < 4; ++g4)
+        for(int n = 0; n < AH; ++n)
         {
-            if(g4 + 1 < 4)
+            read_operand(n);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for(int n = 0; n < NM; ++n)
+        {
+            if(n + AH < NM)
             {
-                read_group(g4 + 1);
+                read_operand(n + AH);
             }
+            const int r = n / DBLOCKS, db = n % DBLOCKS;
+            o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[n], s[r], o[db], 0, 0, 0);
+            between(n);
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for(int x = 0; x < 4; ++x)
-            {
-                const int r = 4 * g4 + x;
-#pragma unroll
-                for(int db = 0; db < DBLOCKS; ++db)
-                {
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[r][db], s[r], o[db],
-                            0, 0, 0);
-                    if(db == 0)
-                    {
-                        between(r);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
-            }
         }
     };
     auto nothing = [](int) {};
@@ -527,97 +515,238 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     if constexpr(SPLIT)
     {
         // ---- every wavefront walks its own key steps wave, wave + 4, ... ---------
-        // through its own K and V buffer.  Loads complete in the order they
-        // were issued: K(i) V(i) K(i+1) V(i+1) ...
-        char *Kw = lds_k0 + wave_u * BLOCK_BYTES;
-        char *Vw = lds_v0 + wave_u * BLOCK_BYTES;
+        // through two buffers of its own and shares nothing with the others
+        // inside the loop, so the loop has no barrier.  The steps are software
+        // pipelined: the softmax of step i runs in the shadow of the score
+        // MFMAs of step i+1, then the output MFMAs of step i follow.
+        //   buffer R (lds_k0): K(i+1) while those scores are computed;
+        //   buffer P (lds_v0): V(i) while that output is computed - and K(0)
+        //                      at the very start, so that nothing waits for it.
+        // Loads complete in the order they were issued:
+        //   K(0)->P K(1)->R | V(0)->P K(2)->R | V(1)->P K(3)->R | ...
+        // V(i) is requested between the score MFMAs of step i+1 (P is free once
+        // the output of step i-1 is done), K(i+2) between the output MFMAs of
+        // step i (R is free once the scores of step i+1 are done): a load
+        // instruction issued behind an MFMA costs the wavefront nothing.
+        char *Rw = lds_k0 + wave_u * BLOCK_BYTES;
+        char *Pw = lds_v0 + wave_u * BLOCK_BYTES;
         const int n_my = wave_u < n_steps ? (n_steps - wave_u + 3) / 4 : 0;
+        // Piece i of a block's LPW load instructions goes out behind the MFMA
+        // group t = i * groups / (LPW * NNTILE_F32_FRONT): spread over all
+        // groups of the phase with 1, over its first half with 2, ...
+        constexpr int FRONT = NNTILE_F32_FRONT;
+        auto pieces = [](int t, int groups, int &lo, int &hi)
+        {
+            lo = t * LPW * FRONT / groups;
+            hi = (t + 1) * LPW * FRONT / groups;
+            lo = lo < LPW ? lo : LPW;
+            hi = hi < LPW ? hi : LPW;
+        };
         if(n_my > 0)
         {
-            const StepSource src = locate(wave_u);
-            fetch(src.K, src.rows_left, k_goff, lds_k0);
-            fetch(src.V, src.rows_left, v_goff, lds_v0);
-        }
-        // The Q values (ordinary loads) have arrived - said with an instruction
-        // the compiler's own wait insertion sees: otherwise it waits for them
-        // at their first use inside the loop, on every pass, with vmcnt(0).
-        f32_wait_vmcnt<0>();
-        // K of the next step is requested between the output MFMAs of this one
-        // (its buffer is free once the scores are done), V between the score
-        // MFMAs of the next (its buffer is free once the output products are):
-        // a load instruction issued behind an MFMA costs the wavefront nothing.
-        constexpr int K_EVERY = 16 / (LPW < 16 ? LPW : 16);     // one K piece every so many keys
-        constexpr int V_EVERY = QSTEPS >= LPW ? QSTEPS / LPW : 1;
-        constexpr int V_PER = QSTEPS >= LPW ? 1 : LPW / QSTEPS;
-        StepSource cur = {nullptr, nullptr, 0};
-        bool v_pending = false;     // V of step i is still to be requested (inside its score MFMAs)
-        for(int i = 0; i < n_my; ++i)
-        {
-            const int g = wave_u + 4 * i;
-            const bool more = i + 1 < n_my;
-            StepSource nxt = {nullptr, nullptr, 0};
-            if(more)
+            const StepSource src0 = locate(wave_u);
+            fetch(src0.K, src0.rows_left, k_goff, lds_v0);         // K(0) into P
+            StepSource src1 = {nullptr, nullptr, 0};
+            if(n_my > 1)
             {
-                nxt = locate(g + 4);
+                src1 = locate(wave_u + 4);
+                fetch(src1.K, src1.rows_left, k_goff, lds_k0);     // K(1) into R
+                // K(0) has landed, K(1) may still be on its way.  (This also
+                // says that the Q values, ordinary loads, have arrived, with an
+                // instruction the compiler's own wait insertion sees: otherwise
+                // it waits for them at their first use inside the loop, on every
+                // pass, with vmcnt(0).)
+                f32_wait_vmcnt<LPW>();
             }
-            const bool skip = hidden(g);
-            f32x16 s;
-            if(v_pending)
+            else
             {
-                // K(i) has landed (everything has); V(i) goes out now
                 f32_wait_vmcnt<0>();
-                if(!skip)
+            }
+            F32_STAMP(1)
+            f32x16 s_cur;
+            scores(wave_u, Pw, s_cur, nothing);
+            F32_STAMP(2)
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // P has been read
+            StepSource cur = src0;      // step i: its V is still to be requested
+            StepSource nxt = src1;      // step i+1: its K is in R or on its way there
+            for(int i = 0; i < n_my; ++i)
+            {
+                const int g = wave_u + 4 * i;
+                const bool more = i + 1 < n_my;
+                const bool more2 = i + 2 < n_my;
+                StepSource nxt2 = {nullptr, nullptr, 0};
+                if(more2)
                 {
-                    scores(g, Kw, s, [&](int t)
+                    nxt2 = locate(g + 8);
+                }
+                // ---- the softmax of step i, in pieces ----------------------------
+                float mc = 0.0f, rs = 0.0f;
+                auto softmax_head = [&]() __attribute__((always_inline))
+                {
+                    float mx = neg_inf();
+#pragma unroll
+                    for(int r = 0; r < 16; ++r)
                     {
-                        if(t % V_EVERY == 0 && t / V_EVERY * V_PER < LPW)
+                        mx = fmaxf(mx, s_cur[r]);
+                    }
+                    mx = max_across_halves(mx);
+                    const float m_new = fmaxf(m_run, mx);
+                    const float m_use = (m_new == neg_inf()) ? 0.0f : m_new;
+                    mc = m_use * c;
+                    // the running maximum rarely moves after the first steps
+                    if(__builtin_amdgcn_ballot_w64(m_new != m_run) != 0)
+                    {
+                        const float alpha = fast_exp2((m_run - m_use) * c);
+                        l_run *= alpha;
+#pragma unroll
+                        for(int db = 0; db < DBLOCKS; ++db)
                         {
 #pragma unroll
-                            for(int x = 0; x < V_PER; ++x)
+                            for(int r = 0; r < 16; ++r)
                             {
-                                fetch_piece(cur.V, cur.rows_left, v_goff, lds_v0, t / V_EVERY * V_PER + x);
+                                o[db][r] *= alpha;
+                            }
+                        }
+                        m_run = m_new;
+                    }
+                    asm volatile("" : "+v"(mc));
+                };
+                // elements [lo, hi) of the 16 scores of a lane
+                auto softmax_part = [&](int lo, int hi) __attribute__((always_inline))
+                {
+#pragma unroll
+                    for(int r = 0; r < 16; ++r)
+                    {
+                        if(r >= lo && r < hi)
+                        {
+                            float e = fast_exp2(fmaf(s_cur[r], c, -mc));
+                            // (keeps the exponential where it is written: its
+                            // result is first used by the output MFMAs, and the
+                            // compiler would otherwise move it down to them,
+                            // out of the shadow of the score MFMAs)
+                            asm volatile("" : "+v"(e));
+                            s_cur[r] = e;
+                            rs += e;
+                        }
+                    }
+                    asm volatile("" : "+v"(rs));
+                };
+                f32x16 s_nxt;
+                F32_STAMP(3 + 4 * i)
+                if(more)
+                {
+                    // K(i+1) has landed in R (everything requested so far has)
+                    f32_wait_vmcnt<0>();
+                    F32_STAMP(4 + 4 * i)
+                    scores(g + 4, Rw, s_nxt, [&](int t)
+                    {
+                        // behind the first MFMA of a group: V(i) goes out, into P;
+                        // behind the second MFMA of all: the head of the softmax;
+                        // behind the others: an element of it or none
+#if NNTILE_F32_FINE
+                        constexpr int NFREE = 3 * QSTEPS - 1;
+                        if(t % 4 == 0)
+                        {
+                            int lo, hi;
+                            pieces(t / 4, QSTEPS, lo, hi);
+#pragma unroll
+                            for(int x = 0; x < LPW; ++x)
+                            {
+                                if(x >= lo && x < hi)
+                                {
+                                    fetch_piece(cur.V, cur.rows_left, v_goff, lds_v0, x);
+                                }
+                            }
+                        }
+                        else if(t == 1)
+                        {
+                            softmax_head();
+                        }
+                        else
+                        {
+                            const int k = t - 2 - t / 4;    // which of the NFREE other places
+                            softmax_part(k * 16 / NFREE, (k + 1) * 16 / NFREE);
+                        }
+#else
+                        if(t % 4 == 0)
+                        {
+                            const int j = t / 4;
+                            int lo, hi;
+                            pieces(j, QSTEPS, lo, hi);
+#pragma unroll
+                            for(int x = 0; x < LPW; ++x)
+                            {
+                                if(x >= lo && x < hi)
+                                {
+                                    fetch_piece(cur.V, cur.rows_left, v_goff, lds_v0, x);
+                                }
+                            }
+                            if(j == 0)
+                            {
+                                softmax_head();
+                            }
+                            else
+                            {
+                                softmax_part((j - 1) * 16 / (QSTEPS - 1), j * 16 / (QSTEPS - 1));
+                            }
+                        }
+#endif
+                    });
+                }
+                else
+                {
+                    fetch(cur.V, cur.rows_left, v_goff, lds_v0);
+                    softmax_head();
+                    softmax_part(0, 16);
+                }
+                l_run += rs;
+                // R has been read, V(i) has landed in P
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                F32_STAMP(5 + 4 * i)
+                f32_wait_vmcnt<0>();
+                F32_STAMP(6 + 4 * i)
+                // (two copies of the phase rather than a branch around every
+                // load instruction inside it)
+                if(more2)
+                {
+                    output(Pw, s_cur, [&](int t)
+                    {
+                        // K(i+2) goes out, into R
+                        if(t % DBLOCKS == 0)
+                        {
+                            int lo, hi;
+                            pieces(t / DBLOCKS, 16, lo, hi);
+#pragma unroll
+                            for(int x = 0; x < LPW; ++x)
+                            {
+                                if(x >= lo && x < hi)
+                                {
+                                    fetch_piece(nxt2.K, nxt2.rows_left, k_goff, lds_k0, x);
+                                }
                             }
                         }
                     });
                 }
                 else
                 {
-                    fetch(cur.V, cur.rows_left, v_goff, lds_v0);
+                    output(Pw, s_cur, nothing);
                 }
-            }
-            else
-            {
-                // first step: K(0) has landed, V(0) is on its way behind it
-                f32_wait_vmcnt<LPW>();
-                if(!skip)
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // P has been read
+                if(more)
                 {
-                    scores(g, Kw, s, nothing);
-                }
-            }
-            if(!skip)
-            {
-                softmax(s);
-            }
-            // V(i) has landed
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            f32_wait_vmcnt<0>();
-            if(!skip)
-            {
-                output(Vw, s, [&](int t)
-                {
-                    if(more && t % K_EVERY == 0 && t / K_EVERY < LPW)
+#pragma unroll
+                    for(int r = 0; r < 16; ++r)
                     {
-                        fetch_piece(nxt.K, nxt.rows_left, k_goff, lds_k0, t / K_EVERY);
+                        s_cur[r] = s_nxt[r];
                     }
-                });
+                }
+                cur = nxt;
+                nxt = nxt2;
             }
-            else if(more)
-            {
-                fetch(nxt.K, nxt.rows_left, k_goff, lds_k0);
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            cur = nxt;
-            v_pending = more;
+        }
+        else
+        {
+            f32_wait_vmcnt<0>();
         }
     }
     else
@@ -669,8 +798,10 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         constexpr int NW = 2 + 16 * DBLOCKS;
         static_assert((NSUB - 1) * NW * 64 * 4 <= NSUB * BLOCK_BYTES, "exchange area does not fit");
         float *xch = reinterpret_cast<float *>(lds_k0);
+        F32_STAMP(43)
         f32_wait_vmcnt<0>();
         __syncthreads();        // everyone is done with the key buffers
+        F32_STAMP(44)
         if(wave > 0)
         {
             float *dst = xch + (wave - 1) * NW * 64 + lane;
@@ -715,6 +846,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     }
 
     // ---- epilogue --------------------------------------------------------------
+    F32_STAMP(45)
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     const bool empty = !(l_tot > 0.0f);     // no visible key for this query
     if(!q_ok || (empty && !p.overwrite))
@@ -762,6 +894,8 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
             *reinterpret_cast<f32x4 *>(dst) = v;
         }
     }
+    F32_STAMP(46)
+    F32_STAMP_DUMP
 }
 
 template<int HEAD, bool SPLIT>
