@@ -44,10 +44,6 @@ namespace nntile_hip
 #define F32_STAMP_DECL
 #define F32_STAMP_DUMP
 #endif
-// SPLIT form: how early in a phase the loads of the next block go out
-#ifndef NNTILE_F32_FRONT
-#define NNTILE_F32_FRONT 1
-#endif
 // SPLIT form: the softmax of the previous step behind every score MFMA (1) or
 // behind the first of each group of four (0)
 #ifndef NNTILE_F32_FINE
@@ -531,17 +527,10 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         char *Rw = lds_k0 + wave_u * BLOCK_BYTES;
         char *Pw = lds_v0 + wave_u * BLOCK_BYTES;
         const int n_my = wave_u < n_steps ? (n_steps - wave_u + 3) / 4 : 0;
-        // Piece i of a block's LPW load instructions goes out behind the MFMA
-        // group t = i * groups / (LPW * NNTILE_F32_FRONT): spread over all
-        // groups of the phase with 1, over its first half with 2, ...
-        constexpr int FRONT = NNTILE_F32_FRONT;
-        auto pieces = [](int t, int groups, int &lo, int &hi)
-        {
-            lo = t * LPW * FRONT / groups;
-            hi = (t + 1) * LPW * FRONT / groups;
-            lo = lo < LPW ? lo : LPW;
-            hi = hi < LPW ? hi : LPW;
-        };
+        // Both phases have 4 * LPW MFMAs: load instruction i of the next block
+        // goes out behind MFMA 4 * i.  (Issuing them earlier in the phase - all
+        // in its first half, its first quarter, or at once - changed nothing.)
+        static_assert(LPW == QSTEPS && 16 * DBLOCKS == 4 * LPW, "one load instruction per four MFMAs");
         if(n_my > 0)
         {
             const StepSource src0 = locate(wave_u);
@@ -647,16 +636,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
                         constexpr int NFREE = 3 * QSTEPS - 1;
                         if(t % 4 == 0)
                         {
-                            int lo, hi;
-                            pieces(t / 4, QSTEPS, lo, hi);
-#pragma unroll
-                            for(int x = 0; x < LPW; ++x)
-                            {
-                                if(x >= lo && x < hi)
-                                {
-                                    fetch_piece(cur.V, cur.rows_left, v_goff, lds_v0, x);
-                                }
-                            }
+                            fetch_piece(cur.V, cur.rows_left, v_goff, lds_v0, t / 4);
                         }
                         else if(t == 1)
                         {
@@ -671,16 +651,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
                         if(t % 4 == 0)
                         {
                             const int j = t / 4;
-                            int lo, hi;
-                            pieces(j, QSTEPS, lo, hi);
-#pragma unroll
-                            for(int x = 0; x < LPW; ++x)
-                            {
-                                if(x >= lo && x < hi)
-                                {
-                                    fetch_piece(cur.V, cur.rows_left, v_goff, lds_v0, x);
-                                }
-                            }
+                            fetch_piece(cur.V, cur.rows_left, v_goff, lds_v0, j);
                             if(j == 0)
                             {
                                 softmax_head();
@@ -712,18 +683,9 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
                     output(Pw, s_cur, [&](int t)
                     {
                         // K(i+2) goes out, into R
-                        if(t % DBLOCKS == 0)
+                        if(t % 4 == 0)
                         {
-                            int lo, hi;
-                            pieces(t / DBLOCKS, 16, lo, hi);
-#pragma unroll
-                            for(int x = 0; x < LPW; ++x)
-                            {
-                                if(x >= lo && x < hi)
-                                {
-                                    fetch_piece(nxt2.K, nxt2.rows_left, k_goff, lds_k0, x);
-                                }
-                            }
+                            fetch_piece(nxt2.K, nxt2.rows_left, k_goff, lds_k0, t / 4);
                         }
                     });
                 }
