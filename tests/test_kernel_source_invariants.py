@@ -94,3 +94,14 @@ def test_no_packed_fp32_instructions(assemblies):
     for name, text in assemblies.items():
         for line in _instructions(text):
             assert not re.match(r"v_pk_(add|mul|fma)_f32\b", line), (name, line)
+
+
+def test_forward_kernels_use_no_scratch_memory(assemblies):
+    """An array that the compiler could not keep in registers (a loop it did
+    not unroll, a register index known only at run time) shows up as private
+    scratch memory: slow, and with run-time indexing an implicit M0 user.  The
+    forward kernels are written to need none."""
+    for name in ("sdpa_prefill_16bit.hip", "sdpa_prefill_fp32.hip", "sdpa_decode_16bit.hip"):
+        sizes = re.findall(r"\.private_segment_fixed_size:\s*(\d+)", assemblies[name])
+        assert sizes, name
+        assert all(int(x) == 0 for x in sizes), (name, sorted(set(sizes)))
