@@ -245,8 +245,10 @@ def bench_reference_grid(steps, warmup, case=None):
     (tests/kernel/flash_sdpa_fwd_cudnn.cc:591-613): seq in {128, 1024, 4096} x
     head in {64, 128} x batch in {4, 8} x {causal, full} x {bf16, fp16}, one
     square tile, random data.  Each case twice: through
-    nntile_hip_flash_sdpa_fwd_* with the additive mask tile the reference
-    passes (merge into an lse of -inf, as its test does), and through the tile
+    nntile_hip_flash_sdpa_fwd_* with the additive mask tile and the two scratch
+    tiles the reference passes (merge into an lse of -inf, as its test does;
+    masks of 1 MiB and more are scanned once per call into the scratch
+    logsumexp tile by a small kernel of its own), and through the tile
     entry point with the same mask given analytically (overwrite mode).
     FLOPs: 4 * head * visible pairs * batch (causal-exact for the causal mask).
     `case` = "dtype,seq,head,batch,mask" restricts the run to that one case
@@ -274,13 +276,15 @@ def bench_reference_grid(steps, warmup, case=None):
                     Q, K, V = (_randn(shape, dt, 42, i) for i in range(3))
                     A = torch.zeros_like(Q)
                     lse = torch.empty((batch, seq), dtype=torch.float32, device="cuda")
+                    # the reference's two scratch tiles (STARPU_SCRATCH handles)
+                    scratch_lse, scratch_A = torch.empty_like(lse), torch.empty_like(A)
                     for mask_type in ("causal", "full"):
                         if not take(4, mask_type):
                             continue
                         pairs = seq * (seq + 1) // 2 if mask_type == "causal" else seq * seq
                         flops = 4.0 * head * pairs * batch
                         m = masks[mask_type]
-                        additive = h.plan_tile(K, Q, m, lse, V, A, h.MASK_ADDITIVE)
+                        additive = h.FlashPlan(K, Q, m, lse, V, A, scratch_lse, scratch_A)
 
                         def with_mask():
                             lse.fill_(float("-inf"))

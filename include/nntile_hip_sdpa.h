@@ -71,8 +71,13 @@ enum nntile_hip_mask_mode
  *  src/kernel/flash_sdpa_fwd_cudnn/cuda.cc:145-202): same argument order and
  * meaning, the cuDNN handle/graph pair replaced by the stream.  One square
  * tile: seq queries against seq keys, additive mask [seq, seq] in T.
- * scratch_lse and scratch_A are accepted for signature compatibility and
- * never touched (the merge is fused into the kernel); they may be null. */
+ * The merge is fused into the kernel, so neither scratch tile is needed for
+ * it and both may be null.  scratch_A is never touched.  scratch_lse (seq *
+ * batch floats, as the reference registers it) may be overwritten: when the
+ * mask is 1 MiB or larger the 16-bit variants scan it once per call with a
+ * small kernel of their own and keep what they found (16 bytes per 128
+ * queries and key range) there, instead of letting the workgroups of every
+ * batch entry scan the same rows.  Same result, bit for bit. */
 int nntile_hip_flash_sdpa_fwd_bf16(void *stream, int64_t seq, int64_t head,
         int64_t batch, const uint16_t *K, const uint16_t *Q,
         const uint16_t *mask, float *scratch_lse, const uint16_t *V,

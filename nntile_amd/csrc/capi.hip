@@ -10,7 +10,8 @@ namespace nntile_hip
 {
 
 template<typename T>
-int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head, int mode);
+int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head, int mode,
+        void *scan_scratch, size_t scan_scratch_bytes);
 int launch_prefill_fp32(hipStream_t stream, PrefillParams &p, int head, int mode);
 
 template<typename T>
@@ -55,7 +56,8 @@ static bool mode_ok(int mode)
 }
 
 static int dispatch_prefill(DType dt, hipStream_t stream, PrefillParams &p,
-        int64_t head, int mode)
+        int64_t head, int mode, void *scan_scratch = nullptr,
+        size_t scan_scratch_bytes = 0)
 {
     if(head != 32 && head != 64 && head != 128)
     {
@@ -65,16 +67,20 @@ static int dispatch_prefill(DType dt, hipStream_t stream, PrefillParams &p,
     switch(dt)
     {
         case DType::bf16:
-            return launch_prefill_16bit<Bf16>(stream, p, (int)head, mode);
+            return launch_prefill_16bit<Bf16>(stream, p, (int)head, mode, scan_scratch,
+                    scan_scratch_bytes);
         case DType::fp16:
-            return launch_prefill_16bit<Fp16>(stream, p, (int)head, mode);
+            return launch_prefill_16bit<Fp16>(stream, p, (int)head, mode, scan_scratch,
+                    scan_scratch_bytes);
         default:
             return launch_prefill_fp32(stream, p, (int)head, mode);
     }
 }
 
+// scan_scratch: device memory the call may overwrite (the reference's
+// scratch_logsumexp tile, scan_scratch_bytes of it), or null
 static int tile_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a,
-        int64_t kv_rows = 0)
+        int64_t kv_rows = 0, void *scan_scratch = nullptr, size_t scan_scratch_bytes = 0)
 {
     if(a == nullptr || a->q_seq <= 0 || a->k_seq <= 0 || a->head <= 0
             || a->batch <= 0 || a->n_batch <= 0 || a->kv_group <= 0
@@ -118,7 +124,7 @@ static int tile_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a,
     p.lse[0] = a->lse;
     p.A[0] = a->A;
     return dispatch_prefill(dt, static_cast<hipStream_t>(stream), p, a->head,
-            a->mask_mode);
+            a->mask_mode, scan_scratch, scan_scratch_bytes);
 }
 
 static int bwd_call(DType dt, void *stream, const nntile_hip_sdpa_bwd_args *a)
@@ -228,9 +234,22 @@ static int flash_bwd_call(DType dt, void *stream, int64_t seq, int64_t head,
     return bwd_call(dt, stream, &a);
 }
 
+// bytes of a [seq, batch] fp32 tile (what the reference registers as
+// scratch_logsumexp); 0 for sizes that are refused anyway
+static size_t tile_floats_bytes(int64_t seq, int64_t batch)
+{
+    return (seq > 0 && batch > 0 && seq <= 0x7fffffff && batch <= 0x7fffffff)
+        ? (size_t)seq * (size_t)batch * sizeof(float) : 0;
+}
+
+// scratch_lse: the reference's scratch tile for the logsumexp of the pair
+// (seq * batch floats, src/starpu/flash_sdpa_fwd_cudnn.cc:128-136); the merge
+// is fused into the kernel, so the tile is free: a large mask is scanned once
+// into it instead of once per batch entry.  May be null.
 static int flash_call(DType dt, void *stream, int64_t seq, int64_t head,
         int64_t batch, const void *K, const void *Q, const void *mask,
-        const void *V, float *lse, void *A)
+        const void *V, float *lse, void *A, float *scratch_lse,
+        size_t scratch_lse_bytes)
 {
     nntile_hip_sdpa_tile_args a;
     std::memset(&a, 0, sizeof(a));
@@ -246,7 +265,7 @@ static int flash_call(DType dt, void *stream, int64_t seq, int64_t head,
     a.V = V;
     a.lse = lse;
     a.A = A;
-    return tile_call(dt, stream, &a);
+    return tile_call(dt, stream, &a, 0, scratch_lse, scratch_lse_bytes);
 }
 
 static int grid_call(DType dt, void *stream, const nntile_hip_sdpa_grid_args *a)
@@ -630,7 +649,10 @@ static void codelet_call(DType dt, const char *name, void *buffers[],
             reinterpret_cast<const void *>(ifs[2]->ptr),
             reinterpret_cast<const void *>(ifs[4]->ptr),
             reinterpret_cast<float *>(ifs[3]->ptr),
-            reinterpret_cast<void *>(ifs[5]->ptr));
+            reinterpret_cast<void *>(ifs[5]->ptr),
+            // buffer 6: the scratch tile for the pair's logsumexp
+            ifs[6] != nullptr ? reinterpret_cast<float *>(ifs[6]->ptr) : nullptr,
+            ifs[6] != nullptr ? ifs[6]->elemsize : 0);
     if(rc != NNTILE_HIP_OK)
     {
         std::fprintf(stderr, "HIP Worker: %s: launch failed with code %d "
@@ -686,25 +708,27 @@ extern "C"
 
 int nntile_hip_flash_sdpa_fwd_bf16(void *stream, int64_t seq, int64_t head,
         int64_t batch, const uint16_t *K, const uint16_t *Q,
-        const uint16_t *mask, float *, const uint16_t *V, uint16_t *,
+        const uint16_t *mask, float *scratch_lse, const uint16_t *V, uint16_t *,
         float *lse, uint16_t *A)
 {
-    return flash_call(DType::bf16, stream, seq, head, batch, K, Q, mask, V, lse, A);
+    return flash_call(DType::bf16, stream, seq, head, batch, K, Q, mask, V, lse, A,
+            scratch_lse, tile_floats_bytes(seq, batch));
 }
 
 int nntile_hip_flash_sdpa_fwd_fp16(void *stream, int64_t seq, int64_t head,
         int64_t batch, const uint16_t *K, const uint16_t *Q,
-        const uint16_t *mask, float *, const uint16_t *V, uint16_t *,
+        const uint16_t *mask, float *scratch_lse, const uint16_t *V, uint16_t *,
         float *lse, uint16_t *A)
 {
-    return flash_call(DType::fp16, stream, seq, head, batch, K, Q, mask, V, lse, A);
+    return flash_call(DType::fp16, stream, seq, head, batch, K, Q, mask, V, lse, A,
+            scratch_lse, tile_floats_bytes(seq, batch));
 }
 
 int nntile_hip_flash_sdpa_fwd_fp32(void *stream, int64_t seq, int64_t head,
         int64_t batch, const float *K, const float *Q, const float *mask,
         float *, const float *V, float *, float *lse, float *A)
 {
-    return flash_call(DType::fp32, stream, seq, head, batch, K, Q, mask, V, lse, A);
+    return flash_call(DType::fp32, stream, seq, head, batch, K, Q, mask, V, lse, A, nullptr, 0);
 }
 
 int nntile_hip_sdpa_fwd_tile_bf16(void *stream, const nntile_hip_sdpa_tile_args *args)

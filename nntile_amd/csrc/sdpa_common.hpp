@@ -38,6 +38,9 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 // Kernel arguments of the prefill kernels (passed by value in the kernarg
 // segment).  Query tile t holds rows [t*q_tile, min((t+1)*q_tile, q_seq)),
 // the same for key tiles.
+// Key ranges a mask is scanned in by mask_step_bits_kernel
+constexpr int kMaskBitSplits = 8;
+
 struct PrefillParams
 {
     int64_t q_seq, k_seq, q_tile, k_tile;
@@ -46,6 +49,13 @@ struct PrefillParams
     int64_t kv_rows;              // rows between two entries of K and V; 0: the tile's own rows
                                   // (a cache's capacity, single key tile only)
     const void *mask;
+    // explicit masks, one query tile: what a scan of the mask rows of every
+    // 128-query block found, written by mask_step_bits_kernel before the
+    // launch - kMaskBitSplits pairs of 64-bit words per block (one pair per
+    // range of keys, to be OR-ed): bit s of the first word: some value of
+    // 64-key step s is not "open", of the second: not "hidden" (steps from 63
+    // on share bit 63).  Null: every workgroup scans its own rows.
+    const unsigned long long *mask_bits;
     int32_t n_q_tiles, n_kv_tiles;
     int32_t batch, n_batch, kv_group;
     int32_t q_blocks_per_tile;    // ceil(q_tile / rows per workgroup)

@@ -214,7 +214,22 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         constexpr uint32_t OPEN = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 0u : 0x01010101u;
         constexpr uint32_t HIDDEN = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? T::kNegInfPair : 0u;
         const int64_t row_bytes = (int64_t)k_seq * ES;
-        if(n_steps > 0 && row_bytes % 16 == 0 && (p.mask_ld * ES) % 16 == 0
+        // bit s: some value of step s (steps >= 63 share bit 63) is not open / not hidden
+        unsigned long long not_open = 0ull, not_hidden = 0ull;
+        bool scanned = false;
+        if(n_steps > 0 && p.mask_bits != nullptr)
+        {
+            // the scan was done once for all batch entries before the launch
+            const unsigned long long *w = p.mask_bits + (int64_t)qb * (2 * kMaskBitSplits);
+#pragma unroll
+            for(int sp = 0; sp < kMaskBitSplits; ++sp)
+            {
+                not_open |= w[2 * sp];
+                not_hidden |= w[2 * sp + 1];
+            }
+            scanned = true;
+        }
+        else if(n_steps > 0 && row_bytes % 16 == 0 && (p.mask_ld * ES) % 16 == 0
                 && reinterpret_cast<uintptr_t>(p.mask) % 16 == 0
                 && p.mask_ld * ES * kQRows < (int64_t)(1 << 30))
         {
@@ -230,8 +245,6 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             const int total = n_rows * n_chunks;
             const char *mbase = static_cast<const char *>(p.mask)
                 + (int64_t)q_row0 * p.mask_ld * ES;
-            // bit s: some value of step s (steps >= 63 share bit 63) is not open / not hidden
-            unsigned long long not_open = 0ull, not_hidden = 0ull;
             // chunk tid, tid + 256, ... of the rows laid end to end: (row, c)
             // advances by 256 chunks per load without a division
             const int d_row = kThreads / n_chunks, d_c = kThreads % n_chunks;
@@ -280,6 +293,10 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             __syncthreads();
             not_open = scan_bits[0];
             not_hidden = scan_bits[1];
+            scanned = true;
+        }
+        if(scanned)
+        {
             if(not_hidden == 0ull)
             {
                 if(!p.overwrite)
@@ -1333,11 +1350,148 @@ static int launch_mode(hipStream_t stream, const PrefillParams &p, int mode,
     return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
 }
 
+// The scan of an explicit mask that every workgroup of the attention kernel
+// would do for its own 128 rows, done once for all batch entries: workgroup
+// (query block, key range) ORs what it finds in its range of 16-byte chunks
+// into one pair of words (see PrefillParams::mask_bits).  ES: bytes per mask
+// element; open / hidden: the 32-bit pattern of four (two) visible / hidden
+// elements.
+template<int ES>
+__global__ __launch_bounds__(kThreads)
+void mask_step_bits_kernel(const char *mask, int ld_bytes, int q_len, int n_chunks,
+        uint32_t open_word, uint32_t hidden_word, unsigned long long *table)
+{
+    constexpr int CHUNKS_PER_STEP = kKeys * ES / 16;
+    __shared__ unsigned long long bits[2];
+    const int tid = threadIdx.x;
+    const int qb = blockIdx.x / kMaskBitSplits;
+    const int sp = blockIdx.x % kMaskBitSplits;
+    if(tid == 0)
+    {
+        bits[0] = 0ull;
+        bits[1] = 0ull;
+    }
+    __syncthreads();
+    const int per_split = (n_chunks + kMaskBitSplits - 1) / kMaskBitSplits;
+    const int c_lo = min(sp * per_split, n_chunks);
+    const int n_loc = min(c_lo + per_split, n_chunks) - c_lo;
+    const int q_row0 = qb * kQRows;
+    const int n_rows = min(kQRows, q_len - q_row0);
+    unsigned long long not_open = 0ull, not_hidden = 0ull;
+    if(n_loc > 0)
+    {
+        const int total = n_rows * n_loc;
+        const char *mbase = mask + (int64_t)q_row0 * ld_bytes + (int64_t)c_lo * 16;
+        // chunk tid, tid + 256, ... of the rows' pieces laid end to end
+        const int d_row = kThreads / n_loc, d_c = kThreads % n_loc;
+        int row = tid / n_loc, c = tid % n_loc;
+        for(int base = 0; base < total; base += 16 * kThreads)
+        {
+            // (rows past the end re-read the last row: no branches, so that
+            // the 16 loads are in flight together)
+            u32x4 v[16];
+            int st[16];
+#pragma unroll
+            for(int u = 0; u < 16; ++u)
+            {
+                const int r = min(row, n_rows - 1);
+                st[u] = min((c_lo + c) / CHUNKS_PER_STEP, 63);
+                v[u] = *reinterpret_cast<const u32x4 *>(
+                        mbase + (uint32_t)(r * ld_bytes + c * 16));
+                row += d_row;
+                c += d_c;
+                if(c >= n_loc)
+                {
+                    c -= n_loc;
+                    row += 1;
+                }
+            }
+#pragma unroll
+            for(int u = 0; u < 16; ++u)
+            {
+                const uint32_t any1 = v[u][0] | v[u][1] | v[u][2] | v[u][3];
+                const uint32_t all1 = v[u][0] & v[u][1] & v[u][2] & v[u][3];
+                const bool open = (any1 == open_word) & (all1 == open_word);
+                const bool hidden = (any1 == hidden_word) & (all1 == hidden_word);
+                not_open |= (unsigned long long)(!open) << st[u];
+                not_hidden |= (unsigned long long)(!hidden) << st[u];
+            }
+        }
+    }
+    if(not_open != 0ull)
+    {
+        atomicOr(&bits[0], not_open);
+    }
+    if(not_hidden != 0ull)
+    {
+        atomicOr(&bits[1], not_hidden);
+    }
+    __syncthreads();
+    if(tid == 0)
+    {
+        table[2 * (int64_t)blockIdx.x] = bits[0];
+        table[2 * (int64_t)blockIdx.x + 1] = bits[1];
+    }
+}
+
+// Masks below this size are scanned by the attention kernel's workgroups
+// themselves: the launch of the scan would cost more than it saves.
+constexpr int64_t kMaskScanLaunchBytes = 1 << 20;
+
+// One-tile calls with an explicit mask and a scratch buffer of the caller's
+// (the reference's scratch_logsumexp tile): scan the mask once, into the
+// scratch, instead of once per batch entry.  Leaves p.mask_bits null when the
+// conditions of the kernel's own scan do not hold or the scratch is too small.
+template<typename T>
+static int scan_mask_once(hipStream_t stream, PrefillParams &p, int mode,
+        void *scratch, size_t scratch_bytes)
+{
+    const bool additive = mode == NNTILE_HIP_MASK_ADDITIVE;
+    if((!additive && mode != NNTILE_HIP_MASK_BOOL) || scratch == nullptr
+            || p.n_q_tiles != 1 || p.n_kv_tiles != 1 || p.mask == nullptr)
+    {
+        return NNTILE_HIP_OK;
+    }
+    const int64_t es = additive ? 2 : 1;
+    const int64_t row_bytes = p.k_seq * es;
+    const int64_t table_bytes = (int64_t)p.q_blocks_per_tile * kMaskBitSplits * 16;
+    if(row_bytes % 16 != 0 || (p.mask_ld * es) % 16 != 0
+            || reinterpret_cast<uintptr_t>(p.mask) % 16 != 0
+            || p.mask_ld * es * kQRows >= (int64_t)(1 << 30)
+            || reinterpret_cast<uintptr_t>(scratch) % 8 != 0
+            || (int64_t)scratch_bytes < table_bytes
+            || p.q_seq * row_bytes < kMaskScanLaunchBytes || p.batch < 2)
+    {
+        return NNTILE_HIP_OK;
+    }
+    auto *table = static_cast<unsigned long long *>(scratch);
+    const dim3 grid((unsigned)(p.q_blocks_per_tile * kMaskBitSplits));
+    if(additive)
+    {
+        hipLaunchKernelGGL((mask_step_bits_kernel<2>), grid, dim3(kThreads), 0, stream,
+                static_cast<const char *>(p.mask), (int)(p.mask_ld * es), (int)p.q_seq,
+                (int)(row_bytes / 16), 0u, T::kNegInfPair, table);
+    }
+    else
+    {
+        hipLaunchKernelGGL((mask_step_bits_kernel<1>), grid, dim3(kThreads), 0, stream,
+                static_cast<const char *>(p.mask), (int)(p.mask_ld * es), (int)p.q_seq,
+                (int)(row_bytes / 16), 0x01010101u, 0u, table);
+    }
+    if(hipGetLastError() != hipSuccess)
+    {
+        return NNTILE_HIP_ELAUNCH;
+    }
+    p.mask_bits = table;
+    return NNTILE_HIP_OK;
+}
+
 // Host launcher shared by the tile and grid entry points.  p must be fully
-// filled except for the block counts and the remap flag.
+// filled except for the block counts and the remap flag.  scan_scratch: device
+// memory the call may use for a scan of an explicit mask (may be null).
 template<typename T>
 int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
-        int mode)
+        int mode, void *scan_scratch, size_t scan_scratch_bytes)
 {
     p.q_blocks_per_tile = (int)((p.q_tile + kQRows - 1) / kQRows);
     p.k_blocks_per_tile = (int)((p.k_tile + kKeys - 1) / kKeys);
@@ -1345,6 +1499,12 @@ int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
     if(n_wg <= 0 || n_wg > 0x7fffffff)
     {
         return NNTILE_HIP_EINVAL;
+    }
+    p.mask_bits = nullptr;
+    const int scan_rc = scan_mask_once<T>(stream, p, mode, scan_scratch, scan_scratch_bytes);
+    if(scan_rc != NNTILE_HIP_OK)
+    {
+        return scan_rc;
     }
     p.xcd_remap = (p.batch % 8 == 0) ? 1 : 0;
     const dim3 grid((unsigned)n_wg);
@@ -1361,7 +1521,7 @@ int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
     }
 }
 
-template int launch_prefill_16bit<Bf16>(hipStream_t, PrefillParams &, int, int);
-template int launch_prefill_16bit<Fp16>(hipStream_t, PrefillParams &, int, int);
+template int launch_prefill_16bit<Bf16>(hipStream_t, PrefillParams &, int, int, void *, size_t);
+template int launch_prefill_16bit<Fp16>(hipStream_t, PrefillParams &, int, int, void *, size_t);
 
 } // namespace nntile_hip

@@ -207,14 +207,18 @@ def _dev(*tensors):
             raise ValueError("tiles must be contiguous device tensors")
 
 
-def flash_sdpa_fwd(K, Q, mask, lse, V, A, stream=None):
+def flash_sdpa_fwd(K, Q, mask, lse, V, A, scratch_lse=None, scratch_A=None, stream=None):
     """One square tile with an additive mask: the reference kernel call
-    (execute_graph) with its argument order K, Q, mask, lse, V, A."""
-    _dev(K, Q, mask, lse, V, A)
+    (execute_graph) with its argument order K, Q, mask, lse, V, A.
+    scratch_lse ([batch, seq] fp32) and scratch_A (like A) are the reference's
+    scratch tiles; the call may overwrite them."""
+    _dev(K, Q, mask, lse, V, A, scratch_lse, scratch_A)
     batch, seq, head = Q.shape
+    if scratch_lse is not None and scratch_lse.numel() * scratch_lse.element_size() < 4 * batch * seq:
+        raise ValueError("scratch_lse is smaller than a logsumexp tile")
     fn = getattr(lib(), "nntile_hip_flash_sdpa_fwd_" + dtype_name(Q))
     _check(fn(_stream(stream), seq, head, batch, _ptr(K), _ptr(Q), _ptr(mask),
-              None, _ptr(V), None, _ptr(lse), _ptr(A)), "flash_sdpa_fwd")
+              _ptr(scratch_lse), _ptr(V), _ptr(scratch_A), _ptr(lse), _ptr(A)), "flash_sdpa_fwd")
 
 
 def _tile_args(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, q_pos0,
@@ -330,6 +334,26 @@ class Plan:
         rc = self._fn(_stream(stream), ctypes.byref(self._args), *self._extra)
         if rc != OK:
             raise SdpaError(rc, self._what)
+
+
+class FlashPlan:
+    """flash_sdpa_fwd (the reference kernel call, scratch tiles included)
+    prepared once; `launch` costs one foreign call."""
+
+    def __init__(self, K, Q, mask, lse, V, A, scratch_lse=None, scratch_A=None):
+        _dev(K, Q, mask, lse, V, A, scratch_lse, scratch_A)
+        batch, seq, head = Q.shape
+        if scratch_lse is not None and scratch_lse.numel() * scratch_lse.element_size() < 4 * batch * seq:
+            raise ValueError("scratch_lse is smaller than a logsumexp tile")
+        self._fn = getattr(lib(), "nntile_hip_flash_sdpa_fwd_" + dtype_name(Q))
+        self._args = (seq, head, batch, _ptr(K), _ptr(Q), _ptr(mask), _ptr(scratch_lse), _ptr(V),
+                      _ptr(scratch_A), _ptr(lse), _ptr(A))
+        self._keep = (K, Q, mask, lse, V, A, scratch_lse, scratch_A)
+
+    def launch(self, stream=None):
+        rc = self._fn(_stream(stream), *self._args)
+        if rc != OK:
+            raise SdpaError(rc, "flash_sdpa_fwd")
 
 
 def plan_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq, q_tile, k_tile,

@@ -168,6 +168,20 @@ Handle::Handle(std::size_t size): nbytes(size)
     stamp = std::make_shared<std::atomic<std::uint64_t>>(next_stamp());
 }
 
+Handle worker_scratch(std::size_t size)
+{
+    static std::mutex guard;
+    static Handle buffer;
+    std::lock_guard<std::mutex> lock(guard);
+    if(buffer.size() < size)
+    {
+        // tasks already enqueued may still use the old buffer
+        task_wait_for_all();
+        buffer = Handle(size < (std::size_t(1) << 20) ? (std::size_t(1) << 20) : size);
+    }
+    return buffer;
+}
+
 void Handle::mark_written() const
 {
     if(stamp)
@@ -438,10 +452,13 @@ void flash_sdpa_fwd_cudnn_async(const Tile<T> &K, const Tile<T> &Q,
     const Index head = K.shape[0];
     // n_batch * kv_group_size * n_head_kv -> one flat batch
     const Index batch = K.shape[2] * K.shape[3] * K.shape[4];
-    // The reference registers two scratch handles per call; the HIP body
-    // never touches them (the merge is fused), so they are empty here and
-    // exist only to keep the submit signature.
-    starpu::VariableHandle scratch_logsumexp, scratch_A;
+    // The reference registers two scratch handles per call
+    // (src/tile/flash_sdpa_fwd_cudnn.cc:176-195).  The HIP body fuses the
+    // merge and needs neither for it; it scans a large mask once into the
+    // first (seq * batch floats).  The second stays empty.
+    starpu::VariableHandle scratch_logsumexp = starpu::worker_scratch(
+            sizeof(float) * static_cast<std::size_t>(seq) * static_cast<std::size_t>(batch));
+    starpu::VariableHandle scratch_A;
     starpu::flash_sdpa_fwd_cudnn<T>().submit(seq, head, batch, K, Q, mask,
             logsumexp, V, A, scratch_logsumexp, scratch_A);
     scratch_logsumexp.unregister_submit();

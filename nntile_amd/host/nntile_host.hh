@@ -98,6 +98,13 @@ public:
 
 using VariableHandle = Handle;
 
+//! Scratch memory of the one worker this stand-in has: at least `size` bytes,
+//! valid until the next call asks for more.  Under StarPU a STARPU_SCRATCH
+//! handle costs a task no allocation (the runtime keeps such buffers per
+//! worker); a Handle(size) here would call hipMalloc per task.  All bodies run
+//! in order on one stream, so consecutive tasks can share the buffer.
+Handle worker_scratch(std::size_t size);
+
 //! Stream every codelet body of this process enqueues on
 void *get_local_stream();
 void task_wait_for_all();

@@ -1,0 +1,85 @@
+"""The reference-signature call with its scratch tile: a large additive mask
+is scanned once per call by a small kernel of its own (into the scratch
+logsumexp tile) instead of once per batch entry by the attention kernel's
+workgroups.  Both ways produce the same bits about the mask, so the results
+must be identical bit for bit, whatever the mask holds; and they must agree
+with the CPU checker."""
+import numpy as np
+import pytest
+import torch
+
+from nntile_amd import hip_sdpa, synth
+from . import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _mask(kind, seq):
+    i = np.arange(seq)[:, None]
+    j = np.arange(seq)[None, :]
+    if kind == "causal":
+        return j <= i
+    if kind == "full":
+        return np.ones((seq, seq), bool)
+    if kind == "window":
+        return np.abs(i - j) <= 100
+    if kind == "upper":                 # every query of the first blocks sees nothing
+        return (j <= i) & (i >= 200)
+    if kind == "holes":                 # open but for single hidden elements
+        m = np.ones((seq, seq), bool)
+        m[5, 70] = m[seq - 1, 0] = m[130, seq - 1] = False
+        m[:, 0] = True
+        return m
+    rng = np.random.Generator(np.random.PCG64(7))
+    m = rng.random((seq, seq)) < 0.5
+    m[:, 0] = True
+    return m
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("kind", ["causal", "full", "window", "upper", "holes", "random"])
+@pytest.mark.parametrize("seq,head,batch", [(1024, 64, 2), (768, 128, 3), (4160, 64, 2)])
+def test_scan_once_equals_scan_per_workgroup(oracle, dtype, kind, seq, head, batch):
+    # (4160 = 65 key steps: steps from 63 on share one bit of the scan)
+    print("case", dtype, kind, seq, head, batch, flush=True)
+    (Q, K, V), f32 = H.make_qkv(31, batch, seq, seq, head, dtype)
+    vis = _mask(kind, seq)
+    m = H.additive_mask(vis, dtype).cuda()
+    Kd, Qd, Vd = K.cuda(), Q.cuda(), V.cuda()
+    outs = []
+    for with_scratch in (False, True):
+        lse, A = H.fresh_outputs(batch, seq, head, dtype)
+        scratch = torch.full((batch, seq), float("nan"), device="cuda") if with_scratch else None
+        hip_sdpa.flash_sdpa_fwd(Kd, Qd, m, lse, Vd, A, scratch_lse=scratch)
+        torch.cuda.synchronize()
+        outs.append((lse, A))
+    (lse0, A0), (lse1, A1) = outs
+    assert torch.equal(lse0, lse1)
+    rows = torch.from_numpy(vis.any(axis=1)).cuda()
+    assert torch.equal(A0[:, rows].view(torch.int16), A1[:, rows].view(torch.int16))
+    if seq <= 1024:
+        qf, kf, vf = f32
+        want, want_lse = oracle.sdpa_vanilla(kf, qf, vf, vis)
+        r = vis.any(axis=1)
+        assert H.rel_fro(H.to_np(A1)[:, r], want[:, r]) < H.TOL[dtype]
+        assert H.rel_fro(H.to_np(lse1)[:, r], want_lse[:, r]) < H.TOL[dtype]
+        assert np.all(np.isneginf(H.to_np(lse1)[:, ~r]))
+
+
+def test_codelet_body_uses_its_scratch_buffer(oracle):
+    # buffer 6 of the codelet is the scratch logsumexp tile; with and without
+    # it the task's result is the same
+    dtype, seq, head, batch = "bf16", 1024, 64, 4
+    (Q, K, V), _ = H.make_qkv(33, batch, seq, seq, head, dtype)
+    m = H.additive_mask(synth.causal_mask(seq, seq), dtype).cuda()
+    Kd, Qd, Vd = K.cuda(), Q.cuda(), V.cuda()
+    outs = []
+    for with_scratch in (False, True):
+        lse, A = H.fresh_outputs(batch, seq, head, dtype)
+        s_lse = torch.empty((batch, seq), device="cuda") if with_scratch else None
+        s_A = torch.empty_like(A) if with_scratch else None
+        hip_sdpa.flash_sdpa_fwd_codelet(Kd, Qd, m, lse, Vd, A, s_lse, s_A)
+        torch.cuda.synchronize()
+        outs.append((lse, A))
+    assert torch.equal(outs[0][0], outs[1][0])
+    assert torch.equal(outs[0][1].view(torch.int16), outs[1][1].view(torch.int16))
