@@ -900,11 +900,13 @@ int launch_prefill_fp32(hipStream_t stream, PrefillParams &p, int head, int mode
     {
         return NNTILE_HIP_EUNSUPPORTED;
     }
-    // with fewer 128-query workgroups than CUs, 32-query workgroups whose
-    // wavefronts share the keys instead
+    // with fewer 128-query workgroups than CUs, or query tiles so short that
+    // half of such a workgroup's wavefronts would have no rows (the new tokens
+    // of a decode step), 32-query workgroups whose wavefronts share the keys
+    // instead
     const int64_t n_wide = (int64_t)p.batch * p.n_q_tiles
         * ((p.q_tile + kQRows32 - 1) / kQRows32);
-    const bool split = n_wide < 256;
+    const bool split = n_wide < 256 || p.q_tile <= 64;
     const int q_rows = split ? 32 : kQRows32;
     p.q_blocks_per_tile = (int)((p.q_tile + q_rows - 1) / q_rows);
     const int64_t n_wg = (int64_t)p.batch * p.n_q_tiles * p.q_blocks_per_tile;
