@@ -124,8 +124,25 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
     const int col = lane & 15;       // row (query) within the wavefront
     const int quad = lane >> 4;      // 0..3
 
-    const int split = blockIdx.x % p.n_splits;
-    const int unit = blockIdx.x / p.n_splits;        // nb + n_batch*hkv
+    // Workgroups are dealt round-robin to the 8 XCDs.  All key splits of a
+    // unit go to one XCD, and so do the workgroups of the merge kernel that
+    // read the unit's partials: the partials then stay within one L2
+    // (cfg4: 50.6 -> 50.0 us per step).
+    int split, unit;
+    {
+        const int units = p.n_batch * p.n_head_kv;
+        if(units % 8 == 0)
+        {
+            const int x = blockIdx.x & 7, j = blockIdx.x >> 3;
+            unit = (j / p.n_splits) * 8 + x;
+            split = j % p.n_splits;
+        }
+        else
+        {
+            split = blockIdx.x % p.n_splits;
+            unit = blockIdx.x / p.n_splits;        // nb + n_batch*hkv
+        }
+    }
     const int nb = unit % p.n_batch;
     const int hkv = unit / p.n_batch;
 
@@ -555,7 +572,23 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
     constexpr int TPR = HEAD / 4;               // threads per row
     constexpr int ROWS_PER_WG = 256 / TPR;
     const int64_t total_rows = (int64_t)p.n_batch * p.n_head_kv * p.rows;
-    const int64_t grow = (int64_t)blockIdx.x * ROWS_PER_WG + threadIdx.x / TPR;
+    // (the unit's row blocks on the XCD that computed its partials)
+    int64_t grow;
+    {
+        const int units = p.n_batch * p.n_head_kv;
+        const int blocks_per_unit = (p.rows + ROWS_PER_WG - 1) / ROWS_PER_WG;
+        if(units % 8 == 0 && p.rows % ROWS_PER_WG == 0)
+        {
+            const int x = blockIdx.x & 7, j = blockIdx.x >> 3;
+            const int u = (j / blocks_per_unit) * 8 + x;
+            const int rb = j % blocks_per_unit;
+            grow = (int64_t)u * p.rows + rb * ROWS_PER_WG + threadIdx.x / TPR;
+        }
+        else
+        {
+            grow = (int64_t)blockIdx.x * ROWS_PER_WG + threadIdx.x / TPR;
+        }
+    }
     if(grow >= total_rows)
     {
         return;
