@@ -414,11 +414,27 @@ def bench_backward(cfg, steps, warmup):
 
     wall, dev = time_steps(step, steps, warmup)
     fl = 2.5 * cfg.flops()
+    # the same gradients over the reference's tiling (separately allocated
+    # sequence tiles, gradients added to the tiles as the reference's
+    # operation does): one call for all tile pairs
+    tile = cfg.seq_tile
+    cut = lambda t: [t[:, s:s + tile].contiguous() for s in range(0, cfg.q_seq, tile)]
+    Kt, Qt, Vt, At, Gt, Lt = (cut(t) for t in (K, Q, V, A, G, lse))
+    dKt, dQt, dVt = ([torch.zeros_like(t) for t in Qt] for _ in range(3))
+    plan = h.plan_bwd_grid(Kt, Qt, Vt, At, Gt, Lt, dKt, dQt, dVt, cfg.q_seq, cfg.q_seq, tile, tile,
+                           h.MASK_CAUSAL, ws)
+    wall_t, dev_t = time_steps(plan.launch, steps, warmup)
     return {"workload": cfg.name, "ms_per_step": round(wall, 4), "flops_per_step": fl,
             "what": "backward of %s in one call (row dots + one launch for dQ, dK, dV), analytic "
                     "causal mask, gradients written; 2.5 x the forward's causal-exact FLOPs" % cfg.name,
             "roofline": roofline("mfma", "sdpa_bwd_rowdot_kernel + sdpa_bwd_kernel<bf16,128,causal>",
-                                 fl, dev, PEAK_BF16_TFLOPS, "TFLOP/s")}
+                                 fl, dev, PEAK_BF16_TFLOPS, "TFLOP/s"),
+            "reference_tiling": {
+                "what": "the same over %d x %d separately allocated tiles of %d rows, gradients "
+                        "added to the tiles: nntile_hip_sdpa_bwd_grid, one call for all tile pairs "
+                        "(row dots per query tile + one launch)" % (len(Qt), len(Kt), tile),
+                "ms_per_step": round(wall_t, 4), "device_ms_per_step": round(dev_t, 4),
+                "frac_of_peak": round(fl / (dev_t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}}
 
 
 def bench_rope(cfg, steps, warmup):

@@ -208,6 +208,47 @@ int nntile_hip_sdpa_fwd_grid_bf16(void *stream, const nntile_hip_sdpa_grid_args 
 int nntile_hip_sdpa_fwd_grid_fp16(void *stream, const nntile_hip_sdpa_grid_args *args);
 int nntile_hip_sdpa_fwd_grid_fp32(void *stream, const nntile_hip_sdpa_grid_args *args);
 
+/* The backward over the same grid of tiles in one call: what
+ * tensor::flash_sdpa_bwd_cudnn_async (src/tensor/flash_sdpa_bwd_cudnn.cc:
+ * 172-247) computes by submitting one task per (dQ tile, key tile) pair, for
+ * one (batch, head) slab whose tiles are all resident on this GPU.  dQ of a
+ * query tile sums over every key tile, dK and dV of a key tile over every
+ * query tile (and, with kv_group > 1, over the query heads of the group); the
+ * sums are carried in fp32 and rounded once, where the pair-by-pair form
+ * rounds after every pair.  Tiles are separate allocations laid out as in
+ * nntile_hip_sdpa_grid_args; A, dA, dQ and lse follow the query tiles, dK and
+ * dV the key tiles.  q_tile and k_tile must be multiples of 128 (the rows a
+ * workgroup owns) unless the axis has a single tile; other sizes get
+ * NNTILE_HIP_EUNSUPPORTED and are served pair by pair through
+ * nntile_hip_sdpa_bwd_tile_*.  Only the analytic masks (NONE, CAUSAL).
+ * flags: NNTILE_HIP_SDPA_OVERWRITE writes the gradients instead of adding to
+ * them.  workspace: q_seq*batch floats of device memory, 4-byte aligned,
+ * private to the call until it has completed. */
+#define NNTILE_HIP_SDPA_BWD_MAX_TILES 32
+
+typedef struct nntile_hip_sdpa_bwd_grid_args
+{
+    int64_t q_seq, k_seq, q_tile, k_tile, head;
+    int64_t batch, n_batch, kv_group;
+    int32_t mask_mode, n_q_tiles, n_kv_tiles, flags;
+    int64_t q_pos0, k_pos0, causal_offset;
+    const void *K[NNTILE_HIP_SDPA_BWD_MAX_TILES];
+    const void *V[NNTILE_HIP_SDPA_BWD_MAX_TILES];
+    const void *Q[NNTILE_HIP_SDPA_BWD_MAX_TILES];
+    const void *A[NNTILE_HIP_SDPA_BWD_MAX_TILES];
+    const void *dA[NNTILE_HIP_SDPA_BWD_MAX_TILES];
+    const float *lse[NNTILE_HIP_SDPA_BWD_MAX_TILES];
+    void *dK[NNTILE_HIP_SDPA_BWD_MAX_TILES];
+    void *dQ[NNTILE_HIP_SDPA_BWD_MAX_TILES];
+    void *dV[NNTILE_HIP_SDPA_BWD_MAX_TILES];
+    void *workspace;
+    size_t workspace_bytes;
+} nntile_hip_sdpa_bwd_grid_args;
+
+size_t nntile_hip_sdpa_bwd_grid_workspace_bytes(const nntile_hip_sdpa_bwd_grid_args *args);
+int nntile_hip_sdpa_bwd_grid_bf16(void *stream, const nntile_hip_sdpa_bwd_grid_args *args);
+int nntile_hip_sdpa_bwd_grid_fp16(void *stream, const nntile_hip_sdpa_bwd_grid_args *args);
+
 /* ---- 4. short-query / long-key decode ----------------------------------------
  * The shape of LlamaAttention.forward_dynamic
  * (wrappers/python/nntile/model/llama_attention.py:627-760), which in the

@@ -19,6 +19,9 @@ int launch_decode_16bit(hipStream_t stream, DecodeParams &p, int head, int mode)
 int decode_choose_splits(int units, int n_steps);
 template<typename T>
 int launch_bwd_16bit(hipStream_t stream, const BwdParams &p, int head, int mode);
+template<typename T>
+int launch_bwd_grid_16bit(hipStream_t stream, const BwdGridParams &p,
+        const void *const *A_tiles, int n_q_tiles, int head, int mode);
 size_t decode_workspace_bytes(int units, int n_splits, int rows, int head);
 size_t decode_partial_o_bytes(int units, int n_splits, int rows, int head);
 
@@ -204,6 +207,91 @@ static int bwd_call(DType dt, void *stream, const nntile_hip_sdpa_bwd_args *a)
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dt == DType::bf16 ? launch_bwd_16bit<Bf16>(s, p, (int)a->head, a->mask_mode)
         : launch_bwd_16bit<Fp16>(s, p, (int)a->head, a->mask_mode);
+}
+
+static int bwd_grid_call(DType dt, void *stream, const nntile_hip_sdpa_bwd_grid_args *a)
+{
+    if(a == nullptr || a->q_seq <= 0 || a->k_seq <= 0 || a->q_tile <= 0
+            || a->k_tile <= 0 || a->head <= 0 || a->batch <= 0
+            || a->n_batch <= 0 || a->kv_group <= 0
+            || a->batch % (a->n_batch * a->kv_group) != 0
+            || a->batch > 0x7fffffff || a->q_seq > 0x7fffffff
+            || a->k_seq > 0x7fffffff
+            || a->n_q_tiles <= 0 || a->n_q_tiles > NNTILE_HIP_SDPA_BWD_MAX_TILES
+            || a->n_kv_tiles <= 0 || a->n_kv_tiles > NNTILE_HIP_SDPA_BWD_MAX_TILES)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(a->mask_mode != NNTILE_HIP_MASK_NONE && a->mask_mode != NNTILE_HIP_MASK_CAUSAL)
+    {
+        return mode_ok(a->mask_mode) ? NNTILE_HIP_EUNSUPPORTED : NNTILE_HIP_EINVAL;
+    }
+    // the tile counts must match the extents
+    if((a->q_seq + a->q_tile - 1) / a->q_tile != a->n_q_tiles
+            || (a->k_seq + a->k_tile - 1) / a->k_tile != a->n_kv_tiles)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(a->head != 32 && a->head != 64 && a->head != 128)
+    {
+        return NNTILE_HIP_EUNSUPPORTED;
+    }
+    // a workgroup's 128 rows must not straddle two allocations
+    if((a->n_q_tiles > 1 && a->q_tile % 128 != 0) || (a->n_kv_tiles > 1 && a->k_tile % 128 != 0))
+    {
+        return NNTILE_HIP_EUNSUPPORTED;
+    }
+    const size_t d_bytes = (size_t)a->q_seq * (size_t)a->batch * sizeof(float);
+    if(a->workspace == nullptr || a->workspace_bytes < d_bytes
+            || (reinterpret_cast<uintptr_t>(a->workspace) & 3u) != 0)
+    {
+        return NNTILE_HIP_EWORKSPACE;
+    }
+    BwdGridParams p;
+    std::memset(static_cast<void *>(&p), 0, sizeof(p));
+    p.q_seq = a->q_seq;
+    p.k_seq = a->k_seq;
+    p.q_tile = a->q_tile;
+    p.k_tile = a->k_tile;
+    p.q_pos0 = a->q_pos0;
+    p.k_pos0 = a->k_pos0;
+    p.causal_offset = a->causal_offset;
+    p.D = static_cast<float *>(a->workspace);
+    p.batch = (int32_t)a->batch;
+    p.n_batch = (int32_t)a->n_batch;
+    p.kv_group = (int32_t)a->kv_group;
+    p.overwrite = (a->flags & NNTILE_HIP_SDPA_OVERWRITE) ? 1 : 0;
+    p.scale = 1.0f / sqrtf(static_cast<float>(a->head));
+    for(int t = 0; t < a->n_kv_tiles; ++t)
+    {
+        if(a->K[t] == nullptr || a->V[t] == nullptr || a->dK[t] == nullptr
+                || a->dV[t] == nullptr || !aligned16(a->K[t]) || !aligned16(a->V[t])
+                || !aligned16(a->dK[t]) || !aligned16(a->dV[t]))
+        {
+            return NNTILE_HIP_EINVAL;
+        }
+        p.Kt[t] = a->K[t];
+        p.Vt[t] = a->V[t];
+        p.dKt[t] = a->dK[t];
+        p.dVt[t] = a->dV[t];
+    }
+    for(int t = 0; t < a->n_q_tiles; ++t)
+    {
+        if(a->Q[t] == nullptr || a->A[t] == nullptr || a->dA[t] == nullptr
+                || a->lse[t] == nullptr || a->dQ[t] == nullptr || !aligned16(a->Q[t])
+                || !aligned16(a->A[t]) || !aligned16(a->dA[t]) || !aligned16(a->dQ[t]))
+        {
+            return NNTILE_HIP_EINVAL;
+        }
+        p.Qt[t] = a->Q[t];
+        p.dAt[t] = a->dA[t];
+        p.lset[t] = a->lse[t];
+        p.dQt[t] = a->dQ[t];
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dt == DType::bf16
+        ? launch_bwd_grid_16bit<Bf16>(s, p, a->A, a->n_q_tiles, (int)a->head, a->mask_mode)
+        : launch_bwd_grid_16bit<Fp16>(s, p, a->A, a->n_q_tiles, (int)a->head, a->mask_mode);
 }
 
 static int flash_bwd_call(DType dt, void *stream, int64_t seq, int64_t head,
@@ -850,6 +938,25 @@ size_t nntile_hip_sdpa_bwd_workspace_bytes(const nntile_hip_sdpa_bwd_args *a)
         bytes += (size_t)((a->q_seq + 63) / 64) * (size_t)((a->k_seq + 63) / 64);
     }
     return bytes;
+}
+
+size_t nntile_hip_sdpa_bwd_grid_workspace_bytes(const nntile_hip_sdpa_bwd_grid_args *a)
+{
+    if(a == nullptr || a->q_seq <= 0 || a->batch <= 0)
+    {
+        return 0;
+    }
+    return (size_t)a->q_seq * (size_t)a->batch * sizeof(float);
+}
+
+int nntile_hip_sdpa_bwd_grid_bf16(void *stream, const nntile_hip_sdpa_bwd_grid_args *args)
+{
+    return bwd_grid_call(DType::bf16, stream, args);
+}
+
+int nntile_hip_sdpa_bwd_grid_fp16(void *stream, const nntile_hip_sdpa_bwd_grid_args *args)
+{
+    return bwd_grid_call(DType::fp16, stream, args);
 }
 
 int nntile_hip_sdpa_bwd_tile_bf16(void *stream, const nntile_hip_sdpa_bwd_args *args)

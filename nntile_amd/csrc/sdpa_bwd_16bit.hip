@@ -289,8 +289,12 @@ void sdpa_bwd_rowdot_kernel(const void *dA, const void *A, float *D, int64_t row
     }
 }
 
-template<typename T, int HEAD, int MODE>
-__device__ __forceinline__ void sdpa_bwd_dq_body(const BwdParams &p, unsigned wg,
+// GRID: the rows of both sequence axes live in separately allocated tiles
+// (BwdGridParams); a workgroup's own 128 rows lie in one tile and every 64-row
+// step of the other axis does too, because tile sizes are multiples of 128.
+template<typename T, int HEAD, int MODE, bool GRID>
+__device__ __forceinline__ void sdpa_bwd_dq_body(
+        const std::conditional_t<GRID, BwdGridParams, BwdParams> &p, unsigned wg,
         char *lds_k0, char *lds_k1, char *lds_v0, char *lds_v1)
 {
     typedef typename T::vec8 vec8;
@@ -316,13 +320,31 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(const BwdParams &p, unsigned wg
     const int q_seq = (int)p.q_seq, k_seq = (int)p.k_seq;
     const int my_q = q_row0 + wave * 32 + col;
     const bool q_ok = my_q < q_seq;
-    const int64_t q_off = ((int64_t)b * q_seq + (q_ok ? my_q : 0)) * HEAD;
+    // the lane's query: its row within the allocation that holds it (of Q, dA,
+    // dQ, and of lse without the head axis), and its place among the row dots
+    int64_t q_elem = (int64_t)b * q_seq + (q_ok ? my_q : 0), d_idx = q_elem;
+    const void *Q_own = p.Q, *dA_own = p.dA;
+    void *dQ_own = p.dQ;
+    const float *lse_own = p.lse;
+    if constexpr(GRID)
+    {
+        const int q_tile = (int)p.q_tile;
+        const int tq = q_row0 / q_tile, t0 = tq * q_tile;
+        const int rows_t = min(q_tile, q_seq - t0);
+        q_elem = (int64_t)b * rows_t + ((q_ok ? my_q : q_row0) - t0);
+        d_idx = (int64_t)p.batch * t0 + q_elem;
+        Q_own = p.Qt[tq];
+        dA_own = p.dAt[tq];
+        dQ_own = p.dQt[tq];
+        lse_own = p.lset[tq];
+    }
+    const int64_t q_off = q_elem * HEAD;
 
     // Q and dA fragments (B operands); the row dot D = dA . A of the query
     vec8 qf[KSTEPS], gf[KSTEPS];
     {
-        const uint16_t *qs = static_cast<const uint16_t *>(p.Q) + q_off + half * 8;
-        const uint16_t *gs = static_cast<const uint16_t *>(p.dA) + q_off + half * 8;
+        const uint16_t *qs = static_cast<const uint16_t *>(Q_own) + q_off + half * 8;
+        const uint16_t *gs = static_cast<const uint16_t *>(dA_own) + q_off + half * 8;
 #pragma unroll
         for(int ks = 0; ks < KSTEPS; ++ks)
         {
@@ -337,8 +359,8 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(const BwdParams &p, unsigned wg
             gf[ks] = __builtin_bit_cast(vec8, g);
         }
     }
-    const float d_row = q_ok ? p.D[(int64_t)b * q_seq + my_q] : 0.0f;
-    const float lse_q = q_ok ? p.lse[(int64_t)b * q_seq + my_q] : neg_inf();
+    const float d_row = q_ok ? p.D[d_idx] : 0.0f;
+    const float lse_q = q_ok ? lse_own[q_elem] : neg_inf();
     // exponent offset in log2 units; a row that saw nothing has P = 0
     const float lse2 = (lse_q == neg_inf()) ? __builtin_huge_valf() : lse_q * kLog2e;
 
@@ -407,11 +429,25 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(const BwdParams &p, unsigned wg
     {
         const int row0 = g * kBwdStep;
         const int last = min(kBwdStep, k_seq - row0) - 1;
+        const char *Kg, *Vg;        // the step's first row of the entry
+        if constexpr(GRID)
+        {
+            const int k_tile = (int)p.k_tile;
+            const int tk = row0 / k_tile, t0 = tk * k_tile;
+            const int64_t off = ((int64_t)kvb * min(k_tile, k_seq - t0) + (row0 - t0)) * RB;
+            Kg = static_cast<const char *>(p.Kt[tk]) + off;
+            Vg = static_cast<const char *>(p.Vt[tk]) + off;
+        }
+        else
+        {
+            Kg = Kb + (int64_t)row0 * RB;
+            Vg = Vb + (int64_t)row0 * RB;
+        }
         char *kdst = kdst_base + wave_u * LOADS_PER_WAVE * 1024;
         char *vdst = vdst_base + wave_u * LOADS_PER_WAVE * 1024;
         const uint32_t back = (uint32_t)(max(ld_row0 + i * ROWS_PER_LOAD - last, 0) * RB);
-        load_to_lds16<0, false>(Kb + (int64_t)row0 * RB, ld_goff[i] - back, kdst + i * 1024);
-        load_to_lds16<0, false>(Vb + (int64_t)row0 * RB, ld_goff[i] - back, vdst + i * 1024);
+        load_to_lds16<0, false>(Kg, ld_goff[i] - back, kdst + i * 1024);
+        load_to_lds16<0, false>(Vg, ld_goff[i] - back, vdst + i * 1024);
     };
     auto fetch = [&](int g, char *kdst_base, char *vdst_base)
     {
@@ -612,7 +648,7 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(const BwdParams &p, unsigned wg
     {
         return;
     }
-    uint16_t *dst = static_cast<uint16_t *>(p.dQ) + q_off;
+    uint16_t *dst = static_cast<uint16_t *>(dQ_own) + q_off;
 #pragma unroll
     for(int db = 0; db < DBLOCKS; ++db)
     {
@@ -653,8 +689,9 @@ constexpr int kDkvWaves = 4;
 constexpr int kDkvThreads = kDkvWaves * 64;
 constexpr int kDkvRows = kDkvWaves * 32;        // keys per workgroup
 
-template<typename T, int HEAD, int MODE, int PART>
-__device__ __forceinline__ void sdpa_bwd_dkv_body(const BwdParams &p, unsigned wg,
+template<typename T, int HEAD, int MODE, int PART, bool GRID>
+__device__ __forceinline__ void sdpa_bwd_dkv_body(
+        const std::conditional_t<GRID, BwdGridParams, BwdParams> &p, unsigned wg,
         char *lds_q0, char *lds_q1, char *lds_g0, char *lds_g1,
         float (*lds_stat)[2][kBwdStep])
 {
@@ -684,13 +721,27 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(const BwdParams &p, unsigned w
     const int nb = kvb % p.n_batch, hkv = kvb / p.n_batch;
     const int my_k = k_row0 + wave * 32 + col;
     const bool k_ok = my_k < k_seq;
-    const int64_t k_off = ((int64_t)kvb * k_seq + (k_ok ? my_k : 0)) * HEAD;
+    // the lane's key: its row within the allocation that holds it (of K, V, dK, dV)
+    int64_t k_elem = (int64_t)kvb * k_seq + (k_ok ? my_k : 0);
+    const void *K_own = p.K, *V_own = p.V;
+    void *dK_own = p.dK, *dV_own = p.dV;
+    if constexpr(GRID)
+    {
+        const int k_tile = (int)p.k_tile;
+        const int tk = k_row0 / k_tile, t0 = tk * k_tile;
+        k_elem = (int64_t)kvb * min(k_tile, k_seq - t0) + ((k_ok ? my_k : k_row0) - t0);
+        K_own = p.Kt[tk];
+        V_own = p.Vt[tk];
+        dK_own = p.dKt[tk];
+        dV_own = p.dVt[tk];
+    }
+    const int64_t k_off = k_elem * HEAD;
 
     // K and V fragments (B operands): lane (col, half) holds head values 16*ks + 8*half..+7
     vec8 kf[KSTEPS], vf[KSTEPS];
     {
-        const uint16_t *ks_ = static_cast<const uint16_t *>(p.K) + k_off + half * 8;
-        const uint16_t *vs_ = static_cast<const uint16_t *>(p.V) + k_off + half * 8;
+        const uint16_t *ks_ = static_cast<const uint16_t *>(K_own) + k_off + half * 8;
+        const uint16_t *vs_ = static_cast<const uint16_t *>(V_own) + k_off + half * 8;
 #pragma unroll
         for(int ks = 0; ks < KSTEPS; ++ks)
         {
@@ -805,11 +856,35 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(const BwdParams &p, unsigned w
     // logsumexp and D of its queries through registers (threads 0..127)
     // (inside the loop the tile loads go between the MFMAs, one Q and one dA
     // load at a time: a wave stands still ~64 cycles per load)
+    // the allocation that holds query row0 of entry bq, the row's index in it
+    // (for lse; times HEAD for Q and dA) and in the row dots
+    struct QueryRows
+    {
+        const void *Q, *dA;
+        const float *lse;
+        int64_t elem, d_idx;
+    };
+    auto query_rows = [&](int bq, int row0) __attribute__((always_inline)) -> QueryRows
+    {
+        if constexpr(GRID)
+        {
+            const int q_tile = (int)p.q_tile;
+            const int tq = row0 / q_tile, t0 = tq * q_tile;
+            const int64_t elem = (int64_t)bq * min(q_tile, q_seq - t0) + (row0 - t0);
+            return QueryRows{p.Qt[tq], p.dAt[tq], p.lset[tq], elem, (int64_t)p.batch * t0 + elem};
+        }
+        else
+        {
+            const int64_t elem = (int64_t)bq * q_seq + row0;
+            return QueryRows{p.Q, p.dA, p.lse, elem, elem};
+        }
+    };
     auto fetch_piece = [&](int bq, int row0, int last, char *qdst_base, char *gdst_base, int j)
         __attribute__((always_inline))
     {
-        const char *Qp = static_cast<const char *>(p.Q) + ((int64_t)bq * q_seq + row0) * RB;
-        const char *Gp = static_cast<const char *>(p.dA) + ((int64_t)bq * q_seq + row0) * RB;
+        const QueryRows at = query_rows(bq, row0);
+        const char *Qp = static_cast<const char *>(at.Q) + at.elem * RB;
+        const char *Gp = static_cast<const char *>(at.dA) + at.elem * RB;
         char *qdst = qdst_base + wave_u * LPW * 1024;
         char *gdst = gdst_base + wave_u * LPW * 1024;
         const uint32_t back = (uint32_t)(max(ld_row[j] - last, 0) * RB);
@@ -821,16 +896,16 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(const BwdParams &p, unsigned w
         if(tid < 2 * kBwdStep)
         {
             const int which = tid / kBwdStep, r = tid % kBwdStep;
-            const int64_t src = (int64_t)bq * q_seq + row0 + min(r, last);
+            const QueryRows at = query_rows(bq, row0);
             float v;
             if(which == 0)
             {
-                const float l = p.lse[src];
+                const float l = at.lse[at.elem + min(r, last)];
                 v = (r > last || l == neg_inf()) ? __builtin_huge_valf() : l * kLog2e;
             }
             else
             {
-                v = r > last ? 0.0f : p.D[src];
+                v = r > last ? 0.0f : p.D[at.d_idx + min(r, last)];
             }
             stat[which][r] = v;
         }
@@ -1104,11 +1179,11 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(const BwdParams &p, unsigned w
     };
     if(DO_DK)
     {
-        store(p.dK, dk, p.scale);
+        store(dK_own, dk, p.scale);
     }
     if(DO_DV)
     {
-        store(p.dV, dv, 1.0f);
+        store(dV_own, dv, 1.0f);
     }
 }
 
@@ -1117,9 +1192,10 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(const BwdParams &p, unsigned w
 // last n_dkv dV.  A tile-pair call has fewer workgroups per gradient than the
 // chip has places (two a CU); together they fill it, and a long call loses
 // the ends of two launches.
-template<typename T, int HEAD, int MODE>
+template<typename T, int HEAD, int MODE, bool GRID>
 __global__ __launch_bounds__(kDkvThreads, 2)
-void sdpa_bwd_kernel(const BwdParams p, unsigned n_dkv, unsigned n_dq)
+void sdpa_bwd_kernel(const std::conditional_t<GRID, BwdGridParams, BwdParams> p, unsigned n_dkv,
+        unsigned n_dq)
 {
     typedef BwdTile<HEAD> G;
     static_assert(kDkvThreads == kBwdThreads, "one block size for the three parts");
@@ -1132,16 +1208,16 @@ void sdpa_bwd_kernel(const BwdParams p, unsigned n_dkv, unsigned n_dq)
     __shared__ __attribute__((aligned(16))) float lds_stat[2][2][kBwdStep];
     if(blockIdx.x < n_dkv)
     {
-        sdpa_bwd_dkv_body<T, HEAD, MODE, BWD_PART_DK>(p, blockIdx.x, lds_0, lds_1, lds_2,
+        sdpa_bwd_dkv_body<T, HEAD, MODE, BWD_PART_DK, GRID>(p, blockIdx.x, lds_0, lds_1, lds_2,
                 lds_3, lds_stat);
     }
     else if(blockIdx.x < n_dkv + n_dq)
     {
-        sdpa_bwd_dq_body<T, HEAD, MODE>(p, blockIdx.x - n_dkv, lds_0, lds_1, lds_2, lds_3);
+        sdpa_bwd_dq_body<T, HEAD, MODE, GRID>(p, blockIdx.x - n_dkv, lds_0, lds_1, lds_2, lds_3);
     }
     else
     {
-        sdpa_bwd_dkv_body<T, HEAD, MODE, BWD_PART_DV>(p, blockIdx.x - n_dkv - n_dq, lds_0,
+        sdpa_bwd_dkv_body<T, HEAD, MODE, BWD_PART_DV, GRID>(p, blockIdx.x - n_dkv - n_dq, lds_0,
                 lds_1, lds_2, lds_3, lds_stat);
     }
 }
@@ -1178,11 +1254,85 @@ static int launch_bwd_mode(hipStream_t stream, const BwdParams &p)
     {
         return NNTILE_HIP_ELAUNCH;
     }
-    hipLaunchKernelGGL((sdpa_bwd_kernel<T, HEAD, MODE>),
+    hipLaunchKernelGGL((sdpa_bwd_kernel<T, HEAD, MODE, false>),
             dim3((unsigned)(2 * n_dkv + n_dq)), dim3(kDkvThreads), 0, stream, p,
             (unsigned)n_dkv, (unsigned)n_dq);
     return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
 }
+
+// The grid form: the row dots tile by tile (each tile's A and dA are one
+// allocation, and D follows the layout of lse), then the one gradient launch.
+template<typename T, int HEAD, int MODE>
+static int launch_bwd_grid_mode(hipStream_t stream, const BwdGridParams &p,
+        const void *const *A_tiles, int n_q_tiles)
+{
+    const int64_t q_blocks = (p.q_seq + kBwdRows - 1) / kBwdRows;
+    const int64_t k_blocks = (p.k_seq + kDkvRows - 1) / kDkvRows;
+    const int64_t kv_batch = p.batch / p.kv_group;
+    const int64_t n_dq = (int64_t)p.batch * q_blocks, n_dkv = kv_batch * k_blocks;
+    if(n_dq <= 0 || n_dkv <= 0 || n_dq > 0x3fffffff || n_dkv > 0x3fffffff
+            || (int64_t)p.batch * p.q_tile * (HEAD / 8) / 256 > 0x7ffffffe)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    for(int t = 0; t < n_q_tiles; ++t)
+    {
+        const int64_t t0 = (int64_t)t * p.q_tile;
+        const int64_t rows = (int64_t)p.batch * (p.q_tile < p.q_seq - t0 ? p.q_tile : p.q_seq - t0);
+        hipLaunchKernelGGL((sdpa_bwd_rowdot_kernel<T, HEAD>),
+                dim3((unsigned)((rows * (HEAD / 8) + 255) / 256)), dim3(256), 0, stream,
+                p.dAt[t], A_tiles[t], p.D + (int64_t)p.batch * t0, rows);
+        if(hipGetLastError() != hipSuccess)
+        {
+            return NNTILE_HIP_ELAUNCH;
+        }
+    }
+    hipLaunchKernelGGL((sdpa_bwd_kernel<T, HEAD, MODE, true>),
+            dim3((unsigned)(2 * n_dkv + n_dq)), dim3(kDkvThreads), 0, stream, p,
+            (unsigned)n_dkv, (unsigned)n_dq);
+    return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
+}
+
+template<typename T, int HEAD>
+static int launch_bwd_grid_head(hipStream_t stream, const BwdGridParams &p,
+        const void *const *A_tiles, int n_q_tiles, int mode)
+{
+    switch(mode)
+    {
+        case NNTILE_HIP_MASK_NONE:
+            return launch_bwd_grid_mode<T, HEAD, NNTILE_HIP_MASK_NONE>(stream, p, A_tiles,
+                    n_q_tiles);
+        case NNTILE_HIP_MASK_CAUSAL:
+            return launch_bwd_grid_mode<T, HEAD, NNTILE_HIP_MASK_CAUSAL>(stream, p, A_tiles,
+                    n_q_tiles);
+        default:
+            return NNTILE_HIP_EINVAL;
+    }
+}
+
+// The caller has checked: every tile but the last of an axis holds q_tile /
+// k_tile rows, both multiples of 128 unless the axis is one tile.
+template<typename T>
+int launch_bwd_grid_16bit(hipStream_t stream, const BwdGridParams &p,
+        const void *const *A_tiles, int n_q_tiles, int head, int mode)
+{
+    switch(head)
+    {
+        case 32:
+            return launch_bwd_grid_head<T, 32>(stream, p, A_tiles, n_q_tiles, mode);
+        case 64:
+            return launch_bwd_grid_head<T, 64>(stream, p, A_tiles, n_q_tiles, mode);
+        case 128:
+            return launch_bwd_grid_head<T, 128>(stream, p, A_tiles, n_q_tiles, mode);
+        default:
+            return NNTILE_HIP_EUNSUPPORTED;
+    }
+}
+
+template int launch_bwd_grid_16bit<Bf16>(hipStream_t, const BwdGridParams &, const void *const *,
+        int, int, int);
+template int launch_bwd_grid_16bit<Fp16>(hipStream_t, const BwdGridParams &, const void *const *,
+        int, int, int);
 
 template<typename T, int HEAD>
 static int launch_bwd_head(hipStream_t stream, const BwdParams &p, int mode)

@@ -114,6 +114,25 @@ struct BwdParams
     float scale;
 };
 
+// The same over a grid of separately allocated tiles along the two sequence
+// axes (analytic masks only): tile t of the query axis holds rows
+// [t*q_tile, min((t+1)*q_tile, q_seq)) of every batch entry, an entry's rows
+// contiguous inside it; likewise the key axis.  The single pointers of the
+// base are unused; D holds the row dots tile after tile in the layout of lse.
+constexpr int kBwdMaxTiles = NNTILE_HIP_SDPA_BWD_MAX_TILES;
+struct BwdGridParams : BwdParams
+{
+    int64_t q_tile, k_tile;
+    const void *Kt[kBwdMaxTiles];
+    const void *Vt[kBwdMaxTiles];
+    const void *Qt[kBwdMaxTiles];
+    const void *dAt[kBwdMaxTiles];
+    const float *lset[kBwdMaxTiles];
+    void *dKt[kBwdMaxTiles];
+    void *dQt[kBwdMaxTiles];
+    void *dVt[kBwdMaxTiles];
+};
+
 // 16 bytes per lane from global memory straight into LDS: lane l reads
 // gaddr + OFF (its own address) and its bytes land at lds_dst + OFF + 16*l
 // (lds_dst is the same for the whole wavefront; it travels in M0).  Written

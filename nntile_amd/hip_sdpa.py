@@ -18,6 +18,7 @@ LIB_PATH = os.path.join(_HERE, "libnntile_hip_sdpa.so")
 
 MASK_ADDITIVE, MASK_NONE, MASK_CAUSAL, MASK_BOOL = 0, 1, 2, 3
 MAX_TILES = 64
+BWD_MAX_TILES = 32
 OVERWRITE = 1
 
 OK, EINVAL, EUNSUPPORTED, ELAUNCH, EWORKSPACE = 0, -1, -2, -3, -4
@@ -61,6 +62,21 @@ class BwdArgs(ctypes.Structure):
                 ("workspace_bytes", ctypes.c_size_t)]
 
 
+class BwdGridArgs(ctypes.Structure):
+    _fields_ = [("q_seq", _i64), ("k_seq", _i64), ("q_tile", _i64),
+                ("k_tile", _i64), ("head", _i64), ("batch", _i64),
+                ("n_batch", _i64), ("kv_group", _i64),
+                ("mask_mode", ctypes.c_int32), ("n_q_tiles", ctypes.c_int32),
+                ("n_kv_tiles", ctypes.c_int32), ("flags", ctypes.c_int32),
+                ("q_pos0", _i64), ("k_pos0", _i64), ("causal_offset", _i64),
+                ("K", _vp * BWD_MAX_TILES), ("V", _vp * BWD_MAX_TILES),
+                ("Q", _vp * BWD_MAX_TILES), ("A", _vp * BWD_MAX_TILES),
+                ("dA", _vp * BWD_MAX_TILES), ("lse", _vp * BWD_MAX_TILES),
+                ("dK", _vp * BWD_MAX_TILES), ("dQ", _vp * BWD_MAX_TILES),
+                ("dV", _vp * BWD_MAX_TILES), ("workspace", _vp),
+                ("workspace_bytes", ctypes.c_size_t)]
+
+
 class VariableInterface(ctypes.Structure):
     _fields_ = [("id", ctypes.c_int), ("ptr", ctypes.c_size_t),
                 ("dev_handle", ctypes.c_size_t), ("offset", ctypes.c_size_t),
@@ -82,6 +98,8 @@ EXPORTS = (
     + ["nntile_hip_flash_sdpa_bwd_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_sdpa_bwd_tile_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_sdpa_bwd_workspace_bytes"]
+    + ["nntile_hip_sdpa_bwd_grid_" + t for t in ("bf16", "fp16")]
+    + ["nntile_hip_sdpa_bwd_grid_workspace_bytes"]
     + ["nntile_hip_flash_sdpa_bwd_codelet_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_accumulate_attn_output_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_flash_sdpa_fwd_codelet_" + t for t in ("bf16", "fp16", "fp32")]
@@ -137,6 +155,9 @@ def lib():
             f = getattr(L, "nntile_hip_sdpa_bwd_tile_" + t)
             f.argtypes = [_vp, ctypes.POINTER(BwdArgs)]
             f.restype = ctypes.c_int
+            f = getattr(L, "nntile_hip_sdpa_bwd_grid_" + t)
+            f.argtypes = [_vp, ctypes.POINTER(BwdGridArgs)]
+            f.restype = ctypes.c_int
         for t in ("bf16", "fp16", "fp32"):
             for name in ("nntile_hip_rope_", "nntile_hip_rope_backward_"):
                 f = getattr(L, name + t)
@@ -158,6 +179,8 @@ def lib():
             f.restype = ctypes.c_int
         L.nntile_hip_sdpa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
         L.nntile_hip_sdpa_bwd_workspace_bytes.restype = ctypes.c_size_t
+        L.nntile_hip_sdpa_bwd_grid_workspace_bytes.argtypes = [ctypes.POINTER(BwdGridArgs)]
+        L.nntile_hip_sdpa_bwd_grid_workspace_bytes.restype = ctypes.c_size_t
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.argtypes = [ctypes.POINTER(TileArgs)]
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.restype = ctypes.c_size_t
         L.nntile_hip_sdpa_fwd_decode_static.argtypes = [_vp, ctypes.c_int32,
@@ -319,6 +342,64 @@ def sdpa_fwd_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq,
     fn = getattr(lib(), "nntile_hip_sdpa_fwd_grid_" + dtype_name(Q_tiles[0]))
     _check(fn(_stream(stream), ctypes.byref(a)), "sdpa_fwd_grid")
     return a
+
+
+def _bwd_grid_args(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles, dQ_tiles,
+                   dV_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, n_batch, kv_group, q_pos0,
+                   k_pos0, causal_offset, flags, workspace):
+    batch, _, head = Q_tiles[0].shape
+    if len(Q_tiles) > BWD_MAX_TILES or len(K_tiles) > BWD_MAX_TILES:
+        raise SdpaError(EINVAL, "sdpa_bwd_grid")
+    a = BwdGridArgs()
+    a.q_seq, a.k_seq, a.q_tile, a.k_tile, a.head = q_seq, k_seq, q_tile, k_tile, head
+    a.batch = batch
+    a.n_batch = batch if n_batch is None else n_batch
+    a.kv_group = kv_group
+    a.mask_mode = mask_mode
+    a.flags = flags
+    a.n_q_tiles, a.n_kv_tiles = len(Q_tiles), len(K_tiles)
+    a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
+    for i, (k, v, dk, dv) in enumerate(zip(K_tiles, V_tiles, dK_tiles, dV_tiles)):
+        a.K[i], a.V[i], a.dK[i], a.dV[i] = (t.data_ptr() for t in (k, v, dk, dv))
+    for i, ts in enumerate(zip(Q_tiles, A_tiles, dA_tiles, lse_tiles, dQ_tiles)):
+        a.Q[i], a.A[i], a.dA[i], a.lse[i], a.dQ[i] = (t.data_ptr() for t in ts)
+    a.workspace = workspace.data_ptr()
+    a.workspace_bytes = workspace.numel() * workspace.element_size()
+    return a
+
+
+def sdpa_bwd_grid(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles, dQ_tiles,
+                  dV_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, n_batch=None, kv_group=1,
+                  q_pos0=0, k_pos0=0, causal_offset=0, flags=0, workspace=None, stream=None):
+    """The backward of every (query tile, key tile) pair in one call: dQ of a
+    query tile sums over the key tiles, dK and dV of a key tile over the query
+    tiles; the gradients are added to dK, dQ, dV (written with
+    flags=OVERWRITE).  Tiles are lists of separately allocated tensors
+    [batch, rows, head] (lse: [batch, rows])."""
+    every = (*K_tiles, *Q_tiles, *V_tiles, *A_tiles, *dA_tiles, *lse_tiles, *dK_tiles,
+             *dQ_tiles, *dV_tiles)
+    _dev(*every, workspace)
+    if workspace is None:
+        workspace = torch.empty(4 * q_seq * Q_tiles[0].shape[0], dtype=torch.uint8,
+                                device=Q_tiles[0].device)
+    a = _bwd_grid_args(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles,
+                       dQ_tiles, dV_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, n_batch,
+                       kv_group, q_pos0, k_pos0, causal_offset, flags, workspace)
+    fn = getattr(lib(), "nntile_hip_sdpa_bwd_grid_" + dtype_name(Q_tiles[0]))
+    _check(fn(_stream(stream), ctypes.byref(a)), "sdpa_bwd_grid")
+
+
+def plan_bwd_grid(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles, dQ_tiles,
+                  dV_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, workspace, n_batch=None,
+                  kv_group=1, q_pos0=0, k_pos0=0, causal_offset=0, flags=0):
+    every = (*K_tiles, *Q_tiles, *V_tiles, *A_tiles, *dA_tiles, *lse_tiles, *dK_tiles,
+             *dQ_tiles, *dV_tiles, workspace)
+    _dev(*every)
+    a = _bwd_grid_args(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles,
+                       dQ_tiles, dV_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, n_batch,
+                       kv_group, q_pos0, k_pos0, causal_offset, flags, workspace)
+    fn = getattr(lib(), "nntile_hip_sdpa_bwd_grid_" + dtype_name(Q_tiles[0]))
+    return Plan(fn, a, "sdpa_bwd_grid", keep=every)
 
 
 class Plan:

@@ -1368,6 +1368,100 @@ static Index bwd_pairs(const Tensor<T> &K, const Tensor<T> &Q,
     return submitted;
 }
 
+template<typename T> struct BwdGridCall;
+template<> struct BwdGridCall<bf16_t>
+{
+    static int run(void *s, const nntile_hip_sdpa_bwd_grid_args *a) { return nntile_hip_sdpa_bwd_grid_bf16(s, a); }
+};
+template<> struct BwdGridCall<fp16_t>
+{
+    static int run(void *s, const nntile_hip_sdpa_bwd_grid_args *a) { return nntile_hip_sdpa_bwd_grid_fp16(s, a); }
+};
+
+// Whether one call can take all tile pairs of a slab: the argument block has
+// room for the tiles, and no workgroup's 128 rows straddle two tiles.
+static bool bwd_grid_fits(const TensorTraits &K, const TensorTraits &Q)
+{
+    const Index n_q = Q.grid.shape[1], n_kv = K.grid.shape[1];
+    return n_q <= NNTILE_HIP_SDPA_BWD_MAX_TILES && n_kv <= NNTILE_HIP_SDPA_BWD_MAX_TILES
+        && (n_q == 1 || Q.basetile_shape[1] % 128 == 0)
+        && (n_kv == 1 || K.basetile_shape[1] % 128 == 0);
+}
+
+// All (dQ tile, key tile) pairs of a slab of the batch grid in one call, for
+// a mask that is the causal rule or hides nothing: the sums over the pairs
+// (src/tensor/flash_sdpa_bwd_cudnn.cc:172-247) are carried in fp32 inside the
+// kernels instead of through the 16-bit gradient tiles.  Returns the calls.
+template<typename T>
+static Index bwd_grid(const Tensor<T> &K, const Tensor<T> &Q,
+        const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
+        int mask_mode, Index causal_offset, const Tensor<fp32_t> &logsumexp,
+        const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV)
+{
+    const Index n_q = Q.grid.shape[1], n_kv = K.grid.shape[1];
+    // One workspace for all calls: they run in order on one stream, and each
+    // call writes what it reads there.
+    const std::size_t ws_bytes = sizeof(float) * static_cast<std::size_t>(Q.shape[1]
+            * Q.basetile_shape[2] * Q.basetile_shape[3] * Q.basetile_shape[4]);
+    starpu::VariableHandle workspace(ws_bytes);
+    Index calls = 0;
+    for(Index g4 = 0; g4 < Q.grid.shape[4]; ++g4)
+    {
+        for(Index g3 = 0; g3 < Q.grid.shape[3]; ++g3)
+        {
+            for(Index g2 = 0; g2 < Q.grid.shape[2]; ++g2)
+            {
+                nntile_hip_sdpa_bwd_grid_args a;
+                std::memset(&a, 0, sizeof(a));
+                const auto &q0 = Q.get_tile({0, 0, g2, g3, g4});
+                a.q_seq = Q.shape[1];
+                a.k_seq = K.shape[1];
+                a.q_tile = Q.basetile_shape[1];
+                a.k_tile = K.basetile_shape[1];
+                a.head = Q.shape[0];
+                a.batch = q0.shape[2] * q0.shape[3] * q0.shape[4];
+                a.n_batch = a.batch;
+                a.kv_group = 1;
+                a.mask_mode = mask_mode;
+                a.n_q_tiles = static_cast<std::int32_t>(n_q);
+                a.n_kv_tiles = static_cast<std::int32_t>(n_kv);
+                a.causal_offset = causal_offset;
+                for(Index t = 0; t < n_kv; ++t)
+                {
+                    a.K[t] = K.get_tile({0, t, g2, g3, g4}).get_ptr();
+                    a.V[t] = V.get_tile({0, t, g2, g3, g4}).get_ptr();
+                    a.dK[t] = dK.get_tile({0, t, g2, g3, g4}).get_ptr();
+                    a.dV[t] = dV.get_tile({0, t, g2, g3, g4}).get_ptr();
+                    dK.get_tile({0, t, g2, g3, g4}).mark_written();
+                    dV.get_tile({0, t, g2, g3, g4}).mark_written();
+                }
+                for(Index t = 0; t < n_q; ++t)
+                {
+                    a.Q[t] = Q.get_tile({0, t, g2, g3, g4}).get_ptr();
+                    a.A[t] = A.get_tile({0, t, g2, g3, g4}).get_ptr();
+                    a.dA[t] = dA.get_tile({0, t, g2, g3, g4}).get_ptr();
+                    a.dQ[t] = dQ.get_tile({0, t, g2, g3, g4}).get_ptr();
+                    a.lse[t] = static_cast<const float *>(
+                            logsumexp.get_tile({t, g2, g3, g4}).get_ptr());
+                    dQ.get_tile({0, t, g2, g3, g4}).mark_written();
+                }
+                a.workspace = workspace.get_ptr();
+                a.workspace_bytes = ws_bytes;
+                starpu::count_direct_launch();
+                const int rc = BwdGridCall<T>::run(starpu::get_local_stream(), &a);
+                if(rc != NNTILE_HIP_OK)
+                {
+                    throw std::runtime_error("Error in flash_sdpa_bwd_hip grid launch (code "
+                            + std::to_string(rc) + ")");
+                }
+                ++calls;
+            }
+        }
+    }
+    workspace.unregister_submit();
+    return calls;
+}
+
 template<typename T>
 Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
@@ -1381,6 +1475,10 @@ Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
     flash_sdpa_bwd_cudnn_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
     require(mask_mode == NNTILE_HIP_MASK_NONE || mask_mode == NNTILE_HIP_MASK_CAUSAL,
             "flash_sdpa_bwd_hip: mask_mode must be NONE or CAUSAL");
+    if(bwd_grid_fits(K, Q))
+    {
+        return bwd_grid<T>(K, Q, V, A, dA, mask_mode, causal_offset, logsumexp, dK, dQ, dV);
+    }
     return bwd_pairs<T>(K, Q, V, A, dA, nullptr, nullptr, mask_mode, causal_offset,
             logsumexp, dK, dQ, dV);
 }
@@ -1395,6 +1493,13 @@ Index flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
     flash_sdpa_bwd_cudnn_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
     require(static_cast<Index>(mask_classes.size()) == mask.grid.nelems,
             "one class per mask tile is required");
+    // A mask that is the causal rule itself, or hides nothing, needs no call
+    // per pair (as in the forward operation above).
+    const int whole = flash_sdpa_mask_rule(mask, mask_classes, causal_offset);
+    if(whole >= 0 && bwd_grid_fits(K, Q))
+    {
+        return bwd_grid<T>(K, Q, V, A, dA, whole, causal_offset, logsumexp, dK, dQ, dV);
+    }
     return bwd_pairs<T>(K, Q, V, A, dA, &mask, &mask_classes, NNTILE_HIP_MASK_CAUSAL,
             causal_offset, logsumexp, dK, dQ, dV);
 }

@@ -380,10 +380,13 @@ void flash_sdpa_bwd_cudnn(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV);
 
 //! Same gradients with an analytic mask (NNTILE_HIP_MASK_NONE, or
-//! NNTILE_HIP_MASK_CAUSAL with `causal_offset`): no mask tensor, one call per
-//! (dQ tile, key tile) pair with the pair's positions, and pairs that a
-//! causal mask hides completely are not submitted.  Gradients are added.
-//! Returns the number of tile pairs submitted.
+//! NNTILE_HIP_MASK_CAUSAL with `causal_offset`): no mask tensor.  Where the
+//! sequence tiles are multiples of 128 rows (or an axis is one tile) and at
+//! most NNTILE_HIP_SDPA_BWD_MAX_TILES an axis, one call per slab of the batch
+//! grid takes all its tile pairs; otherwise one call per (dQ tile, key tile)
+//! pair with the pair's positions, and pairs that a causal mask hides
+//! completely are not submitted.  Gradients are added.  Returns the number
+//! of calls made (slabs, or tile pairs).
 template<typename T>
 Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,
@@ -393,7 +396,9 @@ Index flash_sdpa_bwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
 //! flash_sdpa_bwd_cudnn_async that uses the classes of the mask's tiles
 //! (flash_sdpa_mask_classes): no call for a pair whose mask tile hides
 //! everything, analytic masks for open and causal ones, the reference's tile
-//! operation for the rest.  Gradients are added.  Returns the pairs submitted.
+//! operation for the rest; a mask whose classes say it is the causal rule
+//! itself (or hides nothing) goes the way of flash_sdpa_bwd_hip_async.
+//! Gradients are added.  Returns the calls made (tile pairs, or slabs).
 template<typename T>
 Index flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,

@@ -306,3 +306,61 @@ def test_classified_submission_skips_hidden_tile_pairs(oracle, dtype, kind, offs
                     and not mask[q * tile:(q + 1) * tile, k * tile:(k + 1) * tile].all()
                     and not (kind == "causal" and q == k))
         assert tile_tasks == slabs * mixed
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("kind,offset", [("causal", 0), ("causal", -70), ("full", 0), ("window", 0)])
+def test_tiles_of_128_rows_take_one_call_per_slab(oracle, dtype, kind, offset):
+    """Sequence tiles that are multiples of 128 rows: a mask whose tile classes say it is the causal rule, or hides nothing,
+    costs one call per slab of the batch grid instead of one per tile pair -
+    through the overload that takes the classes, through the reference's own
+    signature, and through the analytic form; any other mask still goes pair
+    by pair.  Gradients as the checker's and as the literal submission's."""
+    head, seq, tile, nb, grp, nkv = 64, 384, 128, 2, 1, 2
+    batch = nb * grp * nkv
+    shape5, base5 = [head, seq, nb, grp, nkv], [head, tile, 1, 1, 2]
+    (Q, K, V), (qf, kf, vf) = H.make_qkv(71, batch, seq, seq, head, dtype)
+    _, gf = H.rounded(synth.randn(72, 0, batch * seq * head).reshape(batch, seq, head), dtype)
+    i = np.arange(seq)
+    mask = {"causal": i[None, :] <= i[:, None] + offset, "window": np.abs(i[None, :] - i[:, None]) <= 150,
+            "full": np.ones((seq, seq), bool)}[kind]
+    add = np.where(mask, 0.0, -np.inf).astype(np.float32)
+    vis = mask.any(axis=1)
+    with np.errstate(all="ignore"):
+        A64, lse64 = oracle.sdpa_bruteforce_f64(kf, qf, vf, add)
+    A64 = np.where(vis[None, :, None], A64, 0.0)
+    lse = np.where(vis[None, :], lse64, -np.inf).astype(np.float32)
+    _, af = H.rounded(A64, dtype)
+    data = {"K": kf, "Q": qf, "V": vf, "A": af, "dA": gf}
+    start = {n: 0.25 * synth.randn(73, j, batch * seq * head).reshape(batch, seq, head)
+             for j, n in enumerate(("dK", "dQ", "dV"))}
+    start = {n: H.rounded(x, dtype)[1] for n, x in start.items()}
+    got, calls, ntiles = _run(hm.OP_CLASSIFIED, dtype, data, lse, add, shape5, base5, grads0=start,
+                              offset=offset)
+    ref, all_pairs, _ = _run(hm.OP_PAIRS_BWD, dtype, data, lse, add, shape5, base5, grads0=start)
+    nt = -(-seq // tile)
+    slabs = ntiles // nt
+    live = sum(1 for q in range(nt) for k in range(nt)
+               if mask[q * tile:(q + 1) * tile, k * tile:(k + 1) * tile].any())
+    assert all_pairs == slabs * nt * nt
+    assert calls == (slabs * live if kind == "window" else slabs)
+    with np.errstate(all="ignore"):
+        want = oracle.sdpa_bwd_flash_f64(kf, qf, vf, af, gf, np.where(vis[None, :], lse, 0.0),
+                                         np.where(vis[:, None], add, -np.inf))
+    tol = 1e-2 if dtype == "bf16" else 2e-3
+    for g, r, w, n in zip(got, ref, want, ("dK", "dQ", "dV")):
+        assert H.rel_fro(g, w + start[n]) < tol, n
+        assert H.rel_fro(g, r) < tol, n
+    if kind != "window":
+        hip, hip_calls, _ = _run(hm.OP_HIP, dtype, data, lse, add, shape5, base5, grads0=start,
+                                 mask_mode=2 if kind == "causal" else 1, offset=offset)
+        assert hip_calls == slabs
+        for g, d, n in zip(got, hip, ("dK", "dQ", "dV")):
+            assert np.array_equal(g, d), n
+    if offset == 0:
+        dflt, tile_tasks, _ = _run(hm.OP_TENSOR, dtype, data, lse, add, shape5, base5, grads0=start)
+        for g, d, n in zip(got, dflt, ("dK", "dQ", "dV")):
+            assert np.array_equal(g, d), n
+        if kind != "window":
+            assert tile_tasks == 0
