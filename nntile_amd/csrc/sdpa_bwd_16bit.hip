@@ -387,6 +387,19 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
         const int r = ld_row0 + i * ROWS_PER_LOAD;
         ld_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ G::swz(r)) * 16);
     }
+    // (only the last step of the keys can be short: its rows past the end read
+    // the last row that exists; the offsets of that step are kept beside the
+    // others rather than computed per load)
+    uint32_t ld_goff_end[LOADS_PER_WAVE];
+    {
+        const int last_of_end = (k_seq - 1) % kBwdStep;
+#pragma unroll
+        for(int i = 0; i < LOADS_PER_WAVE; ++i)
+        {
+            ld_goff_end[i] = ld_goff[i]
+                - (uint32_t)(max(ld_row0 + i * ROWS_PER_LOAD - last_of_end, 0) * RB);
+        }
+    }
     // row operand: lane (col, half) reads row mb*32+col, logical chunk 2*ks+half;
     // 32 rows further on the swizzle is the same, so mb goes into the immediate
     uint32_t row_raddr[KSTEPS];
@@ -424,37 +437,44 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
     // (a wave gets one such load accepted every ~64 cycles and stands still
     // until then: inside the loop the loads go between the MFMAs, one K and
     // one V load at a time)
-    auto fetch_piece = [&](int g, char *kdst_base, char *vdst_base, int i)
-        __attribute__((always_inline))
+    struct KeyRows
+    {
+        const char *K, *V;      // the step's first row of the entry
+        bool at_end;
+    };
+    auto key_rows = [&](int g) __attribute__((always_inline)) -> KeyRows
     {
         const int row0 = g * kBwdStep;
-        const int last = min(kBwdStep, k_seq - row0) - 1;
-        const char *Kg, *Vg;        // the step's first row of the entry
+        const bool at_end = row0 + kBwdStep > k_seq;
         if constexpr(GRID)
         {
             const int k_tile = (int)p.k_tile;
             const int tk = row0 / k_tile, t0 = tk * k_tile;
             const int64_t off = ((int64_t)kvb * min(k_tile, k_seq - t0) + (row0 - t0)) * RB;
-            Kg = static_cast<const char *>(p.Kt[tk]) + off;
-            Vg = static_cast<const char *>(p.Vt[tk]) + off;
+            return KeyRows{static_cast<const char *>(p.Kt[tk]) + off,
+                static_cast<const char *>(p.Vt[tk]) + off, at_end};
         }
         else
         {
-            Kg = Kb + (int64_t)row0 * RB;
-            Vg = Vb + (int64_t)row0 * RB;
+            return KeyRows{Kb + (int64_t)row0 * RB, Vb + (int64_t)row0 * RB, at_end};
         }
+    };
+    auto fetch_piece = [&](const KeyRows &at, char *kdst_base, char *vdst_base, int i)
+        __attribute__((always_inline))
+    {
         char *kdst = kdst_base + wave_u * LOADS_PER_WAVE * 1024;
         char *vdst = vdst_base + wave_u * LOADS_PER_WAVE * 1024;
-        const uint32_t back = (uint32_t)(max(ld_row0 + i * ROWS_PER_LOAD - last, 0) * RB);
-        load_to_lds16<0, false>(Kg, ld_goff[i] - back, kdst + i * 1024);
-        load_to_lds16<0, false>(Vg, ld_goff[i] - back, vdst + i * 1024);
+        const uint32_t goff = at.at_end ? ld_goff_end[i] : ld_goff[i];
+        load_to_lds16<0, false>(at.K, goff, kdst + i * 1024);
+        load_to_lds16<0, false>(at.V, goff, vdst + i * 1024);
     };
     auto fetch = [&](int g, char *kdst_base, char *vdst_base)
     {
+        const KeyRows at = key_rows(g);
 #pragma unroll
         for(int i = 0; i < LOADS_PER_WAVE; ++i)
         {
-            fetch_piece(g, kdst_base, vdst_base, i);
+            fetch_piece(at, kdst_base, vdst_base, i);
         }
     };
     constexpr int FETCH_STRIDE = (NNTILE_BWD_SPREAD == 2 ? 2 : 1) * KSTEPS / LOADS_PER_WAVE;
@@ -500,7 +520,9 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         // the last step loads its own tile once more, rather than branch
-        const int g_fetch = g_next >= 0 ? g_next : g;
+        // (wave-common, computed once here: the loads between the MFMAs below
+        // only add their offsets)
+        const KeyRows at_f = key_rows(g_next >= 0 ? g_next : g);
         if(NNTILE_BWD_SPREAD == 0 && g_next >= 0)
         {
             fetch(g_next, BUF ? lds_k0 : lds_k1, BUF ? lds_v0 : lds_v1);
@@ -545,7 +567,7 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
                 {
                     if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
                     {
-                        fetch_piece(g_fetch, BUF ? lds_k0 : lds_k1, BUF ? lds_v0 : lds_v1, j);
+                        fetch_piece(at_f, BUF ? lds_k0 : lds_k1, BUF ? lds_v0 : lds_v1, j);
                     }
                 }
             }
@@ -770,15 +792,17 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
         first_step = min(q_lo / kBwdStep, n_steps);
     }
 
-    uint32_t ld_goff[LPW];
-    int ld_row[LPW];
+    // (only the last step of the queries can be short: its rows past the end
+    // read the last row that exists; the offsets of that step are kept beside
+    // the others rather than computed per load)
+    uint32_t ld_goff[LPW], ld_goff_end[LPW];
     const int ld_cpos = lane % CPR;
 #pragma unroll
     for(int i = 0; i < LPW; ++i)
     {
         const int r = ((wave % LOADERS) * LPW + i) * ROWS_PER_LOAD + lane / CPR;
-        ld_row[i] = r;
         ld_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ G::swz(r)) * 16);
+        ld_goff_end[i] = ld_goff[i] - (uint32_t)(max(r - (q_seq - 1) % kBwdStep, 0) * RB);
     }
     // row operand: lane (col, half) reads row mb*32+col, logical chunk 2*ks+half;
     // 32 rows further on the swizzle is the same, so mb goes into the immediate
@@ -879,36 +903,53 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             return QueryRows{p.Q, p.dA, p.lse, elem, elem};
         }
     };
-    auto fetch_piece = [&](int bq, int row0, int last, char *qdst_base, char *gdst_base, int j)
-        __attribute__((always_inline))
+    auto fetch_piece = [&](const QueryRows &at, bool at_end, char *qdst_base, char *gdst_base,
+            int j) __attribute__((always_inline))
     {
-        const QueryRows at = query_rows(bq, row0);
         const char *Qp = static_cast<const char *>(at.Q) + at.elem * RB;
         const char *Gp = static_cast<const char *>(at.dA) + at.elem * RB;
         char *qdst = qdst_base + wave_u * LPW * 1024;
         char *gdst = gdst_base + wave_u * LPW * 1024;
-        const uint32_t back = (uint32_t)(max(ld_row[j] - last, 0) * RB);
-        load_to_lds16<0, false>(Qp, ld_goff[j] - back, qdst + j * 1024);
-        load_to_lds16<0, false>(Gp, ld_goff[j] - back, gdst + j * 1024);
+        const uint32_t goff = at_end ? ld_goff_end[j] : ld_goff[j];
+        load_to_lds16<0, false>(Qp, goff, qdst + j * 1024);
+        load_to_lds16<0, false>(Gp, goff, gdst + j * 1024);
     };
-    auto fetch_stat = [&](int bq, int row0, int last, float (*stat)[kBwdStep])
+    // The statistics of a step in two halves, so that the load's latency
+    // passes behind the MFMAs of the step before: stat_load starts the read
+    // of the thread's value (threads 0..63 a logsumexp, 64..127 a row dot),
+    // stat_store turns it into what the step reads from LDS.
+    auto stat_load = [&](const QueryRows &at, int last) __attribute__((always_inline)) -> float
+    {
+        float raw = 0.0f;
+        if(tid < 2 * kBwdStep)
+        {
+            const int which = tid / kBwdStep, r = tid % kBwdStep;
+            const float *src = which == 0 ? at.lse + at.elem : p.D + at.d_idx;
+            raw = src[min(r, last)];
+        }
+        return raw;
+    };
+    auto stat_store = [&](float raw, int last, float (*stat)[kBwdStep])
+        __attribute__((always_inline))
     {
         if(tid < 2 * kBwdStep)
         {
             const int which = tid / kBwdStep, r = tid % kBwdStep;
-            const QueryRows at = query_rows(bq, row0);
             float v;
             if(which == 0)
             {
-                const float l = at.lse[at.elem + min(r, last)];
-                v = (r > last || l == neg_inf()) ? __builtin_huge_valf() : l * kLog2e;
+                v = (r > last || raw == neg_inf()) ? __builtin_huge_valf() : raw * kLog2e;
             }
             else
             {
-                v = r > last ? 0.0f : p.D[at.d_idx + min(r, last)];
+                v = r > last ? 0.0f : -raw;
             }
             stat[which][r] = v;
         }
+    };
+    auto fetch_stat = [&](const QueryRows &at, int last, float (*stat)[kBwdStep])
+    {
+        stat_store(stat_load(at, last), last, stat);
     };
     constexpr int FETCH_STRIDE = (NNTILE_BWD_SPREAD == 2 ? 2 : 1) * KSTEPS / LPW;
     static_assert(FETCH_STRIDE >= 1 && 1 + (LPW - 1) * FETCH_STRIDE < 2 * KSTEPS,
@@ -919,15 +960,16 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
         locate(i, bq, qs);
         const int row0 = qs * kBwdStep;
         const int last = min(kBwdStep, q_seq - row0) - 1;
+        const QueryRows at = query_rows(bq, row0);
         if(LOADERS == kDkvWaves || wave_u < LOADERS)
         {
 #pragma unroll
             for(int j = 0; j < LPW; ++j)
             {
-                fetch_piece(bq, row0, last, qdst_base, gdst_base, j);
+                fetch_piece(at, last + 1 < kBwdStep, qdst_base, gdst_base, j);
             }
         }
-        fetch_stat(bq, row0, last, stat);
+        fetch_stat(at, last, stat);
     };
 
     int i_cur = walk_begin();
@@ -951,15 +993,20 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
         locate(i_next >= 0 ? i_next : i, bq_f, qs_f);
         const int row0_f = qs_f * kBwdStep;
         const int last_f = min(kBwdStep, q_seq - row0_f) - 1;
+        const bool at_end_f = last_f + 1 < kBwdStep;
+        // (wave-common, computed once here: the loads between the MFMAs below
+        // only add their offsets)
+        const QueryRows at_f = query_rows(bq_f, row0_f);
+        float raw_next = 0.0f;
         if(i_next >= 0)
         {
-            fetch_stat(bq_f, row0_f, last_f, lds_stat[BUF ^ 1]);
+            raw_next = stat_load(at_f, last_f);
             if(NNTILE_BWD_SPREAD == 0 && (LOADERS == kDkvWaves || wave_u < LOADERS))
             {
 #pragma unroll
                 for(int j = 0; j < LPW; ++j)
                 {
-                    fetch_piece(bq_f, row0_f, last_f, BUF ? lds_q0 : lds_q1,
+                    fetch_piece(at_f, at_end_f, BUF ? lds_q0 : lds_q1,
                             BUF ? lds_g0 : lds_g1, j);
                 }
             }
@@ -991,6 +1038,22 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                 sv[r] = 0.0f;
                 dpv[r] = 0.0f;
             }
+            if(DO_DK)
+            {
+                // dP - D: the accumulator starts at -D of its row (four
+                // consecutive queries per LDS read), the products add dP
+#pragma unroll
+                for(int rg = 0; rg < 4; ++rg)
+                {
+                    const f32x4 nd4 = *reinterpret_cast<const f32x4 *>(
+                            &stat[1][mb * 32 + 8 * rg + 4 * half]);
+#pragma unroll
+                    for(int e = 0; e < 4; ++e)
+                    {
+                        dpv[4 * rg + e] = nd4[e];
+                    }
+                }
+            }
 #pragma unroll
             for(int ks = 0; ks < KSTEPS; ++ks)
             {
@@ -1009,7 +1072,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                     {
                         if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
                         {
-                            fetch_piece(bq_f, row0_f, last_f, BUF ? lds_q0 : lds_q1,
+                            fetch_piece(at_f, at_end_f, BUF ? lds_q0 : lds_q1,
                                     BUF ? lds_g0 : lds_g1, j);
                         }
                     }
@@ -1040,7 +1103,6 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                 // four consecutive queries: their statistics in one LDS read each
                 const int qr0 = mb * 32 + 8 * rg + 4 * half;
                 const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(&stat[0][qr0]);
-                const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&stat[1][qr0]);
 #pragma unroll
                 for(int e = 0; e < 4; ++e)
                 {
@@ -1072,7 +1134,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                         }
                     }
                     pv[r] = use_mask ? (visible ? fast_exp2(ex) : 0.0f) : fast_exp2(ex);
-                    dsv[r] = pv[r] * (dpv[r] - d4[e]);
+                    dsv[r] = pv[r] * dpv[r];
                 }
             }
 #pragma unroll
@@ -1111,6 +1173,13 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                     }
                 }
             }
+        }
+        // (the other buffer's readers passed this step's barrier; the next
+        // step's barrier orders these writes before its reads)
+        __builtin_amdgcn_sched_barrier(0);
+        if(i_next >= 0)
+        {
+            stat_store(raw_next, last_f, lds_stat[BUF ^ 1]);
         }
     };
     auto run = [&](int i, int i_next, auto buf_tag) __attribute__((always_inline))
@@ -1204,7 +1273,7 @@ void sdpa_bwd_kernel(const std::conditional_t<GRID, BwdGridParams, BwdParams> p,
     __shared__ __attribute__((aligned(1024))) char lds_2[G::BYTES];
     __shared__ __attribute__((aligned(1024))) char lds_3[G::BYTES];
     // dK, dV parts, per query of a step: logsumexp in log2 units (+inf for a
-    // row that saw nothing) and the row dot D; rows past the end hold +inf / 0
+    // row that saw nothing) and minus the row dot D; rows past the end hold +inf / 0
     __shared__ __attribute__((aligned(16))) float lds_stat[2][2][kBwdStep];
     if(blockIdx.x < n_dkv)
     {
