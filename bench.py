@@ -149,13 +149,14 @@ class PowerSampler:
         return round(sum(tail) / len(tail), 0) if tail else None
 
 
-def bench_prefill(cfg, steps, warmup, zeros=False, settle_s=0.0):
-    """One fused launch per independent slab of cfg over its whole tile grid
-    (analytic causal mask, hidden tile pairs skipped, overwrite mode).  Tiles
-    are separate allocations, as NNTile tensors are.  zeros=True replaces the
-    inputs by zeros (for the power comparison only).  settle_s: seconds of the
-    same step run untimed before the warm-up steps, so that clock and power
-    have settled on this load whatever ran before."""
+def bench_prefill(cfg, steps, warmup, zeros=False, settle_s=0.0, one_launch=True):
+    """The tensor-level call over cfg's whole tile grid (analytic causal mask,
+    hidden tile pairs skipped, overwrite mode): one fused launch over all
+    sequence tiles of all slabs of the batch grid (one_launch=False: one
+    launch per slab).  Tiles are separate allocations, as NNTile tensors are.
+    zeros=True replaces the inputs by zeros (for the power comparison only).
+    settle_s: seconds of the same step run untimed before the warm-up steps,
+    so that clock and power have settled on this load whatever ran before."""
     import torch
     from nntile_amd import hip_sdpa as h
     dt = {"fp32": torch.float32, "bf16": torch.bfloat16, "fp16": torch.float16}[cfg.dtype]
@@ -175,8 +176,15 @@ def bench_prefill(cfg, steps, warmup, zeros=False, settle_s=0.0):
         A = [torch.zeros_like(q) for q in Q]
         lse = [torch.full((per_call, cfg.seq_tile), float("-inf"), device="cuda") for _ in range(nt)]
         keep.append((Q, K, V, A, lse))
-        plans.append(h.plan_grid(K, Q, lse, V, A, cfg.q_seq, cfg.k_seq, cfg.seq_tile,
-                                 cfg.seq_tile, h.MASK_CAUSAL, flags=h.OVERWRITE))
+    if one_launch and cfg.calls * nt <= h.MAX_TILES:
+        cat = lambda i: [t for slab in keep for t in slab[i]]
+        plans.append(h.plan_grid(cat(1), cat(0), cat(4), cat(2), cat(3), cfg.q_seq, cfg.k_seq,
+                                 cfg.seq_tile, cfg.seq_tile, h.MASK_CAUSAL, flags=h.OVERWRITE,
+                                 n_slabs=cfg.calls))
+    else:
+        for Q, K, V, A, lse in keep:
+            plans.append(h.plan_grid(K, Q, lse, V, A, cfg.q_seq, cfg.k_seq, cfg.seq_tile,
+                                     cfg.seq_tile, h.MASK_CAUSAL, flags=h.OVERWRITE))
     del q_all, k_all, v_all
 
     def step():
@@ -666,6 +674,8 @@ def main():
     legs = {"prefill": lambda: bench_prefill(cfg3, args.steps, args.warmup),
             "cfg5": lambda: bench_prefill(BY_NAME["cfg5_long_seq_bf16"], args.steps, args.warmup),
             "cfg2": lambda: bench_prefill(BY_NAME["cfg2_gpt2_small_fp32"], args.steps, args.warmup),
+            "cfg2_per_slab": lambda: bench_prefill(BY_NAME["cfg2_gpt2_small_fp32"], args.steps,
+                                                   args.warmup, one_launch=False),
             "decode": lambda: bench_decode(cfg4, args.steps, args.warmup),
             "decode_wide": lambda: bench_decode(cfg4_wide, args.steps, args.warmup),
             "reference_api": lambda: bench_reference_api(cfg3, args.steps, args.warmup),
@@ -711,6 +721,12 @@ def main():
                                  c.flops(), r["device_ms_per_step"],
                                  PEAK_FP32_TFLOPS if fp32 else PEAK_BF16_TFLOPS, "TFLOP/s",
                                  TRAFFIC.get(name))}
+        if c.calls > 1:
+            r1 = bench_prefill(c, few, 3, one_launch=False)
+            extras[name]["one_launch_per_slab"] = {
+                "what": "the same with one launch per slab of the batch grid (%d launches)" % c.calls,
+                "ms_per_step": round(r1["ms_per_step"], 4), "tflops": round(r1["tflops"], 2),
+                "launches_per_step": r1["launches_per_step"]}
     backward = bench_backward(cfg3, max(5, args.steps // 10), 3)
     rope = bench_rope(cfg3, few, 5)
     transpose = bench_transpose(cfg3, few, 5)

@@ -188,7 +188,17 @@ int nntile_hip_sdpa_bwd_tile_fp16(void *stream, const nntile_hip_sdpa_bwd_args *
  * all query tiles hold q_tile rows and all key tiles k_tile rows, except the
  * last of each, which holds the remainder of q_seq / k_seq.  Only the
  * analytic masks (NONE, CAUSAL) are accepted; positions count from row 0 of
- * tile 0 plus q_pos0 / k_pos0. */
+ * tile 0 plus q_pos0 / k_pos0.
+ *
+ * n_slabs > 1 puts several such slabs into the one launch - the tiles the
+ * tensor-level loop walks along the batch axes, each slab a set of separate
+ * allocations with the same extents and `batch` entries: the tables then hold
+ * slab s's tiles at [s*n_q_tiles + t] (Q, lse, A) and [s*n_kv_tiles + t] (K,
+ * V), and n_slabs*n_q_tiles and n_slabs*n_kv_tiles must not exceed
+ * NNTILE_HIP_SDPA_MAX_TILES.  batch, n_batch and kv_group describe one slab.
+ * 0 stands for 1.  (A launch picks its workgroup shape from its total size,
+ * so the fp32 results of a many-slab launch may differ from per-slab launches
+ * in the last bits: the key steps of a row are summed in another order.) */
 #define NNTILE_HIP_SDPA_MAX_TILES 64
 
 typedef struct nntile_hip_sdpa_grid_args
@@ -196,6 +206,7 @@ typedef struct nntile_hip_sdpa_grid_args
     int64_t q_seq, k_seq, q_tile, k_tile, head;
     int64_t batch, n_batch, kv_group;
     int32_t mask_mode, n_q_tiles, n_kv_tiles, flags;
+    int32_t n_slabs, reserved;
     int64_t q_pos0, k_pos0, causal_offset;
     const void *K[NNTILE_HIP_SDPA_MAX_TILES];
     const void *V[NNTILE_HIP_SDPA_MAX_TILES];

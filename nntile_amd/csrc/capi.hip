@@ -117,6 +117,7 @@ static int tile_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a,
     p.mask_ld = a->k_seq;
     p.kv_rows = kv_rows;
     p.n_q_tiles = p.n_kv_tiles = 1;
+    p.n_slabs = 1;
     p.batch = (int32_t)a->batch;
     p.n_batch = (int32_t)a->n_batch;
     p.kv_group = (int32_t)a->kv_group;
@@ -365,7 +366,15 @@ static int grid_call(DType dt, void *stream, const nntile_hip_sdpa_grid_args *a)
             || a->batch > 0x7fffffff || a->q_seq > 0x7fffffff
             || a->k_seq > 0x7fffffff
             || a->n_q_tiles <= 0 || a->n_q_tiles > NNTILE_HIP_SDPA_MAX_TILES
-            || a->n_kv_tiles <= 0 || a->n_kv_tiles > NNTILE_HIP_SDPA_MAX_TILES)
+            || a->n_kv_tiles <= 0 || a->n_kv_tiles > NNTILE_HIP_SDPA_MAX_TILES
+            || a->n_slabs < 0 || a->n_slabs > NNTILE_HIP_SDPA_MAX_TILES)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    const int n_slabs = a->n_slabs == 0 ? 1 : a->n_slabs;
+    const int n_q_all = n_slabs * a->n_q_tiles, n_kv_all = n_slabs * a->n_kv_tiles;
+    if(n_q_all > NNTILE_HIP_SDPA_MAX_TILES || n_kv_all > NNTILE_HIP_SDPA_MAX_TILES
+            || a->batch * n_slabs > 0x7fffffff)
     {
         return NNTILE_HIP_EINVAL;
     }
@@ -392,11 +401,12 @@ static int grid_call(DType dt, void *stream, const nntile_hip_sdpa_grid_args *a)
     p.causal_offset = a->causal_offset;
     p.n_q_tiles = a->n_q_tiles;
     p.n_kv_tiles = a->n_kv_tiles;
+    p.n_slabs = n_slabs;
     p.batch = (int32_t)a->batch;
     p.n_batch = (int32_t)a->n_batch;
     p.kv_group = (int32_t)a->kv_group;
     p.overwrite = (a->flags & NNTILE_HIP_SDPA_OVERWRITE) ? 1 : 0;
-    for(int t = 0; t < a->n_kv_tiles; ++t)
+    for(int t = 0; t < n_kv_all; ++t)
     {
         if(a->K[t] == nullptr || a->V[t] == nullptr || !aligned16(a->K[t])
                 || !aligned16(a->V[t]))
@@ -406,7 +416,7 @@ static int grid_call(DType dt, void *stream, const nntile_hip_sdpa_grid_args *a)
         p.K[t] = a->K[t];
         p.V[t] = a->V[t];
     }
-    for(int t = 0; t < a->n_q_tiles; ++t)
+    for(int t = 0; t < n_q_all; ++t)
     {
         if(a->Q[t] == nullptr || a->A[t] == nullptr || a->lse[t] == nullptr
                 || !aligned16(a->Q[t]) || !aligned16(a->A[t]))

@@ -57,6 +57,8 @@ struct PrefillParams
     // on share bit 63).  Null: every workgroup scans its own rows.
     const unsigned long long *mask_bits;
     int32_t n_q_tiles, n_kv_tiles;
+    int32_t n_slabs;              // slabs of `batch` entries each in this launch; slab s's tiles sit at
+                                  // [s*n_q_tiles + t] / [s*n_kv_tiles + t] of the tables below
     int32_t batch, n_batch, kv_group;
     int32_t q_blocks_per_tile;    // ceil(q_tile / rows per workgroup)
     int32_t k_blocks_per_tile;    // ceil(k_tile / keys per step)
@@ -141,6 +143,9 @@ struct BwdGridParams : BwdParams
 // every wait for an LDS read into a wait for all LDS reads, which undoes
 // reading operands ahead of their use.  The caller waits (vmcnt) and
 // synchronises before anyone reads the target; nothing else here uses M0.
+#ifndef NNTILE_DMA_NT_BITS
+#define NNTILE_DMA_NT_BITS "nt"     // cache-policy bits of the streaming (NT) form
+#endif
 template<int OFF, bool NT>
 __device__ __forceinline__ void load_to_lds16(const void *gaddr, char *lds_dst)
 {
@@ -149,7 +154,7 @@ __device__ __forceinline__ void load_to_lds16(const void *gaddr, char *lds_dst)
     if(NT)
     {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-                "global_load_lds_dwordx4 %1, off offset:%2 nt"
+                "global_load_lds_dwordx4 %1, off offset:%2 " NNTILE_DMA_NT_BITS
                 :: "s"(base), "v"(gaddr), "n"(OFF) : "memory");
     }
     else
@@ -179,7 +184,7 @@ __device__ __forceinline__ void load_to_lds16(const void *gbase_in, uint32_t lan
     if(NT)
     {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-                "global_load_lds_dwordx4 %1, %2 offset:%3 nt"
+                "global_load_lds_dwordx4 %1, %2 offset:%3 " NNTILE_DMA_NT_BITS
                 :: "s"(base), "v"(lane_off), "s"(gbase), "n"(OFF) : "memory");
     }
     else

@@ -122,17 +122,27 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         }
     }
     int b, qblk;
+    const int batch_all = p.batch * p.n_slabs;
     if(p.xcd_remap)
     {
-        const int b_per_xcd = p.batch >> 3;
+        const int b_per_xcd = batch_all >> 3;
         const int i = (int)(wg >> 3);
         b = (int)(wg & 7) * b_per_xcd + i % b_per_xcd;
         qblk = q_blocks - 1 - i / b_per_xcd;
     }
     else
     {
-        b = (int)wg % p.batch;
-        qblk = q_blocks - 1 - (int)wg / p.batch;
+        b = (int)wg % batch_all;
+        qblk = q_blocks - 1 - (int)wg / batch_all;
+    }
+    // the slab of this entry: its tiles are allocations of their own
+    int q_tile0 = 0, k_tile0 = 0;
+    if(p.n_slabs > 1)
+    {
+        const int slab = b / p.batch;
+        b -= slab * p.batch;
+        q_tile0 = slab * p.n_q_tiles;
+        k_tile0 = slab * p.n_kv_tiles;
     }
     const int qt = qblk / p.q_blocks_per_tile;
     const int qb = qblk % p.q_blocks_per_tile;
@@ -144,7 +154,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     }
     const int kvb = kv_entry(b, p.n_batch, p.kv_group);
 
-    const uint16_t *Qt = static_cast<const uint16_t *>(p.Q[qt])
+    const uint16_t *Qt = static_cast<const uint16_t *>(p.Q[q_tile0 + qt])
         + (int64_t)b * q_len * HEAD;
     const int my_q = q_row0 + wave * 32 + col;          // row within tile
     const bool q_ok = my_q < q_len;
@@ -463,8 +473,8 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             if(cur.kt < p.n_kv_tiles)
             {
                 cur.rows_left = tile_rows(cur.kt);
-                cur.Kp = static_cast<const char *>(p.K[cur.kt]) + slab(cur.kt);
-                cur.Vp = static_cast<const char *>(p.V[cur.kt]) + slab(cur.kt);
+                cur.Kp = static_cast<const char *>(p.K[k_tile0 + cur.kt]) + slab(cur.kt);
+                cur.Vp = static_cast<const char *>(p.V[k_tile0 + cur.kt]) + slab(cur.kt);
             }
             else
             {
@@ -573,8 +583,8 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
 
     PHASE_DECL
     StepCursor cur = {0, 0, tile_rows(0),
-        static_cast<const char *>(p.K[0]) + slab(0),
-        static_cast<const char *>(p.V[0]) + slab(0)};     // step being computed
+        static_cast<const char *>(p.K[k_tile0]) + slab(0),
+        static_cast<const char *>(p.V[k_tile0]) + slab(0)};     // step being computed
     StepCursor nxt = cur;                        // step being fetched
     // Leading steps that are complete (64 keys) and visible to every query of
     // the workgroup need no mask at all; they run in the pipelined loop below.
@@ -1230,7 +1240,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     const bool live = q_ok && !(empty && !p.overwrite);
     const float to_ln = p.scale;
     const float lse_new = empty ? neg_inf() : m_run * to_ln + __logf(l_tot);
-    float *lse_ptr = p.lse[qt] + (int64_t)b * q_len + (q_ok ? my_q : 0);
+    float *lse_ptr = p.lse[q_tile0 + qt] + (int64_t)b * q_len + (q_ok ? my_q : 0);
     const float lse_old = (p.overwrite || !live) ? neg_inf() : *lse_ptr;
     float w_old = 0.0f, w_new = 0.0f, lse_out = neg_inf();
     if(live && !empty)
@@ -1267,7 +1277,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         }
         const uint64_t live_rows = __builtin_amdgcn_ballot_w64(live && half == 0);
         constexpr int ROWS_PER_ST = 1024 / RB;      // rows one store instruction covers
-        char *Abase = static_cast<char *>(p.A[qt])
+        char *Abase = static_cast<char *>(p.A[q_tile0 + qt])
             + ((int64_t)b * q_len + q_row0 + wave * 32) * RB;
 #pragma unroll
         for(int i = 0; i < 32 / ROWS_PER_ST; ++i)
@@ -1287,7 +1297,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     {
         return;
     }
-    uint16_t *Arow = static_cast<uint16_t *>(p.A[qt])
+    uint16_t *Arow = static_cast<uint16_t *>(p.A[q_tile0 + qt])
         + ((int64_t)b * q_len + my_q) * HEAD;
 #pragma unroll
     for(int db = 0; db < DBLOCKS; ++db)
@@ -1495,7 +1505,8 @@ int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
 {
     p.q_blocks_per_tile = (int)((p.q_tile + kQRows - 1) / kQRows);
     p.k_blocks_per_tile = (int)((p.k_tile + kKeys - 1) / kKeys);
-    const int64_t n_wg = (int64_t)p.batch * p.n_q_tiles * p.q_blocks_per_tile;
+    const int64_t batch_all = (int64_t)p.batch * p.n_slabs;
+    const int64_t n_wg = batch_all * p.n_q_tiles * p.q_blocks_per_tile;
     if(n_wg <= 0 || n_wg > 0x7fffffff)
     {
         return NNTILE_HIP_EINVAL;
@@ -1506,7 +1517,7 @@ int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
     {
         return scan_rc;
     }
-    p.xcd_remap = (p.batch % 8 == 0) ? 1 : 0;
+    p.xcd_remap = (batch_all % 8 == 0) ? 1 : 0;
     const dim3 grid((unsigned)n_wg);
     switch(head)
     {

@@ -49,6 +49,28 @@ namespace nntile_hip
 #ifndef NNTILE_F32_FINE
 #define NNTILE_F32_FINE 0
 #endif
+// Launches with fewer 128-query workgroups than this take the SPLIT form.
+// Measured crossovers (fused launches of batch x seq x head, 100 launches
+// each): under a causal mask the 32-query workgroups, dealt longest first,
+// fill the triangle far better - head 64: 48 x 1024 81.7 us against 139.5,
+// 32 x 4096 619 against 771, 192 x 2048 1005 against 1087, and only at 384 x
+// 2048 (6144 such workgroups) 2301 against 2022; head 128: 96 x 1024 353
+// against 385, 64 x 2048 809 against 820, 96 x 2048 1227 against 1118.
+// Without a mask the shared key steps win earlier: head 64, 48 x 1024 122
+// against 139, 96 x 1024 243 against 202.
+static int split_below(int head, int mode)
+{
+#ifdef NNTILE_F32_SPLIT_BELOW
+    return NNTILE_F32_SPLIT_BELOW;
+#else
+    const bool causal = mode == NNTILE_HIP_MASK_CAUSAL;
+    if(head >= 128)
+    {
+        return causal ? 1025 : 256;
+    }
+    return causal ? 4096 : 512;
+#endif
+}
 constexpr int kQRows32 = 128;
 constexpr int kKeys32 = 32;
 constexpr int kThreads32 = 256;          // 4 wavefronts in both forms
@@ -99,6 +121,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     F32_STAMP_DECL
 
     const int q_blocks = p.n_q_tiles * p.q_blocks_per_tile;
+    const int batch_all = p.batch * p.n_slabs;
     int wg = blockIdx.x;
     int b, qblk;
     if(SPLIT)
@@ -117,8 +140,8 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
             i = 32 + (per_xcd - 1 - i);
         }
         const int k = (i << 3) | (wg & 7);
-        b = k % p.batch;
-        qblk = q_blocks - 1 - k / p.batch;
+        b = k % batch_all;
+        qblk = q_blocks - 1 - k / batch_all;
     }
     else
     {
@@ -130,6 +153,15 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         b = wg / q_blocks;
         qblk = q_blocks - 1 - (wg % q_blocks);
     }
+    // the slab of this entry: its tiles are allocations of their own
+    int q_tile0 = 0, k_tile0 = 0;
+    if(p.n_slabs > 1)
+    {
+        const int slab = b / p.batch;
+        b -= slab * p.batch;
+        q_tile0 = slab * p.n_q_tiles;
+        k_tile0 = slab * p.n_kv_tiles;
+    }
     const int qt = qblk / p.q_blocks_per_tile;
     const int qb = qblk % p.q_blocks_per_tile;
     const int64_t q_len = min(p.q_tile, p.q_seq - (int64_t)qt * p.q_tile);
@@ -140,7 +172,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     }
     const int kvb = kv_entry(b, p.n_batch, p.kv_group);
 
-    const float *Qt = static_cast<const float *>(p.Q[qt])
+    const float *Qt = static_cast<const float *>(p.Q[q_tile0 + qt])
         + (int64_t)b * q_len * HEAD;
     const int64_t my_q = q_row0 + (SPLIT ? 0 : wave * 32) + col;
     const bool q_ok = my_q < q_len;
@@ -217,8 +249,8 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     const int64_t k_len0 = min(p.k_tile, p.k_seq);
     const bool one_tile = p.n_kv_tiles == 1;
     const int64_t entry_rows0 = p.kv_rows > 0 ? p.kv_rows : k_len0;
-    const char *K0 = static_cast<const char *>(p.K[0]) + ((int64_t)kvb * entry_rows0) * RB;
-    const char *V0 = static_cast<const char *>(p.V[0]) + ((int64_t)kvb * entry_rows0) * RB;
+    const char *K0 = static_cast<const char *>(p.K[k_tile0]) + ((int64_t)kvb * entry_rows0) * RB;
+    const char *V0 = static_cast<const char *>(p.V[k_tile0]) + ((int64_t)kvb * entry_rows0) * RB;
     auto locate = [&](int g) -> StepSource
     {
         StepSource src;
@@ -234,8 +266,8 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
             const int kb = g % p.k_blocks_per_tile;
             const int64_t k_len = min(p.k_tile, p.k_seq - (int64_t)kt * p.k_tile);
             const int64_t off = ((int64_t)kvb * k_len + (int64_t)kb * kKeys32) * RB;
-            src.K = static_cast<const char *>(p.K[kt]) + off;
-            src.V = static_cast<const char *>(p.V[kt]) + off;
+            src.K = static_cast<const char *>(p.K[k_tile0 + kt]) + off;
+            src.V = static_cast<const char *>(p.V[k_tile0 + kt]) + off;
             src.rows_left = (int)k_len - kb * kKeys32;
         }
         return src;
@@ -817,7 +849,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
     }
     const float to_ln = EXPLICIT ? 1.0f : p.scale;
     const float lse_new = empty ? neg_inf() : m_run * to_ln + __logf(l_tot);
-    float *lse_ptr = p.lse[qt] + (int64_t)b * q_len + my_q;
+    float *lse_ptr = p.lse[q_tile0 + qt] + (int64_t)b * q_len + my_q;
     const float lse_old = p.overwrite ? neg_inf() : *lse_ptr;
     float w_old = 0.0f, w_new = 0.0f, lse_out = neg_inf();
     if(!empty)
@@ -829,7 +861,7 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         *lse_ptr = lse_out;
     }
     const float w_o = empty ? 0.0f : w_new / l_tot;
-    float *Arow = static_cast<float *>(p.A[qt])
+    float *Arow = static_cast<float *>(p.A[q_tile0 + qt])
         + ((int64_t)b * q_len + my_q) * HEAD;
 #pragma unroll
     for(int db = 0; db < DBLOCKS; ++db)
@@ -904,12 +936,13 @@ int launch_prefill_fp32(hipStream_t stream, PrefillParams &p, int head, int mode
     // half of such a workgroup's wavefronts would have no rows (the new tokens
     // of a decode step), 32-query workgroups whose wavefronts share the keys
     // instead
-    const int64_t n_wide = (int64_t)p.batch * p.n_q_tiles
+    const int64_t batch_all = (int64_t)p.batch * p.n_slabs;
+    const int64_t n_wide = batch_all * p.n_q_tiles
         * ((p.q_tile + kQRows32 - 1) / kQRows32);
-    const bool split = n_wide < 256 || p.q_tile <= 64;
+    const bool split = n_wide < split_below(head, mode) || p.q_tile <= 64;
     const int q_rows = split ? 32 : kQRows32;
     p.q_blocks_per_tile = (int)((p.q_tile + q_rows - 1) / q_rows);
-    const int64_t n_wg = (int64_t)p.batch * p.n_q_tiles * p.q_blocks_per_tile;
+    const int64_t n_wg = batch_all * p.n_q_tiles * p.q_blocks_per_tile;
     if(n_wg <= 0 || n_wg > 0x7fffffff)
     {
         return NNTILE_HIP_EINVAL;

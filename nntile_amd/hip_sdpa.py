@@ -45,6 +45,7 @@ class GridArgs(ctypes.Structure):
                 ("n_batch", _i64), ("kv_group", _i64),
                 ("mask_mode", ctypes.c_int32), ("n_q_tiles", ctypes.c_int32),
                 ("n_kv_tiles", ctypes.c_int32), ("flags", ctypes.c_int32),
+                ("n_slabs", ctypes.c_int32), ("reserved", ctypes.c_int32),
                 ("q_pos0", _i64), ("k_pos0", _i64), ("causal_offset", _i64),
                 ("K", _vp * MAX_TILES), ("V", _vp * MAX_TILES),
                 ("Q", _vp * MAX_TILES), ("lse", _vp * MAX_TILES),
@@ -317,13 +318,13 @@ def sdpa_bwd_tile(K, Q, V, A, dA, mask, lse, dK, dQ, dV, mask_mode, n_batch=None
     _check(fn(_stream(stream), ctypes.byref(a)), "sdpa_bwd_tile")
 
 
-def sdpa_fwd_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq,
-                  q_tile, k_tile, mask_mode, n_batch=None, kv_group=1,
-                  q_pos0=0, k_pos0=0, causal_offset=0, flags=0, stream=None):
-    """All key tiles merged into all query tiles in one launch.  Tiles are
-    lists of separately allocated tensors [batch, rows, head]."""
+def _grid_args(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq, q_tile, k_tile,
+               mask_mode, n_batch, kv_group, q_pos0, k_pos0, causal_offset, flags, n_slabs):
     _dev(*K_tiles, *Q_tiles, *lse_tiles, *V_tiles, *A_tiles)
     batch, _, head = Q_tiles[0].shape
+    if (len(Q_tiles) > MAX_TILES or len(K_tiles) > MAX_TILES or n_slabs < 1
+            or len(Q_tiles) % n_slabs or len(K_tiles) % n_slabs):
+        raise SdpaError(EINVAL, "sdpa_fwd_grid")
     a = GridArgs()
     a.q_seq, a.k_seq, a.q_tile, a.k_tile, a.head = q_seq, k_seq, q_tile, k_tile, head
     a.batch = batch
@@ -331,14 +332,25 @@ def sdpa_fwd_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq,
     a.kv_group = kv_group
     a.mask_mode = mask_mode
     a.flags = flags
-    a.n_q_tiles, a.n_kv_tiles = len(Q_tiles), len(K_tiles)
+    a.n_slabs = n_slabs
+    a.n_q_tiles, a.n_kv_tiles = len(Q_tiles) // n_slabs, len(K_tiles) // n_slabs
     a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
-    if len(Q_tiles) > MAX_TILES or len(K_tiles) > MAX_TILES:
-        raise SdpaError(EINVAL, "sdpa_fwd_grid")
     for i, (k, v) in enumerate(zip(K_tiles, V_tiles)):
         a.K[i], a.V[i] = k.data_ptr(), v.data_ptr()
     for i, (q, l, o) in enumerate(zip(Q_tiles, lse_tiles, A_tiles)):
         a.Q[i], a.lse[i], a.A[i] = q.data_ptr(), l.data_ptr(), o.data_ptr()
+    return a
+
+
+def sdpa_fwd_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq,
+                  q_tile, k_tile, mask_mode, n_batch=None, kv_group=1,
+                  q_pos0=0, k_pos0=0, causal_offset=0, flags=0, stream=None, n_slabs=1):
+    """All key tiles merged into all query tiles in one launch.  Tiles are
+    lists of separately allocated tensors [batch, rows, head]; with n_slabs > 1
+    the lists hold the tiles of slab 0, then those of slab 1, ... (the tiles
+    along the batch axes, `batch` entries each)."""
+    a = _grid_args(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq, q_tile, k_tile,
+                   mask_mode, n_batch, kv_group, q_pos0, k_pos0, causal_offset, flags, n_slabs)
     fn = getattr(lib(), "nntile_hip_sdpa_fwd_grid_" + dtype_name(Q_tiles[0]))
     _check(fn(_stream(stream), ctypes.byref(a)), "sdpa_fwd_grid")
     return a
@@ -438,24 +450,10 @@ class FlashPlan:
 
 
 def plan_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq, q_tile, k_tile,
-              mask_mode, n_batch=None, kv_group=1, q_pos0=0, k_pos0=0, causal_offset=0, flags=0):
-    _dev(*K_tiles, *Q_tiles, *lse_tiles, *V_tiles, *A_tiles)
-    batch, _, head = Q_tiles[0].shape
-    if len(Q_tiles) > MAX_TILES or len(K_tiles) > MAX_TILES:
-        raise SdpaError(EINVAL, "sdpa_fwd_grid")
-    a = GridArgs()
-    a.q_seq, a.k_seq, a.q_tile, a.k_tile, a.head = q_seq, k_seq, q_tile, k_tile, head
-    a.batch = batch
-    a.n_batch = batch if n_batch is None else n_batch
-    a.kv_group = kv_group
-    a.mask_mode = mask_mode
-    a.flags = flags
-    a.n_q_tiles, a.n_kv_tiles = len(Q_tiles), len(K_tiles)
-    a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
-    for i, (k, v) in enumerate(zip(K_tiles, V_tiles)):
-        a.K[i], a.V[i] = k.data_ptr(), v.data_ptr()
-    for i, (q, l, o) in enumerate(zip(Q_tiles, lse_tiles, A_tiles)):
-        a.Q[i], a.lse[i], a.A[i] = q.data_ptr(), l.data_ptr(), o.data_ptr()
+              mask_mode, n_batch=None, kv_group=1, q_pos0=0, k_pos0=0, causal_offset=0, flags=0,
+              n_slabs=1):
+    a = _grid_args(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq, q_tile, k_tile,
+                   mask_mode, n_batch, kv_group, q_pos0, k_pos0, causal_offset, flags, n_slabs)
     fn = getattr(lib(), "nntile_hip_sdpa_fwd_grid_" + dtype_name(Q_tiles[0]))
     return Plan(fn, a, "sdpa_fwd_grid",
                 keep=(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles))

@@ -875,7 +875,7 @@ template<> struct GridCall<fp32_t>
 };
 
 template<typename T>
-void flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
+Index flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
         int mask_mode, Index causal_offset, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &V, const Tensor<T> &A, bool overwrite)
 {
@@ -889,56 +889,80 @@ void flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
     const Index n_q = Q.grid.shape[1], n_kv = K.grid.shape[1];
     require(n_q <= NNTILE_HIP_SDPA_MAX_TILES && n_kv <= NNTILE_HIP_SDPA_MAX_TILES,
             "flash_sdpa_fwd_hip: too many sequence tiles for one launch");
-    // One launch per slab of the batch grid: all its query and key tiles
+    // The slabs of the batch grid (each with all its query and key tiles) go
+    // into as few launches as the tile tables hold: slabs with the same
+    // number of entries share a launch, up to NNTILE_HIP_SDPA_MAX_TILES
+    // tiles per axis.
+    struct Slab { Index g2, g3, g4, batch; };
+    std::vector<Slab> slabs;
     for(Index g4 = 0; g4 < Q.grid.shape[4]; ++g4)
     {
         for(Index g3 = 0; g3 < Q.grid.shape[3]; ++g3)
         {
             for(Index g2 = 0; g2 < Q.grid.shape[2]; ++g2)
             {
-                nntile_hip_sdpa_grid_args a;
-                std::memset(&a, 0, sizeof(a));
                 const auto &q0 = Q.get_tile({0, 0, g2, g3, g4});
-                a.q_seq = Q.shape[1];
-                a.k_seq = K.shape[1];
-                a.q_tile = Q.basetile_shape[1];
-                a.k_tile = K.basetile_shape[1];
-                a.head = Q.shape[0];
-                a.batch = q0.shape[2] * q0.shape[3] * q0.shape[4];
-                a.n_batch = a.batch;
-                a.kv_group = 1;
-                a.mask_mode = mask_mode;
-                a.flags = overwrite ? NNTILE_HIP_SDPA_OVERWRITE : 0;
-                a.n_q_tiles = static_cast<std::int32_t>(n_q);
-                a.n_kv_tiles = static_cast<std::int32_t>(n_kv);
-                a.causal_offset = causal_offset;
-                for(Index t = 0; t < n_kv; ++t)
-                {
-                    a.K[t] = K.get_tile({0, t, g2, g3, g4}).get_ptr();
-                    a.V[t] = V.get_tile({0, t, g2, g3, g4}).get_ptr();
-                }
-                for(Index t = 0; t < n_q; ++t)
-                {
-                    a.Q[t] = Q.get_tile({0, t, g2, g3, g4}).get_ptr();
-                    a.A[t] = A.get_tile({0, t, g2, g3, g4}).get_ptr();
-                    a.lse[t] = static_cast<float *>(
-                            logsumexp.get_tile({t, g2, g3, g4}).get_ptr());
-                }
-                for(Index t = 0; t < n_q; ++t)
-                {
-                    A.get_tile({0, t, g2, g3, g4}).mark_written();
-                    logsumexp.get_tile({t, g2, g3, g4}).mark_written();
-                }
-                starpu::count_direct_launch();
-                const int rc = GridCall<T>::run(starpu::get_local_stream(), &a);
-                if(rc != NNTILE_HIP_OK)
-                {
-                    throw std::runtime_error("Error in flash_sdpa_fwd_hip launch (code "
-                            + std::to_string(rc) + ")");
-                }
+                slabs.push_back({g2, g3, g4, q0.shape[2] * q0.shape[3] * q0.shape[4]});
             }
         }
     }
+    const std::size_t per_launch = static_cast<std::size_t>(
+            NNTILE_HIP_SDPA_MAX_TILES / std::max(n_q, n_kv));
+    Index launches = 0;
+    for(std::size_t first = 0; first < slabs.size();)
+    {
+        std::size_t count = 1;
+        while(first + count < slabs.size() && count < per_launch
+                && slabs[first + count].batch == slabs[first].batch)
+        {
+            ++count;
+        }
+        nntile_hip_sdpa_grid_args a;
+        std::memset(&a, 0, sizeof(a));
+        a.q_seq = Q.shape[1];
+        a.k_seq = K.shape[1];
+        a.q_tile = Q.basetile_shape[1];
+        a.k_tile = K.basetile_shape[1];
+        a.head = Q.shape[0];
+        a.batch = slabs[first].batch;
+        a.n_batch = a.batch;
+        a.kv_group = 1;
+        a.mask_mode = mask_mode;
+        a.flags = overwrite ? NNTILE_HIP_SDPA_OVERWRITE : 0;
+        a.n_q_tiles = static_cast<std::int32_t>(n_q);
+        a.n_kv_tiles = static_cast<std::int32_t>(n_kv);
+        a.n_slabs = static_cast<std::int32_t>(count);
+        a.causal_offset = causal_offset;
+        for(std::size_t s = 0; s < count; ++s)
+        {
+            const Index g2 = slabs[first + s].g2, g3 = slabs[first + s].g3,
+                  g4 = slabs[first + s].g4;
+            for(Index t = 0; t < n_kv; ++t)
+            {
+                a.K[s * n_kv + t] = K.get_tile({0, t, g2, g3, g4}).get_ptr();
+                a.V[s * n_kv + t] = V.get_tile({0, t, g2, g3, g4}).get_ptr();
+            }
+            for(Index t = 0; t < n_q; ++t)
+            {
+                a.Q[s * n_q + t] = Q.get_tile({0, t, g2, g3, g4}).get_ptr();
+                a.A[s * n_q + t] = A.get_tile({0, t, g2, g3, g4}).get_ptr();
+                a.lse[s * n_q + t] = static_cast<float *>(
+                        logsumexp.get_tile({t, g2, g3, g4}).get_ptr());
+                A.get_tile({0, t, g2, g3, g4}).mark_written();
+                logsumexp.get_tile({t, g2, g3, g4}).mark_written();
+            }
+        }
+        starpu::count_direct_launch();
+        const int rc = GridCall<T>::run(starpu::get_local_stream(), &a);
+        if(rc != NNTILE_HIP_OK)
+        {
+            throw std::runtime_error("Error in flash_sdpa_fwd_hip launch (code "
+                    + std::to_string(rc) + ")");
+        }
+        first += count;
+        ++launches;
+    }
+    return launches;
 }
 
 template<typename T> struct TileCall;
@@ -1095,8 +1119,7 @@ Index flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
     if(whole >= 0 && Q.grid.shape[1] <= NNTILE_HIP_SDPA_MAX_TILES
             && num_k_seq_tiles <= NNTILE_HIP_SDPA_MAX_TILES)
     {
-        flash_sdpa_fwd_hip_async<T>(K, Q, whole, causal_offset, logsumexp, V, A, false);
-        return Q.grid.shape[2] * Q.grid.shape[3] * Q.grid.shape[4];
+        return flash_sdpa_fwd_hip_async<T>(K, Q, whole, causal_offset, logsumexp, V, A, false);
     }
     Index submitted = 0;
     for(Index a_linear = 0; a_linear < A.grid.nelems; ++a_linear)
@@ -1542,7 +1565,7 @@ NNTILE_HOST_INSTANTIATE_TENSOR_BWD(fp16_t)
             const Tensor<T> &, const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &); \
     template void flash_sdpa_fwd_cudnn<T>(const Tensor<T> &, const Tensor<T> &, \
             const Tensor<T> &, const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &); \
-    template void flash_sdpa_fwd_hip_async<T>(const Tensor<T> &, const Tensor<T> &, int, \
+    template Index flash_sdpa_fwd_hip_async<T>(const Tensor<T> &, const Tensor<T> &, int, \
             Index, const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, bool); \
     template std::vector<int> flash_sdpa_mask_classes<T>(const Tensor<T> &, Index); \
     template std::vector<int> flash_sdpa_cached_mask_classes<T>(const Tensor<T> &, Index); \

@@ -317,10 +317,13 @@ void flash_sdpa_fwd_cudnn(const Tensor<T> &K, const Tensor<T> &Q,
 
 //! Same result with an analytic mask (mask_mode NNTILE_HIP_MASK_NONE or
 //! NNTILE_HIP_MASK_CAUSAL with `causal_offset`): for every (batch, group,
-//! head) slab all key tiles are merged into all query tiles in ONE launch.
+//! head) slab all key tiles are merged into all query tiles in ONE launch,
+//! and slabs with the same number of entries share a launch as far as its
+//! tile tables reach (NNTILE_HIP_SDPA_MAX_TILES tiles per axis).
 //! `overwrite` = the running pair need not be initialised by the caller.
+//! Returns the number of launches.
 template<typename T>
-void flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
+Index flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
         int mask_mode, Index causal_offset, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &V, const Tensor<T> &A, bool overwrite);
 
@@ -338,8 +341,8 @@ int flash_sdpa_mask_rule(const TensorTraits &mask, const std::vector<int> &mask_
         Index causal_offset);
 
 //! flash_sdpa_fwd_cudnn_async that uses those classes.  A mask that is the
-//! causal rule itself (or hides nothing) runs as flash_sdpa_fwd_hip_async:
-//! one launch per slab of the batch grid.  Otherwise, per pair: a mask tile
+//! causal rule itself (or hides nothing) runs as flash_sdpa_fwd_hip_async.
+//! Otherwise, per pair: a mask tile
 //! that hides everything - nothing submitted; one that hides nothing - no
 //! mask; one on the causal rule - the analytic mask; the rest as in the
 //! reference.  Returns the number of launches.

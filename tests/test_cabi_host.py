@@ -25,7 +25,8 @@ def test_library_exports_every_declared_symbol():
 
 def test_struct_layouts_match_header():
     assert ctypes.sizeof(h.TileArgs) == 6 * 8 + 8 + 3 * 8 + 6 * 8
-    assert ctypes.sizeof(h.GridArgs) == 8 * 8 + 16 + 3 * 8 + 5 * 64 * 8
+    assert ctypes.sizeof(h.GridArgs) == 8 * 8 + 16 + 8 + 3 * 8 + 5 * 64 * 8
+    assert h.GridArgs.n_slabs.offset == 8 * 8 + 16 and h.GridArgs.q_pos0.offset == 8 * 8 + 24
     assert ctypes.sizeof(h.FlashClArgs) == 32
     assert ctypes.sizeof(h.VariableInterface) == 40
 
@@ -70,6 +71,12 @@ def test_bad_arguments_are_rejected_before_launch(t):
     assert grid(None, ctypes.byref(g)) == h.EUNSUPPORTED
     g.mask_mode = h.MASK_CAUSAL
     assert grid(None, ctypes.byref(g)) == h.EINVAL                         # null tile pointers
+    g.n_slabs = 17                                                          # 17 * 4 tiles > 64
+    for i in range(64):
+        g.K[i] = g.V[i] = g.Q[i] = g.lse[i] = g.A[i] = 4096
+    assert grid(None, ctypes.byref(g)) == h.EINVAL
+    g.n_slabs = -1
+    assert grid(None, ctypes.byref(g)) == h.EINVAL
 
 
 def test_decode_argument_checks():

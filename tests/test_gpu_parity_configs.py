@@ -65,6 +65,27 @@ def test_cfg2_gpt2_small_fp32(oracle):
     H.check_rows(A_all.reshape(want.shape), want, lse_all.reshape(want_lse.shape), want_lse, "fp32", "cfg2")
 
 
+def test_cfg2_gpt2_small_fp32_one_launch(oracle):
+    """The same four (batch, head-tile) slabs as separate allocations in ONE
+    launch with the analytic causal mask (what the tensor-level call submits
+    once the mask's tiles are known to be the causal rule)."""
+    cfg = BY_NAME["cfg2_gpt2_small_fp32"]
+    (Q, K, V), (qf, kf, vf) = _inputs(cfg)
+    want, want_lse = oracle.sdpa_vanilla(kf, qf, vf, synth.causal_mask(cfg.q_seq, cfg.k_seq))
+    shape5 = (cfg.n_head_kv, cfg.n_batch, cfg.q_seq, cfg.head)
+    slab = lambda t: [t.view(shape5)[:, nb].contiguous().cuda() for nb in range(cfg.n_batch)]
+    outs = [H.fresh_outputs(cfg.n_head_kv, cfg.q_seq, cfg.head, "fp32") for _ in range(cfg.n_batch)]
+    hip_sdpa.sdpa_fwd_grid(slab(K), slab(Q), [o[0] for o in outs], slab(V), [o[1] for o in outs],
+                           cfg.q_seq, cfg.k_seq, cfg.seq_tile, cfg.seq_tile, hip_sdpa.MASK_CAUSAL,
+                           n_slabs=cfg.n_batch)
+    torch.cuda.synchronize()
+    A = np.stack([H.to_np(o[1]) for o in outs], axis=1).reshape(want.shape)
+    lse = np.stack([H.to_np(o[0]) for o in outs], axis=1).reshape(want_lse.shape)
+    assert H.rel_fro(A, want) < 1e-4
+    assert H.rel_fro(lse, want_lse) < 1e-4
+    H.check_rows(A, want, lse, want_lse, "fp32", "cfg2 one launch")
+
+
 def _split(t, tile):
     return [t[:, s:s + tile].contiguous().cuda() for s in range(0, t.shape[1], tile)]
 
