@@ -34,8 +34,7 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 TRAFFIC = {
     "cfg3_llama_prefill_bf16": (175127911, "profiles/sdpa_prefill_16bit_kernel_cfg3_llama_prefill_bf16.txt"),
     "cfg4_gqa_decode_bf16": (288075448, "profiles/sdpa_decode_16bit_kernel_cfg4_gqa_decode_bf16.txt"),
-    # per step = four launches
-    "cfg2_gpt2_small_fp32": (75873356, "profiles/sdpa_prefill_fp32_kernel_cfg2_gpt2_small_fp32.txt"),
+    "cfg2_gpt2_small_fp32": (55549952, "profiles/sdpa_prefill_fp32_kernel_cfg2_gpt2_small_fp32.txt"),
 }
 
 

@@ -44,7 +44,22 @@ constexpr int kDecodeCUs = 256;   // MI355X
 #ifndef NNTILE_DEC_PART16
 #define NNTILE_DEC_PART16 1
 #endif
+// How the partial outputs are stored: 0 plain, 1 non-temporal, 2 / 3 written
+// through at system / device scope
+#ifndef NNTILE_DEC_PART_STORE
+#define NNTILE_DEC_PART_STORE 0
+#endif
 typedef __attribute__((ext_vector_type(4))) float acc4;
+
+// Developer build (-DNNTILE_DEC_TRACE): wall-clock stamps (100 MHz) of every
+// workgroup of the last launch, read back with nntile_hip_debug_dec_trace.
+#ifdef NNTILE_DEC_TRACE
+__device__ unsigned long long dec_trace[8 * 2048];
+#define DEC_STAMP(i) do { if(__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) == 0 \
+        && blockIdx.x < 2048) { dec_trace[8 * blockIdx.x + (i)] = wall_clock64(); } } while(0)
+#else
+#define DEC_STAMP(i)
+#endif
 
 template<typename T> struct Mfma16;
 template<> struct Mfma16<Bf16>
@@ -118,6 +133,7 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         else { return ring3; }
     };
 
+    DEC_STAMP(0);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -303,6 +319,10 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         // ring is there to avoid.  LDS reads are ordered by lgkmcnt, the
         // loads by the explicit vmcnt above.
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#ifdef NNTILE_DEC_TRACE
+        if(it == 0) { DEC_STAMP(1); }
+        if(it == n_local - 1) { DEC_STAMP(2); }
+#endif
         {
             const int ahead = it + STAGES - 1;
             if(ahead < n_local)
@@ -469,6 +489,7 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
     }
 
     // ---- write the partial ---------------------------------------------------------
+    DEC_STAMP(3);
     float l_tot = l_run + __shfl_xor(l_run, 16);
     l_tot = sum_across_halves(l_tot);
     if(!row_ok)
@@ -550,8 +571,22 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         u32x2 w;
         w[0] = T::pack2(o[db][0] * inv, o[db][1] * inv);
         w[1] = T::pack2(o[db][2] * inv, o[db][3] * inv);
+#if NNTILE_DEC_PART_STORE == 1
+        __builtin_nontemporal_store(w, reinterpret_cast<u32x2 *>(dst + 16 * db));
+#elif NNTILE_DEC_PART_STORE == 2
+        __hip_atomic_store(reinterpret_cast<unsigned long long *>(dst + 16 * db),
+                __builtin_bit_cast(unsigned long long, w), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+#elif NNTILE_DEC_PART_STORE == 3
+        __hip_atomic_store(reinterpret_cast<unsigned long long *>(dst + 16 * db),
+                __builtin_bit_cast(unsigned long long, w), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#else
         *reinterpret_cast<u32x2 *>(dst + 16 * db) = w;
+#endif
     }
+#ifdef NNTILE_DEC_TRACE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    DEC_STAMP(4);
+#endif
 #else
     float *dst = p.part_o + prow * HEAD + 4 * quad;
 #pragma unroll
@@ -569,6 +604,7 @@ template<typename T, int HEAD>
 __global__ __launch_bounds__(256)
 void sdpa_decode_reduce_kernel(const DecodeParams p)
 {
+    DEC_STAMP(5);
     constexpr int TPR = HEAD / 4;               // threads per row
     constexpr int ROWS_PER_WG = 256 / TPR;
     const int64_t total_rows = (int64_t)p.n_batch * p.n_head_kv * p.rows;
@@ -728,7 +764,18 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
     {
         p.lse[row] = lse_out;
     }
+#ifdef NNTILE_DEC_TRACE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    DEC_STAMP(6);
+#endif
 }
+
+#ifdef NNTILE_DEC_TRACE
+extern "C" int nntile_hip_debug_dec_trace(unsigned long long *host)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(dec_trace), sizeof(dec_trace));
+}
+#endif
 
 template<typename T, int HEAD, int MODE, int STAGES>
 static void launch_decode_main(hipStream_t stream, const DecodeParams &p, dim3 grid)
