@@ -64,10 +64,30 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const char *lds_ptr)
     return __builtin_bit_cast(u32x2, v);
 }
 
+// Developer build (-DNNTILE_PF_TRACE): wall-clock stamps (100 MHz) of every
+// workgroup of the last launch - start, first step in LDS, end of the
+// pipelined loop, end of the key steps, end - plus where it ran and how many
+// steps it had; read back with nntile_hip_debug_pf_trace.
+#ifdef NNTILE_PF_TRACE
+__device__ unsigned long long pf_trace[8 * 4096];
+#define PF_STAMP(i) do { if(__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) == 0 \
+        && blockIdx.x < 4096) { pf_trace[8 * blockIdx.x + (i)] = wall_clock64(); } } while(0)
+#define PF_NOTE(i, v) do { if(__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) == 0 \
+        && blockIdx.x < 4096) { pf_trace[8 * blockIdx.x + (i)] = (unsigned long long)(v); } } while(0)
+extern "C" int nntile_hip_debug_pf_trace(unsigned long long *host)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(pf_trace), sizeof(pf_trace));
+}
+#else
+#define PF_STAMP(i)
+#define PF_NOTE(i, v)
+#endif
+
 template<typename T, int HEAD, int MODE>
 __global__ __launch_bounds__(kThreads, 2)
 void sdpa_prefill_16bit_kernel(const PrefillParams p)
 {
+    PF_STAMP(0);
     typedef typename T::vec8 vec8;
     constexpr int KSTEPS = HEAD / 16;       // MFMA steps along head for S
     constexpr int DBLOCKS = HEAD / 32;      // 32-row blocks of O^T
@@ -621,6 +641,10 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    PF_STAMP(1);
+    PF_NOTE(5, ((unsigned long long)__builtin_amdgcn_s_getreg(63508) << 32)
+            | (unsigned)__builtin_amdgcn_s_getreg(63492));
+    PF_NOTE(6, ((unsigned long long)(unsigned)n_steps << 32) | (unsigned)(b * 1024 + qblk));
 
     // One key step on LDS buffer BUF (a compile-time constant, so that every
     // LDS address is a fixed register plus an immediate).
@@ -1215,6 +1239,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         __syncthreads();
     }
 
+    PF_STAMP(2);
     {
         int g = g_first;
         if(g < n_steps && (g & 1))
@@ -1232,6 +1257,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         }
     }
     NNTILE_PHASE_DUMP()
+    PF_STAMP(3);
 
     // ---- epilogue: normalise, merge into the running (lse, A) ----------------
     const float l_tot = sum_across_halves(l_run);
@@ -1291,6 +1317,10 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 *reinterpret_cast<u32x4 *>(Abase + (int64_t)r * RB + c * 16) = v;
             }
         }
+#ifdef NNTILE_PF_TRACE
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        PF_STAMP(4);
+#endif
         return;
     }
     if(!live)
