@@ -45,6 +45,12 @@ extern "C" {
  * A = 0.  Saves the fill of lse (wrappers/python/nntile/layer/sdpa.py:538-539)
  * and one read of A when the caller knows this is the first key tile. */
 #define NNTILE_HIP_SDPA_OVERWRITE 1
+/* fp32 tile and grid calls, for tests and tuning: fix the workgroup shape
+ * instead of letting the size of the launch pick it - 128 queries sharing
+ * every key step (SHARED), or 32 queries whose four wavefronts split the key
+ * steps (SPLIT).  Both set, or a 16-bit call: ignored. */
+#define NNTILE_HIP_SDPA_FORM_SHARED 0x100
+#define NNTILE_HIP_SDPA_FORM_SPLIT  0x200
 
 /* How visibility of key k to query q is given. */
 enum nntile_hip_mask_mode

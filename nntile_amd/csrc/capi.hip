@@ -58,6 +58,14 @@ static bool mode_ok(int mode)
     return mode >= NNTILE_HIP_MASK_ADDITIVE && mode <= NNTILE_HIP_MASK_BOOL;
 }
 
+// the workgroup shape a caller asked for (fp32 kernels): 0 none, 1 shared, 2 split
+static int prefill_form(int32_t flags)
+{
+    const bool shared = (flags & NNTILE_HIP_SDPA_FORM_SHARED) != 0;
+    const bool split = (flags & NNTILE_HIP_SDPA_FORM_SPLIT) != 0;
+    return shared == split ? 0 : (shared ? 1 : 2);
+}
+
 static int dispatch_prefill(DType dt, hipStream_t stream, PrefillParams &p,
         int64_t head, int mode, void *scan_scratch = nullptr,
         size_t scan_scratch_bytes = 0)
@@ -122,6 +130,7 @@ static int tile_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a,
     p.n_batch = (int32_t)a->n_batch;
     p.kv_group = (int32_t)a->kv_group;
     p.overwrite = (a->flags & NNTILE_HIP_SDPA_OVERWRITE) ? 1 : 0;
+    p.form = prefill_form(a->flags);
     p.K[0] = a->K;
     p.V[0] = a->V;
     p.Q[0] = a->Q;
@@ -406,6 +415,7 @@ static int grid_call(DType dt, void *stream, const nntile_hip_sdpa_grid_args *a)
     p.n_batch = (int32_t)a->n_batch;
     p.kv_group = (int32_t)a->kv_group;
     p.overwrite = (a->flags & NNTILE_HIP_SDPA_OVERWRITE) ? 1 : 0;
+    p.form = prefill_form(a->flags);
     for(int t = 0; t < n_kv_all; ++t)
     {
         if(a->K[t] == nullptr || a->V[t] == nullptr || !aligned16(a->K[t])

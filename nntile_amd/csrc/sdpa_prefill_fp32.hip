@@ -939,7 +939,8 @@ int launch_prefill_fp32(hipStream_t stream, PrefillParams &p, int head, int mode
     const int64_t batch_all = (int64_t)p.batch * p.n_slabs;
     const int64_t n_wide = batch_all * p.n_q_tiles
         * ((p.q_tile + kQRows32 - 1) / kQRows32);
-    const bool split = n_wide < split_below(head, mode) || p.q_tile <= 64;
+    const bool split = p.form != 0 ? p.form == 2
+        : (n_wide < split_below(head, mode) || p.q_tile <= 64);
     const int q_rows = split ? 32 : kQRows32;
     p.q_blocks_per_tile = (int)((p.q_tile + q_rows - 1) / q_rows);
     const int64_t n_wg = batch_all * p.n_q_tiles * p.q_blocks_per_tile;

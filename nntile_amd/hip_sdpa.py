@@ -20,6 +20,7 @@ MASK_ADDITIVE, MASK_NONE, MASK_CAUSAL, MASK_BOOL = 0, 1, 2, 3
 MAX_TILES = 64
 BWD_MAX_TILES = 32
 OVERWRITE = 1
+FORM_SHARED, FORM_SPLIT = 0x100, 0x200     # fp32 calls: fix the workgroup shape (tests, tuning)
 
 OK, EINVAL, EUNSUPPORTED, ELAUNCH, EWORKSPACE = 0, -1, -2, -3, -4
 TILE_MIXED, TILE_OPEN, TILE_HIDDEN, TILE_CAUSAL = 0, 1, 2, 3
