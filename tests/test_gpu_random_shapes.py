@@ -9,6 +9,8 @@ sequence lengths against every head size and type, grouped heads with ragged
 key tiles, causal offsets that hide whole query rows (negative) or nothing,
 random masks with rows that see no key, overwrite against merge into a fresh
 pair, and positions of the pair inside a larger sequence."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -18,8 +20,10 @@ from . import helpers as H
 
 pytestmark = pytest.mark.gpu
 
-N_FORWARD = 160
-N_BACKWARD = 48
+# (the environment variables widen the sweep for a one-off run; the cases of
+# the default run are a prefix of it)
+N_FORWARD = int(os.environ.get("NNTILE_SWEEP_FORWARD", "160"))
+N_BACKWARD = int(os.environ.get("NNTILE_SWEEP_BACKWARD", "48"))
 BWD_TOL = {"bf16": 1e-2, "fp16": 2e-3}
 
 
