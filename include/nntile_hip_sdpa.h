@@ -239,8 +239,14 @@ int nntile_hip_sdpa_fwd_grid_fp32(void *stream, const nntile_hip_sdpa_grid_args 
  * NNTILE_HIP_EUNSUPPORTED and are served pair by pair through
  * nntile_hip_sdpa_bwd_tile_*.  Only the analytic masks (NONE, CAUSAL).
  * flags: NNTILE_HIP_SDPA_OVERWRITE writes the gradients instead of adding to
- * them.  workspace: q_seq*batch floats of device memory, 4-byte aligned,
- * private to the call until it has completed. */
+ * them.  n_slabs > 1 (0 stands for 1) puts several slabs of the batch grid,
+ * each `batch` entries in tiles of its own with the same extents, into the
+ * one call, slab s's tiles at [s*n_q_tiles + t] / [s*n_kv_tiles + t] of the
+ * tables as in nntile_hip_sdpa_grid_args; n_slabs*n_q_tiles and
+ * n_slabs*n_kv_tiles must not exceed NNTILE_HIP_SDPA_BWD_MAX_TILES.
+ * workspace: n_slabs*q_seq*batch floats of device memory
+ * (nntile_hip_sdpa_bwd_grid_workspace_bytes), 4-byte aligned, private to the
+ * call until it has completed. */
 #define NNTILE_HIP_SDPA_BWD_MAX_TILES 32
 
 typedef struct nntile_hip_sdpa_bwd_grid_args
@@ -248,6 +254,7 @@ typedef struct nntile_hip_sdpa_bwd_grid_args
     int64_t q_seq, k_seq, q_tile, k_tile, head;
     int64_t batch, n_batch, kv_group;
     int32_t mask_mode, n_q_tiles, n_kv_tiles, flags;
+    int32_t n_slabs, reserved;
     int64_t q_pos0, k_pos0, causal_offset;
     const void *K[NNTILE_HIP_SDPA_BWD_MAX_TILES];
     const void *V[NNTILE_HIP_SDPA_BWD_MAX_TILES];

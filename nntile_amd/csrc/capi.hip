@@ -228,7 +228,15 @@ static int bwd_grid_call(DType dt, void *stream, const nntile_hip_sdpa_bwd_grid_
             || a->batch > 0x7fffffff || a->q_seq > 0x7fffffff
             || a->k_seq > 0x7fffffff
             || a->n_q_tiles <= 0 || a->n_q_tiles > NNTILE_HIP_SDPA_BWD_MAX_TILES
-            || a->n_kv_tiles <= 0 || a->n_kv_tiles > NNTILE_HIP_SDPA_BWD_MAX_TILES)
+            || a->n_kv_tiles <= 0 || a->n_kv_tiles > NNTILE_HIP_SDPA_BWD_MAX_TILES
+            || a->n_slabs < 0 || a->n_slabs > NNTILE_HIP_SDPA_BWD_MAX_TILES)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    const int n_slabs = a->n_slabs == 0 ? 1 : a->n_slabs;
+    const int n_q_all = n_slabs * a->n_q_tiles, n_kv_all = n_slabs * a->n_kv_tiles;
+    if(n_q_all > NNTILE_HIP_SDPA_BWD_MAX_TILES || n_kv_all > NNTILE_HIP_SDPA_BWD_MAX_TILES
+            || a->batch * n_slabs > 0x7fffffff)
     {
         return NNTILE_HIP_EINVAL;
     }
@@ -251,7 +259,7 @@ static int bwd_grid_call(DType dt, void *stream, const nntile_hip_sdpa_bwd_grid_
     {
         return NNTILE_HIP_EUNSUPPORTED;
     }
-    const size_t d_bytes = (size_t)a->q_seq * (size_t)a->batch * sizeof(float);
+    const size_t d_bytes = (size_t)n_slabs * (size_t)a->q_seq * (size_t)a->batch * sizeof(float);
     if(a->workspace == nullptr || a->workspace_bytes < d_bytes
             || (reinterpret_cast<uintptr_t>(a->workspace) & 3u) != 0)
     {
@@ -259,6 +267,9 @@ static int bwd_grid_call(DType dt, void *stream, const nntile_hip_sdpa_bwd_grid_
     }
     BwdGridParams p;
     std::memset(static_cast<void *>(&p), 0, sizeof(p));
+    p.n_slabs = n_slabs;
+    p.n_q_tiles = a->n_q_tiles;
+    p.n_kv_tiles = a->n_kv_tiles;
     p.q_seq = a->q_seq;
     p.k_seq = a->k_seq;
     p.q_tile = a->q_tile;
@@ -272,7 +283,7 @@ static int bwd_grid_call(DType dt, void *stream, const nntile_hip_sdpa_bwd_grid_
     p.kv_group = (int32_t)a->kv_group;
     p.overwrite = (a->flags & NNTILE_HIP_SDPA_OVERWRITE) ? 1 : 0;
     p.scale = 1.0f / sqrtf(static_cast<float>(a->head));
-    for(int t = 0; t < a->n_kv_tiles; ++t)
+    for(int t = 0; t < n_kv_all; ++t)
     {
         if(a->K[t] == nullptr || a->V[t] == nullptr || a->dK[t] == nullptr
                 || a->dV[t] == nullptr || !aligned16(a->K[t]) || !aligned16(a->V[t])
@@ -285,7 +296,7 @@ static int bwd_grid_call(DType dt, void *stream, const nntile_hip_sdpa_bwd_grid_
         p.dKt[t] = a->dK[t];
         p.dVt[t] = a->dV[t];
     }
-    for(int t = 0; t < a->n_q_tiles; ++t)
+    for(int t = 0; t < n_q_all; ++t)
     {
         if(a->Q[t] == nullptr || a->A[t] == nullptr || a->dA[t] == nullptr
                 || a->lse[t] == nullptr || a->dQ[t] == nullptr || !aligned16(a->Q[t])
@@ -966,7 +977,8 @@ size_t nntile_hip_sdpa_bwd_grid_workspace_bytes(const nntile_hip_sdpa_bwd_grid_a
     {
         return 0;
     }
-    return (size_t)a->q_seq * (size_t)a->batch * sizeof(float);
+    const size_t n_slabs = a->n_slabs <= 0 ? 1 : (size_t)a->n_slabs;
+    return n_slabs * (size_t)a->q_seq * (size_t)a->batch * sizeof(float);
 }
 
 int nntile_hip_sdpa_bwd_grid_bf16(void *stream, const nntile_hip_sdpa_bwd_grid_args *args)

@@ -314,7 +314,26 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
     const int q_blocks = (int)((p.q_seq + kBwdRows - 1) / kBwdRows);
     // the last query blocks see the most keys under a causal mask: first
     int b, q_block;
-    map_workgroup(wg, p.batch, q_blocks, true, b, q_block);
+    // (the grid form: the slab of the entry, whose tiles are allocations of
+    // their own)
+    int q_tile0 = 0, k_tile0 = 0;
+    int64_t d_slab = 0;
+    if constexpr(GRID)
+    {
+        map_workgroup(wg, p.batch * p.n_slabs, q_blocks, true, b, q_block);
+        if(p.n_slabs > 1)
+        {
+            const int slab = b / p.batch;
+            b -= slab * p.batch;
+            q_tile0 = slab * p.n_q_tiles;
+            k_tile0 = slab * p.n_kv_tiles;
+            d_slab = (int64_t)slab * p.q_seq * p.batch;
+        }
+    }
+    else
+    {
+        map_workgroup(wg, p.batch, q_blocks, true, b, q_block);
+    }
     const int q_row0 = q_block * kBwdRows;
     const int kvb = kv_entry(b, p.n_batch, p.kv_group);
     const int q_seq = (int)p.q_seq, k_seq = (int)p.k_seq;
@@ -332,11 +351,11 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
         const int tq = q_row0 / q_tile, t0 = tq * q_tile;
         const int rows_t = min(q_tile, q_seq - t0);
         q_elem = (int64_t)b * rows_t + ((q_ok ? my_q : q_row0) - t0);
-        d_idx = (int64_t)p.batch * t0 + q_elem;
-        Q_own = p.Qt[tq];
-        dA_own = p.dAt[tq];
-        dQ_own = p.dQt[tq];
-        lse_own = p.lset[tq];
+        d_idx = d_slab + (int64_t)p.batch * t0 + q_elem;
+        Q_own = p.Qt[q_tile0 + tq];
+        dA_own = p.dAt[q_tile0 + tq];
+        dQ_own = p.dQt[q_tile0 + tq];
+        lse_own = p.lset[q_tile0 + tq];
     }
     const int64_t q_off = q_elem * HEAD;
 
@@ -451,8 +470,8 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
             const int k_tile = (int)p.k_tile;
             const int tk = row0 / k_tile, t0 = tk * k_tile;
             const int64_t off = ((int64_t)kvb * min(k_tile, k_seq - t0) + (row0 - t0)) * RB;
-            return KeyRows{static_cast<const char *>(p.Kt[tk]) + off,
-                static_cast<const char *>(p.Vt[tk]) + off, at_end};
+            return KeyRows{static_cast<const char *>(p.Kt[k_tile0 + tk]) + off,
+                static_cast<const char *>(p.Vt[k_tile0 + tk]) + off, at_end};
         }
         else
         {
@@ -738,7 +757,25 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
     const int k_blocks = (k_seq + kDkvRows - 1) / kDkvRows;
     // the first key blocks are seen by the most queries under a causal mask
     int kvb, k_block;                               // kvb = nb + n_batch*hkv
-    map_workgroup(wg, p.batch / p.kv_group, k_blocks, false, kvb, k_block);
+    int q_tile0 = 0, k_tile0 = 0;
+    int64_t d_slab = 0;
+    if constexpr(GRID)
+    {
+        const int kv_entries = p.batch / p.kv_group;
+        map_workgroup(wg, kv_entries * p.n_slabs, k_blocks, false, kvb, k_block);
+        if(p.n_slabs > 1)
+        {
+            const int slab = kvb / kv_entries;
+            kvb -= slab * kv_entries;
+            q_tile0 = slab * p.n_q_tiles;
+            k_tile0 = slab * p.n_kv_tiles;
+            d_slab = (int64_t)slab * p.q_seq * p.batch;
+        }
+    }
+    else
+    {
+        map_workgroup(wg, p.batch / p.kv_group, k_blocks, false, kvb, k_block);
+    }
     const int k_row0 = k_block * kDkvRows;
     const int nb = kvb % p.n_batch, hkv = kvb / p.n_batch;
     const int my_k = k_row0 + wave * 32 + col;
@@ -752,10 +789,10 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
         const int k_tile = (int)p.k_tile;
         const int tk = k_row0 / k_tile, t0 = tk * k_tile;
         k_elem = (int64_t)kvb * min(k_tile, k_seq - t0) + ((k_ok ? my_k : k_row0) - t0);
-        K_own = p.Kt[tk];
-        V_own = p.Vt[tk];
-        dK_own = p.dKt[tk];
-        dV_own = p.dVt[tk];
+        K_own = p.Kt[k_tile0 + tk];
+        V_own = p.Vt[k_tile0 + tk];
+        dK_own = p.dKt[k_tile0 + tk];
+        dV_own = p.dVt[k_tile0 + tk];
     }
     const int64_t k_off = k_elem * HEAD;
 
@@ -895,7 +932,8 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             const int q_tile = (int)p.q_tile;
             const int tq = row0 / q_tile, t0 = tq * q_tile;
             const int64_t elem = (int64_t)bq * min(q_tile, q_seq - t0) + (row0 - t0);
-            return QueryRows{p.Qt[tq], p.dAt[tq], p.lset[tq], elem, (int64_t)p.batch * t0 + elem};
+            return QueryRows{p.Qt[q_tile0 + tq], p.dAt[q_tile0 + tq], p.lset[q_tile0 + tq], elem,
+                d_slab + (int64_t)p.batch * t0 + elem};
         }
         else
         {
@@ -1337,23 +1375,28 @@ static int launch_bwd_grid_mode(hipStream_t stream, const BwdGridParams &p,
 {
     const int64_t q_blocks = (p.q_seq + kBwdRows - 1) / kBwdRows;
     const int64_t k_blocks = (p.k_seq + kDkvRows - 1) / kDkvRows;
-    const int64_t kv_batch = p.batch / p.kv_group;
-    const int64_t n_dq = (int64_t)p.batch * q_blocks, n_dkv = kv_batch * k_blocks;
+    const int64_t kv_batch = p.batch / p.kv_group * p.n_slabs;
+    const int64_t n_dq = (int64_t)p.batch * p.n_slabs * q_blocks, n_dkv = kv_batch * k_blocks;
     if(n_dq <= 0 || n_dkv <= 0 || n_dq > 0x3fffffff || n_dkv > 0x3fffffff
             || (int64_t)p.batch * p.q_tile * (HEAD / 8) / 256 > 0x7ffffffe)
     {
         return NNTILE_HIP_EINVAL;
     }
-    for(int t = 0; t < n_q_tiles; ++t)
+    for(int s = 0; s < p.n_slabs; ++s)
     {
-        const int64_t t0 = (int64_t)t * p.q_tile;
-        const int64_t rows = (int64_t)p.batch * (p.q_tile < p.q_seq - t0 ? p.q_tile : p.q_seq - t0);
-        hipLaunchKernelGGL((sdpa_bwd_rowdot_kernel<T, HEAD>),
-                dim3((unsigned)((rows * (HEAD / 8) + 255) / 256)), dim3(256), 0, stream,
-                p.dAt[t], A_tiles[t], p.D + (int64_t)p.batch * t0, rows);
-        if(hipGetLastError() != hipSuccess)
+        for(int t = 0; t < n_q_tiles; ++t)
         {
-            return NNTILE_HIP_ELAUNCH;
+            const int64_t t0 = (int64_t)t * p.q_tile;
+            const int64_t rows = (int64_t)p.batch
+                * (p.q_tile < p.q_seq - t0 ? p.q_tile : p.q_seq - t0);
+            hipLaunchKernelGGL((sdpa_bwd_rowdot_kernel<T, HEAD>),
+                    dim3((unsigned)((rows * (HEAD / 8) + 255) / 256)), dim3(256), 0, stream,
+                    p.dAt[s * n_q_tiles + t], A_tiles[s * n_q_tiles + t],
+                    p.D + (int64_t)s * p.q_seq * p.batch + (int64_t)p.batch * t0, rows);
+            if(hipGetLastError() != hipSuccess)
+            {
+                return NNTILE_HIP_ELAUNCH;
+            }
         }
     }
     hipLaunchKernelGGL((sdpa_bwd_kernel<T, HEAD, MODE, true>),

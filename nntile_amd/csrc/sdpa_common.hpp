@@ -126,6 +126,9 @@ constexpr int kBwdMaxTiles = NNTILE_HIP_SDPA_BWD_MAX_TILES;
 struct BwdGridParams : BwdParams
 {
     int64_t q_tile, k_tile;
+    // slabs of `batch` entries each: slab s's tiles sit at [s*n_q_tiles + t] /
+    // [s*n_kv_tiles + t] of the tables, its row dots at D + s*q_seq*batch
+    int32_t n_slabs, n_q_tiles, n_kv_tiles;
     const void *Kt[kBwdMaxTiles];
     const void *Vt[kBwdMaxTiles];
     const void *Qt[kBwdMaxTiles];

@@ -70,6 +70,7 @@ class BwdGridArgs(ctypes.Structure):
                 ("n_batch", _i64), ("kv_group", _i64),
                 ("mask_mode", ctypes.c_int32), ("n_q_tiles", ctypes.c_int32),
                 ("n_kv_tiles", ctypes.c_int32), ("flags", ctypes.c_int32),
+                ("n_slabs", ctypes.c_int32), ("reserved", ctypes.c_int32),
                 ("q_pos0", _i64), ("k_pos0", _i64), ("causal_offset", _i64),
                 ("K", _vp * BWD_MAX_TILES), ("V", _vp * BWD_MAX_TILES),
                 ("Q", _vp * BWD_MAX_TILES), ("A", _vp * BWD_MAX_TILES),
@@ -359,9 +360,10 @@ def sdpa_fwd_grid(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq,
 
 def _bwd_grid_args(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles, dQ_tiles,
                    dV_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, n_batch, kv_group, q_pos0,
-                   k_pos0, causal_offset, flags, workspace):
+                   k_pos0, causal_offset, flags, workspace, n_slabs=1):
     batch, _, head = Q_tiles[0].shape
-    if len(Q_tiles) > BWD_MAX_TILES or len(K_tiles) > BWD_MAX_TILES:
+    if (len(Q_tiles) > BWD_MAX_TILES or len(K_tiles) > BWD_MAX_TILES or n_slabs < 1
+            or len(Q_tiles) % n_slabs or len(K_tiles) % n_slabs):
         raise SdpaError(EINVAL, "sdpa_bwd_grid")
     a = BwdGridArgs()
     a.q_seq, a.k_seq, a.q_tile, a.k_tile, a.head = q_seq, k_seq, q_tile, k_tile, head
@@ -370,7 +372,8 @@ def _bwd_grid_args(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_t
     a.kv_group = kv_group
     a.mask_mode = mask_mode
     a.flags = flags
-    a.n_q_tiles, a.n_kv_tiles = len(Q_tiles), len(K_tiles)
+    a.n_slabs = n_slabs
+    a.n_q_tiles, a.n_kv_tiles = len(Q_tiles) // n_slabs, len(K_tiles) // n_slabs
     a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
     for i, (k, v, dk, dv) in enumerate(zip(K_tiles, V_tiles, dK_tiles, dV_tiles)):
         a.K[i], a.V[i], a.dK[i], a.dV[i] = (t.data_ptr() for t in (k, v, dk, dv))
@@ -383,34 +386,36 @@ def _bwd_grid_args(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_t
 
 def sdpa_bwd_grid(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles, dQ_tiles,
                   dV_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, n_batch=None, kv_group=1,
-                  q_pos0=0, k_pos0=0, causal_offset=0, flags=0, workspace=None, stream=None):
+                  q_pos0=0, k_pos0=0, causal_offset=0, flags=0, workspace=None, stream=None,
+                  n_slabs=1):
     """The backward of every (query tile, key tile) pair in one call: dQ of a
     query tile sums over the key tiles, dK and dV of a key tile over the query
     tiles; the gradients are added to dK, dQ, dV (written with
     flags=OVERWRITE).  Tiles are lists of separately allocated tensors
-    [batch, rows, head] (lse: [batch, rows])."""
+    [batch, rows, head] (lse: [batch, rows]); with n_slabs > 1 the lists hold
+    the tiles of slab 0, then those of slab 1, ..."""
     every = (*K_tiles, *Q_tiles, *V_tiles, *A_tiles, *dA_tiles, *lse_tiles, *dK_tiles,
              *dQ_tiles, *dV_tiles)
     _dev(*every, workspace)
     if workspace is None:
-        workspace = torch.empty(4 * q_seq * Q_tiles[0].shape[0], dtype=torch.uint8,
+        workspace = torch.empty(4 * n_slabs * q_seq * Q_tiles[0].shape[0], dtype=torch.uint8,
                                 device=Q_tiles[0].device)
     a = _bwd_grid_args(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles,
                        dQ_tiles, dV_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, n_batch,
-                       kv_group, q_pos0, k_pos0, causal_offset, flags, workspace)
+                       kv_group, q_pos0, k_pos0, causal_offset, flags, workspace, n_slabs)
     fn = getattr(lib(), "nntile_hip_sdpa_bwd_grid_" + dtype_name(Q_tiles[0]))
     _check(fn(_stream(stream), ctypes.byref(a)), "sdpa_bwd_grid")
 
 
 def plan_bwd_grid(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles, dQ_tiles,
                   dV_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, workspace, n_batch=None,
-                  kv_group=1, q_pos0=0, k_pos0=0, causal_offset=0, flags=0):
+                  kv_group=1, q_pos0=0, k_pos0=0, causal_offset=0, flags=0, n_slabs=1):
     every = (*K_tiles, *Q_tiles, *V_tiles, *A_tiles, *dA_tiles, *lse_tiles, *dK_tiles,
              *dQ_tiles, *dV_tiles, workspace)
     _dev(*every)
     a = _bwd_grid_args(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles,
                        dQ_tiles, dV_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, n_batch,
-                       kv_group, q_pos0, k_pos0, causal_offset, flags, workspace)
+                       kv_group, q_pos0, k_pos0, causal_offset, flags, workspace, n_slabs)
     fn = getattr(lib(), "nntile_hip_sdpa_bwd_grid_" + dtype_name(Q_tiles[0]))
     return Plan(fn, a, "sdpa_bwd_grid", keep=every)
 

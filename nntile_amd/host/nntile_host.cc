@@ -1411,8 +1411,9 @@ static bool bwd_grid_fits(const TensorTraits &K, const TensorTraits &Q)
         && (n_kv == 1 || K.basetile_shape[1] % 128 == 0);
 }
 
-// All (dQ tile, key tile) pairs of a slab of the batch grid in one call, for
-// a mask that is the causal rule or hides nothing: the sums over the pairs
+// All (dQ tile, key tile) pairs of the slabs of the batch grid in as few
+// calls as the tile tables allow, for a mask that is the causal rule or
+// hides nothing: the sums over the pairs
 // (src/tensor/flash_sdpa_bwd_cudnn.cc:172-247) are carried in fp32 inside the
 // kernels instead of through the 16-bit gradient tiles.  Returns the calls.
 template<typename T>
@@ -1422,64 +1423,87 @@ static Index bwd_grid(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV)
 {
     const Index n_q = Q.grid.shape[1], n_kv = K.grid.shape[1];
-    // One workspace for all calls: they run in order on one stream, and each
-    // call writes what it reads there.
-    const std::size_t ws_bytes = sizeof(float) * static_cast<std::size_t>(Q.shape[1]
-            * Q.basetile_shape[2] * Q.basetile_shape[3] * Q.basetile_shape[4]);
-    starpu::VariableHandle workspace(ws_bytes);
-    Index calls = 0;
+    // The slabs of the batch grid go into as few calls as the tile tables
+    // hold: slabs with the same number of entries share a call.
+    struct Slab { Index g2, g3, g4, batch; };
+    std::vector<Slab> slabs;
     for(Index g4 = 0; g4 < Q.grid.shape[4]; ++g4)
     {
         for(Index g3 = 0; g3 < Q.grid.shape[3]; ++g3)
         {
             for(Index g2 = 0; g2 < Q.grid.shape[2]; ++g2)
             {
-                nntile_hip_sdpa_bwd_grid_args a;
-                std::memset(&a, 0, sizeof(a));
                 const auto &q0 = Q.get_tile({0, 0, g2, g3, g4});
-                a.q_seq = Q.shape[1];
-                a.k_seq = K.shape[1];
-                a.q_tile = Q.basetile_shape[1];
-                a.k_tile = K.basetile_shape[1];
-                a.head = Q.shape[0];
-                a.batch = q0.shape[2] * q0.shape[3] * q0.shape[4];
-                a.n_batch = a.batch;
-                a.kv_group = 1;
-                a.mask_mode = mask_mode;
-                a.n_q_tiles = static_cast<std::int32_t>(n_q);
-                a.n_kv_tiles = static_cast<std::int32_t>(n_kv);
-                a.causal_offset = causal_offset;
-                for(Index t = 0; t < n_kv; ++t)
-                {
-                    a.K[t] = K.get_tile({0, t, g2, g3, g4}).get_ptr();
-                    a.V[t] = V.get_tile({0, t, g2, g3, g4}).get_ptr();
-                    a.dK[t] = dK.get_tile({0, t, g2, g3, g4}).get_ptr();
-                    a.dV[t] = dV.get_tile({0, t, g2, g3, g4}).get_ptr();
-                    dK.get_tile({0, t, g2, g3, g4}).mark_written();
-                    dV.get_tile({0, t, g2, g3, g4}).mark_written();
-                }
-                for(Index t = 0; t < n_q; ++t)
-                {
-                    a.Q[t] = Q.get_tile({0, t, g2, g3, g4}).get_ptr();
-                    a.A[t] = A.get_tile({0, t, g2, g3, g4}).get_ptr();
-                    a.dA[t] = dA.get_tile({0, t, g2, g3, g4}).get_ptr();
-                    a.dQ[t] = dQ.get_tile({0, t, g2, g3, g4}).get_ptr();
-                    a.lse[t] = static_cast<const float *>(
-                            logsumexp.get_tile({t, g2, g3, g4}).get_ptr());
-                    dQ.get_tile({0, t, g2, g3, g4}).mark_written();
-                }
-                a.workspace = workspace.get_ptr();
-                a.workspace_bytes = ws_bytes;
-                starpu::count_direct_launch();
-                const int rc = BwdGridCall<T>::run(starpu::get_local_stream(), &a);
-                if(rc != NNTILE_HIP_OK)
-                {
-                    throw std::runtime_error("Error in flash_sdpa_bwd_hip grid launch (code "
-                            + std::to_string(rc) + ")");
-                }
-                ++calls;
+                slabs.push_back({g2, g3, g4, q0.shape[2] * q0.shape[3] * q0.shape[4]});
             }
         }
+    }
+    const std::size_t per_call = static_cast<std::size_t>(
+            NNTILE_HIP_SDPA_BWD_MAX_TILES / std::max(n_q, n_kv));
+    // One workspace for all calls: they run in order on one stream, and each
+    // call writes what it reads there.
+    const std::size_t ws_bytes = sizeof(float) * per_call * static_cast<std::size_t>(Q.shape[1]
+            * Q.basetile_shape[2] * Q.basetile_shape[3] * Q.basetile_shape[4]);
+    starpu::VariableHandle workspace(ws_bytes);
+    Index calls = 0;
+    for(std::size_t first = 0; first < slabs.size();)
+    {
+        std::size_t count = 1;
+        while(first + count < slabs.size() && count < per_call
+                && slabs[first + count].batch == slabs[first].batch)
+        {
+            ++count;
+        }
+        nntile_hip_sdpa_bwd_grid_args a;
+        std::memset(&a, 0, sizeof(a));
+        a.q_seq = Q.shape[1];
+        a.k_seq = K.shape[1];
+        a.q_tile = Q.basetile_shape[1];
+        a.k_tile = K.basetile_shape[1];
+        a.head = Q.shape[0];
+        a.batch = slabs[first].batch;
+        a.n_batch = a.batch;
+        a.kv_group = 1;
+        a.mask_mode = mask_mode;
+        a.n_q_tiles = static_cast<std::int32_t>(n_q);
+        a.n_kv_tiles = static_cast<std::int32_t>(n_kv);
+        a.n_slabs = static_cast<std::int32_t>(count);
+        a.causal_offset = causal_offset;
+        for(std::size_t s = 0; s < count; ++s)
+        {
+            const Index g2 = slabs[first + s].g2, g3 = slabs[first + s].g3,
+                  g4 = slabs[first + s].g4;
+            for(Index t = 0; t < n_kv; ++t)
+            {
+                a.K[s * n_kv + t] = K.get_tile({0, t, g2, g3, g4}).get_ptr();
+                a.V[s * n_kv + t] = V.get_tile({0, t, g2, g3, g4}).get_ptr();
+                a.dK[s * n_kv + t] = dK.get_tile({0, t, g2, g3, g4}).get_ptr();
+                a.dV[s * n_kv + t] = dV.get_tile({0, t, g2, g3, g4}).get_ptr();
+                dK.get_tile({0, t, g2, g3, g4}).mark_written();
+                dV.get_tile({0, t, g2, g3, g4}).mark_written();
+            }
+            for(Index t = 0; t < n_q; ++t)
+            {
+                a.Q[s * n_q + t] = Q.get_tile({0, t, g2, g3, g4}).get_ptr();
+                a.A[s * n_q + t] = A.get_tile({0, t, g2, g3, g4}).get_ptr();
+                a.dA[s * n_q + t] = dA.get_tile({0, t, g2, g3, g4}).get_ptr();
+                a.dQ[s * n_q + t] = dQ.get_tile({0, t, g2, g3, g4}).get_ptr();
+                a.lse[s * n_q + t] = static_cast<const float *>(
+                        logsumexp.get_tile({t, g2, g3, g4}).get_ptr());
+                dQ.get_tile({0, t, g2, g3, g4}).mark_written();
+            }
+        }
+        a.workspace = workspace.get_ptr();
+        a.workspace_bytes = ws_bytes;
+        starpu::count_direct_launch();
+        const int rc = BwdGridCall<T>::run(starpu::get_local_stream(), &a);
+        if(rc != NNTILE_HIP_OK)
+        {
+            throw std::runtime_error("Error in flash_sdpa_bwd_hip grid launch (code "
+                    + std::to_string(rc) + ")");
+        }
+        ++calls;
+        first += count;
     }
     workspace.unregister_submit();
     return calls;

@@ -27,6 +27,8 @@ def test_struct_layouts_match_header():
     assert ctypes.sizeof(h.TileArgs) == 6 * 8 + 8 + 3 * 8 + 6 * 8
     assert ctypes.sizeof(h.GridArgs) == 8 * 8 + 16 + 8 + 3 * 8 + 5 * 64 * 8
     assert h.GridArgs.n_slabs.offset == 8 * 8 + 16 and h.GridArgs.q_pos0.offset == 8 * 8 + 24
+    assert ctypes.sizeof(h.BwdGridArgs) == 8 * 8 + 16 + 8 + 3 * 8 + 9 * 32 * 8 + 16
+    assert h.BwdGridArgs.n_slabs.offset == 8 * 8 + 16 and h.BwdGridArgs.q_pos0.offset == 8 * 8 + 24
     assert ctypes.sizeof(h.FlashClArgs) == 32
     assert ctypes.sizeof(h.VariableInterface) == 40
 

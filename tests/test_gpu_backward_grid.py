@@ -198,3 +198,61 @@ def test_refusals():
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     assert hip_sdpa.lib().nntile_hip_sdpa_bwd_grid_bf16(None, ctypes.byref(a)) == hip_sdpa.EINVAL
     assert hip_sdpa.lib().nntile_hip_sdpa_bwd_grid_workspace_bytes(ctypes.byref(a)) == 4 * 128 * batch
+
+
+@pytest.mark.parametrize("dtype,head", [("bf16", 64), ("bf16", 128), ("fp16", 32)])
+@pytest.mark.parametrize("mode", ["causal", "none"])
+@pytest.mark.parametrize("n_slabs,shape", [
+    (4, (256, 256, 256, 256, 3, 1, 1)),     # one tile an axis, slabs along the batch
+    (3, (384, 640, 128, 256, 1, 2, 2)),     # sequence tiles as well, grouped queries
+    (2, (300, 520, 128, 384, 2, 1, 1)),     # ragged last tiles
+    (8, (200, 200, 200, 200, 1, 1, 1)),     # one entry per slab
+])
+def test_slabs_in_one_call(dtype, head, mode, n_slabs, shape):
+    """Several slabs of the batch grid in one call (n_slabs) give, bit for
+    bit, what one call per slab gives; the workspace grows with the slabs."""
+    q_seq, k_seq, q_tile, k_tile, n_batch, group, n_kv = shape
+    print("case bwd slabs", dtype, head, mode, n_slabs, shape, flush=True)
+    offset = max(k_seq - q_seq, 0)
+    mm = hip_sdpa.MASK_CAUSAL if mode == "causal" else hip_sdpa.MASK_NONE
+    ins_all = [[] for _ in range(6)]        # K, Q, V, A, dA, lse
+    acc_all, acc_one = [[] for _ in range(3)], [[] for _ in range(3)]
+    for s in range(n_slabs):
+        (Q, K, V, G), _, init = _case(400 + 3 * s, n_batch, group, n_kv, q_seq, k_seq, head, dtype)
+        # any A and lse of the right shape do: both ways read the same ones
+        A, _ = _rounded(0.5 * synth.randn(900 + s, 0, Q.numel()).reshape(Q.shape), dtype)
+        lse = torch.from_numpy(np.log(np.arange(1, q_seq + 1, dtype=np.float32)
+                                      )[None].repeat(Q.shape[0], 0).copy())
+        tiles = [_split(t.cuda(), step) for t, step in
+                 ((K, k_tile), (Q, q_tile), (V, k_tile), (A, q_tile), (G, q_tile), (lse, q_tile))]
+        one = [_split(x[0].clone().cuda(), step)
+               for x, step in zip(init, (k_tile, q_tile, k_tile))]
+        hip_sdpa.sdpa_bwd_grid(*tiles, *one, q_seq, k_seq, q_tile, k_tile, mm, n_batch=n_batch,
+                               kv_group=group, causal_offset=offset)
+        for dst, src in zip(ins_all, tiles):
+            dst += src
+        for dst, src in zip(acc_one, one):
+            dst += src
+        for dst, x, step in zip(acc_all, init, (k_tile, q_tile, k_tile)):
+            dst += _split(x[0].clone().cuda(), step)
+    batch = n_batch * group * n_kv
+    a = hip_sdpa.plan_bwd_grid(*ins_all, *acc_all, q_seq, k_seq, q_tile, k_tile, mm,
+                               n_batch=n_batch, kv_group=group, causal_offset=offset,
+                               n_slabs=n_slabs, workspace=torch.empty(1, dtype=torch.uint8,
+                                                                      device="cuda"))
+    assert (hip_sdpa.lib().nntile_hip_sdpa_bwd_grid_workspace_bytes(ctypes.byref(a._args))
+            == 4 * n_slabs * q_seq * batch)
+    hip_sdpa.sdpa_bwd_grid(*ins_all, *acc_all, q_seq, k_seq, q_tile, k_tile, mm, n_batch=n_batch,
+                           kv_group=group, causal_offset=offset, n_slabs=n_slabs)
+    torch.cuda.synchronize()
+    for got, want, name in zip(acc_all, acc_one, ("dK", "dQ", "dV")):
+        for t, (x, y) in enumerate(zip(got, want)):
+            assert torch.equal(_bits(x), _bits(y)), (name, t)
+    # a workspace sized for one slab is refused
+    with pytest.raises(hip_sdpa.SdpaError) as e:
+        hip_sdpa.sdpa_bwd_grid(*ins_all, *acc_all, q_seq, k_seq, q_tile, k_tile, mm,
+                               n_batch=n_batch, kv_group=group, causal_offset=offset,
+                               n_slabs=n_slabs,
+                               workspace=torch.empty(4 * q_seq * batch, dtype=torch.uint8,
+                                                     device="cuda"))
+    assert e.value.code == hip_sdpa.EWORKSPACE
