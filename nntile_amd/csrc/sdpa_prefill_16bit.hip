@@ -642,6 +642,9 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     PF_STAMP(1);
+#ifdef NNTILE_PF_TRACE
+    const unsigned long long pf_cycles0 = clock64();
+#endif
     PF_NOTE(5, ((unsigned long long)__builtin_amdgcn_s_getreg(63508) << 32)
             | (unsigned)__builtin_amdgcn_s_getreg(63492));
     PF_NOTE(6, ((unsigned long long)(unsigned)n_steps << 32) | (unsigned)(b * 1024 + qblk));
@@ -1258,6 +1261,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     }
     NNTILE_PHASE_DUMP()
     PF_STAMP(3);
+    PF_NOTE(7, clock64() - pf_cycles0);     // shader-clock cycles between stamps 1 and 3
 
     // ---- epilogue: normalise, merge into the running (lse, A) ----------------
     const float l_tot = sum_across_halves(l_run);
