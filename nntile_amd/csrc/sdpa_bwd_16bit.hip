@@ -41,6 +41,9 @@ namespace nntile_hip
 #ifndef NNTILE_BWD_PIPE
 #define NNTILE_BWD_PIPE 1
 #endif
+#ifndef NNTILE_BWD_PIPE_DQ
+#define NNTILE_BWD_PIPE_DQ 1        // the same in the dQ workgroups
+#endif
 #ifndef NNTILE_BWD_AHEAD
 #define NNTILE_BWD_AHEAD 2          // LDS operands are read this many MFMAs early
 #endif
@@ -572,93 +575,264 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
         // exists and the last key the workgroup's first query sees)
         const bool bounds = keys_here < kBwdStep
             || (MODE == NNTILE_HIP_MASK_CAUSAL && kg0 + kBwdStep - 1 > rel + q_row0);
-#pragma unroll
-        for(int mb = 0; mb < 2; ++mb)
+        if constexpr(EXPLICIT || NNTILE_BWD_PIPE_DQ == 0)
         {
-            f32x16 sv, dpv;
-#pragma unroll
-            for(int r = 0; r < 16; ++r)
+    #pragma unroll
+            for(int mb = 0; mb < 2; ++mb)
             {
-                sv[r] = 0.0f;
-                dpv[r] = 0.0f;
-            }
-#pragma unroll
-            for(int ks = 0; ks < KSTEPS; ++ks)
-            {
-                const vec8 ka = *reinterpret_cast<const vec8 *>(Ks + row_raddr[ks] + mb * 32 * RB);
-                const vec8 va = *reinterpret_cast<const vec8 *>(Vs + row_raddr[ks] + mb * 32 * RB);
-                sv = T::mfma(ka, qf[ks], sv);
-                dpv = T::mfma(va, gf[ks], dpv);
-#pragma unroll
-                for(int j = 0; j < LOADS_PER_WAVE; ++j)
+                f32x16 sv, dpv;
+    #pragma unroll
+                for(int r = 0; r < 16; ++r)
                 {
-                    if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
+                    sv[r] = 0.0f;
+                    dpv[r] = 0.0f;
+                }
+    #pragma unroll
+                for(int ks = 0; ks < KSTEPS; ++ks)
+                {
+                    const vec8 ka = *reinterpret_cast<const vec8 *>(Ks + row_raddr[ks] + mb * 32 * RB);
+                    const vec8 va = *reinterpret_cast<const vec8 *>(Vs + row_raddr[ks] + mb * 32 * RB);
+                    sv = T::mfma(ka, qf[ks], sv);
+                    dpv = T::mfma(va, gf[ks], dpv);
+    #pragma unroll
+                    for(int j = 0; j < LOADS_PER_WAVE; ++j)
                     {
-                        fetch_piece(at_f, BUF ? lds_k0 : lds_k1, BUF ? lds_v0 : lds_v1, j);
+                        if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
+                        {
+                            fetch_piece(at_f, BUF ? lds_k0 : lds_k1, BUF ? lds_v0 : lds_v1, j);
+                        }
+                    }
+                }
+                // Keys past the end and keys the causal mask hides: their scores
+                // become -inf in a pass of their own, which only the steps at the
+                // end of the keys and on the diagonal run (a wave-common branch).
+                if(bounds)
+                {
+    #pragma unroll
+                    for(int r = 0; r < 16; ++r)
+                    {
+                        const int key = mb * 32 + tile_row(r, half);
+                        sv[r] = key <= lim ? sv[r] : neg_inf();
+                    }
+                }
+                float dsv[16];
+    #pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    float e = fmaf(sv[r], c, -lse2);        // -inf: hidden, or a row that saw nothing
+                    bool visible = true;
+                    if(use_mask)
+                    {
+                        // wave-common address of the step's first key in the
+                        // workgroup's first row + the lane's 32-bit offset;
+                        // keys past the end read the last key, and are hidden
+                        const uint32_t key_off = (uint32_t)(mb * 32 + tile_row(r, 0)) * MASK_ES;
+                        const char *mp = mask_step + min(mask_off + key_off, mask_off_last);
+                        if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                        {
+                            const float add = T::to_float(*reinterpret_cast<const uint16_t *>(mp));
+                            visible = visible && (add != neg_inf());
+                            e = fmaf(add, kLog2e, e);
+                        }
+                        else
+                        {
+                            const uint8_t shown = *reinterpret_cast<const uint8_t *>(mp);
+                            visible = visible && (shown != 0);
+                        }
+                    }
+                    const float pr = use_mask ? (visible ? fast_exp2(e) : 0.0f) : fast_exp2(e);
+                    dsv[r] = pr * (dpv[r] - d_row);
+                }
+                uint32_t ds_pk[8];
+    #pragma unroll
+                for(int k = 0; k < 8; ++k)
+                {
+                    ds_pk[k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
+                }
+                // ---- dQ^T += K^T dS^T: the block's two sub-steps of 16 keys ------------------
+    #pragma unroll
+                for(int tt = 0; tt < 2; ++tt)
+                {
+                    const int t = 2 * mb + tt;
+                    const u32x4 braw = {ds_pk[4 * tt], ds_pk[4 * tt + 1], ds_pk[4 * tt + 2],
+                        ds_pk[4 * tt + 3]};
+                    const vec8 bop = __builtin_bit_cast(vec8, braw);
+    #pragma unroll
+                    for(int db = 0; db < DBLOCKS; ++db)
+                    {
+                        const u32x2 lo = bwd_lds_read_tr16(Ks + tr_raddr[0][db] + (16 * t) * RB);
+                        const u32x2 hi = bwd_lds_read_tr16(Ks + tr_raddr[1][db] + (16 * t) * RB);
+                        const u32x4 araw = {lo[0], lo[1], hi[0], hi[1]};
+                        acc[db] = T::mfma(__builtin_bit_cast(vec8, araw), bop, acc[db]);
                     }
                 }
             }
+        }
+        else
+        {
+            // The step's two 32-key blocks in three phases each - A: the two
+            // score products, B: dS on the vector ALU, C: dQ^T += K^T dS^T -
+            // issued as A0 | A1 with B0 | C0 with B1 | C1 (see the dK / dV body).
+            f32x16 sv[2], dpv[2];
+            uint32_t ds_pk[2][8];
+            constexpr int A_MFMAS = 2 * KSTEPS, C_MFMAS = 2 * DBLOCKS;
+            constexpr int AHEAD = NNTILE_BWD_AHEAD;
+            auto a_init = [&](int mb) __attribute__((always_inline))
+            {
+    #pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    sv[mb][r] = 0.0f;
+                    dpv[mb][r] = 0.0f;
+                }
+            };
+            auto a_read = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
+            {
+                if(i >= A_MFMAS)
+                {
+                    return;
+                }
+                ring[i % (AHEAD + 1)] = *reinterpret_cast<const vec8 *>(((i & 1) ? Vs : Ks)
+                        + row_raddr[i / 2] + mb * 32 * RB);
+            };
+            auto a_mfma = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
+            {
+                const int ks = i / 2;
+                if(i & 1)
+                {
+                    dpv[mb] = T::mfma(ring[i % (AHEAD + 1)], gf[ks], dpv[mb]);
+    #pragma unroll
+                    for(int j = 0; j < LOADS_PER_WAVE; ++j)
+                    {
+                        if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
+                        {
+                            fetch_piece(at_f, BUF ? lds_k0 : lds_k1, BUF ? lds_v0 : lds_v1, j);
+                        }
+                    }
+                }
+                else
+                {
+                    sv[mb] = T::mfma(ring[i % (AHEAD + 1)], qf[ks], sv[mb]);
+                }
+            };
             // Keys past the end and keys the causal mask hides: their scores
             // become -inf in a pass of their own, which only the steps at the
             // end of the keys and on the diagonal run (a wave-common branch).
-            if(bounds)
+            auto hide = [&](int mb) __attribute__((always_inline))
             {
-#pragma unroll
-                for(int r = 0; r < 16; ++r)
+                if(bounds)
                 {
-                    const int key = mb * 32 + tile_row(r, half);
-                    sv[r] = key <= lim ? sv[r] : neg_inf();
-                }
-            }
-            float dsv[16];
-#pragma unroll
-            for(int r = 0; r < 16; ++r)
-            {
-                float e = fmaf(sv[r], c, -lse2);        // -inf: hidden, or a row that saw nothing
-                bool visible = true;
-                if(use_mask)
-                {
-                    // wave-common address of the step's first key in the
-                    // workgroup's first row + the lane's 32-bit offset;
-                    // keys past the end read the last key, and are hidden
-                    const uint32_t key_off = (uint32_t)(mb * 32 + tile_row(r, 0)) * MASK_ES;
-                    const char *mp = mask_step + min(mask_off + key_off, mask_off_last);
-                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+    #pragma unroll
+                    for(int r = 0; r < 16; ++r)
                     {
-                        const float add = T::to_float(*reinterpret_cast<const uint16_t *>(mp));
-                        visible = visible && (add != neg_inf());
-                        e = fmaf(add, kLog2e, e);
-                    }
-                    else
-                    {
-                        const uint8_t shown = *reinterpret_cast<const uint8_t *>(mp);
-                        visible = visible && (shown != 0);
+                        const int key = mb * 32 + tile_row(r, half);
+                        sv[mb][r] = key <= lim ? sv[mb][r] : neg_inf();
                     }
                 }
-                const float pr = use_mask ? (visible ? fast_exp2(e) : 0.0f) : fast_exp2(e);
-                dsv[r] = pr * (dpv[r] - d_row);
-            }
-            uint32_t ds_pk[8];
-#pragma unroll
-            for(int k = 0; k < 8; ++k)
+            };
+            float ds_even = 0.0f;
+            auto b_item = [&](int mb, int r) __attribute__((always_inline))
             {
-                ds_pk[k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
-            }
-            // ---- dQ^T += K^T dS^T: the block's two sub-steps of 16 keys ------------------
-#pragma unroll
-            for(int tt = 0; tt < 2; ++tt)
-            {
-                const int t = 2 * mb + tt;
-                const u32x4 braw = {ds_pk[4 * tt], ds_pk[4 * tt + 1], ds_pk[4 * tt + 2],
-                    ds_pk[4 * tt + 3]};
-                const vec8 bop = __builtin_bit_cast(vec8, braw);
-#pragma unroll
-                for(int db = 0; db < DBLOCKS; ++db)
+                const float e = fmaf(sv[mb][r], c, -lse2);        // -inf: hidden, or a row that saw nothing
+                const float pr = fast_exp2(e);
+                const float dsr = pr * (dpv[mb][r] - d_row);
+                if(r % 2 == 0)
                 {
-                    const u32x2 lo = bwd_lds_read_tr16(Ks + tr_raddr[0][db] + (16 * t) * RB);
-                    const u32x2 hi = bwd_lds_read_tr16(Ks + tr_raddr[1][db] + (16 * t) * RB);
-                    const u32x4 araw = {lo[0], lo[1], hi[0], hi[1]};
-                    acc[db] = T::mfma(__builtin_bit_cast(vec8, araw), bop, acc[db]);
+                    ds_even = dsr;
+                }
+                else
+                {
+                    ds_pk[mb][r / 2] = T::pack2(ds_even, dsr);
+                    asm volatile("" : "+v"(ds_pk[mb][r / 2]));
+                }
+            };
+            // the block's two sub-steps of 16 keys
+            auto c_read = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
+            {
+                if(i >= C_MFMAS)
+                {
+                    return;
+                }
+                const int t = 2 * mb + i / DBLOCKS, db = i % DBLOCKS;
+                const u32x2 lo = bwd_lds_read_tr16(Ks + tr_raddr[0][db] + (16 * t) * RB);
+                const u32x2 hi = bwd_lds_read_tr16(Ks + tr_raddr[1][db] + (16 * t) * RB);
+                const u32x4 araw = {lo[0], lo[1], hi[0], hi[1]};
+                ring[i % (AHEAD + 1)] = __builtin_bit_cast(vec8, araw);
+            };
+            auto c_mfma = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
+            {
+                const int tt = i / DBLOCKS, db = i % DBLOCKS;
+                const u32x4 braw = {ds_pk[mb][4 * tt], ds_pk[mb][4 * tt + 1], ds_pk[mb][4 * tt + 2],
+                    ds_pk[mb][4 * tt + 3]};
+                acc[db] = T::mfma(ring[i % (AHEAD + 1)], __builtin_bit_cast(vec8, braw), acc[db]);
+            };
+            {
+                vec8 ring[AHEAD + 1];
+                a_init(0);
+    #pragma unroll
+                for(int i = 0; i < AHEAD; ++i)
+                {
+                    a_read(0, i, ring);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+                for(int i = 0; i < A_MFMAS; ++i)
+                {
+                    a_read(0, i + AHEAD, ring);
+                    a_mfma(0, i, ring);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                hide(0);
+                a_init(1);
+    #pragma unroll
+                for(int i = 0; i < AHEAD; ++i)
+                {
+                    a_read(1, i, ring);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+                for(int i = 0; i < A_MFMAS; ++i)
+                {
+                    a_read(1, i + AHEAD, ring);
+                    a_mfma(1, i, ring);
+    #pragma unroll
+                    for(int r = i * 16 / A_MFMAS; r < (i + 1) * 16 / A_MFMAS; ++r)
+                    {
+                        b_item(0, r);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                hide(1);
+    #pragma unroll
+                for(int i = 0; i < AHEAD; ++i)
+                {
+                    c_read(0, i, ring);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+                for(int i = 0; i < C_MFMAS; ++i)
+                {
+                    c_read(0, i + AHEAD, ring);
+                    c_mfma(0, i, ring);
+    #pragma unroll
+                    for(int r = i * 16 / C_MFMAS; r < (i + 1) * 16 / C_MFMAS; ++r)
+                    {
+                        b_item(1, r);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+    #pragma unroll
+                for(int i = 0; i < AHEAD; ++i)
+                {
+                    c_read(1, i, ring);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+                for(int i = 0; i < C_MFMAS; ++i)
+                {
+                    c_read(1, i + AHEAD, ring);
+                    c_mfma(1, i, ring);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
@@ -1070,386 +1244,397 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             + (int64_t)q0 * (int64_t)mask_row_bytes;
         const uint32_t mask_last_row = (uint32_t)(rows_here - 1) * mask_row_bytes;
 
-        // The step's two 32-query blocks in three phases each - A: S = Q K^T and
-        // dP = dA V^T (rows are queries, the lane's column its key), B: P and dS
-        // on the vector ALU, C: dV^T += dA^T P, dK^T += Q^T dS - issued as
-        // A0 | A1 with B0 | C0 with B1 | C1, so that the matrix unit works
-        // through a block's neighbours while the vector ALU turns its scores
-        // into probabilities.  P, dS: register r of block mb is query
-        // q0 + mb*32 + tile_row(r, half).
-        f32x16 sv[2], dpv[2];
-        uint32_t p_pk[2][8], ds_pk[2][8];
-        auto phase_a = [&](int mb) __attribute__((always_inline))
+        if constexpr(EXPLICIT || NNTILE_BWD_PIPE == 0)
         {
-#pragma unroll
-            for(int r = 0; r < 16; ++r)
+            // (one 32-query block at a time: half the accumulators live)
+            // ---- S = Q K^T, dP = dA V^T: rows are queries, the lane's column its key;
+            // P, dS: register r of block mb is query q0 + mb*32 + tile_row(r, half) --------------
+    #pragma unroll
+            for(int mb = 0; mb < 2; ++mb)
             {
-                sv[mb][r] = 0.0f;
-                dpv[mb][r] = 0.0f;
-            }
-            if(DO_DK)
-            {
-                // dP - D: the accumulator starts at -D of its row (four
-                // consecutive queries per LDS read), the products add dP
-#pragma unroll
+                uint32_t p_pk[8], ds_pk[8];
+                f32x16 sv, dpv;
+    #pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    sv[r] = 0.0f;
+                    dpv[r] = 0.0f;
+                }
+                if(DO_DK)
+                {
+                    // dP - D: the accumulator starts at -D of its row (four
+                    // consecutive queries per LDS read), the products add dP
+    #pragma unroll
+                    for(int rg = 0; rg < 4; ++rg)
+                    {
+                        const f32x4 nd4 = *reinterpret_cast<const f32x4 *>(
+                                &stat[1][mb * 32 + 8 * rg + 4 * half]);
+    #pragma unroll
+                        for(int e = 0; e < 4; ++e)
+                        {
+                            dpv[4 * rg + e] = nd4[e];
+                        }
+                    }
+                }
+    #pragma unroll
+                for(int ks = 0; ks < KSTEPS; ++ks)
+                {
+                    const vec8 qa = *reinterpret_cast<const vec8 *>(Qs + row_raddr[ks] + mb * 32 * RB);
+                    sv = T::mfma(qa, kf[ks], sv);
+                    if(DO_DK)
+                    {
+                        const vec8 ga = *reinterpret_cast<const vec8 *>(Gs + row_raddr[ks]
+                                + mb * 32 * RB);
+                        dpv = T::mfma(ga, vf[ks], dpv);
+                    }
+                    if(LOADERS == kDkvWaves || wave_u < LOADERS)
+                    {
+    #pragma unroll
+                        for(int j = 0; j < LPW; ++j)
+                        {
+                            if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
+                            {
+                                fetch_piece(at_f, at_end_f, BUF ? lds_q0 : lds_q1,
+                                        BUF ? lds_g0 : lds_g1, j);
+                            }
+                        }
+                    }
+                }
+                // Keys past the end and pairs the causal mask hides: their scores
+                // become -inf in a pass of their own, which only the workgroups at
+                // the end of the keys and the steps on the diagonal run (a
+                // wave-common branch).
+                if(bounds)
+                {
+    #pragma unroll
+                    for(int r = 0; r < 16; ++r)
+                    {
+                        const int qr = mb * 32 + tile_row(r, half);
+                        bool vis = k_ok;
+                        if(MODE == NNTILE_HIP_MASK_CAUSAL)
+                        {
+                            vis = vis && (my_k <= rel + q0 + qr);
+                        }
+                        sv[r] = vis ? sv[r] : neg_inf();
+                    }
+                }
+                float pv[16], dsv[16];
+    #pragma unroll
                 for(int rg = 0; rg < 4; ++rg)
                 {
-                    const f32x4 nd4 = *reinterpret_cast<const f32x4 *>(
-                            &stat[1][mb * 32 + 8 * rg + 4 * half]);
-#pragma unroll
+                    // four consecutive queries: their statistics in one LDS read each
+                    const int qr0 = mb * 32 + 8 * rg + 4 * half;
+                    const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(&stat[0][qr0]);
+    #pragma unroll
                     for(int e = 0; e < 4; ++e)
                     {
-                        dpv[mb][4 * rg + e] = nd4[e];
+                        const int r = 4 * rg + e;
+                        float ex = fmaf(sv[r], c, -lse4[e]);    // -inf: hidden, or a row past the end
+                        bool visible = true;
+                        if(use_mask)
+                        {
+                            // the row is the same for the lanes of one half: its
+                            // address is wave-common, the lane adds its key (and
+                            // four rows in the upper half, while those exist;
+                            // rows past the end read a row that exists and are
+                            // dropped by their logsumexp of +inf)
+                            const int rb = mb * 32 + 8 * rg + e;
+                            const char *mrow = mask_step
+                                + min((uint32_t)rb * mask_row_bytes, mask_last_row);
+                            const char *mp = mrow + (rb + 4 < rows_here ? mask_off_hi : mask_off_lo);
+                            if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                            {
+                                const float add = T::to_float(
+                                        *reinterpret_cast<const uint16_t *>(mp));
+                                visible = visible && (add != neg_inf());
+                                ex = fmaf(add, kLog2e, ex);
+                            }
+                            else
+                            {
+                                const uint8_t shown = *reinterpret_cast<const uint8_t *>(mp);
+                            visible = visible && (shown != 0);
+                            }
+                        }
+                        pv[r] = use_mask ? (visible ? fast_exp2(ex) : 0.0f) : fast_exp2(ex);
+                        dsv[r] = pv[r] * dpv[r];
+                    }
+                }
+    #pragma unroll
+                for(int k = 0; k < 8; ++k)
+                {
+                    p_pk[k] = T::pack2(pv[2 * k], pv[2 * k + 1]);
+                    ds_pk[k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
+                }
+                // ---- dV^T += dA^T P, dK^T += Q^T dS: the block's two sub-steps of 16 queries ----
+    #pragma unroll
+                for(int tt = 0; tt < 2; ++tt)
+                {
+                    const int t = 2 * mb + tt;
+                    const u32x4 praw = {p_pk[4 * tt], p_pk[4 * tt + 1], p_pk[4 * tt + 2],
+                        p_pk[4 * tt + 3]};
+                    const u32x4 sraw = {ds_pk[4 * tt], ds_pk[4 * tt + 1], ds_pk[4 * tt + 2],
+                        ds_pk[4 * tt + 3]};
+                    const vec8 pb = __builtin_bit_cast(vec8, praw);
+                    const vec8 sb = __builtin_bit_cast(vec8, sraw);
+    #pragma unroll
+                    for(int db = 0; db < DBLOCKS; ++db)
+                    {
+                        if(DO_DV)
+                        {
+                            const u32x2 glo = bwd_lds_read_tr16(Gs + tr_raddr[0][db] + (16 * t) * RB);
+                            const u32x2 ghi = bwd_lds_read_tr16(Gs + tr_raddr[1][db] + (16 * t) * RB);
+                            const u32x4 graw = {glo[0], glo[1], ghi[0], ghi[1]};
+                            dv[db] = T::mfma(__builtin_bit_cast(vec8, graw), pb, dv[db]);
+                        }
+                        if(DO_DK)
+                        {
+                            const u32x2 qlo = bwd_lds_read_tr16(Qs + tr_raddr[0][db] + (16 * t) * RB);
+                            const u32x2 qhi = bwd_lds_read_tr16(Qs + tr_raddr[1][db] + (16 * t) * RB);
+                            const u32x4 qraw = {qlo[0], qlo[1], qhi[0], qhi[1]};
+                            dk[db] = T::mfma(__builtin_bit_cast(vec8, qraw), sb, dk[db]);
+                        }
                     }
                 }
             }
-#pragma unroll
-            for(int ks = 0; ks < KSTEPS; ++ks)
+        }
+        else
+        {
+            // The step's two 32-query blocks in three phases each - A: S = Q K^T and
+            // dP = dA V^T (rows are queries, the lane's column its key), B: P and dS
+            // on the vector ALU, C: dV^T += dA^T P, dK^T += Q^T dS - issued as
+            // A0 | A1 with B0 | C0 with B1 | C1, so that the matrix unit works
+            // through a block's neighbours while the vector ALU turns its scores
+            // into probabilities.  P, dS: register r of block mb is query
+            // q0 + mb*32 + tile_row(r, half).
+            f32x16 sv[2], dpv[2];
+            uint32_t p_pk[2][8], ds_pk[2][8];
+            // Keys past the end and pairs the causal mask hides: their scores
+            // become -inf in a pass of their own, which only the workgroups at
+            // the end of the keys and the steps on the diagonal run (a
+            // wave-common branch).
+            auto hide = [&](int mb) __attribute__((always_inline))
             {
-                const vec8 qa = *reinterpret_cast<const vec8 *>(Qs + row_raddr[ks] + mb * 32 * RB);
-                sv[mb] = T::mfma(qa, kf[ks], sv[mb]);
-                if(DO_DK)
+                if(bounds)
                 {
-                    const vec8 ga = *reinterpret_cast<const vec8 *>(Gs + row_raddr[ks]
-                            + mb * 32 * RB);
-                    dpv[mb] = T::mfma(ga, vf[ks], dpv[mb]);
+    #pragma unroll
+                    for(int r = 0; r < 16; ++r)
+                    {
+                        const int qr = mb * 32 + tile_row(r, half);
+                        bool vis = k_ok;
+                        if(MODE == NNTILE_HIP_MASK_CAUSAL)
+                        {
+                            vis = vis && (my_k <= rel + q0 + qr);
+                        }
+                        sv[mb][r] = vis ? sv[mb][r] : neg_inf();
+                    }
                 }
-                if(LOADERS == kDkvWaves || wave_u < LOADERS)
+            };
+            // The overlapped order, written out slot by slot (one MFMA, the operand
+            // read of a later slot, a slice of the vector work) with a scheduling
+            // barrier after each, or the compiler regroups it into phases.
+            constexpr int A_MFMAS = (DO_DK ? 2 : 1) * KSTEPS, C_MFMAS = 2 * DBLOCKS;
+            constexpr int AHEAD = NNTILE_BWD_AHEAD;
+            auto a_read = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
+            {
+                if(i >= A_MFMAS)
                 {
-#pragma unroll
+                    return;
+                }
+                const int ks = DO_DK ? i / 2 : i;
+                const char *src = (DO_DK && (i & 1)) ? Gs : Qs;
+                ring[i % (AHEAD + 1)] = *reinterpret_cast<const vec8 *>(src + row_raddr[ks]
+                        + mb * 32 * RB);
+            };
+            auto a_mfma = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
+            {
+                const int ks = DO_DK ? i / 2 : i;
+                if(DO_DK && (i & 1))
+                {
+                    dpv[mb] = T::mfma(ring[i % (AHEAD + 1)], vf[ks], dpv[mb]);
+                }
+                else
+                {
+                    sv[mb] = T::mfma(ring[i % (AHEAD + 1)], kf[ks], sv[mb]);
+                }
+                // the tile loads of the next step, spread over the products
+                if((LOADERS == kDkvWaves || wave_u < LOADERS) && NNTILE_BWD_SPREAD != 0
+                        && (!DO_DK || (i & 1)))
+                {
+    #pragma unroll
                     for(int j = 0; j < LPW; ++j)
                     {
-                        if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
+                        if(mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
                         {
                             fetch_piece(at_f, at_end_f, BUF ? lds_q0 : lds_q1,
                                     BUF ? lds_g0 : lds_g1, j);
                         }
                     }
                 }
-            }
-        };
-        // Keys past the end and pairs the causal mask hides: their scores
-        // become -inf in a pass of their own, which only the workgroups at
-        // the end of the keys and the steps on the diagonal run (a
-        // wave-common branch).
-        auto hide = [&](int mb) __attribute__((always_inline))
-        {
-            if(bounds)
+            };
+            auto a_init = [&](int mb) __attribute__((always_inline))
             {
-#pragma unroll
+    #pragma unroll
                 for(int r = 0; r < 16; ++r)
                 {
-                    const int qr = mb * 32 + tile_row(r, half);
-                    bool vis = k_ok;
-                    if(MODE == NNTILE_HIP_MASK_CAUSAL)
-                    {
-                        vis = vis && (my_k <= rel + q0 + qr);
-                    }
-                    sv[mb][r] = vis ? sv[mb][r] : neg_inf();
+                    sv[mb][r] = 0.0f;
+                    dpv[mb][r] = 0.0f;
                 }
-            }
-        };
-        auto phase_b = [&](int mb) __attribute__((always_inline))
-        {
-            float pv[16], dsv[16];
-#pragma unroll
-            for(int rg = 0; rg < 4; ++rg)
-            {
-                // four consecutive queries: their statistics in one LDS read each
-                const int qr0 = mb * 32 + 8 * rg + 4 * half;
-                const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(&stat[0][qr0]);
-#pragma unroll
-                for(int e = 0; e < 4; ++e)
+                if(DO_DK)
                 {
-                    const int r = 4 * rg + e;
-                    float ex = fmaf(sv[mb][r], c, -lse4[e]);    // -inf: hidden, or a row past the end
-                    bool visible = true;
-                    if(use_mask)
+    #pragma unroll
+                    for(int rg = 0; rg < 4; ++rg)
                     {
-                        // the row is the same for the lanes of one half: its
-                        // address is wave-common, the lane adds its key (and
-                        // four rows in the upper half, while those exist;
-                        // rows past the end read a row that exists and are
-                        // dropped by their logsumexp of +inf)
-                        const int rb = mb * 32 + 8 * rg + e;
-                        const char *mrow = mask_step
-                            + min((uint32_t)rb * mask_row_bytes, mask_last_row);
-                        const char *mp = mrow + (rb + 4 < rows_here ? mask_off_hi : mask_off_lo);
-                        if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                        const f32x4 nd4 = *reinterpret_cast<const f32x4 *>(
+                                &stat[1][mb * 32 + 8 * rg + 4 * half]);
+    #pragma unroll
+                        for(int e = 0; e < 4; ++e)
                         {
-                            const float add = T::to_float(
-                                    *reinterpret_cast<const uint16_t *>(mp));
-                            visible = visible && (add != neg_inf());
-                            ex = fmaf(add, kLog2e, ex);
-                        }
-                        else
-                        {
-                            const uint8_t shown = *reinterpret_cast<const uint8_t *>(mp);
-                            visible = visible && (shown != 0);
+                            dpv[mb][4 * rg + e] = nd4[e];
                         }
                     }
-                    pv[r] = use_mask ? (visible ? fast_exp2(ex) : 0.0f) : fast_exp2(ex);
-                    dsv[r] = pv[r] * dpv[mb][r];
                 }
-            }
-#pragma unroll
-            for(int k = 0; k < 8; ++k)
+            };
+            auto c_read = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
             {
-                p_pk[mb][k] = T::pack2(pv[2 * k], pv[2 * k + 1]);
-                ds_pk[mb][k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
-            }
-        };
-        // the block's two sub-steps of 16 queries
-        auto phase_c = [&](int mb) __attribute__((always_inline))
-        {
-#pragma unroll
-            for(int tt = 0; tt < 2; ++tt)
-            {
-                const int t = 2 * mb + tt;
-                const u32x4 praw = {p_pk[mb][4 * tt], p_pk[mb][4 * tt + 1], p_pk[mb][4 * tt + 2],
-                    p_pk[mb][4 * tt + 3]};
-                const u32x4 sraw = {ds_pk[mb][4 * tt], ds_pk[mb][4 * tt + 1],
-                    ds_pk[mb][4 * tt + 2], ds_pk[mb][4 * tt + 3]};
-                const vec8 pb = __builtin_bit_cast(vec8, praw);
-                const vec8 sb = __builtin_bit_cast(vec8, sraw);
-#pragma unroll
-                for(int db = 0; db < DBLOCKS; ++db)
+                if(i >= C_MFMAS)
                 {
-                    if(DO_DV)
-                    {
-                        const u32x2 glo = bwd_lds_read_tr16(Gs + tr_raddr[0][db] + (16 * t) * RB);
-                        const u32x2 ghi = bwd_lds_read_tr16(Gs + tr_raddr[1][db] + (16 * t) * RB);
-                        const u32x4 graw = {glo[0], glo[1], ghi[0], ghi[1]};
-                        dv[db] = T::mfma(__builtin_bit_cast(vec8, graw), pb, dv[db]);
-                    }
-                    if(DO_DK)
-                    {
-                        const u32x2 qlo = bwd_lds_read_tr16(Qs + tr_raddr[0][db] + (16 * t) * RB);
-                        const u32x2 qhi = bwd_lds_read_tr16(Qs + tr_raddr[1][db] + (16 * t) * RB);
-                        const u32x4 qraw = {qlo[0], qlo[1], qhi[0], qhi[1]};
-                        dk[db] = T::mfma(__builtin_bit_cast(vec8, qraw), sb, dk[db]);
-                    }
+                    return;
                 }
-            }
-        };
-        // The overlapped order, written out slot by slot (one MFMA, the operand
-        // read of a later slot, a slice of the vector work) with a scheduling
-        // barrier after each, or the compiler regroups it into phases.
-        constexpr int A_MFMAS = (DO_DK ? 2 : 1) * KSTEPS, C_MFMAS = 2 * DBLOCKS;
-        constexpr int AHEAD = NNTILE_BWD_AHEAD;
-        auto a_read = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
-        {
-            if(i >= A_MFMAS)
+                const int t = 2 * mb + i / DBLOCKS, db = i % DBLOCKS;
+                const char *src = (DO_DV ? Gs : Qs) + (16 * t) * RB;
+                const u32x2 lo = bwd_lds_read_tr16(src + tr_raddr[0][db]);
+                const u32x2 hi = bwd_lds_read_tr16(src + tr_raddr[1][db]);
+                const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
+                ring[i % (AHEAD + 1)] = __builtin_bit_cast(vec8, raw);
+            };
+            auto c_mfma = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
             {
-                return;
-            }
-            const int ks = DO_DK ? i / 2 : i;
-            const char *src = (DO_DK && (i & 1)) ? Gs : Qs;
-            ring[i % (AHEAD + 1)] = *reinterpret_cast<const vec8 *>(src + row_raddr[ks]
-                    + mb * 32 * RB);
-        };
-        auto a_mfma = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
-        {
-            const int ks = DO_DK ? i / 2 : i;
-            if(DO_DK && (i & 1))
-            {
-                dpv[mb] = T::mfma(ring[i % (AHEAD + 1)], vf[ks], dpv[mb]);
-            }
-            else
-            {
-                sv[mb] = T::mfma(ring[i % (AHEAD + 1)], kf[ks], sv[mb]);
-            }
-            // the tile loads of the next step, spread over the products
-            if((LOADERS == kDkvWaves || wave_u < LOADERS) && NNTILE_BWD_SPREAD != 0
-                    && (!DO_DK || (i & 1)))
-            {
-#pragma unroll
-                for(int j = 0; j < LPW; ++j)
-                {
-                    if(mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
-                    {
-                        fetch_piece(at_f, at_end_f, BUF ? lds_q0 : lds_q1,
-                                BUF ? lds_g0 : lds_g1, j);
-                    }
-                }
-            }
-        };
-        auto a_init = [&](int mb) __attribute__((always_inline))
-        {
-#pragma unroll
-            for(int r = 0; r < 16; ++r)
-            {
-                sv[mb][r] = 0.0f;
-                dpv[mb][r] = 0.0f;
-            }
-            if(DO_DK)
-            {
-#pragma unroll
-                for(int rg = 0; rg < 4; ++rg)
-                {
-                    const f32x4 nd4 = *reinterpret_cast<const f32x4 *>(
-                            &stat[1][mb * 32 + 8 * rg + 4 * half]);
-#pragma unroll
-                    for(int e = 0; e < 4; ++e)
-                    {
-                        dpv[mb][4 * rg + e] = nd4[e];
-                    }
-                }
-            }
-        };
-        auto c_read = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
-        {
-            if(i >= C_MFMAS)
-            {
-                return;
-            }
-            const int t = 2 * mb + i / DBLOCKS, db = i % DBLOCKS;
-            const char *src = (DO_DV ? Gs : Qs) + (16 * t) * RB;
-            const u32x2 lo = bwd_lds_read_tr16(src + tr_raddr[0][db]);
-            const u32x2 hi = bwd_lds_read_tr16(src + tr_raddr[1][db]);
-            const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
-            ring[i % (AHEAD + 1)] = __builtin_bit_cast(vec8, raw);
-        };
-        auto c_mfma = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
-        {
-            const int tt = i / DBLOCKS, db = i % DBLOCKS;
-            const uint32_t (&pk)[8] = DO_DV ? p_pk[mb] : ds_pk[mb];
-            const u32x4 braw = {pk[4 * tt], pk[4 * tt + 1], pk[4 * tt + 2], pk[4 * tt + 3]};
-            if(DO_DV)
-            {
-                dv[db] = T::mfma(ring[i % (AHEAD + 1)], __builtin_bit_cast(vec8, braw), dv[db]);
-            }
-            else
-            {
-                dk[db] = T::mfma(ring[i % (AHEAD + 1)], __builtin_bit_cast(vec8, braw), dk[db]);
-            }
-        };
-        // vector work of query r of block mb (statistics of four queries per
-        // LDS read, read one group ahead)
-        f32x4 lse_cur = {0.0f, 0.0f, 0.0f, 0.0f}, lse_nxt = lse_cur;
-        float pv_even = 0.0f, ds_even = 0.0f;
-        auto b_begin = [&](int mb) __attribute__((always_inline))
-        {
-            lse_nxt = *reinterpret_cast<const f32x4 *>(&stat[0][mb * 32 + 4 * half]);
-        };
-        auto b_item = [&](int mb, int r) __attribute__((always_inline))
-        {
-            if(r % 4 == 0)
-            {
-                lse_cur = lse_nxt;
-                if(r + 4 < 16)
-                {
-                    lse_nxt = *reinterpret_cast<const f32x4 *>(
-                            &stat[0][mb * 32 + 8 * (r / 4 + 1) + 4 * half]);
-                }
-            }
-            const float pr = fast_exp2(fmaf(sv[mb][r], c, -lse_cur[r % 4]));
-            const float dsr = pr * dpv[mb][r];
-            if(r % 2 == 0)
-            {
-                pv_even = pr;
-                ds_even = dsr;
-            }
-            else
-            {
+                const int tt = i / DBLOCKS, db = i % DBLOCKS;
+                const uint32_t (&pk)[8] = DO_DV ? p_pk[mb] : ds_pk[mb];
+                const u32x4 braw = {pk[4 * tt], pk[4 * tt + 1], pk[4 * tt + 2], pk[4 * tt + 3]};
                 if(DO_DV)
                 {
-                    p_pk[mb][r / 2] = T::pack2(pv_even, pr);
-                    asm volatile("" : "+v"(p_pk[mb][r / 2]));
+                    dv[db] = T::mfma(ring[i % (AHEAD + 1)], __builtin_bit_cast(vec8, braw), dv[db]);
                 }
                 else
                 {
-                    ds_pk[mb][r / 2] = T::pack2(ds_even, dsr);
-                    asm volatile("" : "+v"(ds_pk[mb][r / 2]));
+                    dk[db] = T::mfma(ring[i % (AHEAD + 1)], __builtin_bit_cast(vec8, braw), dk[db]);
                 }
-            }
-        };
-        if(NNTILE_BWD_PIPE != 0 && !use_mask)
-        {
-            vec8 ring[AHEAD + 1];
-            // A0
-            a_init(0);
-#pragma unroll
-            for(int i = 0; i < AHEAD; ++i)
+            };
+            // vector work of query r of block mb (statistics of four queries per
+            // LDS read, read one group ahead)
+            f32x4 lse_cur = {0.0f, 0.0f, 0.0f, 0.0f}, lse_nxt = lse_cur;
+            float pv_even = 0.0f, ds_even = 0.0f;
+            auto b_begin = [&](int mb) __attribute__((always_inline))
             {
-                a_read(0, i, ring);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for(int i = 0; i < A_MFMAS; ++i)
+                lse_nxt = *reinterpret_cast<const f32x4 *>(&stat[0][mb * 32 + 4 * half]);
+            };
+            auto b_item = [&](int mb, int r) __attribute__((always_inline))
             {
-                a_read(0, i + AHEAD, ring);
-                a_mfma(0, i, ring);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            hide(0);
-            // A1 with B0
-            a_init(1);
-            b_begin(0);
-#pragma unroll
-            for(int i = 0; i < AHEAD; ++i)
-            {
-                a_read(1, i, ring);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for(int i = 0; i < A_MFMAS; ++i)
-            {
-                a_read(1, i + AHEAD, ring);
-                a_mfma(1, i, ring);
-#pragma unroll
-                for(int r = i * 16 / A_MFMAS; r < (i + 1) * 16 / A_MFMAS; ++r)
+                if(r % 4 == 0)
                 {
-                    b_item(0, r);
+                    lse_cur = lse_nxt;
+                    if(r + 4 < 16)
+                    {
+                        lse_nxt = *reinterpret_cast<const f32x4 *>(
+                                &stat[0][mb * 32 + 8 * (r / 4 + 1) + 4 * half]);
+                    }
                 }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            hide(1);
-            // C0 with B1
-            b_begin(1);
-#pragma unroll
-            for(int i = 0; i < AHEAD; ++i)
-            {
-                c_read(0, i, ring);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for(int i = 0; i < C_MFMAS; ++i)
-            {
-                c_read(0, i + AHEAD, ring);
-                c_mfma(0, i, ring);
-#pragma unroll
-                for(int r = i * 16 / C_MFMAS; r < (i + 1) * 16 / C_MFMAS; ++r)
+                const float pr = fast_exp2(fmaf(sv[mb][r], c, -lse_cur[r % 4]));
+                const float dsr = pr * dpv[mb][r];
+                if(r % 2 == 0)
                 {
-                    b_item(1, r);
+                    pv_even = pr;
+                    ds_even = dsr;
+                }
+                else
+                {
+                    if(DO_DV)
+                    {
+                        p_pk[mb][r / 2] = T::pack2(pv_even, pr);
+                        asm volatile("" : "+v"(p_pk[mb][r / 2]));
+                    }
+                    else
+                    {
+                        ds_pk[mb][r / 2] = T::pack2(ds_even, dsr);
+                        asm volatile("" : "+v"(ds_pk[mb][r / 2]));
+                    }
+                }
+            };
+            {
+                vec8 ring[AHEAD + 1];
+                // A0
+                a_init(0);
+    #pragma unroll
+                for(int i = 0; i < AHEAD; ++i)
+                {
+                    a_read(0, i, ring);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-            }
-            // C1
-#pragma unroll
-            for(int i = 0; i < AHEAD; ++i)
-            {
-                c_read(1, i, ring);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for(int i = 0; i < C_MFMAS; ++i)
-            {
-                c_read(1, i + AHEAD, ring);
-                c_mfma(1, i, ring);
+    #pragma unroll
+                for(int i = 0; i < A_MFMAS; ++i)
+                {
+                    a_read(0, i + AHEAD, ring);
+                    a_mfma(0, i, ring);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                hide(0);
+                // A1 with B0
+                a_init(1);
+                b_begin(0);
+    #pragma unroll
+                for(int i = 0; i < AHEAD; ++i)
+                {
+                    a_read(1, i, ring);
+                }
                 __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        else
-        {
-            // (one 32-query block at a time: fewer registers live)
-#pragma unroll
-            for(int mb = 0; mb < 2; ++mb)
-            {
-                phase_a(mb);
-                hide(mb);
-                phase_b(mb);
-                phase_c(mb);
+    #pragma unroll
+                for(int i = 0; i < A_MFMAS; ++i)
+                {
+                    a_read(1, i + AHEAD, ring);
+                    a_mfma(1, i, ring);
+    #pragma unroll
+                    for(int r = i * 16 / A_MFMAS; r < (i + 1) * 16 / A_MFMAS; ++r)
+                    {
+                        b_item(0, r);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                hide(1);
+                // C0 with B1
+                b_begin(1);
+    #pragma unroll
+                for(int i = 0; i < AHEAD; ++i)
+                {
+                    c_read(0, i, ring);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+                for(int i = 0; i < C_MFMAS; ++i)
+                {
+                    c_read(0, i + AHEAD, ring);
+                    c_mfma(0, i, ring);
+    #pragma unroll
+                    for(int r = i * 16 / C_MFMAS; r < (i + 1) * 16 / C_MFMAS; ++r)
+                    {
+                        b_item(1, r);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // C1
+    #pragma unroll
+                for(int i = 0; i < AHEAD; ++i)
+                {
+                    c_read(1, i, ring);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+                for(int i = 0; i < C_MFMAS; ++i)
+                {
+                    c_read(1, i + AHEAD, ring);
+                    c_mfma(1, i, ring);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
         // (the other buffer's readers passed this step's barrier; the next
