@@ -367,3 +367,31 @@ def test_tiles_of_128_rows_take_one_call_per_slab(oracle, dtype, kind, offset):
             assert np.array_equal(g, d), n
         if kind != "window":
             assert tile_tasks == 0
+
+
+@pytest.mark.gpu
+def test_slabs_of_unequal_size_share_calls_only_with_their_like(oracle):
+    """A batch grid whose last tiles are smaller: slabs of 4, 2, 2 and 1
+    entries.  Only neighbours of equal size share a call (4 | 2, 2 | 1), and
+    the gradients are those of the pair-by-pair submission and the checker."""
+    dtype, head, seq, tile, nb, grp, nkv = "bf16", 64, 256, 128, 3, 1, 3
+    batch = nb * grp * nkv
+    shape5, base5 = [head, seq, nb, grp, nkv], [head, tile, 2, 1, 2]
+    (Q, K, V), (qf, kf, vf) = H.make_qkv(91, batch, seq, seq, head, dtype)
+    _, gf = H.rounded(synth.randn(92, 0, batch * seq * head).reshape(batch, seq, head), dtype)
+    i = np.arange(seq)
+    mask = i[None, :] <= i[:, None]
+    add = np.where(mask, 0.0, -np.inf).astype(np.float32)
+    A64, lse64 = oracle.sdpa_bruteforce_f64(kf, qf, vf, add)
+    lse = lse64.astype(np.float32)
+    _, af = H.rounded(A64, dtype)
+    data = {"K": kf, "Q": qf, "V": vf, "A": af, "dA": gf}
+    got, calls, ntiles = _run(hm.OP_CLASSIFIED, dtype, data, lse, add, shape5, base5)
+    ref, all_pairs, _ = _run(hm.OP_PAIRS_BWD, dtype, data, lse, add, shape5, base5)
+    nt = seq // tile
+    assert ntiles // nt == 4 and all_pairs == 4 * nt * nt
+    assert calls == 3
+    want = oracle.sdpa_bwd_flash_f64(kf, qf, vf, af, gf, lse, add)
+    for g, r, w, n in zip(got, ref, want, ("dK", "dQ", "dV")):
+        assert H.rel_fro(g, w) < 1e-2, n
+        assert H.rel_fro(g, r) < 1e-2, n
