@@ -123,7 +123,9 @@ def _run(dtype, arrs, mask_bool, head, seq, nb, grp, nkv, tile, op, **kw):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])
 @pytest.mark.parametrize("head,seq,nb,grp,nkv,tile", [(32, 64, 2, 1, 2, 64), (128, 256, 2, 1, 2, 128),
-                                                     (32, 512, 4, 3, 4, 64), (64, 200, 2, 1, 2, 96)])
+                                                     (32, 512, 4, 3, 4, 64), (64, 200, 2, 1, 2, 96),
+                                                     # batch tiles of 2, 2 and 1 entries: slabs of unequal size
+                                                     (64, 256, 5, 1, 3, 128)])
 def test_tensor_level_tiles_match_oracle(oracle, dtype, head, seq, nb, grp, nkv, tile):
     arrs, (qf, kf, vf) = _case(dtype, head, seq, nb, grp, nkv)
     mask = synth.causal_mask(seq, seq)
