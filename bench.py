@@ -444,6 +444,45 @@ def bench_backward(cfg, steps, warmup):
                 "frac_of_peak": round(fl / (dev_t * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}}
 
 
+def bench_backward_slabs(cfg, steps, warmup):
+    """Backward over a tensor whose batch axes are tiled (cfg.calls slabs of
+    the batch grid, one sequence tile each): all slabs in one call (n_slabs of
+    nntile_hip_sdpa_bwd_grid_args) against one call per slab."""
+    import torch
+    from nntile_amd import hip_sdpa as h
+    dt = {"bf16": torch.bfloat16, "fp16": torch.float16}[cfg.dtype]
+    per = cfg.batch_flat // cfg.calls
+    seq = cfg.q_seq
+    mk = lambda i: [_randn((per, seq, cfg.head), dt, cfg.seed, 10 * s + i) for s in range(cfg.calls)]
+    Q, K, V, G = mk(0), mk(1), mk(2), mk(3)
+    A = [torch.zeros_like(q) for q in Q]
+    L = [torch.full((per, seq), float("-inf"), device="cuda") for _ in Q]
+    h.sdpa_fwd_grid(K, Q, L, V, A, seq, seq, seq, seq, h.MASK_CAUSAL, flags=h.OVERWRITE,
+                    n_slabs=cfg.calls)
+    dK, dQ, dV = ([torch.zeros_like(q) for q in Q] for _ in range(3))
+    ws = torch.empty(4 * cfg.calls * seq * per, dtype=torch.uint8, device="cuda")
+    one = h.plan_bwd_grid(K, Q, V, A, G, L, dK, dQ, dV, seq, seq, seq, seq, h.MASK_CAUSAL, ws,
+                          flags=h.OVERWRITE, n_slabs=cfg.calls)
+    each = [h.plan_bwd_grid([K[i]], [Q[i]], [V[i]], [A[i]], [G[i]], [L[i]], [dK[i]], [dQ[i]],
+                            [dV[i]], seq, seq, seq, seq, h.MASK_CAUSAL, ws, flags=h.OVERWRITE)
+            for i in range(cfg.calls)]
+
+    def per_slab():
+        for pl in each:
+            pl.launch()
+
+    _, dev1 = time_steps(one.launch, steps, warmup)
+    _, dev2 = time_steps(per_slab, steps, warmup)
+    fl = 2.5 * cfg.flops()
+    return {"what": "backward of %d slabs of %d heads x %d x %d (%s), causal, gradients written: one "
+                    "call for all slabs against one call per slab" % (cfg.calls, per, seq, cfg.head,
+                                                                       cfg.dtype),
+            "one_call": {"device_ms_per_step": round(dev1, 4),
+                         "tflops": round(fl / (dev1 * 1e-3) / 1e12, 1)},
+            "one_call_per_slab": {"device_ms_per_step": round(dev2, 4),
+                                  "tflops": round(fl / (dev2 * 1e-3) / 1e12, 1)}}
+
+
 def bench_rope(cfg, steps, warmup):
     """Rotary embedding of the Q tensor of the workload (the step before the
     attention kernel): sin, cos of shape [head/2, seq], src and dst
@@ -646,7 +685,7 @@ def main():
                          "(e.g. bf16,4096,64,8,causal)")
     ap.add_argument("--only", default=None,
                     help="run only this leg (for profiling): prefill | cfg5 | cfg2 | decode | decode_wide | "
-                         "reference_api | reference_grid | power_context | copy_context | backward | rope | transpose | accumulate | "
+                         "reference_api | reference_grid | power_context | copy_context | backward | backward_slabs | rope | transpose | accumulate | "
                          "kv_cache | copy")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -685,6 +724,10 @@ def main():
             "rope": lambda: bench_rope(cfg3, args.steps, args.warmup),
             "transpose": lambda: bench_transpose(cfg3, args.steps, args.warmup),
             "accumulate": lambda: bench_accumulate(cfg3, args.steps, args.warmup),
+            "backward_slabs": lambda: bench_backward_slabs(
+                __import__("dataclasses").replace(BY_NAME["cfg2_gpt2_small_fp32"],
+                                                  name="cfg2_shape_in_bf16", dtype="bf16"),
+                args.steps, args.warmup),
             "kv_cache": lambda: bench_kv_cache(cfg4, args.steps, args.warmup)}
     if only == "copy":
         # calibration leg for the HBM traffic counters: a plain device copy
@@ -726,6 +769,21 @@ def main():
                 "what": "the same with one launch per slab of the batch grid (%d launches)" % c.calls,
                 "ms_per_step": round(r1["ms_per_step"], 4), "tflops": round(r1["tflops"], 2),
                 "launches_per_step": r1["launches_per_step"]}
+    # cfg2's tiling on 16-bit tiles (the shape of the reference's GPT-2 flash
+    # path): the slabs of the batch grid in one launch and one by one
+    import dataclasses
+    gpt2_bf16 = dataclasses.replace(BY_NAME["cfg2_gpt2_small_fp32"], name="cfg2_shape_in_bf16",
+                                    dtype="bf16")
+    r, r1 = bench_prefill(gpt2_bf16, few, 3), bench_prefill(gpt2_bf16, few, 3, one_launch=False)
+    extras[gpt2_bf16.name] = {
+        "what": "for information: cfg2's shape and tiling on bf16 tiles",
+        "ms_per_step": round(r["ms_per_step"], 4), "tflops": round(r["tflops"], 2),
+        "launches_per_step": r["launches_per_step"],
+        "frac_of_peak": round(r["tflops"] / PEAK_BF16_TFLOPS, 4),
+        "one_launch_per_slab": {"ms_per_step": round(r1["ms_per_step"], 4),
+                                "tflops": round(r1["tflops"], 2),
+                                "launches_per_step": r1["launches_per_step"]},
+        "backward": bench_backward_slabs(gpt2_bf16, few, 3)}
     backward = bench_backward(cfg3, max(5, args.steps // 10), 3)
     rope = bench_rope(cfg3, few, 5)
     transpose = bench_transpose(cfg3, few, 5)
