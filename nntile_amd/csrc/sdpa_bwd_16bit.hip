@@ -908,6 +908,12 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
 // One set of workgroups per gradient (dK: S, dP, dK^T; dV: S, dV^T - the
 // scores are computed once more) fits two workgroups of 4 wavefronts on a CU.
 enum { BWD_PART_DK = 1, BWD_PART_DV = 2 };
+// Head sizes at which one workgroup holds both gradients of its keys.
+#ifndef NNTILE_BWD_FUSED_KEYS_HEAD
+#define NNTILE_BWD_FUSED_KEYS_HEAD 64
+#endif
+template<int HEAD> constexpr bool kBwdFusedKeys = HEAD <= NNTILE_BWD_FUSED_KEYS_HEAD;
+constexpr int kBwdCUs = 256;
 constexpr int kDkvWaves = 4;
 constexpr int kDkvThreads = kDkvWaves * 64;
 constexpr int kDkvRows = kDkvWaves * 32;        // keys per workgroup
@@ -918,7 +924,8 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
         char *lds_q0, char *lds_q1, char *lds_g0, char *lds_g1,
         float (*lds_stat)[2][kBwdStep])
 {
-    constexpr bool DO_DK = PART == BWD_PART_DK, DO_DV = PART == BWD_PART_DV;
+    constexpr bool DO_DK = (PART & BWD_PART_DK) != 0, DO_DV = (PART & BWD_PART_DV) != 0;
+    constexpr bool BOTH = DO_DK && DO_DV;
     typedef typename T::vec8 vec8;
     typedef BwdTile<HEAD> G;
     constexpr int KSTEPS = G::KSTEPS, DBLOCKS = G::DBLOCKS, RB = G::RB, CPR = G::CPR;
@@ -1432,7 +1439,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             // The overlapped order, written out slot by slot (one MFMA, the operand
             // read of a later slot, a slice of the vector work) with a scheduling
             // barrier after each, or the compiler regroups it into phases.
-            constexpr int A_MFMAS = (DO_DK ? 2 : 1) * KSTEPS, C_MFMAS = 2 * DBLOCKS;
+            constexpr int A_MFMAS = (DO_DK ? 2 : 1) * KSTEPS, C_MFMAS = (BOTH ? 2 : 1) * 2 * DBLOCKS;
             constexpr int AHEAD = NNTILE_BWD_AHEAD;
             auto a_read = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
             {
@@ -1500,8 +1507,11 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                 {
                     return;
                 }
-                const int t = 2 * mb + i / DBLOCKS, db = i % DBLOCKS;
-                const char *src = (DO_DV ? Gs : Qs) + (16 * t) * RB;
+                // (both gradients: dV and dK products alternate)
+                const int j = BOTH ? i / 2 : i;
+                const bool for_dv = BOTH ? (i & 1) == 0 : DO_DV;
+                const int t = 2 * mb + j / DBLOCKS, db = j % DBLOCKS;
+                const char *src = (for_dv ? Gs : Qs) + (16 * t) * RB;
                 const u32x2 lo = bwd_lds_read_tr16(src + tr_raddr[0][db]);
                 const u32x2 hi = bwd_lds_read_tr16(src + tr_raddr[1][db]);
                 const u32x4 raw = {lo[0], lo[1], hi[0], hi[1]};
@@ -1509,10 +1519,12 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             };
             auto c_mfma = [&](int mb, int i, vec8 (&ring)[AHEAD + 1]) __attribute__((always_inline))
             {
-                const int tt = i / DBLOCKS, db = i % DBLOCKS;
-                const uint32_t (&pk)[8] = DO_DV ? p_pk[mb] : ds_pk[mb];
+                const int j = BOTH ? i / 2 : i;
+                const bool for_dv = BOTH ? (i & 1) == 0 : DO_DV;
+                const int tt = j / DBLOCKS, db = j % DBLOCKS;
+                const uint32_t (&pk)[8] = for_dv ? p_pk[mb] : ds_pk[mb];
                 const u32x4 braw = {pk[4 * tt], pk[4 * tt + 1], pk[4 * tt + 2], pk[4 * tt + 3]};
-                if(DO_DV)
+                if(for_dv)
                 {
                     dv[db] = T::mfma(ring[i % (AHEAD + 1)], __builtin_bit_cast(vec8, braw), dv[db]);
                 }
@@ -1554,7 +1566,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                         p_pk[mb][r / 2] = T::pack2(pv_even, pr);
                         asm volatile("" : "+v"(p_pk[mb][r / 2]));
                     }
-                    else
+                    if(DO_DK)
                     {
                         ds_pk[mb][r / 2] = T::pack2(ds_even, dsr);
                         asm volatile("" : "+v"(ds_pk[mb][r / 2]));
@@ -1724,7 +1736,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
 // last n_dkv dV.  A tile-pair call has fewer workgroups per gradient than the
 // chip has places (two a CU); together they fill it, and a long call loses
 // the ends of two launches.
-template<typename T, int HEAD, int MODE, bool GRID>
+template<typename T, int HEAD, int MODE, bool GRID, bool FUSED_KEYS = false>
 __global__ __launch_bounds__(kDkvThreads, 2)
 void sdpa_bwd_kernel(const std::conditional_t<GRID, BwdGridParams, BwdParams> p, unsigned n_dkv,
         unsigned n_dq)
@@ -1738,7 +1750,22 @@ void sdpa_bwd_kernel(const std::conditional_t<GRID, BwdGridParams, BwdParams> p,
     // dK, dV parts, per query of a step: logsumexp in log2 units (+inf for a
     // row that saw nothing) and minus the row dot D; rows past the end hold +inf / 0
     __shared__ __attribute__((aligned(16))) float lds_stat[2][2][kBwdStep];
-    if(blockIdx.x < n_dkv)
+    if constexpr(FUSED_KEYS)
+    {
+        // (K and V fragments and both accumulators fit beside the rest: one
+        // set of key-owning workgroups computes dK and dV from one pass over
+        // the scores, seven products a call instead of eight)
+        if(blockIdx.x < n_dkv)
+        {
+            sdpa_bwd_dkv_body<T, HEAD, MODE, BWD_PART_DK | BWD_PART_DV, GRID>(p, blockIdx.x, lds_0,
+                    lds_1, lds_2, lds_3, lds_stat);
+        }
+        else
+        {
+            sdpa_bwd_dq_body<T, HEAD, MODE, GRID>(p, blockIdx.x - n_dkv, lds_0, lds_1, lds_2, lds_3);
+        }
+    }
+    else if(blockIdx.x < n_dkv)
     {
         sdpa_bwd_dkv_body<T, HEAD, MODE, BWD_PART_DK, GRID>(p, blockIdx.x, lds_0, lds_1, lds_2,
                 lds_3, lds_stat);
@@ -1786,6 +1813,20 @@ static int launch_bwd_mode(hipStream_t stream, const BwdParams &p)
     {
         return NNTILE_HIP_ELAUNCH;
     }
+    if constexpr(kBwdFusedKeys<HEAD>)
+    {
+        // One set of key-owning workgroups for both gradients (seven products
+        // instead of eight) once the three sets would not all be resident at
+        // the same time; below that the longest workgroup sets the time, and
+        // the separate sets have the shorter ones.
+        if(2 * n_dkv + n_dq > 2 * kBwdCUs)
+        {
+            hipLaunchKernelGGL((sdpa_bwd_kernel<T, HEAD, MODE, false, true>),
+                    dim3((unsigned)(n_dkv + n_dq)), dim3(kDkvThreads), 0, stream, p,
+                    (unsigned)n_dkv, (unsigned)n_dq);
+            return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
+        }
+    }
     hipLaunchKernelGGL((sdpa_bwd_kernel<T, HEAD, MODE, false>),
             dim3((unsigned)(2 * n_dkv + n_dq)), dim3(kDkvThreads), 0, stream, p,
             (unsigned)n_dkv, (unsigned)n_dq);
@@ -1822,6 +1863,20 @@ static int launch_bwd_grid_mode(hipStream_t stream, const BwdGridParams &p,
             {
                 return NNTILE_HIP_ELAUNCH;
             }
+        }
+    }
+    if constexpr(kBwdFusedKeys<HEAD>)
+    {
+        // One set of key-owning workgroups for both gradients (seven products
+        // instead of eight) once the three sets would not all be resident at
+        // the same time; below that the longest workgroup sets the time, and
+        // the separate sets have the shorter ones.
+        if(2 * n_dkv + n_dq > 2 * kBwdCUs)
+        {
+            hipLaunchKernelGGL((sdpa_bwd_kernel<T, HEAD, MODE, true, true>),
+                    dim3((unsigned)(n_dkv + n_dq)), dim3(kDkvThreads), 0, stream, p,
+                    (unsigned)n_dkv, (unsigned)n_dq);
+            return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
         }
     }
     hipLaunchKernelGGL((sdpa_bwd_kernel<T, HEAD, MODE, true>),

@@ -77,15 +77,24 @@ def test_reference_kernel_test_cases(oracle, dtype, mask_kind, strategy, seq, he
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("head", [32, 64])
+@pytest.mark.parametrize("mode", ["causal", "none", "additive"])
+def test_more_workgroups_than_places(oracle, dtype, head, mode):
+    """A batch large enough that the workgroups of the three gradients would
+    not all be resident at once: at these head sizes dK and dV then come from
+    one set of workgroups (masks given as values included)."""
+    test_modes_and_shapes(oracle, dtype, head, 300, 512, mode, batch=72)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
 @pytest.mark.parametrize("head", [32, 64, 128])
 @pytest.mark.parametrize("q_seq,k_seq", [(128, 128), (200, 333), (64, 520), (257, 100)])
 @pytest.mark.parametrize("mode", ["causal", "none", "additive", "bool"])
-def test_modes_and_shapes(oracle, dtype, head, q_seq, k_seq, mode):
+def test_modes_and_shapes(oracle, dtype, head, q_seq, k_seq, mode, batch=2):
     """Every mask mode on rectangular and ragged shapes, with A and lse from a
     forward pass of the same inputs, gradients accumulated onto non-zero
     tiles and, second, written in overwrite mode."""
-    print("case bwd", dtype, head, q_seq, k_seq, mode, flush=True)
-    batch = 2
+    print("case bwd", dtype, head, q_seq, k_seq, mode, batch, flush=True)
     offset = max(k_seq - q_seq, 0)
     (Q, K, V), (qf, kf, vf) = H.make_qkv(91, batch, q_seq, k_seq, head, dtype)
     G, gf = _rounded(synth.randn(92, 0, batch * q_seq * head).reshape(batch, q_seq, head), dtype)

@@ -207,6 +207,10 @@ def test_refusals():
     (3, (384, 640, 128, 256, 1, 2, 2)),     # sequence tiles as well, grouped queries
     (2, (300, 520, 128, 384, 2, 1, 1)),     # ragged last tiles
     (8, (200, 200, 200, 200, 1, 1, 1)),     # one entry per slab
+    # more workgroups than the chip holds at once: at head sizes up to 64 the
+    # call over all slabs takes the workgroups that compute dK and dV
+    # together, the calls per slab the separate ones
+    (4, (1024, 1024, 1024, 1024, 12, 1, 1)),
 ])
 def test_slabs_in_one_call(dtype, head, mode, n_slabs, shape):
     """Several slabs of the batch grid in one call (n_slabs) give, bit for
@@ -248,6 +252,22 @@ def test_slabs_in_one_call(dtype, head, mode, n_slabs, shape):
     for got, want, name in zip(acc_all, acc_one, ("dK", "dQ", "dV")):
         for t, (x, y) in enumerate(zip(got, want)):
             assert torch.equal(_bits(x), _bits(y)), (name, t)
+    if q_tile == q_seq and k_tile == k_seq and group == 1:
+        # one tile an axis: the slabs side by side in one allocation are a
+        # batch of n_slabs * batch entries for the one-allocation form
+        K1, Q1, V1, A1, G1, L1 = (torch.cat(t, dim=0) for t in ins_all)
+        init1 = [torch.cat(t, dim=0) for t in acc_one]      # (shapes only)
+        start = []
+        for s in range(n_slabs):
+            _, _, init = _case(400 + 3 * s, n_batch, group, n_kv, q_seq, k_seq, head, dtype)
+            start.append([x[0].clone().cuda() for x in init])
+        dK1, dQ1, dV1 = (torch.cat([st[i] for st in start], dim=0) for i in range(3))
+        assert dK1.shape == init1[0].shape
+        hip_sdpa.sdpa_bwd_tile(K1, Q1, V1, A1, G1, None, L1, dK1, dQ1, dV1, mm,
+                               causal_offset=offset)
+        torch.cuda.synchronize()
+        for got, one, name in zip(acc_all, (dK1, dQ1, dV1), ("dK", "dQ", "dV")):
+            assert torch.equal(_bits(torch.cat(got, dim=0)), _bits(one)), name
     # a workspace sized for one slab is refused
     with pytest.raises(hip_sdpa.SdpaError) as e:
         hip_sdpa.sdpa_bwd_grid(*ins_all, *acc_all, q_seq, k_seq, q_tile, k_tile, mm,
