@@ -1541,38 +1541,57 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             {
                 lse_nxt = *reinterpret_cast<const f32x4 *>(&stat[0][mb * 32 + 4 * half]);
             };
-            auto b_item = [&](int mb, int r) __attribute__((always_inline))
+            // (in three stages a tick apart - exponent, exponential, products and
+            // packing - so that a lone wavefront does not wait for its own
+            // results: tick t takes query t, t-1 and t-2 through one stage each)
+            float ex_stage[2] = {0.0f, 0.0f}, pr_stage[2] = {0.0f, 0.0f};
+            auto b_tick = [&](int mb, int t) __attribute__((always_inline))
             {
-                if(r % 4 == 0)
+                if(t - 2 >= 0 && t - 2 < 16)
                 {
-                    lse_cur = lse_nxt;
-                    if(r + 4 < 16)
+                    const int r = t - 2;
+                    const float pr = pr_stage[r % 2];
+                    const float dsr = pr * dpv[mb][r];
+                    if(r % 2 == 0)
                     {
-                        lse_nxt = *reinterpret_cast<const f32x4 *>(
-                                &stat[0][mb * 32 + 8 * (r / 4 + 1) + 4 * half]);
+                        pv_even = pr;
+                        ds_even = dsr;
+                    }
+                    else
+                    {
+                        if(DO_DV)
+                        {
+                            p_pk[mb][r / 2] = T::pack2(pv_even, pr);
+                            asm volatile("" : "+v"(p_pk[mb][r / 2]));
+                        }
+                        if(DO_DK)
+                        {
+                            ds_pk[mb][r / 2] = T::pack2(ds_even, dsr);
+                            asm volatile("" : "+v"(ds_pk[mb][r / 2]));
+                        }
                     }
                 }
-                const float pr = fast_exp2(fmaf(sv[mb][r], c, -lse_cur[r % 4]));
-                const float dsr = pr * dpv[mb][r];
-                if(r % 2 == 0)
+                if(t - 1 >= 0 && t - 1 < 16)
                 {
-                    pv_even = pr;
-                    ds_even = dsr;
+                    const int r = t - 1;
+                    pr_stage[r % 2] = fast_exp2(ex_stage[r % 2]);
                 }
-                else
+                if(t < 16)
                 {
-                    if(DO_DV)
+                    const int r = t;
+                    if(r % 4 == 0)
                     {
-                        p_pk[mb][r / 2] = T::pack2(pv_even, pr);
-                        asm volatile("" : "+v"(p_pk[mb][r / 2]));
+                        lse_cur = lse_nxt;
+                        if(r + 4 < 16)
+                        {
+                            lse_nxt = *reinterpret_cast<const f32x4 *>(
+                                    &stat[0][mb * 32 + 8 * (r / 4 + 1) + 4 * half]);
+                        }
                     }
-                    if(DO_DK)
-                    {
-                        ds_pk[mb][r / 2] = T::pack2(ds_even, dsr);
-                        asm volatile("" : "+v"(ds_pk[mb][r / 2]));
-                    }
+                    ex_stage[r % 2] = fmaf(sv[mb][r], c, -lse_cur[r % 4]);
                 }
             };
+            constexpr int B_TICKS = 18;
             {
                 vec8 ring[AHEAD + 1];
                 // A0
@@ -1606,9 +1625,9 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                     a_read(1, i + AHEAD, ring);
                     a_mfma(1, i, ring);
     #pragma unroll
-                    for(int r = i * 16 / A_MFMAS; r < (i + 1) * 16 / A_MFMAS; ++r)
+                    for(int t = i * B_TICKS / A_MFMAS; t < (i + 1) * B_TICKS / A_MFMAS; ++t)
                     {
-                        b_item(0, r);
+                        b_tick(0, t);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -1627,9 +1646,9 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                     c_read(0, i + AHEAD, ring);
                     c_mfma(0, i, ring);
     #pragma unroll
-                    for(int r = i * 16 / C_MFMAS; r < (i + 1) * 16 / C_MFMAS; ++r)
+                    for(int t = i * B_TICKS / C_MFMAS; t < (i + 1) * B_TICKS / C_MFMAS; ++t)
                     {
-                        b_item(1, r);
+                        b_tick(1, t);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
