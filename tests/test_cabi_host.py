@@ -81,6 +81,37 @@ def test_bad_arguments_are_rejected_before_launch(t):
     assert grid(None, ctypes.byref(g)) == h.EINVAL
 
 
+@pytest.mark.parametrize("t", ["bf16", "fp16"])
+def test_backward_grid_argument_checks(t):
+    """Refused before anything is launched: a null block, slab counts that
+    overflow the tile tables, a workspace that does not grow with the slabs."""
+    L = h.lib()
+    grid = getattr(L, "nntile_hip_sdpa_bwd_grid_" + t)
+    assert grid(None, None) == h.EINVAL
+    g = h.BwdGridArgs()
+    g.q_seq = g.k_seq = 512
+    g.q_tile = g.k_tile = 128
+    g.head, g.batch, g.n_batch, g.kv_group = 64, 2, 2, 1
+    g.n_q_tiles = g.n_kv_tiles = 4
+    g.mask_mode = h.MASK_CAUSAL
+    for i in range(h.BWD_MAX_TILES):
+        for name in ("K", "V", "Q", "A", "dA", "lse", "dK", "dQ", "dV"):
+            getattr(g, name)[i] = 4096
+    g.workspace, g.workspace_bytes = 4096, 4 * 512 * 2
+    assert L.nntile_hip_sdpa_bwd_grid_workspace_bytes(ctypes.byref(g)) == 4 * 512 * 2
+    g.n_slabs = 9                                                           # 9 * 4 tiles > 32
+    assert grid(None, ctypes.byref(g)) == h.EINVAL
+    g.n_slabs = -1
+    assert grid(None, ctypes.byref(g)) == h.EINVAL
+    g.n_slabs = 8                                                           # fits, but the workspace is for one slab
+    assert L.nntile_hip_sdpa_bwd_grid_workspace_bytes(ctypes.byref(g)) == 8 * 4 * 512 * 2
+    assert grid(None, ctypes.byref(g)) == h.EWORKSPACE
+    g.n_slabs = 1
+    g.q_tile = 96                                                           # not a multiple of 128
+    g.n_q_tiles = 6
+    assert grid(None, ctypes.byref(g)) == h.EUNSUPPORTED
+
+
 def test_decode_argument_checks():
     L = h.lib()
     a = _tile(q_seq=16, k_seq=512, head=128, batch=16, n_batch=2, kv_group=4)
