@@ -577,24 +577,24 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
             || (MODE == NNTILE_HIP_MASK_CAUSAL && kg0 + kBwdStep - 1 > rel + q_row0);
         if constexpr(EXPLICIT || NNTILE_BWD_PIPE_DQ == 0)
         {
-    #pragma unroll
+#pragma unroll
             for(int mb = 0; mb < 2; ++mb)
             {
                 f32x16 sv, dpv;
-    #pragma unroll
+#pragma unroll
                 for(int r = 0; r < 16; ++r)
                 {
                     sv[r] = 0.0f;
                     dpv[r] = 0.0f;
                 }
-    #pragma unroll
+#pragma unroll
                 for(int ks = 0; ks < KSTEPS; ++ks)
                 {
                     const vec8 ka = *reinterpret_cast<const vec8 *>(Ks + row_raddr[ks] + mb * 32 * RB);
                     const vec8 va = *reinterpret_cast<const vec8 *>(Vs + row_raddr[ks] + mb * 32 * RB);
                     sv = T::mfma(ka, qf[ks], sv);
                     dpv = T::mfma(va, gf[ks], dpv);
-    #pragma unroll
+#pragma unroll
                     for(int j = 0; j < LOADS_PER_WAVE; ++j)
                     {
                         if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
@@ -608,7 +608,7 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
                 // end of the keys and on the diagonal run (a wave-common branch).
                 if(bounds)
                 {
-    #pragma unroll
+#pragma unroll
                     for(int r = 0; r < 16; ++r)
                     {
                         const int key = mb * 32 + tile_row(r, half);
@@ -616,7 +616,7 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
                     }
                 }
                 float dsv[16];
-    #pragma unroll
+#pragma unroll
                 for(int r = 0; r < 16; ++r)
                 {
                     float e = fmaf(sv[r], c, -lse2);        // -inf: hidden, or a row that saw nothing
@@ -644,20 +644,20 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
                     dsv[r] = pr * (dpv[r] - d_row);
                 }
                 uint32_t ds_pk[8];
-    #pragma unroll
+#pragma unroll
                 for(int k = 0; k < 8; ++k)
                 {
                     ds_pk[k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
                 }
                 // ---- dQ^T += K^T dS^T: the block's two sub-steps of 16 keys ------------------
-    #pragma unroll
+#pragma unroll
                 for(int tt = 0; tt < 2; ++tt)
                 {
                     const int t = 2 * mb + tt;
                     const u32x4 braw = {ds_pk[4 * tt], ds_pk[4 * tt + 1], ds_pk[4 * tt + 2],
                         ds_pk[4 * tt + 3]};
                     const vec8 bop = __builtin_bit_cast(vec8, braw);
-    #pragma unroll
+#pragma unroll
                     for(int db = 0; db < DBLOCKS; ++db)
                     {
                         const u32x2 lo = bwd_lds_read_tr16(Ks + tr_raddr[0][db] + (16 * t) * RB);
@@ -679,7 +679,7 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
             constexpr int AHEAD = NNTILE_BWD_AHEAD;
             auto a_init = [&](int mb) __attribute__((always_inline))
             {
-    #pragma unroll
+#pragma unroll
                 for(int r = 0; r < 16; ++r)
                 {
                     sv[mb][r] = 0.0f;
@@ -701,7 +701,7 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
                 if(i & 1)
                 {
                     dpv[mb] = T::mfma(ring[i % (AHEAD + 1)], gf[ks], dpv[mb]);
-    #pragma unroll
+#pragma unroll
                     for(int j = 0; j < LOADS_PER_WAVE; ++j)
                     {
                         if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
@@ -722,7 +722,7 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
             {
                 if(bounds)
                 {
-    #pragma unroll
+#pragma unroll
                     for(int r = 0; r < 16; ++r)
                     {
                         const int key = mb * 32 + tile_row(r, half);
@@ -769,13 +769,13 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
             {
                 vec8 ring[AHEAD + 1];
                 a_init(0);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < AHEAD; ++i)
                 {
                     a_read(0, i, ring);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < A_MFMAS; ++i)
                 {
                     a_read(0, i + AHEAD, ring);
@@ -784,18 +784,18 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
                 }
                 hide(0);
                 a_init(1);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < AHEAD; ++i)
                 {
                     a_read(1, i, ring);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < A_MFMAS; ++i)
                 {
                     a_read(1, i + AHEAD, ring);
                     a_mfma(1, i, ring);
-    #pragma unroll
+#pragma unroll
                     for(int r = i * 16 / A_MFMAS; r < (i + 1) * 16 / A_MFMAS; ++r)
                     {
                         b_item(0, r);
@@ -803,31 +803,31 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 hide(1);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < AHEAD; ++i)
                 {
                     c_read(0, i, ring);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < C_MFMAS; ++i)
                 {
                     c_read(0, i + AHEAD, ring);
                     c_mfma(0, i, ring);
-    #pragma unroll
+#pragma unroll
                     for(int r = i * 16 / C_MFMAS; r < (i + 1) * 16 / C_MFMAS; ++r)
                     {
                         b_item(1, r);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < AHEAD; ++i)
                 {
                     c_read(1, i, ring);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < C_MFMAS; ++i)
                 {
                     c_read(1, i + AHEAD, ring);
@@ -1256,12 +1256,12 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             // (one 32-query block at a time: half the accumulators live)
             // ---- S = Q K^T, dP = dA V^T: rows are queries, the lane's column its key;
             // P, dS: register r of block mb is query q0 + mb*32 + tile_row(r, half) --------------
-    #pragma unroll
+#pragma unroll
             for(int mb = 0; mb < 2; ++mb)
             {
                 uint32_t p_pk[8], ds_pk[8];
                 f32x16 sv, dpv;
-    #pragma unroll
+#pragma unroll
                 for(int r = 0; r < 16; ++r)
                 {
                     sv[r] = 0.0f;
@@ -1271,19 +1271,19 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                 {
                     // dP - D: the accumulator starts at -D of its row (four
                     // consecutive queries per LDS read), the products add dP
-    #pragma unroll
+#pragma unroll
                     for(int rg = 0; rg < 4; ++rg)
                     {
                         const f32x4 nd4 = *reinterpret_cast<const f32x4 *>(
                                 &stat[1][mb * 32 + 8 * rg + 4 * half]);
-    #pragma unroll
+#pragma unroll
                         for(int e = 0; e < 4; ++e)
                         {
                             dpv[4 * rg + e] = nd4[e];
                         }
                     }
                 }
-    #pragma unroll
+#pragma unroll
                 for(int ks = 0; ks < KSTEPS; ++ks)
                 {
                     const vec8 qa = *reinterpret_cast<const vec8 *>(Qs + row_raddr[ks] + mb * 32 * RB);
@@ -1296,7 +1296,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                     }
                     if(LOADERS == kDkvWaves || wave_u < LOADERS)
                     {
-    #pragma unroll
+#pragma unroll
                         for(int j = 0; j < LPW; ++j)
                         {
                             if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
@@ -1313,7 +1313,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                 // wave-common branch).
                 if(bounds)
                 {
-    #pragma unroll
+#pragma unroll
                     for(int r = 0; r < 16; ++r)
                     {
                         const int qr = mb * 32 + tile_row(r, half);
@@ -1326,13 +1326,13 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                     }
                 }
                 float pv[16], dsv[16];
-    #pragma unroll
+#pragma unroll
                 for(int rg = 0; rg < 4; ++rg)
                 {
                     // four consecutive queries: their statistics in one LDS read each
                     const int qr0 = mb * 32 + 8 * rg + 4 * half;
                     const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(&stat[0][qr0]);
-    #pragma unroll
+#pragma unroll
                     for(int e = 0; e < 4; ++e)
                     {
                         const int r = 4 * rg + e;
@@ -1366,14 +1366,14 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                         dsv[r] = pv[r] * dpv[r];
                     }
                 }
-    #pragma unroll
+#pragma unroll
                 for(int k = 0; k < 8; ++k)
                 {
                     p_pk[k] = T::pack2(pv[2 * k], pv[2 * k + 1]);
                     ds_pk[k] = T::pack2(dsv[2 * k], dsv[2 * k + 1]);
                 }
                 // ---- dV^T += dA^T P, dK^T += Q^T dS: the block's two sub-steps of 16 queries ----
-    #pragma unroll
+#pragma unroll
                 for(int tt = 0; tt < 2; ++tt)
                 {
                     const int t = 2 * mb + tt;
@@ -1383,7 +1383,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                         ds_pk[4 * tt + 3]};
                     const vec8 pb = __builtin_bit_cast(vec8, praw);
                     const vec8 sb = __builtin_bit_cast(vec8, sraw);
-    #pragma unroll
+#pragma unroll
                     for(int db = 0; db < DBLOCKS; ++db)
                     {
                         if(DO_DV)
@@ -1423,7 +1423,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             {
                 if(bounds)
                 {
-    #pragma unroll
+#pragma unroll
                     for(int r = 0; r < 16; ++r)
                     {
                         const int qr = mb * 32 + tile_row(r, half);
@@ -1467,7 +1467,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                 if((LOADERS == kDkvWaves || wave_u < LOADERS) && NNTILE_BWD_SPREAD != 0
                         && (!DO_DK || (i & 1)))
                 {
-    #pragma unroll
+#pragma unroll
                     for(int j = 0; j < LPW; ++j)
                     {
                         if(mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
@@ -1480,7 +1480,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             };
             auto a_init = [&](int mb) __attribute__((always_inline))
             {
-    #pragma unroll
+#pragma unroll
                 for(int r = 0; r < 16; ++r)
                 {
                     sv[mb][r] = 0.0f;
@@ -1488,12 +1488,12 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                 }
                 if(DO_DK)
                 {
-    #pragma unroll
+#pragma unroll
                     for(int rg = 0; rg < 4; ++rg)
                     {
                         const f32x4 nd4 = *reinterpret_cast<const f32x4 *>(
                                 &stat[1][mb * 32 + 8 * rg + 4 * half]);
-    #pragma unroll
+#pragma unroll
                         for(int e = 0; e < 4; ++e)
                         {
                             dpv[mb][4 * rg + e] = nd4[e];
@@ -1596,13 +1596,13 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                 vec8 ring[AHEAD + 1];
                 // A0
                 a_init(0);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < AHEAD; ++i)
                 {
                     a_read(0, i, ring);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < A_MFMAS; ++i)
                 {
                     a_read(0, i + AHEAD, ring);
@@ -1613,18 +1613,18 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                 // A1 with B0
                 a_init(1);
                 b_begin(0);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < AHEAD; ++i)
                 {
                     a_read(1, i, ring);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < A_MFMAS; ++i)
                 {
                     a_read(1, i + AHEAD, ring);
                     a_mfma(1, i, ring);
-    #pragma unroll
+#pragma unroll
                     for(int t = i * B_TICKS / A_MFMAS; t < (i + 1) * B_TICKS / A_MFMAS; ++t)
                     {
                         b_tick(0, t);
@@ -1634,18 +1634,18 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                 hide(1);
                 // C0 with B1
                 b_begin(1);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < AHEAD; ++i)
                 {
                     c_read(0, i, ring);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < C_MFMAS; ++i)
                 {
                     c_read(0, i + AHEAD, ring);
                     c_mfma(0, i, ring);
-    #pragma unroll
+#pragma unroll
                     for(int t = i * B_TICKS / C_MFMAS; t < (i + 1) * B_TICKS / C_MFMAS; ++t)
                     {
                         b_tick(1, t);
@@ -1653,13 +1653,13 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 // C1
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < AHEAD; ++i)
                 {
                     c_read(1, i, ring);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
+#pragma unroll
                 for(int i = 0; i < C_MFMAS; ++i)
                 {
                     c_read(1, i + AHEAD, ring);
