@@ -205,14 +205,16 @@ def bench_power_context(cfg, seconds=1.5):
     """What the chip sustains under its power cap, for context: the cfg3
     prefill launch and a plain library GEMM (torch.matmul, 8192^3 bf16), each
     on N(0,1) data and on zeros, in loops of about `seconds`, with the board
-    power read beside them.  The matrix units' power depends on the data: on
+    power read beside them, and the matrix instruction alone on operands that
+    stay in registers.  The matrix units' power depends on the data: on
     zeros both run at the full clock, on random data both are held at the
     power cap.  Not a roofline - the published peak stays the yardstick - but
     it says how much of the distance to it any kernel can cover on such data."""
     import torch
     out = {"what": "loops of ~%.1f s; TFLOP/s and board power (W, amdgpu hwmon); the GEMM is the "
                    "library's (torch.matmul 8192^3 bf16), shown only as the sustained matrix rate "
-                   "of this GPU on the same kind of data" % seconds}
+                   "of this GPU on the same kind of data; mfma_only: v_mfma_f32_32x32x16_bf16 on "
+                   "operands held in registers, two wavefronts per SIMD, nothing else" % seconds}
     for key, zeros in (("prefill_cfg3_randn", False), ("prefill_cfg3_zeros", True)):
         with PowerSampler() as ps:
             r = bench_prefill(cfg, int(seconds / 130e-6), 50, zeros=zeros)
@@ -228,6 +230,30 @@ def bench_power_context(cfg, seconds=1.5):
             _, dev = time_steps(lambda: torch.matmul(a, b.t(), out=c), int(seconds / 0.6e-3), 20)
         out[key] = {"tflops": round(2.0 * n ** 3 / (dev * 1e-3) / 1e12, 1), "kernel_ms": round(dev, 4),
                     "watts": ps.watts()}
+    # the matrix units alone: v_mfma_f32_32x32x16_bf16 on operands held in
+    # registers, two wavefronts per SIMD (nntile_amd/csrc/mfma_probe.hip)
+    import ctypes
+    from nntile_amd import build as hip_build
+    if os.path.exists(hip_build.PROBE_LIB):
+        probe = ctypes.CDLL(hip_build.PROBE_LIB).nntile_hip_probe_mfma
+        probe.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32,
+                          ctypes.c_int32]
+        sink = torch.zeros(1, device="cuda")
+        iters, wgs = 20000, 512
+        for key, zeros in (("mfma_only_randn", False), ("mfma_only_zeros", True)):
+            ops = torch.zeros(8192, dtype=torch.bfloat16, device="cuda") if zeros else \
+                _randn((8192,), torch.bfloat16, 9, 0)
+            stream = torch.cuda.current_stream().cuda_stream
+
+            def step():
+                if probe(stream, ops.data_ptr(), sink.data_ptr(), iters, wgs) != 0:
+                    raise RuntimeError("mfma probe failed")
+
+            with PowerSampler() as ps:
+                _, dev = time_steps(step, max(3, int(seconds / 2.5e-3)), 3)
+            fl = wgs * 4 * iters * 4 * 32768.0
+            out[key] = {"tflops": round(fl / (dev * 1e-3) / 1e12, 1), "kernel_ms": round(dev, 4),
+                        "watts": ps.watts()}
     return out
 
 
