@@ -1009,6 +1009,17 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                     return;
                 }
                 const int i = slot_idx(sl);
+#ifdef NNTILE_PF_KO_LDSREAD     // (power attribution only: wrong results)
+                opnd[sl] = qf[i % KSTEPS];
+                return;
+#endif
+#ifdef NNTILE_PF_KO_HALFREAD    // (every second operand read only)
+                if(sl & 1)
+                {
+                    opnd[sl] = opnd[sl - 1];
+                    return;
+                }
+#endif
                 if(slot_kind(sl) == 1)
                 {
                     if(DO_S)
@@ -1042,7 +1053,13 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 const int k = it / 3, r = it % 3;
                 if(r < 2)
                 {
+#if defined(NNTILE_PF_KO_EXP)
+                    pe[r] = fmaf(s_cur[2 * k + r], c, -mc);
+#elif defined(NNTILE_PF_KO_SOFTMAX)
+                    pe[r] = s_cur[2 * k + r];
+#else
                     pe[r] = fast_exp2(fmaf(s_cur[2 * k + r], c, -mc));
+#endif
                 }
                 else
                 {
@@ -1081,7 +1098,11 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                     o[db] = T::mfma(opnd[sl], __builtin_bit_cast(vec8, praw), o[db]);
                 }
                 // the softmax items are spread over the slots 1 .. NSLOT-1
+#ifdef NNTILE_PF_KO_ITEMS
+                if(false)
+#else
                 if(DO_SM && sl >= 1)
+#endif
                 {
 #pragma unroll
                     for(int it = (sl - 1) * NITEM / (NSLOT - 1);
@@ -1090,16 +1111,23 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                         item(it);
                     }
                 }
+#ifndef NNTILE_PF_KO_DMA
                 if(DO_FETCH && (sl & 1))
                 {
                     fetch_piece(sl >> 1);
                 }
+#endif
                 __builtin_amdgcn_sched_barrier(0);
             }
             rescale_pending = false;
             if(DO_SM)
             {
+#if defined(NNTILE_PF_KO_EXP) || defined(NNTILE_PF_KO_SOFTMAX) || defined(NNTILE_PF_KO_ITEMS) \
+    || defined(NNTILE_PF_KO_LDSREAD)
+                if(false)       // (the knocked-out variants never redo a sub-block)
+#else
                 if(__builtin_amdgcn_ballot_w64(!(rs <= kLazyLimit)) != 0)
+#endif
                 {
                     float mx = s_cur[0];
 #pragma unroll
