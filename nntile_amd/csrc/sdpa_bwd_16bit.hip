@@ -34,6 +34,44 @@
 namespace nntile_hip
 {
 
+// Developer build (-DNNTILE_BWD_TRACE): shader-clock cycles that the first
+// wavefront of every key-owning workgroup spends in each phase of its steps,
+// summed over the steps; read back with nntile_hip_debug_bwd_trace.
+#ifdef NNTILE_BWD_TRACE
+__device__ unsigned long long bwd_trace[8 * 4096];
+__device__ unsigned long long bwd_wall[4 * 4096];
+#define BWD_WALL(i, part) do { if(threadIdx.x == 0 && blockIdx.x < 4096) { \
+        bwd_wall[4 * blockIdx.x + (i)] = wall_clock64(); bwd_wall[4 * blockIdx.x + 2] = (part); } } while(0)
+#define BWD_TRACE_DECL unsigned long long bt_sum[7] = {0, 0, 0, 0, 0, 0, 0}, bt_last = 0; int bt_steps = 0;
+#define BWD_TRACE_START() do { bt_last = clock64(); } while(0)
+#define BWD_TRACE_MARK(i) do { const unsigned long long now_ = clock64(); bt_sum[i] += now_ - bt_last; \
+        bt_last = now_; } while(0)
+#define BWD_TRACE_STEP() do { bt_steps += 1; } while(0)
+#define BWD_TRACE_FLUSH(part) do { if(threadIdx.x == 0 && blockIdx.x < 4096) { \
+        for(int i_ = 0; i_ < 6; ++i_) { bwd_trace[8 * blockIdx.x + i_] = bt_sum[i_]; } \
+        bwd_trace[8 * blockIdx.x + 6] = (unsigned long long)bt_steps; \
+        bwd_trace[8 * blockIdx.x + 7] = (unsigned long long)(part); } } while(0)
+}
+extern "C" int nntile_hip_debug_bwd_wall(unsigned long long *host)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(nntile_hip::bwd_wall), sizeof(nntile_hip::bwd_wall));
+}
+extern "C" int nntile_hip_debug_bwd_trace(unsigned long long *host)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(nntile_hip::bwd_trace), sizeof(nntile_hip::bwd_trace));
+}
+namespace nntile_hip
+{
+#else
+#define BWD_TRACE_DECL
+#define BWD_TRACE_START()
+#define BWD_TRACE_MARK(i)
+#define BWD_TRACE_STEP()
+#define BWD_TRACE_FLUSH(part)
+#define BWD_WALL(i, part)
+#endif
+
+
 // Where the tile loads of the next step are issued: 0 = all at the start of
 // the step, 1 = between the MFMAs of the step's first half, 2 = of the whole
 // 1: a step's two query (key) blocks overlap - the matrix products of one
@@ -926,6 +964,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
 {
     constexpr bool DO_DK = (PART & BWD_PART_DK) != 0, DO_DV = (PART & BWD_PART_DV) != 0;
     constexpr bool BOTH = DO_DK && DO_DV;
+    BWD_TRACE_DECL
     typedef typename T::vec8 vec8;
     typedef BwdTile<HEAD> G;
     constexpr int KSTEPS = G::KSTEPS, DBLOCKS = G::DBLOCKS, RB = G::RB, CPR = G::CPR;
@@ -1211,8 +1250,11 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
         const char *Qs = BUF ? lds_q1 : lds_q0;
         const char *Gs = BUF ? lds_g1 : lds_g0;
         const float (*stat)[kBwdStep] = lds_stat[BUF];
+        BWD_TRACE_START();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+        BWD_TRACE_MARK(0);
+        BWD_TRACE_STEP();
         // the statistics of the next step now, its tiles between the MFMAs
         // below (the last step loads its own tiles once more, rather than
         // branch)
@@ -1609,6 +1651,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                     a_mfma(0, i, ring);
                     __builtin_amdgcn_sched_barrier(0);
                 }
+                BWD_TRACE_MARK(1);
                 hide(0);
                 // A1 with B0
                 a_init(1);
@@ -1631,6 +1674,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
+                BWD_TRACE_MARK(2);
                 hide(1);
                 // C0 with B1
                 b_begin(1);
@@ -1652,6 +1696,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
+                BWD_TRACE_MARK(3);
                 // C1
 #pragma unroll
                 for(int i = 0; i < AHEAD; ++i)
@@ -1668,6 +1713,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
                 }
             }
         }
+        BWD_TRACE_MARK(4);
         // (the other buffer's readers passed this step's barrier; the next
         // step's barrier orders these writes before its reads)
         __builtin_amdgcn_sched_barrier(0);
@@ -1675,6 +1721,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
         {
             stat_store(raw_next, last_f, lds_stat[BUF ^ 1]);
         }
+        BWD_TRACE_MARK(5);
     };
     auto run = [&](int i, int i_next, auto buf_tag) __attribute__((always_inline))
     {
@@ -1704,6 +1751,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
     // workgroup's LDS can be given away)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
+    BWD_TRACE_FLUSH(PART);
     // ---- dK (+)= scale dk, dV (+)= dv -------------------------------------------------
     if(!k_ok)
     {
@@ -1760,6 +1808,7 @@ __global__ __launch_bounds__(kDkvThreads, 2)
 void sdpa_bwd_kernel(const std::conditional_t<GRID, BwdGridParams, BwdParams> p, unsigned n_dkv,
         unsigned n_dq)
 {
+    BWD_WALL(0, blockIdx.x < n_dkv ? 1 : (blockIdx.x < n_dkv + n_dq ? 0 : 2));
     typedef BwdTile<HEAD> G;
     static_assert(kDkvThreads == kBwdThreads, "one block size for the three parts");
     __shared__ __attribute__((aligned(1024))) char lds_0[G::BYTES];
@@ -1798,6 +1847,10 @@ void sdpa_bwd_kernel(const std::conditional_t<GRID, BwdGridParams, BwdParams> p,
         sdpa_bwd_dkv_body<T, HEAD, MODE, BWD_PART_DV, GRID>(p, blockIdx.x - n_dkv - n_dq, lds_0,
                 lds_1, lds_2, lds_3, lds_stat);
     }
+#ifdef NNTILE_BWD_TRACE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    BWD_WALL(1, blockIdx.x < n_dkv ? 1 : (blockIdx.x < n_dkv + n_dq ? 0 : 2));
+#endif
 }
 
 template<typename T, int HEAD, int MODE>
