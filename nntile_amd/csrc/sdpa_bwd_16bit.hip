@@ -42,6 +42,8 @@ __device__ unsigned long long bwd_trace[8 * 4096];
 __device__ unsigned long long bwd_wall[4 * 4096];
 #define BWD_WALL(i, part) do { if(threadIdx.x == 0 && blockIdx.x < 4096) { \
         bwd_wall[4 * blockIdx.x + (i)] = wall_clock64(); bwd_wall[4 * blockIdx.x + 2] = (part); } } while(0)
+#define BWD_WALL_AT(i) do { if(threadIdx.x == 0 && blockIdx.x < 4096) { \
+        bwd_wall[4 * blockIdx.x + (i)] = wall_clock64(); } } while(0)
 #define BWD_TRACE_DECL unsigned long long bt_sum[7] = {0, 0, 0, 0, 0, 0, 0}, bt_last = 0; int bt_steps = 0;
 #define BWD_TRACE_START() do { bt_last = clock64(); } while(0)
 #define BWD_TRACE_MARK(i) do { const unsigned long long now_ = clock64(); bt_sum[i] += now_ - bt_last; \
@@ -69,6 +71,7 @@ namespace nntile_hip
 #define BWD_TRACE_STEP()
 #define BWD_TRACE_FLUSH(part)
 #define BWD_WALL(i, part)
+#define BWD_WALL_AT(i)
 #endif
 
 
@@ -1243,6 +1246,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
     {
         fetch(i_cur, lds_q0, lds_g0, lds_stat[0]);
     }
+    BWD_WALL_AT(3);     // (developer trace: the workgroup is set up, its first tile requested)
     auto step = [&](int i, int i_next, auto buf_tag, auto masked_tag)
         __attribute__((always_inline))
     {
