@@ -949,11 +949,20 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
 // One set of workgroups per gradient (dK: S, dP, dK^T; dV: S, dV^T - the
 // scores are computed once more) fits two workgroups of 4 wavefronts on a CU.
 enum { BWD_PART_DK = 1, BWD_PART_DV = 2 };
-// Head sizes at which one workgroup holds both gradients of its keys.
+// Where one workgroup holds both gradients of its keys: at head sizes up to 64
+// under every mask mode; at head 128 (K and V fragments and the two
+// accumulators are 192 of a lane's 256 registers there) under the analytic
+// modes, with the blocks of a step one after the other and a few registers
+// spilled - 12 scratch accesses a step beside its 64 MFMAs.
 #ifndef NNTILE_BWD_FUSED_KEYS_HEAD
 #define NNTILE_BWD_FUSED_KEYS_HEAD 64
 #endif
-template<int HEAD> constexpr bool kBwdFusedKeys = HEAD <= NNTILE_BWD_FUSED_KEYS_HEAD;
+#ifndef NNTILE_BWD_FUSED_KEYS_HEAD_ANALYTIC
+#define NNTILE_BWD_FUSED_KEYS_HEAD_ANALYTIC 128
+#endif
+template<int HEAD, int MODE> constexpr bool kBwdFusedKeys = HEAD <= NNTILE_BWD_FUSED_KEYS_HEAD
+    || (HEAD <= NNTILE_BWD_FUSED_KEYS_HEAD_ANALYTIC
+            && (MODE == NNTILE_HIP_MASK_NONE || MODE == NNTILE_HIP_MASK_CAUSAL));
 constexpr int kBwdCUs = 256;
 constexpr int kDkvWaves = 4;
 constexpr int kDkvThreads = kDkvWaves * 64;
@@ -1297,7 +1306,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             + (int64_t)q0 * (int64_t)mask_row_bytes;
         const uint32_t mask_last_row = (uint32_t)(rows_here - 1) * mask_row_bytes;
 
-        if constexpr(EXPLICIT || NNTILE_BWD_PIPE == 0)
+        if constexpr(EXPLICIT || NNTILE_BWD_PIPE == 0 || (BOTH && HEAD > 64))
         {
             // (one 32-query block at a time: half the accumulators live)
             // ---- S = Q K^T, dP = dA V^T: rows are queries, the lane's column its key;
@@ -1889,7 +1898,7 @@ static int launch_bwd_mode(hipStream_t stream, const BwdParams &p)
     {
         return NNTILE_HIP_ELAUNCH;
     }
-    if constexpr(kBwdFusedKeys<HEAD>)
+    if constexpr(kBwdFusedKeys<HEAD, MODE>)
     {
         // One set of key-owning workgroups for both gradients (seven products
         // instead of eight) once the three sets would not all be resident at
@@ -1941,7 +1950,7 @@ static int launch_bwd_grid_mode(hipStream_t stream, const BwdGridParams &p,
             }
         }
     }
-    if constexpr(kBwdFusedKeys<HEAD>)
+    if constexpr(kBwdFusedKeys<HEAD, MODE>)
     {
         // One set of key-owning workgroups for both gradients (seven products
         // instead of eight) once the three sets would not all be resident at
