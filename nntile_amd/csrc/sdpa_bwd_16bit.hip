@@ -957,6 +957,9 @@ enum { BWD_PART_DK = 1, BWD_PART_DV = 2 };
 #ifndef NNTILE_BWD_FUSED_KEYS_HEAD
 #define NNTILE_BWD_FUSED_KEYS_HEAD 64
 #endif
+#ifndef NNTILE_BWD_FUSED_ORDER
+#define NNTILE_BWD_FUSED_ORDER 1      // 1: product by product at head 128; 0: S with dP, then dV with dK
+#endif
 #ifndef NNTILE_BWD_FUSED_KEYS_HEAD_ANALYTIC
 #define NNTILE_BWD_FUSED_KEYS_HEAD_ANALYTIC 128
 #endif
@@ -1306,7 +1309,133 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             + (int64_t)q0 * (int64_t)mask_row_bytes;
         const uint32_t mask_last_row = (uint32_t)(rows_here - 1) * mask_row_bytes;
 
-        if constexpr(EXPLICIT || NNTILE_BWD_PIPE == 0 || (BOTH && HEAD > 64))
+        if constexpr(!EXPLICIT && BOTH && HEAD > 64 && NNTILE_BWD_FUSED_ORDER == 1)
+        {
+            // Both gradients at head 128: 192 registers hold fragments and
+            // accumulators, so a block goes product by product - S, P, dV, then
+            // dP, dS, dK - and the probabilities in fp32 are all that crosses
+            // from the first half to the second.
+#pragma unroll
+            for(int mb = 0; mb < 2; ++mb)
+            {
+                f32x16 sv;
+#pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    sv[r] = 0.0f;
+                }
+#pragma unroll
+                for(int ks = 0; ks < KSTEPS; ++ks)
+                {
+                    const vec8 qa = *reinterpret_cast<const vec8 *>(Qs + row_raddr[ks]
+                            + mb * 32 * RB);
+                    sv = T::mfma(qa, kf[ks], sv);
+                    if(LOADERS == kDkvWaves || wave_u < LOADERS)
+                    {
+#pragma unroll
+                        for(int j = 0; j < LPW; ++j)
+                        {
+                            if(NNTILE_BWD_SPREAD != 0 && mb * KSTEPS + ks == 1 + j * FETCH_STRIDE)
+                            {
+                                fetch_piece(at_f, at_end_f, BUF ? lds_q0 : lds_q1,
+                                        BUF ? lds_g0 : lds_g1, j);
+                            }
+                        }
+                    }
+                }
+                if(bounds)
+                {
+#pragma unroll
+                    for(int r = 0; r < 16; ++r)
+                    {
+                        const int qr = mb * 32 + tile_row(r, half);
+                        bool vis = k_ok;
+                        if(MODE == NNTILE_HIP_MASK_CAUSAL)
+                        {
+                            vis = vis && (my_k <= rel + q0 + qr);
+                        }
+                        sv[r] = vis ? sv[r] : neg_inf();
+                    }
+                }
+                // P in place of S
+                uint32_t pk[8];
+#pragma unroll
+                for(int rg = 0; rg < 4; ++rg)
+                {
+                    const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(
+                            &stat[0][mb * 32 + 8 * rg + 4 * half]);
+#pragma unroll
+                    for(int e = 0; e < 4; ++e)
+                    {
+                        sv[4 * rg + e] = fast_exp2(fmaf(sv[4 * rg + e], c, -lse4[e]));
+                    }
+                }
+#pragma unroll
+                for(int k = 0; k < 8; ++k)
+                {
+                    pk[k] = T::pack2(sv[2 * k], sv[2 * k + 1]);
+                }
+                // dV^T += dA^T P
+#pragma unroll
+                for(int tt = 0; tt < 2; ++tt)
+                {
+                    const int t = 2 * mb + tt;
+                    const u32x4 praw = {pk[4 * tt], pk[4 * tt + 1], pk[4 * tt + 2], pk[4 * tt + 3]};
+                    const vec8 pb = __builtin_bit_cast(vec8, praw);
+#pragma unroll
+                    for(int db = 0; db < DBLOCKS; ++db)
+                    {
+                        const u32x2 glo = bwd_lds_read_tr16(Gs + tr_raddr[0][db] + (16 * t) * RB);
+                        const u32x2 ghi = bwd_lds_read_tr16(Gs + tr_raddr[1][db] + (16 * t) * RB);
+                        const u32x4 graw = {glo[0], glo[1], ghi[0], ghi[1]};
+                        dv[db] = T::mfma(__builtin_bit_cast(vec8, graw), pb, dv[db]);
+                    }
+                }
+                // dP - D
+                f32x16 dpv;
+#pragma unroll
+                for(int rg = 0; rg < 4; ++rg)
+                {
+                    const f32x4 nd4 = *reinterpret_cast<const f32x4 *>(
+                            &stat[1][mb * 32 + 8 * rg + 4 * half]);
+#pragma unroll
+                    for(int e = 0; e < 4; ++e)
+                    {
+                        dpv[4 * rg + e] = nd4[e];
+                    }
+                }
+#pragma unroll
+                for(int ks = 0; ks < KSTEPS; ++ks)
+                {
+                    const vec8 ga = *reinterpret_cast<const vec8 *>(Gs + row_raddr[ks]
+                            + mb * 32 * RB);
+                    dpv = T::mfma(ga, vf[ks], dpv);
+                }
+                // dS, in the registers of the packed P
+#pragma unroll
+                for(int k = 0; k < 8; ++k)
+                {
+                    pk[k] = T::pack2(sv[2 * k] * dpv[2 * k], sv[2 * k + 1] * dpv[2 * k + 1]);
+                }
+                // dK^T += Q^T dS
+#pragma unroll
+                for(int tt = 0; tt < 2; ++tt)
+                {
+                    const int t = 2 * mb + tt;
+                    const u32x4 sraw = {pk[4 * tt], pk[4 * tt + 1], pk[4 * tt + 2], pk[4 * tt + 3]};
+                    const vec8 sb = __builtin_bit_cast(vec8, sraw);
+#pragma unroll
+                    for(int db = 0; db < DBLOCKS; ++db)
+                    {
+                        const u32x2 qlo = bwd_lds_read_tr16(Qs + tr_raddr[0][db] + (16 * t) * RB);
+                        const u32x2 qhi = bwd_lds_read_tr16(Qs + tr_raddr[1][db] + (16 * t) * RB);
+                        const u32x4 qraw = {qlo[0], qlo[1], qhi[0], qhi[1]};
+                        dk[db] = T::mfma(__builtin_bit_cast(vec8, qraw), sb, dk[db]);
+                    }
+                }
+            }
+        }
+        else if constexpr(EXPLICIT || NNTILE_BWD_PIPE == 0 || (BOTH && HEAD > 64))
         {
             // (one 32-query block at a time: half the accumulators live)
             // ---- S = Q K^T, dP = dA V^T: rows are queries, the lane's column its key;
