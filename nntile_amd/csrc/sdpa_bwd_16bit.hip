@@ -957,6 +957,9 @@ enum { BWD_PART_DK = 1, BWD_PART_DV = 2 };
 #ifndef NNTILE_BWD_FUSED_KEYS_HEAD
 #define NNTILE_BWD_FUSED_KEYS_HEAD 64
 #endif
+#ifndef NNTILE_BWD_GOFF_IN_LDS
+#define NNTILE_BWD_GOFF_IN_LDS 1
+#endif
 #ifndef NNTILE_BWD_FUSED_ORDER
 #define NNTILE_BWD_FUSED_ORDER 1      // 1: product by product at head 128; 0: S with dP, then dV with dK
 #endif
@@ -1084,6 +1087,22 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
         ld_goff[i] = (uint32_t)(r * RB + (ld_cpos ^ G::swz(r)) * 16);
         ld_goff_end[i] = ld_goff[i] - (uint32_t)(max(r - (q_seq - 1) % kBwdStep, 0) * RB);
     }
+    // Both gradients at head 128 leave no registers for these tables, and a
+    // spilled entry is reloaded from scratch with a wait for every load in
+    // flight, the next step's tile loads included: they go to LDS, whose reads
+    // have a counter of their own.
+    constexpr bool GOFF_IN_LDS = BOTH && HEAD > 64 && NNTILE_BWD_GOFF_IN_LDS != 0;
+    __shared__ uint32_t lds_goff[GOFF_IN_LDS ? 2 * LPW * kDkvThreads : 1];
+    if constexpr(GOFF_IN_LDS)
+    {
+#pragma unroll
+        for(int i = 0; i < LPW; ++i)
+        {
+            lds_goff[i * kDkvThreads + tid] = ld_goff[i];
+            lds_goff[(LPW + i) * kDkvThreads + tid] = ld_goff_end[i];
+        }
+        // (each thread reads back what it wrote: no barrier needed)
+    }
     // row operand: lane (col, half) reads row mb*32+col, logical chunk 2*ks+half;
     // 32 rows further on the swizzle is the same, so mb goes into the immediate
     uint32_t row_raddr[KSTEPS];
@@ -1191,7 +1210,15 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
         const char *Gp = static_cast<const char *>(at.dA) + at.elem * RB;
         char *qdst = qdst_base + wave_u * LPW * 1024;
         char *gdst = gdst_base + wave_u * LPW * 1024;
-        const uint32_t goff = at_end ? ld_goff_end[j] : ld_goff[j];
+        uint32_t goff;
+        if constexpr(GOFF_IN_LDS)
+        {
+            goff = lds_goff[((at_end ? LPW : 0) + j) * kDkvThreads + tid];
+        }
+        else
+        {
+            goff = at_end ? ld_goff_end[j] : ld_goff[j];
+        }
         load_to_lds16<0, false>(Qp, goff, qdst + j * 1024);
         load_to_lds16<0, false>(Gp, goff, gdst + j * 1024);
     };
