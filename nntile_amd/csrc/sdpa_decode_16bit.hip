@@ -356,30 +356,73 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         // ---- mask: s[kb][r] is key 16*kb + 4*quad + r ----------------------------
         if(EXPLICIT)
         {
-            // the mask is [k_seq, q_seq]: row index = token
+            // the mask is [k_seq, q_seq]: row index = token.  Each block gives
+            // a lane four consecutive keys: a full step of an aligned mask
+            // takes one 8-byte (additive) or 4-byte (boolean) load per block.
+            // Otherwise element by element: keys past the end of a ragged step
+            // are hidden, and their loads are clamped to the step's last key
+            // instead of being branched around, so that a lane's loads are
+            // independent and overlap.
+            const int64_t mrow = (int64_t)tok * p.mask_ld + k_row0;
+            constexpr int ES = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 2 : 1;
+            const bool wide = (p.mask_ld % 4 == 0) && (k_row0 % 4 == 0)
+                && (reinterpret_cast<uintptr_t>(p.mask) % (4 * ES) == 0)
+                && keys_here == kDecKeys;
 #pragma unroll
             for(int kb = 0; kb < KB; ++kb)
             {
                 const int key0 = 16 * kb + 4 * quad;
-#pragma unroll
-                for(int e = 0; e < 4; ++e)
+                float add[4];
+                if(wide)
                 {
-                    float add;
-                    const int64_t mi = (int64_t)tok * p.mask_ld + k_row0 + key0 + e;
                     if(MODE == NNTILE_HIP_MASK_ADDITIVE)
                     {
-                        add = (key0 + e < keys_here)
-                            ? T::to_float(static_cast<const uint16_t *>(p.mask)[mi])
-                            : neg_inf();
+                        const u32x2 w = *reinterpret_cast<const u32x2 *>(
+                                static_cast<const uint16_t *>(p.mask) + mrow + key0);
+#pragma unroll
+                        for(int e = 0; e < 4; ++e)
+                        {
+                            add[e] = T::to_float((uint16_t)(
+                                        (e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu)));
+                        }
                     }
                     else
                     {
-                        add = (key0 + e < keys_here
-                                && static_cast<const uint8_t *>(p.mask)[mi] != 0)
-                            ? 0.0f : neg_inf();
+                        const uint32_t w = *reinterpret_cast<const uint32_t *>(
+                                static_cast<const uint8_t *>(p.mask) + mrow + key0);
+#pragma unroll
+                        for(int e = 0; e < 4; ++e)
+                        {
+                            add[e] = ((w >> (8 * e)) & 0xffu) != 0u ? 0.0f : neg_inf();
+                        }
                     }
-                    const float v = s[kb][e] * p.scale + add;
-                    s[kb][e] = (add == neg_inf()) ? neg_inf() : v;
+                }
+                else
+                {
+#pragma unroll
+                    for(int e = 0; e < 4; ++e)
+                    {
+                        const int64_t mi = mrow + max(min(key0 + e, keys_here - 1), 0);
+                        if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                        {
+                            add[e] = T::to_float(static_cast<const uint16_t *>(p.mask)[mi]);
+                        }
+                        else
+                        {
+                            add[e] = static_cast<const uint8_t *>(p.mask)[mi] != 0
+                                ? 0.0f : neg_inf();
+                        }
+                        if(key0 + e >= keys_here)
+                        {
+                            add[e] = neg_inf();
+                        }
+                    }
+                }
+#pragma unroll
+                for(int e = 0; e < 4; ++e)
+                {
+                    const float v = s[kb][e] * p.scale + add[e];
+                    s[kb][e] = (add[e] == neg_inf()) ? neg_inf() : v;
                 }
             }
         }

@@ -748,26 +748,30 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                         for(int rg = 0; rg < 4; ++rg)
                         {
                             const int key0 = mb * 32 + 8 * rg + 4 * half;
-                            const int64_t krow = k_row0 + key0;
 #pragma unroll
                             for(int e = 0; e < 4; ++e)
                             {
-                                // out-of-range keys of a ragged step are hidden
-                                // and their mask element is not touched
-                                float add = neg_inf();
-                                if(key0 + e < keys_here)
+                                // out-of-range keys of a ragged step are hidden;
+                                // their loads are clamped to the step's last key
+                                // instead of being branched around, so that the
+                                // 32 loads of a lane are independent and overlap
+                                const int64_t at = mask_row + k_row0
+                                    + max(min(key0 + e, keys_here - 1), 0);
+                                float add;
+                                if(MODE == NNTILE_HIP_MASK_ADDITIVE)
                                 {
-                                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
-                                    {
-                                        add = T::to_float(static_cast<const uint16_t *>(
-                                                    p.mask)[mask_row + krow + e]);
-                                    }
-                                    else
-                                    {
-                                        add = static_cast<const uint8_t *>(
-                                                p.mask)[mask_row + krow + e] != 0
-                                            ? 0.0f : neg_inf();
-                                    }
+                                    add = T::to_float(static_cast<const uint16_t *>(
+                                                p.mask)[at]);
+                                }
+                                else
+                                {
+                                    add = static_cast<const uint8_t *>(
+                                            p.mask)[at] != 0
+                                        ? 0.0f : neg_inf();
+                                }
+                                if(key0 + e >= keys_here)
+                                {
+                                    add = neg_inf();
                                 }
                                 s[mb][4 * rg + e] = fmaf(add, inv_scale,
                                         s[mb][4 * rg + e]);

@@ -347,6 +347,75 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         const int64_t k_row0 = (int64_t)kb * kKeys32;
         const int64_t k_pos_base = p.k_pos0 + (int64_t)kt * p.k_tile + k_row0;
         const int keys_here = (int)min((int64_t)kKeys32, k_len - k_row0);
+        // Explicit mask: the step's 16 values of this lane are loaded here,
+        // ahead of the chain of MFMAs.  Register r holds key
+        // 8*(r/4) + 4*half + r%4: four groups of four consecutive keys.  A full
+        // step of an aligned mask takes one 16-byte (additive) or 4-byte
+        // (boolean) load per group; lanes are queries, a mask row apart, so
+        // the cost of a load is the cache lines it touches, not its width.
+        // Otherwise element by element: keys past the end of a ragged step
+        // are hidden, and their loads are clamped to the step's last key
+        // instead of being branched around, so that the loads are independent.
+        float madd[EXPLICIT ? 16 : 1];
+        if(EXPLICIT)
+        {
+            const int64_t mrow = (q_ok ? my_q : 0) * p.mask_ld + k_row0;
+            constexpr int ES = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 4 : 1;
+            const bool wide = (p.mask_ld % 4 == 0) && (k_row0 % 4 == 0)
+                && (reinterpret_cast<uintptr_t>(p.mask) % (4 * ES) == 0)
+                && keys_here == kKeys32;
+            if(wide)
+            {
+#pragma unroll
+                for(int rg = 0; rg < 4; ++rg)
+                {
+                    const int64_t at = mrow + 8 * rg + 4 * half;
+                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                    {
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>(
+                                static_cast<const float *>(p.mask) + at);
+#pragma unroll
+                        for(int e = 0; e < 4; ++e)
+                        {
+                            madd[4 * rg + e] = v[e];
+                        }
+                    }
+                    else
+                    {
+                        const uint32_t w = *reinterpret_cast<const uint32_t *>(
+                                static_cast<const uint8_t *>(p.mask) + at);
+#pragma unroll
+                        for(int e = 0; e < 4; ++e)
+                        {
+                            madd[4 * rg + e] = ((w >> (8 * e)) & 0xffu) != 0u
+                                ? 0.0f : neg_inf();
+                        }
+                    }
+                }
+            }
+            else
+            {
+#pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    const int key = 8 * (r >> 2) + 4 * half + (r & 3);
+                    const int64_t at = mrow + max(min(key, keys_here - 1), 0);
+                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                    {
+                        madd[r] = static_cast<const float *>(p.mask)[at];
+                    }
+                    else
+                    {
+                        madd[r] = static_cast<const uint8_t *>(p.mask)[at] != 0
+                            ? 0.0f : neg_inf();
+                    }
+                    if(key >= keys_here)
+                    {
+                        madd[r] = neg_inf();
+                    }
+                }
+            }
+        }
         // One accumulator chain: a dependent MFMA of this shape issues right
         // behind its predecessor (64 cycles apart, measured), and the first one
         // takes a constant zero, so nothing is cleared or added up afterwards.
@@ -389,33 +458,11 @@ void sdpa_prefill_fp32_kernel(const PrefillParams p)
         // ---- mask: register r holds key 8*(r/4) + 4*half + r%4 ---------------
         if(EXPLICIT)
         {
-            const int64_t qrow = q_ok ? my_q : 0;
 #pragma unroll
-            for(int rg = 0; rg < 4; ++rg)
+            for(int r = 0; r < 16; ++r)
             {
-                const int key0 = 8 * rg + 4 * half;
-                const int64_t krow = k_row0 + key0;
-#pragma unroll
-                for(int e = 0; e < 4; ++e)
-                {
-                    float add;
-                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
-                    {
-                        add = (key0 + e < keys_here)
-                            ? static_cast<const float *>(p.mask)[
-                                qrow * p.mask_ld + krow + e]
-                            : neg_inf();
-                    }
-                    else
-                    {
-                        add = (key0 + e < keys_here
-                                && static_cast<const uint8_t *>(p.mask)[
-                                    qrow * p.mask_ld + krow + e] != 0)
-                            ? 0.0f : neg_inf();
-                    }
-                    const float v = s[4 * rg + e] * p.scale + add;
-                    s[4 * rg + e] = (add == neg_inf()) ? neg_inf() : v;
-                }
+                const float v = s[r] * p.scale + madd[r];
+                s[r] = (madd[r] == neg_inf()) ? neg_inf() : v;
             }
         }
         else
