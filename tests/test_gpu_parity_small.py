@@ -153,7 +153,7 @@ def test_grid_entry_matches_oracle(oracle, dtype, q_seq, k_seq, q_tile, k_tile, 
 @pytest.mark.parametrize("q_seq,k_seq,n_batch,group,n_kv,head", [
     (16, 512, 2, 4, 2, 128), (1, 300, 3, 4, 2, 128), (16, 1000, 1, 4, 1, 64),
     (5, 77, 2, 8, 3, 128), (16, 64, 1, 2, 2, 128), (64, 200, 2, 1, 2, 64)])
-@pytest.mark.parametrize("mode", ["causal", "bool", "none"])
+@pytest.mark.parametrize("mode", ["causal", "bool", "additive", "none"])
 def test_decode_entry_matches_oracle(oracle, dtype, q_seq, k_seq, n_batch, group, n_kv, head, mode):
     print("case", dtype, q_seq, k_seq, n_batch, group, n_kv, head, mode, flush=True)
     batch = n_batch * group * n_kv
@@ -166,7 +166,9 @@ def test_decode_entry_matches_oracle(oracle, dtype, q_seq, k_seq, n_batch, group
                      device="cuda")
     lse, A = H.fresh_outputs(batch, q_seq, head, dtype)
     m, mm = {"causal": (None, hip_sdpa.MASK_CAUSAL), "none": (None, hip_sdpa.MASK_NONE),
-             "bool": (None if mask is None else torch.from_numpy(mask).cuda(), hip_sdpa.MASK_BOOL)}[mode]
+             "bool": (None if mask is None else torch.from_numpy(mask).cuda(), hip_sdpa.MASK_BOOL),
+             "additive": (None if mask is None else H.additive_mask(mask, dtype).cuda(),
+                          hip_sdpa.MASK_ADDITIVE)}[mode]
     hip_sdpa.sdpa_fwd_decode(Kd, Qd, m, lse, Vd, A, mm, n_batch, group, ws, causal_offset=offset)
     torch.cuda.synchronize()
     assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
