@@ -292,6 +292,51 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         return step_lo + (j >= n_local ? j - n_local : j);
     };
 
+    // Explicit mask: the raw values of a full step of an aligned mask - per
+    // block of 16 keys the lane's four consecutive keys, one 8-byte (additive)
+    // or 4-byte (boolean) load - are requested one step ahead, BEFORE that
+    // step's K/V loads are issued.  Waiting for a load also waits for every
+    // load issued before it, so mask values requested behind the K/V loads of
+    // the next step would make each step wait for its successor's data.
+    u32x2 mnext[KB];
+#pragma unroll
+    for(int kb = 0; kb < KB; ++kb)
+    {
+        mnext[kb] = u32x2{0u, 0u};
+    }
+    bool mnext_wide = false;
+    const bool mask_aligned = EXPLICIT && (p.mask_ld % 4 == 0)
+        && (reinterpret_cast<uintptr_t>(p.mask)
+                % (MODE == NNTILE_HIP_MASK_ADDITIVE ? 8 : 4) == 0);
+    auto mask_request = [&](int it_req)
+    {
+        mnext_wide = false;
+        if(EXPLICIT && mask_aligned && it_req < n_local)
+        {
+            const int64_t kr = (int64_t)actual(it_req) * kDecKeys;
+            if(p.k_seq - kr >= kDecKeys)
+            {
+                mnext_wide = true;
+                const int64_t at = (int64_t)tok * p.mask_ld + kr + 4 * quad;
+#pragma unroll
+                for(int kb = 0; kb < KB; ++kb)
+                {
+                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
+                    {
+                        mnext[kb] = *reinterpret_cast<const u32x2 *>(
+                                static_cast<const uint16_t *>(p.mask) + at + 16 * kb);
+                    }
+                    else
+                    {
+                        mnext[kb][0] = *reinterpret_cast<const uint32_t *>(
+                                static_cast<const uint8_t *>(p.mask) + at + 16 * kb);
+                    }
+                }
+            }
+        }
+    };
+    mask_request(0);
+
     // prologue: STAGES-1 steps in flight
     if(0 < n_local) { fetch(actual(0), ring(std::integral_constant<int, 0>{})); }
     if(STAGES > 2 && 1 < n_local) { fetch(actual(1), ring(std::integral_constant<int, 1>{})); }
@@ -323,6 +368,21 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         if(it == 0) { DEC_STAMP(1); }
         if(it == n_local - 1) { DEC_STAMP(2); }
 #endif
+        // this step's mask values (they arrived with the wait above: the use
+        // below is where the compiler puts its own wait), then the request
+        // for the next step's
+        u32x2 mcur[KB];
+        const bool cur_wide = mnext_wide;
+        if(EXPLICIT)
+        {
+#pragma unroll
+            for(int kb = 0; kb < KB; ++kb)
+            {
+                mcur[kb] = mnext[kb];
+                asm volatile("" : "+v"(mcur[kb]));
+            }
+            mask_request(it + 1);
+        }
         {
             const int ahead = it + STAGES - 1;
             if(ahead < n_local)
@@ -356,44 +416,31 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         // ---- mask: s[kb][r] is key 16*kb + 4*quad + r ----------------------------
         if(EXPLICIT)
         {
-            // the mask is [k_seq, q_seq]: row index = token.  Each block gives
-            // a lane four consecutive keys: a full step of an aligned mask
-            // takes one 8-byte (additive) or 4-byte (boolean) load per block.
-            // Otherwise element by element: keys past the end of a ragged step
-            // are hidden, and their loads are clamped to the step's last key
-            // instead of being branched around, so that a lane's loads are
-            // independent and overlap.
+            // the mask is [k_seq, q_seq]: row index = token.  A full step of
+            // an aligned mask finds its values in mcur.  Otherwise element by
+            // element: keys past the end of a ragged step are hidden, and
+            // their loads are clamped to the step's last key instead of being
+            // branched around, so that a lane's loads are independent.
             const int64_t mrow = (int64_t)tok * p.mask_ld + k_row0;
-            constexpr int ES = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 2 : 1;
-            const bool wide = (p.mask_ld % 4 == 0) && (k_row0 % 4 == 0)
-                && (reinterpret_cast<uintptr_t>(p.mask) % (4 * ES) == 0)
-                && keys_here == kDecKeys;
 #pragma unroll
             for(int kb = 0; kb < KB; ++kb)
             {
                 const int key0 = 16 * kb + 4 * quad;
                 float add[4];
-                if(wide)
+                if(cur_wide)
                 {
-                    if(MODE == NNTILE_HIP_MASK_ADDITIVE)
-                    {
-                        const u32x2 w = *reinterpret_cast<const u32x2 *>(
-                                static_cast<const uint16_t *>(p.mask) + mrow + key0);
+                    const u32x2 w = mcur[kb];
 #pragma unroll
-                        for(int e = 0; e < 4; ++e)
+                    for(int e = 0; e < 4; ++e)
+                    {
+                        if(MODE == NNTILE_HIP_MASK_ADDITIVE)
                         {
                             add[e] = T::to_float((uint16_t)(
                                         (e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu)));
                         }
-                    }
-                    else
-                    {
-                        const uint32_t w = *reinterpret_cast<const uint32_t *>(
-                                static_cast<const uint8_t *>(p.mask) + mrow + key0);
-#pragma unroll
-                        for(int e = 0; e < 4; ++e)
+                        else
                         {
-                            add[e] = ((w >> (8 * e)) & 0xffu) != 0u ? 0.0f : neg_inf();
+                            add[e] = ((w[0] >> (8 * e)) & 0xffu) != 0u ? 0.0f : neg_inf();
                         }
                     }
                 }
