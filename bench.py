@@ -201,41 +201,47 @@ def bench_prefill(cfg, steps, warmup, zeros=False, settle_s=0.0, one_launch=True
             "tflops": cfg.flops() / (wall * 1e-3) / 1e12}
 
 
-def bench_power_context(cfg, seconds=1.5):
-    """What the chip sustains under its power cap, for context: the cfg3
-    prefill launch and a plain library GEMM (torch.matmul, 8192^3 bf16), each
-    on N(0,1) data and on zeros, in loops of about `seconds`, with the board
-    power read beside them, and the matrix instruction alone on operands that
-    stay in registers.  The matrix units' power depends on the data: on
-    zeros both run at the full clock, on random data both are held at the
-    power cap.  Not a roofline - the published peak stays the yardstick - but
-    it says how much of the distance to it any kernel can cover on such data."""
+def bench_library_gemm(seconds, zeros=False):
+    """A plain library GEMM (torch.matmul, 8192^3 bf16) in a loop of about
+    `seconds` with the board power read beside it: the matrix rate this GPU
+    sustains under its power cap on the benchmark's kind of data."""
+    import torch
+    n = 8192
+    a = torch.zeros(n, n, dtype=torch.bfloat16, device="cuda") if zeros else \
+        _randn((n, n), torch.bfloat16, 7, 0)
+    b = torch.zeros_like(a) if zeros else _randn((n, n), torch.bfloat16, 7, 1)
+    c = torch.empty_like(a)
+    with PowerSampler() as ps:
+        _, dev = time_steps(lambda: torch.matmul(a, b.t(), out=c), max(20, int(seconds / 0.6e-3)), 20)
+    return {"tflops": round(2.0 * n ** 3 / (dev * 1e-3) / 1e12, 1), "kernel_ms": round(dev, 4),
+            "watts": ps.watts()}
+
+
+def bench_power_context(cfg, seconds=1.5, probe_lib=None):
+    """What the chip sustains under its power cap, for context (--only
+    power_context): the cfg3 prefill launch and a plain library GEMM, each on
+    N(0,1) data and on zeros, in loops of about `seconds`, with the board power
+    read beside them; with --probe-lib PATH also the matrix instruction alone
+    on operands that stay in registers (PATH: a shared library that exports
+    nntile_hip_probe_mfma(stream, operands, sink, iters, workgroups); none is
+    built or shipped with the product).  The matrix units' power depends on
+    the data: on zeros both run at the full clock, on random data both are
+    held at the power cap.  Not a roofline - the published peak stays the
+    yardstick."""
     import torch
     out = {"what": "loops of ~%.1f s; TFLOP/s and board power (W, amdgpu hwmon); the GEMM is the "
-                   "library's (torch.matmul 8192^3 bf16), shown only as the sustained matrix rate "
-                   "of this GPU on the same kind of data; mfma_only: v_mfma_f32_32x32x16_bf16 on "
+                   "library's (torch.matmul 8192^3 bf16); mfma_only: v_mfma_f32_32x32x16_bf16 on "
                    "operands held in registers, two wavefronts per SIMD, nothing else" % seconds}
     for key, zeros in (("prefill_cfg3_randn", False), ("prefill_cfg3_zeros", True)):
         with PowerSampler() as ps:
             r = bench_prefill(cfg, int(seconds / 130e-6), 50, zeros=zeros)
         out[key] = {"tflops": round(cfg.flops() / (r["device_ms_per_step"] * 1e-3) / 1e12, 1),
                     "kernel_ms": round(r["device_ms_per_step"], 4), "watts": ps.watts()}
-    n = 8192
-    for key, zeros in (("library_gemm_randn", False), ("library_gemm_zeros", True)):
-        a = torch.zeros(n, n, dtype=torch.bfloat16, device="cuda") if zeros else \
-            _randn((n, n), torch.bfloat16, 7, 0)
-        b = torch.zeros_like(a) if zeros else _randn((n, n), torch.bfloat16, 7, 1)
-        c = torch.empty_like(a)
-        with PowerSampler() as ps:
-            _, dev = time_steps(lambda: torch.matmul(a, b.t(), out=c), int(seconds / 0.6e-3), 20)
-        out[key] = {"tflops": round(2.0 * n ** 3 / (dev * 1e-3) / 1e12, 1), "kernel_ms": round(dev, 4),
-                    "watts": ps.watts()}
-    # the matrix units alone: v_mfma_f32_32x32x16_bf16 on operands held in
-    # registers, two wavefronts per SIMD (nntile_amd/csrc/mfma_probe.hip)
-    import ctypes
-    from nntile_amd import build as hip_build
-    if os.path.exists(hip_build.PROBE_LIB):
-        probe = ctypes.CDLL(hip_build.PROBE_LIB).nntile_hip_probe_mfma
+    out["library_gemm_randn"] = bench_library_gemm(seconds)
+    out["library_gemm_zeros"] = bench_library_gemm(seconds, zeros=True)
+    if probe_lib:
+        import ctypes
+        probe = ctypes.CDLL(os.path.abspath(probe_lib)).nntile_hip_probe_mfma
         probe.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32,
                           ctypes.c_int32]
         sink = torch.zeros(1, device="cuda")
@@ -700,15 +706,89 @@ def cpu_baseline(cfg, target_seconds=15.0):
             "seconds": dt}
 
 
+DETAIL_FILE = os.path.join("gpurun_out", "bench_detail.json")
+LINE_LIMIT = 4000     # bytes; the driver keeps only the tail of stdout
+
+
+def compact_line(main_leg, dec, ref_api, backward, gemm, cpu, args, cfg3, cfg4, watts=None):
+    """The ONE line printed last: the headline, both rooflines, the
+    reference-signature path, the backward and the CPU baseline.  Everything
+    else goes to DETAIL_FILE."""
+    r3 = lambda x: round(x, 3)
+    out = {
+        "metric": "sdpa_fwd_tflops",
+        "value": round(main_leg["tflops"], 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_leg["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic N(0,1), counter-based generator of the parity tests, seed 42 + config index, "
+                "rounded to bf16",
+        "config": {"workload": cfg3.name, "head_size": cfg3.head, "n_head": cfg3.n_head_kv,
+                   "seq_len": cfg3.q_seq, "batch": cfg3.n_batch, "seq_tile": cfg3.seq_tile,
+                   "mask": "causal", "flops_per_step_causal_exact": cfg3.flops(),
+                   "launches_per_step": main_leg["launches_per_step"],
+                   "timed": "one fused launch over the 4x4 grid of separately allocated tiles, analytic "
+                            "causal mask, overwrite mode; value = causal-exact FLOPs / wall time per step"},
+        "roofline": roofline("mfma", "sdpa_prefill_16bit_kernel<bf16,128,causal>", cfg3.flops(),
+                             main_leg["device_ms_per_step"], PEAK_BF16_TFLOPS, "TFLOP/s",
+                             TRAFFIC[cfg3.name]),
+        "decode": {"workload": cfg4.name, "ms_per_step": round(dec["ms_per_step"], 4),
+                   "value": round(dec["gbs"], 1), "unit": "GB/s",
+                   "roofline": roofline("hbm", dec.get("kernel", "sdpa_decode_16bit_kernel"),
+                                        dec["algorithmic_bytes"], dec["device_ms_per_step"],
+                                        PEAK_HBM_GBS, "GB/s", TRAFFIC[cfg4.name])},
+        "detail_file": DETAIL_FILE,
+    }
+    if gemm is not None:
+        # the matrix rate the board sustains on this kind of data under its
+        # power cap, measured in this run: context for roofline.frac, no
+        # replacement for the published peak
+        out["roofline"]["context"] = {"library_gemm_randn_tflops": gemm["tflops"],
+                                      "library_gemm_watts": gemm["watts"], "prefill_watts": watts}
+    if ref_api is not None:
+        out["per_task_path"] = {
+            "what": "cfg3 through tensor::flash_sdpa_fwd_cudnn_async with the reference's six arguments "
+                    "and a materialised causal mask (C++ host mirror); every_pair = its literal "
+                    "one-task-per-tile-pair submission",
+            "ms_per_step": ref_api["default_overload"]["ms_per_step"],
+            "launches": ref_api["default_overload"]["launches_per_step"],
+            "every_pair_ms_per_step": ref_api["every_pair"]["ms_per_step"],
+            "every_pair_launches": ref_api["every_pair"]["launches_per_step"]}
+    if backward is not None:
+        out["backward"] = {"ms_per_step": backward["ms_per_step"],
+                           "frac": backward["roofline"]["frac"],
+                           "kernel_ms": backward["roofline"]["kernel_ms"]}
+    if cpu is not None:
+        out["cpu_baseline"] = {"value": round(cpu["value"], 5), "unit": cpu["unit"], "cores": cpu["cores"],
+                               "kind": cpu["kind"], "sample": cpu["sample"],
+                               "seconds": round(cpu["seconds"], 2)}
+    line = json.dumps(out)
+    if len(line) > LINE_LIMIT:
+        raise RuntimeError("bench.py: the result line is %d bytes, limit %d" % (len(line), LINE_LIMIT))
+    return line
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--brief", action="store_true",
+                    help="only the legs of the result line (headline, decode, reference signature, "
+                         "backward, CPU baseline); no detail file")
     ap.add_argument("--case", default=None,
                     help="with --only reference_grid: one case, as dtype,seq,head,batch,mask "
                          "(e.g. bf16,4096,64,8,causal)")
+    ap.add_argument("--probe-lib", default=None,
+                    help="with --only power_context: a shared library exporting nntile_hip_probe_mfma "
+                         "(the matrix instruction alone); not part of the product")
     ap.add_argument("--only", default=None,
                     help="run only this leg (for profiling): prefill | cfg5 | cfg2 | decode | decode_wide | "
                          "reference_api | reference_grid | power_context | copy_context | backward | backward_slabs | rope | transpose | accumulate | "
@@ -744,7 +824,7 @@ def main():
             "decode_wide": lambda: bench_decode(cfg4_wide, args.steps, args.warmup),
             "reference_api": lambda: bench_reference_api(cfg3, args.steps, args.warmup),
             "reference_grid": lambda: bench_reference_grid(args.steps, args.warmup, args.case),
-            "power_context": lambda: bench_power_context(cfg3),
+            "power_context": lambda: bench_power_context(cfg3, probe_lib=args.probe_lib),
             "copy_context": lambda: bench_copy_context(args.steps, args.warmup),
             "backward": lambda: bench_backward(cfg3, args.steps, args.warmup),
             "rope": lambda: bench_rope(cfg3, args.steps, args.warmup),
@@ -771,132 +851,85 @@ def main():
         show(legs[only]())
         return
 
-    few = max(5, args.steps // 5)
-    dec = bench_decode(cfg4, args.steps, args.warmup)
-    dec_wide = bench_decode(cfg4_wide, few, 5)
+    # every leg is timed over at least 20 steps after at least 5 warm-up
+    # steps, whatever --steps says; the secondary legs take a fifth of it
+    steps = max(20, args.steps)
+    warmup = max(5, args.warmup)
+    few = max(20, args.steps // 5)
+    dec = bench_decode(cfg4, max(steps, 100), max(warmup, 20))
     ref_api = bench_reference_api(cfg3, few, 5)
-    ref_grid = bench_reference_grid(max(5, args.steps // 25), 3)
-    extras = {}
-    for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):
-        c = BY_NAME[name]
-        r = bench_prefill(c, few, 3)
-        fp32 = c.dtype == "fp32"
-        extras[name] = {
+    backward = bench_backward(cfg3, max(20, args.steps // 10), 5)
+    detail = {}
+    if not args.brief:
+        detail["decode_many_sequences"] = (lambda r: {
+            "workload": cfg4_wide.name,
+            "what": "for information: cfg4's bytes as 64 sequences x 8 kv heads x 1024 keys, 16 new "
+                    "tokens each; one key split per unit, no merge launch",
+            "roofline": roofline("hbm", "sdpa_decode_16bit_kernel (single split)",
+                                 r["algorithmic_bytes"], r["device_ms_per_step"],
+                                 PEAK_HBM_GBS, "GB/s")})(bench_decode(cfg4_wide, few, 5))
+        detail["reference_bench_grid"] = bench_reference_grid(20, 5)
+        extras = {}
+        for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):
+            c = BY_NAME[name]
+            r = bench_prefill(c, few, 5)
+            fp32 = c.dtype == "fp32"
+            extras[name] = {
+                "ms_per_step": round(r["ms_per_step"], 4), "tflops": round(r["tflops"], 2),
+                "flops_causal_exact": c.flops(), "launches_per_step": r["launches_per_step"],
+                "roofline": roofline("mfma", "sdpa_prefill_fp32_kernel<%d,causal>" % c.head if fp32
+                                     else "sdpa_prefill_16bit_kernel<bf16,%d,causal>" % c.head,
+                                     c.flops(), r["device_ms_per_step"],
+                                     PEAK_FP32_TFLOPS if fp32 else PEAK_BF16_TFLOPS, "TFLOP/s",
+                                     TRAFFIC.get(name))}
+            if c.calls > 1:
+                r1 = bench_prefill(c, few, 5, one_launch=False)
+                extras[name]["one_launch_per_slab"] = {
+                    "what": "the same with one launch per slab of the batch grid (%d launches)" % c.calls,
+                    "ms_per_step": round(r1["ms_per_step"], 4), "tflops": round(r1["tflops"], 2),
+                    "launches_per_step": r1["launches_per_step"]}
+        # cfg2's tiling on 16-bit tiles (the shape of the reference's GPT-2 flash
+        # path): the slabs of the batch grid in one launch and one by one
+        import dataclasses
+        gpt2_bf16 = dataclasses.replace(BY_NAME["cfg2_gpt2_small_fp32"], name="cfg2_shape_in_bf16",
+                                        dtype="bf16")
+        r, r1 = bench_prefill(gpt2_bf16, few, 5), bench_prefill(gpt2_bf16, few, 5, one_launch=False)
+        extras[gpt2_bf16.name] = {
+            "what": "for information: cfg2's shape and tiling on bf16 tiles",
             "ms_per_step": round(r["ms_per_step"], 4), "tflops": round(r["tflops"], 2),
-            "flops_causal_exact": c.flops(), "launches_per_step": r["launches_per_step"],
-            "roofline": roofline("mfma", "sdpa_prefill_fp32_kernel<%d,causal>" % c.head if fp32
-                                 else "sdpa_prefill_16bit_kernel<bf16,%d,causal>" % c.head,
-                                 c.flops(), r["device_ms_per_step"],
-                                 PEAK_FP32_TFLOPS if fp32 else PEAK_BF16_TFLOPS, "TFLOP/s",
-                                 TRAFFIC.get(name))}
-        if c.calls > 1:
-            r1 = bench_prefill(c, few, 3, one_launch=False)
-            extras[name]["one_launch_per_slab"] = {
-                "what": "the same with one launch per slab of the batch grid (%d launches)" % c.calls,
-                "ms_per_step": round(r1["ms_per_step"], 4), "tflops": round(r1["tflops"], 2),
-                "launches_per_step": r1["launches_per_step"]}
-    # cfg2's tiling on 16-bit tiles (the shape of the reference's GPT-2 flash
-    # path): the slabs of the batch grid in one launch and one by one
-    import dataclasses
-    gpt2_bf16 = dataclasses.replace(BY_NAME["cfg2_gpt2_small_fp32"], name="cfg2_shape_in_bf16",
-                                    dtype="bf16")
-    r, r1 = bench_prefill(gpt2_bf16, few, 3), bench_prefill(gpt2_bf16, few, 3, one_launch=False)
-    extras[gpt2_bf16.name] = {
-        "what": "for information: cfg2's shape and tiling on bf16 tiles",
-        "ms_per_step": round(r["ms_per_step"], 4), "tflops": round(r["tflops"], 2),
-        "launches_per_step": r["launches_per_step"],
-        "frac_of_peak": round(r["tflops"] / PEAK_BF16_TFLOPS, 4),
-        "one_launch_per_slab": {"ms_per_step": round(r1["ms_per_step"], 4),
-                                "tflops": round(r1["tflops"], 2),
-                                "launches_per_step": r1["launches_per_step"]},
-        "backward": bench_backward_slabs(gpt2_bf16, few, 3)}
-    backward = bench_backward(cfg3, max(5, args.steps // 10), 3)
-    rope = bench_rope(cfg3, few, 5)
-    transpose = bench_transpose(cfg3, few, 5)
-    kv_cache = bench_kv_cache(cfg4, few, 5)
-    accumulate = bench_accumulate(cfg3, few, 5)
-    power = bench_power_context(cfg3)
-    copy_ctx = bench_copy_context(few, 5)
+            "launches_per_step": r["launches_per_step"],
+            "frac_of_peak": round(r["tflops"] / PEAK_BF16_TFLOPS, 4),
+            "one_launch_per_slab": {"ms_per_step": round(r1["ms_per_step"], 4),
+                                    "tflops": round(r1["tflops"], 2),
+                                    "launches_per_step": r1["launches_per_step"]},
+            "backward": bench_backward_slabs(gpt2_bf16, few, 5)}
+        detail["other_configs"] = extras
+        detail["rope"] = bench_rope(cfg3, few, 5)
+        detail["transpose"] = bench_transpose(cfg3, few, 5)
+        detail["kv_cache"] = bench_kv_cache(cfg4, few, 5)
+        detail["accumulate_attn_output"] = bench_accumulate(cfg3, few, 5)
+    # the sustained matrix rate of the board on the same kind of data, for
+    # roofline.context (a library GEMM for about half a second)
+    gemm = bench_library_gemm(0.5)
     # The headline leg runs last and after 0.3 s of its own launch, untimed:
     # the first timed loop of a process, and a loop that follows another kind
     # of load (a copy, a library GEMM), measure up to 5 % slower than the same
     # loop a moment later (clock and power still settling), whatever the
     # warm-up count.  The W warm-up steps and the K timed steps follow.
-    main_leg = bench_prefill(cfg3, args.steps, args.warmup, settle_s=0.3)
-
-    out = {
-        "metric": "sdpa_fwd_tflops",
-        "value": round(main_leg["tflops"], 2),
-        "unit": "TFLOP/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(main_leg["ms_per_step"], 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": DATA,
-        "config": {"workload": cfg3.name, "head_size": cfg3.head, "n_head": cfg3.n_head_kv,
-                   "seq_len": cfg3.q_seq, "batch": cfg3.n_batch, "seq_tile": cfg3.seq_tile,
-                   "mask": "causal", "flops_per_step_causal_exact": cfg3.flops(),
-                   "flops_per_step_dense": cfg3.flops(False),
-                   "launches_per_step": main_leg["launches_per_step"],
-                   "timed": "one fused launch over the 4x4 grid of separately allocated tiles, "
-                            "analytic causal mask (6 fully hidden tile pairs skipped), overwrite mode: "
-                            "the launch defines (lse, A), which replaces the caller's fills of lse "
-                            "with -inf and of A with 0 (layer/sdpa.py:538-539); value = causal-exact "
-                            "FLOPs / wall time per step; roofline.kernel_ms = HIP-event time per "
-                            "step of the same loop; the W warm-up steps are preceded by 0.3 s of the "
-                            "same launch, untimed (clock and power settle on this load)"},
-        "roofline": roofline("mfma", "sdpa_prefill_16bit_kernel<bf16,128,causal>", cfg3.flops(),
-                             main_leg["device_ms_per_step"], PEAK_BF16_TFLOPS, "TFLOP/s",
-                             TRAFFIC[cfg3.name]),
-        "decode": {"workload": cfg4.name, "ms_per_step": round(dec["ms_per_step"], 4),
-                   "value": round(dec["gbs"], 1), "unit": "GB/s",
-                   "tflops": round(dec["tflops"], 2),
-                   "roofline": roofline("hbm", "sdpa_decode_16bit_kernel + sdpa_decode_reduce_kernel",
-                                        dec["algorithmic_bytes"], dec["device_ms_per_step"],
-                                        PEAK_HBM_GBS, "GB/s", TRAFFIC[cfg4.name],
-                                        {"algorithmic_bytes": dec["algorithmic_bytes"],
-                                         "workspace_bytes": dec["workspace_bytes"]})},
-        "decode_many_sequences": {
-            "workload": cfg4_wide.name,
-            "what": "for information: cfg4's bytes as 64 sequences x 8 kv heads x 1024 keys, 16 new "
-                    "tokens each; one key split per unit, no merge launch",
-            "roofline": roofline("hbm", "sdpa_decode_16bit_kernel (single split)",
-                                 dec_wide["algorithmic_bytes"], dec_wide["device_ms_per_step"],
-                                 PEAK_HBM_GBS, "GB/s")},
-        "per_task_path": {
-            "what": "cfg3 as an unchanged caller runs it, through the C++ mirror of the reference's "
-                    "tensor layer: tiled tensors, a materialised additive causal mask, per pass the "
-                    "-inf fill of logsumexp and tensor::flash_sdpa_fwd_cudnn_async(K, Q, mask, "
-                    "logsumexp, V, A) with the reference's six arguments.  The mask's tiles are "
-                    "classified the first time the mask is seen and the classes kept with its "
-                    "handles: the causal rule -> one launch in merge mode",
-            "ms_per_step": ref_api["default_overload"]["ms_per_step"],
-            "tflops": ref_api["default_overload"]["tflops"],
-            "launches_per_step": ref_api["default_overload"]["launches_per_step"],
-            "mask_classifications": ref_api["default_overload"]["mask_classifications"],
-            "every_pair": dict(ref_api["every_pair"],
-                               what="the reference's submission literally "
-                                    "(tensor::flash_sdpa_fwd_cudnn_pairs_async): 16 tile tasks with "
-                                    "their additive mask tiles, (lse, A) handed over in bf16")},
-        "reference_bench_grid": ref_grid,
-        "other_configs": extras,
-        "backward": backward,
-        "rope": rope,
-        "transpose": transpose,
-        "kv_cache": kv_cache,
-        "accumulate_attn_output": accumulate,
-        "power_context": power,
-        "copy_context": copy_ctx,
-    }
-    if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(cfg3)
-        out["cpu_baseline"]["value"] = round(out["cpu_baseline"]["value"], 5)
-        out["cpu_baseline"]["seconds"] = round(out["cpu_baseline"]["seconds"], 2)
-    print(json.dumps(out))
+    with PowerSampler() as ps:
+        main_leg = bench_prefill(cfg3, args.steps, args.warmup, settle_s=0.3)
+    cpu = None if args.no_cpu else cpu_baseline(cfg3)
+    line = compact_line(main_leg, dec, ref_api, backward, gemm, cpu, args, cfg3, cfg4, ps.watts())
+    if not args.brief:
+        detail = dict({"headline": json.loads(line), "per_task_path": ref_api, "backward": backward,
+                       "decode": dec}, **detail)
+        try:
+            os.makedirs(os.path.dirname(DETAIL_FILE), exist_ok=True)
+            with open(DETAIL_FILE, "w") as f:
+                json.dump(detail, f, indent=1)
+        except OSError as e:
+            sys.stderr.write("bench.py: detail file not written: %s\n" % e)
+    print(line)
 
 
 if __name__ == "__main__":

@@ -12,8 +12,6 @@ LIB = os.path.join(HERE, "libnntile_hip_sdpa.so")
 SOURCES = ["sdpa_prefill_16bit.hip", "sdpa_prefill_fp32.hip",
            "sdpa_decode_16bit.hip", "sdpa_bwd_16bit.hip", "rope.hip", "transpose.hip", "kv_cache.hip", "mask_classify.hip",
            "accumulate_attn_output.hip", "capi.hip"]
-PROBE_SOURCE = "mfma_probe.hip"
-PROBE_LIB = os.path.join(HERE, "libnntile_hip_probe.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -60,16 +58,6 @@ def build(force=False, verbose=True):
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)
-    # the measurement aid of bench.py's power_context leg: a library of its own
-    src = os.path.join(CSRC, PROBE_SOURCE)
-    if force or not os.path.exists(PROBE_LIB) or os.path.getmtime(src) > os.path.getmtime(PROBE_LIB):
-        cmd = [HIPCC] + FLAGS + ["-shared", src, "-o", PROBE_LIB]
-        if verbose:
-            print(" ".join(cmd), flush=True)
-        out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
-        if out.returncode != 0:
-            print(out.stdout.decode())
-            raise RuntimeError("hipcc failed")
     return LIB
 
 
