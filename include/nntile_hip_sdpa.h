@@ -51,6 +51,12 @@ extern "C" {
  * steps (SPLIT).  Both set, or a 16-bit call: ignored. */
 #define NNTILE_HIP_SDPA_FORM_SHARED 0x100
 #define NNTILE_HIP_SDPA_FORM_SPLIT  0x200
+/* decode calls, for tests and tuning: merge the key splits in a second launch
+ * instead of inside the main one (SEPARATE_MERGE); exchange the partials of
+ * the in-launch merge through device-scope fences whatever XCD the
+ * workgroups run on (FENCED). */
+#define NNTILE_HIP_SDPA_DECODE_SEPARATE_MERGE 0x400
+#define NNTILE_HIP_SDPA_DECODE_FENCED         0x800
 
 /* How visibility of key k to query q is given. */
 enum nntile_hip_mask_mode

@@ -24,6 +24,7 @@ int launch_bwd_grid_16bit(hipStream_t stream, const BwdGridParams &p,
         const void *const *A_tiles, int n_q_tiles, int head, int mode);
 size_t decode_workspace_bytes(int units, int n_splits, int rows, int head);
 size_t decode_partial_o_bytes(int units, int n_splits, int rows, int head);
+size_t decode_partial_ml_bytes(int units, int n_splits, int rows);
 
 struct F32Store;
 struct Bf16Store;
@@ -515,6 +516,10 @@ static int decode_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *
     p.part_o = static_cast<float *>(workspace);
     p.part_ml = reinterpret_cast<float *>(static_cast<char *>(workspace)
             + decode_partial_o_bytes(units, splits, rows, (int)a->head));
+    p.sync = reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.part_ml)
+            + decode_partial_ml_bytes(units, splits, rows));
+    p.fused = (a->flags & NNTILE_HIP_SDPA_DECODE_SEPARATE_MERGE) ? 0 : 1;
+    p.fenced = (a->flags & NNTILE_HIP_SDPA_DECODE_FENCED) ? 1 : 0;
     p.n_batch = (int32_t)a->n_batch;
     p.kv_group = (int32_t)a->kv_group;
     p.n_head_kv = (int32_t)(units / a->n_batch);

@@ -92,6 +92,16 @@ struct DecodeParams
     int32_t n_splits, steps_per_split, n_steps;
     int32_t overwrite;
     float scale;
+    // Merge inside the main launch (fused != 0): the grid holds n_main main
+    // workgroups followed by merge_blocks_per_unit merge workgroups per unit.
+    // sync: per unit sync_stride 64-bit words - word 0 is reserved, word
+    // 1 + rb*n_splits + s is the flag that split s raises for merge workgroup
+    // rb of the unit (the launch's tag; the merge workgroup sets it back to 0).
+    unsigned long long *sync;
+    unsigned long long tag;         // unique per call, never 0
+    unsigned long long spin_limit;  // longest wait for a flag, in 100 MHz ticks
+    int32_t fused, fenced;
+    int32_t n_main, merge_blocks_per_unit, sync_stride;
 };
 
 // Kernel arguments of the backward kernels.  K, V, dK, dV: [head, k_seq,

@@ -17,6 +17,8 @@
 //    O^T += V^T P^T with P^T taken from the S^T accumulators); LDS rows are
 //    unpadded and XOR-swizzled by 16-byte chunks against bank conflicts, and
 //    the V operand is gathered with the transposing ds_read_b64_tr_b16.
+#include <atomic>
+#include <random>
 #include <type_traits>
 
 #include "sdpa_common.hpp"
@@ -93,6 +95,242 @@ template<int N> __device__ __forceinline__ void wait_vmcnt()
     asm volatile("" ::: "memory");
 }
 
+// Loads that are served by the L2 (never by a CU's own cache): what one
+// workgroup reads of memory another workgroup of the same launch has written.
+template<bool COH>
+__device__ __forceinline__ unsigned long long ld64(const void *ptr)
+{
+    if(COH)
+    {
+        return __hip_atomic_load(
+                const_cast<unsigned long long *>(static_cast<const unsigned long long *>(ptr)),
+                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return *static_cast<const unsigned long long *>(ptr);
+}
+
+template<bool COH>
+__device__ __forceinline__ float ld32f(const float *ptr)
+{
+    if(COH)
+    {
+        return __hip_atomic_load(const_cast<float *>(ptr), __ATOMIC_RELAXED,
+                __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return *ptr;
+}
+
+// The XCD this wavefront runs on (hardware register XCC_ID, bits 3:0).
+__device__ __forceinline__ int xcc_id()
+{
+    return (int)(__builtin_amdgcn_s_getreg((31 << 11) | 20) & 15u);
+}
+
+// Merge workgroups of the fused form that gave up waiting for a flag (they
+// leave their rows untouched); read with nntile_hip_debug_decode_sync_timeouts.
+__device__ unsigned int decode_sync_timeouts;
+
+// Merge the split partials of row rr of a unit and fold the result into
+// (lse, A).  The calling thread handles head values d4 .. d4+3.  COH: the
+// partials were written by other workgroups of this launch.
+template<typename T, int HEAD, bool COH>
+__device__ __forceinline__ void decode_merge_row(const DecodeParams &p, int unit, int rr, int d4)
+{
+    static_assert(!COH || NNTILE_DEC_PART16, "the fused merge reads 16-bit partials");
+    const int nb = unit % p.n_batch;
+    const int hkv = unit / p.n_batch;
+    const int g = rr / (int)p.q_seq, tok = rr % (int)p.q_seq;
+    const int64_t qb = nb + (int64_t)p.n_batch * (g + (int64_t)p.kv_group * hkv);
+
+    const int64_t base = (int64_t)unit * p.n_splits * p.rows + rr;
+    const int last_split = p.n_splits - 1;
+    typedef __attribute__((ext_vector_type(2))) float f32x2;
+    // The loads of up to 8 splits are issued together (indices past the last
+    // split are clamped and get weight 0): the latency of the partials is
+    // paid once per 8 splits, not once per split; with at most 8 splits the
+    // maxima and the values travel in the same round trip.
+    const int64_t row = qb * p.q_seq + tok;
+    uint16_t *Adst = static_cast<uint16_t *>(p.A) + row * HEAD + d4;
+    float top = neg_inf();
+    float l = 0.0f;
+    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto load8 = [&](int s0, f32x2 (&ml)[8], f32x4 (&v)[8])
+    {
+#pragma unroll
+        for(int j = 0; j < 8; ++j)
+        {
+            const int sidx = min(s0 + j, last_split);
+            const int64_t prow = base + (int64_t)sidx * p.rows;
+            ml[j] = __builtin_bit_cast(f32x2, ld64<COH>(p.part_ml + 2 * prow));
+#if NNTILE_DEC_PART16
+            const u32x2 raw = __builtin_bit_cast(u32x2, ld64<COH>(
+                    reinterpret_cast<const uint16_t *>(p.part_o) + prow * HEAD + d4));
+            v[j] = f32x4{T::to_float((uint16_t)(raw[0] & 0xffffu)), T::to_float((uint16_t)(raw[0] >> 16)),
+                T::to_float((uint16_t)(raw[1] & 0xffffu)), T::to_float((uint16_t)(raw[1] >> 16))};
+#else
+            v[j] = *reinterpret_cast<const f32x4 *>(p.part_o + prow * HEAD + d4);
+#endif
+        }
+    };
+    auto add8 = [&](int s0, const f32x2 (&ml)[8], const f32x4 (&v)[8])
+    {
+#pragma unroll
+        for(int j = 0; j < 8; ++j)
+        {
+            const bool live = (s0 + j <= last_split) && (ml[j][0] != neg_inf());
+#if NNTILE_DEC_PART16
+            const float w = live ? __expf(ml[j][0] - top) * ml[j][1] : 0.0f;
+            l += w;
+#else
+            const float w = live ? __expf(ml[j][0] - top) : 0.0f;
+            l += w * ml[j][1];
+#endif
+            acc += w * v[j];
+        }
+    };
+    if(p.n_splits <= 8)
+    {
+        f32x2 ml[8];
+        f32x4 v[8];
+        load8(0, ml, v);
+#pragma unroll
+        for(int j = 0; j < 8; ++j)
+        {
+            top = fmaxf(top, ml[j][0]);
+        }
+        if(top != neg_inf())
+        {
+            add8(0, ml, v);
+        }
+    }
+    else
+    {
+        for(int s0 = 0; s0 < p.n_splits; s0 += 8)
+        {
+            float m[8];
+#pragma unroll
+            for(int j = 0; j < 8; ++j)
+            {
+                const int sidx = min(s0 + j, last_split);
+                m[j] = ld32f<COH>(p.part_ml + 2 * (base + (int64_t)sidx * p.rows));
+            }
+#pragma unroll
+            for(int j = 0; j < 8; ++j)
+            {
+                top = fmaxf(top, m[j]);
+            }
+        }
+        if(top != neg_inf())
+        {
+            for(int s0 = 0; s0 < p.n_splits; s0 += 8)
+            {
+                f32x2 ml[8];
+                f32x4 v[8];
+                load8(s0, ml, v);
+                add8(s0, ml, v);
+            }
+        }
+    }
+    if(top == neg_inf())
+    {
+        // no visible key at all: leave lse and A untouched, or write the
+        // empty row when the running pair is being overwritten
+        if(p.overwrite)
+        {
+            *reinterpret_cast<u32x2 *>(Adst) = u32x2{0, 0};
+            if(d4 == 0)
+            {
+                p.lse[row] = neg_inf();
+            }
+        }
+        return;
+    }
+    const float lse_new = top + __logf(l);
+    const float lse_old = p.overwrite ? neg_inf() : p.lse[row];
+    float w_old, w_new, lse_out;
+    merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
+    const float sc = w_new / l;
+    float v[4] = {acc[0] * sc, acc[1] * sc, acc[2] * sc, acc[3] * sc};
+    if(w_old != 0.0f)
+    {
+        const u32x2 old = *reinterpret_cast<const u32x2 *>(Adst);
+        v[0] += w_old * T::to_float((uint16_t)(old[0] & 0xffffu));
+        v[1] += w_old * T::to_float((uint16_t)(old[0] >> 16));
+        v[2] += w_old * T::to_float((uint16_t)(old[1] & 0xffffu));
+        v[3] += w_old * T::to_float((uint16_t)(old[1] >> 16));
+    }
+    u32x2 out;
+    out[0] = T::pack2(v[0], v[1]);
+    out[1] = T::pack2(v[2], v[3]);
+    *reinterpret_cast<u32x2 *>(Adst) = out;
+    // The threads of a row sit in one wavefront (TPR <= 32 divides 64) and
+    // run in lock step: all of them have read lse_old by now.
+    if(d4 == 0)
+    {
+        p.lse[row] = lse_out;
+    }
+}
+
+// A merge workgroup of the fused form: block `idx` behind the main workgroups.
+// It is dispatched when main workgroups have left (the hardware starts the
+// workgroups of a launch in index order, and the main ones never wait for
+// anything), waits until every split of its unit has raised its flag, merges
+// its rows and lowers the flags again.  Unit and merge workgroup sit on the
+// XCD of the unit's main workgroups, so flags and partials are exchanged
+// through that XCD's L2; should the hardware have placed either side
+// elsewhere (the XCC_ID register says), both fall back to device-scope fences.
+template<typename T, int HEAD>
+__device__ __forceinline__ void decode_merge_workgroup(const DecodeParams &p, int idx)
+{
+    constexpr int TPR = HEAD / 4;               // threads per row
+    constexpr int ROWS_PER_WG = 256 / TPR;
+    const int tid = threadIdx.x;
+    const int x = idx & 7, j = idx >> 3;
+    const int unit = (j / p.merge_blocks_per_unit) * 8 + x;
+    const int rb = j % p.merge_blocks_per_unit;
+    unsigned long long *flags = p.sync + (int64_t)unit * p.sync_stride + 1 + rb * p.n_splits;
+    int bad = 0;
+    if(tid < p.n_splits)
+    {
+        const unsigned long long t0 = wall_clock64();
+        while(ld64<true>(flags + tid) != p.tag)
+        {
+            __builtin_amdgcn_s_sleep(4);
+            if(wall_clock64() - t0 > p.spin_limit)
+            {
+                bad = 1;
+                break;
+            }
+        }
+    }
+    bad = __syncthreads_or(bad);
+    if(bad)
+    {
+        if(tid == 0)
+        {
+            atomicAdd(&decode_sync_timeouts, 1u);
+        }
+        return;
+    }
+    if(p.fenced || xcc_id() != x)
+    {
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
+    const int rr = rb * ROWS_PER_WG + tid / TPR;
+    if(rr < p.rows)
+    {
+        decode_merge_row<T, HEAD, true>(p, unit, rr, (tid % TPR) * 4);
+    }
+    // every partial of these rows has been read: the flags go down for the
+    // next call on this workspace (a replay of a captured graph has this
+    // call's tag again)
+    __syncthreads();
+    if(tid < p.n_splits)
+    {
+        __hip_atomic_store(flags + tid, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 // DIRECT: the unit has one key split, so the partial is the result and is
 // folded into (lse, A) here; no partials are written and no merge kernel runs.
 template<typename T, int HEAD, int MODE, int STAGES, bool DIRECT = false>
@@ -133,6 +371,19 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         else { return ring3; }
     };
 
+    if constexpr(!DIRECT)
+    {
+        if(p.fused && (int)blockIdx.x >= p.n_main)
+        {
+            DEC_STAMP(5);
+            decode_merge_workgroup<T, HEAD>(p, (int)blockIdx.x - p.n_main);
+#ifdef NNTILE_DEC_TRACE
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            DEC_STAMP(6);
+#endif
+            return;
+        }
+    }
     DEC_STAMP(0);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -582,12 +833,12 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
     DEC_STAMP(3);
     float l_tot = l_run + __shfl_xor(l_run, 16);
     l_tot = sum_across_halves(l_tot);
-    if(!row_ok)
-    {
-        return;
-    }
     if constexpr(DIRECT)
     {
+        if(!row_ok)
+        {
+            return;
+        }
         const int g = rr / (int)p.q_seq, tok = rr % (int)p.q_seq;
         const int64_t qb = nb + (int64_t)p.n_batch * (g + (int64_t)p.kv_group * hkv);
         const int64_t row = qb * p.q_seq + tok;
@@ -641,6 +892,8 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         }
         return;
     }
+    if(row_ok)
+    {
     const int64_t prow = ((int64_t)unit * p.n_splits + split) * p.rows + rr;
     if(quad == 0)
     {
@@ -673,10 +926,6 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         *reinterpret_cast<u32x2 *>(dst + 16 * db) = w;
 #endif
     }
-#ifdef NNTILE_DEC_TRACE
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    DEC_STAMP(4);
-#endif
 #else
     float *dst = p.part_o + prow * HEAD + 4 * quad;
 #pragma unroll
@@ -685,6 +934,27 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         *reinterpret_cast<acc4 *>(dst + 16 * db) = o[db];
     }
 #endif
+    }
+#ifdef NNTILE_DEC_TRACE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    DEC_STAMP(4);
+#endif
+    if(p.fused)
+    {
+        // The partial is complete in this XCD's L2 once every wavefront's
+        // stores have been acknowledged (the barrier's release waits for
+        // them); then one flag per merge workgroup of the unit goes up.
+        __syncthreads();
+        if(p.fenced || xcc_id() != (int)(blockIdx.x & 7))
+        {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        }
+        if(tid < p.merge_blocks_per_unit)
+        {
+            __hip_atomic_store(p.sync + (int64_t)unit * p.sync_stride + 1 + tid * p.n_splits + split,
+                    p.tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
 }
 
 // Merge the split partials of each row and fold the result into (lse, A).
@@ -719,141 +989,8 @@ void sdpa_decode_reduce_kernel(const DecodeParams p)
     {
         return;
     }
-    const int d4 = (threadIdx.x % TPR) * 4;
-    const int rr = (int)(grow % p.rows);
-    const int unit = (int)(grow / p.rows);
-    const int nb = unit % p.n_batch;
-    const int hkv = unit / p.n_batch;
-    const int g = rr / (int)p.q_seq, tok = rr % (int)p.q_seq;
-    const int64_t qb = nb + (int64_t)p.n_batch * (g + (int64_t)p.kv_group * hkv);
-
-    const int64_t base = (int64_t)unit * p.n_splits * p.rows + rr;
-    const int last_split = p.n_splits - 1;
-    typedef __attribute__((ext_vector_type(2))) float f32x2;
-    // The loads of up to 8 splits are issued together (indices past the last
-    // split are clamped and get weight 0): the latency of the partials is
-    // paid once per 8 splits, not once per split; with at most 8 splits the
-    // maxima and the values travel in the same round trip.
-    const int64_t row = qb * p.q_seq + tok;
-    uint16_t *Adst = static_cast<uint16_t *>(p.A) + row * HEAD + d4;
-    float top = neg_inf();
-    float l = 0.0f;
-    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-    auto load8 = [&](int s0, f32x2 (&ml)[8], f32x4 (&v)[8])
-    {
-#pragma unroll
-        for(int j = 0; j < 8; ++j)
-        {
-            const int sidx = min(s0 + j, last_split);
-            const int64_t prow = base + (int64_t)sidx * p.rows;
-            ml[j] = *reinterpret_cast<const f32x2 *>(p.part_ml + 2 * prow);
-#if NNTILE_DEC_PART16
-            const u32x2 raw = *reinterpret_cast<const u32x2 *>(
-                    reinterpret_cast<const uint16_t *>(p.part_o) + prow * HEAD + d4);
-            v[j] = f32x4{T::to_float((uint16_t)(raw[0] & 0xffffu)), T::to_float((uint16_t)(raw[0] >> 16)),
-                T::to_float((uint16_t)(raw[1] & 0xffffu)), T::to_float((uint16_t)(raw[1] >> 16))};
-#else
-            v[j] = *reinterpret_cast<const f32x4 *>(p.part_o + prow * HEAD + d4);
-#endif
-        }
-    };
-    auto add8 = [&](int s0, const f32x2 (&ml)[8], const f32x4 (&v)[8])
-    {
-#pragma unroll
-        for(int j = 0; j < 8; ++j)
-        {
-            const bool live = (s0 + j <= last_split) && (ml[j][0] != neg_inf());
-#if NNTILE_DEC_PART16
-            const float w = live ? __expf(ml[j][0] - top) * ml[j][1] : 0.0f;
-            l += w;
-#else
-            const float w = live ? __expf(ml[j][0] - top) : 0.0f;
-            l += w * ml[j][1];
-#endif
-            acc += w * v[j];
-        }
-    };
-    if(p.n_splits <= 8)
-    {
-        f32x2 ml[8];
-        f32x4 v[8];
-        load8(0, ml, v);
-#pragma unroll
-        for(int j = 0; j < 8; ++j)
-        {
-            top = fmaxf(top, ml[j][0]);
-        }
-        if(top != neg_inf())
-        {
-            add8(0, ml, v);
-        }
-    }
-    else
-    {
-        for(int s0 = 0; s0 < p.n_splits; s0 += 8)
-        {
-            float m[8];
-#pragma unroll
-            for(int j = 0; j < 8; ++j)
-            {
-                const int sidx = min(s0 + j, last_split);
-                m[j] = p.part_ml[2 * (base + (int64_t)sidx * p.rows)];
-            }
-#pragma unroll
-            for(int j = 0; j < 8; ++j)
-            {
-                top = fmaxf(top, m[j]);
-            }
-        }
-        if(top != neg_inf())
-        {
-            for(int s0 = 0; s0 < p.n_splits; s0 += 8)
-            {
-                f32x2 ml[8];
-                f32x4 v[8];
-                load8(s0, ml, v);
-                add8(s0, ml, v);
-            }
-        }
-    }
-    if(top == neg_inf())
-    {
-        // no visible key at all: leave lse and A untouched, or write the
-        // empty row when the running pair is being overwritten
-        if(p.overwrite)
-        {
-            *reinterpret_cast<u32x2 *>(Adst) = u32x2{0, 0};
-            if(d4 == 0)
-            {
-                p.lse[row] = neg_inf();
-            }
-        }
-        return;
-    }
-    const float lse_new = top + __logf(l);
-    const float lse_old = p.overwrite ? neg_inf() : p.lse[row];
-    float w_old, w_new, lse_out;
-    merge_weights(lse_old, lse_new, w_old, w_new, lse_out);
-    const float sc = w_new / l;
-    float v[4] = {acc[0] * sc, acc[1] * sc, acc[2] * sc, acc[3] * sc};
-    if(w_old != 0.0f)
-    {
-        const u32x2 old = *reinterpret_cast<const u32x2 *>(Adst);
-        v[0] += w_old * T::to_float((uint16_t)(old[0] & 0xffffu));
-        v[1] += w_old * T::to_float((uint16_t)(old[0] >> 16));
-        v[2] += w_old * T::to_float((uint16_t)(old[1] & 0xffffu));
-        v[3] += w_old * T::to_float((uint16_t)(old[1] >> 16));
-    }
-    u32x2 out;
-    out[0] = T::pack2(v[0], v[1]);
-    out[1] = T::pack2(v[2], v[3]);
-    *reinterpret_cast<u32x2 *>(Adst) = out;
-    // The threads of a row sit in one wavefront (TPR <= 32 divides 64) and
-    // run in lock step: all of them have read lse_old by now.
-    if(d4 == 0)
-    {
-        p.lse[row] = lse_out;
-    }
+    decode_merge_row<T, HEAD, false>(p, (int)(grow / p.rows), (int)(grow % p.rows),
+            (threadIdx.x % TPR) * 4);
 #ifdef NNTILE_DEC_TRACE
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     DEC_STAMP(6);
@@ -866,6 +1003,49 @@ extern "C" int nntile_hip_debug_dec_trace(unsigned long long *host)
     return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(dec_trace), sizeof(dec_trace));
 }
 #endif
+
+// 64-bit words of the sync area per unit (fused merge): one reserved word and
+// a flag per (merge workgroup of the unit, split), rounded to 64 bytes.
+int decode_sync_stride(int n_splits, int rows, int head)
+{
+    const int rows_per_wg = 256 / (head / 4);
+    const int merge_blocks = (rows + rows_per_wg - 1) / rows_per_wg;
+    return (1 + merge_blocks * n_splits + 7) / 8 * 8;
+}
+
+// A value no earlier call of this process has used and that memory left
+// behind by anything else is unlikely to hold: a random upper half fixed at
+// load time, a counter below it.
+static unsigned long long next_decode_tag()
+{
+    static const unsigned long long salt = []
+    {
+        std::random_device rd;
+        return ((unsigned long long)rd() << 32) | 0x80000000ull;
+    }();
+    static std::atomic<unsigned long long> counter{0};
+    unsigned long long tag = salt + counter.fetch_add(1, std::memory_order_relaxed) + 1ull;
+    return tag == 0ull ? 1ull : tag;
+}
+
+// Longest wait of a merge workgroup for a flag, in ticks of the 100 MHz clock
+// (2 s unless a test sets it).
+static std::atomic<unsigned long long> decode_spin_limit{200000000ull};
+
+extern "C" unsigned long long nntile_hip_debug_decode_spin_limit(unsigned long long ticks)
+{
+    return decode_spin_limit.exchange(ticks);
+}
+
+extern "C" long long nntile_hip_debug_decode_sync_timeouts(void)
+{
+    unsigned int n = 0;
+    if(hipMemcpyFromSymbol(&n, HIP_SYMBOL(decode_sync_timeouts), sizeof(n)) != hipSuccess)
+    {
+        return -1;
+    }
+    return (long long)n;
+}
 
 template<typename T, int HEAD, int MODE, int STAGES>
 static void launch_decode_main(hipStream_t stream, const DecodeParams &p, dim3 grid)
@@ -881,10 +1061,24 @@ static void launch_decode_main(hipStream_t stream, const DecodeParams &p, dim3 g
 }
 
 template<typename T, int HEAD, int STAGES>
-static int launch_decode_stages(hipStream_t stream, const DecodeParams &p, int mode)
+static int launch_decode_stages(hipStream_t stream, DecodeParams &p, int mode)
 {
     const int units = p.n_batch * p.n_head_kv;
-    const dim3 grid((unsigned)(units * p.n_splits));
+    constexpr int rows_per_wg = 256 / (HEAD / 4);
+    const int merge_blocks = (p.rows + rows_per_wg - 1) / rows_per_wg;
+    // The merge rides in the main launch when the caller allows it, the unit
+    // has several splits and the units map onto the XCDs (8 at a time).
+    p.fused = (p.fused && p.n_splits > 1 && units % 8 == 0 && p.sync != nullptr
+            && NNTILE_DEC_PART16) ? 1 : 0;
+    p.n_main = units * p.n_splits;
+    p.merge_blocks_per_unit = merge_blocks;
+    p.sync_stride = decode_sync_stride(p.n_splits, p.rows, HEAD);
+    if(p.fused)
+    {
+        p.tag = next_decode_tag();
+        p.spin_limit = decode_spin_limit.load(std::memory_order_relaxed);
+    }
+    const dim3 grid((unsigned)(p.n_main + (p.fused ? units * merge_blocks : 0)));
     switch(mode)
     {
         case NNTILE_HIP_MASK_ADDITIVE:
@@ -906,9 +1100,8 @@ static int launch_decode_stages(hipStream_t stream, const DecodeParams &p, int m
     {
         return NNTILE_HIP_ELAUNCH;
     }
-    if(p.n_splits > 1)
+    if(p.n_splits > 1 && !p.fused)
     {
-        constexpr int rows_per_wg = 256 / (HEAD / 4);
         const int64_t total_rows = (int64_t)units * p.rows;
         hipLaunchKernelGGL((sdpa_decode_reduce_kernel<T, HEAD>),
                 dim3((unsigned)((total_rows + rows_per_wg - 1) / rows_per_wg)),
@@ -920,7 +1113,7 @@ static int launch_decode_stages(hipStream_t stream, const DecodeParams &p, int m
 // Ring depth 2 (64 KB of LDS at head 128) lets two workgroups share a CU, which
 // measured faster than one workgroup with a deeper ring.
 template<typename T, int HEAD>
-static int launch_decode_head(hipStream_t stream, const DecodeParams &p, int mode)
+static int launch_decode_head(hipStream_t stream, DecodeParams &p, int mode)
 {
     return launch_decode_stages<T, HEAD, NNTILE_DEC_STAGES>(stream, p, mode);
 }
@@ -944,10 +1137,16 @@ size_t decode_partial_o_bytes(int units, int n_splits, int rows, int head)
     return (size_t)units * n_splits * rows * head * (NNTILE_DEC_PART16 ? 2 : sizeof(float));
 }
 
+size_t decode_partial_ml_bytes(int units, int n_splits, int rows)
+{
+    return (size_t)units * n_splits * rows * 2 * sizeof(float);
+}
+
 size_t decode_workspace_bytes(int units, int n_splits, int rows, int head)
 {
     return decode_partial_o_bytes(units, n_splits, rows, head)
-        + (size_t)units * n_splits * rows * 2 * sizeof(float);
+        + decode_partial_ml_bytes(units, n_splits, rows)
+        + (size_t)units * decode_sync_stride(n_splits, rows, head) * sizeof(unsigned long long);
 }
 
 template<typename T>

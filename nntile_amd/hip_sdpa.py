@@ -21,6 +21,9 @@ MAX_TILES = 64
 BWD_MAX_TILES = 32
 OVERWRITE = 1
 FORM_SHARED, FORM_SPLIT = 0x100, 0x200     # fp32 calls: fix the workgroup shape (tests, tuning)
+# decode calls (tests, tuning): merge the key splits in a second launch; exchange
+# the partials of the in-launch merge through device-scope fences
+DECODE_SEPARATE_MERGE, DECODE_FENCED = 0x400, 0x800
 
 OK, EINVAL, EUNSUPPORTED, ELAUNCH, EWORKSPACE = 0, -1, -2, -3, -4
 TILE_MIXED, TILE_OPEN, TILE_HIDDEN, TILE_CAUSAL = 0, 1, 2, 3
@@ -483,6 +486,22 @@ def plan_decode(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group, workspace, 
     nbytes = workspace.numel() * workspace.element_size()
     return Plan(fn, a, "sdpa_fwd_decode", extra=(_ptr(workspace), nbytes),
                 keep=(K, Q, mask, lse, V, A, workspace))
+
+
+def decode_sync_timeouts():
+    """Merge workgroups of in-launch decode merges that gave up waiting for a
+    split since the library was loaded (diagnostic; blocks)."""
+    f = lib().nntile_hip_debug_decode_sync_timeouts
+    f.restype = ctypes.c_longlong
+    return int(f())
+
+
+def decode_spin_limit(ticks):
+    """Sets the longest wait of a merge workgroup for a split, in ticks of the
+    100 MHz clock; returns the previous value (diagnostic)."""
+    f = lib().nntile_hip_debug_decode_spin_limit
+    f.argtypes, f.restype = [ctypes.c_ulonglong], ctypes.c_ulonglong
+    return int(f(ticks))
 
 
 def decode_workspace_bytes(K, Q, n_batch, kv_group):
