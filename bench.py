@@ -398,10 +398,11 @@ def bench_reference_api(cfg, steps, warmup):
     return out
 
 
-def bench_decode(cfg, steps, warmup):
-    """The GQA decode shape: main kernel + merge of the key splits per step.
-    Four (K, V) sets rotate (4 x 256 MiB at cfg4: the 256 MiB last-level cache
-    cannot serve a pass)."""
+def bench_decode(cfg, steps, warmup, more_flags=0):
+    """The GQA decode shape: one launch per step (the key splits of a unit
+    are merged inside it).  Four (K, V) sets rotate (4 x 256 MiB at cfg4: the
+    256 MiB last-level cache cannot serve a pass).  more_flags: further flags
+    of the decode call (the merge as a second launch)."""
     import torch
     from nntile_amd import hip_sdpa as h
     kvb = cfg.n_batch * cfg.n_head_kv
@@ -414,7 +415,7 @@ def bench_decode(cfg, steps, warmup):
     ws = torch.empty(h.decode_workspace_bytes(Ks[0], Q, cfg.n_batch, cfg.kv_group),
                      dtype=torch.uint8, device="cuda")
     plans = [h.plan_decode(Ks[j], Q, None, lse, Vs[j], A, h.MASK_CAUSAL, cfg.n_batch, cfg.kv_group,
-                           ws, causal_offset=cfg.causal_offset, flags=h.OVERWRITE)
+                           ws, causal_offset=cfg.causal_offset, flags=h.OVERWRITE | more_flags)
              for j in range(nrot)]
     i = [0]
 
@@ -790,7 +791,7 @@ def main():
                     help="with --only power_context: a shared library exporting nntile_hip_probe_mfma "
                          "(the matrix instruction alone); not part of the product")
     ap.add_argument("--only", default=None,
-                    help="run only this leg (for profiling): prefill | cfg5 | cfg2 | decode | decode_wide | "
+                    help="run only this leg (for profiling): prefill | cfg5 | cfg2 | decode | decode_separate_merge | decode_wide | "
                          "reference_api | reference_grid | power_context | copy_context | backward | backward_slabs | rope | transpose | accumulate | "
                          "kv_cache | copy")
     args = ap.parse_args()
@@ -821,6 +822,8 @@ def main():
             "cfg2_per_slab": lambda: bench_prefill(BY_NAME["cfg2_gpt2_small_fp32"], args.steps,
                                                    args.warmup, one_launch=False),
             "decode": lambda: bench_decode(cfg4, args.steps, args.warmup),
+            "decode_separate_merge": lambda: bench_decode(cfg4, args.steps, args.warmup,
+                                                          h.DECODE_SEPARATE_MERGE),
             "decode_wide": lambda: bench_decode(cfg4_wide, args.steps, args.warmup),
             "reference_api": lambda: bench_reference_api(cfg3, args.steps, args.warmup),
             "reference_grid": lambda: bench_reference_grid(args.steps, args.warmup, args.case),

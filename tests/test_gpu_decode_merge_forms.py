@@ -93,6 +93,29 @@ def test_workspace_contents_do_not_matter_and_calls_repeat(oracle, fill):
     assert H.rel_fro(H.to_np(lse), want_lse2) < H.TOL[dtype]
 
 
+def test_other_inputs_on_the_same_workspace(oracle):
+    """Calls with different inputs take turns on one workspace: every call
+    must merge the partials written by this call, not what an earlier call
+    left at the same addresses."""
+    dtype, q_seq, k_seq, n_batch, group, n_kv, head = "bf16", 16, 1536, 4, 4, 2, 128
+    cases = [_case(oracle, dtype, q_seq, k_seq, n_batch, group, n_kv, head, "causal", seed=40 + i)
+             for i in range(3)]
+    ws = torch.empty(hip_sdpa.decode_workspace_bytes(cases[0][0][0], cases[0][0][1], n_batch, group),
+                     dtype=torch.uint8, device="cuda")
+    outs = [H.fresh_outputs(cases[0][0][1].shape[0], q_seq, head, dtype) for _ in range(9)]
+    # enqueued back to back, checked afterwards
+    for rep, out in enumerate(outs):
+        (Kd, Qd, Vd), (m, mm, offset), _ = cases[rep % 3]
+        hip_sdpa.sdpa_fwd_decode(Kd, Qd, m, out[0], Vd, out[1], mm, n_batch, group, ws,
+                                 causal_offset=offset)
+    torch.cuda.synchronize()
+    for rep, (lse, A) in enumerate(outs):
+        want, want_lse = cases[rep % 3][2]
+        assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype], rep
+        assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype], rep
+        H.check_rows(H.to_np(A), want, H.to_np(lse), want_lse, dtype, "rep %d" % rep)
+
+
 def test_merge_inside_the_launch_into_running_pair(oracle):
     """Two calls over two halves of the cache == one call over all of it."""
     dtype, q_seq, k_seq, n_batch, group, n_kv, head = "bf16", 16, 1024, 4, 4, 2, 128

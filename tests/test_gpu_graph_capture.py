@@ -26,8 +26,13 @@ def _replays(graph, check, disturb):
         check()
 
 
-def test_decode_step_through_the_cache_in_a_graph():
-    n_batch, n_kv, group, head, cap, old, new = 2, 2, 4, 128, 1024, 600, 16
+@pytest.mark.parametrize("n_batch", [2, 4])
+def test_decode_step_through_the_cache_in_a_graph(n_batch):
+    """n_batch 2: 4 units, the merge of the key splits is a launch of its own.
+    n_batch 4: 8 units, the merge rides in the main launch and its flags live
+    in the workspace - a replay carries the captured call's tag again and
+    finds them as the previous replay (or `disturb`) left them."""
+    n_kv, group, head, cap, old, new = 2, 4, 128, 1024, 600, 16
     kvb, batch = n_batch * n_kv, n_batch * n_kv * group
     dt = torch.bfloat16
     Kc, Vc = _randn((kvb, cap, head), dt, 1), _randn((kvb, cap, head), dt, 2)

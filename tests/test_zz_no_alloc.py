@@ -58,6 +58,13 @@ def test_static_scratch_decode_head64_and_merge(oracle):
     _both(oracle, "bf16", 1, 300, 3, 4, 2, 64, 55, False)
 
 
+def test_static_scratch_decode_with_the_merge_inside_the_launch(oracle):
+    # 8 units: the merge rides in the main launch and its flags live in the
+    # array as well; then a smaller input
+    _both(oracle, "bf16", 16, 2048, 4, 4, 2, 128, 56, False)
+    _both(oracle, "bf16", 3, 900, 8, 2, 1, 128, 57, True)
+
+
 def test_static_scratch_refuses_what_does_not_fit():
     # 64 rows x 4096 units x 1 split of bf16 partials alone are 64 MiB
     n_batch, group, n_kv, head, q_seq, k_seq = 1024, 4, 4, 128, 16, 8192
