@@ -316,6 +316,17 @@ int nntile_hip_sdpa_fwd_decode_fp16(void *stream, const nntile_hip_sdpa_tile_arg
 int nntile_hip_sdpa_fwd_decode_static(void *stream, int32_t dtype,
         const nntile_hip_sdpa_tile_args *args);
 
+/* ---- 4c. diagnostics of the decode entry points ------------------------------
+ * No counterpart in the reference.  When a (batch entry, kv head) unit has
+ * several key splits and the units come in multiples of 8, the merge of the
+ * splits runs inside the main launch: merge workgroups behind the main ones
+ * wait for flags in the workspace.  That wait is bounded (2 s of the 100 MHz
+ * device clock unless set otherwise here; returns the previous bound); a merge
+ * workgroup that gives up leaves its rows untouched and is counted.  The
+ * count since the library was loaded (blocking; -1 on error): */
+unsigned long long nntile_hip_debug_decode_spin_limit(unsigned long long ticks);
+long long nntile_hip_debug_decode_sync_timeouts(void);
+
 /* ---- 5. the running-statistics hand-off on its own ---------------------------
  * Replaces kernel::accumulate_attn_output::cuda<T>
  * (src/kernel/accumulate_attn_output/cuda.cu:115-135; CPU statement
@@ -371,6 +382,42 @@ void nntile_hip_flash_sdpa_fwd_codelet_fp32(void *buffers[], void *cl_args);
  * (include/nntile/starpu/flash_sdpa_bwd_cudnn.hh:48-57). */
 void nntile_hip_flash_sdpa_bwd_codelet_bf16(void *buffers[], void *cl_args);
 void nntile_hip_flash_sdpa_bwd_codelet_fp16(void *buffers[], void *cl_args);
+
+/* ---- 6b. StarPU codelet bodies of the whole-grid calls ---------------------------
+ * The fused launches as tasks: what tensor::flash_sdpa_fwd_cudnn_async
+ * (src/tensor/flash_sdpa_fwd_cudnn.cc:246-274) submits as one task per (output
+ * tile, key tile) pair becomes ONE task per group of slabs, submitted like the
+ * reference's (src/starpu/flash_sdpa_fwd_cudnn.cc:181-210: starpu_task_insert
+ * on a codelet with nbuffers = STARPU_VARIABLE_NBUFFERS, src/starpu/codelet.cc:
+ * 58, so the number of handles is free).  buffers[] point at StarPU variable
+ * interfaces, tile after tile, in this order and with these access modes
+ * (nK = n_slabs*n_kv_tiles, nQ = n_slabs*n_q_tiles, slab s's tiles at
+ * [s*n_kv_tiles + t] / [s*n_q_tiles + t] as in nntile_hip_sdpa_grid_args):
+ *   forward : K[nK](R) V[nK](R) Q[nQ](R) lse[nQ](RW) A[nQ](RW)
+ *             (with NNTILE_HIP_SDPA_OVERWRITE in flags lse and A may be W)
+ *   backward: K[nK](R) V[nK](R) Q[nQ](R) A[nQ](R) dA[nQ](R) lse[nQ](R)
+ *             dK[nK](RW) dQ[nQ](RW) dV[nK](RW) workspace(SCRATCH, at least
+ *             nntile_hip_sdpa_bwd_grid_workspace_bytes)
+ * cl_args points at nntile_hip_sdpa_grid_cl_args: the reference's args_t
+ * members first (seq = rows of a full query tile, head, batch = entries of one
+ * slab), then the geometry of nntile_hip_sdpa_grid_args.  Same error
+ * behaviour as the per-pair bodies: a line on stderr, the task does nothing. */
+typedef struct nntile_hip_sdpa_grid_cl_args
+{
+    void *owner;
+    int64_t seq, head, batch;           /* args_t of the reference */
+    int64_t q_seq, k_seq, q_tile, k_tile;
+    int64_t n_batch, kv_group;
+    int64_t q_pos0, k_pos0, causal_offset;
+    int32_t mask_mode, flags;
+    int32_t n_q_tiles, n_kv_tiles, n_slabs, reserved;
+} nntile_hip_sdpa_grid_cl_args;
+
+void nntile_hip_sdpa_fwd_grid_codelet_bf16(void *buffers[], void *cl_args);
+void nntile_hip_sdpa_fwd_grid_codelet_fp16(void *buffers[], void *cl_args);
+void nntile_hip_sdpa_fwd_grid_codelet_fp32(void *buffers[], void *cl_args);
+void nntile_hip_sdpa_bwd_grid_codelet_bf16(void *buffers[], void *cl_args);
+void nntile_hip_sdpa_bwd_grid_codelet_fp16(void *buffers[], void *cl_args);
 
 /* ---- 7. The step before the attention kernel: rotary position embedding ----
  * Replace kernel::rope::cuda<T> (include/nntile/kernel/rope/cuda.hh:24-27,

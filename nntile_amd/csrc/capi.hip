@@ -823,6 +823,139 @@ static void bwd_codelet_call(DType dt, const char *name, void *buffers[],
     }
 }
 
+// Geometry of a grid call out of the codelet arguments; false (after a line on
+// stderr) when the task cannot be run.
+static bool grid_codelet_geometry(const char *name, void *buffers[], void *cl_args,
+        int max_tiles, const nntile_hip_sdpa_grid_cl_args *&args, int &n_k, int &n_q)
+{
+    if(buffers == nullptr || cl_args == nullptr)
+    {
+        std::fprintf(stderr, "HIP Worker: %s: null buffers or arguments, "
+                "skipping task\n", name);
+        return false;
+    }
+    args = static_cast<const nntile_hip_sdpa_grid_cl_args *>(cl_args);
+    const int n_slabs = args->n_slabs > 0 ? args->n_slabs : 1;
+    if(args->n_q_tiles <= 0 || args->n_kv_tiles <= 0
+            || (int64_t)n_slabs * args->n_q_tiles > max_tiles
+            || (int64_t)n_slabs * args->n_kv_tiles > max_tiles)
+    {
+        std::fprintf(stderr, "HIP Worker: %s: %d slabs of %d x %d tiles do not fit one "
+                "call, skipping task\n", name, n_slabs, args->n_q_tiles, args->n_kv_tiles);
+        return false;
+    }
+    n_k = n_slabs * args->n_kv_tiles;
+    n_q = n_slabs * args->n_q_tiles;
+    return true;
+}
+
+template<typename A>
+static void grid_codelet_fill(A &a, const nntile_hip_sdpa_grid_cl_args *args)
+{
+    std::memset(&a, 0, sizeof(a));
+    a.q_seq = args->q_seq;
+    a.k_seq = args->k_seq;
+    a.q_tile = args->q_tile;
+    a.k_tile = args->k_tile;
+    a.head = args->head;
+    a.batch = args->batch;
+    a.n_batch = args->n_batch;
+    a.kv_group = args->kv_group;
+    a.mask_mode = args->mask_mode;
+    a.n_q_tiles = args->n_q_tiles;
+    a.n_kv_tiles = args->n_kv_tiles;
+    a.flags = args->flags;
+    a.n_slabs = args->n_slabs;
+    a.q_pos0 = args->q_pos0;
+    a.k_pos0 = args->k_pos0;
+    a.causal_offset = args->causal_offset;
+}
+
+static void fwd_grid_codelet_call(DType dt, const char *name, void *buffers[], void *cl_args)
+{
+    const nntile_hip_sdpa_grid_cl_args *args = nullptr;
+    int n_k = 0, n_q = 0;
+    if(!grid_codelet_geometry(name, buffers, cl_args, NNTILE_HIP_SDPA_MAX_TILES, args, n_k, n_q))
+    {
+        return;
+    }
+    auto **ifs = reinterpret_cast<nntile_hip_variable_interface **>(buffers);
+    const int n_buffers = 2 * n_k + 3 * n_q;
+    for(int i = 0; i < n_buffers; ++i)
+    {
+        if(ifs[i] == nullptr)
+        {
+            std::fprintf(stderr, "HIP Worker: %s: buffer %d is null, skipping task\n", name, i);
+            return;
+        }
+    }
+    nntile_hip_sdpa_grid_args a;
+    grid_codelet_fill(a, args);
+    for(int t = 0; t < n_k; ++t)
+    {
+        a.K[t] = reinterpret_cast<const void *>(ifs[t]->ptr);
+        a.V[t] = reinterpret_cast<const void *>(ifs[n_k + t]->ptr);
+    }
+    for(int t = 0; t < n_q; ++t)
+    {
+        a.Q[t] = reinterpret_cast<const void *>(ifs[2 * n_k + t]->ptr);
+        a.lse[t] = reinterpret_cast<float *>(ifs[2 * n_k + n_q + t]->ptr);
+        a.A[t] = reinterpret_cast<void *>(ifs[2 * n_k + 2 * n_q + t]->ptr);
+    }
+    void *stream = g_stream_provider ? g_stream_provider() : nullptr;
+    const int rc = grid_call(dt, stream, &a);
+    if(rc != NNTILE_HIP_OK)
+    {
+        std::fprintf(stderr, "HIP Worker: %s: launch failed with code %d (q_seq=%lld k_seq=%lld "
+                "head=%lld batch=%lld), skipping task\n", name, rc, (long long)args->q_seq,
+                (long long)args->k_seq, (long long)args->head, (long long)args->batch);
+    }
+}
+
+static void bwd_grid_codelet_call(DType dt, const char *name, void *buffers[], void *cl_args)
+{
+    const nntile_hip_sdpa_grid_cl_args *args = nullptr;
+    int n_k = 0, n_q = 0;
+    if(!grid_codelet_geometry(name, buffers, cl_args, NNTILE_HIP_SDPA_BWD_MAX_TILES, args, n_k,
+                n_q))
+    {
+        return;
+    }
+    auto **ifs = reinterpret_cast<nntile_hip_variable_interface **>(buffers);
+    const int n_buffers = 4 * n_k + 5 * n_q + 1;
+    for(int i = 0; i < n_buffers; ++i)
+    {
+        if(ifs[i] == nullptr)
+        {
+            std::fprintf(stderr, "HIP Worker: %s: buffer %d is null, skipping task\n", name, i);
+            return;
+        }
+    }
+    nntile_hip_sdpa_bwd_grid_args a;
+    grid_codelet_fill(a, args);
+    int at = 0;
+    auto take = [&]() { return reinterpret_cast<void *>(ifs[at++]->ptr); };
+    for(int t = 0; t < n_k; ++t) { a.K[t] = take(); }
+    for(int t = 0; t < n_k; ++t) { a.V[t] = take(); }
+    for(int t = 0; t < n_q; ++t) { a.Q[t] = take(); }
+    for(int t = 0; t < n_q; ++t) { a.A[t] = take(); }
+    for(int t = 0; t < n_q; ++t) { a.dA[t] = take(); }
+    for(int t = 0; t < n_q; ++t) { a.lse[t] = static_cast<const float *>(take()); }
+    for(int t = 0; t < n_k; ++t) { a.dK[t] = take(); }
+    for(int t = 0; t < n_q; ++t) { a.dQ[t] = take(); }
+    for(int t = 0; t < n_k; ++t) { a.dV[t] = take(); }
+    a.workspace_bytes = ifs[at]->elemsize;
+    a.workspace = take();
+    void *stream = g_stream_provider ? g_stream_provider() : nullptr;
+    const int rc = bwd_grid_call(dt, stream, &a);
+    if(rc != NNTILE_HIP_OK)
+    {
+        std::fprintf(stderr, "HIP Worker: %s: launch failed with code %d (q_seq=%lld k_seq=%lld "
+                "head=%lld batch=%lld), skipping task\n", name, rc, (long long)args->q_seq,
+                (long long)args->k_seq, (long long)args->head, (long long)args->batch);
+    }
+}
+
 } // namespace nntile_hip
 
 using namespace nntile_hip;
@@ -1024,6 +1157,31 @@ int nntile_hip_flash_sdpa_bwd_fp16(void *stream, int64_t seq, int64_t head,
 {
     return flash_bwd_call(DType::fp16, stream, seq, head, batch, K, Q, V, A, dA, mask,
             lse, scratch_dQ, dK, dQ, dV);
+}
+
+void nntile_hip_sdpa_fwd_grid_codelet_bf16(void *buffers[], void *cl_args)
+{
+    fwd_grid_codelet_call(DType::bf16, "nntile_sdpa_fwd_grid_hip_bf16", buffers, cl_args);
+}
+
+void nntile_hip_sdpa_fwd_grid_codelet_fp16(void *buffers[], void *cl_args)
+{
+    fwd_grid_codelet_call(DType::fp16, "nntile_sdpa_fwd_grid_hip_fp16", buffers, cl_args);
+}
+
+void nntile_hip_sdpa_fwd_grid_codelet_fp32(void *buffers[], void *cl_args)
+{
+    fwd_grid_codelet_call(DType::fp32, "nntile_sdpa_fwd_grid_hip_fp32", buffers, cl_args);
+}
+
+void nntile_hip_sdpa_bwd_grid_codelet_bf16(void *buffers[], void *cl_args)
+{
+    bwd_grid_codelet_call(DType::bf16, "nntile_sdpa_bwd_grid_hip_bf16", buffers, cl_args);
+}
+
+void nntile_hip_sdpa_bwd_grid_codelet_fp16(void *buffers[], void *cl_args)
+{
+    bwd_grid_codelet_call(DType::fp16, "nntile_sdpa_bwd_grid_hip_fp16", buffers, cl_args);
 }
 
 void nntile_hip_flash_sdpa_bwd_codelet_bf16(void *buffers[], void *cl_args)

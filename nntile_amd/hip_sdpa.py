@@ -93,6 +93,18 @@ class FlashClArgs(ctypes.Structure):
     _fields_ = [("owner", _vp), ("seq", _i64), ("head", _i64), ("batch", _i64)]
 
 
+class GridClArgs(ctypes.Structure):
+    """nntile_hip_sdpa_grid_cl_args: the reference's args_t members, then the
+    geometry of the tile grid."""
+    _fields_ = [("owner", _vp), ("seq", _i64), ("head", _i64), ("batch", _i64),
+                ("q_seq", _i64), ("k_seq", _i64), ("q_tile", _i64), ("k_tile", _i64),
+                ("n_batch", _i64), ("kv_group", _i64),
+                ("q_pos0", _i64), ("k_pos0", _i64), ("causal_offset", _i64),
+                ("mask_mode", ctypes.c_int32), ("flags", ctypes.c_int32),
+                ("n_q_tiles", ctypes.c_int32), ("n_kv_tiles", ctypes.c_int32),
+                ("n_slabs", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+
+
 STREAM_PROVIDER = ctypes.CFUNCTYPE(_vp)
 
 EXPORTS = (
@@ -116,6 +128,9 @@ EXPORTS = (
     + ["nntile_hip_sdpa_fwd_decode_cache_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_sdpa_fwd_tile_cache_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_mask_tile_class_" + t for t in ("bf16", "fp16", "fp32", "bool")]
+    + ["nntile_hip_sdpa_fwd_grid_codelet_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_sdpa_bwd_grid_codelet_" + t for t in ("bf16", "fp16")]
+    + ["nntile_hip_debug_decode_spin_limit", "nntile_hip_debug_decode_sync_timeouts"]
     + ["nntile_hip_set_stream_provider", "nntile_hip_sdpa_version"])
 
 _lib = None
@@ -701,6 +716,72 @@ def flash_sdpa_fwd_codelet(K, Q, mask, lse, V, A, scratch_lse=None, scratch_A=No
                        b if batch is None else batch)
     fn = getattr(lib(), "nntile_hip_flash_sdpa_fwd_codelet_" + dtype_name(Q))
     fn(bufs, ctypes.addressof(args))
+
+
+def _interfaces(tensors):
+    """Look-alike StarPU variable interfaces of device tensors and the
+    buffers[] array that points at them (keep both alive during the call)."""
+    ifs = []
+    for t in tensors:
+        v = VariableInterface()
+        v.id = 2
+        v.ptr = 0 if t is None else t.data_ptr()
+        v.dev_handle = v.ptr
+        v.offset = 0
+        v.elemsize = 0 if t is None else t.numel() * t.element_size()
+        ifs.append(v)
+    return ifs, (_vp * len(ifs))(*[ctypes.addressof(v) for v in ifs])
+
+
+def _grid_cl_args(Q_tiles, K_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, n_batch, kv_group,
+                  q_pos0, k_pos0, causal_offset, flags, n_slabs):
+    batch, _, head = Q_tiles[0].shape
+    a = GridClArgs()
+    a.owner = None
+    a.seq, a.head, a.batch = q_tile, head, batch
+    a.q_seq, a.k_seq, a.q_tile, a.k_tile = q_seq, k_seq, q_tile, k_tile
+    a.n_batch = batch if n_batch is None else n_batch
+    a.kv_group = kv_group
+    a.q_pos0, a.k_pos0, a.causal_offset = q_pos0, k_pos0, causal_offset
+    a.mask_mode, a.flags = mask_mode, flags
+    a.n_slabs = n_slabs
+    a.n_q_tiles, a.n_kv_tiles = len(Q_tiles) // n_slabs, len(K_tiles) // n_slabs
+    return a
+
+
+def sdpa_fwd_grid_codelet(K_tiles, Q_tiles, lse_tiles, V_tiles, A_tiles, q_seq, k_seq, q_tile,
+                          k_tile, mask_mode, n_batch=None, kv_group=1, q_pos0=0, k_pos0=0,
+                          causal_offset=0, flags=0, n_slabs=1, n_q_tiles=None):
+    """Calls the StarPU-shaped body of the whole-grid forward as a HIP worker
+    would: buffers K tiles, V tiles, Q tiles, lse tiles, A tiles (null stream
+    unless a provider was registered).  n_q_tiles overrides the tile count in
+    the arguments (to provoke the body's error path)."""
+    _dev(*K_tiles, *Q_tiles, *lse_tiles, *V_tiles, *A_tiles)
+    a = _grid_cl_args(Q_tiles, K_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, n_batch, kv_group,
+                      q_pos0, k_pos0, causal_offset, flags, n_slabs)
+    if n_q_tiles is not None:
+        a.n_q_tiles = n_q_tiles
+    ifs, bufs = _interfaces(list(K_tiles) + list(V_tiles) + list(Q_tiles) + list(lse_tiles)
+                            + list(A_tiles))
+    fn = getattr(lib(), "nntile_hip_sdpa_fwd_grid_codelet_" + dtype_name(Q_tiles[0]))
+    fn.argtypes, fn.restype = [_vp, _vp], None
+    fn(bufs, ctypes.addressof(a))
+
+
+def sdpa_bwd_grid_codelet(K_tiles, Q_tiles, V_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles,
+                          dQ_tiles, dV_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, workspace,
+                          n_batch=None, kv_group=1, q_pos0=0, k_pos0=0, causal_offset=0, flags=0,
+                          n_slabs=1):
+    """The body of the whole-grid backward: buffers K, V, Q, A, dA, lse tiles
+    (read), dK, dQ, dV tiles (read-write), one scratch buffer."""
+    groups = [K_tiles, V_tiles, Q_tiles, A_tiles, dA_tiles, lse_tiles, dK_tiles, dQ_tiles, dV_tiles]
+    _dev(*[t for g in groups for t in g], workspace)
+    a = _grid_cl_args(Q_tiles, K_tiles, q_seq, k_seq, q_tile, k_tile, mask_mode, n_batch, kv_group,
+                      q_pos0, k_pos0, causal_offset, flags, n_slabs)
+    ifs, bufs = _interfaces([t for g in groups for t in g] + [workspace])
+    fn = getattr(lib(), "nntile_hip_sdpa_bwd_grid_codelet_" + dtype_name(Q_tiles[0]))
+    fn.argtypes, fn.restype = [_vp, _vp], None
+    fn(bufs, ctypes.addressof(a))
 
 
 def flash_sdpa_bwd_codelet(K, Q, V, A, dA, mask, lse, dK, dQ, dV, scratch_dK=None,

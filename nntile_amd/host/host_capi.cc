@@ -409,6 +409,33 @@ int64_t nntile_host_tasks_submitted(int dtype)
     return starpu::flash_sdpa_fwd_cudnn<fp32_t>().submitted;
 }
 
+// Tasks of the whole-grid codelets (one per group of slabs) submitted so far
+int64_t nntile_host_grid_tasks_submitted(int dtype, int backward)
+{
+    if(backward)
+    {
+        if(dtype == DT_BF16) return starpu::sdpa_bwd_grid<bf16_t>().submitted;
+        if(dtype == DT_FP16) return starpu::sdpa_bwd_grid<fp16_t>().submitted;
+        return -1;
+    }
+    if(dtype == DT_BF16) return starpu::sdpa_fwd_grid<bf16_t>().submitted;
+    if(dtype == DT_FP16) return starpu::sdpa_fwd_grid<fp16_t>().submitted;
+    return starpu::sdpa_fwd_grid<fp32_t>().submitted;
+}
+
+const char *nntile_host_grid_codelet_name(int dtype, int backward)
+{
+    if(backward)
+    {
+        if(dtype == DT_BF16) return starpu::sdpa_bwd_grid<bf16_t>().name.c_str();
+        if(dtype == DT_FP16) return starpu::sdpa_bwd_grid<fp16_t>().name.c_str();
+        return "";
+    }
+    if(dtype == DT_BF16) return starpu::sdpa_fwd_grid<bf16_t>().name.c_str();
+    if(dtype == DT_FP16) return starpu::sdpa_fwd_grid<fp16_t>().name.c_str();
+    return starpu::sdpa_fwd_grid<fp32_t>().name.c_str();
+}
+
 const char *nntile_host_codelet_name(int dtype)
 {
     if(dtype == DT_BF16) return starpu::flash_sdpa_fwd_cudnn<bf16_t>().name.c_str();
@@ -449,7 +476,7 @@ void nntile_host_tensor_mark_written(void *t_)
 // then tensor::flash_sdpa_fwd_cudnn_async (op 0) or
 // tensor::flash_sdpa_fwd_cudnn_pairs_async (op 3), with HIP events on the
 // mirror's stream.  *ms = milliseconds per pass, *launches = attention
-// launches per pass (tile tasks + direct launches).
+// launches per pass (tile tasks + whole-grid tasks + direct launches).
 int nntile_host_time_flash_sdpa_fwd(int op, int dtype, void *K, void *Q, void *mask,
         void *lse, void *V, void *A, int steps, int warmup, double *ms, int64_t *launches,
         char *err, int errlen)
@@ -459,8 +486,12 @@ int nntile_host_time_flash_sdpa_fwd(int op, int dtype, void *K, void *Q, void *m
         auto k = static_cast<AnyTensor *>(K), q = static_cast<AnyTensor *>(Q),
              m = static_cast<AnyTensor *>(mask), l = static_cast<AnyTensor *>(lse),
              v = static_cast<AnyTensor *>(V), a = static_cast<AnyTensor *>(A);
-        const int64_t before = nntile_host_tasks_submitted(dtype)
-            + starpu::direct_launches();
+        auto count = [&]()
+        {
+            return nntile_host_tasks_submitted(dtype) + nntile_host_grid_tasks_submitted(dtype, 0)
+                + starpu::direct_launches();
+        };
+        const int64_t before = count();
         double total = 0.0;
         auto pass = [&]()
         {
@@ -474,7 +505,7 @@ int nntile_host_time_flash_sdpa_fwd(int op, int dtype, void *K, void *Q, void *m
             pass();
         }
         starpu::task_wait_for_all();
-        const int64_t mid = nntile_host_tasks_submitted(dtype) + starpu::direct_launches();
+        const int64_t mid = count();
         total = starpu::time_on_stream_ms([&]()
         {
             for(int i = 0; i < steps; ++i)
@@ -482,7 +513,7 @@ int nntile_host_time_flash_sdpa_fwd(int op, int dtype, void *K, void *Q, void *m
                 pass();
             }
         });
-        const int64_t after = nntile_host_tasks_submitted(dtype) + starpu::direct_launches();
+        const int64_t after = count();
         (void)before;
         *ms = total / (steps > 0 ? steps : 1);
         *launches = steps > 0 ? (after - mid) / steps : 0;

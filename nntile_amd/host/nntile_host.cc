@@ -389,6 +389,171 @@ template class FlashSdpaBwdCudnn<std::tuple<fp16_t>>;
 template FlashSdpaBwdCudnn<std::tuple<bf16_t>> &flash_sdpa_bwd_cudnn<bf16_t>();
 template FlashSdpaBwdCudnn<std::tuple<fp16_t>> &flash_sdpa_bwd_cudnn<fp16_t>();
 
+// ---- codelets of the whole-grid calls ------------------------------------------
+
+// "Task execution" of a codelet with a free number of handles: look-alike
+// variable interfaces in the order given, the body called at once on the
+// context's stream (it only enqueues).
+static void run_body(void (*body)(void **, void *),
+        const std::vector<const Handle *> &handles, void *args)
+{
+    std::vector<nntile_hip_variable_interface> ifs(handles.size());
+    std::vector<void *> buffers(handles.size());
+    for(std::size_t i = 0; i < handles.size(); ++i)
+    {
+        ifs[i].id = 2;      // STARPU_VARIABLE_INTERFACE_ID
+        ifs[i].ptr = reinterpret_cast<std::uintptr_t>(handles[i]->get_ptr());
+        ifs[i].dev_handle = ifs[i].ptr;
+        ifs[i].offset = 0;
+        ifs[i].elemsize = handles[i]->size();
+        buffers[i] = &ifs[i];
+    }
+    (void)get_local_stream();       // makes sure the provider is registered
+    body(buffers.data(), args);
+}
+
+static void check_tile_counts(const nntile_hip_sdpa_grid_cl_args &g, std::size_t n_k,
+        std::size_t n_q, const char *what)
+{
+    const std::size_t n_slabs = g.n_slabs > 0 ? static_cast<std::size_t>(g.n_slabs) : 1;
+    if(n_k != n_slabs * static_cast<std::size_t>(g.n_kv_tiles)
+            || n_q != n_slabs * static_cast<std::size_t>(g.n_q_tiles))
+    {
+        throw std::runtime_error(std::string("Error in ") + what
+                + " task submission: handle counts do not match the tile grid");
+    }
+}
+
+template<typename T>
+SdpaFwdGrid<std::tuple<T>>::SdpaFwdGrid():
+    name(std::string("nntile_sdpa_fwd_grid_hip_") + T::short_name)
+{
+}
+
+template<> void SdpaFwdGrid<std::tuple<bf16_t>>::hip(void *buffers[], void *cl_args) noexcept
+{
+    nntile_hip_sdpa_fwd_grid_codelet_bf16(buffers, cl_args);
+}
+
+template<> void SdpaFwdGrid<std::tuple<fp16_t>>::hip(void *buffers[], void *cl_args) noexcept
+{
+    nntile_hip_sdpa_fwd_grid_codelet_fp16(buffers, cl_args);
+}
+
+template<> void SdpaFwdGrid<std::tuple<fp32_t>>::hip(void *buffers[], void *cl_args) noexcept
+{
+    nntile_hip_sdpa_fwd_grid_codelet_fp32(buffers, cl_args);
+}
+
+template<typename T>
+void SdpaFwdGrid<std::tuple<T>>::submit(const args_t &geometry,
+        const std::vector<Handle> &K, const std::vector<Handle> &V,
+        const std::vector<Handle> &Q, const std::vector<Handle> &logsumexp,
+        const std::vector<Handle> &A)
+{
+    check_tile_counts(geometry, K.size(), Q.size(), "sdpa_fwd_grid");
+    if(V.size() != K.size() || logsumexp.size() != Q.size() || A.size() != Q.size())
+    {
+        throw std::runtime_error("Error in sdpa_fwd_grid task submission: handle counts differ");
+    }
+    // arguments malloc'ed and owned by the task, as in the reference
+    auto *args = static_cast<args_t *>(std::malloc(sizeof(args_t)));
+    if(args == nullptr)
+    {
+        throw std::runtime_error("Error in sdpa_fwd_grid task submission");
+    }
+    *args = geometry;
+    args->owner = this;
+    std::vector<const Handle *> handles;
+    handles.reserve(2 * K.size() + 3 * Q.size());
+    for(const auto &h : K) { handles.push_back(&h); }              // R
+    for(const auto &h : V) { handles.push_back(&h); }              // R
+    for(const auto &h : Q) { handles.push_back(&h); }              // R
+    for(const auto &h : logsumexp) { handles.push_back(&h); h.mark_written(); }    // RW
+    for(const auto &h : A) { handles.push_back(&h); h.mark_written(); }            // RW
+    run_body(&hip, handles, args);
+    std::free(args);
+    ++submitted;
+}
+
+template<typename T> SdpaFwdGrid<std::tuple<T>> &sdpa_fwd_grid()
+{
+    static SdpaFwdGrid<std::tuple<T>> codelet;
+    return codelet;
+}
+
+template class SdpaFwdGrid<std::tuple<bf16_t>>;
+template class SdpaFwdGrid<std::tuple<fp16_t>>;
+template class SdpaFwdGrid<std::tuple<fp32_t>>;
+template SdpaFwdGrid<std::tuple<bf16_t>> &sdpa_fwd_grid<bf16_t>();
+template SdpaFwdGrid<std::tuple<fp16_t>> &sdpa_fwd_grid<fp16_t>();
+template SdpaFwdGrid<std::tuple<fp32_t>> &sdpa_fwd_grid<fp32_t>();
+
+template<typename T>
+SdpaBwdGrid<std::tuple<T>>::SdpaBwdGrid():
+    name(std::string("nntile_sdpa_bwd_grid_hip_") + T::short_name)
+{
+}
+
+template<> void SdpaBwdGrid<std::tuple<bf16_t>>::hip(void *buffers[], void *cl_args) noexcept
+{
+    nntile_hip_sdpa_bwd_grid_codelet_bf16(buffers, cl_args);
+}
+
+template<> void SdpaBwdGrid<std::tuple<fp16_t>>::hip(void *buffers[], void *cl_args) noexcept
+{
+    nntile_hip_sdpa_bwd_grid_codelet_fp16(buffers, cl_args);
+}
+
+template<typename T>
+void SdpaBwdGrid<std::tuple<T>>::submit(const args_t &geometry,
+        const std::vector<Handle> &K, const std::vector<Handle> &V,
+        const std::vector<Handle> &Q, const std::vector<Handle> &A,
+        const std::vector<Handle> &dA, const std::vector<Handle> &logsumexp,
+        const std::vector<Handle> &dK, const std::vector<Handle> &dQ,
+        const std::vector<Handle> &dV, Handle scratch)
+{
+    check_tile_counts(geometry, K.size(), Q.size(), "sdpa_bwd_grid");
+    if(V.size() != K.size() || dK.size() != K.size() || dV.size() != K.size()
+            || A.size() != Q.size() || dA.size() != Q.size() || logsumexp.size() != Q.size()
+            || dQ.size() != Q.size())
+    {
+        throw std::runtime_error("Error in sdpa_bwd_grid task submission: handle counts differ");
+    }
+    auto *args = static_cast<args_t *>(std::malloc(sizeof(args_t)));
+    if(args == nullptr)
+    {
+        throw std::runtime_error("Error in sdpa_bwd_grid task submission");
+    }
+    *args = geometry;
+    args->owner = this;
+    std::vector<const Handle *> handles;
+    handles.reserve(4 * K.size() + 5 * Q.size() + 1);
+    for(const auto *group : {&K, &V, &Q, &A, &dA, &logsumexp})     // R
+    {
+        for(const auto &h : *group) { handles.push_back(&h); }
+    }
+    for(const auto *group : {&dK, &dQ, &dV})                        // RW
+    {
+        for(const auto &h : *group) { handles.push_back(&h); h.mark_written(); }
+    }
+    handles.push_back(&scratch);                                     // SCRATCH
+    run_body(&hip, handles, args);
+    std::free(args);
+    ++submitted;
+}
+
+template<typename T> SdpaBwdGrid<std::tuple<T>> &sdpa_bwd_grid()
+{
+    static SdpaBwdGrid<std::tuple<T>> codelet;
+    return codelet;
+}
+
+template class SdpaBwdGrid<std::tuple<bf16_t>>;
+template class SdpaBwdGrid<std::tuple<fp16_t>>;
+template SdpaBwdGrid<std::tuple<bf16_t>> &sdpa_bwd_grid<bf16_t>();
+template SdpaBwdGrid<std::tuple<fp16_t>> &sdpa_bwd_grid<fp16_t>();
+
 } // namespace starpu
 
 // ---------------------------------------------------------------------------
@@ -917,14 +1082,16 @@ Index flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
         {
             ++count;
         }
-        nntile_hip_sdpa_grid_args a;
+        // one task of the whole-grid codelet for these slabs
+        nntile_hip_sdpa_grid_cl_args a;
         std::memset(&a, 0, sizeof(a));
+        a.seq = Q.basetile_shape[1];
+        a.head = Q.shape[0];
+        a.batch = slabs[first].batch;
         a.q_seq = Q.shape[1];
         a.k_seq = K.shape[1];
         a.q_tile = Q.basetile_shape[1];
         a.k_tile = K.basetile_shape[1];
-        a.head = Q.shape[0];
-        a.batch = slabs[first].batch;
         a.n_batch = a.batch;
         a.kv_group = 1;
         a.mask_mode = mask_mode;
@@ -933,32 +1100,24 @@ Index flash_sdpa_fwd_hip_async(const Tensor<T> &K, const Tensor<T> &Q,
         a.n_kv_tiles = static_cast<std::int32_t>(n_kv);
         a.n_slabs = static_cast<std::int32_t>(count);
         a.causal_offset = causal_offset;
+        std::vector<starpu::Handle> Kh, Vh, Qh, Lh, Ah;
         for(std::size_t s = 0; s < count; ++s)
         {
             const Index g2 = slabs[first + s].g2, g3 = slabs[first + s].g3,
                   g4 = slabs[first + s].g4;
             for(Index t = 0; t < n_kv; ++t)
             {
-                a.K[s * n_kv + t] = K.get_tile({0, t, g2, g3, g4}).get_ptr();
-                a.V[s * n_kv + t] = V.get_tile({0, t, g2, g3, g4}).get_ptr();
+                Kh.push_back(K.get_tile({0, t, g2, g3, g4}));
+                Vh.push_back(V.get_tile({0, t, g2, g3, g4}));
             }
             for(Index t = 0; t < n_q; ++t)
             {
-                a.Q[s * n_q + t] = Q.get_tile({0, t, g2, g3, g4}).get_ptr();
-                a.A[s * n_q + t] = A.get_tile({0, t, g2, g3, g4}).get_ptr();
-                a.lse[s * n_q + t] = static_cast<float *>(
-                        logsumexp.get_tile({t, g2, g3, g4}).get_ptr());
-                A.get_tile({0, t, g2, g3, g4}).mark_written();
-                logsumexp.get_tile({t, g2, g3, g4}).mark_written();
+                Qh.push_back(Q.get_tile({0, t, g2, g3, g4}));
+                Ah.push_back(A.get_tile({0, t, g2, g3, g4}));
+                Lh.push_back(logsumexp.get_tile({t, g2, g3, g4}));
             }
         }
-        starpu::count_direct_launch();
-        const int rc = GridCall<T>::run(starpu::get_local_stream(), &a);
-        if(rc != NNTILE_HIP_OK)
-        {
-            throw std::runtime_error("Error in flash_sdpa_fwd_hip launch (code "
-                    + std::to_string(rc) + ")");
-        }
+        starpu::sdpa_fwd_grid<T>().submit(a, Kh, Vh, Qh, Lh, Ah);
         first += count;
         ++launches;
     }
@@ -1444,7 +1603,7 @@ static Index bwd_grid(const Tensor<T> &K, const Tensor<T> &Q,
     // call writes what it reads there.
     const std::size_t ws_bytes = sizeof(float) * per_call * static_cast<std::size_t>(Q.shape[1]
             * Q.basetile_shape[2] * Q.basetile_shape[3] * Q.basetile_shape[4]);
-    starpu::VariableHandle workspace(ws_bytes);
+    starpu::VariableHandle workspace = starpu::worker_scratch(ws_bytes);
     Index calls = 0;
     for(std::size_t first = 0; first < slabs.size();)
     {
@@ -1454,14 +1613,16 @@ static Index bwd_grid(const Tensor<T> &K, const Tensor<T> &Q,
         {
             ++count;
         }
-        nntile_hip_sdpa_bwd_grid_args a;
+        // one task of the whole-grid codelet for these slabs
+        nntile_hip_sdpa_grid_cl_args a;
         std::memset(&a, 0, sizeof(a));
+        a.seq = Q.basetile_shape[1];
+        a.head = Q.shape[0];
+        a.batch = slabs[first].batch;
         a.q_seq = Q.shape[1];
         a.k_seq = K.shape[1];
         a.q_tile = Q.basetile_shape[1];
         a.k_tile = K.basetile_shape[1];
-        a.head = Q.shape[0];
-        a.batch = slabs[first].batch;
         a.n_batch = a.batch;
         a.kv_group = 1;
         a.mask_mode = mask_mode;
@@ -1469,39 +1630,28 @@ static Index bwd_grid(const Tensor<T> &K, const Tensor<T> &Q,
         a.n_kv_tiles = static_cast<std::int32_t>(n_kv);
         a.n_slabs = static_cast<std::int32_t>(count);
         a.causal_offset = causal_offset;
+        std::vector<starpu::Handle> Kh, Vh, Qh, Ah, dAh, Lh, dKh, dQh, dVh;
         for(std::size_t s = 0; s < count; ++s)
         {
             const Index g2 = slabs[first + s].g2, g3 = slabs[first + s].g3,
                   g4 = slabs[first + s].g4;
             for(Index t = 0; t < n_kv; ++t)
             {
-                a.K[s * n_kv + t] = K.get_tile({0, t, g2, g3, g4}).get_ptr();
-                a.V[s * n_kv + t] = V.get_tile({0, t, g2, g3, g4}).get_ptr();
-                a.dK[s * n_kv + t] = dK.get_tile({0, t, g2, g3, g4}).get_ptr();
-                a.dV[s * n_kv + t] = dV.get_tile({0, t, g2, g3, g4}).get_ptr();
-                dK.get_tile({0, t, g2, g3, g4}).mark_written();
-                dV.get_tile({0, t, g2, g3, g4}).mark_written();
+                Kh.push_back(K.get_tile({0, t, g2, g3, g4}));
+                Vh.push_back(V.get_tile({0, t, g2, g3, g4}));
+                dKh.push_back(dK.get_tile({0, t, g2, g3, g4}));
+                dVh.push_back(dV.get_tile({0, t, g2, g3, g4}));
             }
             for(Index t = 0; t < n_q; ++t)
             {
-                a.Q[s * n_q + t] = Q.get_tile({0, t, g2, g3, g4}).get_ptr();
-                a.A[s * n_q + t] = A.get_tile({0, t, g2, g3, g4}).get_ptr();
-                a.dA[s * n_q + t] = dA.get_tile({0, t, g2, g3, g4}).get_ptr();
-                a.dQ[s * n_q + t] = dQ.get_tile({0, t, g2, g3, g4}).get_ptr();
-                a.lse[s * n_q + t] = static_cast<const float *>(
-                        logsumexp.get_tile({t, g2, g3, g4}).get_ptr());
-                dQ.get_tile({0, t, g2, g3, g4}).mark_written();
+                Qh.push_back(Q.get_tile({0, t, g2, g3, g4}));
+                Ah.push_back(A.get_tile({0, t, g2, g3, g4}));
+                dAh.push_back(dA.get_tile({0, t, g2, g3, g4}));
+                dQh.push_back(dQ.get_tile({0, t, g2, g3, g4}));
+                Lh.push_back(logsumexp.get_tile({t, g2, g3, g4}));
             }
         }
-        a.workspace = workspace.get_ptr();
-        a.workspace_bytes = ws_bytes;
-        starpu::count_direct_launch();
-        const int rc = BwdGridCall<T>::run(starpu::get_local_stream(), &a);
-        if(rc != NNTILE_HIP_OK)
-        {
-            throw std::runtime_error("Error in flash_sdpa_bwd_hip grid launch (code "
-                    + std::to_string(rc) + ")");
-        }
+        starpu::sdpa_bwd_grid<T>().submit(a, Kh, Vh, Qh, Ah, dAh, Lh, dKh, dQh, dVh, workspace);
         ++calls;
         first += count;
     }

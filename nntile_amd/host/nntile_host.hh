@@ -109,7 +109,9 @@ Handle worker_scratch(std::size_t size);
 void *get_local_stream();
 void task_wait_for_all();
 //! Launches that tensor-level functions made through the C ABI directly
-//! (not as codelet tasks) since the start of the process
+//! (not as codelet tasks) since the start of the process: single tile pairs
+//! whose mask tile is open or on the causal rule (the whole-grid calls are
+//! tasks of the SdpaFwdGrid / SdpaBwdGrid codelets)
 std::int64_t direct_launches();
 void count_direct_launch();
 //! Milliseconds the stream needs for what `enqueue` puts on it (HIP events
@@ -177,6 +179,59 @@ public:
 };
 
 template<typename T> FlashSdpaBwdCudnn<std::tuple<T>> &flash_sdpa_bwd_cudnn();
+
+//! Codelets of the whole-grid calls: ONE task for all (query tile, key tile)
+//! pairs of a group of slabs of the batch grid.  No counterpart object in the
+//! reference, which submits a FlashSdpaFwdCudnn / FlashSdpaBwdCudnn task per
+//! pair (src/tensor/flash_sdpa_fwd_cudnn.cc:246-274,
+//! src/tensor/flash_sdpa_bwd_cudnn.cc:172-247); built like those: a body with
+//! the codelet signature, arguments malloc'ed per task and owned by it, the
+//! number of handles free (nbuffers = STARPU_VARIABLE_NBUFFERS,
+//! src/starpu/codelet.cc:58).  Handles travel tile after tile:
+//!   forward : K tiles (R), V tiles (R), Q tiles (R), logsumexp tiles (RW),
+//!             A tiles (RW)
+//!   backward: K, V, Q, A, dA, logsumexp tiles (R), dK, dQ, dV tiles (RW),
+//!             one scratch buffer
+template<typename T> class SdpaFwdGrid;
+
+template<typename T>
+class SdpaFwdGrid<std::tuple<T>>
+{
+public:
+    std::string name;       // "nntile_sdpa_fwd_grid_hip_<type>"
+    //! the reference's args_t members first, then the geometry of the grid
+    using args_t = nntile_hip_sdpa_grid_cl_args;
+    SdpaFwdGrid();
+    static constexpr std::array<void (*)(void **, void *), 1> cpu_funcs = {nullptr};
+    static void hip(void *buffers[], void *cl_args) noexcept;
+    void submit(const args_t &geometry, const std::vector<Handle> &K,
+            const std::vector<Handle> &V, const std::vector<Handle> &Q,
+            const std::vector<Handle> &logsumexp, const std::vector<Handle> &A);
+    Index submitted = 0;
+};
+
+template<typename T> SdpaFwdGrid<std::tuple<T>> &sdpa_fwd_grid();
+
+template<typename T> class SdpaBwdGrid;
+
+template<typename T>
+class SdpaBwdGrid<std::tuple<T>>
+{
+public:
+    std::string name;       // "nntile_sdpa_bwd_grid_hip_<type>"
+    using args_t = nntile_hip_sdpa_grid_cl_args;
+    SdpaBwdGrid();
+    static constexpr std::array<void (*)(void **, void *), 1> cpu_funcs = {nullptr};
+    static void hip(void *buffers[], void *cl_args) noexcept;
+    void submit(const args_t &geometry, const std::vector<Handle> &K,
+            const std::vector<Handle> &V, const std::vector<Handle> &Q,
+            const std::vector<Handle> &A, const std::vector<Handle> &dA,
+            const std::vector<Handle> &logsumexp, const std::vector<Handle> &dK,
+            const std::vector<Handle> &dQ, const std::vector<Handle> &dV, Handle scratch);
+    Index submitted = 0;
+};
+
+template<typename T> SdpaBwdGrid<std::tuple<T>> &sdpa_bwd_grid();
 
 } // namespace starpu
 

@@ -12,6 +12,7 @@
 #include <cstdint>
 
 #include "../../include/nntile_hip_sdpa.h"
+#include "../../include/nntile_hip_starpu.h"
 
 #if defined(__has_include)
 #if __has_include(<starpu.h>) && __has_include(<starpu_hip.h>)
@@ -106,6 +107,47 @@ extern "C" int nntile_hip_starpu_register(void *cl_fwd, void *cl_bwd, int dtype)
     return 0;
 }
 
+// The codelets of the whole-grid calls take any number of handles
+extern "C" int nntile_hip_starpu_register_grid(void *cl_fwd_grid, void *cl_bwd_grid, int dtype)
+{
+    nntile_hip_set_stream_provider(&local_stream);
+    void (*fwd)(void **, void *) = nullptr;
+    void (*bwd)(void **, void *) = nullptr;
+    switch(dtype)
+    {
+        case NNTILE_HIP_DTYPE_BF16:
+            fwd = nntile_hip_sdpa_fwd_grid_codelet_bf16;
+            bwd = nntile_hip_sdpa_bwd_grid_codelet_bf16;
+            break;
+        case NNTILE_HIP_DTYPE_FP16:
+            fwd = nntile_hip_sdpa_fwd_grid_codelet_fp16;
+            bwd = nntile_hip_sdpa_bwd_grid_codelet_fp16;
+            break;
+        case 2:
+            fwd = nntile_hip_sdpa_fwd_grid_codelet_fp32;
+            break;
+        default:
+            return -1;
+    }
+    if(cl_fwd_grid != nullptr)
+    {
+        auto *cl = static_cast<struct starpu_codelet *>(cl_fwd_grid);
+        cl->nbuffers = STARPU_VARIABLE_NBUFFERS;
+        add_hip(cl, fwd);
+    }
+    if(cl_bwd_grid != nullptr)
+    {
+        if(bwd == nullptr)
+        {
+            return -1;
+        }
+        auto *cl = static_cast<struct starpu_codelet *>(cl_bwd_grid);
+        cl->nbuffers = STARPU_VARIABLE_NBUFFERS;
+        add_hip(cl, bwd);
+    }
+    return 0;
+}
+
 #else // no StarPU in this build
 
 extern "C" int nntile_hip_starpu_available(void)
@@ -116,6 +158,11 @@ extern "C" int nntile_hip_starpu_available(void)
 extern "C" int nntile_hip_starpu_register(void *, void *, int)
 {
     return -1;      // built without StarPU
+}
+
+extern "C" int nntile_hip_starpu_register_grid(void *, void *, int)
+{
+    return -1;
 }
 
 #endif

@@ -59,6 +59,10 @@ def lib():
         L.nntile_host_footprint.restype = ctypes.c_uint32
         L.nntile_host_tasks_submitted.argtypes = [ctypes.c_int]
         L.nntile_host_tasks_submitted.restype = i64
+        L.nntile_host_grid_tasks_submitted.argtypes = [ctypes.c_int, ctypes.c_int]
+        L.nntile_host_grid_tasks_submitted.restype = i64
+        L.nntile_host_grid_codelet_name.argtypes = [ctypes.c_int, ctypes.c_int]
+        L.nntile_host_grid_codelet_name.restype = ctypes.c_char_p
         L.nntile_host_codelet_name.argtypes = [ctypes.c_int]
         L.nntile_host_codelet_name.restype = ctypes.c_char_p
         L.nntile_host_mask_cache_stats.argtypes = [ctypes.POINTER(ctypes.c_uint64)] * 2
@@ -220,6 +224,15 @@ def tasks_submitted_bwd(dtype):
 
 def codelet_name_bwd(dtype):
     return lib().nntile_host_codelet_name_bwd(DTYPES[dtype]).decode()
+
+
+def grid_tasks_submitted(dtype, backward=False):
+    """Tasks of the whole-grid codelets (one per group of slabs) so far."""
+    return int(lib().nntile_host_grid_tasks_submitted(DTYPES[dtype], int(backward)))
+
+
+def grid_codelet_name(dtype, backward=False):
+    return lib().nntile_host_grid_codelet_name(DTYPES[dtype], int(backward)).decode()
 
 
 def tasks_submitted(dtype):

@@ -152,6 +152,37 @@ def test_starpu_registration_unit_compiles_to_stubs_here():
     L = hm.lib()
     assert L.nntile_hip_starpu_available() == 0
     assert L.nntile_hip_starpu_register(None, None, 0) == -1
+    assert L.nntile_hip_starpu_register_grid(None, None, 0) == -1
+
+
+def test_host_library_exports_what_its_header_declares():
+    from nntile_amd import host_mirror as hm
+    header = open(os.path.join(ROOT, "include", "nntile_hip_starpu.h")).read()
+    declared = set(re.findall(r"\b(nntile_hip_[a-z0-9_]+)\s*\(", header))
+    assert declared == {"nntile_hip_starpu_available", "nntile_hip_starpu_register",
+                        "nntile_hip_starpu_register_grid"}
+    L = hm.lib()
+    for name in sorted(declared):
+        assert hasattr(L, name), name
+
+
+def test_grid_codelet_bodies_report_and_return_on_bad_arguments(capfd):
+    """Error behaviour of the reference body (src/starpu/flash_sdpa_fwd_cudnn.cc:
+    69-115): a line on stderr, the task does nothing."""
+    L = h.lib()
+    for name in ("nntile_hip_sdpa_fwd_grid_codelet_bf16", "nntile_hip_sdpa_bwd_grid_codelet_fp16"):
+        fn = getattr(L, name)
+        fn.argtypes, fn.restype = [ctypes.c_void_p, ctypes.c_void_p], None
+        fn(None, None)
+        a = h.GridClArgs()
+        a.n_q_tiles, a.n_kv_tiles, a.n_slabs = 40, 40, 2        # 80 tiles an axis
+        bufs = (ctypes.c_void_p * 4)()
+        fn(bufs, ctypes.addressof(a))
+        a.n_q_tiles, a.n_kv_tiles, a.n_slabs = 1, 1, 1
+        fn(bufs, ctypes.addressof(a))                            # null buffers
+    err = capfd.readouterr().err
+    assert err.count("skipping task") == 6
+    assert ctypes.sizeof(h.GridClArgs) == 13 * 8 + 6 * 4
 
 
 def test_starpu_registration_unit_is_valid_against_the_api_it_names(tmp_path):
@@ -170,9 +201,9 @@ def test_starpu_registration_unit_is_valid_against_the_api_it_names(tmp_path):
     (tmp_path / "starpu.h").write_text(
         "#pragma once\n#include <stddef.h>\n#include <stdint.h>\n"
         "#define STARPU_MAXIMPLEMENTATIONS 4\n#define STARPU_HIP (1 << 7)\n"
-        "#define STARPU_HIP_ASYNC 1\n"
+        "#define STARPU_HIP_ASYNC 1\n#define STARPU_VARIABLE_NBUFFERS (-1)\n"
         "struct starpu_codelet { uint32_t where; void (*hip_funcs[STARPU_MAXIMPLEMENTATIONS])(void **, void *);"
-        " char hip_flags[STARPU_MAXIMPLEMENTATIONS]; };\n"
+        " char hip_flags[STARPU_MAXIMPLEMENTATIONS]; int nbuffers; };\n"
         "struct starpu_variable_interface { int id; uintptr_t ptr; uintptr_t dev_handle; size_t offset;"
         " size_t elemsize; };\n")
     (tmp_path / "starpu_hip.h").write_text(

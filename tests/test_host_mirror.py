@@ -222,8 +222,12 @@ def test_reference_signature_caches_the_mask_classes_and_drops_them_on_a_write(o
 
     arr, M = _mask_tensor(dtype, causal, tile)
     M.from_array(arr)
-    # first sight: classified (a miss); the causal rule: no tile tasks
+    # first sight: classified (a miss); the causal rule: no tile tasks, one
+    # task of the whole-grid codelet instead (all slabs have the same extents)
+    grid0 = hm.grid_tasks_submitted(dtype)
     assert run(M, causal) == (0, 0, 1)
+    assert hm.grid_tasks_submitted(dtype) - grid0 == 1
+    assert hm.grid_codelet_name(dtype) == "nntile_sdpa_fwd_grid_hip_" + dtype
     # the same mask again: found, nothing re-read
     assert run(M, causal) == (0, 1, 0)
     assert run(M, causal) == (0, 1, 0)
