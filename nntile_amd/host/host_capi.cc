@@ -453,6 +453,55 @@ void nntile_host_mask_cache_stats(uint64_t *hits, uint64_t *misses)
     *misses = st.misses;
 }
 
+uint64_t nntile_host_mask_classifications(void)
+{
+    return tensor::flash_sdpa_mask_cache_stats().classifications;
+}
+
+// tensor::flash_sdpa_mask_declare_constant (forget != 0: flash_sdpa_mask_forget)
+int nntile_host_mask_declare_constant(void *mask_, int forget, char *err, int errlen)
+{
+    try
+    {
+        auto *m = static_cast<AnyTensor *>(mask_);
+        if(m->dtype == DT_BF16)
+        {
+            forget ? tensor::flash_sdpa_mask_forget<bf16_t>(*m->bf16)
+                : tensor::flash_sdpa_mask_declare_constant<bf16_t>(*m->bf16);
+        }
+        else if(m->dtype == DT_FP16)
+        {
+            forget ? tensor::flash_sdpa_mask_forget<fp16_t>(*m->fp16)
+                : tensor::flash_sdpa_mask_declare_constant<fp16_t>(*m->fp16);
+        }
+        else
+        {
+            forget ? tensor::flash_sdpa_mask_forget<fp32_t>(*m->fp32)
+                : tensor::flash_sdpa_mask_declare_constant<fp32_t>(*m->fp32);
+        }
+        return 0;
+    }
+    catch(const std::exception &e) { return fail(err, errlen, e); }
+}
+
+// Device address of tile `i` of a tensor (for tests that write a tile by
+// means the runtime does not see)
+void *nntile_host_tensor_tile_ptr(void *t_, int64_t i)
+{
+    auto *t = static_cast<AnyTensor *>(t_);
+    if(t->dtype == DT_BF16) return t->bf16->get_tile(i).get_ptr();
+    if(t->dtype == DT_FP16) return t->fp16->get_tile(i).get_ptr();
+    return t->fp32->get_tile(i).get_ptr();
+}
+
+int64_t nntile_host_tensor_tile_bytes(void *t_, int64_t i)
+{
+    auto *t = static_cast<AnyTensor *>(t_);
+    if(t->dtype == DT_BF16) return static_cast<int64_t>(t->bf16->get_tile(i).size());
+    if(t->dtype == DT_FP16) return static_cast<int64_t>(t->fp16->get_tile(i).size());
+    return static_cast<int64_t>(t->fp32->get_tile(i).size());
+}
+
 void nntile_host_mask_cache_clear(void)
 {
     tensor::flash_sdpa_mask_cache_clear();

@@ -990,11 +990,16 @@ void flash_sdpa_fwd_cudnn(const Tensor<T> &K, const Tensor<T> &Q,
 
 // ---- what is known about a mask, kept with its handles ----------------------
 // A layer builds its mask once and passes the same tensor to every call
-// (wrappers/python/nntile/model/gpt2_attention.py:72-87), so the classes of
-// its tiles are worth one blocking pass on first sight.  An entry is valid as
-// long as every tile of the mask is the allocation it was and has not been
-// given to a writer since (Handle::write_stamp); the key is the first tile's
-// address.
+// (wrappers/python/nntile/model/gpt2_attention.py:72-87).  When it says so
+// (flash_sdpa_mask_declare_constant, once, after building the mask) the classes
+// of the mask's tiles are computed in one blocking pass and kept here; the
+// calls with the reference's signature look them up and never block.  An
+// entry is dropped by flash_sdpa_mask_forget, and - in this runtime, where
+// every write access goes through Handle::mark_written - when a tile is given
+// to a writer or its memory is reallocated (Handle::write_stamp); the key is
+// the first tile's address.  A mask that was not declared is never looked at
+// ahead of time: its pairs are submitted with their mask tiles, as the
+// reference does, whatever the tiles hold at that moment.
 namespace
 {
 
@@ -1008,7 +1013,7 @@ struct MaskCacheEntry
 
 std::mutex mask_cache_mutex;
 std::vector<MaskCacheEntry> mask_cache;         // few masks per process: linear search
-std::uint64_t mask_cache_hits = 0, mask_cache_misses = 0;
+std::uint64_t mask_cache_hits = 0, mask_cache_misses = 0, mask_cache_classifications = 0;
 constexpr std::size_t kMaskCacheEntries = 64;
 
 } // namespace
@@ -1016,7 +1021,7 @@ constexpr std::size_t kMaskCacheEntries = 64;
 MaskCacheStats flash_sdpa_mask_cache_stats()
 {
     std::lock_guard<std::mutex> guard(mask_cache_mutex);
-    return MaskCacheStats{mask_cache_hits, mask_cache_misses};
+    return MaskCacheStats{mask_cache_hits, mask_cache_misses, mask_cache_classifications};
 }
 
 void flash_sdpa_mask_cache_clear()
@@ -1179,58 +1184,131 @@ std::vector<int> flash_sdpa_mask_classes(const Tensor<T> &mask, Index causal_off
 }
 
 template<typename T>
-std::vector<int> flash_sdpa_cached_mask_classes(const Tensor<T> &mask, Index causal_offset)
+static std::vector<std::pair<const void *, std::uint64_t>> mask_identity(const Tensor<T> &mask)
 {
-    require(mask.ndim == 2, "mask must be 2-dimensional");
     std::vector<std::pair<const void *, std::uint64_t>> ident(mask.grid.nelems);
     for(Index i = 0; i < mask.grid.nelems; ++i)
     {
         const auto &tile = mask.get_tile(i);
         ident[i] = {tile.get_ptr(), tile.write_stamp()};
     }
+    return ident;
+}
+
+template<typename T>
+bool flash_sdpa_mask_known_classes(const Tensor<T> &mask, Index causal_offset,
+        std::vector<int> &classes)
+{
+    require(mask.ndim == 2, "mask must be 2-dimensional");
+    const auto ident = mask_identity(mask);
+    std::lock_guard<std::mutex> guard(mask_cache_mutex);
+    for(std::size_t e = 0; e < mask_cache.size(); )
     {
-        std::lock_guard<std::mutex> guard(mask_cache_mutex);
-        for(std::size_t e = 0; e < mask_cache.size(); )
+        auto &entry = mask_cache[e];
+        if(entry.tiles.empty() || ident.empty() || entry.tiles[0].first != ident[0].first)
         {
-            auto &entry = mask_cache[e];
-            if(entry.tiles.empty() || ident.empty() || entry.tiles[0].first != ident[0].first)
-            {
-                ++e;
-                continue;
-            }
-            if(entry.tiles == ident && entry.causal_offset == causal_offset
-                    && entry.shape == mask.shape && entry.basetile == mask.basetile_shape)
-            {
-                ++mask_cache_hits;
-                return entry.classes;
-            }
-            if(entry.tiles[0].second != ident[0].second)
-            {
-                // the memory at this address was written or reallocated
-                mask_cache.erase(mask_cache.begin() + static_cast<std::ptrdiff_t>(e));
-                continue;
-            }
             ++e;
+            continue;
         }
-        ++mask_cache_misses;
+        if(entry.tiles == ident && entry.causal_offset == causal_offset
+                && entry.shape == mask.shape && entry.basetile == mask.basetile_shape)
+        {
+            ++mask_cache_hits;
+            classes = entry.classes;
+            return true;
+        }
+        if(entry.tiles[0].second != ident[0].second)
+        {
+            // the memory at this address was given to a writer or reallocated
+            mask_cache.erase(mask_cache.begin() + static_cast<std::ptrdiff_t>(e));
+            continue;
+        }
+        ++e;
     }
+    ++mask_cache_misses;
+    return false;
+}
+
+template<typename T>
+void flash_sdpa_mask_declare_constant(const Tensor<T> &mask, Index causal_offset)
+{
+    require(mask.ndim == 2, "mask must be 2-dimensional");
     // (outside the lock: this blocks on the device)
     MaskCacheEntry fresh;
     fresh.classes = flash_sdpa_mask_classes<T>(mask, causal_offset);
-    fresh.tiles = std::move(ident);
+    fresh.tiles = mask_identity(mask);
     fresh.causal_offset = causal_offset;
     fresh.shape = mask.shape;
     fresh.basetile = mask.basetile_shape;
-    std::vector<int> classes = fresh.classes;
+    std::lock_guard<std::mutex> guard(mask_cache_mutex);
+    ++mask_cache_classifications;
+    // one entry per mask and offset: an earlier declaration is replaced
+    for(std::size_t e = 0; e < mask_cache.size(); )
     {
-        std::lock_guard<std::mutex> guard(mask_cache_mutex);
-        if(mask_cache.size() >= kMaskCacheEntries)
+        const auto &entry = mask_cache[e];
+        if(!entry.tiles.empty() && !fresh.tiles.empty()
+                && entry.tiles[0].first == fresh.tiles[0].first
+                && entry.causal_offset == causal_offset)
         {
-            mask_cache.erase(mask_cache.begin());
+            mask_cache.erase(mask_cache.begin() + static_cast<std::ptrdiff_t>(e));
+            continue;
         }
-        mask_cache.push_back(std::move(fresh));
+        ++e;
     }
-    return classes;
+    if(mask_cache.size() >= kMaskCacheEntries)
+    {
+        mask_cache.erase(mask_cache.begin());
+    }
+    mask_cache.push_back(std::move(fresh));
+}
+
+template<typename T>
+void flash_sdpa_mask_forget(const Tensor<T> &mask)
+{
+    if(mask.grid.nelems == 0)
+    {
+        return;
+    }
+    const void *first = mask.get_tile(0).get_ptr();
+    std::lock_guard<std::mutex> guard(mask_cache_mutex);
+    for(std::size_t e = 0; e < mask_cache.size(); )
+    {
+        if(!mask_cache[e].tiles.empty() && mask_cache[e].tiles[0].first == first)
+        {
+            mask_cache.erase(mask_cache.begin() + static_cast<std::ptrdiff_t>(e));
+            continue;
+        }
+        ++e;
+    }
+}
+
+bool flash_sdpa_classify_on_first_sight()
+{
+    static const bool on = []
+    {
+        const char *v = std::getenv("NNTILE_HIP_SDPA_CLASSIFY_ON_FIRST_SIGHT");
+        return v != nullptr && v[0] != '\0' && v[0] != '0';
+    }();
+    return on;
+}
+
+// The classes of a mask for the calls with the reference's signature: known
+// if the mask was declared constant (and neither written through this runtime
+// nor forgotten since); with the opt-in above an unknown mask is declared on
+// the spot (blocking).
+template<typename T>
+static bool classes_for_reference_call(const Tensor<T> &mask, std::vector<int> &classes)
+{
+    if(flash_sdpa_mask_known_classes<T>(mask, 0, classes))
+    {
+        return true;
+    }
+    if(!flash_sdpa_classify_on_first_sight())
+    {
+        return false;
+    }
+    flash_sdpa_mask_declare_constant<T>(mask, 0);
+    return flash_sdpa_mask_known_classes<T>(mask, 0, classes);
 }
 
 // What the classes say about the mask as a whole: NNTILE_HIP_MASK_NONE when
@@ -1347,9 +1425,15 @@ void flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
     flash_sdpa_fwd_cudnn_check(K, Q, mask, logsumexp, V, A);
     // The reference's signature carries no offset: its masks are square
     // (K.shape[1] == Q.shape[1] is one of its checks), the rule to look for is
-    // key <= query.
-    const std::vector<int> classes = flash_sdpa_cached_mask_classes<T>(mask, 0);
-    (void)flash_sdpa_fwd_cudnn_async<T>(K, Q, mask, classes, 0, logsumexp, V, A);
+    // key <= query.  A mask nothing is known about is read as the reference
+    // reads it: one task per pair with the pair's mask tile.
+    std::vector<int> classes;
+    if(classes_for_reference_call<T>(mask, classes))
+    {
+        (void)flash_sdpa_fwd_cudnn_async<T>(K, Q, mask, classes, 0, logsumexp, V, A);
+        return;
+    }
+    flash_sdpa_fwd_cudnn_pairs_async<T>(K, Q, mask, logsumexp, V, A);
 }
 
 // ---- backward: src/tensor/flash_sdpa_bwd_cudnn.cc:22-261 -------------------
@@ -1708,9 +1792,14 @@ void flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &dK, const Tensor<T> &dQ, const Tensor<T> &dV)
 {
     flash_sdpa_bwd_cudnn_check(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
-    const std::vector<int> classes = flash_sdpa_cached_mask_classes<T>(mask, 0);
-    (void)flash_sdpa_bwd_cudnn_async<T>(K, Q, V, A, dA, mask, classes, 0, logsumexp,
-            dK, dQ, dV);
+    std::vector<int> classes;
+    if(classes_for_reference_call<T>(mask, classes))
+    {
+        (void)flash_sdpa_bwd_cudnn_async<T>(K, Q, V, A, dA, mask, classes, 0, logsumexp,
+                dK, dQ, dV);
+        return;
+    }
+    flash_sdpa_bwd_cudnn_pairs_async<T>(K, Q, V, A, dA, mask, logsumexp, dK, dQ, dV);
 }
 
 #define NNTILE_HOST_INSTANTIATE_TENSOR_BWD(T) \
@@ -1742,7 +1831,9 @@ NNTILE_HOST_INSTANTIATE_TENSOR_BWD(fp16_t)
     template Index flash_sdpa_fwd_hip_async<T>(const Tensor<T> &, const Tensor<T> &, int, \
             Index, const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &, bool); \
     template std::vector<int> flash_sdpa_mask_classes<T>(const Tensor<T> &, Index); \
-    template std::vector<int> flash_sdpa_cached_mask_classes<T>(const Tensor<T> &, Index); \
+    template bool flash_sdpa_mask_known_classes<T>(const Tensor<T> &, Index, std::vector<int> &); \
+    template void flash_sdpa_mask_declare_constant<T>(const Tensor<T> &, Index); \
+    template void flash_sdpa_mask_forget<T>(const Tensor<T> &); \
     template void flash_sdpa_fwd_cudnn_pairs_async<T>(const Tensor<T> &, const Tensor<T> &, \
             const Tensor<T> &, const Tensor<fp32_t> &, const Tensor<T> &, const Tensor<T> &); \
     template Index flash_sdpa_fwd_cudnn_async<T>(const Tensor<T> &, const Tensor<T> &, \

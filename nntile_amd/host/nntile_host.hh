@@ -331,15 +331,17 @@ void flash_sdpa_fwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
 
 //! The reference's operation with the reference's arguments
 //! (src/tensor/flash_sdpa_fwd_cudnn.cc:210-279).  What it computes is the
-//! reference's result; how it is submitted depends on what the mask holds.
-//! The first call that sees a mask classifies its tiles (blocking, once:
-//! flash_sdpa_mask_classes against the rule key <= query) and keeps the
-//! classes keyed on the mask tiles' handles; later calls with the same,
-//! unwritten mask find them.  Then, as the overload that takes the classes
-//! does: a mask that is the causal rule or hides nothing - one launch per slab
-//! of the batch grid; otherwise per pair, hidden pairs not submitted, open and
-//! causal pairs without mask memory, the rest (a mask with bias values: every
-//! pair) exactly as flash_sdpa_fwd_cudnn_pairs_async.
+//! reference's result; how it is submitted depends on what is known about the
+//! mask.  Nothing known (the default): one task per (output tile, key tile)
+//! pair with the pair's mask tile, exactly as flash_sdpa_fwd_cudnn_pairs_async
+//! - the mask is read by the kernels when they run, so a mask that any task,
+//! kernel or copy has rewritten in the meantime is honoured.  Declared constant
+//! (flash_sdpa_mask_declare_constant): as the overload that takes the classes -
+//! a mask that is the causal rule or hides nothing becomes one task of the
+//! whole-grid codelet per group of slabs, otherwise hidden pairs are not
+//! submitted, open and causal pairs run without mask memory, the rest (a mask
+//! with bias values: every pair) as the reference does.  Never blocks: only
+//! the declaration does.
 template<typename T>
 void flash_sdpa_fwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
@@ -353,15 +355,43 @@ void flash_sdpa_fwd_cudnn_pairs_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &mask, const Tensor<fp32_t> &logsumexp,
         const Tensor<T> &V, const Tensor<T> &A);
 
-//! The classes of flash_sdpa_mask_classes(mask, causal_offset), computed on
-//! first sight of the mask and kept until one of its tiles is written or
-//! freed (Handle::write_stamp).  Blocking on a miss.
+//! The caller's statement that the contents of `mask` stay as they are from
+//! now on - what a layer says once after it has built its mask (the reference
+//! builds it at construction and never writes it again:
+//! wrappers/python/nntile/model/gpt2_attention.py:72-87).  BLOCKING: the
+//! mask's tiles are classified against the rule key <= query + causal_offset
+//! (one pass over the mask, one word per tile read back) and the classes are
+//! kept with the tiles' handles until flash_sdpa_mask_forget, until this
+//! runtime hands a tile to a writer (Handle::mark_written), or until the
+//! memory is freed.  The contract is the caller's: whoever rewrites a declared
+//! mask by means this runtime does not see (a kernel or copy of its own on
+//! get_ptr()) must call flash_sdpa_mask_forget first, exactly as it would have
+//! to tell StarPU about such a write.  Under StarPU the entry is keyed on the
+//! tiles' starpu_data_handle_t and dropped where the tensor unregisters or
+//! invalidates them (include/nntile/starpu/handle.hh: unregister,
+//! invalidate_submit).
 template<typename T>
-std::vector<int> flash_sdpa_cached_mask_classes(const Tensor<T> &mask, Index causal_offset);
+void flash_sdpa_mask_declare_constant(const Tensor<T> &mask, Index causal_offset = 0);
 
-//! Counters of that cache since the start of the process, and a reset of the
-//! cache (not of the counters)
-struct MaskCacheStats { std::uint64_t hits, misses; };
+//! Drops what flash_sdpa_mask_declare_constant stored for this mask
+template<typename T>
+void flash_sdpa_mask_forget(const Tensor<T> &mask);
+
+//! The classes stored for this mask and offset, if any; never blocks
+template<typename T>
+bool flash_sdpa_mask_known_classes(const Tensor<T> &mask, Index causal_offset,
+        std::vector<int> &classes);
+
+//! Opt-in for callers that cannot add the declaration: with the environment
+//! variable NNTILE_HIP_SDPA_CLASSIFY_ON_FIRST_SIGHT set (not "0"), a call with
+//! the reference's signature declares an unknown mask constant itself - it
+//! BLOCKS on that first call, and foreign writes to the mask go unnoticed.
+bool flash_sdpa_classify_on_first_sight();
+
+//! Counters of the store since the start of the process (look-ups that found
+//! an entry, look-ups that did not, blocking classifications), and a reset of
+//! the store (not of the counters)
+struct MaskCacheStats { std::uint64_t hits, misses, classifications; };
 MaskCacheStats flash_sdpa_mask_cache_stats();
 void flash_sdpa_mask_cache_clear();
 
@@ -414,9 +444,10 @@ void flash_sdpa_bwd_cudnn_check(const TensorTraits &K, const TensorTraits &Q,
         const TensorTraits &dK, const TensorTraits &dQ, const TensorTraits &dV);
 
 //! The reference's operation with the reference's arguments
-//! (src/tensor/flash_sdpa_bwd_cudnn.cc:172-247); submitted through the cached
-//! classes of the mask's tiles like the forward (hidden pairs not submitted,
-//! open and causal pairs without mask memory, the rest as the reference does)
+//! (src/tensor/flash_sdpa_bwd_cudnn.cc:172-247); a mask declared constant is
+//! submitted through the classes of its tiles like the forward (hidden pairs
+//! not submitted, open and causal pairs without mask memory, the rest as the
+//! reference does), any other mask pair by pair as the reference does
 template<typename T>
 void flash_sdpa_bwd_cudnn_async(const Tensor<T> &K, const Tensor<T> &Q,
         const Tensor<T> &V, const Tensor<T> &A, const Tensor<T> &dA,

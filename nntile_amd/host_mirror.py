@@ -69,6 +69,15 @@ def lib():
         L.nntile_host_mask_cache_stats.restype = None
         L.nntile_host_mask_cache_clear.argtypes = []
         L.nntile_host_mask_cache_clear.restype = None
+        L.nntile_host_mask_classifications.argtypes = []
+        L.nntile_host_mask_classifications.restype = ctypes.c_uint64
+        L.nntile_host_mask_declare_constant.argtypes = [ctypes.c_void_p, ctypes.c_int,
+                                                        ctypes.c_char_p, ctypes.c_int]
+        L.nntile_host_mask_declare_constant.restype = ctypes.c_int
+        L.nntile_host_tensor_tile_ptr.argtypes = [ctypes.c_void_p, i64]
+        L.nntile_host_tensor_tile_ptr.restype = ctypes.c_void_p
+        L.nntile_host_tensor_tile_bytes.argtypes = [ctypes.c_void_p, i64]
+        L.nntile_host_tensor_tile_bytes.restype = i64
         L.nntile_host_tensor_mark_written.argtypes = [vp]
         L.nntile_host_tensor_mark_written.restype = None
         L.nntile_host_time_flash_sdpa_fwd.argtypes = [
@@ -133,9 +142,33 @@ def flash_sdpa_fwd(op, K, Q, mask, lse, V, A, mask_mode=0, offset=0, overwrite=F
           None if mask is None else mask.h, lse.h, V.h, A.h, mask_mode, offset, int(overwrite))
 
 
+def mask_declare_constant(mask):
+    """tensor::flash_sdpa_mask_declare_constant: the mask's contents stay as
+    they are; its tiles are classified now (blocking) and the calls with the
+    reference's signature use the classes from here on."""
+    _call(lib().nntile_host_mask_declare_constant, mask.h, 0)
+
+
+def mask_forget(mask):
+    """tensor::flash_sdpa_mask_forget."""
+    _call(lib().nntile_host_mask_declare_constant, mask.h, 1)
+
+
+def mask_classifications():
+    """Blocking classifications of a mask since the start of the process."""
+    return int(lib().nntile_host_mask_classifications())
+
+
+def tile_ptr(tensor, i):
+    """(device address, bytes) of tile i: for writes the runtime does not see."""
+    return (int(lib().nntile_host_tensor_tile_ptr(tensor.h, i)),
+            int(lib().nntile_host_tensor_tile_bytes(tensor.h, i)))
+
+
 def mask_cache_stats():
-    """(hits, misses) of the mask-class cache behind the reference-signature
-    tensor operations (OP_TENSOR), since the start of the process."""
+    """(look-ups that found the mask's classes, look-ups that did not) behind
+    the reference-signature tensor operations (OP_TENSOR), since the start of
+    the process."""
     hits, misses = ctypes.c_uint64(0), ctypes.c_uint64(0)
     lib().nntile_host_mask_cache_stats(ctypes.byref(hits), ctypes.byref(misses))
     return hits.value, misses.value

@@ -110,6 +110,9 @@ def _run(dtype, arrs, mask_bool, head, seq, nb, grp, nkv, tile, op, **kw):
         m_t, _ = H.rounded(add, dtype)
         m_np = m_t.numpy() if dtype == "fp32" else m_t.view(__import__("torch").int16).numpy().view(np.uint16)
         mask = hm.Tensor(dtype, [seq, seq], [tile, tile]).from_array(np.asfortranarray(m_np))
+    if op == hm.OP_TENSOR and kw.pop("declare", True):
+        # what the layer says once after building its mask
+        hm.mask_declare_constant(mask)
     before = hm.tasks_submitted(dtype)
     hm.flash_sdpa_fwd(op, T["K"], T["Q"], mask, lse, T["V"], A, **kw)
     a = A.to_array()
@@ -135,10 +138,15 @@ def test_tensor_level_tiles_match_oracle(oracle, dtype, head, seq, nb, grp, nkv,
         # one task per (output tile, key tile), none skipped (src/tensor/...:221-274)
         assert tasks == ntiles * (seq // tile)
         assert H.rel_fro(got, want) < H.TOL[dtype] and H.rel_fro(got_lse, want_lse) < H.TOL[dtype]
-        # the reference's signature: the mask's tiles are classified on first
-        # sight, a causal mask then needs no tile tasks at all
+        # the reference's signature on a mask declared constant: its tiles were
+        # classified at the declaration, a causal mask needs no tile tasks at all
         got, got_lse, tasks, ntiles = _run(dtype, arrs, mask, head, seq, nb, grp, nkv, tile, hm.OP_TENSOR)
         assert tasks == 0
+        assert H.rel_fro(got, want) < H.TOL[dtype] and H.rel_fro(got_lse, want_lse) < H.TOL[dtype]
+        # ... and on a mask nothing was said about: the reference's submission
+        got, got_lse, tasks, ntiles = _run(dtype, arrs, mask, head, seq, nb, grp, nkv, tile,
+                                           hm.OP_TENSOR, declare=False)
+        assert tasks == ntiles * (seq // tile)
         assert H.rel_fro(got, want) < H.TOL[dtype] and H.rel_fro(got_lse, want_lse) < H.TOL[dtype]
     # the single-launch path on the same tiling, ragged last tile included
     got, got_lse, tasks, _ = _run(dtype, arrs, mask, head, seq, nb, grp, nkv, tile, hm.OP_HIP,
@@ -199,7 +207,7 @@ def _read_out(dtype, A, lse, head, seq):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["bf16", "fp32"])
-def test_reference_signature_caches_the_mask_classes_and_drops_them_on_a_write(oracle, dtype):
+def test_reference_signature_uses_the_classes_of_a_declared_mask_and_drops_them_on_a_write(oracle, dtype):
     head, seq, nb, grp, nkv, tile = 64, 256, 2, 1, 2, 64
     arrs, (qf, kf, vf) = _case(dtype, head, seq, nb, grp, nkv, seed=21)
     s5, b5 = [head, seq, nb, grp, nkv], [head, tile, 1, 1, 1]
@@ -209,55 +217,126 @@ def test_reference_signature_caches_the_mask_classes_and_drops_them_on_a_write(o
     window = np.abs(i[None, :] - i[:, None]) <= 40
     n_t = seq // tile
     slabs = nb * grp * nkv
+    every_pair = slabs * n_t * n_t
 
     def run(M, mask_bool):
+        """(tile tasks, look-ups that found classes, look-ups that did not,
+        blocking classifications) of one call with the reference's signature"""
         A, lse = _outputs(dtype, s5, b5)
-        tasks0, (h0, m0) = hm.tasks_submitted(dtype), hm.mask_cache_stats()
+        tasks0, (h0, m0), c0 = hm.tasks_submitted(dtype), hm.mask_cache_stats(), hm.mask_classifications()
         hm.flash_sdpa_fwd(hm.OP_TENSOR, T["K"], T["Q"], M, lse, T["V"], A)
-        (h1, m1) = hm.mask_cache_stats()
+        (h1, m1), c1 = hm.mask_cache_stats(), hm.mask_classifications()
         got, got_lse = _read_out(dtype, A, lse, head, seq)
         want, want_lse = oracle.sdpa_vanilla(kf, qf, vf, mask_bool, k_tile=tile)
         assert H.rel_fro(got, want) < H.TOL[dtype] and H.rel_fro(got_lse, want_lse) < H.TOL[dtype]
-        return hm.tasks_submitted(dtype) - tasks0, h1 - h0, m1 - m0
+        return hm.tasks_submitted(dtype) - tasks0, h1 - h0, m1 - m0, c1 - c0
 
     arr, M = _mask_tensor(dtype, causal, tile)
     M.from_array(arr)
-    # first sight: classified (a miss); the causal rule: no tile tasks, one
-    # task of the whole-grid codelet instead (all slabs have the same extents)
+    # nothing said about the mask: the reference's submission, and the call
+    # never classifies anything itself
+    assert run(M, causal) == (every_pair, 0, 1, 0)
+    # declared constant: classified once, there and then; the causal rule needs
+    # no tile tasks, one task of the whole-grid codelet instead (all slabs have
+    # the same extents)
+    c0 = hm.mask_classifications()
+    hm.mask_declare_constant(M)
+    assert hm.mask_classifications() - c0 == 1
     grid0 = hm.grid_tasks_submitted(dtype)
-    assert run(M, causal) == (0, 0, 1)
+    assert run(M, causal) == (0, 1, 0, 0)
     assert hm.grid_tasks_submitted(dtype) - grid0 == 1
     assert hm.grid_codelet_name(dtype) == "nntile_sdpa_fwd_grid_hip_" + dtype
-    # the same mask again: found, nothing re-read
-    assert run(M, causal) == (0, 1, 0)
-    assert run(M, causal) == (0, 1, 0)
-    # the mask is rewritten with a window: the classes are dropped, the result
-    # follows the new contents, pairs the window hides are not submitted and
-    # the others take the tile path (their tiles are MIXED) or the open path
+    assert run(M, causal) == (0, 1, 0, 0)
+    # the mask is rewritten through the runtime with a window: the classes are
+    # dropped with the write, the call goes back to the reference's submission
+    # and follows the new contents
     arr_w, _ = _mask_tensor(dtype, window, tile)
     M.from_array(arr_w)
-    tasks, hits, misses = run(M, window)
-    assert (hits, misses) == (0, 1)
+    assert run(M, window) == (every_pair, 0, 1, 0)
+    # declared again: pairs the window hides are not submitted, the others take
+    # the tile path (their tiles are MIXED) or the open path
+    hm.mask_declare_constant(M)
+    tasks, hits, misses, classified = run(M, window)
+    assert (hits, misses, classified) == (1, 0, 0)
     live = sum(1 for q in range(n_t) for k in range(n_t)
                if window[q * tile:(q + 1) * tile, k * tile:(k + 1) * tile].any())
     mixed = sum(1 for q in range(n_t) for k in range(n_t)
                 if window[q * tile:(q + 1) * tile, k * tile:(k + 1) * tile].any()
                 and not window[q * tile:(q + 1) * tile, k * tile:(k + 1) * tile].all())
     assert live < n_t * n_t and 0 < tasks <= slabs * mixed
-    assert run(M, window)[1:] == (1, 0)
-    # a writer got the tiles (same contents): classified again, same answer
+    # a writer got the tiles (same contents): dropped again
     M.mark_written()
-    assert run(M, window)[1:] == (0, 1)
-    # back to the causal contents
-    M.from_array(arr)
-    assert run(M, causal) == (0, 0, 1)
+    assert run(M, window)[1:] == (0, 1, 0)
+    # forgotten on request
+    hm.mask_declare_constant(M)
+    assert run(M, window)[1:] == (1, 0, 0)
+    hm.mask_forget(M)
+    assert run(M, window) == (every_pair, 0, 1, 0)
     # another tensor, freed and re-created in between (its memory may be
     # the one the freed tensor had): never served from the old entry
+    hm.mask_declare_constant(M)
     for mask_bool in (window, causal, window):
         arr2, M2 = _mask_tensor(dtype, mask_bool, tile)
         M2.from_array(arr2)
-        assert run(M2, mask_bool)[1:] == (0, 1)
+        assert run(M2, mask_bool)[1:] == (0, 1, 0)
+        hm.mask_declare_constant(M2)
+        assert run(M2, mask_bool)[1:] == (1, 0, 0)
         del M2
+
+
+@pytest.mark.gpu
+def test_a_mask_rewritten_behind_the_runtimes_back_is_honoured(oracle):
+    """The mask's tiles are overwritten by a kernel the runtime knows nothing
+    about (the transpose kernel of the C ABI, launched by the test on the
+    tiles' device addresses): the next call with the reference's signature
+    reads the mask as it then is, because an undeclared mask is never
+    classified ahead of time."""
+    import ctypes
+    import torch
+    from nntile_amd import hip_sdpa
+    dtype, head, seq, nb, grp, nkv, tile = "bf16", 64, 256, 2, 1, 2, 128
+    arrs, (qf, kf, vf) = _case(dtype, head, seq, nb, grp, nkv, seed=23)
+    s5, b5 = [head, seq, nb, grp, nkv], [head, tile, 1, 1, 1]
+    T = {n: hm.Tensor(dtype, s5, b5).from_array(arrs[n]) for n in ("K", "Q", "V")}
+    causal = synth.causal_mask(seq, seq)
+    i = np.arange(seq)
+    window = np.abs(i[None, :] - i[:, None]) <= 40
+    arr, M = _mask_tensor(dtype, causal, tile)
+    M.from_array(arr)
+
+    def run(mask_bool):
+        A, lse = _outputs(dtype, s5, b5)
+        hm.flash_sdpa_fwd(hm.OP_TENSOR, T["K"], T["Q"], M, lse, T["V"], A)
+        got, got_lse = _read_out(dtype, A, lse, head, seq)
+        want, want_lse = oracle.sdpa_vanilla(kf, qf, vf, mask_bool, k_tile=tile)
+        return H.rel_fro(got, want), H.rel_fro(got_lse, want_lse)
+
+    assert max(run(causal)) < H.TOL[dtype]
+    # tile (kt, qt) of the mask is Fortran [k, q] = the transpose of the C-ordered
+    # [k, q] block the test builds; dst = 1.0 * src^T writes it in place
+    add = np.where(window, 0.0, -np.inf).astype(np.float32)          # [q, k]
+    n_t = seq // tile
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # (the calls above are blocking: nothing of the runtime's is in flight)
+    keep = []
+    for qt in range(n_t):
+        for kt in range(n_t):
+            block = add[qt * tile:(qt + 1) * tile, kt * tile:(kt + 1) * tile]    # [q, k]
+            src = torch.from_numpy(np.ascontiguousarray(block.T)).to(torch.bfloat16).cuda()   # C [k, q]
+            ptr, nbytes = hm.tile_ptr(M, kt + qt * n_t)
+            assert nbytes == tile * tile * 2
+            # src as Fortran [q, k] (m = q, n = k) -> dst Fortran [k, q]
+            rc = hip_sdpa.lib().nntile_hip_transpose_bf16(stream, tile, tile, ctypes.c_float(1.0),
+                                                          ctypes.c_void_p(src.data_ptr()),
+                                                          ctypes.c_void_p(ptr))
+            assert rc == 0
+            keep.append(src)
+    torch.cuda.synchronize()
+    assert max(run(window)) < H.TOL[dtype]
+    # the same write behind a DECLARED mask breaks the caller's contract, and
+    # the caller's remedy is to say so before writing: forget, write, declare
+    hm.mask_declare_constant(M)
+    assert max(run(window)) < H.TOL[dtype]
 
 
 @pytest.mark.gpu
@@ -268,10 +347,12 @@ def test_reference_signature_with_a_bias_mask_is_the_reference_submission_bit_fo
     i = np.arange(seq)
     bias = (-0.25 * np.abs(i[:, None] - i[None, :]) - 0.25).astype(np.float32)
     outs = []
-    for op in (hm.OP_PAIRS, hm.OP_TENSOR, hm.OP_TENSOR):
+    for declare, op in ((False, hm.OP_PAIRS), (False, hm.OP_TENSOR), (True, hm.OP_TENSOR)):
         T = {n: hm.Tensor(dtype, s5, b5).from_array(arrs[n]) for n in ("K", "Q", "V")}
         arr, M = _mask_tensor(dtype, np.ones((seq, seq), bool), tile, values=bias)
         M.from_array(arr)
+        if declare:
+            hm.mask_declare_constant(M)
         A, lse = _outputs(dtype, s5, b5)
         before = hm.tasks_submitted(dtype)
         hm.flash_sdpa_fwd(op, T["K"], T["Q"], M, lse, T["V"], A)

@@ -139,6 +139,8 @@ def _run(op, dtype, data, lse, add_mask, shape5, base5, grads0=None, mask_mode=0
         pairs = hm.flash_sdpa_bwd(op, T["K"], T["Q"], T["V"], T["A"], T["dA"], M, L, T["dK"], T["dQ"],
                                   T["dV"], offset=offset)
     else:
+        if op == hm.OP_TENSOR:
+            hm.mask_declare_constant(M)     # what the layer says once after building its mask
         hm.flash_sdpa_bwd(op, T["K"], T["Q"], T["V"], T["A"], T["dA"], M, L, T["dK"], T["dQ"], T["dV"])
         pairs = hm.tasks_submitted_bwd(dtype) - before
     out = [_flat(_values(T[n].to_array(), dtype), head, seq) for n in ("dK", "dQ", "dV")]
@@ -296,8 +298,9 @@ def test_classified_submission_skips_hidden_tile_pairs(oracle, dtype, kind, offs
         assert H.rel_fro(g, w) < tol, n
         assert H.rel_fro(g, r) < tol, n
     if offset == 0:
-        # the reference's signature classifies the mask itself (rule key <= query)
-        # and submits the same calls: same bits, and only MIXED pairs as tile tasks
+        # the reference's signature on the mask declared constant (classified
+        # against the rule key <= query) submits the same calls: same bits, and
+        # only MIXED pairs as tile tasks
         dflt, tile_tasks, _ = _run(hm.OP_TENSOR, dtype, data, lse, add, shape5, base5)
         for g, d, n in zip(got, dflt, ("dK", "dQ", "dV")):
             assert np.array_equal(g, d), n
