@@ -148,7 +148,7 @@ class PowerSampler:
         return round(sum(tail) / len(tail), 0) if tail else None
 
 
-def bench_prefill(cfg, steps, warmup, zeros=False, settle_s=0.0, one_launch=True):
+def bench_prefill(cfg, steps, warmup, zeros=False, settle_s=0.0, one_launch=True, more_flags=0):
     """The tensor-level call over cfg's whole tile grid (analytic causal mask,
     hidden tile pairs skipped, overwrite mode): one fused launch over all
     sequence tiles of all slabs of the batch grid (one_launch=False: one
@@ -178,12 +178,12 @@ def bench_prefill(cfg, steps, warmup, zeros=False, settle_s=0.0, one_launch=True
     if one_launch and cfg.calls * nt <= h.MAX_TILES:
         cat = lambda i: [t for slab in keep for t in slab[i]]
         plans.append(h.plan_grid(cat(1), cat(0), cat(4), cat(2), cat(3), cfg.q_seq, cfg.k_seq,
-                                 cfg.seq_tile, cfg.seq_tile, h.MASK_CAUSAL, flags=h.OVERWRITE,
-                                 n_slabs=cfg.calls))
+                                 cfg.seq_tile, cfg.seq_tile, h.MASK_CAUSAL,
+                                 flags=h.OVERWRITE | more_flags, n_slabs=cfg.calls))
     else:
         for Q, K, V, A, lse in keep:
             plans.append(h.plan_grid(K, Q, lse, V, A, cfg.q_seq, cfg.k_seq, cfg.seq_tile,
-                                     cfg.seq_tile, h.MASK_CAUSAL, flags=h.OVERWRITE))
+                                     cfg.seq_tile, h.MASK_CAUSAL, flags=h.OVERWRITE | more_flags))
     del q_all, k_all, v_all
 
     def step():
@@ -804,7 +804,7 @@ def main():
                     help="with --only power_context: a shared library exporting nntile_hip_probe_mfma "
                          "(the matrix instruction alone); not part of the product")
     ap.add_argument("--only", default=None,
-                    help="run only this leg (for profiling): prefill | cfg5 | cfg2 | decode | decode_separate_merge | decode_wide | "
+                    help="run only this leg (for profiling): prefill | prefill_128_queries | cfg5 | cfg2 | decode | decode_separate_merge | decode_wide | "
                          "reference_api | reference_grid | power_context | copy_context | backward | backward_slabs | rope | transpose | accumulate | "
                          "kv_cache | copy")
     args = ap.parse_args()
@@ -830,6 +830,10 @@ def main():
     show = lambda r: print(json.dumps({k: (round(v, 4) if isinstance(v, float) else v)
                                        for k, v in r.items()}))
     legs = {"prefill": lambda: bench_prefill(cfg3, args.steps, args.warmup),
+            "prefill_128_queries": lambda: bench_prefill(cfg3, args.steps, args.warmup,
+                                                         more_flags=h.FORM_SHARED),
+            "cfg5_128_queries": lambda: bench_prefill(BY_NAME["cfg5_long_seq_bf16"], args.steps,
+                                                      args.warmup, more_flags=h.FORM_SHARED),
             "cfg5": lambda: bench_prefill(BY_NAME["cfg5_long_seq_bf16"], args.steps, args.warmup),
             "cfg2": lambda: bench_prefill(BY_NAME["cfg2_gpt2_small_fp32"], args.steps, args.warmup),
             "cfg2_per_slab": lambda: bench_prefill(BY_NAME["cfg2_gpt2_small_fp32"], args.steps,

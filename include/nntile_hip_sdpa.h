@@ -51,6 +51,12 @@ extern "C" {
  * steps (SPLIT).  Both set, or a 16-bit call: ignored. */
 #define NNTILE_HIP_SDPA_FORM_SHARED 0x100
 #define NNTILE_HIP_SDPA_FORM_SPLIT  0x200
+/* 16-bit tile and grid calls with an analytic mask, head 64 or 128, for tests
+ * and tuning: workgroups of 256 queries (eight wavefronts, one workgroup per
+ * CU) instead of 128 (four, two per CU).  Without it a launch picks the form
+ * from its size (256 queries at head 128 when every CU gets two workgroups);
+ * NNTILE_HIP_SDPA_FORM_SHARED keeps such a call at 128 queries. */
+#define NNTILE_HIP_SDPA_FORM_WIDE   0x4000
 /* decode calls, for tests and tuning: merge the key splits in a second launch
  * instead of inside the main one (SEPARATE_MERGE); exchange the partials of
  * the in-launch merge through device-scope fences whatever XCD the

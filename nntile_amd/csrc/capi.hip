@@ -64,6 +64,10 @@ static int prefill_form(int32_t flags)
 {
     const bool shared = (flags & NNTILE_HIP_SDPA_FORM_SHARED) != 0;
     const bool split = (flags & NNTILE_HIP_SDPA_FORM_SPLIT) != 0;
+    if(flags & NNTILE_HIP_SDPA_FORM_WIDE)
+    {
+        return 8;       // 16-bit kernels: 256-query workgroups
+    }
     return shared == split ? 0 : (shared ? 1 : 2);
 }
 

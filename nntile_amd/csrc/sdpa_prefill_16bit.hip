@@ -40,7 +40,7 @@
 namespace nntile_hip
 {
 
-constexpr int kQRows = 128;     // queries per workgroup
+constexpr int kQRows = 128;     // queries per workgroup of four wavefronts
 constexpr int kKeys = 64;       // keys per step
 constexpr int kThreads = 256;
 constexpr unsigned kCUsPerXCD = 32;   // MI355X: 256 CUs in 8 XCDs
@@ -83,11 +83,17 @@ extern "C" int nntile_hip_debug_pf_trace(unsigned long long *host)
 #define PF_NOTE(i, v)
 #endif
 
-template<typename T, int HEAD, int MODE>
-__global__ __launch_bounds__(kThreads, 2)
+// WAVES: wavefronts per workgroup, 32 queries each.  4: two workgroups share a
+// CU.  8 (analytic masks, head 64 and 128): one workgroup of 256 queries per
+// CU, whose eight wavefronts share every K/V step - a CU then brings each step
+// into LDS once where two workgroups of four bring it twice.
+template<typename T, int HEAD, int MODE, int WAVES = 4>
+__global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1)
 void sdpa_prefill_16bit_kernel(const PrefillParams p)
 {
     PF_STAMP(0);
+    constexpr int kQRows = WAVES * 32;
+    constexpr int kThreads = WAVES * 64;
     typedef typename T::vec8 vec8;
     constexpr int KSTEPS = HEAD / 16;       // MFMA steps along head for S
     constexpr int DBLOCKS = HEAD / 32;      // 32-row blocks of O^T
@@ -96,12 +102,14 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     constexpr int RPL = 16 / CPR;           // rows per 256-byte line of LDS banks
     constexpr int ROWS_PER_LOAD = 1024 / RB;   // rows one load instruction fills
     constexpr int LOADS = kKeys / ROWS_PER_LOAD;  // load instructions per K (or V) step
-    constexpr int LOADS_PER_WAVE = LOADS / 4;
+    constexpr int LOADS_PER_WAVE = LOADS / WAVES;
     constexpr int K_BYTES = kKeys * RB;
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
-    static_assert(LOADS_PER_WAVE == 1 || LOADS_PER_WAVE == 2 || LOADS_PER_WAVE == 4,
+    static_assert(LOADS_PER_WAVE * WAVES == LOADS
+            && (LOADS_PER_WAVE == 1 || LOADS_PER_WAVE == 2 || LOADS_PER_WAVE == 4),
             "head size does not fit this tiling");
+    static_assert(WAVES == 4 || (WAVES == 8 && !EXPLICIT), "eight wavefronts: analytic masks only");
 
     // Separate arrays, not one: the compiler then knows that the loads
     // streaming into one of them cannot alias the reads of the others and
@@ -133,7 +141,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // workgroup shares its CU with the shortest of the first 64.
     const int q_blocks = p.n_q_tiles * p.q_blocks_per_tile;
     unsigned wg = blockIdx.x;
-    if(gridDim.x >= 8u * 2u * kCUsPerXCD)
+    if(WAVES == 4 && gridDim.x >= 8u * 2u * kCUsPerXCD)
     {
         const unsigned i = wg >> 3;
         if(i >= kCUsPerXCD && i < 2u * kCUsPerXCD)
@@ -1013,17 +1021,6 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                     return;
                 }
                 const int i = slot_idx(sl);
-#ifdef NNTILE_PF_KO_LDSREAD     // (power attribution only: wrong results)
-                opnd[sl] = qf[i % KSTEPS];
-                return;
-#endif
-#ifdef NNTILE_PF_KO_HALFREAD    // (every second operand read only)
-                if(sl & 1)
-                {
-                    opnd[sl] = opnd[sl - 1];
-                    return;
-                }
-#endif
                 if(slot_kind(sl) == 1)
                 {
                     if(DO_S)
@@ -1057,13 +1054,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                 const int k = it / 3, r = it % 3;
                 if(r < 2)
                 {
-#if defined(NNTILE_PF_KO_EXP)
-                    pe[r] = fmaf(s_cur[2 * k + r], c, -mc);
-#elif defined(NNTILE_PF_KO_SOFTMAX)
-                    pe[r] = s_cur[2 * k + r];
-#else
                     pe[r] = fast_exp2(fmaf(s_cur[2 * k + r], c, -mc));
-#endif
                 }
                 else
                 {
@@ -1102,11 +1093,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                     o[db] = T::mfma(opnd[sl], __builtin_bit_cast(vec8, praw), o[db]);
                 }
                 // the softmax items are spread over the slots 1 .. NSLOT-1
-#ifdef NNTILE_PF_KO_ITEMS
-                if(false)
-#else
                 if(DO_SM && sl >= 1)
-#endif
                 {
 #pragma unroll
                     for(int it = (sl - 1) * NITEM / (NSLOT - 1);
@@ -1115,23 +1102,16 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
                         item(it);
                     }
                 }
-#ifndef NNTILE_PF_KO_DMA
                 if(DO_FETCH && (sl & 1))
                 {
                     fetch_piece(sl >> 1);
                 }
-#endif
                 __builtin_amdgcn_sched_barrier(0);
             }
             rescale_pending = false;
             if(DO_SM)
             {
-#if defined(NNTILE_PF_KO_EXP) || defined(NNTILE_PF_KO_SOFTMAX) || defined(NNTILE_PF_KO_ITEMS) \
-    || defined(NNTILE_PF_KO_LDSREAD)
-                if(false)       // (the knocked-out variants never redo a sub-block)
-#else
                 if(__builtin_amdgcn_ballot_w64(!(rs <= kLazyLimit)) != 0)
-#endif
                 {
                     float mx = s_cur[0];
 #pragma unroll
@@ -1323,7 +1303,9 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         // any more after the last barrier) so that they leave as whole rows,
         // 16 bytes per lane, instead of 8-byte pieces 2*HEAD bytes apart.
         // 16-byte chunk c of row r sits at chunk position c ^ (r % CPR).
-        char *xch = (wave < 2 ? lds_k0 : lds_k1) + (wave & 1) * 32 * RB;
+        // (two wavefronts per buffer: K0, K1, then V0, V1 for wavefronts 4 to 7)
+        char *xch = ((wave >> 1) == 0 ? lds_k0 : (wave >> 1) == 1 ? lds_k1
+                : (wave >> 1) == 2 ? lds_v0 : lds_v1) + (wave & 1) * 32 * RB;
 #pragma unroll
         for(int db = 0; db < DBLOCKS; ++db)
         {
@@ -1396,8 +1378,9 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
 
 template<typename T, int HEAD>
 static int launch_mode(hipStream_t stream, const PrefillParams &p, int mode,
-        dim3 grid)
+        dim3 grid, bool wide)
 {
+    constexpr int kThreads = 256;
     switch(mode)
     {
         case NNTILE_HIP_MASK_ADDITIVE:
@@ -1406,11 +1389,29 @@ static int launch_mode(hipStream_t stream, const PrefillParams &p, int mode,
                     stream, p);
             break;
         case NNTILE_HIP_MASK_NONE:
+            if constexpr(HEAD >= 64)
+            {
+                if(wide)
+                {
+                    hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
+                                NNTILE_HIP_MASK_NONE, 8>), grid, dim3(512), 0, stream, p);
+                    break;
+                }
+            }
             hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
                         NNTILE_HIP_MASK_NONE>), grid, dim3(kThreads), 0,
                     stream, p);
             break;
         case NNTILE_HIP_MASK_CAUSAL:
+            if constexpr(HEAD >= 64)
+            {
+                if(wide)
+                {
+                    hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
+                                NNTILE_HIP_MASK_CAUSAL, 8>), grid, dim3(512), 0, stream, p);
+                    break;
+                }
+            }
             hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
                         NNTILE_HIP_MASK_CAUSAL>), grid, dim3(kThreads), 0,
                     stream, p);
@@ -1569,7 +1570,24 @@ template<typename T>
 int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
         int mode, void *scan_scratch, size_t scan_scratch_bytes)
 {
-    p.q_blocks_per_tile = (int)((p.q_tile + kQRows - 1) / kQRows);
+    // 256-query workgroups (eight wavefronts, one workgroup a CU): when asked
+    // for (p.form == 8), and by themselves where they measured faster - head
+    // 128, whole 256-query blocks, and enough of them that every CU gets two
+    // under a causal mask (one workgroup a CU has nobody to share the CU with
+    // while it starts and ends, and a causal launch of one round is set by its
+    // longest workgroup), or a whole number of rounds without a mask.
+    // p.form == 1 keeps the 128-query form.
+    const bool can_wide = (head == 64 || head == 128)
+        && (mode == NNTILE_HIP_MASK_NONE || mode == NNTILE_HIP_MASK_CAUSAL);
+    bool wide = can_wide && p.form == 8;
+    if(can_wide && p.form == 0 && head == 128 && (p.q_tile % 256 == 0 || p.n_q_tiles == 1))
+    {
+        const int64_t n_w = (int64_t)p.batch * p.n_slabs * p.n_q_tiles * ((p.q_tile + 255) / 256);
+        wide = mode == NNTILE_HIP_MASK_CAUSAL ? n_w >= 512
+            : (n_w >= 256 && (n_w % 256 == 0 || n_w >= 1024));
+    }
+    const int q_rows = wide ? 256 : kQRows;
+    p.q_blocks_per_tile = (int)((p.q_tile + q_rows - 1) / q_rows);
     p.k_blocks_per_tile = (int)((p.k_tile + kKeys - 1) / kKeys);
     const int64_t batch_all = (int64_t)p.batch * p.n_slabs;
     const int64_t n_wg = batch_all * p.n_q_tiles * p.q_blocks_per_tile;
@@ -1588,11 +1606,11 @@ int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
     switch(head)
     {
         case 32:
-            return launch_mode<T, 32>(stream, p, mode, grid);
+            return launch_mode<T, 32>(stream, p, mode, grid, false);
         case 64:
-            return launch_mode<T, 64>(stream, p, mode, grid);
+            return launch_mode<T, 64>(stream, p, mode, grid, wide);
         case 128:
-            return launch_mode<T, 128>(stream, p, mode, grid);
+            return launch_mode<T, 128>(stream, p, mode, grid, wide);
         default:
             return NNTILE_HIP_EUNSUPPORTED;
     }

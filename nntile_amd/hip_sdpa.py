@@ -21,6 +21,7 @@ MAX_TILES = 64
 BWD_MAX_TILES = 32
 OVERWRITE = 1
 FORM_SHARED, FORM_SPLIT = 0x100, 0x200     # fp32 calls: fix the workgroup shape (tests, tuning)
+FORM_WIDE = 0x4000                         # 16-bit analytic-mask calls: 256-query workgroups
 # decode calls (tests, tuning): merge the key splits in a second launch; exchange
 # the partials of the in-launch merge through device-scope fences
 DECODE_SEPARATE_MERGE, DECODE_FENCED = 0x400, 0x800
