@@ -95,7 +95,15 @@ enum nntile_hip_mask_mode
  * mask is 1 MiB or larger the 16-bit variants scan it once per call with a
  * small kernel of their own and keep what they found (16 bytes per 128
  * queries and key range) there, instead of letting the workgroups of every
- * batch entry scan the same rows.  Same result, bit for bit. */
+ * batch entry scan the same rows.  Same result, bit for bit.
+ *
+ * SIZE OF scratch_lse: the call has no argument for it and takes it to be
+ * what the reference registers, seq * batch floats.  Pass NULL or a buffer of
+ * at least seq * batch * 4 bytes - never a smaller dummy: the device would
+ * write past its end.  (The codelet bodies of section 6 know the size of
+ * their scratch buffer from its interface and leave a smaller one alone; a
+ * pointer that is not 8-byte aligned is left alone as well.  The fp32
+ * variant never touches it.) */
 int nntile_hip_flash_sdpa_fwd_bf16(void *stream, int64_t seq, int64_t head,
         int64_t batch, const uint16_t *K, const uint16_t *Q,
         const uint16_t *mask, float *scratch_lse, const uint16_t *V,
@@ -314,7 +322,7 @@ int nntile_hip_sdpa_fwd_decode_fp16(void *stream, const nntile_hip_sdpa_tile_arg
  * NNTILE_HIP_EWORKSPACE and a line on stderr.  The array's address on the
  * current device is looked up on the first call made with that device current
  * (make that call outside a capture); the stream must belong to the current
- * device.  All calls on one GPU share the array: two of them in flight at the
+ * device - a stream of another GPU is refused with NNTILE_HIP_EINVAL.  All calls on one GPU share the array: two of them in flight at the
  * same time (different streams) race, calls on one stream do not. */
 #define NNTILE_HIP_DECODE_STATIC_SCRATCH_BYTES (16u << 20)
 #define NNTILE_HIP_DTYPE_BF16 0

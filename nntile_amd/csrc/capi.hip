@@ -553,13 +553,32 @@ static std::atomic<void *> scratch_ptr[kMaxDevices];
 static std::mutex scratch_mutex;
 
 // Device address of `scratch` on the current device, resolved on the first
-// call per device.
-static int static_scratch(void **out)
+// call per device; `stream` must be a stream of that device.
+static int static_scratch(hipStream_t stream, void **out)
 {
     int dev = -1;
     if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
     {
         return NNTILE_HIP_ELAUNCH;
+    }
+    // The array of the CURRENT device is the one handed to the kernels, so a
+    // stream of another GPU would run them on an address of the wrong device:
+    // refused.  (A query only: legal on a capturing stream; the null stream
+    // reports the current device.)
+    if(stream != nullptr)
+    {
+        hipDevice_t stream_dev = -1;
+        if(hipStreamGetDevice(stream, &stream_dev) != hipSuccess)
+        {
+            (void)hipGetLastError();
+            return NNTILE_HIP_EINVAL;
+        }
+        if((int)stream_dev != dev)
+        {
+            std::fprintf(stderr, "nntile_hip_sdpa_fwd_decode_static: the stream belongs to "
+                    "device %d, the current device is %d\n", (int)stream_dev, dev);
+            return NNTILE_HIP_EINVAL;
+        }
     }
     void *ptr = scratch_ptr[dev].load(std::memory_order_acquire);
     if(ptr == nullptr)
@@ -608,7 +627,7 @@ static int decode_static_call(void *stream, int32_t dtype,
         return NNTILE_HIP_EWORKSPACE;
     }
     void *ws = nullptr;
-    const int rc = static_scratch(&ws);
+    const int rc = static_scratch(static_cast<hipStream_t>(stream), &ws);
     if(rc != NNTILE_HIP_OK)
     {
         return rc;

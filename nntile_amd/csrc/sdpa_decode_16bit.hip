@@ -87,6 +87,22 @@ __device__ __forceinline__ u32x2 dec_lds_read_tr16(const char *lds_ptr)
     return __builtin_bit_cast(u32x2, v);
 }
 
+// The wait of the K/V ring, counted by hand: vmcnt retires in issue order, so
+// "at most N outstanding" means everything but the N youngest loads is done.
+// What a wavefront issues, in order (f(i) = the VM_PER_STEP global->LDS loads
+// of key step i, m(i) = the KB ordinary loads of step i's mask values; the
+// compiler's own wait counting sees m, not f, which is inline asm):
+//   prologue   m(0) f(0) .. f(STAGES-2)
+//   step it    wait_vmcnt<(STAGES-2)*VM_PER_STEP>   -> f(it) and m(it) are done:
+//                  younger than them are only f(it+1) .. f(it+STAGES-2)
+//              mcur = m(it)   (the compiler adds vmcnt(0) here, as it knows of
+//                  no younger load: with two stages nothing is outstanding at
+//                  that point; with three or four it drains f(it+1).., one
+//                  step more than needed, for explicit masks only)
+//              m(it+1) f(it+STAGES-1)
+// so the most a wavefront ever has outstanding is (STAGES-1)*VM_PER_STEP + KB,
+// which must stay below the counter's 64 (checked where VM_PER_STEP is defined).
+// In the tail (fewer than STAGES-1 steps ahead) the wait is for everything.
 template<int N> __device__ __forceinline__ void wait_vmcnt()
 {
     static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
@@ -350,6 +366,8 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
     constexpr int K_BYTES = kDecKeys * RB;
     constexpr int STAGE_BYTES = 2 * K_BYTES;            // K then V
     constexpr int VM_PER_STEP = 2 * LOADS_PER_WAVE;     // load instructions a wave issues per step
+    static_assert((STAGES - 1) * VM_PER_STEP + kDecKeys / 16 < 64,
+            "the ring's loads and one step's mask loads must fit the 6-bit vmcnt");
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
     static_assert(LOADS_PER_WAVE >= 1, "head size too small for this tiling");
@@ -543,7 +561,7 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         return step_lo + (j >= n_local ? j - n_local : j);
     };
 
-    // Explicit mask: the raw values of a full step of an aligned mask - per
+    // Explicit mask: the raw values of a full step of the mask - per
     // block of 16 keys the lane's four consecutive keys, one 8-byte (additive)
     // or 4-byte (boolean) load - are requested one step ahead, BEFORE that
     // step's K/V loads are issued.  Waiting for a load also waits for every
@@ -556,9 +574,11 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         mnext[kb] = u32x2{0u, 0u};
     }
     bool mnext_wide = false;
-    const bool mask_aligned = EXPLICIT && (p.mask_ld % 4 == 0)
-        && (reinterpret_cast<uintptr_t>(p.mask)
-                % (MODE == NNTILE_HIP_MASK_ADDITIVE ? 8 : 4) == 0);
+    // (masks of any row length and start: the loads carry the alignment of one
+    // element, which global memory accepts)
+    const bool mask_aligned = EXPLICIT;
+    typedef u32x2 __attribute__((aligned(2))) u32x2_any;
+    typedef uint32_t __attribute__((aligned(1))) u32_any;
     auto mask_request = [&](int it_req)
     {
         mnext_wide = false;
@@ -574,12 +594,12 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
                 {
                     if(MODE == NNTILE_HIP_MASK_ADDITIVE)
                     {
-                        mnext[kb] = *reinterpret_cast<const u32x2 *>(
+                        mnext[kb] = *reinterpret_cast<const u32x2_any *>(
                                 static_cast<const uint16_t *>(p.mask) + at + 16 * kb);
                     }
                     else
                     {
-                        mnext[kb][0] = *reinterpret_cast<const uint32_t *>(
+                        mnext[kb][0] = *reinterpret_cast<const u32_any *>(
                                 static_cast<const uint8_t *>(p.mask) + at + 16 * kb);
                     }
                 }

@@ -535,19 +535,23 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         mraw[i] = 0;
     }
     const int64_t mask_row = (int64_t)(q_ok ? my_q : 0) * p.mask_ld;
-    const bool mask_wide = EXPLICIT && (p.mask_ld % 4 == 0)
-        && (reinterpret_cast<uintptr_t>(p.mask) % 8 == 0);
+    // (every full step of any mask: the wide loads below carry the alignment
+    // of one element, and global memory takes unaligned accesses - a row
+    // length that is not a multiple of 4 costs some loads a second cache
+    // line, not a load per element)
+    const bool mask_wide = EXPLICIT;
     // loads of the mask values of key step kb (a full step) into mraw
     auto mask_fetch = [&](int kb)
     {
         if(MODE == NNTILE_HIP_MASK_ADDITIVE)
         {
+            typedef u32x2 __attribute__((aligned(2))) u32x2_any;
             const uint16_t *mp = static_cast<const uint16_t *>(p.mask) + mask_row
                 + kb * kKeys + 4 * half;
 #pragma unroll
             for(int i = 0; i < 8; ++i)
             {
-                const u32x2 v = *reinterpret_cast<const u32x2 *>(
+                const u32x2 v = *reinterpret_cast<const u32x2_any *>(
                         mp + (i >> 2) * 32 + (i & 3) * 8);
                 mraw[2 * i] = v[0];
                 mraw[2 * i + 1] = v[1];
@@ -555,12 +559,13 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         }
         else if(MODE == NNTILE_HIP_MASK_BOOL)
         {
+            typedef uint32_t __attribute__((aligned(1))) u32_any;
             const uint8_t *mp = static_cast<const uint8_t *>(p.mask) + mask_row
                 + kb * kKeys + 4 * half;
 #pragma unroll
             for(int i = 0; i < 8; ++i)
             {
-                mraw[i] = *reinterpret_cast<const uint32_t *>(
+                mraw[i] = *reinterpret_cast<const u32_any *>(
                         mp + (i >> 2) * 32 + (i & 3) * 8);
             }
         }

@@ -83,3 +83,28 @@ def test_codelet_body_uses_its_scratch_buffer(oracle):
         outs.append((lse, A))
     assert torch.equal(outs[0][0], outs[1][0])
     assert torch.equal(outs[0][1].view(torch.int16), outs[1][1].view(torch.int16))
+
+
+def test_a_scratch_smaller_than_a_logsumexp_tile_is_refused_or_left_alone():
+    """The tile call cannot know the size of its scratch (it takes it to be a
+    logsumexp tile), so the Python wrapper refuses a smaller tensor before the
+    call; the codelet body reads the size from the buffer's interface and
+    leaves a smaller one untouched - same result as without it."""
+    seq, head, batch, dtype = 1024, 64, 2, "bf16"
+    (Q, K, V), _ = H.make_qkv(37, batch, seq, seq, head, dtype)
+    m = H.additive_mask(_mask("window", seq), dtype).cuda()
+    Kd, Qd, Vd = K.cuda(), Q.cuda(), V.cuda()
+    lse, A = H.fresh_outputs(batch, seq, head, dtype)
+    small = torch.full((batch * seq - 1,), float("nan"), device="cuda")
+    with pytest.raises(ValueError):
+        hip_sdpa.flash_sdpa_fwd(Kd, Qd, m, lse, Vd, A, scratch_lse=small)
+    torch.cuda.synchronize()
+    assert torch.isneginf(lse).all()          # nothing ran
+    lse0, A0 = H.fresh_outputs(batch, seq, head, dtype)
+    hip_sdpa.flash_sdpa_fwd_codelet(Kd, Qd, m, lse0, Vd, A0)
+    lse1, A1 = H.fresh_outputs(batch, seq, head, dtype)
+    tiny = torch.full((4,), float("nan"), device="cuda")      # less than the scan's table
+    hip_sdpa.flash_sdpa_fwd_codelet(Kd, Qd, m, lse1, Vd, A1, scratch_lse=tiny)
+    torch.cuda.synchronize()
+    assert torch.isnan(tiny).all()            # left alone
+    assert torch.equal(lse0, lse1) and torch.equal(A0.view(torch.int16), A1.view(torch.int16))

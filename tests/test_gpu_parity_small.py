@@ -175,6 +175,38 @@ def test_decode_entry_matches_oracle(oracle, dtype, q_seq, k_seq, n_batch, group
     assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("form", ["additive", "bool"])
+@pytest.mark.parametrize("q_seq,k_seq,shift,head", [(16, 1001, 0, 128), (5, 333, 1, 128), (16, 2050, 3, 64),
+                                                    (3, 67, 1, 128), (16, 1024, 1, 128), (7, 130, 0, 64)])
+def test_decode_explicit_masks_of_any_alignment(oracle, dtype, form, q_seq, k_seq, shift, head):
+    """Decode with a mask given as values that is not a causal one (holes and
+    hidden stretches, so that a wrong mask element changes the result), whose
+    rows are not a multiple of 4 elements, that starts `shift` elements into
+    its allocation, and whose last key step is ragged; both mask tile types."""
+    print("case decode mask", dtype, form, q_seq, k_seq, shift, head, flush=True)
+    n_batch, group, n_kv = 2, 4, 2
+    batch = n_batch * group * n_kv
+    (Q, K, V), f32 = H.make_qkv(29, batch, q_seq, k_seq, head, dtype, kv_batch=n_batch * n_kv)
+    i = np.arange(q_seq)[:, None]
+    j = np.arange(k_seq)[None, :]
+    mask = np.ascontiguousarray(((i * 5 + j) % 7 != 0) & ((j // 50) % 3 != (i % 3)) & (j >= i))
+    want, want_lse = _oracle(oracle, f32, mask, n_batch=n_batch, kv_repeat=group)
+    flat = (H.additive_mask(mask, dtype) if form == "additive" else torch.from_numpy(mask.copy())).reshape(-1)
+    room = torch.zeros(flat.numel() + 8, dtype=flat.dtype)
+    room[shift:shift + flat.numel()] = flat
+    m = room.cuda()[shift:shift + flat.numel()].view(q_seq, k_seq)
+    Kd, Qd, Vd = K.cuda(), Q.cuda(), V.cuda()
+    ws = torch.empty(hip_sdpa.decode_workspace_bytes(Kd, Qd, n_batch, group), dtype=torch.uint8,
+                     device="cuda")
+    lse, A = H.fresh_outputs(batch, q_seq, head, dtype)
+    mode = hip_sdpa.MASK_ADDITIVE if form == "additive" else hip_sdpa.MASK_BOOL
+    hip_sdpa.sdpa_fwd_decode(Kd, Qd, m, lse, Vd, A, mode, n_batch, group, ws)
+    torch.cuda.synchronize()
+    assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
+    assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+
+
 def test_decode_merges_into_running_pair(oracle):
     """Two decode calls over two halves of the cache == one call over all of it."""
     dtype, q_seq, k_seq, n_batch, group, n_kv, head = "bf16", 16, 512, 2, 4, 2, 128
@@ -462,6 +494,40 @@ def test_explicit_mask_scan_paths(oracle, dtype, form, q_seq, k_seq, pattern):
     got2, got2_lse = H.to_np(A2), H.to_np(lse2)
     assert np.all(got2[:, ~vis] == 0) and np.all(np.isneginf(got2_lse[:, ~vis]))
     assert np.array_equal(got2[:, vis], got[:, vis]) and np.array_equal(got2_lse[:, vis], got_lse[:, vis])
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("form", ["additive", "bool"])
+@pytest.mark.parametrize("head", [64, 128])
+@pytest.mark.parametrize("q_seq,k_seq,shift", [(130, 333, 0), (130, 1001, 0), (257, 1001, 1),
+                                               (64, 67, 3), (200, 130, 1), (128, 1024, 1)])
+def test_explicit_mask_rows_of_any_alignment(oracle, dtype, form, head, q_seq, k_seq, shift):
+    """Mask rows whose length is not a multiple of 4 elements, and a mask that
+    starts `shift` elements into its allocation: the full key steps still take
+    the wide mask loads (at the alignment of one element), only the ragged
+    last step goes element by element.  A band pattern, so that steps with
+    nothing masked, mixed steps and fully hidden steps all occur."""
+    print("case unaligned mask", dtype, form, head, q_seq, k_seq, shift, flush=True)
+    batch = 3
+    i = np.arange(q_seq)[:, None]
+    j = np.arange(k_seq)[None, :]
+    mask = np.ascontiguousarray((j <= (k_seq // 3 + 2 * i)) & ((i + j) % 11 != 0))
+    (Q, K, V), f32 = H.make_qkv(91, batch, q_seq, k_seq, head, dtype)
+    want, want_lse = _oracle(oracle, f32, mask)
+    flat = (H.additive_mask(mask, dtype) if form == "additive" else torch.from_numpy(mask.copy())).reshape(-1)
+    room = torch.zeros(flat.numel() + 8, dtype=flat.dtype)
+    room[shift:shift + flat.numel()] = flat
+    m = room.cuda()[shift:shift + flat.numel()].view(q_seq, k_seq)
+    assert m.is_contiguous() and m.data_ptr() % 8 == (shift * m.element_size()) % 8
+    mode = hip_sdpa.MASK_ADDITIVE if form == "additive" else hip_sdpa.MASK_BOOL
+    lse, A = H.fresh_outputs(batch, q_seq, head, dtype)
+    hip_sdpa.sdpa_fwd_tile(K.cuda(), Q.cuda(), m, lse, V.cuda(), A, mode, flags=hip_sdpa.OVERWRITE)
+    torch.cuda.synchronize()
+    got, got_lse = H.to_np(A), H.to_np(lse)
+    vis = mask.any(axis=1)
+    assert np.all(got[:, ~vis] == 0) and np.all(np.isneginf(got_lse[:, ~vis]))
+    assert H.rel_fro(got[:, vis], want[:, vis]) < H.TOL[dtype]
+    assert H.rel_fro(got_lse[:, vis], want_lse[:, vis]) < H.TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16"])

@@ -65,6 +65,69 @@ def test_static_scratch_decode_with_the_merge_inside_the_launch(oracle):
     _both(oracle, "bf16", 3, 900, 8, 2, 1, 128, 57, True)
 
 
+def _inputs(n_batch, group, n_kv, q_seq, k_seq, head, seed):
+    batch = n_batch * group * n_kv
+    (Q, K, V), _ = H.make_qkv(seed, batch, q_seq, k_seq, head, "bf16", kv_batch=n_batch * n_kv)
+    return K.cuda(), Q.cuda(), V.cuda(), batch
+
+
+def test_static_scratch_decode_allocates_nothing():
+    """Across a call (after the warm-up call that looks the array up) the
+    device's free memory as the runtime reports it, and what torch's allocator
+    holds, stay what they were - for the form with the merge in a launch of
+    its own and for the one with the merge inside the main launch."""
+    for n_batch in (2, 4):
+        Kd, Qd, Vd, batch = _inputs(n_batch, 4, 2, 16, 2048, 128, 60 + n_batch)
+        lse, A = H.fresh_outputs(batch, 16, 128, "bf16")
+        call = lambda: hip_sdpa.sdpa_fwd_decode_static(
+            Kd, Qd, None, lse, Vd, A, hip_sdpa.MASK_CAUSAL, n_batch, 4, causal_offset=2032,
+            flags=hip_sdpa.OVERWRITE)
+        call()
+        torch.cuda.synchronize()
+        free0, _ = torch.cuda.mem_get_info()
+        reserved0, allocated0 = torch.cuda.memory_reserved(), torch.cuda.memory_allocated()
+        for _ in range(3):
+            call()
+        torch.cuda.synchronize()
+        free1, _ = torch.cuda.mem_get_info()
+        assert free1 == free0
+        assert torch.cuda.memory_reserved() == reserved0
+        assert torch.cuda.memory_allocated() == allocated0
+
+
+@pytest.mark.parametrize("n_batch", [2, 4])
+def test_static_scratch_decode_under_stream_capture(n_batch):
+    """One call recorded into a graph, after a warm-up call outside the capture
+    (the look-up of the array's address is not legal inside one).  Replays
+    with eager work and synchronisations in between, each compared bit for
+    bit with the eager result."""
+    q_seq, k_seq, head, group = 16, 2048, 128, 4
+    Kd, Qd, Vd, batch = _inputs(n_batch, group, 2, q_seq, k_seq, head, 70 + n_batch)
+    offset = k_seq - q_seq
+    lse0, A0 = H.fresh_outputs(batch, q_seq, head, "bf16")
+    hip_sdpa.sdpa_fwd_decode_static(Kd, Qd, None, lse0, Vd, A0, hip_sdpa.MASK_CAUSAL, n_batch, group,
+                                    causal_offset=offset, flags=hip_sdpa.OVERWRITE)
+    torch.cuda.synchronize()
+    lse, A = H.fresh_outputs(batch, q_seq, head, "bf16")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        hip_sdpa.sdpa_fwd_decode_static(Kd, Qd, None, lse, Vd, A, hip_sdpa.MASK_CAUSAL, n_batch,
+                                        group, causal_offset=offset, flags=hip_sdpa.OVERWRITE)
+    small = _inputs(1, group, 2, 3, 500, head, 79)
+    for _ in range(3):
+        A.fill_(float("nan"))
+        lse.fill_(float("nan"))
+        # an eager call on another shape leaves its partials (and flags) in the array
+        lse_s, A_s = H.fresh_outputs(small[3], 3, head, "bf16")
+        hip_sdpa.sdpa_fwd_decode_static(small[0], small[1], None, lse_s, small[2], A_s,
+                                        hip_sdpa.MASK_CAUSAL, 1, group, causal_offset=497,
+                                        flags=hip_sdpa.OVERWRITE)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(A.view(torch.int16), A0.view(torch.int16)) and torch.equal(lse, lse0)
+
+
 def test_static_scratch_refuses_what_does_not_fit():
     # 64 rows x 4096 units x 1 split of bf16 partials alone are 64 MiB
     n_batch, group, n_kv, head, q_seq, k_seq = 1024, 4, 4, 128, 16, 8192
