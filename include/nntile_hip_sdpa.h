@@ -45,10 +45,13 @@ extern "C" {
  * A = 0.  Saves the fill of lse (wrappers/python/nntile/layer/sdpa.py:538-539)
  * and one read of A when the caller knows this is the first key tile. */
 #define NNTILE_HIP_SDPA_OVERWRITE 1
-/* fp32 tile and grid calls, for tests and tuning: fix the workgroup shape
- * instead of letting the size of the launch pick it - 128 queries sharing
- * every key step (SHARED), or 32 queries whose four wavefronts split the key
- * steps (SPLIT).  Both set, or a 16-bit call: ignored. */
+/* Tile and grid calls, for tests and tuning: fix the workgroup shape instead
+ * of letting the size of the launch pick it.  fp32: 128 queries sharing every
+ * key step (SHARED), or 32 queries whose four wavefronts split the key steps
+ * (SPLIT).  16-bit: 128 queries and four wavefronts (SHARED), or the same 128
+ * queries held by two groups of four wavefronts that take every second key
+ * step each and merge through LDS (SPLIT; head 64 and 128; what a launch of
+ * at most one workgroup per CU takes by itself).  Both set: ignored. */
 #define NNTILE_HIP_SDPA_FORM_SHARED 0x100
 #define NNTILE_HIP_SDPA_FORM_SPLIT  0x200
 /* 16-bit tile and grid calls with an analytic mask, head 64 or 128, for tests

@@ -59,7 +59,7 @@ static bool mode_ok(int mode)
     return mode >= NNTILE_HIP_MASK_ADDITIVE && mode <= NNTILE_HIP_MASK_BOOL;
 }
 
-// the workgroup shape a caller asked for (fp32 kernels): 0 none, 1 shared, 2 split
+// the workgroup shape a caller asked for: 0 none, 1 shared, 2 split, 8 wide (16-bit kernels)
 static int prefill_form(int32_t flags)
 {
     const bool shared = (flags & NNTILE_HIP_SDPA_FORM_SHARED) != 0;

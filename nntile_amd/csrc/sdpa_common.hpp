@@ -65,7 +65,7 @@ struct PrefillParams
     int32_t xcd_remap;            // 1: regroup workgroups so a slab stays on one XCD
     int32_t overwrite;            // 1: ignore the running pair, write every row
     int32_t form;                 // fp32 launcher: 0 pick by size, 1 shared key steps, 2 split key steps
-                                  // 16-bit launcher: 0 pick by size, 1 128-query workgroups, 8 256-query
+                                  // 16-bit launcher: 0 pick by size, 1 128-query workgroups, 2 the same with the key steps split over two groups of wavefronts, 8 256-query
     float scale;                  // 1/sqrt(head)
     const void *K[kMaxTiles];
     const void *V[kMaxTiles];

@@ -87,12 +87,19 @@ extern "C" int nntile_hip_debug_pf_trace(unsigned long long *host)
 // CU.  8 (analytic masks, head 64 and 128): one workgroup of 256 queries per
 // CU, whose eight wavefronts share every K/V step - a CU then brings each step
 // into LDS once where two workgroups of four bring it twice.
-template<typename T, int HEAD, int MODE, int WAVES = 4>
+template<typename T, int HEAD, int MODE, int WAVES = 4, int GROUPS = 1>
 __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1)
 void sdpa_prefill_16bit_kernel(const PrefillParams p)
 {
     PF_STAMP(0);
-    constexpr int kQRows = WAVES * 32;
+    // GROUPS == 2: the eight wavefronts are two groups of four; both groups
+    // hold the same 128 queries, group g takes the key steps g, g + 2, ...
+    // through a K/V ring of its own, and the two (maximum, sum, output)
+    // triples are merged through LDS before the epilogue.  For launches that
+    // have no second workgroup to put on a CU: two wavefronts per SIMD (one's
+    // softmax beside the other's MFMAs) and half the chain of dependent steps.
+    constexpr int QW = WAVES / GROUPS;      // wavefronts that share a key step
+    constexpr int kQRows = QW * 32;
     constexpr int kThreads = WAVES * 64;
     typedef typename T::vec8 vec8;
     constexpr int KSTEPS = HEAD / 16;       // MFMA steps along head for S
@@ -102,27 +109,33 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     constexpr int RPL = 16 / CPR;           // rows per 256-byte line of LDS banks
     constexpr int ROWS_PER_LOAD = 1024 / RB;   // rows one load instruction fills
     constexpr int LOADS = kKeys / ROWS_PER_LOAD;  // load instructions per K (or V) step
-    constexpr int LOADS_PER_WAVE = LOADS / WAVES;
+    constexpr int LOADS_PER_WAVE = LOADS / QW;
     constexpr int K_BYTES = kKeys * RB;
     constexpr bool EXPLICIT = (MODE == NNTILE_HIP_MASK_ADDITIVE
             || MODE == NNTILE_HIP_MASK_BOOL);
-    static_assert(LOADS_PER_WAVE * WAVES == LOADS
+    static_assert(LOADS_PER_WAVE * QW == LOADS
             && (LOADS_PER_WAVE == 1 || LOADS_PER_WAVE == 2 || LOADS_PER_WAVE == 4),
             "head size does not fit this tiling");
-    static_assert(WAVES == 4 || (WAVES == 8 && !EXPLICIT), "eight wavefronts: analytic masks only");
+    static_assert(GROUPS == 1 || (GROUPS == 2 && WAVES == 8), "two groups of four wavefronts");
+    static_assert(WAVES == 4 || (WAVES == 8 && (GROUPS == 2 || !EXPLICIT)),
+            "eight wavefronts on 256 queries: analytic masks only");
 
     // Separate arrays, not one: the compiler then knows that the loads
     // streaming into one of them cannot alias the reads of the others and
     // does not make those reads wait for the loads.  Key step g lives in
     // lds_k[g % 2] and lds_v[g % 2].
-    __shared__ __attribute__((aligned(1024))) char lds_k0[K_BYTES];
-    __shared__ __attribute__((aligned(1024))) char lds_k1[K_BYTES];
-    __shared__ __attribute__((aligned(1024))) char lds_v0[K_BYTES];
-    __shared__ __attribute__((aligned(1024))) char lds_v1[K_BYTES];
+    // (GROUPS == 2: group g's half of every array starts at g * K_BYTES; that
+    // offset is part of the lanes' read addresses and of the loads' targets)
+    __shared__ __attribute__((aligned(1024))) char lds_k0[K_BYTES * GROUPS];
+    __shared__ __attribute__((aligned(1024))) char lds_k1[K_BYTES * GROUPS];
+    __shared__ __attribute__((aligned(1024))) char lds_v0[K_BYTES * GROUPS];
+    __shared__ __attribute__((aligned(1024))) char lds_v1[K_BYTES * GROUPS];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int grp = GROUPS > 1 ? (tid >> 6) / QW : 0;      // which key steps
+    const int wave = (tid >> 6) - grp * QW;                 // which 32 queries
+    const int lds_grp_off = GROUPS > 1 ? __builtin_amdgcn_readfirstlane(grp) * K_BYTES : 0;
     const int col = lane & 31;      // query within the wavefront / row of a block
     const int half = lane >> 5;
 
@@ -389,7 +402,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
 #pragma unroll
         for(int ks = 0; ks < KSTEPS; ++ks)
         {
-            k_raddr[mb][ks] = (uint32_t)(r * RB
+            k_raddr[mb][ks] = (uint32_t)(grp * K_BYTES + r * RB
                     + ((2 * ks + half) ^ ((r / RPL) % CPR)) * 16);
         }
     }
@@ -410,7 +423,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         for(int db = 0; db < DBLOCKS; ++db)
         {
             const int c = 4 * db + 2 * dblk + (r4 >> 1);
-            v_raddr[db] = (uint32_t)(r * RB + (c ^ swz) * 16
+            v_raddr[db] = (uint32_t)(grp * K_BYTES + r * RB + (c ^ swz) * 16
                     + 8 * (r4 & 1));
         }
     }
@@ -433,7 +446,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     auto fetch_k = [&](const StepCursor &cur, char *dst_base)
     {
         // (wave index made visibly uniform: the LDS target goes into M0)
-        char *dst = dst_base
+        char *dst = dst_base + lds_grp_off
             + __builtin_amdgcn_readfirstlane(wave) * LOADS_PER_WAVE * 1024;
         if(cur.rows_left >= kKeys)
         {
@@ -458,7 +471,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     };
     auto fetch_v = [&](const StepCursor &cur, char *dst_base)
     {
-        char *dst = dst_base
+        char *dst = dst_base + lds_grp_off
             + __builtin_amdgcn_readfirstlane(wave) * LOADS_PER_WAVE * 1024;
         if(cur.rows_left >= kKeys)
         {
@@ -488,7 +501,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     };
 
     // Next step; the tile base pointers are re-read only when the tile changes.
-    auto advance = [&](StepCursor &cur)
+    auto advance_one = [&](StepCursor &cur)
     {
         cur.kb += 1;
         cur.rows_left -= kKeys;
@@ -508,6 +521,15 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             {
                 cur.rows_left = 0;
             }
+        }
+    };
+    // ... the next step of this wavefront's group
+    auto advance = [&](StepCursor &cur)
+    {
+        advance_one(cur);
+        if(GROUPS > 1)
+        {
+            advance_one(cur);
         }
     };
 
@@ -618,6 +640,10 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     StepCursor cur = {0, 0, tile_rows(0),
         static_cast<const char *>(p.K[k_tile0]) + slab(0),
         static_cast<const char *>(p.V[k_tile0]) + slab(0)};     // step being computed
+    if(GROUPS > 1 && grp == 1)
+    {
+        advance_one(cur);       // the second group starts at step 1
+    }
     StepCursor nxt = cur;                        // step being fetched
     // Leading steps that are complete (64 keys) and visible to every query of
     // the workgroup need no mask at all; they run in the pipelined loop below.
@@ -636,7 +662,23 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         {
             n_fast = min(n_fast, n_open);
         }
+        if(GROUPS > 1)
+        {
+            // counted in the group's own steps (its step j is step
+            // GROUPS * j + grp), and the same for both groups: the barriers of
+            // the pipelined loop are the workgroup's
+            n_fast /= GROUPS;
+            n_spread /= GROUPS;
+        }
         n_fast = n_fast >= 2 ? n_fast : 0;
+    }
+    // Rounds of the workgroup; from here on n_steps counts the group's own
+    // steps.  A group that has one step fewer than the other goes through the
+    // last round idle: every wavefront meets every barrier.
+    const int n_rounds = (n_steps + GROUPS - 1) / GROUPS;
+    if(GROUPS > 1)
+    {
+        n_steps = max(n_steps - grp + GROUPS - 1, 0) / GROUPS;
     }
     if(n_steps > 0)
     {
@@ -649,7 +691,7 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         }
         if(mask_wide && n_fast == 0 && cur.rows_left >= kKeys)
         {
-            mask_fetch(0);
+            mask_fetch(cur.kb);
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -679,9 +721,11 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         {
             mask_class = mask_classify();
         }
-        // nothing of this step is visible to this wavefront
-        const bool idle = EXPLICIT ? (mask_class == MASK_HIDDEN)
-            : ((MODE == NNTILE_HIP_MASK_CAUSAL) && (kg0 > wave_rel_lo + 31));
+        // nothing of this step is visible to this wavefront, or the step is
+        // the other group's last one and this group has none in this round
+        const bool idle = (GROUPS > 1 && g >= n_steps)
+            || (EXPLICIT ? (mask_class == MASK_HIDDEN)
+            : ((MODE == NNTILE_HIP_MASK_CAUSAL) && (kg0 > wave_rel_lo + 31)));
 
         // ---- loads of the next step into the other buffer ----------------------
         // (every wavefront passed the barrier that ended step g-1, so nobody
@@ -877,9 +921,9 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         }
         // mask values of the next step (this step's have been consumed)
         if(EXPLICIT && mask_wide && g + 1 < n_steps
-                && cur.rows_left - kKeys >= kKeys)
+                && cur.rows_left - GROUPS * kKeys >= kKeys)
         {
-            mask_fetch(cur.kb + 1);
+            mask_fetch(cur.kb + GROUPS);
         }
         NNTILE_PHASE(2)
 
@@ -1204,8 +1248,8 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             {
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __syncthreads();
-                char *kdst = (BUF ? lds_k1 : lds_k0) + wave_u * LOADS_PER_WAVE * 1024;
-                char *vdst = (BUF ? lds_v0 : lds_v1) + wave_u * LOADS_PER_WAVE * 1024;
+                char *kdst = (BUF ? lds_k1 : lds_k0) + lds_grp_off + wave_u * LOADS_PER_WAVE * 1024;
+                char *vdst = (BUF ? lds_v0 : lds_v1) + lds_grp_off + wave_u * LOADS_PER_WAVE * 1024;
                 body(Yes{}, Yes{}, Yes{}, Yes{}, BUF ? lds_k0 : lds_k1, 0,
                         BUF ? lds_v1 : lds_v0, 0, sb, sa, kdst, vdst);
                 c1 = c2;
@@ -1262,15 +1306,15 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     PF_STAMP(2);
     {
         int g = g_first;
-        if(g < n_steps && (g & 1))
+        if(g < n_rounds && (g & 1))
         {
             step(g, std::integral_constant<int, 1>{});
             g += 1;
         }
-        for(; g < n_steps; g += 2)
+        for(; g < n_rounds; g += 2)
         {
             step(g, std::integral_constant<int, 0>{});
-            if(g + 1 < n_steps)
+            if(g + 1 < n_rounds)
             {
                 step(g + 1, std::integral_constant<int, 1>{});
             }
@@ -1279,6 +1323,57 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     NNTILE_PHASE_DUMP()
     PF_STAMP(3);
     PF_NOTE(7, clock64() - pf_cycles0);     // shader-clock cycles between stamps 1 and 3
+
+    // ---- the second group hands its triple to the first -------------------------
+    // Through the K/V arrays, which nobody reads any more: wavefront w of the
+    // second group writes (O, maximum, sum) lane by lane into array w, its
+    // counterpart in the first group - same queries, same lanes - combines
+    // them with its own as two partial softmaxes are combined.
+    if constexpr(GROUPS > 1)
+    {
+        constexpr int NO = 16 * DBLOCKS;
+        static_assert(GROUPS == 1 || (NO + 2) * 256 <= K_BYTES * GROUPS - 32 * RB,
+                "the triple and the epilogue's staging rows share an array");
+        float *mrg = reinterpret_cast<float *>(wave == 0 ? lds_k0 : wave == 1 ? lds_k1
+                : wave == 2 ? lds_v0 : lds_v1) + lane;
+        __syncthreads();
+        if(grp == 1)
+        {
+#pragma unroll
+            for(int db = 0; db < DBLOCKS; ++db)
+            {
+#pragma unroll
+                for(int r = 0; r < 16; ++r)
+                {
+                    mrg[(16 * db + r) * 64] = o[db][r];
+                }
+            }
+            mrg[NO * 64] = m_run;
+            mrg[(NO + 1) * 64] = l_run;
+        }
+        __syncthreads();
+        if(grp == 1)
+        {
+            return;
+        }
+        const float m_other = mrg[NO * 64];
+        const float l_other = mrg[(NO + 1) * 64];
+        const float m_new = fmaxf(m_run, m_other);
+        // (a group that saw no visible key has maximum -inf and weight 0)
+        const float a_mine = (m_run == neg_inf()) ? 0.0f : fast_exp2((m_run - m_new) * c);
+        const float a_other = (m_other == neg_inf()) ? 0.0f : fast_exp2((m_other - m_new) * c);
+#pragma unroll
+        for(int db = 0; db < DBLOCKS; ++db)
+        {
+#pragma unroll
+            for(int r = 0; r < 16; ++r)
+            {
+                o[db][r] = o[db][r] * a_mine + mrg[(16 * db + r) * 64] * a_other;
+            }
+        }
+        l_run = l_run * a_mine + l_other * a_other;
+        m_run = m_new;
+    }
 
     // ---- epilogue: normalise, merge into the running (lse, A) ----------------
     const float l_tot = sum_across_halves(l_run);
@@ -1309,7 +1404,12 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         // 16 bytes per lane, instead of 8-byte pieces 2*HEAD bytes apart.
         // 16-byte chunk c of row r sits at chunk position c ^ (r % CPR).
         // (two wavefronts per buffer: K0, K1, then V0, V1 for wavefronts 4 to 7)
-        char *xch = ((wave >> 1) == 0 ? lds_k0 : (wave >> 1) == 1 ? lds_k1
+        // (two groups: wavefront w uses the end of array w, behind the triple
+        // it has just read - a neighbour may still be reading its own)
+        char *xch = GROUPS > 1
+            ? (wave == 0 ? lds_k0 : wave == 1 ? lds_k1 : wave == 2 ? lds_v0 : lds_v1)
+                + (K_BYTES * GROUPS - 32 * RB)
+            : ((wave >> 1) == 0 ? lds_k0 : (wave >> 1) == 1 ? lds_k1
                 : (wave >> 1) == 2 ? lds_v0 : lds_v1) + (wave & 1) * 32 * RB;
 #pragma unroll
         for(int db = 0; db < DBLOCKS; ++db)
@@ -1383,9 +1483,37 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
 
 template<typename T, int HEAD>
 static int launch_mode(hipStream_t stream, const PrefillParams &p, int mode,
-        dim3 grid, bool wide)
+        dim3 grid, bool wide, bool key_split)
 {
     constexpr int kThreads = 256;
+    if constexpr(HEAD >= 64)
+    {
+        if(key_split)
+        {
+            switch(mode)
+            {
+                case NNTILE_HIP_MASK_ADDITIVE:
+                    hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
+                                NNTILE_HIP_MASK_ADDITIVE, 8, 2>), grid, dim3(512), 0, stream, p);
+                    break;
+                case NNTILE_HIP_MASK_NONE:
+                    hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
+                                NNTILE_HIP_MASK_NONE, 8, 2>), grid, dim3(512), 0, stream, p);
+                    break;
+                case NNTILE_HIP_MASK_CAUSAL:
+                    hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
+                                NNTILE_HIP_MASK_CAUSAL, 8, 2>), grid, dim3(512), 0, stream, p);
+                    break;
+                case NNTILE_HIP_MASK_BOOL:
+                    hipLaunchKernelGGL((sdpa_prefill_16bit_kernel<T, HEAD,
+                                NNTILE_HIP_MASK_BOOL, 8, 2>), grid, dim3(512), 0, stream, p);
+                    break;
+                default:
+                    return NNTILE_HIP_EINVAL;
+            }
+            return hipGetLastError() == hipSuccess ? NNTILE_HIP_OK : NNTILE_HIP_ELAUNCH;
+        }
+    }
     switch(mode)
     {
         case NNTILE_HIP_MASK_ADDITIVE:
@@ -1600,6 +1728,19 @@ int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
     {
         return NNTILE_HIP_EINVAL;
     }
+    // Two groups of four wavefronts per workgroup, each taking every second
+    // key step (p.form == 2, or by itself): when the launch has at most one
+    // 128-query workgroup per CU, so that a CU would otherwise hold one
+    // wavefront per SIMD, and enough key steps to share (with a mask given as
+    // values a 1024-key tile measured no gain or a small loss - the scan of
+    // the mask rows and the mask loads weigh more there - 4096 keys 7-11 %;
+    // analytic masks: 3-8 % at 1024 keys and 256 workgroups, 12-20 % on
+    // longer rows or fewer workgroups).
+    const bool can_split = (head == 64 || head == 128) && !wide;
+    const bool explicit_mask = mode == NNTILE_HIP_MASK_ADDITIVE || mode == NNTILE_HIP_MASK_BOOL;
+    const bool key_split = can_split && (p.form == 2
+            || (p.form == 0 && n_wg <= 8 * (int64_t)kCUsPerXCD
+                && p.k_seq >= (explicit_mask ? 32 : 4) * kKeys));
     p.mask_bits = nullptr;
     const int scan_rc = scan_mask_once<T>(stream, p, mode, scan_scratch, scan_scratch_bytes);
     if(scan_rc != NNTILE_HIP_OK)
@@ -1611,11 +1752,11 @@ int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
     switch(head)
     {
         case 32:
-            return launch_mode<T, 32>(stream, p, mode, grid, false);
+            return launch_mode<T, 32>(stream, p, mode, grid, false, false);
         case 64:
-            return launch_mode<T, 64>(stream, p, mode, grid, wide);
+            return launch_mode<T, 64>(stream, p, mode, grid, wide, key_split);
         case 128:
-            return launch_mode<T, 128>(stream, p, mode, grid, wide);
+            return launch_mode<T, 128>(stream, p, mode, grid, wide, key_split);
         default:
             return NNTILE_HIP_EUNSUPPORTED;
     }

@@ -20,7 +20,7 @@ MASK_ADDITIVE, MASK_NONE, MASK_CAUSAL, MASK_BOOL = 0, 1, 2, 3
 MAX_TILES = 64
 BWD_MAX_TILES = 32
 OVERWRITE = 1
-FORM_SHARED, FORM_SPLIT = 0x100, 0x200     # fp32 calls: fix the workgroup shape (tests, tuning)
+FORM_SHARED, FORM_SPLIT = 0x100, 0x200     # fix the workgroup shape (tests, tuning); 16-bit SPLIT: two groups of four wavefronts
 FORM_WIDE = 0x4000                         # 16-bit analytic-mask calls: 256-query workgroups
 # decode calls (tests, tuning): merge the key splits in a second launch; exchange
 # the partials of the in-launch merge through device-scope fences
