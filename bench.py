@@ -32,8 +32,8 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # properties of the kernel and the workload, not of one timing run; each names
 # the committed rocprofv3 summary it was read from.
 TRAFFIC = {
-    "cfg3_llama_prefill_bf16": (175127911, "profiles/sdpa_prefill_16bit_kernel_cfg3_llama_prefill_bf16.txt"),
-    "cfg4_gqa_decode_bf16": (288075448, "profiles/sdpa_decode_16bit_kernel_cfg4_gqa_decode_bf16.txt"),
+    "cfg3_llama_prefill_bf16": (176977920, "profiles/sdpa_prefill_16bit_kernel_cfg3_llama_prefill_bf16.txt"),
+    "cfg4_gqa_decode_bf16": (288403456, "profiles/sdpa_decode_16bit_kernel_cfg4_gqa_decode_bf16.txt"),
     "cfg2_gpt2_small_fp32": (55549952, "profiles/sdpa_prefill_fp32_kernel_cfg2_gpt2_small_fp32.txt"),
 }
 
@@ -748,7 +748,7 @@ def compact_line(main_leg, dec, ref_api, backward, gemm, cpu, args, cfg3, cfg4, 
                    "launches_per_step": main_leg["launches_per_step"],
                    "timed": "one fused launch over the 4x4 grid of separately allocated tiles, analytic "
                             "causal mask, overwrite mode; value = causal-exact FLOPs / wall time per step"},
-        "roofline": roofline("mfma", "sdpa_prefill_16bit_kernel<bf16,128,causal>", cfg3.flops(),
+        "roofline": roofline("mfma", "sdpa_prefill_16bit_kernel<bf16,128,causal,8 wavefronts>", cfg3.flops(),
                              main_leg["device_ms_per_step"], PEAK_BF16_TFLOPS, "TFLOP/s",
                              TRAFFIC[cfg3.name]),
         "decode": {"workload": cfg4.name, "ms_per_step": round(dec["ms_per_step"], 4),
