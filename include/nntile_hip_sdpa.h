@@ -343,6 +343,14 @@ int nntile_hip_sdpa_fwd_decode_static(void *stream, int32_t dtype,
  * count since the library was loaded (blocking; -1 on error): */
 unsigned long long nntile_hip_debug_decode_spin_limit(unsigned long long ticks);
 long long nntile_hip_debug_decode_sync_timeouts(void);
+/* The partials reach the merge workgroups through the L2 of the XCD that the
+ * unit's main workgroups ran on: a launch's workgroups go round the XCDs in
+ * index order, and a unit's main and merge workgroups have equal indices
+ * modulo 8.  Every flag carries the number of the XCD that raised it; a merge
+ * workgroup that finds a split of its unit raised elsewhere than on its own
+ * XCD leaves its rows untouched and is counted here (never observed, also not
+ * with several queues dispatching at once; blocking; -1 on error): */
+long long nntile_hip_debug_decode_sync_misplaced(void);
 
 /* ---- 5. the running-statistics hand-off on its own ---------------------------
  * Replaces kernel::accumulate_attn_output::cuda<T>

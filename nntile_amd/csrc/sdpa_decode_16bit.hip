@@ -46,11 +46,6 @@ constexpr int kDecodeCUs = 256;   // MI355X
 #ifndef NNTILE_DEC_PART16
 #define NNTILE_DEC_PART16 1
 #endif
-// How the partial outputs are stored: 0 plain, 1 non-temporal, 2 / 3 written
-// through at system / device scope
-#ifndef NNTILE_DEC_PART_STORE
-#define NNTILE_DEC_PART_STORE 0
-#endif
 typedef __attribute__((ext_vector_type(4))) float acc4;
 
 // Developer build (-DNNTILE_DEC_TRACE): wall-clock stamps (100 MHz) of every
@@ -145,6 +140,9 @@ __device__ __forceinline__ int xcc_id()
 // Merge workgroups of the fused form that gave up waiting for a flag (they
 // leave their rows untouched); read with nntile_hip_debug_decode_sync_timeouts.
 __device__ unsigned int decode_sync_timeouts;
+// ... and those that found a split of their unit on another XCD than their own
+// (rows untouched as well); read with nntile_hip_debug_decode_sync_misplaced.
+__device__ unsigned int decode_sync_misplaced;
 
 // Merge the split partials of row rr of a unit and fold the result into
 // (lse, A).  The calling thread handles head values d4 .. d4+3.  COH: the
@@ -291,10 +289,22 @@ __device__ __forceinline__ void decode_merge_row(const DecodeParams &p, int unit
 // It is dispatched when main workgroups have left (the hardware starts the
 // workgroups of a launch in index order, and the main ones never wait for
 // anything), waits until every split of its unit has raised its flag, merges
-// its rows and lowers the flags again.  Unit and merge workgroup sit on the
-// XCD of the unit's main workgroups, so flags and partials are exchanged
-// through that XCD's L2; should the hardware have placed either side
-// elsewhere (the XCC_ID register says), both fall back to device-scope fences.
+// its rows and lowers the flags again.
+//
+// Placement: the workgroups of one launch go round the 8 XCDs in index order,
+// so the main workgroups of a unit and its merge workgroups, whose indices
+// are equal modulo 8 by construction, share an XCD and its L2: partials
+// written by plain stores are there for plain loads once the writer's stores
+// are acknowledged, no cache has to be written back or invalidated.  Where
+// the round starts is not the launch's to say (XCD 0 on a fresh queue, another
+// one after a graph launch or on a second stream - but one start per launch,
+// also with several queues dispatching at once), so nothing here assumes a
+// particular XCD: every main workgroup puts the number of the XCD it ran on
+// (hardware register XCC_ID) into its flag and the merge workgroup compares
+// it with its own.  A difference - never seen - is counted and the rows are
+// left alone rather than merged from data that may not have arrived.  With
+// p.fenced both sides use device-scope fences instead and placement is not
+// looked at (for comparison: the fences write back and invalidate whole L2s).
 template<typename T, int HEAD>
 __device__ __forceinline__ void decode_merge_workgroup(const DecodeParams &p, int idx)
 {
@@ -308,8 +318,10 @@ __device__ __forceinline__ void decode_merge_workgroup(const DecodeParams &p, in
     int bad = 0;
     if(tid < p.n_splits)
     {
+        // (the tag's low four bits are clear: the flag carries the writer's XCD there)
         const unsigned long long t0 = wall_clock64();
-        while(ld64<true>(flags + tid) != p.tag)
+        unsigned long long seen;
+        while(((seen = ld64<true>(flags + tid)) & ~15ull) != p.tag)
         {
             __builtin_amdgcn_s_sleep(4);
             if(wall_clock64() - t0 > p.spin_limit)
@@ -318,17 +330,21 @@ __device__ __forceinline__ void decode_merge_workgroup(const DecodeParams &p, in
                 break;
             }
         }
+        if(!bad && !p.fenced && (int)(seen & 15ull) != xcc_id())
+        {
+            bad = 2;
+        }
     }
     bad = __syncthreads_or(bad);
     if(bad)
     {
         if(tid == 0)
         {
-            atomicAdd(&decode_sync_timeouts, 1u);
+            atomicAdd((bad & 1) ? &decode_sync_timeouts : &decode_sync_misplaced, 1u);
         }
         return;
     }
-    if(p.fenced || xcc_id() != x)
+    if(p.fenced)
     {
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     }
@@ -934,17 +950,7 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         u32x2 w;
         w[0] = T::pack2(o[db][0] * inv, o[db][1] * inv);
         w[1] = T::pack2(o[db][2] * inv, o[db][3] * inv);
-#if NNTILE_DEC_PART_STORE == 1
-        __builtin_nontemporal_store(w, reinterpret_cast<u32x2 *>(dst + 16 * db));
-#elif NNTILE_DEC_PART_STORE == 2
-        __hip_atomic_store(reinterpret_cast<unsigned long long *>(dst + 16 * db),
-                __builtin_bit_cast(unsigned long long, w), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-#elif NNTILE_DEC_PART_STORE == 3
-        __hip_atomic_store(reinterpret_cast<unsigned long long *>(dst + 16 * db),
-                __builtin_bit_cast(unsigned long long, w), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#else
         *reinterpret_cast<u32x2 *>(dst + 16 * db) = w;
-#endif
     }
 #else
     float *dst = p.part_o + prow * HEAD + 4 * quad;
@@ -963,16 +969,18 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
     {
         // The partial is complete in this XCD's L2 once every wavefront's
         // stores have been acknowledged (the barrier's release waits for
-        // them); then one flag per merge workgroup of the unit goes up.
+        // them); then one flag per merge workgroup of the unit goes up, with
+        // the number of this XCD in its low bits.
         __syncthreads();
-        if(p.fenced || xcc_id() != (int)(blockIdx.x & 7))
+        if(p.fenced)
         {
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         }
         if(tid < p.merge_blocks_per_unit)
         {
             __hip_atomic_store(p.sync + (int64_t)unit * p.sync_stride + 1 + tid * p.n_splits + split,
-                    p.tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    p.tag | (unsigned long long)xcc_id(), __ATOMIC_RELAXED,
+                    __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }
@@ -1035,7 +1043,8 @@ int decode_sync_stride(int n_splits, int rows, int head)
 
 // A value no earlier call of this process has used and that memory left
 // behind by anything else is unlikely to hold: a random upper half fixed at
-// load time, a counter below it.
+// load time, a counter below it; the low four bits stay clear (a flag holds
+// the tag plus the number of the XCD that raised it).
 static unsigned long long next_decode_tag()
 {
     static const unsigned long long salt = []
@@ -1044,8 +1053,8 @@ static unsigned long long next_decode_tag()
         return ((unsigned long long)rd() << 32) | 0x80000000ull;
     }();
     static std::atomic<unsigned long long> counter{0};
-    unsigned long long tag = salt + counter.fetch_add(1, std::memory_order_relaxed) + 1ull;
-    return tag == 0ull ? 1ull : tag;
+    unsigned long long tag = salt + ((counter.fetch_add(1, std::memory_order_relaxed) + 1ull) << 4);
+    return tag == 0ull ? 16ull : tag;
 }
 
 // Longest wait of a merge workgroup for a flag, in ticks of the 100 MHz clock
@@ -1055,6 +1064,17 @@ static std::atomic<unsigned long long> decode_spin_limit{200000000ull};
 extern "C" unsigned long long nntile_hip_debug_decode_spin_limit(unsigned long long ticks)
 {
     return decode_spin_limit.exchange(ticks);
+}
+
+extern "C" long long nntile_hip_debug_decode_sync_misplaced(void)
+{
+    unsigned int n = 0;
+    if(hipMemcpyFromSymbol(&n, HIP_SYMBOL(decode_sync_misplaced), sizeof(n)) != hipSuccess)
+    {
+        (void)hipGetLastError();
+        return -1;
+    }
+    return (long long)n;
 }
 
 extern "C" long long nntile_hip_debug_decode_sync_timeouts(void)

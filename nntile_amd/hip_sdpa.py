@@ -131,7 +131,8 @@ EXPORTS = (
     + ["nntile_hip_mask_tile_class_" + t for t in ("bf16", "fp16", "fp32", "bool")]
     + ["nntile_hip_sdpa_fwd_grid_codelet_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_bwd_grid_codelet_" + t for t in ("bf16", "fp16")]
-    + ["nntile_hip_debug_decode_spin_limit", "nntile_hip_debug_decode_sync_timeouts"]
+    + ["nntile_hip_debug_decode_spin_limit", "nntile_hip_debug_decode_sync_timeouts",
+       "nntile_hip_debug_decode_sync_misplaced"]
     + ["nntile_hip_set_stream_provider", "nntile_hip_sdpa_version"])
 
 _lib = None
@@ -508,6 +509,15 @@ def decode_sync_timeouts():
     """Merge workgroups of in-launch decode merges that gave up waiting for a
     split since the library was loaded (diagnostic; blocks)."""
     f = lib().nntile_hip_debug_decode_sync_timeouts
+    f.restype = ctypes.c_longlong
+    return int(f())
+
+
+def decode_sync_misplaced():
+    """Merge workgroups of in-launch decode merges that found a split of their
+    unit on another XCD than their own since the library was loaded (they
+    leave their rows untouched; diagnostic; blocks)."""
+    f = lib().nntile_hip_debug_decode_sync_misplaced
     f.restype = ctypes.c_longlong
     return int(f())
 

@@ -51,7 +51,7 @@ def _bits(t):
 @pytest.mark.parametrize("mode", ["causal", "bool", "additive", "none"])
 def test_merge_inside_the_launch(oracle, dtype, q_seq, k_seq, n_batch, group, n_kv, head, mode):
     print("case", dtype, q_seq, k_seq, n_batch, group, n_kv, head, mode, flush=True)
-    before = hip_sdpa.decode_sync_timeouts()
+    before = hip_sdpa.decode_sync_timeouts(), hip_sdpa.decode_sync_misplaced()
     dev, msk, (want, want_lse) = _case(oracle, dtype, q_seq, k_seq, n_batch, group, n_kv, head, mode)
     lse, A = _run(dev, msk, n_batch, group, head, dtype, 0)
     assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
@@ -60,7 +60,7 @@ def test_merge_inside_the_launch(oracle, dtype, q_seq, k_seq, n_batch, group, n_
         lse2, A2 = _run(dev, msk, n_batch, group, head, dtype, flags)
         assert np.array_equal(_bits(A), _bits(A2)), flags
         assert np.array_equal(_bits(lse), _bits(lse2)), flags
-    assert hip_sdpa.decode_sync_timeouts() == before
+    assert (hip_sdpa.decode_sync_timeouts(), hip_sdpa.decode_sync_misplaced()) == before
 
 
 @pytest.mark.parametrize("fill", [0x00, 0xFF, "random"])
@@ -135,3 +135,64 @@ def test_merge_inside_the_launch_into_running_pair(oracle):
     torch.cuda.synchronize()
     assert H.rel_fro(H.to_np(A), want) < H.TOL[dtype]
     assert H.rel_fro(H.to_np(lse), want_lse) < H.TOL[dtype]
+
+
+def test_merge_inside_the_launch_wherever_the_round_of_the_xcds_starts(oracle):
+    """A launch's workgroups go round the XCDs in index order, but the XCD of
+    workgroup 0 depends on the queue and on what ran on it before (a graph
+    launch moves it).  The in-launch merge only needs a unit's main and merge
+    workgroups on one XCD, whichever: on the default stream, on side streams,
+    after a graph launch, and with two streams running decode calls at the
+    same time (each on a workspace of its own) the results are those of the
+    two-launch form, bit for bit, and no merge workgroup reports a split on
+    another XCD."""
+    dtype, q_seq, k_seq, n_batch, group, n_kv, head = "bf16", 16, 4096, 4, 4, 2, 128
+    before = hip_sdpa.decode_sync_timeouts(), hip_sdpa.decode_sync_misplaced()
+    dev, msk, (want, want_lse) = _case(oracle, dtype, q_seq, k_seq, n_batch, group, n_kv, head,
+                                       "causal", seed=57)
+    Kd, Qd, Vd = dev
+    m, mm, offset = msk
+    lse0, A0 = _run(dev, msk, n_batch, group, head, dtype,
+                    hip_sdpa.DECODE_SEPARATE_MERGE | hip_sdpa.OVERWRITE)
+    assert H.rel_fro(H.to_np(A0), want) < H.TOL[dtype]
+    nbytes = hip_sdpa.decode_workspace_bytes(Kd, Qd, n_batch, group)
+
+    def call(out, ws, stream=None):
+        hip_sdpa.sdpa_fwd_decode(Kd, Qd, m, out[0], Vd, out[1], mm, n_batch, group, ws,
+                                 causal_offset=offset, flags=hip_sdpa.OVERWRITE, stream=stream)
+
+    def same(out):
+        return np.array_equal(_bits(out[0]), _bits(lse0)) and np.array_equal(_bits(out[1]), _bits(A0))
+
+    ws = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(3)]
+    out = H.fresh_outputs(Qd.shape[0], q_seq, head, dtype)
+    call(out, ws[0])
+    torch.cuda.synchronize()
+    assert same(out)
+    # a graph launch, then the default stream again
+    gout = H.fresh_outputs(Qd.shape[0], q_seq, head, dtype)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(gout, ws[0])
+    for _ in range(2):
+        gout[0].fill_(float("nan"))
+        gout[1].fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert same(gout)
+    out = H.fresh_outputs(Qd.shape[0], q_seq, head, dtype)
+    call(out, ws[0])
+    torch.cuda.synchronize()
+    assert same(out)
+    # two side streams at the same time, several calls each
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[H.fresh_outputs(Qd.shape[0], q_seq, head, dtype) for _ in range(4)] for _ in streams]
+    torch.cuda.synchronize()
+    for rep in range(4):
+        for k, st in enumerate(streams):
+            call(outs[k][rep], ws[1 + k], stream=st)
+    torch.cuda.synchronize()
+    for k in range(2):
+        for rep in range(4):
+            assert same(outs[k][rep]), (k, rep)
+    assert (hip_sdpa.decode_sync_timeouts(), hip_sdpa.decode_sync_misplaced()) == before
