@@ -410,18 +410,20 @@ def bench_reference_api(cfg, steps, warmup):
     return out
 
 
-def bench_decode(cfg, steps, warmup, more_flags=0):
+def bench_decode(cfg, steps, warmup, more_flags=0, fp32=False):
     """The GQA decode shape: one launch per step (the key splits of a unit
     are merged inside it).  Four (K, V) sets rotate (4 x 256 MiB at cfg4: the
     256 MiB last-level cache cannot serve a pass).  more_flags: further flags
-    of the decode call (the merge as a second launch)."""
+    of the decode call (the merge as a second launch).  fp32: the same shape
+    on fp32 tiles through the fp32 decode kernel (twice the bytes)."""
     import torch
     from nntile_amd import hip_sdpa as h
     kvb = cfg.n_batch * cfg.n_head_kv
-    nrot = 4
-    Ks = [_randn((kvb, cfg.k_seq, cfg.head), torch.bfloat16, cfg.seed, 1 + 10 * j) for j in range(nrot)]
-    Vs = [_randn((kvb, cfg.k_seq, cfg.head), torch.bfloat16, cfg.seed, 2 + 10 * j) for j in range(nrot)]
-    Q = _randn((cfg.batch_flat, cfg.q_seq, cfg.head), torch.bfloat16, cfg.seed, 0)
+    dt = torch.float32 if fp32 else torch.bfloat16
+    nrot = 2 if fp32 else 4
+    Ks = [_randn((kvb, cfg.k_seq, cfg.head), dt, cfg.seed, 1 + 10 * j) for j in range(nrot)]
+    Vs = [_randn((kvb, cfg.k_seq, cfg.head), dt, cfg.seed, 2 + 10 * j) for j in range(nrot)]
+    Q = _randn((cfg.batch_flat, cfg.q_seq, cfg.head), dt, cfg.seed, 0)
     A = torch.zeros_like(Q)
     lse = torch.full((cfg.batch_flat, cfg.q_seq), float("-inf"), device="cuda")
     ws = torch.empty(h.decode_workspace_bytes(Ks[0], Q, cfg.n_batch, cfg.kv_group),
@@ -437,6 +439,10 @@ def bench_decode(cfg, steps, warmup, more_flags=0):
 
     wall, dev = time_steps(step, steps, warmup)
     nbytes = cfg.algorithmic_bytes()
+    if fp32:
+        # K, V, Q, A at 4 bytes an element; lse as before
+        lse_bytes = 4 * cfg.batch_flat * cfg.q_seq
+        nbytes = 2 * (nbytes - lse_bytes) + lse_bytes
     return {"ms_per_step": wall, "device_ms_per_step": dev,
             "gbs": nbytes / (wall * 1e-3) / 1e9, "algorithmic_bytes": nbytes,
             "workspace_bytes": ws.numel(), "tflops": cfg.flops() / (wall * 1e-3) / 1e12}
@@ -804,7 +810,7 @@ def main():
                     help="with --only power_context: a shared library exporting nntile_hip_probe_mfma "
                          "(the matrix instruction alone); not part of the product")
     ap.add_argument("--only", default=None,
-                    help="run only this leg (for profiling): prefill | prefill_128_queries | cfg5 | cfg2 | decode | decode_separate_merge | decode_wide | "
+                    help="run only this leg (for profiling): prefill | prefill_128_queries | cfg5 | cfg2 | decode | decode_separate_merge | decode_wide | decode_fp32 | "
                          "reference_api | reference_grid | power_context | copy_context | backward | backward_slabs | rope | transpose | accumulate | "
                          "kv_cache | copy")
     args = ap.parse_args()
@@ -842,6 +848,7 @@ def main():
             "decode_separate_merge": lambda: bench_decode(cfg4, args.steps, args.warmup,
                                                           h.DECODE_SEPARATE_MERGE),
             "decode_wide": lambda: bench_decode(cfg4_wide, args.steps, args.warmup),
+            "decode_fp32": lambda: bench_decode(cfg4, args.steps, args.warmup, fp32=True),
             "reference_api": lambda: bench_reference_api(cfg3, args.steps, args.warmup),
             "reference_grid": lambda: bench_reference_grid(args.steps, args.warmup, args.case),
             "power_context": lambda: bench_power_context(cfg3, probe_lib=args.probe_lib),
@@ -888,6 +895,16 @@ def main():
             "roofline": roofline("hbm", "sdpa_decode_16bit_kernel (single split)",
                                  r["algorithmic_bytes"], r["device_ms_per_step"],
                                  PEAK_HBM_GBS, "GB/s")})(bench_decode(cfg4_wide, few, 5))
+        detail["decode_fp32"] = (lambda r: {
+            "what": "for information: cfg4's shape on fp32 tiles through the fp32 split-key decode "
+                    "(twice the bytes; 17.2 GFLOP of fp32 matrix work)",
+            "device_ms_per_step": round(r["device_ms_per_step"], 4),
+            "algorithmic_bytes": r["algorithmic_bytes"],
+            "gbs": round(r["algorithmic_bytes"] / (r["device_ms_per_step"] * 1e-3) / 1e9, 1),
+            "tflops": round(cfg4.flops() / (r["device_ms_per_step"] * 1e-3) / 1e12, 1),
+            "frac_of_fp32_mfma_peak": round(cfg4.flops() / (r["device_ms_per_step"] * 1e-3) / 1e12
+                                            / PEAK_FP32_TFLOPS, 4)})(
+            bench_decode(cfg4, few, 5, fp32=True))
         detail["reference_bench_grid"] = bench_reference_grid(20, 5)
         extras = {}
         for name in ("cfg1_single_head_fp32", "cfg2_gpt2_small_fp32", "cfg5_long_seq_bf16"):

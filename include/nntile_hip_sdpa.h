@@ -311,6 +311,14 @@ int nntile_hip_sdpa_fwd_decode_bf16(void *stream, const nntile_hip_sdpa_tile_arg
         void *workspace, size_t workspace_bytes);
 int nntile_hip_sdpa_fwd_decode_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
         void *workspace, size_t workspace_bytes);
+/* fp32 tiles (the reference runs forward_dynamic in fp32 as well,
+ * wrappers/python/tests/model/test_llama_attention.py:296-345): the same
+ * sharing of K/V among the query heads of a group and the same split of the
+ * keys, with v_mfma_f32_16x16x4_f32; the partials are fp32, so the workspace
+ * has a size function of its own, and the merge is always a second launch. */
+size_t nntile_hip_sdpa_fwd_decode_workspace_bytes_fp32(const nntile_hip_sdpa_tile_args *args);
+int nntile_hip_sdpa_fwd_decode_fp32(void *stream, const nntile_hip_sdpa_tile_args *args,
+        void *workspace, size_t workspace_bytes);
 
 /* ---- 4b. decode for callers that cannot allocate -------------------------------
  * No counterpart in the reference.  For callers that cannot call hipMalloc
@@ -513,6 +521,8 @@ int nntile_hip_kv_cache_append_fp32(void *stream, int64_t head, int64_t rows, in
 int nntile_hip_sdpa_fwd_decode_cache_bf16(void *stream, const nntile_hip_sdpa_tile_args *args,
         int64_t capacity, void *workspace, size_t workspace_bytes);
 int nntile_hip_sdpa_fwd_decode_cache_fp16(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity, void *workspace, size_t workspace_bytes);
+int nntile_hip_sdpa_fwd_decode_cache_fp32(void *stream, const nntile_hip_sdpa_tile_args *args,
         int64_t capacity, void *workspace, size_t workspace_bytes);
 
 /* nntile_hip_sdpa_fwd_tile_* reading the cache the same way, for what the

@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libnntile_hip_sdpa.so")
 SOURCES = ["sdpa_prefill_16bit.hip", "sdpa_prefill_fp32.hip",
-           "sdpa_decode_16bit.hip", "sdpa_bwd_16bit.hip", "rope.hip", "transpose.hip", "kv_cache.hip", "mask_classify.hip",
+           "sdpa_decode_16bit.hip", "sdpa_decode_fp32.hip", "sdpa_bwd_16bit.hip", "rope.hip", "transpose.hip", "kv_cache.hip", "mask_classify.hip",
            "accumulate_attn_output.hip", "capi.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -25,6 +25,10 @@ int launch_bwd_grid_16bit(hipStream_t stream, const BwdGridParams &p,
 size_t decode_workspace_bytes(int units, int n_splits, int rows, int head);
 size_t decode_partial_o_bytes(int units, int n_splits, int rows, int head);
 size_t decode_partial_ml_bytes(int units, int n_splits, int rows);
+int launch_decode_fp32(hipStream_t stream, const DecodeParams &p, int head, int mode);
+int decode_fp32_steps(int64_t k_seq);
+int decode_fp32_choose_splits(int units, int n_steps);
+size_t decode_fp32_workspace_bytes(int units, int n_splits, int rows, int head);
 
 struct F32Store;
 struct Bf16Store;
@@ -536,6 +540,73 @@ static int decode_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dt == DType::bf16 ? launch_decode_16bit<Bf16>(s, p, (int)a->head, a->mask_mode)
         : launch_decode_16bit<Fp16>(s, p, (int)a->head, a->mask_mode);
+}
+
+// The fp32 twin: steps of 32 keys, partials in fp32, the merge always a second
+// launch.
+static void decode_fp32_geometry(const nntile_hip_sdpa_tile_args *a, int &units,
+        int &n_steps, int &splits, int &rows)
+{
+    units = (int)(a->batch / a->kv_group);
+    n_steps = decode_fp32_steps(a->k_seq);
+    splits = decode_fp32_choose_splits(units, n_steps);
+    rows = (int)(a->q_seq * a->kv_group);
+}
+
+static int decode_fp32_call(void *stream, const nntile_hip_sdpa_tile_args *a,
+        int64_t kv_rows, void *workspace, size_t workspace_bytes)
+{
+    if(!decode_args_ok(a) || kv_rows < a->k_seq || !mode_ok(a->mask_mode) || a->K == nullptr
+            || a->Q == nullptr || a->V == nullptr || a->lse == nullptr
+            || a->A == nullptr || !aligned16(a->K) || !aligned16(a->Q)
+            || !aligned16(a->V) || !aligned16(a->A))
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    const bool explicit_mask = a->mask_mode == NNTILE_HIP_MASK_ADDITIVE
+        || a->mask_mode == NNTILE_HIP_MASK_BOOL;
+    if(explicit_mask && a->mask == nullptr)
+    {
+        return NNTILE_HIP_EINVAL;
+    }
+    if(a->head != 64 && a->head != 128)
+    {
+        return NNTILE_HIP_EUNSUPPORTED;
+    }
+    int units, n_steps, splits, rows;
+    decode_fp32_geometry(a, units, n_steps, splits, rows);
+    const size_t need = decode_fp32_workspace_bytes(units, splits, rows, (int)a->head);
+    if(workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+    {
+        return NNTILE_HIP_EWORKSPACE;
+    }
+    DecodeParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.q_seq = a->q_seq;
+    p.k_seq = a->k_seq;
+    p.kv_rows = kv_rows;
+    p.q_pos0 = a->q_pos0;
+    p.k_pos0 = a->k_pos0;
+    p.causal_offset = a->causal_offset;
+    p.mask = a->mask;
+    p.mask_ld = a->k_seq;
+    p.K = a->K;
+    p.V = a->V;
+    p.Q = a->Q;
+    p.lse = a->lse;
+    p.A = a->A;
+    p.part_o = static_cast<float *>(workspace);
+    p.part_ml = p.part_o + (size_t)units * splits * rows * a->head;
+    p.n_batch = (int32_t)a->n_batch;
+    p.kv_group = (int32_t)a->kv_group;
+    p.n_head_kv = (int32_t)(units / a->n_batch);
+    p.rows = rows;
+    p.n_splits = splits;
+    p.n_steps = n_steps;
+    p.overwrite = (a->flags & NNTILE_HIP_SDPA_OVERWRITE) ? 1 : 0;
+    p.steps_per_split = (n_steps + splits - 1) / splits;
+    p.scale = 1.0f / sqrtf(static_cast<float>(a->head));
+    return launch_decode_fp32(static_cast<hipStream_t>(stream), p, (int)a->head, a->mask_mode);
 }
 
 // ---- decode with the split partials in memory the library owns ---------------
@@ -1066,6 +1137,23 @@ int nntile_hip_sdpa_fwd_decode_fp16(void *stream, const nntile_hip_sdpa_tile_arg
             workspace_bytes);
 }
 
+size_t nntile_hip_sdpa_fwd_decode_workspace_bytes_fp32(const nntile_hip_sdpa_tile_args *args)
+{
+    if(!decode_args_ok(args))
+    {
+        return 0;
+    }
+    int units, n_steps, splits, rows;
+    decode_fp32_geometry(args, units, n_steps, splits, rows);
+    return decode_fp32_workspace_bytes(units, splits, rows, (int)args->head);
+}
+
+int nntile_hip_sdpa_fwd_decode_fp32(void *stream, const nntile_hip_sdpa_tile_args *args,
+        void *workspace, size_t workspace_bytes)
+{
+    return decode_fp32_call(stream, args, args ? args->k_seq : 0, workspace, workspace_bytes);
+}
+
 int nntile_hip_sdpa_fwd_decode_static(void *stream, int32_t dtype,
         const nntile_hip_sdpa_tile_args *args)
 {
@@ -1306,6 +1394,12 @@ int nntile_hip_sdpa_fwd_decode_cache_fp16(void *stream, const nntile_hip_sdpa_ti
         int64_t capacity, void *workspace, size_t workspace_bytes)
 {
     return decode_call(DType::fp16, stream, args, capacity, workspace, workspace_bytes);
+}
+
+int nntile_hip_sdpa_fwd_decode_cache_fp32(void *stream, const nntile_hip_sdpa_tile_args *args,
+        int64_t capacity, void *workspace, size_t workspace_bytes)
+{
+    return decode_fp32_call(stream, args, capacity, workspace, workspace_bytes);
 }
 
 int nntile_hip_mask_tile_class_bf16(void *stream, int64_t k_rows, int64_t q_cols,

@@ -112,8 +112,9 @@ EXPORTS = (
     ["nntile_hip_flash_sdpa_fwd_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_fwd_tile_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_fwd_grid_" + t for t in ("bf16", "fp16", "fp32")]
-    + ["nntile_hip_sdpa_fwd_decode_" + t for t in ("bf16", "fp16")]
-    + ["nntile_hip_sdpa_fwd_decode_workspace_bytes", "nntile_hip_sdpa_fwd_decode_static"]
+    + ["nntile_hip_sdpa_fwd_decode_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_sdpa_fwd_decode_workspace_bytes", "nntile_hip_sdpa_fwd_decode_workspace_bytes_fp32",
+       "nntile_hip_sdpa_fwd_decode_static"]
     + ["nntile_hip_flash_sdpa_bwd_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_sdpa_bwd_tile_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_sdpa_bwd_workspace_bytes"]
@@ -126,7 +127,7 @@ EXPORTS = (
     + ["nntile_hip_rope_backward_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_transpose_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_kv_cache_append_" + t for t in ("bf16", "fp16", "fp32")]
-    + ["nntile_hip_sdpa_fwd_decode_cache_" + t for t in ("bf16", "fp16")]
+    + ["nntile_hip_sdpa_fwd_decode_cache_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_fwd_tile_cache_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_mask_tile_class_" + t for t in ("bf16", "fp16", "fp32", "bool")]
     + ["nntile_hip_sdpa_fwd_grid_codelet_" + t for t in ("bf16", "fp16", "fp32")]
@@ -162,13 +163,14 @@ def lib():
             f = getattr(L, "nntile_hip_flash_sdpa_fwd_codelet_" + t)
             f.argtypes = [ctypes.POINTER(_vp), _vp]
             f.restype = None
-        for t in ("bf16", "fp16"):
+        for t in ("bf16", "fp16", "fp32"):
             f = getattr(L, "nntile_hip_sdpa_fwd_decode_" + t)
             f.argtypes = [_vp, ctypes.POINTER(TileArgs), _vp, ctypes.c_size_t]
             f.restype = ctypes.c_int
             f = getattr(L, "nntile_hip_sdpa_fwd_decode_cache_" + t)
             f.argtypes = [_vp, ctypes.POINTER(TileArgs), _i64, _vp, ctypes.c_size_t]
             f.restype = ctypes.c_int
+        for t in ("bf16", "fp16"):
             f = getattr(L, "nntile_hip_flash_sdpa_bwd_" + t)
             f.argtypes = [_vp, _i64, _i64, _i64] + [_vp] * 13
             f.restype = ctypes.c_int
@@ -206,6 +208,8 @@ def lib():
         L.nntile_hip_sdpa_bwd_grid_workspace_bytes.restype = ctypes.c_size_t
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.argtypes = [ctypes.POINTER(TileArgs)]
         L.nntile_hip_sdpa_fwd_decode_workspace_bytes.restype = ctypes.c_size_t
+        L.nntile_hip_sdpa_fwd_decode_workspace_bytes_fp32.argtypes = [ctypes.POINTER(TileArgs)]
+        L.nntile_hip_sdpa_fwd_decode_workspace_bytes_fp32.restype = ctypes.c_size_t
         L.nntile_hip_sdpa_fwd_decode_static.argtypes = [_vp, ctypes.c_int32,
                                                         ctypes.POINTER(TileArgs)]
         L.nntile_hip_sdpa_fwd_decode_static.restype = ctypes.c_int
@@ -530,9 +534,14 @@ def decode_spin_limit(ticks):
     return int(f(ticks))
 
 
+def _decode_ws_fn(Q):
+    return getattr(lib(), "nntile_hip_sdpa_fwd_decode_workspace_bytes"
+                   + ("_fp32" if dtype_name(Q) == "fp32" else ""))
+
+
 def decode_workspace_bytes(K, Q, n_batch, kv_group):
     a = _tile_args(K, Q, None, Q, K, Q, MASK_NONE, n_batch, kv_group, 0, 0, 0)
-    return int(lib().nntile_hip_sdpa_fwd_decode_workspace_bytes(ctypes.byref(a)))
+    return int(_decode_ws_fn(Q)(ctypes.byref(a)))
 
 
 def sdpa_fwd_decode(K, Q, mask, lse, V, A, mask_mode, n_batch, kv_group,
@@ -653,7 +662,7 @@ def decode_cache_workspace_bytes(k_seq, Q, n_batch, kv_group):
     a = TileArgs()
     a.batch, a.q_seq, a.head = Q.shape
     a.k_seq, a.n_batch, a.kv_group = k_seq, n_batch, kv_group
-    return int(lib().nntile_hip_sdpa_fwd_decode_workspace_bytes(ctypes.byref(a)))
+    return int(_decode_ws_fn(Q)(ctypes.byref(a)))
 
 
 def mask_tile_class(mask, offset=0, workspace=None, stream=None):

@@ -102,10 +102,9 @@ class KVCache:
         last q_seq tokens of the cache (append first).  lse and A are
         overwritten.  mask: None (the causal rule when `causal`, else nothing
         hidden) or a bool mask as for `mask_slice`, whose slice is then passed
-        as values.  Few rows of a 16-bit type (kv_group * q_seq <= 64, head 64
-        or 128) take the split-key decode kernel, everything else - longer
-        chunks, fp32, head 32 - the tile kernel; both read the caches in
-        place."""
+        as values.  Few rows (kv_group * q_seq <= 64, head 64 or 128) take the
+        split-key decode kernel of the tile type, everything else - longer
+        chunks, head 32 - the tile kernel; both read the caches in place."""
         k_seq = len(self)
         q_seq = Q.shape[1]
         mode = hip_sdpa.MASK_CAUSAL if causal else hip_sdpa.MASK_NONE
@@ -123,8 +122,7 @@ class KVCache:
             return t
 
         self._mask_in_use = keep(sliced)
-        decode = (Q.dtype != torch.float32 and kv_group * q_seq <= 64
-                  and Q.shape[2] in (64, 128))
+        decode = kv_group * q_seq <= 64 and Q.shape[2] in (64, 128)
         if not decode:
             hip_sdpa.sdpa_fwd_tile_cache(
                 self.k, self.v, k_seq, Q, sliced, lse, A, mode, n_batch, kv_group,

@@ -103,7 +103,8 @@ def test_forward_kernels_use_no_scratch_memory(assemblies):
     fp32 and the decode kernels need none; of the 16-bit prefill kernel only
     the explicit-mask variants at head 128 spill a few registers (at most 18
     dwords a lane)."""
-    limits = {"sdpa_prefill_fp32.hip": 0, "sdpa_decode_16bit.hip": 0, "sdpa_prefill_16bit.hip": 72}
+    limits = {"sdpa_prefill_fp32.hip": 0, "sdpa_decode_16bit.hip": 0, "sdpa_decode_fp32.hip": 0,
+              "sdpa_prefill_16bit.hip": 72}
     for name, limit in limits.items():
         sizes = re.findall(r"\.private_segment_fixed_size:\s*(\d+)", assemblies[name])
         assert sizes, name
