@@ -95,10 +95,12 @@ enum nntile_hip_mask_mode
  * The merge is fused into the kernel, so neither scratch tile is needed for
  * it and both may be null.  scratch_A is never touched.  scratch_lse (seq *
  * batch floats, as the reference registers it) may be overwritten: when the
- * mask is 1 MiB or larger the 16-bit variants scan it once per call with a
- * small kernel of their own and keep what they found (16 bytes per 128
- * queries and key range) there, instead of letting the workgroups of every
- * batch entry scan the same rows.  Same result, bit for bit.
+ * mask is 1 MiB or larger the 16-bit variants scan it once per call - by the
+ * first workgroups of the attention launch, or, on a stream that is being
+ * captured, by a small launch of their own - and keep what they found (24
+ * bytes per 128 queries and key range) there, instead of letting the
+ * workgroups of every batch entry scan the same rows.  Same result, bit for
+ * bit.
  *
  * SIZE OF scratch_lse: the call has no argument for it and takes it to be
  * what the reference registers, seq * batch floats.  Pass NULL or a buffer of

@@ -55,7 +55,14 @@ struct PrefillParams
     // range of keys, to be OR-ed): bit s of the first word: some value of
     // 64-key step s is not "open", of the second: not "hidden" (steps from 63
     // on share bit 63).  Null: every workgroup scans its own rows.
-    const unsigned long long *mask_bits;
+    unsigned long long *mask_bits;
+    // The scan riding in the attention launch (n_scan_wgs > 0): the first
+    // n_scan_wgs workgroups of the grid do the scan and publish, per (block,
+    // key range), the two words and then a flag word holding mask_tag (unique
+    // to the call); the attention workgroups wait for the flags of their block,
+    // at most mask_spin_limit ticks of the 100 MHz clock (then they scan their
+    // own rows).  Three words per (block, key range) in either form.
+    unsigned long long mask_tag, mask_spin_limit;
     int32_t n_q_tiles, n_kv_tiles;
     int32_t n_slabs;              // slabs of `batch` entries each in this launch; slab s's tiles sit at
                                   // [s*n_q_tiles + t] / [s*n_kv_tiles + t] of the tables below
@@ -64,6 +71,7 @@ struct PrefillParams
     int32_t k_blocks_per_tile;    // ceil(k_tile / keys per step)
     int32_t xcd_remap;            // 1: regroup workgroups so a slab stays on one XCD
     int32_t overwrite;            // 1: ignore the running pair, write every row
+    int32_t n_scan_wgs;
     int32_t form;                 // fp32 launcher: 0 pick by size, 1 shared key steps, 2 split key steps
                                   // 16-bit launcher: 0 pick by size, 1 128-query workgroups, 2 the same with the key steps split over two groups of wavefronts, 8 256-query
     float scale;                  // 1/sqrt(head)

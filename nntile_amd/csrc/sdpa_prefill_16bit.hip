@@ -29,6 +29,8 @@
 // query tile; the epilogue merges the result into the (lse, A) pair in memory
 // (the hand-off between NNTile tasks), so one launch can stand for one task or
 // for a whole row of tasks.
+#include <atomic>
+#include <random>
 #include <type_traits>
 
 #include "sdpa_common.hpp"
@@ -87,6 +89,103 @@ extern "C" int nntile_hip_debug_pf_trace(unsigned long long *host)
 // CU.  8 (analytic masks, head 64 and 128): one workgroup of 256 queries per
 // CU, whose eight wavefronts share every K/V step - a CU then brings each step
 // into LDS once where two workgroups of four bring it twice.
+// Scan of the mask rows of query block qb over key range sp of kMaskBitSplits:
+// the workgroup (THREADS threads) ORs what it finds in its range of 16-byte
+// chunks into bits[0] (bit s: some value of 64-key step s is not "open") and
+// bits[1] (not "hidden"); steps from 63 on share bit 63.  ES: bytes per mask
+// element; open / hidden: the 32-bit pattern of four (two) visible / hidden
+// elements.  bits is valid for every thread on return.
+template<int ES, int THREADS>
+__device__ __forceinline__ void mask_scan_range(const char *mask, int ld_bytes, int q_len,
+        int n_chunks, uint32_t open_word, uint32_t hidden_word, int qb, int sp,
+        unsigned long long *bits)
+{
+    constexpr int CHUNKS_PER_STEP = kKeys * ES / 16;
+    const int tid = threadIdx.x;
+    if(tid == 0)
+    {
+        bits[0] = 0ull;
+        bits[1] = 0ull;
+    }
+    __syncthreads();
+    const int per_split = (n_chunks + kMaskBitSplits - 1) / kMaskBitSplits;
+    const int c_lo = min(sp * per_split, n_chunks);
+    const int n_loc = min(c_lo + per_split, n_chunks) - c_lo;
+    const int q_row0 = qb * kQRows;
+    const int n_rows = min(kQRows, q_len - q_row0);
+    unsigned long long not_open = 0ull, not_hidden = 0ull;
+    if(n_loc > 0)
+    {
+        const int total = n_rows * n_loc;
+        const char *mbase = mask + (int64_t)q_row0 * ld_bytes + (int64_t)c_lo * 16;
+        // chunk tid, tid + THREADS, ... of the rows' pieces laid end to end
+        const int d_row = THREADS / n_loc, d_c = THREADS % n_loc;
+        int row = tid / n_loc, c = tid % n_loc;
+        for(int base = 0; base < total; base += 16 * THREADS)
+        {
+            // (rows past the end re-read the last row: no branches, so that
+            // the 16 loads are in flight together)
+            u32x4 v[16];
+            int st[16];
+#pragma unroll
+            for(int u = 0; u < 16; ++u)
+            {
+                const int r = min(row, n_rows - 1);
+                st[u] = min((c_lo + c) / CHUNKS_PER_STEP, 63);
+                v[u] = *reinterpret_cast<const u32x4 *>(
+                        mbase + (uint32_t)(r * ld_bytes + c * 16));
+                row += d_row;
+                c += d_c;
+                if(c >= n_loc)
+                {
+                    c -= n_loc;
+                    row += 1;
+                }
+            }
+#pragma unroll
+            for(int u = 0; u < 16; ++u)
+            {
+                const uint32_t any1 = v[u][0] | v[u][1] | v[u][2] | v[u][3];
+                const uint32_t all1 = v[u][0] & v[u][1] & v[u][2] & v[u][3];
+                const bool open = (any1 == open_word) & (all1 == open_word);
+                const bool hidden = (any1 == hidden_word) & (all1 == hidden_word);
+                not_open |= (unsigned long long)(!open) << st[u];
+                not_hidden |= (unsigned long long)(!hidden) << st[u];
+            }
+        }
+    }
+    // One LDS atomic per wavefront and word, not one per lane: the range
+    // covers few steps, and a ballot per step says whether any lane has its bit.
+    {
+        const int s_lo = min(c_lo / CHUNKS_PER_STEP, 63);
+        const int s_hi = min((c_lo + max(n_loc, 1) - 1) / CHUNKS_PER_STEP, 63);
+        unsigned long long w_open = 0ull, w_hidden = 0ull;
+        for(int st = s_lo; st <= s_hi; ++st)
+        {
+            if(__builtin_amdgcn_ballot_w64(((not_open >> st) & 1ull) != 0ull) != 0ull)
+            {
+                w_open |= 1ull << st;
+            }
+            if(__builtin_amdgcn_ballot_w64(((not_hidden >> st) & 1ull) != 0ull) != 0ull)
+            {
+                w_hidden |= 1ull << st;
+            }
+        }
+        if((tid & 63) == 0)
+        {
+            if(w_open != 0ull)
+            {
+                atomicOr(&bits[0], w_open);
+            }
+            if(w_hidden != 0ull)
+            {
+                atomicOr(&bits[1], w_hidden);
+            }
+        }
+    }
+    __syncthreads();
+}
+
 template<typename T, int HEAD, int MODE, int WAVES = 4, int GROUPS = 1>
 __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1)
 void sdpa_prefill_16bit_kernel(const PrefillParams p)
@@ -154,6 +253,40 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     // workgroup shares its CU with the shortest of the first 64.
     const int q_blocks = p.n_q_tiles * p.q_blocks_per_tile;
     unsigned wg = blockIdx.x;
+    if constexpr(EXPLICIT)
+    {
+        // The first workgroups of the grid scan the mask for everybody (one
+        // query tile, one key tile): they wait for nothing, so the attention
+        // workgroups behind them can wait for their flags.
+        if(p.n_scan_wgs > 0)
+        {
+            if((int)blockIdx.x < p.n_scan_wgs)
+            {
+                constexpr int ES = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 2 : 1;
+                __shared__ unsigned long long pub_bits[2];
+                mask_scan_range<ES, kThreads>(static_cast<const char *>(p.mask),
+                        (int)(p.mask_ld * ES), (int)p.q_seq, (int)(p.k_seq * ES / 16),
+                        (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 0u : 0x01010101u,
+                        (MODE == NNTILE_HIP_MASK_ADDITIVE) ? T::kNegInfPair : 0u,
+                        (int)blockIdx.x / kMaskBitSplits, (int)blockIdx.x % kMaskBitSplits,
+                        pub_bits);
+                if(tid == 0)
+                {
+                    // written through to memory (device scope), acknowledged,
+                    // then the flag: readers on any XCD find the words
+                    unsigned long long *e = p.mask_bits + 3 * (int64_t)blockIdx.x;
+                    __hip_atomic_store(e, pub_bits[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(e + 1, pub_bits[1], __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_AGENT);
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __hip_atomic_store(e + 2, p.mask_tag, __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_AGENT);
+                }
+                return;
+            }
+            wg -= (unsigned)p.n_scan_wgs;
+        }
+    }
     if(WAVES == 4 && gridDim.x >= 8u * 2u * kCUsPerXCD)
     {
         const unsigned i = wg >> 3;
@@ -246,121 +379,6 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
             const int kt_hi = hi / k_tile;
             n_steps = min(n_steps, kt_hi * p.k_blocks_per_tile
                     + (hi - kt_hi * k_tile) / kKeys + 1);
-        }
-    }
-    // Explicit masks: number of leading key steps in which the mask changes
-    // nothing for any query of the workgroup (they run in the pipelined loop).
-    int n_open = 0;
-    if(EXPLICIT)
-    {
-        // The workgroup's rows of the mask are scanned once, 16 bytes per
-        // thread and load, 16 loads in flight, before anything is fetched.
-        // Per key step the scan records whether every value is "open" (+0 /
-        // true) and whether every value is "hidden" (-inf / false).  Hidden
-        // steps at the end are dropped - a tile pair above the diagonal of a
-        // causal mask given as values costs this scan instead of a pass over K
-        // and V - and the open steps at the start need no mask handling.
-        constexpr int ES = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 2 : 1;
-        constexpr int CHUNKS_PER_STEP = kKeys * ES / 16;
-        constexpr uint32_t OPEN = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 0u : 0x01010101u;
-        constexpr uint32_t HIDDEN = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? T::kNegInfPair : 0u;
-        const int64_t row_bytes = (int64_t)k_seq * ES;
-        // bit s: some value of step s (steps >= 63 share bit 63) is not open / not hidden
-        unsigned long long not_open = 0ull, not_hidden = 0ull;
-        bool scanned = false;
-        if(n_steps > 0 && p.mask_bits != nullptr)
-        {
-            // the scan was done once for all batch entries before the launch
-            const unsigned long long *w = p.mask_bits + (int64_t)qb * (2 * kMaskBitSplits);
-#pragma unroll
-            for(int sp = 0; sp < kMaskBitSplits; ++sp)
-            {
-                not_open |= w[2 * sp];
-                not_hidden |= w[2 * sp + 1];
-            }
-            scanned = true;
-        }
-        else if(n_steps > 0 && row_bytes % 16 == 0 && (p.mask_ld * ES) % 16 == 0
-                && reinterpret_cast<uintptr_t>(p.mask) % 16 == 0
-                && p.mask_ld * ES * kQRows < (int64_t)(1 << 30))
-        {
-            __shared__ unsigned long long scan_bits[2];
-            if(tid == 0)
-            {
-                scan_bits[0] = 0ull;
-                scan_bits[1] = 0ull;
-            }
-            __syncthreads();
-            const int n_chunks = (int)(row_bytes / 16);
-            const int n_rows = min(kQRows, q_len - q_row0);
-            const int total = n_rows * n_chunks;
-            const char *mbase = static_cast<const char *>(p.mask)
-                + (int64_t)q_row0 * p.mask_ld * ES;
-            // chunk tid, tid + 256, ... of the rows laid end to end: (row, c)
-            // advances by 256 chunks per load without a division
-            const int d_row = kThreads / n_chunks, d_c = kThreads % n_chunks;
-            const int ld_bytes = (int)(p.mask_ld * ES);     // fits: checked above
-            int row = tid / n_chunks, c = tid % n_chunks;
-            for(int base = 0; base < total; base += 16 * kThreads)
-            {
-                // (rows past the end re-read the last row: no branches, so
-                // that the 16 loads are in flight together)
-                u32x4 v[16];
-                int st[16];
-#pragma unroll
-                for(int u = 0; u < 16; ++u)
-                {
-                    const int r = min(row, n_rows - 1);
-                    st[u] = min(c / CHUNKS_PER_STEP, 63);
-                    v[u] = *reinterpret_cast<const u32x4 *>(
-                            mbase + (uint32_t)(r * ld_bytes + c * 16));
-                    row += d_row;
-                    c += d_c;
-                    if(c >= n_chunks)
-                    {
-                        c -= n_chunks;
-                        row += 1;
-                    }
-                }
-#pragma unroll
-                for(int u = 0; u < 16; ++u)
-                {
-                    const uint32_t any1 = v[u][0] | v[u][1] | v[u][2] | v[u][3];
-                    const uint32_t all1 = v[u][0] & v[u][1] & v[u][2] & v[u][3];
-                    const bool open = (any1 == OPEN) & (all1 == OPEN);
-                    const bool hidden = (any1 == HIDDEN) & (all1 == HIDDEN);
-                    not_open |= (unsigned long long)(!open) << st[u];
-                    not_hidden |= (unsigned long long)(!hidden) << st[u];
-                }
-            }
-            if(not_open != 0ull)
-            {
-                atomicOr(&scan_bits[0], not_open);
-            }
-            if(not_hidden != 0ull)
-            {
-                atomicOr(&scan_bits[1], not_hidden);
-            }
-            __syncthreads();
-            not_open = scan_bits[0];
-            not_hidden = scan_bits[1];
-            scanned = true;
-        }
-        if(scanned)
-        {
-            if(not_hidden == 0ull)
-            {
-                if(!p.overwrite)
-                {
-                    return;
-                }
-                n_steps = 0;    // the epilogue writes empty rows
-            }
-            else if((not_hidden >> 63) == 0ull)
-            {
-                n_steps = min(n_steps, 64 - __builtin_clzll(not_hidden));
-            }
-            n_open = not_open == 0ull ? 63 : min(__builtin_ctzll(not_open), 63);
         }
     }
     const int wave_rel_lo = rel0 + wave * 32;       // first query of the wavefront
@@ -645,6 +663,191 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
         advance_one(cur);       // the second group starts at step 1
     }
     StepCursor nxt = cur;                        // step being fetched
+    // Masks given as values: the first step's K and V are requested before the
+    // mask is looked at (below: a wait for the scanning workgroups' flags, or a
+    // scan of this workgroup's own rows).  What the mask then says may make
+    // the step unnecessary, which costs nothing but the request.
+    bool first_requested = false;
+    if(EXPLICIT)
+    {
+        const int own = GROUPS > 1 ? max(n_steps - grp + GROUPS - 1, 0) / GROUPS : n_steps;
+        if(own > 0)
+        {
+            fetch_k(nxt, lds_k0);
+            fetch_v(nxt, lds_v0);
+            first_requested = true;
+        }
+    }
+    // Explicit masks: number of leading key steps in which the mask changes
+    // nothing for any query of the workgroup (they run in the pipelined loop).
+    int n_open = 0;
+    if(EXPLICIT)
+    {
+        // The workgroup's rows of the mask are scanned once, 16 bytes per
+        // thread and load, 16 loads in flight, beside the first step's loads.
+        // Per key step the scan records whether every value is "open" (+0 /
+        // true) and whether every value is "hidden" (-inf / false).  Hidden
+        // steps at the end are dropped - a tile pair above the diagonal of a
+        // causal mask given as values costs this scan instead of a pass over K
+        // and V - and the open steps at the start need no mask handling.
+        constexpr int ES = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 2 : 1;
+        constexpr int CHUNKS_PER_STEP = kKeys * ES / 16;
+        constexpr uint32_t OPEN = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? 0u : 0x01010101u;
+        constexpr uint32_t HIDDEN = (MODE == NNTILE_HIP_MASK_ADDITIVE) ? T::kNegInfPair : 0u;
+        const int64_t row_bytes = (int64_t)k_seq * ES;
+        // bit s: some value of step s (steps >= 63 share bit 63) is not open / not hidden
+        unsigned long long not_open = 0ull, not_hidden = 0ull;
+        bool scanned = false;
+        if(n_steps > 0 && p.mask_bits != nullptr && p.n_scan_wgs == 0)
+        {
+            // the scan was done once for all batch entries before the launch
+            const unsigned long long *w = p.mask_bits + (int64_t)qb * (3 * kMaskBitSplits);
+#pragma unroll
+            for(int sp = 0; sp < kMaskBitSplits; ++sp)
+            {
+                not_open |= w[3 * sp];
+                not_hidden |= w[3 * sp + 1];
+            }
+            scanned = true;
+        }
+        else if(n_steps > 0 && p.mask_bits != nullptr)
+        {
+            // ... or is being done by the first workgroups of this launch: one
+            // thread per key range waits for that range's flag (bounded; the
+            // Q fragments are on their way meanwhile), then everybody ORs
+            __shared__ unsigned long long got_bits[2];
+            __shared__ int got_all;
+            if(tid == 0)
+            {
+                got_bits[0] = 0ull;
+                got_bits[1] = 0ull;
+                got_all = 1;
+            }
+            __syncthreads();
+            if(tid < kMaskBitSplits)
+            {
+                unsigned long long *e = p.mask_bits
+                    + 3 * ((int64_t)qb * kMaskBitSplits + tid);
+                const unsigned long long t0 = wall_clock64();
+                bool ok = true;
+                while(__hip_atomic_load(e + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                        != p.mask_tag)
+                {
+                    __builtin_amdgcn_s_sleep(2);
+                    if(wall_clock64() - t0 > p.mask_spin_limit)
+                    {
+                        ok = false;
+                        break;
+                    }
+                }
+                if(ok)
+                {
+                    atomicOr(&got_bits[0], __hip_atomic_load(e, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_AGENT));
+                    atomicOr(&got_bits[1], __hip_atomic_load(e + 1, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_AGENT));
+                }
+                else
+                {
+                    got_all = 0;
+                }
+            }
+            __syncthreads();
+            if(got_all)
+            {
+                not_open = got_bits[0];
+                not_hidden = got_bits[1];
+                scanned = true;
+            }
+        }
+        // (rows whose length or start is not a multiple of 16 bytes are not
+        // scanned: with loads at the alignment of one element the scan cost
+        // what it saved - 49.6 against 48.1 us on 32 x 1001 x 128)
+        if(!scanned && n_steps > 0 && row_bytes % 16 == 0 && (p.mask_ld * ES) % 16 == 0
+                && reinterpret_cast<uintptr_t>(p.mask) % 16 == 0
+                && p.mask_ld * ES * kQRows < (int64_t)(1 << 30))
+        {
+            __shared__ unsigned long long scan_bits[2];
+            if(tid == 0)
+            {
+                scan_bits[0] = 0ull;
+                scan_bits[1] = 0ull;
+            }
+            __syncthreads();
+            const int n_chunks = (int)(row_bytes / 16);
+            const int n_rows = min(kQRows, q_len - q_row0);
+            const int total = n_rows * n_chunks;
+            const char *mbase = static_cast<const char *>(p.mask)
+                + (int64_t)q_row0 * p.mask_ld * ES;
+            // chunk tid, tid + 256, ... of the rows laid end to end: (row, c)
+            // advances by 256 chunks per load without a division
+            const int d_row = kThreads / n_chunks, d_c = kThreads % n_chunks;
+            const int ld_bytes = (int)(p.mask_ld * ES);     // fits: checked above
+            int row = tid / n_chunks, c = tid % n_chunks;
+            for(int base = 0; base < total; base += 16 * kThreads)
+            {
+                // (rows past the end re-read the last row: no branches, so
+                // that the 16 loads are in flight together)
+                u32x4 v[16];
+                int st[16];
+#pragma unroll
+                for(int u = 0; u < 16; ++u)
+                {
+                    const int r = min(row, n_rows - 1);
+                    st[u] = min(c / CHUNKS_PER_STEP, 63);
+                    v[u] = *reinterpret_cast<const u32x4 *>(
+                            mbase + (uint32_t)(r * ld_bytes + c * 16));
+                    row += d_row;
+                    c += d_c;
+                    if(c >= n_chunks)
+                    {
+                        c -= n_chunks;
+                        row += 1;
+                    }
+                }
+#pragma unroll
+                for(int u = 0; u < 16; ++u)
+                {
+                    const uint32_t any1 = v[u][0] | v[u][1] | v[u][2] | v[u][3];
+                    const uint32_t all1 = v[u][0] & v[u][1] & v[u][2] & v[u][3];
+                    const bool open = (any1 == OPEN) & (all1 == OPEN);
+                    const bool hidden = (any1 == HIDDEN) & (all1 == HIDDEN);
+                    not_open |= (unsigned long long)(!open) << st[u];
+                    not_hidden |= (unsigned long long)(!hidden) << st[u];
+                }
+            }
+            if(not_open != 0ull)
+            {
+                atomicOr(&scan_bits[0], not_open);
+            }
+            if(not_hidden != 0ull)
+            {
+                atomicOr(&scan_bits[1], not_hidden);
+            }
+            __syncthreads();
+            not_open = scan_bits[0];
+            not_hidden = scan_bits[1];
+            scanned = true;
+        }
+        if(scanned)
+        {
+            if(not_hidden == 0ull)
+            {
+                if(!p.overwrite)
+                {
+                    // (the first step's loads may be on their way into LDS)
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    return;
+                }
+                n_steps = 0;    // the epilogue writes empty rows
+            }
+            else if((not_hidden >> 63) == 0ull)
+            {
+                n_steps = min(n_steps, 64 - __builtin_clzll(not_hidden));
+            }
+            n_open = not_open == 0ull ? 63 : min(__builtin_ctzll(not_open), 63);
+        }
+    }
     // Leading steps that are complete (64 keys) and visible to every query of
     // the workgroup need no mask at all; they run in the pipelined loop below.
     int n_fast = 0;
@@ -682,8 +885,11 @@ void sdpa_prefill_16bit_kernel(const PrefillParams p)
     }
     if(n_steps > 0)
     {
-        fetch_k(nxt, lds_k0);
-        fetch_v(nxt, lds_v0);
+        if(!first_requested)
+        {
+            fetch_k(nxt, lds_k0);
+            fetch_v(nxt, lds_v0);
+        }
         advance(nxt);
         if(n_fast > 0)
         {
@@ -1561,86 +1767,23 @@ static int launch_mode(hipStream_t stream, const PrefillParams &p, int mode,
 }
 
 // The scan of an explicit mask that every workgroup of the attention kernel
-// would do for its own 128 rows, done once for all batch entries: workgroup
-// (query block, key range) ORs what it finds in its range of 16-byte chunks
-// into one pair of words (see PrefillParams::mask_bits).  ES: bytes per mask
-// element; open / hidden: the 32-bit pattern of four (two) visible / hidden
-// elements.
+// would do for its own 128 rows, done once for all batch entries, as a launch
+// of its own (calls under stream capture; otherwise the scan rides in the
+// attention launch): workgroup (query block, key range) writes its two words
+// to entry blockIdx.x of the table (three words an entry, the third unused
+// here; see PrefillParams::mask_bits).
 template<int ES>
 __global__ __launch_bounds__(kThreads)
 void mask_step_bits_kernel(const char *mask, int ld_bytes, int q_len, int n_chunks,
         uint32_t open_word, uint32_t hidden_word, unsigned long long *table)
 {
-    constexpr int CHUNKS_PER_STEP = kKeys * ES / 16;
     __shared__ unsigned long long bits[2];
-    const int tid = threadIdx.x;
-    const int qb = blockIdx.x / kMaskBitSplits;
-    const int sp = blockIdx.x % kMaskBitSplits;
-    if(tid == 0)
+    mask_scan_range<ES, kThreads>(mask, ld_bytes, q_len, n_chunks, open_word, hidden_word,
+            (int)blockIdx.x / kMaskBitSplits, (int)blockIdx.x % kMaskBitSplits, bits);
+    if(threadIdx.x == 0)
     {
-        bits[0] = 0ull;
-        bits[1] = 0ull;
-    }
-    __syncthreads();
-    const int per_split = (n_chunks + kMaskBitSplits - 1) / kMaskBitSplits;
-    const int c_lo = min(sp * per_split, n_chunks);
-    const int n_loc = min(c_lo + per_split, n_chunks) - c_lo;
-    const int q_row0 = qb * kQRows;
-    const int n_rows = min(kQRows, q_len - q_row0);
-    unsigned long long not_open = 0ull, not_hidden = 0ull;
-    if(n_loc > 0)
-    {
-        const int total = n_rows * n_loc;
-        const char *mbase = mask + (int64_t)q_row0 * ld_bytes + (int64_t)c_lo * 16;
-        // chunk tid, tid + 256, ... of the rows' pieces laid end to end
-        const int d_row = kThreads / n_loc, d_c = kThreads % n_loc;
-        int row = tid / n_loc, c = tid % n_loc;
-        for(int base = 0; base < total; base += 16 * kThreads)
-        {
-            // (rows past the end re-read the last row: no branches, so that
-            // the 16 loads are in flight together)
-            u32x4 v[16];
-            int st[16];
-#pragma unroll
-            for(int u = 0; u < 16; ++u)
-            {
-                const int r = min(row, n_rows - 1);
-                st[u] = min((c_lo + c) / CHUNKS_PER_STEP, 63);
-                v[u] = *reinterpret_cast<const u32x4 *>(
-                        mbase + (uint32_t)(r * ld_bytes + c * 16));
-                row += d_row;
-                c += d_c;
-                if(c >= n_loc)
-                {
-                    c -= n_loc;
-                    row += 1;
-                }
-            }
-#pragma unroll
-            for(int u = 0; u < 16; ++u)
-            {
-                const uint32_t any1 = v[u][0] | v[u][1] | v[u][2] | v[u][3];
-                const uint32_t all1 = v[u][0] & v[u][1] & v[u][2] & v[u][3];
-                const bool open = (any1 == open_word) & (all1 == open_word);
-                const bool hidden = (any1 == hidden_word) & (all1 == hidden_word);
-                not_open |= (unsigned long long)(!open) << st[u];
-                not_hidden |= (unsigned long long)(!hidden) << st[u];
-            }
-        }
-    }
-    if(not_open != 0ull)
-    {
-        atomicOr(&bits[0], not_open);
-    }
-    if(not_hidden != 0ull)
-    {
-        atomicOr(&bits[1], not_hidden);
-    }
-    __syncthreads();
-    if(tid == 0)
-    {
-        table[2 * (int64_t)blockIdx.x] = bits[0];
-        table[2 * (int64_t)blockIdx.x + 1] = bits[1];
+        table[3 * (int64_t)blockIdx.x] = bits[0];
+        table[3 * (int64_t)blockIdx.x + 1] = bits[1];
     }
 }
 
@@ -1648,14 +1791,32 @@ void mask_step_bits_kernel(const char *mask, int ld_bytes, int q_len, int n_chun
 // themselves: the launch of the scan would cost more than it saves.
 constexpr int64_t kMaskScanLaunchBytes = 1 << 20;
 
+// A value no earlier call of this process has used and that memory left
+// behind by anything else is unlikely to hold (never 0).
+static unsigned long long next_scan_tag()
+{
+    static const unsigned long long salt = []
+    {
+        std::random_device rd;
+        return ((unsigned long long)rd() << 32) | 0x40000000ull;
+    }();
+    static std::atomic<unsigned long long> counter{0};
+    const unsigned long long tag = salt + counter.fetch_add(1, std::memory_order_relaxed) + 1ull;
+    return tag == 0ull ? 1ull : tag;
+}
+
 // One-tile calls with an explicit mask and a scratch buffer of the caller's
 // (the reference's scratch_logsumexp tile): scan the mask once, into the
-// scratch, instead of once per batch entry.  Leaves p.mask_bits null when the
-// conditions of the kernel's own scan do not hold or the scratch is too small.
+// scratch, instead of once per batch entry - by the first workgroups of the
+// attention launch itself, or, on a stream that is being captured (a replay
+// would carry this call's tag again and find the flags of the replay before
+// it), by a launch of its own.  Leaves p.mask_bits null when the conditions of
+// the kernel's own scan do not hold or the scratch is too small.
 template<typename T>
 static int scan_mask_once(hipStream_t stream, PrefillParams &p, int mode,
         void *scratch, size_t scratch_bytes)
 {
+    p.n_scan_wgs = 0;
     const bool additive = mode == NNTILE_HIP_MASK_ADDITIVE;
     if((!additive && mode != NNTILE_HIP_MASK_BOOL) || scratch == nullptr
             || p.n_q_tiles != 1 || p.n_kv_tiles != 1 || p.mask == nullptr)
@@ -1664,7 +1825,7 @@ static int scan_mask_once(hipStream_t stream, PrefillParams &p, int mode,
     }
     const int64_t es = additive ? 2 : 1;
     const int64_t row_bytes = p.k_seq * es;
-    const int64_t table_bytes = (int64_t)p.q_blocks_per_tile * kMaskBitSplits * 16;
+    const int64_t table_bytes = (int64_t)p.q_blocks_per_tile * kMaskBitSplits * 24;
     if(row_bytes % 16 != 0 || (p.mask_ld * es) % 16 != 0
             || reinterpret_cast<uintptr_t>(p.mask) % 16 != 0
             || p.mask_ld * es * kQRows >= (int64_t)(1 << 30)
@@ -1676,6 +1837,20 @@ static int scan_mask_once(hipStream_t stream, PrefillParams &p, int mode,
     }
     auto *table = static_cast<unsigned long long *>(scratch);
     const dim3 grid((unsigned)(p.q_blocks_per_tile * kMaskBitSplits));
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if(hipStreamIsCapturing(stream, &capturing) != hipSuccess)
+    {
+        (void)hipGetLastError();
+        capturing = hipStreamCaptureStatusActive;       // the careful form
+    }
+    if(capturing == hipStreamCaptureStatusNone)
+    {
+        p.mask_bits = table;
+        p.n_scan_wgs = (int32_t)grid.x;
+        p.mask_tag = next_scan_tag();
+        p.mask_spin_limit = 100000000ull;       // 1 s of the 100 MHz clock
+        return NNTILE_HIP_OK;
+    }
     if(additive)
     {
         hipLaunchKernelGGL((mask_step_bits_kernel<2>), grid, dim3(kThreads), 0, stream,
@@ -1748,7 +1923,9 @@ int launch_prefill_16bit(hipStream_t stream, PrefillParams &p, int head,
         return scan_rc;
     }
     p.xcd_remap = (batch_all % 8 == 0) ? 1 : 0;
-    const dim3 grid((unsigned)n_wg);
+    // (the scanning workgroups come first; their number is a multiple of 8, so
+    // the attention workgroups keep their places in the round of the XCDs)
+    const dim3 grid((unsigned)(n_wg + p.n_scan_wgs));
     switch(head)
     {
         case 32:

@@ -118,3 +118,52 @@ def test_prefill_and_backward_in_a_graph():
         assert torch.allclose(torch.cat(got[1], dim=1).float(), got[2].float(), rtol=2e-2, atol=2e-2)
 
     _replays(graph, check, disturb)
+
+
+def test_reference_call_with_a_mask_tile_and_scratch_in_a_graph():
+    """The reference-signature call scans a large mask once per call.  Outside a
+    capture the scan rides in the attention launch behind a tag unique to the
+    call; a captured call would carry its tag into every replay, so under
+    capture the scan is a launch of its own.  Replays after the mask has been
+    rewritten in place must follow the new mask, and so must eager calls in
+    between (the scratch keeps what the other form left there)."""
+    import numpy as np
+    batch, seq, head = 3, 1024, 128
+    dt = torch.bfloat16
+    Q, K, V = (_randn((batch, seq, head), dt, 20 + i) for i in range(3))
+    i = np.arange(seq)[:, None]
+    j = np.arange(seq)[None, :]
+    masks = [np.ascontiguousarray(np.broadcast_to(m, (seq, seq)))
+             for m in (j <= i, np.abs(i - j) <= 100, (j <= i) & (i >= 300), j >= 0)]
+    as_tile = lambda vis: torch.from_numpy(np.where(vis, 0.0, -np.inf).astype(np.float32)).to(dt).cuda()
+    mask = as_tile(masks[0]).clone()
+    scratch = torch.full((batch, seq), float("nan"), device="cuda")
+
+    def call(lse, A):
+        lse.fill_(float("-inf"))
+        A.zero_()
+        hip_sdpa.flash_sdpa_fwd(K, Q, mask, lse, V, A, scratch_lse=scratch)
+
+    lse_g, A_g = H.fresh_outputs(batch, seq, head, "bf16")
+    call(lse_g, A_g)                      # warm-up, eager
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(lse_g, A_g)
+    for vis in masks[1:] + masks[:1]:
+        mask.copy_(as_tile(vis))
+        # eager, without the scratch: every workgroup scans its own rows
+        lse_e, A_e = H.fresh_outputs(batch, seq, head, "bf16")
+        lse_e.fill_(float("-inf"))
+        A_e.zero_()
+        hip_sdpa.flash_sdpa_fwd(K, Q, mask, lse_e, V, A_e)
+        # eager with the scratch (the scan rides in the launch), then the replay
+        lse_s, A_s = H.fresh_outputs(batch, seq, head, "bf16")
+        call(lse_s, A_s)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        rows = torch.from_numpy(vis.any(axis=1)).cuda()
+        for lse_x, A_x in ((lse_s, A_s), (lse_g, A_g)):
+            assert torch.equal(lse_x, lse_e)
+            assert torch.equal(A_x[:, rows].view(torch.int16), A_e[:, rows].view(torch.int16))
