@@ -90,7 +90,9 @@ def test_static_scratch_decode_allocates_nothing():
             call()
         torch.cuda.synchronize()
         free1, _ = torch.cuda.mem_get_info()
-        assert free1 == free0
+        # (a workspace for this shape would be 8 MiB and more; the runtime's own
+        # pools may move by a page or two)
+        assert free1 >= free0 - (1 << 20)
         assert torch.cuda.memory_reserved() == reserved0
         assert torch.cuda.memory_allocated() == allocated0
 
