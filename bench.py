@@ -665,8 +665,18 @@ def bench_kv_cache(cfg, steps, warmup):
         appends[i[0] % nrot].launch()
         i[0] += 1
 
+    fused = [h.plan_decode_append_cache(k_new, v_new, Ks[j], Vs[j], cfg.k_seq, Q, None, lse, A,
+                                        h.MASK_CAUSAL, cfg.n_batch, cfg.kv_group, ws,
+                                        causal_offset=cfg.causal_offset, flags=h.OVERWRITE)
+             for j in range(nrot)]
+
+    def one_launch():
+        fused[i[0] % nrot].launch()
+        i[0] += 1
+
     wall, dev = time_steps(step, steps, warmup)
     _, dev_append = time_steps(append_only, steps, 2)
+    _, dev_one = time_steps(one_launch, steps, 5)
     # the same step as a HIP graph (one per cache pair), replayed
     graphs = []
     for j in range(nrot):
@@ -687,6 +697,8 @@ def bench_kv_cache(cfg, steps, warmup):
                     % (cfg.q_seq, cfg.k_seq, cfg.name, cap),
             "ms_per_step": round(wall, 4), "device_ms_per_step": round(dev, 4),
             "append_device_ms": round(dev_append, 4),
+            "one_launch_device_ms_per_step": round(dev_one, 4),
+            "one_launch_frac_of_hbm_peak": round(nbytes / (dev_one * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
             "graph_replay_device_ms_per_step": round(dev_graph, 4), "algorithmic_bytes": nbytes,
             "gbs": round(nbytes / (dev * 1e-3) / 1e9, 1),
             "frac_of_hbm_peak": round(nbytes / (dev * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),

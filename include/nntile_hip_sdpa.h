@@ -526,6 +526,24 @@ int nntile_hip_sdpa_fwd_decode_cache_fp16(void *stream, const nntile_hip_sdpa_ti
         int64_t capacity, void *workspace, size_t workspace_bytes);
 int nntile_hip_sdpa_fwd_decode_cache_fp32(void *stream, const nntile_hip_sdpa_tile_args *args,
         int64_t capacity, void *workspace, size_t workspace_bytes);
+/* The append and the attention of a decode step in ONE launch (no counterpart
+ * in the reference, where they are the copy_intersection calls of
+ * cache_utils.py:146-175 followed by the attention): k_new, v_new
+ * [head, rows_new, n_batch, n_head_kv] are the keys and values of the newest
+ * rows_new tokens, args->k_seq counts the rows of the caches INCLUDING them,
+ * i.e. they belong at rows [k_seq - rows_new, k_seq) of every entry.  The
+ * attention reads those rows from k_new / v_new and the rest from the caches;
+ * workgroups at the end of the launch copy the new rows into the caches, so
+ * after the call the caches are what nntile_hip_kv_cache_append_* would have
+ * made them, and (lse, A) what nntile_hip_sdpa_fwd_decode_cache_* would then
+ * have computed, bit for bit.  NNTILE_HIP_EINVAL when rows_new exceeds k_seq
+ * or the capacity is smaller than k_seq. */
+int nntile_hip_sdpa_fwd_decode_append_cache_bf16(void *stream,
+        const nntile_hip_sdpa_tile_args *args, int64_t capacity, const uint16_t *k_new,
+        const uint16_t *v_new, int64_t rows_new, void *workspace, size_t workspace_bytes);
+int nntile_hip_sdpa_fwd_decode_append_cache_fp16(void *stream,
+        const nntile_hip_sdpa_tile_args *args, int64_t capacity, const uint16_t *k_new,
+        const uint16_t *v_new, int64_t rows_new, void *workspace, size_t workspace_bytes);
 
 /* nntile_hip_sdpa_fwd_tile_* reading the cache the same way, for what the
  * decode form does not take: fp32 caches (the reference runs forward_dynamic

@@ -479,9 +479,19 @@ static void decode_geometry(const nntile_hip_sdpa_tile_args *a, int &units,
     rows = (int)(a->q_seq * a->kv_group);
 }
 
+// k_new, v_new, n_new: rows [k_seq - n_new, k_seq) of every entry are not in
+// the caches yet; the launch reads them from k_new / v_new and writes them
+// into the caches as well (n_new == 0: nothing of the kind)
 static int decode_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *a,
-        int64_t kv_rows, void *workspace, size_t workspace_bytes)
+        int64_t kv_rows, void *workspace, size_t workspace_bytes,
+        const void *k_new = nullptr, const void *v_new = nullptr, int64_t n_new = 0)
 {
+    if(n_new != 0 && (a == nullptr || n_new < 0 || n_new > a->k_seq || n_new > 0x7fffffff
+                || k_new == nullptr || v_new == nullptr || !aligned16(k_new)
+                || !aligned16(v_new)))
+    {
+        return NNTILE_HIP_EINVAL;
+    }
     if(!decode_args_ok(a) || kv_rows < a->k_seq || !mode_ok(a->mask_mode) || a->K == nullptr
             || a->Q == nullptr || a->V == nullptr || a->lse == nullptr
             || a->A == nullptr || !aligned16(a->K) || !aligned16(a->Q)
@@ -528,6 +538,9 @@ static int decode_call(DType dt, void *stream, const nntile_hip_sdpa_tile_args *
             + decode_partial_ml_bytes(units, splits, rows));
     p.fused = (a->flags & NNTILE_HIP_SDPA_DECODE_SEPARATE_MERGE) ? 0 : 1;
     p.fenced = (a->flags & NNTILE_HIP_SDPA_DECODE_FENCED) ? 1 : 0;
+    p.k_new = k_new;
+    p.v_new = v_new;
+    p.n_new = (int32_t)n_new;
     p.n_batch = (int32_t)a->n_batch;
     p.kv_group = (int32_t)a->kv_group;
     p.n_head_kv = (int32_t)(units / a->n_batch);
@@ -1394,6 +1407,22 @@ int nntile_hip_sdpa_fwd_decode_cache_fp16(void *stream, const nntile_hip_sdpa_ti
         int64_t capacity, void *workspace, size_t workspace_bytes)
 {
     return decode_call(DType::fp16, stream, args, capacity, workspace, workspace_bytes);
+}
+
+int nntile_hip_sdpa_fwd_decode_append_cache_bf16(void *stream,
+        const nntile_hip_sdpa_tile_args *args, int64_t capacity, const uint16_t *k_new,
+        const uint16_t *v_new, int64_t rows_new, void *workspace, size_t workspace_bytes)
+{
+    return decode_call(DType::bf16, stream, args, capacity, workspace, workspace_bytes, k_new,
+            v_new, rows_new);
+}
+
+int nntile_hip_sdpa_fwd_decode_append_cache_fp16(void *stream,
+        const nntile_hip_sdpa_tile_args *args, int64_t capacity, const uint16_t *k_new,
+        const uint16_t *v_new, int64_t rows_new, void *workspace, size_t workspace_bytes)
+{
+    return decode_call(DType::fp16, stream, args, capacity, workspace, workspace_bytes, k_new,
+            v_new, rows_new);
 }
 
 int nntile_hip_sdpa_fwd_decode_cache_fp32(void *stream, const nntile_hip_sdpa_tile_args *args,

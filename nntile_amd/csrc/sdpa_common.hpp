@@ -111,6 +111,13 @@ struct DecodeParams
     unsigned long long spin_limit;  // longest wait for a flag, in 100 MHz ticks
     int32_t fused, fenced;
     int32_t n_main, merge_blocks_per_unit, sync_stride;
+    // The append riding in the launch (n_new > 0): K and V are caches whose
+    // rows [k_seq - n_new, k_seq) of every entry have not been written yet;
+    // they are k_new / v_new ([entry][n_new][head]).  The main workgroups read
+    // those rows from k_new / v_new, and n_append workgroups at the end of the
+    // grid (one per unit) copy them into the caches for the calls to come.
+    const void *k_new, *v_new;
+    int32_t n_new, n_append;
 };
 
 // Kernel arguments of the backward kernels.  K, V, dK, dV: [head, k_seq,

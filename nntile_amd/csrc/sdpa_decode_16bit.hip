@@ -405,18 +405,42 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         else { return ring3; }
     };
 
-    if constexpr(!DIRECT)
+    // The grid: n_main main workgroups, then (merge in the launch) the merge
+    // workgroups, then (append in the launch) one copying workgroup per unit.
+    if((int)blockIdx.x >= p.n_main)
     {
-        if(p.fused && (int)blockIdx.x >= p.n_main)
+        const int n_merge = p.fused ? p.n_batch * p.n_head_kv * p.merge_blocks_per_unit : 0;
+        const int behind = (int)blockIdx.x - p.n_main;
+        if(behind >= n_merge)
+        {
+            // New rows into the caches: 16 bytes a thread and piece.  Nobody in
+            // this launch reads them there (the main workgroups take them from
+            // k_new / v_new), so there is nothing to wait for or to signal.
+            const int unit_a = behind - n_merge;
+            const int64_t filled = p.k_seq - p.n_new;
+            const int n16 = p.n_new * (RB / 16);
+            for(int t = threadIdx.x; t < 2 * n16; t += kDecThreads)
+            {
+                const int which = t >= n16 ? 1 : 0;
+                const int piece = t - which * n16;
+                const char *src = static_cast<const char *>(which ? p.v_new : p.k_new)
+                    + ((int64_t)unit_a * p.n_new * RB + (int64_t)piece * 16);
+                char *dst = static_cast<char *>(const_cast<void *>(which ? p.V : p.K))
+                    + (((int64_t)unit_a * p.kv_rows + filled) * RB + (int64_t)piece * 16);
+                *reinterpret_cast<u32x4 *>(dst) = *reinterpret_cast<const u32x4 *>(src);
+            }
+            return;
+        }
+        if constexpr(!DIRECT)
         {
             DEC_STAMP(5);
-            decode_merge_workgroup<T, HEAD>(p, (int)blockIdx.x - p.n_main);
+            decode_merge_workgroup<T, HEAD>(p, behind);
 #ifdef NNTILE_DEC_TRACE
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             DEC_STAMP(6);
 #endif
-            return;
         }
+        return;
     }
     DEC_STAMP(0);
     const int tid = threadIdx.x;
@@ -529,7 +553,28 @@ void sdpa_decode_16bit_kernel(const DecodeParams p)
         char *kdst = slot_base + wave_u * LOADS_PER_WAVE * 1024;
         char *vdst = kdst + K_BYTES;
         const int rows_left = (int)min((int64_t)kDecKeys, p.k_seq - row0);
-        if(rows_left >= kDecKeys)
+        if(p.n_new > 0 && row0 + kDecKeys > p.k_seq - p.n_new)
+        {
+            // some rows of this step are new tokens: they are not in the caches
+            // yet and are read from where the caller holds them (rows past
+            // the end clamped to the last row, as below)
+            const int64_t filled = p.k_seq - p.n_new;
+            const char *Kn = static_cast<const char *>(p.k_new) + (int64_t)unit * p.n_new * RB;
+            const char *Vn = static_cast<const char *>(p.v_new) + (int64_t)unit * p.n_new * RB;
+#pragma unroll
+            for(int i = 0; i < LOADS_PER_WAVE; ++i)
+            {
+                const int64_t g = min(row0 + ld_row[i], p.k_seq - 1);
+                const uint32_t kc = k_goff[i] - (uint32_t)(ld_row[i] * RB);     // the chunk within the row
+                const uint32_t vc = v_goff[i] - (uint32_t)(ld_row[i] * RB);
+                const bool fresh = g >= filled;
+                const char *ks = fresh ? Kn + (g - filled) * RB : Kb + g * RB;
+                const char *vs = fresh ? Vn + (g - filled) * RB : Vb + g * RB;
+                load_to_lds16<0, NNTILE_DMA_NT>(ks + kc, kdst + i * 1024);
+                load_to_lds16<0, NNTILE_DMA_NT>(vs + vc, vdst + i * 1024);
+            }
+        }
+        else if(rows_left >= kDecKeys)
         {
 #pragma unroll
             for(int i = 0; i < LOADS_PER_WAVE; ++i)
@@ -1118,7 +1163,8 @@ static int launch_decode_stages(hipStream_t stream, DecodeParams &p, int mode)
         p.tag = next_decode_tag();
         p.spin_limit = decode_spin_limit.load(std::memory_order_relaxed);
     }
-    const dim3 grid((unsigned)(p.n_main + (p.fused ? units * merge_blocks : 0)));
+    p.n_append = p.n_new > 0 ? units : 0;
+    const dim3 grid((unsigned)(p.n_main + (p.fused ? units * merge_blocks : 0) + p.n_append));
     switch(mode)
     {
         case NNTILE_HIP_MASK_ADDITIVE:

@@ -128,6 +128,7 @@ EXPORTS = (
     + ["nntile_hip_transpose_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_kv_cache_append_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_fwd_decode_cache_" + t for t in ("bf16", "fp16", "fp32")]
+    + ["nntile_hip_sdpa_fwd_decode_append_cache_" + t for t in ("bf16", "fp16")]
     + ["nntile_hip_sdpa_fwd_tile_cache_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_mask_tile_class_" + t for t in ("bf16", "fp16", "fp32", "bool")]
     + ["nntile_hip_sdpa_fwd_grid_codelet_" + t for t in ("bf16", "fp16", "fp32")]
@@ -171,6 +172,9 @@ def lib():
             f.argtypes = [_vp, ctypes.POINTER(TileArgs), _i64, _vp, ctypes.c_size_t]
             f.restype = ctypes.c_int
         for t in ("bf16", "fp16"):
+            f = getattr(L, "nntile_hip_sdpa_fwd_decode_append_cache_" + t)
+            f.argtypes = [_vp, ctypes.POINTER(TileArgs), _i64, _vp, _vp, _i64, _vp, ctypes.c_size_t]
+            f.restype = ctypes.c_int
             f = getattr(L, "nntile_hip_flash_sdpa_bwd_" + t)
             f.argtypes = [_vp, _i64, _i64, _i64] + [_vp] * 13
             f.restype = ctypes.c_int
@@ -656,6 +660,44 @@ def plan_decode_cache(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_bat
     return Plan(fn, a, "sdpa_fwd_decode_cache",
                 extra=(K_cache.shape[1], _ptr(workspace), nbytes),
                 keep=(K_cache, V_cache, Q, mask, lse, A, workspace))
+
+
+def _append_cache_call(k_new, v_new, K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch,
+                       kv_group, workspace, q_pos0, k_pos0, causal_offset, flags):
+    _dev(k_new, v_new, K_cache, V_cache, Q, mask, lse, A, workspace)
+    entries, rows, head = k_new.shape
+    if (K_cache.shape != V_cache.shape or tuple(v_new.shape) != (entries, rows, head)
+            or K_cache.shape[0] != entries or K_cache.shape[2] != head or rows > k_seq
+            or k_new.dtype != K_cache.dtype):
+        raise SdpaError(EINVAL, "sdpa_fwd_decode_append_cache")
+    a = _cache_args(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch, kv_group,
+                    q_pos0, k_pos0, causal_offset, flags)
+    fn = getattr(lib(), "nntile_hip_sdpa_fwd_decode_append_cache_" + dtype_name(Q))
+    nbytes = workspace.numel() * workspace.element_size()
+    extra = (K_cache.shape[1], _ptr(k_new), _ptr(v_new), rows, _ptr(workspace), nbytes)
+    return fn, a, extra
+
+
+def sdpa_fwd_decode_append_cache(k_new, v_new, K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode,
+                                 n_batch, kv_group, workspace, q_pos0=0, k_pos0=0,
+                                 causal_offset=0, flags=0, stream=None):
+    """kv_cache_append of k_new, v_new ([entries, rows, head]) behind the
+    k_seq - rows filled rows of the caches and sdpa_fwd_decode_cache over the
+    k_seq rows, in one launch (16-bit types)."""
+    fn, a, extra = _append_cache_call(k_new, v_new, K_cache, V_cache, k_seq, Q, mask, lse, A,
+                                      mask_mode, n_batch, kv_group, workspace, q_pos0, k_pos0,
+                                      causal_offset, flags)
+    _check(fn(_stream(stream), ctypes.byref(a), *extra), "sdpa_fwd_decode_append_cache")
+
+
+def plan_decode_append_cache(k_new, v_new, K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode,
+                             n_batch, kv_group, workspace, q_pos0=0, k_pos0=0, causal_offset=0,
+                             flags=0):
+    fn, a, extra = _append_cache_call(k_new, v_new, K_cache, V_cache, k_seq, Q, mask, lse, A,
+                                      mask_mode, n_batch, kv_group, workspace, q_pos0, k_pos0,
+                                      causal_offset, flags)
+    return Plan(fn, a, "sdpa_fwd_decode_append_cache", extra=extra,
+                keep=(k_new, v_new, K_cache, V_cache, Q, mask, lse, A, workspace))
 
 
 def decode_cache_workspace_bytes(k_seq, Q, n_batch, kv_group):

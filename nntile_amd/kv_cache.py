@@ -62,6 +62,50 @@ class KVCache:
         self.k_cache_size += rows
         self.v_cache_size += rows
 
+    def append_attend(self, k_partial, v_partial, Q, lse, A, n_batch, kv_group, causal=True,
+                      mask=None, stream=None):
+        """`append` followed by `attend`, same results bit for bit; on the
+        decode kernel's shapes with a 16-bit type the two are ONE launch (the
+        attention reads the new rows from k_partial / v_partial while other
+        workgroups of the launch write them into the caches)."""
+        rows, q_seq = k_partial.shape[1], Q.shape[1]
+        one_launch = (self.k is not None and v_partial.shape[1] == rows
+                      and Q.dtype in (torch.bfloat16, torch.float16)
+                      and kv_group * q_seq <= 64 and Q.shape[2] in (64, 128)
+                      and rows + self.k_cache_size <= self.max_cache_size
+                      and k_partial.is_contiguous() and v_partial.is_contiguous())
+        if not one_launch:
+            self.append(k_partial, v_partial, stream=stream)
+            self.attend(Q, lse, A, n_batch, kv_group, causal=causal, mask=mask, stream=stream)
+            return
+        self.k_cache_size += rows
+        self.v_cache_size += rows
+        k_seq = self.k_cache_size
+        mode = hip_sdpa.MASK_CAUSAL if causal else hip_sdpa.MASK_NONE
+        sliced = None
+        if mask is not None:
+            sliced, mode = self.mask_slice(mask, q_seq), hip_sdpa.MASK_BOOL
+        if stream is not None:
+            for t in (sliced, k_partial, v_partial):
+                if t is not None:
+                    t.record_stream(stream)
+        self._mask_in_use = sliced
+        workspace = self._decode_workspace(k_seq, Q, n_batch, kv_group, stream)
+        hip_sdpa.sdpa_fwd_decode_append_cache(
+            k_partial, v_partial, self.k, self.v, k_seq, Q, sliced, lse, A, mode, n_batch, kv_group,
+            workspace, causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)
+
+    def _decode_workspace(self, k_seq, Q, n_batch, kv_group, stream):
+        need = hip_sdpa.decode_cache_workspace_bytes(k_seq, Q, n_batch, kv_group)
+        if self._workspace is None or self._workspace.numel() < need:
+            # (a launch of an earlier call may still read the old workspace:
+            # it is kept until the one after next replaces it)
+            self._retired_workspace = self._workspace
+            self._workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
+        if stream is not None:
+            self._workspace.record_stream(stream)
+        return self._workspace
+
     @property
     def k_partial(self):
         """The filled rows, as a view (the reference returns a copy)."""
@@ -128,13 +172,7 @@ class KVCache:
                 self.k, self.v, k_seq, Q, sliced, lse, A, mode, n_batch, kv_group,
                 causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)
             return
-        need = hip_sdpa.decode_cache_workspace_bytes(k_seq, Q, n_batch, kv_group)
-        if self._workspace is None or self._workspace.numel() < need:
-            # (a launch of an earlier call may still read the old workspace:
-            # it is kept until the one after next replaces it)
-            self._retired_workspace = self._workspace
-            self._workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
-        keep(self._workspace)
+        workspace = self._decode_workspace(k_seq, Q, n_batch, kv_group, stream)
         hip_sdpa.sdpa_fwd_decode_cache(
-            self.k, self.v, k_seq, Q, sliced, lse, A, mode, n_batch, kv_group, self._workspace,
+            self.k, self.v, k_seq, Q, sliced, lse, A, mode, n_batch, kv_group, workspace,
             causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)
