@@ -163,7 +163,21 @@ __device__ __forceinline__ void map_workgroup(unsigned wg, int entries, int bloc
         entry = (int)(wg % (unsigned)entries);
         i = (int)(wg / (unsigned)entries);
     }
-    block = last_first ? blocks - 1 - i : i;
+    // (the same for every lane: into scalar registers, whatever the divisions
+    // were computed with)
+    entry = __builtin_amdgcn_readfirstlane(entry);
+    block = __builtin_amdgcn_readfirstlane(last_first ? blocks - 1 - i : i);
+}
+
+// The lane's index within its wavefront, asked of the hardware where it is
+// needed again after a long loop (the thread index the kernel started with
+// would have to sit in a register all the way through, and at head 128 there
+// is none to spare).  Does not depend on which lanes are active.
+__device__ __forceinline__ int lane_index_again()
+{
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
 }
 
 __device__ __forceinline__ int tile_row(int r, int half)
@@ -393,7 +407,21 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
     const bool q_ok = my_q < q_seq;
     // the lane's query: its row within the allocation that holds it (of Q, dA,
     // dQ, and of lse without the head axis), and its place among the row dots
-    int64_t q_elem = (int64_t)b * q_seq + (q_ok ? my_q : 0), d_idx = q_elem;
+    // (a function of the row, so that the stores at the end can work it out
+    // again instead of keeping it through the loop)
+    int own_t0 = 0, own_rows = q_seq;           // the tile that holds the block's rows
+    if constexpr(GRID)
+    {
+        const int q_tile = (int)p.q_tile;
+        own_t0 = __builtin_amdgcn_readfirstlane((q_row0 / q_tile) * q_tile);
+        own_rows = min(q_tile, q_seq - own_t0);
+    }
+    auto row_elem = [&](int row, bool ok) __attribute__((always_inline)) -> int64_t
+    {
+        return (int64_t)b * own_rows + ((ok ? row : (GRID ? q_row0 : 0)) - own_t0);
+    };
+    const int64_t q_elem = row_elem(my_q, q_ok);
+    int64_t d_idx = q_elem;
     const void *Q_own = p.Q, *dA_own = p.dA;
     void *dQ_own = p.dQ;
     const float *lse_own = p.lse;
@@ -401,8 +429,6 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
     {
         const int q_tile = (int)p.q_tile;
         const int tq = q_row0 / q_tile, t0 = tq * q_tile;
-        const int rows_t = min(q_tile, q_seq - t0);
-        q_elem = (int64_t)b * rows_t + ((q_ok ? my_q : q_row0) - t0);
         d_idx = d_slab + (int64_t)p.batch * t0 + q_elem;
         Q_own = p.Qt[q_tile0 + tq];
         dA_own = p.dAt[q_tile0 + tq];
@@ -570,7 +596,7 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
     const char *mask_wg = static_cast<const char *>(p.mask)
         + (int64_t)q_row0 * p.mask_ld * (int64_t)MASK_ES;
     const uint32_t mask_row_off = (uint32_t)(q_ok ? my_q - q_row0 : 0) * (uint32_t)p.mask_ld * MASK_ES;
-    const uint32_t mask_off = mask_row_off + (uint32_t)(4 * half) * MASK_ES;
+    const uint32_t mask_off_wg = mask_row_off + (uint32_t)(4 * half) * MASK_ES;
 
     // the workgroup's two query blocks of 64 against the key blocks 0 .. n_steps-1
     const StepSet steps = make_step_set(p, EXPLICIT, q_row0 / kBwdStep,
@@ -603,6 +629,14 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
         const int keys_here = min(kBwdStep, k_seq - kg0);
         const char *mask_step = mask_wg + (int64_t)kg0 * MASK_ES;
         const uint32_t mask_off_last = mask_row_off + (uint32_t)(keys_here - 1) * MASK_ES;
+        // (through an empty asm statement: the 32 offsets that a step adds
+        // constants to are then made where the step uses them instead of once
+        // before the loop and kept, which at head 128 means spilled)
+        uint32_t mask_off = mask_off_wg;
+        if(use_mask)
+        {
+            asm volatile("" : "+v"(mask_off));
+        }
 
         // ---- S^T = K Q^T, dP^T = V dA^T -------------------------------------------------
         // (one 32-key block at a time: half the accumulators live)
@@ -612,6 +646,7 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
         {
             lim = min(lim, my_lim - kg0);
         }
+        const int lim_less_half = lim - 4 * half;
         // (wave-common: the last key of the step against the last key that
         // exists and the last key the workgroup's first query sees)
         const bool bounds = keys_here < kBwdStep
@@ -652,8 +687,8 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
 #pragma unroll
                     for(int r = 0; r < 16; ++r)
                     {
-                        const int key = mb * 32 + tile_row(r, half);
-                        sv[r] = key <= lim ? sv[r] : neg_inf();
+                        // (key mb*32 + tile_row(r, half) <= lim, the lane's part on the right)
+                        sv[r] = mb * 32 + tile_row(r, 0) <= lim_less_half ? sv[r] : neg_inf();
                     }
                 }
                 float dsv[16];
@@ -766,8 +801,9 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
 #pragma unroll
                     for(int r = 0; r < 16; ++r)
                     {
-                        const int key = mb * 32 + tile_row(r, half);
-                        sv[mb][r] = key <= lim ? sv[mb][r] : neg_inf();
+                        // (key mb*32 + tile_row(r, half) <= lim, the lane's part on the right)
+                        sv[mb][r] = mb * 32 + tile_row(r, 0) <= lim_less_half ? sv[mb][r]
+                            : neg_inf();
                     }
                 }
             };
@@ -912,14 +948,17 @@ __device__ __forceinline__ void sdpa_bwd_dq_body(
     {
         return;
     }
-    uint16_t *dst = static_cast<uint16_t *>(dQ_own) + q_off;
+    const int lane_again = lane_index_again();
+    const int my_q_again = q_row0 + wave_u * 32 + (lane_again & 31);
+    const int half_again = lane_again >> 5;
+    uint16_t *dst = static_cast<uint16_t *>(dQ_own) + row_elem(my_q_again, true) * HEAD;
 #pragma unroll
     for(int db = 0; db < DBLOCKS; ++db)
     {
 #pragma unroll
         for(int rg = 0; rg < 4; ++rg)
         {
-            uint16_t *ptr = dst + db * 32 + 8 * rg + 4 * half;
+            uint16_t *ptr = dst + db * 32 + 8 * rg + 4 * half_again;
             float v[4];
 #pragma unroll
             for(int e = 0; e < 4; ++e)
@@ -978,7 +1017,7 @@ template<typename T, int HEAD, int MODE, int PART, bool GRID>
 __device__ __forceinline__ void sdpa_bwd_dkv_body(
         const std::conditional_t<GRID, BwdGridParams, BwdParams> &p, unsigned wg,
         char *lds_q0, char *lds_q1, char *lds_g0, char *lds_g1,
-        float (*lds_stat)[2][kBwdStep])
+        float (*lds_stat_arg)[2][kBwdStep])
 {
     constexpr bool DO_DK = (PART & BWD_PART_DK) != 0, DO_DV = (PART & BWD_PART_DV) != 0;
     constexpr bool BOTH = DO_DK && DO_DV;
@@ -1026,15 +1065,29 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
     const int nb = kvb % p.n_batch, hkv = kvb / p.n_batch;
     const int my_k = k_row0 + wave * 32 + col;
     const bool k_ok = my_k < k_seq;
+    // key kg is visible to query q0 + qr + 4*half iff kg - 4*half <= rel + q0 + qr
+    const int my_k_less_half = my_k - 4 * half;
     // the lane's key: its row within the allocation that holds it (of K, V, dK, dV)
-    int64_t k_elem = (int64_t)kvb * k_seq + (k_ok ? my_k : 0);
+    // (a function of the row, so that the stores at the end can work it out
+    // again instead of keeping it through the loop)
+    int own_t0 = 0, own_rows = k_seq;           // the tile that holds the block's rows
+    if constexpr(GRID)
+    {
+        const int k_tile = (int)p.k_tile;
+        own_t0 = __builtin_amdgcn_readfirstlane((k_row0 / k_tile) * k_tile);
+        own_rows = min(k_tile, k_seq - own_t0);
+    }
+    auto row_elem = [&](int row, bool ok) __attribute__((always_inline)) -> int64_t
+    {
+        return (int64_t)kvb * own_rows + ((ok ? row : (GRID ? k_row0 : 0)) - own_t0);
+    };
+    const int64_t k_elem = row_elem(my_k, k_ok);
     const void *K_own = p.K, *V_own = p.V;
     void *dK_own = p.dK, *dV_own = p.dV;
     if constexpr(GRID)
     {
         const int k_tile = (int)p.k_tile;
-        const int tk = k_row0 / k_tile, t0 = tk * k_tile;
-        k_elem = (int64_t)kvb * min(k_tile, k_seq - t0) + ((k_ok ? my_k : k_row0) - t0);
+        const int tk = k_row0 / k_tile;
         K_own = p.Kt[k_tile0 + tk];
         V_own = p.Vt[k_tile0 + tk];
         dK_own = p.dKt[k_tile0 + tk];
@@ -1092,7 +1145,13 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
     // flight, the next step's tile loads included: they go to LDS, whose reads
     // have a counter of their own.
     constexpr bool GOFF_IN_LDS = BOTH && HEAD > 64 && NNTILE_BWD_GOFF_IN_LDS != 0;
-    __shared__ uint32_t lds_goff[GOFF_IN_LDS ? 2 * LPW * kDkvThreads : 1];
+    // (the statistics of the two buffers behind them in the same array: one
+    // register, the thread's place in the array, then addresses all of it)
+    __shared__ __attribute__((aligned(16))) uint32_t lds_goff[GOFF_IN_LDS
+        ? (2 * LPW + 1) * kDkvThreads : 1];
+    static_assert(2 * 2 * kBwdStep <= kDkvThreads, "two buffers of statistics in one row of the table");
+    float (*lds_stat)[2][kBwdStep] = GOFF_IN_LDS
+        ? reinterpret_cast<float (*)[2][kBwdStep]>(lds_goff + 2 * LPW * kDkvThreads) : lds_stat_arg;
     if constexpr(GOFF_IN_LDS)
     {
 #pragma unroll
@@ -1144,9 +1203,9 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
     // for the rows of the lower and of the upper half of the wave (the
     // launcher keeps 64 rows of the mask within 32 bits)
     constexpr uint32_t MASK_ES = MODE == NNTILE_HIP_MASK_ADDITIVE ? 2u : 1u;
-    const uint32_t mask_row_bytes = (uint32_t)p.mask_ld * MASK_ES;
+    const uint32_t mask_row_bytes_wg = (uint32_t)p.mask_ld * MASK_ES;
     const uint32_t mask_off_lo = (uint32_t)(k_ok ? my_k : 0) * MASK_ES;
-    const uint32_t mask_off_hi = mask_off_lo + (uint32_t)(4 * half) * mask_row_bytes;
+    const uint32_t mask_off_hi = mask_off_lo + (uint32_t)(4 * half) * mask_row_bytes_wg;
     // the workgroup's key blocks of 64 against the query blocks
     // first_step .. n_steps-1, once per head of the group: walk position
     // i = head * 64K + query step
@@ -1252,7 +1311,7 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
             {
                 v = r > last ? 0.0f : -raw;
             }
-            stat[which][r] = v;
+            (&stat[0][0])[tid] = v;        // = stat[which][r]
         }
     };
     auto fetch_stat = [&](const QueryRows &at, int last, float (*stat)[kBwdStep])
@@ -1332,6 +1391,14 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
         // exists and the last key the step's first query sees)
         const bool bounds = k_row0 + kDkvRows > k_seq
             || (MODE == NNTILE_HIP_MASK_CAUSAL && k_row0 + kDkvRows - 1 > rel + q0);
+        // (the row stride through an empty asm statement: its multiples are
+        // then computed where a step uses them - 32 scalar products - instead
+        // of once before the loop and kept, which at head 128 means spilled)
+        uint32_t mask_row_bytes = mask_row_bytes_wg;
+        if(use_mask)
+        {
+            asm volatile("" : "+s"(mask_row_bytes));
+        }
         const char *mask_step = static_cast<const char *>(p.mask)
             + (int64_t)q0 * (int64_t)mask_row_bytes;
         const uint32_t mask_last_row = (uint32_t)(rows_here - 1) * mask_row_bytes;
@@ -1375,11 +1442,12 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
 #pragma unroll
                     for(int r = 0; r < 16; ++r)
                     {
-                        const int qr = mb * 32 + tile_row(r, half);
+                        // (the lane's part on the left, the rest is wave-common)
+                        const int qr = mb * 32 + tile_row(r, 0);
                         bool vis = k_ok;
                         if(MODE == NNTILE_HIP_MASK_CAUSAL)
                         {
-                            vis = vis && (my_k <= rel + q0 + qr);
+                            vis = vis && (my_k_less_half <= rel + q0 + qr);
                         }
                         sv[r] = vis ? sv[r] : neg_inf();
                     }
@@ -1527,11 +1595,12 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
 #pragma unroll
                     for(int r = 0; r < 16; ++r)
                     {
-                        const int qr = mb * 32 + tile_row(r, half);
+                        // (the lane's part on the left, the rest is wave-common)
+                        const int qr = mb * 32 + tile_row(r, 0);
                         bool vis = k_ok;
                         if(MODE == NNTILE_HIP_MASK_CAUSAL)
                         {
-                            vis = vis && (my_k <= rel + q0 + qr);
+                            vis = vis && (my_k_less_half <= rel + q0 + qr);
                         }
                         sv[r] = vis ? sv[r] : neg_inf();
                     }
@@ -1637,11 +1706,12 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
 #pragma unroll
                     for(int r = 0; r < 16; ++r)
                     {
-                        const int qr = mb * 32 + tile_row(r, half);
+                        // (the lane's part on the left, the rest is wave-common)
+                        const int qr = mb * 32 + tile_row(r, 0);
                         bool vis = k_ok;
                         if(MODE == NNTILE_HIP_MASK_CAUSAL)
                         {
-                            vis = vis && (my_k <= rel + q0 + qr);
+                            vis = vis && (my_k_less_half <= rel + q0 + qr);
                         }
                         sv[mb][r] = vis ? sv[mb][r] : neg_inf();
                     }
@@ -1926,16 +1996,20 @@ __device__ __forceinline__ void sdpa_bwd_dkv_body(
     {
         return;
     }
+    const int lane_again = lane_index_again();
+    const int my_k_again = k_row0 + wave_u * 32 + (lane_again & 31);
+    const int half_again = lane_again >> 5;
+    const int64_t k_off_again = row_elem(my_k_again, true) * HEAD;
     auto store = [&](void *base, const f32x16 (&acc)[DBLOCKS], float factor)
     {
-        uint16_t *dst = static_cast<uint16_t *>(base) + k_off;
+        uint16_t *dst = static_cast<uint16_t *>(base) + k_off_again;
 #pragma unroll
         for(int db = 0; db < DBLOCKS; ++db)
         {
 #pragma unroll
             for(int rg = 0; rg < 4; ++rg)
             {
-                uint16_t *ptr = dst + db * 32 + 8 * rg + 4 * half;
+                uint16_t *ptr = dst + db * 32 + 8 * rg + 4 * half_again;
                 float v[4];
 #pragma unroll
                 for(int e = 0; e < 4; ++e)

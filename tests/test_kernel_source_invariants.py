@@ -109,3 +109,26 @@ def test_forward_kernels_use_no_scratch_memory(assemblies):
         sizes = re.findall(r"\.private_segment_fixed_size:\s*(\d+)", assemblies[name])
         assert sizes, name
         assert all(int(x) <= limit for x in sizes), (name, sorted(set(sizes)))
+
+
+def test_backward_kernels_use_no_scratch_memory_without_an_explicit_mask(assemblies):
+    """The backward at head 128 holds K and V fragments and both accumulators
+    in 192 registers of a lane; what else lives through its loops was arranged
+    so that nothing spills in the kernels without a mask and with the causal
+    rule (every head size), and in every kernel below head 128.  The kernels
+    that read mask values at head 128 keep at most 28 dwords a lane in
+    scratch memory."""
+    text = assemblies["sdpa_bwd_16bit.hip"].split("amdhsa.kernels:")[1]
+    seen = 0
+    for entry in text.split(".agpr_count:")[1:]:
+        name = re.search(r"\.name:\s+(\S+)", entry).group(1)
+        size = int(re.search(r"\.private_segment_fixed_size:\s*(\d+)", entry).group(1))
+        m = re.match(r"_ZN10nntile_hip15sdpa_bwd_kernelINS_\w+?ELi(\d+)ELi(\d+)E", name)
+        if m is None:
+            assert size == 0, (name, size)
+            continue
+        seen += 1
+        head, mode = int(m.group(1)), int(m.group(2))
+        explicit = mode in (0, 3)           # NNTILE_HIP_MASK_ADDITIVE, NNTILE_HIP_MASK_BOOL
+        assert size <= (112 if explicit and head == 128 else 0), (name, size)
+    assert seen >= 48
