@@ -626,7 +626,7 @@ def bench_accumulate(cfg, steps, warmup):
             "frac_of_hbm_peak": round(nbytes / (dev * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
 
 
-def bench_kv_cache(cfg, steps, warmup):
+def bench_kv_cache(cfg, steps, warmup, one_launch_only=False):
     """One decode step through a preallocated key/value cache: the keys and
     values of the q_seq new tokens are appended (one launch for both), then
     the decode kernel reads the filled rows of the caches where they lie.  The
@@ -674,6 +674,16 @@ def bench_kv_cache(cfg, steps, warmup):
         fused[i[0] % nrot].launch()
         i[0] += 1
 
+    append_bytes = 2 * 2 * k_new.numel() * k_new.element_size()
+    nbytes = cfg.algorithmic_bytes() + append_bytes
+    if one_launch_only:
+        # (for the profiler: the launch that appends and attends, nothing else)
+        wall, dev_one = time_steps(one_launch, steps, warmup)
+        return {"what": "append %d new tokens + decode over %d cached rows of %s in one launch"
+                        % (cfg.q_seq, cfg.k_seq, cfg.name),
+                "ms_per_step": round(wall, 4), "device_ms_per_step": round(dev_one, 4),
+                "algorithmic_bytes": nbytes,
+                "frac_of_hbm_peak": round(nbytes / (dev_one * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
     wall, dev = time_steps(step, steps, warmup)
     _, dev_append = time_steps(append_only, steps, 2)
     _, dev_one = time_steps(one_launch, steps, 5)
@@ -691,8 +701,6 @@ def bench_kv_cache(cfg, steps, warmup):
         i[0] += 1
 
     _, dev_graph = time_steps(replay, steps, 5)
-    append_bytes = 2 * 2 * k_new.numel() * k_new.element_size()
-    nbytes = cfg.algorithmic_bytes() + append_bytes
     return {"what": "append %d new tokens + decode over %d cached rows of %s, cache capacity %d"
                     % (cfg.q_seq, cfg.k_seq, cfg.name, cap),
             "ms_per_step": round(wall, 4), "device_ms_per_step": round(dev, 4),
@@ -824,7 +832,7 @@ def main():
     ap.add_argument("--only", default=None,
                     help="run only this leg (for profiling): prefill | prefill_128_queries | cfg5 | cfg2 | decode | decode_separate_merge | decode_wide | decode_fp32 | "
                          "reference_api | reference_grid | power_context | copy_context | backward | backward_slabs | rope | transpose | accumulate | "
-                         "kv_cache | copy")
+                         "kv_cache | kv_cache_one_launch | copy")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py: this path runs on ONE GPU; --gpus %d is not supported "
@@ -873,7 +881,8 @@ def main():
                 __import__("dataclasses").replace(BY_NAME["cfg2_gpt2_small_fp32"],
                                                   name="cfg2_shape_in_bf16", dtype="bf16"),
                 args.steps, args.warmup),
-            "kv_cache": lambda: bench_kv_cache(cfg4, args.steps, args.warmup)}
+            "kv_cache": lambda: bench_kv_cache(cfg4, args.steps, args.warmup),
+            "kv_cache_one_launch": lambda: bench_kv_cache(cfg4, args.steps, args.warmup, True)}
     if only == "copy":
         # calibration leg for the HBM traffic counters: a plain device copy
         # of 1 GiB (reads 2^30 bytes, writes 2^30 bytes per launch)
