@@ -673,7 +673,7 @@ def _append_cache_call(k_new, v_new, K_cache, V_cache, k_seq, Q, mask, lse, A, m
     a = _cache_args(K_cache, V_cache, k_seq, Q, mask, lse, A, mask_mode, n_batch, kv_group,
                     q_pos0, k_pos0, causal_offset, flags)
     fn = getattr(lib(), "nntile_hip_sdpa_fwd_decode_append_cache_" + dtype_name(Q))
-    nbytes = workspace.numel() * workspace.element_size()
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     extra = (K_cache.shape[1], _ptr(k_new), _ptr(v_new), rows, _ptr(workspace), nbytes)
     return fn, a, extra
 
