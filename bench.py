@@ -35,6 +35,8 @@ TRAFFIC = {
     "cfg3_llama_prefill_bf16": (176977920, "profiles/sdpa_prefill_16bit_kernel_cfg3_llama_prefill_bf16.txt"),
     "cfg4_gqa_decode_bf16": (288403456, "profiles/sdpa_decode_16bit_kernel_cfg4_gqa_decode_bf16.txt"),
     "cfg2_gpt2_small_fp32": (55549952, "profiles/sdpa_prefill_fp32_kernel_cfg2_gpt2_small_fp32.txt"),
+    # row dots (64 MiB read, 0.5 MiB written) + the gradient launch (488.9 MiB read, 96.1 MiB written)
+    "cfg3_backward": (680994816, "profiles/sdpa_bwd_kernels_cfg3_llama_prefill_bf16.txt"),
 }
 
 
@@ -486,7 +488,7 @@ def bench_backward(cfg, steps, warmup):
             "what": "backward of %s in one call (row dots + one launch for dQ, dK, dV), analytic "
                     "causal mask, gradients written; 2.5 x the forward's causal-exact FLOPs" % cfg.name,
             "roofline": roofline("mfma", "sdpa_bwd_rowdot_kernel + sdpa_bwd_kernel<bf16,128,causal>",
-                                 fl, dev, PEAK_BF16_TFLOPS, "TFLOP/s"),
+                                 fl, dev, PEAK_BF16_TFLOPS, "TFLOP/s", TRAFFIC["cfg3_backward"]),
             "reference_tiling": {
                 "what": "the same over %d x %d separately allocated tiles of %d rows, gradients "
                         "added to the tiles: nntile_hip_sdpa_bwd_grid, one call for all tile pairs "
