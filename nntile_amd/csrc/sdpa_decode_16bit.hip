@@ -6,9 +6,14 @@
 //    together (rows = kv_group * q_seq <= 64), so K and V are read once, not
 //    once per query head;
 //  * the key axis of each (batch entry, kv head) unit is split over
-//    workgroups so that every CU streams; each workgroup writes an
-//    un-normalised partial (max, sum, O) and a second small kernel merges the
-//    partials and folds them into the running (lse, A) pair;
+//    workgroups so that every CU streams; each workgroup writes a partial
+//    (the output normalised and rounded to the tile type, max and sum in
+//    fp32), and merge workgroups at the end of the same grid - or a second
+//    small kernel - merge the partials and fold them into the running
+//    (lse, A) pair; a unit with a single split writes (lse, A) itself;
+//  * rows that are being appended to a cache by the same call are read from
+//    the caller's tensors, and one more workgroup per unit at the very end
+//    of the grid copies them into the caches;
 //  * K and V steps go from global memory straight into LDS (global_load_lds,
 //    16 bytes per lane, 1 KB contiguous per instruction, no registers in
 //    between) through a ring of STAGES buffers, so that STAGES-1 steps of 32 KB

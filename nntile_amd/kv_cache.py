@@ -11,7 +11,8 @@ into fresh dense tensors before every attention call (`k_partial`,
 `v_partial`) and materialises a bool mask slice for the new queries; here
 `attend` hands the caches to the decode kernel with their capacity and the
 visibility rule `key <= query + (len - q_seq)`, so a decode step reads the
-filled rows once and writes only the new ones.
+filled rows once and writes only the new ones; `append_attend` does the
+append and the attention of a decode step in one launch.
 
 Tensors are C-ordered torch device tensors: K, V `[entries, seq, head]`
 (entries = n_batch * n_head_kv, NNTile's `[head, seq, n_batch, n_head_kv]`),
