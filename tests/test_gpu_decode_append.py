@@ -133,3 +133,35 @@ def test_cache_object_steps_one_launch_against_two(dtype):
         assert np.array_equal(res[0][0], res[1][0]) and np.array_equal(res[0][1], res[1][1])
         assert np.array_equal(_bits(a.k[:, :pos]), _bits(b.k[:, :pos]))
         assert np.array_equal(_bits(a.v[:, :pos]), _bits(b.v[:, :pos]))
+
+
+def test_cache_object_on_a_side_stream():
+    """append_attend enqueued on a stream of its own (default priority) while
+    the default stream is busy with something else: same bits as on the
+    default stream."""
+    n_batch, group, n_kv, head, cap = 2, 4, 4, 128, 96
+    batch, kvb = n_batch * group * n_kv, n_batch * n_kv
+    (Q, K, V), _ = H.make_qkv(13, batch, cap, cap, head, "bf16", kv_batch=kvb)
+    Qd, Kd, Vd = Q.cuda(), K.cuda(), V.cuda()
+    side = torch.cuda.Stream()
+    out = []
+    for stream in (None, side):
+        cache = KVCache(cap)
+        cache.append(Kd[:, :40].contiguous(), Vd[:, :40].contiguous())
+        torch.cuda.synchronize()
+        res, pos = [], 40
+        for chunk in (1, 16, 1, 3):
+            kn, vn = Kd[:, pos:pos + chunk].contiguous(), Vd[:, pos:pos + chunk].contiguous()
+            q = Qd[:, pos:pos + chunk].contiguous()
+            lse, A = H.fresh_outputs(batch, chunk, head, "bf16")
+            torch.cuda.synchronize()
+            busy = torch.ones(1 << 22, device="cuda").cumsum(0)      # the default stream's own work
+            cache.append_attend(kn, vn, q, lse, A, n_batch, group, stream=stream)
+            torch.cuda.synchronize()
+            res.append((_bits(lse), _bits(A)))
+            pos += chunk
+            del busy
+        out.append((res, _bits(cache.k[:, :pos]), _bits(cache.v[:, :pos])))
+    for (a_lse, a_A), (b_lse, b_A) in zip(out[0][0], out[1][0]):
+        assert np.array_equal(a_lse, b_lse) and np.array_equal(a_A, b_A)
+    assert np.array_equal(out[0][1], out[1][1]) and np.array_equal(out[0][2], out[1][2])
