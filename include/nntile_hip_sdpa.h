@@ -537,13 +537,17 @@ int nntile_hip_sdpa_fwd_decode_cache_fp32(void *stream, const nntile_hip_sdpa_ti
  * after the call the caches are what nntile_hip_kv_cache_append_* would have
  * made them, and (lse, A) what nntile_hip_sdpa_fwd_decode_cache_* would then
  * have computed, bit for bit.  NNTILE_HIP_EINVAL when rows_new exceeds k_seq
- * or the capacity is smaller than k_seq. */
+ * or the capacity is smaller than k_seq.  The fp32 form is the fp32 decode
+ * kernel with the same two additions. */
 int nntile_hip_sdpa_fwd_decode_append_cache_bf16(void *stream,
         const nntile_hip_sdpa_tile_args *args, int64_t capacity, const uint16_t *k_new,
         const uint16_t *v_new, int64_t rows_new, void *workspace, size_t workspace_bytes);
 int nntile_hip_sdpa_fwd_decode_append_cache_fp16(void *stream,
         const nntile_hip_sdpa_tile_args *args, int64_t capacity, const uint16_t *k_new,
         const uint16_t *v_new, int64_t rows_new, void *workspace, size_t workspace_bytes);
+int nntile_hip_sdpa_fwd_decode_append_cache_fp32(void *stream,
+        const nntile_hip_sdpa_tile_args *args, int64_t capacity, const float *k_new,
+        const float *v_new, int64_t rows_new, void *workspace, size_t workspace_bytes);
 
 /* nntile_hip_sdpa_fwd_tile_* reading the cache the same way, for what the
  * decode form does not take: fp32 caches (the reference runs forward_dynamic

@@ -567,8 +567,15 @@ static void decode_fp32_geometry(const nntile_hip_sdpa_tile_args *a, int &units,
 }
 
 static int decode_fp32_call(void *stream, const nntile_hip_sdpa_tile_args *a,
-        int64_t kv_rows, void *workspace, size_t workspace_bytes)
+        int64_t kv_rows, void *workspace, size_t workspace_bytes,
+        const void *k_new = nullptr, const void *v_new = nullptr, int64_t n_new = 0)
 {
+    if(n_new != 0 && (a == nullptr || n_new < 0 || n_new > a->k_seq || n_new > 0x7fffffff
+                || k_new == nullptr || v_new == nullptr || !aligned16(k_new)
+                || !aligned16(v_new)))
+    {
+        return NNTILE_HIP_EINVAL;
+    }
     if(!decode_args_ok(a) || kv_rows < a->k_seq || !mode_ok(a->mask_mode) || a->K == nullptr
             || a->Q == nullptr || a->V == nullptr || a->lse == nullptr
             || a->A == nullptr || !aligned16(a->K) || !aligned16(a->Q)
@@ -619,6 +626,9 @@ static int decode_fp32_call(void *stream, const nntile_hip_sdpa_tile_args *a,
     p.overwrite = (a->flags & NNTILE_HIP_SDPA_OVERWRITE) ? 1 : 0;
     p.steps_per_split = (n_steps + splits - 1) / splits;
     p.scale = 1.0f / sqrtf(static_cast<float>(a->head));
+    p.k_new = k_new;
+    p.v_new = v_new;
+    p.n_new = (int32_t)n_new;
     return launch_decode_fp32(static_cast<hipStream_t>(stream), p, (int)a->head, a->mask_mode);
 }
 
@@ -1423,6 +1433,14 @@ int nntile_hip_sdpa_fwd_decode_append_cache_fp16(void *stream,
 {
     return decode_call(DType::fp16, stream, args, capacity, workspace, workspace_bytes, k_new,
             v_new, rows_new);
+}
+
+int nntile_hip_sdpa_fwd_decode_append_cache_fp32(void *stream,
+        const nntile_hip_sdpa_tile_args *args, int64_t capacity, const float *k_new,
+        const float *v_new, int64_t rows_new, void *workspace, size_t workspace_bytes)
+{
+    return decode_fp32_call(stream, args, capacity, workspace, workspace_bytes, k_new, v_new,
+            rows_new);
 }
 
 int nntile_hip_sdpa_fwd_decode_cache_fp32(void *stream, const nntile_hip_sdpa_tile_args *args,

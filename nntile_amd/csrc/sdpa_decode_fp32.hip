@@ -81,6 +81,32 @@ void sdpa_decode_fp32_kernel(const DecodeParams p)
     const int col = lane & 15;       // row (query) within the wavefront; key within a block for operand reads
     const int quad = lane >> 4;      // 0..3
 
+    // Behind the units x splits attention workgroups the grid holds, when rows
+    // are being appended to the caches by this call, one copying workgroup per
+    // unit: the new rows into the caches, 16 bytes a thread and piece.  Nobody
+    // in this launch reads them there (the attention takes them from k_new /
+    // v_new), so there is nothing to wait for or to signal.
+    {
+        const int n_main = p.n_batch * p.n_head_kv * p.n_splits;
+        if((int)blockIdx.x >= n_main)
+        {
+            const int unit_a = (int)blockIdx.x - n_main;
+            const int64_t filled = p.k_seq - p.n_new;
+            const int n16 = p.n_new * (RB / 16);
+            for(int t = tid; t < 2 * n16; t += kDecF32Threads)
+            {
+                const int which = t >= n16 ? 1 : 0;
+                const int piece = t - which * n16;
+                const char *src = static_cast<const char *>(which ? p.v_new : p.k_new)
+                    + ((int64_t)unit_a * p.n_new * RB + (int64_t)piece * 16);
+                char *dst = static_cast<char *>(const_cast<void *>(which ? p.V : p.K))
+                    + (((int64_t)unit_a * p.kv_rows + filled) * RB + (int64_t)piece * 16);
+                *reinterpret_cast<f32x4 *>(dst) = *reinterpret_cast<const f32x4 *>(src);
+            }
+            return;
+        }
+    }
+
     // Workgroups go round the 8 XCDs in index order: all key splits of a unit
     // get indices that are equal modulo 8, i.e. one XCD and one L2 for the
     // unit's K/V (the four wavefronts' query heads read them once).
@@ -173,6 +199,28 @@ void sdpa_decode_fp32_kernel(const DecodeParams p)
         char *kdst = slot_base + wave_u * LOADS_PER_WAVE * 1024;
         char *vdst = kdst + K_BYTES;
         const int last = (int)min((int64_t)kDecF32Keys, p.k_seq - row0) - 1;
+        if(p.n_new > 0 && row0 + kDecF32Keys > p.k_seq - p.n_new)
+        {
+            // some rows of this step are new tokens: they are not in the caches
+            // yet and are read from where the caller holds them (rows past
+            // the end clamped to the last row, as below)
+            const int64_t filled = p.k_seq - p.n_new;
+            const char *Kn = static_cast<const char *>(p.k_new) + (int64_t)unit * p.n_new * RB;
+            const char *Vn = static_cast<const char *>(p.v_new) + (int64_t)unit * p.n_new * RB;
+#pragma unroll
+            for(int i = 0; i < LOADS_PER_WAVE; ++i)
+            {
+                const int64_t g = min(row0 + ld_row[i], p.k_seq - 1);
+                const uint32_t kc = k_goff[i] - (uint32_t)(ld_row[i] * RB);     // the chunk within the row
+                const uint32_t vc = v_goff[i] - (uint32_t)(ld_row[i] * RB);
+                const bool fresh = g >= filled;
+                const char *ks = fresh ? Kn + (g - filled) * RB : Kb + g * RB;
+                const char *vs = fresh ? Vn + (g - filled) * RB : Vb + g * RB;
+                load_to_lds16<0, true>(ks + kc, kdst + i * 1024);
+                load_to_lds16<0, true>(vs + vc, vdst + i * 1024);
+            }
+            return;
+        }
 #pragma unroll
         for(int i = 0; i < LOADS_PER_WAVE; ++i)
         {
@@ -526,7 +574,9 @@ template<int HEAD>
 static int launch_decode_fp32_head(hipStream_t stream, const DecodeParams &p, int mode)
 {
     const int units = p.n_batch * p.n_head_kv;
-    const dim3 grid((unsigned)(units * p.n_splits)), block(kDecF32Threads);
+    // (one more workgroup per unit when the call appends rows to the caches)
+    const dim3 grid((unsigned)(units * p.n_splits + (p.n_new > 0 ? units : 0))),
+        block(kDecF32Threads);
     switch(mode)
     {
         case NNTILE_HIP_MASK_ADDITIVE:

@@ -128,7 +128,7 @@ EXPORTS = (
     + ["nntile_hip_transpose_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_kv_cache_append_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_fwd_decode_cache_" + t for t in ("bf16", "fp16", "fp32")]
-    + ["nntile_hip_sdpa_fwd_decode_append_cache_" + t for t in ("bf16", "fp16")]
+    + ["nntile_hip_sdpa_fwd_decode_append_cache_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_sdpa_fwd_tile_cache_" + t for t in ("bf16", "fp16", "fp32")]
     + ["nntile_hip_mask_tile_class_" + t for t in ("bf16", "fp16", "fp32", "bool")]
     + ["nntile_hip_sdpa_fwd_grid_codelet_" + t for t in ("bf16", "fp16", "fp32")]
@@ -171,10 +171,11 @@ def lib():
             f = getattr(L, "nntile_hip_sdpa_fwd_decode_cache_" + t)
             f.argtypes = [_vp, ctypes.POINTER(TileArgs), _i64, _vp, ctypes.c_size_t]
             f.restype = ctypes.c_int
-        for t in ("bf16", "fp16"):
+        for t in ("bf16", "fp16", "fp32"):
             f = getattr(L, "nntile_hip_sdpa_fwd_decode_append_cache_" + t)
             f.argtypes = [_vp, ctypes.POINTER(TileArgs), _i64, _vp, _vp, _i64, _vp, ctypes.c_size_t]
             f.restype = ctypes.c_int
+        for t in ("bf16", "fp16"):
             f = getattr(L, "nntile_hip_flash_sdpa_bwd_" + t)
             f.argtypes = [_vp, _i64, _i64, _i64] + [_vp] * 13
             f.restype = ctypes.c_int
@@ -683,7 +684,7 @@ def sdpa_fwd_decode_append_cache(k_new, v_new, K_cache, V_cache, k_seq, Q, mask,
                                  causal_offset=0, flags=0, stream=None):
     """kv_cache_append of k_new, v_new ([entries, rows, head]) behind the
     k_seq - rows filled rows of the caches and sdpa_fwd_decode_cache over the
-    k_seq rows, in one launch (16-bit types)."""
+    k_seq rows, in one launch."""
     fn, a, extra = _append_cache_call(k_new, v_new, K_cache, V_cache, k_seq, Q, mask, lse, A,
                                       mask_mode, n_batch, kv_group, workspace, q_pos0, k_pos0,
                                       causal_offset, flags)

@@ -66,12 +66,11 @@ class KVCache:
     def append_attend(self, k_partial, v_partial, Q, lse, A, n_batch, kv_group, causal=True,
                       mask=None, stream=None):
         """`append` followed by `attend`, same results bit for bit; on the
-        decode kernel's shapes with a 16-bit type the two are ONE launch (the
+        decode kernels' shapes the two are ONE launch (the
         attention reads the new rows from k_partial / v_partial while other
         workgroups of the launch write them into the caches)."""
         rows, q_seq = k_partial.shape[1], Q.shape[1]
         one_launch = (self.k is not None and v_partial.shape[1] == rows
-                      and Q.dtype in (torch.bfloat16, torch.float16)
                       and kv_group * q_seq <= 64 and Q.shape[2] in (64, 128)
                       and rows + self.k_cache_size <= self.max_cache_size
                       and k_partial.is_contiguous() and v_partial.is_contiguous())

@@ -54,7 +54,7 @@ def _two_ways(dtype, q_seq, rows_new, k_seq, cap, n_batch, group, n_kv, head, mo
     return out
 
 
-@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
 @pytest.mark.parametrize("q_seq,rows_new,k_seq,cap,n_batch,group,n_kv,head", [
     (16, 16, 512, 1024, 2, 4, 4, 128),      # new rows fill the last part of a key step
     (1, 1, 300, 301, 3, 4, 2, 128),         # one token, ragged last step, units not a multiple of 8
@@ -104,7 +104,7 @@ def test_refusals_leave_everything_alone():
     assert np.array_equal(_bits(A), before)
 
 
-@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
 def test_cache_object_steps_one_launch_against_two(dtype):
     """Token by token through two KVCache objects, one with append + attend,
     one with append_attend: same caches, same outputs at every step."""
