@@ -412,12 +412,14 @@ def bench_reference_api(cfg, steps, warmup):
     return out
 
 
-def bench_decode(cfg, steps, warmup, more_flags=0, fp32=False):
+def bench_decode(cfg, steps, warmup, more_flags=0, fp32=False, settle_s=0.0):
     """The GQA decode shape: one launch per step (the key splits of a unit
     are merged inside it).  Four (K, V) sets rotate (4 x 256 MiB at cfg4: the
     256 MiB last-level cache cannot serve a pass).  more_flags: further flags
     of the decode call (the merge as a second launch).  fp32: the same shape
-    on fp32 tiles through the fp32 decode kernel (twice the bytes)."""
+    on fp32 tiles through the fp32 decode kernel (twice the bytes).
+    settle_s: seconds of the same step run untimed before the warm-up steps
+    (the first loop of a process runs before the clocks have settled)."""
     import torch
     from nntile_amd import hip_sdpa as h
     kvb = cfg.n_batch * cfg.n_head_kv
@@ -439,6 +441,12 @@ def bench_decode(cfg, steps, warmup, more_flags=0, fp32=False):
         plans[i[0] % nrot].launch()
         i[0] += 1
 
+    if settle_s > 0:
+        t_end = time.perf_counter() + settle_s
+        while time.perf_counter() < t_end:
+            for _ in range(50):
+                step()
+            torch.cuda.synchronize()
     wall, dev = time_steps(step, steps, warmup)
     nbytes = cfg.algorithmic_bytes()
     if fp32:
@@ -906,7 +914,7 @@ def main():
     steps = max(20, args.steps)
     warmup = max(5, args.warmup)
     few = max(20, args.steps // 5)
-    dec = bench_decode(cfg4, max(steps, 100), max(warmup, 20))
+    dec = bench_decode(cfg4, max(steps, 100), max(warmup, 20), settle_s=0.3)
     ref_api = bench_reference_api(cfg3, few, 5)
     backward = bench_backward(cfg3, max(20, args.steps // 10), 5)
     detail = {}
