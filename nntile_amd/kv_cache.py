@@ -78,13 +78,12 @@ class KVCache:
             self.append(k_partial, v_partial, stream=stream)
             self.attend(Q, lse, A, n_batch, kv_group, causal=causal, mask=mask, stream=stream)
             return
-        self.k_cache_size += rows
-        self.v_cache_size += rows
-        k_seq = self.k_cache_size
+        k_seq = self.k_cache_size + rows
         mode = hip_sdpa.MASK_CAUSAL if causal else hip_sdpa.MASK_NONE
         sliced = None
         if mask is not None:
-            sliced, mode = self.mask_slice(mask, q_seq), hip_sdpa.MASK_BOOL
+            # (the slice that goes with the cache as it will be after the append)
+            sliced, mode = self._mask_slice_for(mask, q_seq, k_seq), hip_sdpa.MASK_BOOL
         if stream is not None:
             for t in (sliced, k_partial, v_partial):
                 if t is not None:
@@ -94,6 +93,9 @@ class KVCache:
         hip_sdpa.sdpa_fwd_decode_append_cache(
             k_partial, v_partial, self.k, self.v, k_seq, Q, sliced, lse, A, mode, n_batch, kv_group,
             workspace, causal_offset=k_seq - q_seq, flags=hip_sdpa.OVERWRITE, stream=stream)
+        # (only now: a refused call leaves the cache as it was)
+        self.k_cache_size += rows
+        self.v_cache_size += rows
 
     def _decode_workspace(self, k_seq, Q, n_batch, kv_group, stream):
         need = hip_sdpa.decode_cache_workspace_bytes(k_seq, Q, n_batch, kv_group)
@@ -130,7 +132,10 @@ class KVCache:
         [q_seq, len] is used as it is; otherwise everything is visible except
         where the mask, read at query position len - q_seq + j, says
         otherwise."""
-        k_seq = len(self)
+        return self._mask_slice_for(mask, q_seq, len(self))
+
+    @staticmethod
+    def _mask_slice_for(mask, q_seq, k_seq):
         if tuple(mask.shape) == (q_seq, k_seq):
             return mask.contiguous()
         out = torch.ones((q_seq, k_seq), dtype=torch.bool, device=mask.device)

@@ -165,3 +165,39 @@ def test_cache_object_on_a_side_stream():
     for (a_lse, a_A), (b_lse, b_A) in zip(out[0][0], out[1][0]):
         assert np.array_equal(a_lse, b_lse) and np.array_equal(a_A, b_A)
     assert np.array_equal(out[0][1], out[1][1]) and np.array_equal(out[0][2], out[1][2])
+
+
+def test_cache_object_with_a_mask_given_as_values():
+    """append_attend with a bool mask of the whole sequence (a window): the
+    slice that goes with the cache AFTER the append, same bits as append +
+    attend; a refused call leaves the cache object as it was."""
+    n_batch, group, n_kv, head, cap = 1, 4, 8, 64, 80
+    batch, kvb = n_batch * group * n_kv, n_batch * n_kv
+    (Q, K, V), _ = H.make_qkv(17, batch, cap, cap, head, "fp16", kv_batch=kvb)
+    Qd, Kd, Vd = Q.cuda(), K.cuda(), V.cuda()
+    i, j = np.arange(cap)[:, None], np.arange(cap)[None, :]
+    mask = torch.from_numpy((j <= i) & (i - j <= 24)).cuda()
+    a, b = KVCache(cap), KVCache(cap)
+    pos = 0
+    for chunk in (30, 1, 7, 1, 16):
+        kn, vn = Kd[:, pos:pos + chunk].contiguous(), Vd[:, pos:pos + chunk].contiguous()
+        q = Qd[:, pos:pos + chunk].contiguous()
+        res = []
+        for cache, fused in ((a, False), (b, True)):
+            lse, A = H.fresh_outputs(batch, chunk, head, "fp16")
+            if fused:
+                cache.append_attend(kn, vn, q, lse, A, n_batch, group, causal=False, mask=mask)
+            else:
+                cache.append(kn, vn)
+                cache.attend(q, lse, A, n_batch, group, causal=False, mask=mask)
+            torch.cuda.synchronize()
+            res.append((_bits(lse), _bits(A)))
+        pos += chunk
+        assert len(a) == len(b) == pos
+        assert np.array_equal(res[0][0], res[1][0]) and np.array_equal(res[0][1], res[1][1])
+    # 25 rows left; 26 are refused by the two-launch path taken for them, and nothing moves
+    kn = Kd[:, :26].contiguous()
+    lse, A = H.fresh_outputs(batch, 26, head, "fp16")
+    with pytest.raises(hip_sdpa.SdpaError):
+        b.append_attend(kn, kn, Qd[:, :26].contiguous(), lse, A, n_batch, group)
+    assert len(b) == pos
