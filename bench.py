@@ -759,7 +759,8 @@ DETAIL_FILE = os.path.join("gpurun_out", "bench_detail.json")
 LINE_LIMIT = 4000     # bytes; the driver keeps only the tail of stdout
 
 
-def compact_line(main_leg, dec, ref_api, backward, gemm, cpu, args, cfg3, cfg4, watts=None):
+def compact_line(main_leg, dec, ref_api, backward, gemm, cpu, args, cfg3, cfg4, watts=None,
+                 kv_cache=None):
     """The ONE line printed last: the headline, both rooflines, the
     reference-signature path, the backward and the CPU baseline.  Everything
     else goes to DETAIL_FILE."""
@@ -814,6 +815,13 @@ def compact_line(main_leg, dec, ref_api, backward, gemm, cpu, args, cfg3, cfg4, 
         out["backward"] = {"ms_per_step": backward["ms_per_step"],
                            "frac": backward["roofline"]["frac"],
                            "kernel_ms": backward["roofline"]["kernel_ms"]}
+    if kv_cache is not None:
+        # the decode step through the key/value cache: append + decode as two
+        # launches and as one
+        out["decode"]["through_cache"] = {
+            "two_launches_ms": kv_cache["device_ms_per_step"],
+            "one_launch_ms": kv_cache["one_launch_device_ms_per_step"],
+            "one_launch_frac": kv_cache["one_launch_frac_of_hbm_peak"]}
     if cpu is not None:
         out["cpu_baseline"] = {"value": round(cpu["value"], 5), "unit": cpu["unit"], "cores": cpu["cores"],
                                "kind": cpu["kind"], "sample": cpu["sample"],
@@ -987,7 +995,8 @@ def main():
     with PowerSampler() as ps:
         main_leg = bench_prefill(cfg3, args.steps, args.warmup, settle_s=0.3)
     cpu = None if args.no_cpu else cpu_baseline(cfg3)
-    line = compact_line(main_leg, dec, ref_api, backward, gemm, cpu, args, cfg3, cfg4, ps.watts())
+    line = compact_line(main_leg, dec, ref_api, backward, gemm, cpu, args, cfg3, cfg4, ps.watts(),
+                        detail.get("kv_cache"))
     if not args.brief:
         detail = dict({"headline": json.loads(line), "per_task_path": ref_api, "backward": backward,
                        "decode": dec}, **detail)

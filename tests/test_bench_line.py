@@ -33,9 +33,12 @@ def test_result_line_is_short_and_complete():
            "sample": "16 of 32 (batch,head) slabs of cfg3_llama_prefill_bf16 x 1 passes, all 4096 "
                      "queries, key tiles of 1024; FLOPs counted causal-exact as for the GPU (the CPU "
                      "path computes the dense score matrix)", "seconds": 15.912345}
-    line = b.compact_line(main_leg, dec, ref_api, backward, gemm, cpu, args, cfg3, cfg4, 1300.0)
+    kv = {"device_ms_per_step": 0.0531, "one_launch_device_ms_per_step": 0.0487,
+          "one_launch_frac_of_hbm_peak": 0.6971}
+    line = b.compact_line(main_leg, dec, ref_api, backward, gemm, cpu, args, cfg3, cfg4, 1300.0, kv)
     assert "\n" not in line and len(line) < b.LINE_LIMIT <= 4096
     out = json.loads(line)
+    assert out["decode"]["through_cache"]["one_launch_ms"] == 0.0487
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
                 "higher_is_better", "scaling", "vs_baseline", "dtype", "data", "config", "roofline",
                 "decode", "cpu_baseline"):
